@@ -1,0 +1,14 @@
+"""MI355X (gfx950) implementation of craftax.cu's batched policy path.
+
+The product is libcfpolicy.so (hand-written HIP behind the C ABI of
+include/cfp.h); this package is the thin host-side mirror of the reference's
+CuPolicy call surface used by the tests and the benchmark.  Importing it loads
+the shared library and fails if it has not been built.
+"""
+from . import _lib
+from . import policy
+from .policy import Policy, lib
+
+lib()  # fail at import time, not at first use, when the HIP library is missing
+
+__all__ = ["Policy", "policy", "lib", "_lib"]

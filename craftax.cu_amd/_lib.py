@@ -1,0 +1,76 @@
+"""ctypes binding of libcfpolicy.so (the C ABI declared in include/cfp.h).
+
+The library is built in-tree by build.py (hipcc --offload-arch=gfx950).  There
+is no fallback: if the shared object is missing or a symbol is absent the
+import fails, so a GPU run can never silently measure something else.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libcfpolicy.so")
+
+c_f32p = C.POINTER(C.c_float)
+c_u8p = C.POINTER(C.c_uint8)
+vp = C.c_void_p
+
+# name -> (restype, argtypes); one entry per declaration in include/cfp.h
+PROTOTYPES = {
+    "cfp_last_error": (C.c_char_p, []),
+    "cfp_abi_version": (C.c_int, []),
+    "cfp_policy_create": (C.c_int, [C.POINTER(vp), C.c_int, C.c_int, C.c_uint64]),
+    "cfp_policy_destroy": (None, [vp]),
+    "cfp_policy_num_envs": (C.c_int, [vp]),
+    "cfp_policy_layers": (C.c_int, [vp]),
+    "cfp_policy_param_count": (C.c_size_t, [vp]),
+    "cfp_policy_set_params": (C.c_int, [vp, vp, C.c_size_t]),
+    "cfp_policy_get_params": (C.c_int, [vp, vp, C.c_size_t]),
+    "cfp_policy_refresh_weights": (C.c_int, [vp, vp]),
+    "cfp_policy_params": (vp, [vp]),
+    "cfp_policy_state": (vp, [vp]),
+    "cfp_policy_rec": (vp, [vp]),
+    "cfp_policy_h_enc": (vp, [vp]),
+    "cfp_policy_h3": (vp, [vp]),
+    "cfp_policy_logits": (vp, [vp]),
+    "cfp_policy_stream": (vp, [vp]),
+    "cfp_encode_step": (C.c_int, [vp, vp, C.c_int, vp]),
+    "cfp_gru_chain": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int, C.c_int, vp]),
+    "cfp_head": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "cfp_policy_forward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int,
+                                     C.c_int, vp]),
+    "cfp_gemm_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
+    "cfp_gemm_enc_fwd": (C.c_int, [C.c_int, vp, vp, vp, vp]),
+    "cfp_gemm_dh": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),
+    "cfp_gemm_dw": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),
+    "cfp_gemv_dwv": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "cfp_expand_obs": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int,
+                                 C.c_int, vp]),
+    "cfp_add_bias": (C.c_int, [vp, vp, C.c_int, vp]),
+    "cfp_mingru_epi_fwd": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int, vp]),
+    "cfp_record_obs": (C.c_int, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp,
+                                 C.c_int, vp]),
+    "cfp_synth_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),
+}
+
+
+class CfpError(RuntimeError):
+    pass
+
+
+def load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import "
+            "__graft_entry__ as g; g.build()'` (hipcc, gfx950); there is no "
+            "CPU fallback for the policy path")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in PROTOTYPES.items():
+        fn = getattr(lib, name)   # AttributeError = header/library mismatch
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def check(lib, rc):
+    if rc != 0:
+        raise CfpError(lib.cfp_last_error().decode("utf-8", "replace"))

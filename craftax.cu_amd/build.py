@@ -1,0 +1,43 @@
+"""In-tree build of libcfpolicy.so for gfx950 (hipcc cross-compiles without a GPU)."""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OUT = os.path.join(HERE, "libcfpolicy.so")
+SOURCES = ["policy_forward.hip", "cfp_api.hip", "gemm.hip", "record.hip"]
+ARCH = "gfx950"
+
+
+def hipcc_path():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (looked at $HIPCC, PATH, /opt/rocm/bin)")
+
+
+def build(verbose=False):
+    """Compile every HIP source into one shared library; always recompiles."""
+    cmd = [
+        hipcc_path(), f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
+        "-shared", "-Wall", "-Wno-unused-function",
+        # packed fp32 VALU ops are kept off for gfx950 device code
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-o", OUT,
+    ] + [os.path.join(CSRC, s) for s in SOURCES]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return OUT
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

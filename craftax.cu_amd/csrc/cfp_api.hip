@@ -1,0 +1,351 @@
+// C ABI: policy object lifetime, parameter upload, and the forward entry
+// points.  Host-side mirror of the reference's CuPolicy layer
+// (craftax_full.cu:11758-12092): every device buffer is allocated here at
+// create time and owned by the object; step entry points only enqueue work.
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "cfp_common.h"
+
+namespace cfp {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+
+// Counter-based generator shared with the host-side test utilities:
+// value(seed, stream, index) is a splitmix64 finalizer of a linear counter.
+__host__ __device__ inline uint64_t mix64(uint64_t seed, uint64_t stream,
+                                          uint64_t index) {
+    uint64_t z = seed + stream * 0xD1B54A32D192ED03ULL +
+                 (index + 1) * 0x9E3779B97F4A7C15ULL;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
+    return z ^ (z >> 31);
+}
+__host__ __device__ inline float unit24(uint64_t z) {
+    return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+}  // namespace cfp
+
+struct cfp_policy {
+    int n = 0;
+    int layers = 0;
+    size_t param_count = 0;
+    float* params = nullptr;
+    float* we_pk = nullptr;
+    float* wg_pk = nullptr;
+    float* wav_pk = nullptr;
+    float* h_state = nullptr;
+    uint8_t* rec = nullptr;
+    float* h_enc = nullptr;
+    float* h3 = nullptr;
+    float* logits = nullptr;
+    hipStream_t stream = nullptr;
+};
+
+using namespace cfp;
+
+extern "C" {
+
+const char* cfp_last_error(void) { return g_err; }
+int cfp_abi_version(void) { return 1; }
+
+static void policy_release(cfp_policy* p) {
+    if (!p) return;
+    if (p->stream) (void)hipStreamDestroy(p->stream);
+    (void)hipFree(p->params);
+    (void)hipFree(p->we_pk);
+    (void)hipFree(p->wg_pk);
+    (void)hipFree(p->wav_pk);
+    (void)hipFree(p->h_state);
+    (void)hipFree(p->rec);
+    (void)hipFree(p->h_enc);
+    (void)hipFree(p->h3);
+    (void)hipFree(p->logits);
+    delete p;
+}
+
+// Xavier-uniform weights, U(+-1/sqrt(fan_in)) biases; segment order is the
+// arena order (craftax_full.cu:11832-11840).
+static void init_params_host(std::vector<float>& w, int layers, uint64_t seed) {
+    struct Seg { size_t off, count; float bound; };
+    const float xe = sqrtf(6.0f / (float)(CFP_OBS + CFP_HIDDEN));
+    const float xg = sqrtf(6.0f / (float)(CFP_HIDDEN + CFP_GRU));
+    const float xa = sqrtf(6.0f / (float)(CFP_HIDDEN + CFP_ACTIONS));
+    const float xv = sqrtf(6.0f / (float)(CFP_HIDDEN + 1));
+    const float be = 1.0f / sqrtf((float)CFP_OBS);
+    const float bh = 1.0f / sqrtf((float)CFP_HIDDEN);
+    const Seg segs[7] = {
+        {CFP_OFF_W_ENC, (size_t)CFP_OBS * CFP_HIDDEN, xe},
+        {CFP_OFF_B_ENC, CFP_HIDDEN, be},
+        {CFP_OFF_W_GRU, (size_t)layers * CFP_GRU * CFP_HIDDEN, xg},
+        {(size_t)CFP_OFF_W_A(layers), (size_t)CFP_ACTIONS * CFP_HIDDEN, xa},
+        {(size_t)CFP_OFF_B_A(layers), CFP_ACTIONS, bh},
+        {(size_t)CFP_OFF_W_V(layers), CFP_HIDDEN, xv},
+        {(size_t)CFP_OFF_B_V(layers), 1, bh},
+    };
+    for (int s = 0; s < 7; s++)
+        for (size_t i = 0; i < segs[s].count; i++) {
+            float u = unit24(mix64(seed, (uint64_t)s, i));
+            w[segs[s].off + i] = (2.0f * u - 1.0f) * segs[s].bound;
+        }
+}
+
+int cfp_policy_create(cfp_policy** out, int num_envs, int layers,
+                      uint64_t seed) {
+    CFP_REQUIRE(out != nullptr, "cfp_policy_create: out is NULL");
+    *out = nullptr;
+    CFP_REQUIRE(num_envs > 0 && num_envs % 32 == 0,
+                "policy modes need the env count to be a positive multiple of "
+                "32 (got %d)", num_envs);
+    CFP_REQUIRE(layers >= 1 && layers <= CFP_MAX_LAYERS,
+                "layers must be in 1..%d (got %d)", CFP_MAX_LAYERS, layers);
+    cfp_policy* p = new cfp_policy();
+    p->n = num_envs;
+    p->layers = layers;
+    p->param_count = (size_t)CFP_PARAM_COUNT(layers);
+    const size_t hn = (size_t)CFP_HIDDEN * num_envs;
+#define CFP_ALLOC(ptr, bytes)                                                 \
+    do {                                                                      \
+        hipError_t e_ = hipMalloc((void**)&(ptr), (bytes));                   \
+        if (e_ != hipSuccess) {                                               \
+            set_error("hipMalloc(%zu bytes) for %s failed: %s",               \
+                      (size_t)(bytes), #ptr, hipGetErrorString(e_));          \
+            policy_release(p);                                                \
+            return 1;                                                         \
+        }                                                                     \
+    } while (0)
+    CFP_ALLOC(p->params, p->param_count * sizeof(float));
+    CFP_ALLOC(p->we_pk, (size_t)(kKbEnc + 2) * 2048 * sizeof(float));
+    CFP_ALLOC(p->wg_pk,
+              ((size_t)layers * kGruPackFloats + 4 * 6 * 64 * 4) * sizeof(float));
+    CFP_ALLOC(p->wav_pk, kAvPackFloats * sizeof(float));
+    CFP_ALLOC(p->h_state, (size_t)layers * hn * sizeof(float));
+    CFP_ALLOC(p->rec, (size_t)num_envs * CFP_REC_BYTES);
+    CFP_ALLOC(p->h_enc, hn * sizeof(float));
+    CFP_ALLOC(p->h3, hn * sizeof(float));
+    CFP_ALLOC(p->logits, (size_t)CFP_AV * num_envs * sizeof(float));
+#undef CFP_ALLOC
+    hipError_t e = hipStreamCreateWithFlags(&p->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        set_error("hipStreamCreateWithFlags failed: %s", hipGetErrorString(e));
+        policy_release(p);
+        return 1;
+    }
+    e = hipMemset(p->h_state, 0, (size_t)layers * hn * sizeof(float));
+    if (e == hipSuccess) e = hipMemset(p->rec, 0, (size_t)num_envs * CFP_REC_BYTES);
+    if (e != hipSuccess) {
+        set_error("hipMemset failed: %s", hipGetErrorString(e));
+        policy_release(p);
+        return 1;
+    }
+    std::vector<float> w(p->param_count);
+    init_params_host(w, layers, seed);
+    if (cfp_policy_set_params(p, w.data(), w.size()) != 0) {
+        policy_release(p);
+        return 1;
+    }
+    *out = p;
+    return 0;
+}
+
+void cfp_policy_destroy(cfp_policy* p) { policy_release(p); }
+
+int cfp_policy_num_envs(const cfp_policy* p) { return p ? p->n : 0; }
+int cfp_policy_layers(const cfp_policy* p) { return p ? p->layers : 0; }
+size_t cfp_policy_param_count(const cfp_policy* p) {
+    return p ? p->param_count : 0;
+}
+
+int cfp_policy_set_params(cfp_policy* p, const float* host_params,
+                          size_t count) {
+    CFP_REQUIRE(p && host_params, "cfp_policy_set_params: NULL argument");
+    CFP_REQUIRE(count == p->param_count,
+                "param count mismatch: got %zu, policy has %zu", count,
+                p->param_count);
+    CFP_HIP_TRY(hipMemcpy(p->params, host_params, count * sizeof(float),
+                          hipMemcpyHostToDevice));
+    if (cfp_policy_refresh_weights(p, nullptr) != 0) return 1;
+    CFP_HIP_TRY(hipDeviceSynchronize());
+    return 0;
+}
+
+int cfp_policy_get_params(const cfp_policy* p, float* host_params,
+                          size_t count) {
+    CFP_REQUIRE(p && host_params, "cfp_policy_get_params: NULL argument");
+    CFP_REQUIRE(count == p->param_count,
+                "param count mismatch: got %zu, policy has %zu", count,
+                p->param_count);
+    CFP_HIP_TRY(hipMemcpy(host_params, p->params, count * sizeof(float),
+                          hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int cfp_policy_refresh_weights(cfp_policy* p, void* stream) {
+    CFP_REQUIRE(p, "cfp_policy_refresh_weights: NULL policy");
+    return launch_pack_weights(p->params, p->layers, p->we_pk, p->wg_pk,
+                               p->wav_pk, (hipStream_t)stream);
+}
+
+float* cfp_policy_params(cfp_policy* p) { return p->params; }
+float* cfp_policy_state(cfp_policy* p) { return p->h_state; }
+uint8_t* cfp_policy_rec(cfp_policy* p) { return p->rec; }
+float* cfp_policy_h_enc(cfp_policy* p) { return p->h_enc; }
+float* cfp_policy_h3(cfp_policy* p) { return p->h3; }
+float* cfp_policy_logits(cfp_policy* p) { return p->logits; }
+void* cfp_policy_stream(cfp_policy* p) { return (void*)p->stream; }
+
+static void fill_weights(const cfp_policy* p, FwdArgs& a) {
+    a.we_pk = reinterpret_cast<const f4*>(p->we_pk);
+    a.b_enc = p->params + CFP_OFF_B_ENC;
+    a.wg_pk = reinterpret_cast<const f4*>(p->wg_pk);
+    a.wav_pk = reinterpret_cast<const f4*>(p->wav_pk);
+    a.b_a = p->params + CFP_OFF_B_A(p->layers);
+    a.b_v = p->params + CFP_OFF_B_V(p->layers);
+}
+
+// Launch over [0, n) in chunks; every per-env pointer is advanced by the
+// chunk start, the layer stride of state / r_state stays that of the full n.
+static int run_chunked(FwdArgs a, int n, int chunk, hipStream_t st) {
+    CFP_REQUIRE(n > 0 && n % 32 == 0,
+                "env count must be a positive multiple of 32 (got %d)", n);
+    if (chunk <= 0 || chunk > n) chunk = n;
+    CFP_REQUIRE(chunk % 32 == 0, "chunk must be a multiple of 32 (got %d)",
+                chunk);
+    for (int e0 = 0; e0 < n; e0 += chunk) {
+        FwdArgs c = a;
+        c.n = n - e0 < chunk ? n - e0 : chunk;
+        const size_t off = (size_t)e0;
+        if (a.rec) c.rec = a.rec + off * CFP_REC_BYTES;
+        if (a.x0) c.x0 = a.x0 + off * CFP_HIDDEN;
+        if (a.state) c.state = a.state + off * CFP_HIDDEN;
+        if (a.terminals) c.terminals = a.terminals + off;
+        if (a.r_state) c.r_state = a.r_state + off * CFP_HIDDEN;
+        if (a.h_enc_out) c.h_enc_out = a.h_enc_out + off * CFP_HIDDEN;
+        if (a.h3_out) c.h3_out = a.h3_out + off * CFP_HIDDEN;
+        if (a.av_out) c.av_out = a.av_out + off * CFP_AV;
+        if (launch_forward(c, st) != 0) return 1;
+    }
+    return 0;
+}
+
+int cfp_encode_step(cfp_policy* p, const uint8_t* d_rec_row, int n,
+                    void* stream) {
+    CFP_REQUIRE(p, "cfp_encode_step: NULL policy");
+    CFP_REQUIRE(n <= p->n, "cfp_encode_step: n=%d exceeds the policy's %d envs",
+                n, p->n);
+    FwdArgs a{};
+    fill_weights(p, a);
+    a.rec = d_rec_row ? d_rec_row : p->rec;
+    a.h_enc_out = p->h_enc;
+    a.layers = 0;
+    a.do_head = 0;
+    return run_chunked(a, n, 0, (hipStream_t)stream);
+}
+
+int cfp_gru_chain(cfp_policy* p, const float* d_x0, float* d_state,
+                  const float* d_terminals, float* d_r_state_t, float* d_h3,
+                  int n, int chunk, void* stream) {
+    CFP_REQUIRE(p && d_x0 && d_state && d_h3, "cfp_gru_chain: NULL argument");
+    FwdArgs a{};
+    fill_weights(p, a);
+    a.x0 = d_x0;
+    a.state = d_state;
+    a.terminals = d_terminals;
+    a.r_state = d_r_state_t;
+    a.h3_out = d_h3;
+    a.layer_stride = (size_t)n * CFP_HIDDEN;
+    a.layers = p->layers;
+    a.do_head = 0;
+    return run_chunked(a, n, chunk, (hipStream_t)stream);
+}
+
+int cfp_head(cfp_policy* p, const float* d_h3, float* d_av, int n,
+             void* stream) {
+    CFP_REQUIRE(p && d_h3 && d_av, "cfp_head: NULL argument");
+    FwdArgs a{};
+    fill_weights(p, a);
+    a.x0 = d_h3;
+    a.av_out = d_av;
+    a.layers = 0;
+    a.do_head = 1;
+    return run_chunked(a, n, 0, (hipStream_t)stream);
+}
+
+int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
+                       const float* d_terminals, float* d_state,
+                       float* d_r_state_t, float* d_h_enc, float* d_h3,
+                       float* d_av, int n, int chunk, void* stream) {
+    CFP_REQUIRE(p, "cfp_policy_forward: NULL policy");
+    CFP_REQUIRE(d_state != nullptr || n == p->n,
+                "cfp_policy_forward: the object's live state covers %d envs, "
+                "n=%d needs an explicit state buffer", p->n, n);
+    CFP_REQUIRE(d_rec_row != nullptr || n <= p->n,
+                "cfp_policy_forward: n=%d exceeds the record scratch (%d envs)",
+                n, p->n);
+    CFP_REQUIRE(d_av != nullptr || n <= p->n,
+                "cfp_policy_forward: n=%d exceeds the logits buffer (%d envs)",
+                n, p->n);
+    FwdArgs a{};
+    fill_weights(p, a);
+    a.rec = d_rec_row ? d_rec_row : p->rec;
+    a.terminals = d_terminals;
+    a.state = d_state ? d_state : p->h_state;
+    a.r_state = d_r_state_t;
+    a.h_enc_out = d_h_enc;
+    a.h3_out = d_h3;
+    a.av_out = d_av ? d_av : p->logits;
+    a.layer_stride = (size_t)n * CFP_HIDDEN;
+    a.layers = p->layers;
+    a.do_head = 1;
+    return run_chunked(a, n, chunk, (hipStream_t)stream);
+}
+
+}  // extern "C"
+
+// ---- synthetic records -------------------------------------------------------
+namespace cfp {
+// One thread per (env, dword): dwords 0..197 are four map bytes U{0..40},
+// dwords 198..248 one tail float U[0,1) on a 24-bit grid.
+__global__ void k_synth_records(uint32_t* __restrict__ rec, size_t total_dw,
+                                int n, uint64_t seed, uint64_t step) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total_dw) return;
+    size_t env = i / 249;
+    int d = (int)(i - env * 249);
+    uint64_t z = mix64(seed, step, env * 249 + (uint64_t)d);
+    uint32_t w;
+    if (d < CFP_OBS_MAP / 4) {
+        w = (uint32_t)(z & 0xffff) % 41u;
+        w |= ((uint32_t)((z >> 16) & 0xffff) % 41u) << 8;
+        w |= ((uint32_t)((z >> 32) & 0xffff) % 41u) << 16;
+        w |= ((uint32_t)((z >> 48) & 0xffff) % 41u) << 24;
+    } else {
+        w = __float_as_uint(unit24(z));
+    }
+    rec[i] = w;
+}
+}  // namespace cfp
+
+extern "C" int cfp_synth_records(uint8_t* d_rec, int n, uint64_t seed,
+                                 uint64_t step, void* stream) {
+    CFP_REQUIRE(d_rec && n > 0, "cfp_synth_records: bad argument");
+    CFP_REQUIRE((reinterpret_cast<uintptr_t>(d_rec) & 3u) == 0,
+                "records must be 4-byte aligned");
+    size_t total = (size_t)n * 249;
+    hipLaunchKernelGGL(cfp::k_synth_records, dim3((unsigned)((total + 255) / 256)),
+                       dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<uint32_t*>(d_rec), total, n, seed, step);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}

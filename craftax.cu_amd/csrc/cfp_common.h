@@ -1,0 +1,80 @@
+// Shared host/device definitions for the gfx950 policy-path library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "../../include/cfp.h"
+
+namespace cfp {
+
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+
+// Workgroup tile of the fused forward: 32 envs x all 256 hidden units,
+// 4 wavefronts, wave w owns units [64w, 64w+64).
+constexpr int kTileEnvs = 32;
+constexpr int kFwdThreads = 256;
+// K is consumed in blocks of 8: one 16-byte operand fragment per lane feeds
+// four 32x32x2 MFMA steps (lanes 0-31 carry k = 8b+j, lanes 32-63 k = 8b+4+j).
+constexpr int kKBlock = 8;
+constexpr int kObsPad = 848;                       // 843 rounded up to 8
+constexpr int kKbEnc = kObsPad / kKBlock;          // 106
+constexpr int kKbMap = CFP_OBS_MAP / kKBlock;      // 99: map bytes end on a block edge
+constexpr int kKbHid = CFP_HIDDEN / kKBlock;       // 32
+constexpr int kAvPad = 64;                         // head rows padded 44 -> 64
+
+// MFMA-ordered weight mirror sizes, in floats.
+constexpr size_t kEncPackFloats = (size_t)kObsPad * CFP_HIDDEN;
+constexpr size_t kGruPackFloats = (size_t)CFP_GRU * CFP_HIDDEN;   // per layer
+constexpr size_t kAvPackFloats = (size_t)kAvPad * CFP_HIDDEN;
+
+void set_error(const char* fmt, ...);
+
+#define CFP_HIP_TRY(expr)                                                     \
+    do {                                                                      \
+        hipError_t e_ = (expr);                                               \
+        if (e_ != hipSuccess) {                                               \
+            cfp::set_error("%s:%d: %s -> %s", __FILE__, __LINE__, #expr,      \
+                           hipGetErrorString(e_));                            \
+            return 1;                                                         \
+        }                                                                     \
+    } while (0)
+
+#define CFP_REQUIRE(cond, ...)                                                \
+    do {                                                                      \
+        if (!(cond)) {                                                        \
+            cfp::set_error(__VA_ARGS__);                                      \
+            return 1;                                                         \
+        }                                                                     \
+    } while (0)
+
+// ---- launchers implemented in the .hip files -------------------------------
+struct FwdArgs {
+    const uint8_t* rec;      // [n][996] or null (then x0 is the layer-0 input)
+    const float* x0;         // [n][256] or null
+    const f4* we_pk;         // packed encoder weights
+    const float* b_enc;
+    const f4* wg_pk;         // packed gate weights, layers back to back
+    const f4* wav_pk;        // packed head weights
+    const float* b_a;
+    const float* b_v;
+    float* state;            // [layers][state_envs][256] in/out, or null
+    const float* terminals;  // [n] or null (= no terminal)
+    float* r_state;          // like state, or null
+    float* h_enc_out;        // [n][256] or null
+    float* h3_out;           // [n][256] or null
+    float* av_out;           // [n][44] or null
+    size_t layer_stride;     // floats between layers in state / r_state
+    int n;                   // envs in this launch (multiple of 32)
+    int layers;              // MinGRU layers to run (0 = encoder only)
+    int do_head;
+};
+int launch_forward(const FwdArgs& a, hipStream_t st);
+
+int launch_pack_weights(const float* params, int layers, float* we_pk,
+                        float* wg_pk, float* wav_pk, hipStream_t st);
+
+}  // namespace cfp

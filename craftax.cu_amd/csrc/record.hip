@@ -1,0 +1,281 @@
+// Observation-record kernels: state -> 996-byte compact record, record ->
+// fp32 features, and the unfused elementwise pieces of the forward
+// (bias add, MinGRU gate/blend epilogue) kept for parity tests and for the
+// PPO update's window recompute.
+//
+// Record format (craftax_full.c:578-581, encoder :2721-2844): 99 view cells
+// (9 rows x 11 cols, row-major) x 8 bytes {block, item+1, visible, melee+1,
+// passive+1, ranged+1, mob-projectile+1, player-projectile+1}, then 51 raw
+// little-endian fp32 scalars.  All of it is integer/byte work bound by HBM
+// gathers; one wavefront encodes one env, a lane per view cell.
+#include "cfp_common.h"
+
+namespace cfp {
+namespace {
+
+constexpr int MAP = 48;
+constexpr int ROWS = 9, COLS = 11, CELLS = ROWS * COLS;
+
+__device__ __forceinline__ int jax_index(int index, int size) {
+    // craftax_wg_jax_index, craftax_full.c:2180
+    if (index < 0) index += size;
+    if (index < 0) return 0;
+    if (index >= size) return size - 1;
+    return index;
+}
+
+// How each of the 51 tail scalars is derived (craftax_full.c:2646-2703).
+enum TailKind : uint8_t {
+    T_SQRT10,   // sqrtf((float)i) * 0.1f
+    T_HALF,     // (float)i * 0.5f
+    T_QUARTER,  // (float)i * 0.25f
+    T_INT,      // (float)i
+    T_F10,      // f * 0.1f          (float field)
+    T_I10,      // (float)i * 0.1f
+    T_DIR,      // one-hot of player_direction - 1, slot in `aux`
+    T_FLOAT,    // f
+    T_BOOL,     // i != 0
+    T_KILLED,   // i >= 8
+    T_BOSS,     // boss vulnerable
+};
+struct TailSpec { uint8_t kind, field, aux; };
+
+#define FLD(name) ((uint8_t)(offsetof(cfp_env_scalars, name) / 4))
+__constant__ TailSpec kTail[CFP_OBS_TAIL] = {
+    {T_SQRT10, FLD(wood), 0},      {T_SQRT10, FLD(stone), 0},
+    {T_SQRT10, FLD(coal), 0},      {T_SQRT10, FLD(iron), 0},
+    {T_SQRT10, FLD(diamond), 0},   {T_SQRT10, FLD(sapphire), 0},
+    {T_SQRT10, FLD(ruby), 0},      {T_SQRT10, FLD(sapling), 0},
+    {T_SQRT10, FLD(torches), 0},   {T_SQRT10, FLD(arrows), 0},
+    {T_HALF, FLD(books), 0},       {T_QUARTER, FLD(pickaxe), 0},
+    {T_QUARTER, FLD(sword), 0},    {T_INT, FLD(sword_enchantment), 0},
+    {T_INT, FLD(bow_enchantment), 0}, {T_INT, FLD(bow), 0},
+    {T_SQRT10, FLD(potions[0]), 0}, {T_SQRT10, FLD(potions[1]), 0},
+    {T_SQRT10, FLD(potions[2]), 0}, {T_SQRT10, FLD(potions[3]), 0},
+    {T_SQRT10, FLD(potions[4]), 0}, {T_SQRT10, FLD(potions[5]), 0},
+    {T_F10, FLD(player_health), 0}, {T_I10, FLD(player_food), 0},
+    {T_I10, FLD(player_drink), 0}, {T_I10, FLD(player_energy), 0},
+    {T_I10, FLD(player_mana), 0},  {T_I10, FLD(player_xp), 0},
+    {T_I10, FLD(player_dexterity), 0}, {T_I10, FLD(player_strength), 0},
+    {T_I10, FLD(player_intelligence), 0},
+    {T_DIR, FLD(player_direction), 0}, {T_DIR, FLD(player_direction), 1},
+    {T_DIR, FLD(player_direction), 2}, {T_DIR, FLD(player_direction), 3},
+    {T_HALF, FLD(armour[0]), 0},   {T_HALF, FLD(armour[1]), 0},
+    {T_HALF, FLD(armour[2]), 0},   {T_HALF, FLD(armour[3]), 0},
+    {T_INT, FLD(armour_enchantments[0]), 0}, {T_INT, FLD(armour_enchantments[1]), 0},
+    {T_INT, FLD(armour_enchantments[2]), 0}, {T_INT, FLD(armour_enchantments[3]), 0},
+    {T_FLOAT, FLD(light_level), 0}, {T_BOOL, FLD(is_sleeping), 0},
+    {T_BOOL, FLD(is_resting), 0},  {T_BOOL, FLD(learned_spells[0]), 0},
+    {T_BOOL, FLD(learned_spells[1]), 0}, {T_I10, FLD(player_level), 0},
+    {T_KILLED, FLD(monsters_killed_level), 0}, {T_BOSS, 0, 0},
+};
+#undef FLD
+
+// class (record channel - 3) of each of the 14 mob slots
+__constant__ uint8_t kSlotClass[CFP_MOB_SLOTS] = {0, 0, 0, 1, 1, 1, 2, 2,
+                                                  3, 3, 3, 4, 4, 4};
+
+__global__ __launch_bounds__(256) void k_record_obs(
+    const cfp_env_scalars* __restrict__ scalars,
+    const uint8_t* __restrict__ map, const uint8_t* __restrict__ item_map,
+    const uint8_t* __restrict__ light_map, size_t env_stride,
+    size_t level_stride, uint8_t* __restrict__ rec_row, int n) {
+    const int lane = threadIdx.x & 63;
+    const int env = __builtin_amdgcn_readfirstlane(
+        (int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
+    if (env >= n) return;
+    const cfp_env_scalars* s = scalars + env;
+    const int pr = s->player_position[0], pc = s->player_position[1];
+    const int level = s->player_level;
+    const int mlevel = jax_index(level, 9);
+    const size_t cell_plane = (size_t)env * env_stride + (size_t)level * level_stride;
+    const size_t mob_plane = (size_t)env * env_stride + (size_t)mlevel * level_stride;
+    const uint8_t* light_m = light_map + mob_plane;
+
+    // Mob list: slot s contributes (cell, channel, value) when it passes the
+    // predicates of craftax_encode_mobs{3,2}_compact (craftax_full.c:2747-2825);
+    // evaluated identically by every lane, ascending slot order = last wins.
+    int mob_cell[CFP_MOB_SLOTS];
+    int mob_val[CFP_MOB_SLOTS];
+#pragma unroll
+    for (int m = 0; m < CFP_MOB_SLOTS; m++) {
+        const int type = s->mob_type_id[m];
+        const int mr = s->mob_position[m][0], mc = s->mob_position[m][1];
+        const int lr = mr - pr + ROWS / 2, lc = mc - pc + COLS / 2;
+        bool ok = type >= 0 && type < 8 && s->mob_mask[m] != 0 && lr >= 0 &&
+                  lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
+                  mc >= 0 && mc < MAP;
+        if (ok) ok = light_m[mr * MAP + mc] > 12;
+        mob_cell[m] = ok ? lr * COLS + lc : -1;
+        mob_val[m] = type + 1;
+    }
+
+    uint32_t* out = reinterpret_cast<uint32_t*>(rec_row + (size_t)env * CFP_REC_BYTES);
+    for (int cell = lane; cell < CELLS; cell += 64) {
+        const int row = cell / COLS, col = cell - row * COLS;
+        const int wr = pr - ROWS / 2 + row, wc = pc - COLS / 2 + col;
+        uint32_t lo = 0, hi = 0;
+        if (wr >= 0 && wr < MAP && wc >= 0 && wc < MAP) {
+            const size_t o = cell_plane + (size_t)(wr * MAP + wc);
+            if (light_map[o] > 12)
+                lo = (uint32_t)map[o] | ((uint32_t)(uint8_t)(item_map[o] + 1) << 8) |
+                     (1u << 16);
+        }
+        uint32_t ch[5] = {0, 0, 0, 0, 0};
+#pragma unroll
+        for (int m = 0; m < CFP_MOB_SLOTS; m++)
+            if (mob_cell[m] == cell) ch[kSlotClass[m]] = (uint32_t)(uint8_t)mob_val[m];
+        lo |= ch[0] << 24;
+        hi = ch[1] | (ch[2] << 8) | (ch[3] << 16) | (ch[4] << 24);
+        out[2 * cell] = lo;
+        out[2 * cell + 1] = hi;
+    }
+
+    if (lane < CFP_OBS_TAIL) {
+        const TailSpec ts = kTail[lane];
+        const int32_t* fi = reinterpret_cast<const int32_t*>(s);
+        const int iv = fi[ts.field];
+        const float fv = __int_as_float(iv);
+        const float xi = (float)iv;
+        float v = 0.0f;
+        switch (ts.kind) {
+            case T_SQRT10: v = __fsqrt_rn(xi) * 0.1f; break;
+            case T_HALF: v = xi * 0.5f; break;
+            case T_QUARTER: v = xi * 0.25f; break;
+            case T_INT: v = xi; break;
+            case T_F10: v = fv * 0.1f; break;
+            case T_I10: v = xi * 0.1f; break;
+            case T_DIR: v = (iv - 1 == (int)ts.aux) ? 1.0f : 0.0f; break;
+            case T_FLOAT: v = fv; break;
+            case T_BOOL: v = iv != 0 ? 1.0f : 0.0f; break;
+            case T_KILLED: v = iv >= 8 ? 1.0f : 0.0f; break;
+            case T_BOSS: {
+                // craftax_wg_is_boss_vulnerable, craftax_full.c:2205: no live
+                // melee (slots 0..2) or ranged (slots 6..7) mob, spawn timer <= 0
+                bool any = false;
+                for (int m = 0; m < 3; m++) any = any || s->mob_mask[m] != 0;
+                for (int m = 6; m < 8; m++) any = any || s->mob_mask[m] != 0;
+                v = (!any && s->boss_timesteps_to_spawn_this_round <= 0) ? 1.0f : 0.0f;
+            } break;
+        }
+        out[CFP_OBS_MAP / 4 + lane] = __float_as_uint(v);
+    }
+}
+
+__global__ void k_expand_obs(const uint8_t* __restrict__ r_obs,
+                             float* __restrict__ xobs, int t0, size_t total,
+                             int mb, int n, int env_start) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int f = (int)(idx % CFP_OBS);
+    const size_t w = idx / CFP_OBS;
+    const size_t t = (size_t)t0 + w / (size_t)mb;
+    const size_t el = w % (size_t)mb;
+    const uint8_t* rec = r_obs + (t * (size_t)n + env_start + el) * CFP_REC_BYTES;
+    float x;
+    if (f < CFP_OBS_MAP) {
+        x = (float)rec[f];
+    } else {
+        const uint32_t* tail = reinterpret_cast<const uint32_t*>(rec + CFP_OBS_MAP);
+        x = __uint_as_float(tail[f - CFP_OBS_MAP]);
+    }
+    xobs[idx] = x;
+}
+
+__global__ void k_add_bias(float* __restrict__ h, const float* __restrict__ b,
+                           size_t total) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    h[idx] += b[idx & (CFP_HIDDEN - 1)];
+}
+
+__device__ __forceinline__ float sigmoid_fast(float z) {
+    return __builtin_amdgcn_rcpf(1.0f + __expf(-z));
+}
+
+__global__ void k_mingru_epi_fwd(const float* __restrict__ pre,
+                                 const float* __restrict__ x,
+                                 float* __restrict__ state,
+                                 float* __restrict__ h_out,
+                                 float* __restrict__ r_state_store,
+                                 const float* __restrict__ prev_terminals,
+                                 size_t total) {
+    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int k = (int)(idx & (CFP_HIDDEN - 1));
+    const size_t col = idx / CFP_HIDDEN;
+    float st = state[idx];
+    if (prev_terminals && prev_terminals[col] != 0.0f) st = 0.0f;
+    if (r_state_store) r_state_store[idx] = st;
+    const size_t o3 = col * CFP_GRU + k;
+    const float zh = pre[o3], zg = pre[o3 + CFP_HIDDEN], zp = pre[o3 + 2 * CFP_HIDDEN];
+    const float gh = zh >= 0.0f ? zh + 0.5f : sigmoid_fast(zh);
+    const float out = st + sigmoid_fast(zg) * (gh - st);
+    const float p = sigmoid_fast(zp);
+    h_out[idx] = p * out + (1.0f - p) * x[idx];
+    state[idx] = out;
+}
+
+}  // namespace
+}  // namespace cfp
+
+using namespace cfp;
+
+extern "C" {
+
+int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
+                   const uint8_t* d_item_map, const uint8_t* d_light_map,
+                   size_t env_stride, size_t level_stride, uint8_t* d_rec_row,
+                   int n, void* stream) {
+    CFP_REQUIRE(d_scalars && d_map && d_item_map && d_light_map && d_rec_row,
+                "cfp_record_obs: NULL argument");
+    CFP_REQUIRE(n > 0, "cfp_record_obs: n must be positive (got %d)", n);
+    CFP_REQUIRE((reinterpret_cast<uintptr_t>(d_rec_row) & 3u) == 0,
+                "record rows must be 4-byte aligned");
+    CFP_REQUIRE(env_stride >= (size_t)MAP * MAP,
+                "cfp_record_obs: env_stride smaller than one 48x48 plane");
+    hipLaunchKernelGGL(k_record_obs, dim3((n + 3) / 4), dim3(256), 0,
+                       (hipStream_t)stream, d_scalars, d_map, d_item_map,
+                       d_light_map, env_stride, level_stride, d_rec_row, n);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int cfp_expand_obs(const uint8_t* d_r_obs, float* d_xobs, int t0, int count,
+                   int mb, int n, int env_start, void* stream) {
+    CFP_REQUIRE(d_r_obs && d_xobs && count > 0 && mb > 0 && n > 0 && t0 >= 0 &&
+                    env_start >= 0 && env_start + mb <= n,
+                "cfp_expand_obs: bad argument");
+    CFP_REQUIRE((reinterpret_cast<uintptr_t>(d_r_obs) & 3u) == 0,
+                "records must be 4-byte aligned");
+    const size_t total = (size_t)count * CFP_OBS;
+    hipLaunchKernelGGL(k_expand_obs, dim3((unsigned)((total + 255) / 256)),
+                       dim3(256), 0, (hipStream_t)stream, d_r_obs, d_xobs, t0,
+                       total, mb, n, env_start);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int cfp_add_bias(float* d_h, const float* d_b, int cols, void* stream) {
+    CFP_REQUIRE(d_h && d_b && cols > 0, "cfp_add_bias: bad argument");
+    const size_t total = (size_t)cols * CFP_HIDDEN;
+    hipLaunchKernelGGL(k_add_bias, dim3((unsigned)((total + 255) / 256)),
+                       dim3(256), 0, (hipStream_t)stream, d_h, d_b, total);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int cfp_mingru_epi_fwd(const float* d_pre, const float* d_x, float* d_state,
+                       float* d_h_out, float* d_r_state_store,
+                       const float* d_prev_terminals, int cols, void* stream) {
+    CFP_REQUIRE(d_pre && d_x && d_state && d_h_out && cols > 0,
+                "cfp_mingru_epi_fwd: bad argument");
+    const size_t total = (size_t)cols * CFP_HIDDEN;
+    hipLaunchKernelGGL(k_mingru_epi_fwd, dim3((unsigned)((total + 255) / 256)),
+                       dim3(256), 0, (hipStream_t)stream, d_pre, d_x, d_state,
+                       d_h_out, d_r_state_store, d_prev_terminals, total);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,259 @@
+"""Host-side mirror of the reference's CuPolicy call surface over the C ABI.
+
+Names follow craftax_full.cu: encode_step (:11931), gru_chain (:11978), the
+policy half of rollout_step (:12022) and the GEMM wrappers (:11604-11666).
+PyTorch is used only to own device memory and streams; every computation is a
+call into libcfpolicy.so.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib
+
+HIDDEN, GRU, OBS, OBS_MAP, OBS_TAIL = 256, 768, 843, 792, 51
+REC_BYTES, ACTIONS, AV = 996, 43, 44
+
+_cfp = None
+
+
+def lib():
+    global _cfp
+    if _cfp is None:
+        _cfp = _lib.load()
+    return _cfp
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensor required"
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _check(rc):
+    _lib.check(lib(), rc)
+
+
+def param_offsets(layers):
+    """Flat arena layout, craftax_full.cu:9094-9102."""
+    o = {"W_enc": 0, "b_enc": OBS * HIDDEN}
+    o["W_gru"] = o["b_enc"] + HIDDEN
+    o["W_a"] = o["W_gru"] + layers * GRU * HIDDEN
+    o["b_a"] = o["W_a"] + ACTIONS * HIDDEN
+    o["W_v"] = o["b_a"] + ACTIONS
+    o["b_v"] = o["W_v"] + HIDDEN
+    o["count"] = o["b_v"] + 1
+    return o
+
+
+def split_params(params, layers):
+    """Views of a flat host params array, shaped as the reference documents them."""
+    o = param_offsets(layers)
+    p = np.asarray(params)
+    return {
+        "W_enc": p[o["W_enc"]:o["b_enc"]].reshape(OBS, HIDDEN),
+        "b_enc": p[o["b_enc"]:o["W_gru"]],
+        "W_gru": p[o["W_gru"]:o["W_a"]].reshape(layers, GRU, HIDDEN),
+        "W_a": p[o["W_a"]:o["b_a"]].reshape(ACTIONS, HIDDEN),
+        "b_a": p[o["b_a"]:o["W_v"]],
+        "W_v": p[o["W_v"]:o["b_v"]],
+        "b_v": p[o["b_v"]:o["count"]],
+    }
+
+
+class Policy:
+    """cfp_policy handle (CuPolicy, craftax_full.cu:11758)."""
+
+    def __init__(self, num_envs, layers=3, seed=1):
+        self._h = C.c_void_p()
+        _check(lib().cfp_policy_create(C.byref(self._h), num_envs, layers, seed))
+        self.n = num_envs
+        self.layers = layers
+        self.param_count = lib().cfp_policy_param_count(self._h)
+
+    def close(self):
+        if getattr(self, "_h", None) and self._h.value:
+            lib().cfp_policy_destroy(self._h)
+            self._h = C.c_void_p()
+
+    __del__ = close
+
+    # -- parameters ----------------------------------------------------
+    def set_params(self, host_params):
+        a = np.ascontiguousarray(host_params, dtype=np.float32)
+        _check(lib().cfp_policy_set_params(self._h, a.ctypes.data_as(C.c_void_p), a.size))
+
+    def get_params(self):
+        a = np.empty(self.param_count, dtype=np.float32)
+        _check(lib().cfp_policy_get_params(self._h, a.ctypes.data_as(C.c_void_p), a.size))
+        return a
+
+    def refresh_weights(self):
+        _check(lib().cfp_policy_refresh_weights(self._h, _stream()))
+
+    # -- forward entry points ------------------------------------------------
+    def encode_step(self, rec=None, n=None):
+        """records [n][996] u8 (None = the object's scratch) -> the object's h_enc."""
+        if rec is not None:
+            n = rec.shape[0]
+        elif n is None:
+            n = self.n
+        _check(lib().cfp_encode_step(self._h, _ptr(rec), n, _stream()))
+        return self.h_enc[:n]
+
+    # -- library-owned device buffers, viewed as tensors (no copy) ---------------
+    @property
+    def params(self):
+        return _wrap(lib().cfp_policy_params(self._h), (self.param_count,), "<f4")
+
+    @property
+    def state(self):
+        return _wrap(lib().cfp_policy_state(self._h), (self.layers, self.n, HIDDEN), "<f4")
+
+    @property
+    def rec(self):
+        return _wrap(lib().cfp_policy_rec(self._h), (self.n, REC_BYTES), "|u1")
+
+    @property
+    def h_enc(self):
+        return _wrap(lib().cfp_policy_h_enc(self._h), (self.n, HIDDEN), "<f4")
+
+    @property
+    def h3(self):
+        return _wrap(lib().cfp_policy_h3(self._h), (self.n, HIDDEN), "<f4")
+
+    @property
+    def logits(self):
+        return _wrap(lib().cfp_policy_logits(self._h), (self.n, AV), "<f4")
+
+    def gru_chain(self, x0, state, terminals, r_state_t=None, h3=None, chunk=0):
+        n = x0.shape[0]
+        if h3 is None:
+            h3 = torch.empty((n, HIDDEN), dtype=torch.float32, device=x0.device)
+        _check(lib().cfp_gru_chain(self._h, _ptr(x0), _ptr(state), _ptr(terminals),
+                                   _ptr(r_state_t), _ptr(h3), n, chunk, _stream()))
+        return h3
+
+    def head(self, h3, av=None):
+        n = h3.shape[0]
+        if av is None:
+            av = torch.empty((n, AV), dtype=torch.float32, device=h3.device)
+        _check(lib().cfp_head(self._h, _ptr(h3), _ptr(av), n, _stream()))
+        return av
+
+    def forward(self, rec, terminals, state, r_state_t=None, h_enc=None, h3=None,
+                av=None, chunk=0):
+        """Policy half of rollout_step: records -> logits/value, state updated in place."""
+        n = rec.shape[0]
+        if av is None:
+            av = torch.empty((n, AV), dtype=torch.float32, device=rec.device)
+        _check(lib().cfp_policy_forward(self._h, _ptr(rec), _ptr(terminals), _ptr(state),
+                                        _ptr(r_state_t), _ptr(h_enc), _ptr(h3),
+                                        _ptr(av), n, chunk, _stream()))
+        return av
+
+
+class _DevBuf:
+    """Borrowed device memory exposed through __cuda_array_interface__."""
+
+    def __init__(self, ptr, shape, typestr):
+        self.__cuda_array_interface__ = {
+            "shape": tuple(shape), "typestr": typestr, "data": (int(ptr), False),
+            "version": 2, "strides": None}
+
+
+def _wrap(ptr, shape, typestr):
+    return torch.as_tensor(_DevBuf(ptr, shape, typestr), device="cuda")
+
+
+# -- the dense-math seam -------------------------------------------------------
+def gemm_fwd(W, x, y=None):
+    """y[cols][m] = x[cols][k] . W[m][k]^T (cu_gemm_fwd :11604)."""
+    m, k = W.shape
+    cols = x.shape[0]
+    if y is None:
+        y = torch.empty((cols, m), dtype=torch.float32, device=x.device)
+    _check(lib().cfp_gemm_fwd(m, cols, k, _ptr(W), _ptr(x), _ptr(y), _stream()))
+    return y
+
+
+def gemm_enc_fwd(W_enc, xobs, h=None):
+    cols = xobs.shape[0]
+    if h is None:
+        h = torch.empty((cols, HIDDEN), dtype=torch.float32, device=xobs.device)
+    _check(lib().cfp_gemm_enc_fwd(cols, _ptr(W_enc), _ptr(xobs), _ptr(h), _stream()))
+    return h
+
+
+def gemm_dh(W, dpre, dh=None):
+    m3 = W.shape[0]
+    cols = dpre.shape[0]
+    if dh is None:
+        dh = torch.empty((cols, HIDDEN), dtype=torch.float32, device=dpre.device)
+    _check(lib().cfp_gemm_dh(m3, cols, _ptr(W), _ptr(dpre), _ptr(dh), _stream()))
+    return dh
+
+
+def gemm_dw(x, dpre, dW):
+    """dW[rows][256] += dpre[cols][rows]^T . x[cols][256] (cu_gemm_dw :11642)."""
+    cols, rows = dpre.shape
+    _check(lib().cfp_gemm_dw(rows, cols, _ptr(x), _ptr(dpre), _ptr(dW), _stream()))
+    return dW
+
+
+def gemv_dwv(x, dv, dWv):
+    cols = x.shape[0]
+    _check(lib().cfp_gemv_dwv(_ptr(x), _ptr(dv), _ptr(dWv), cols, _stream()))
+    return dWv
+
+
+def expand_obs(r_obs, count, t0=0, mb=None, n=None, env_start=0, xobs=None):
+    """k_expand_obs (:10028): records -> fp32 features [count][843]."""
+    flat = r_obs.reshape(-1, REC_BYTES)
+    if n is None:
+        n = flat.shape[0]
+    if mb is None:
+        mb = count
+    if xobs is None:
+        xobs = torch.empty((count, OBS), dtype=torch.float32, device=r_obs.device)
+    _check(lib().cfp_expand_obs(_ptr(flat), _ptr(xobs), t0, count, mb, n, env_start,
+                                _stream()))
+    return xobs
+
+
+def add_bias(h, b):
+    _check(lib().cfp_add_bias(_ptr(h), _ptr(b), h.shape[0], _stream()))
+    return h
+
+
+def mingru_epi_fwd(pre, x, state, terminals, r_state_store=None, h_out=None):
+    cols = x.shape[0]
+    if h_out is None:
+        h_out = torch.empty_like(x)
+    _check(lib().cfp_mingru_epi_fwd(_ptr(pre), _ptr(x), _ptr(state), _ptr(h_out),
+                                    _ptr(r_state_store), _ptr(terminals), cols, _stream()))
+    return h_out
+
+
+def record_obs(scalars_u8, maps, item_maps, light_maps, n, env_stride, level_stride,
+               rec=None):
+    """k_record_obs (:9284): encoder-input state -> [n][996] records."""
+    if rec is None:
+        rec = torch.empty((n, REC_BYTES), dtype=torch.uint8, device=maps.device)
+    _check(lib().cfp_record_obs(_ptr(scalars_u8), _ptr(maps), _ptr(item_maps),
+                                _ptr(light_maps), env_stride, level_stride, _ptr(rec),
+                                n, _stream()))
+    return rec
+
+
+def synth_records(n, seed, step, rec=None, device="cuda"):
+    if rec is None:
+        rec = torch.empty((n, REC_BYTES), dtype=torch.uint8, device=device)
+    _check(lib().cfp_synth_records(_ptr(rec), n, seed, step, _stream()))
+    return rec

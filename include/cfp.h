@@ -1,0 +1,204 @@
+/*
+ * cfp.h -- C ABI of the MI355X (gfx950) batched Craftax policy path.
+ *
+ * Every entry point replaces one static function of the reference's single
+ * translation unit craftax_full.cu (cited as file:line at each declaration).
+ * The reference exposes no FFI for this path, so the seam kept here is the
+ * call surface of its rollout/trainer layers: same argument order, same
+ * tensor layouts, same "all work is enqueued on the given stream, nothing is
+ * allocated inside a step" contract.
+ *
+ * Conventions
+ *   - All pointers named d_* / documented "device" are HIP device pointers.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the legacy default stream).
+ *   - Activations are env-major: element (k, env) of a [rows]-wide tensor
+ *     sits at env*rows + k (the reference calls this col-major [rows][cols]).
+ *   - Return value: 0 on success, nonzero on error; cfp_last_error() returns
+ *     a thread-local message.  A library must not exit(); the reference's
+ *     CU_CHECK (craftax_full.cu:8635) prints and exit(1)s instead.
+ *   - Env counts must be multiples of 32, as in the reference
+ *     (craftax_full.cu:11820).
+ */
+#ifndef CFP_H_
+#define CFP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- fixed architecture (craftax_full.cu:9086-9105) ---------------------- */
+#define CFP_HIDDEN 256
+#define CFP_GRU (3 * CFP_HIDDEN)        /* [zh | zg | zp] rows per layer      */
+#define CFP_OBS 843                     /* 792 map features + 51 tail floats  */
+#define CFP_OBS_MAP 792
+#define CFP_OBS_TAIL 51
+#define CFP_REC_BYTES 996               /* compact record, craftax_full.c:578 */
+#define CFP_ACTIONS 43
+#define CFP_AV (CFP_ACTIONS + 1)        /* fused head: 43 logits + value      */
+#define CFP_MAX_LAYERS 3
+
+/* Flat fp32 parameter arena offsets for `layers` MinGRU layers
+ * (craftax_full.cu:9094-9102). */
+#define CFP_OFF_W_ENC 0
+#define CFP_OFF_B_ENC (CFP_OBS * CFP_HIDDEN)
+#define CFP_OFF_W_GRU (CFP_OFF_B_ENC + CFP_HIDDEN)
+#define CFP_OFF_W_A(layers) (CFP_OFF_W_GRU + (layers) * CFP_GRU * CFP_HIDDEN)
+#define CFP_OFF_B_A(layers) (CFP_OFF_W_A(layers) + CFP_ACTIONS * CFP_HIDDEN)
+#define CFP_OFF_W_V(layers) (CFP_OFF_B_A(layers) + CFP_ACTIONS)
+#define CFP_OFF_B_V(layers) (CFP_OFF_W_V(layers) + CFP_HIDDEN)
+#define CFP_PARAM_COUNT(layers) (CFP_OFF_B_V(layers) + 1)
+
+const char* cfp_last_error(void);
+/* Library/ABI version, bumped when a signature changes. */
+int cfp_abi_version(void);
+
+/* ---- policy object: replaces CuPolicy (craftax_full.cu:11758-11796) ------ */
+typedef struct cfp_policy cfp_policy;
+
+/* cu_policy_init (craftax_full.cu:11819): allocates every device buffer the
+ * forward needs for `num_envs` envs (params, packed weight mirrors, live
+ * state [layers][n][256] zeroed, record scratch, h_enc, h3, fused head
+ * output), fills params from `seed` (Xavier-uniform; the reference draws
+ * U(+-1/sqrt(fan_in)) from cuRAND Philox, which is not reproducible off CUDA)
+ * and builds the MFMA-ordered weight mirrors.  layers in 1..3. */
+int cfp_policy_create(cfp_policy** out, int num_envs, int layers, uint64_t seed);
+/* cu_policy_free (craftax_full.cu:11907). */
+void cfp_policy_destroy(cfp_policy* p);
+
+int cfp_policy_num_envs(const cfp_policy* p);
+int cfp_policy_layers(const cfp_policy* p);
+size_t cfp_policy_param_count(const cfp_policy* p);
+
+/* Host <-> device copies of the flat params arena (the payload of the
+ * reference's CFW1 checkpoint, cu_save_weights/cu_load_weights
+ * craftax_full.cu:12248/12264).  set_params also rebuilds the mirrors. */
+int cfp_policy_set_params(cfp_policy* p, const float* host_params, size_t count);
+int cfp_policy_get_params(const cfp_policy* p, float* host_params, size_t count);
+/* Rebuild the MFMA-ordered weight mirrors from the params arena after the
+ * arena changed on device: the role of cu_params_refresh_bf16 + cu_pack_wav
+ * (craftax_full.cu:11805-11817) after init / Adam. */
+int cfp_policy_refresh_weights(cfp_policy* p, void* stream);
+
+/* Borrowed device pointers owned by the policy object. */
+float* cfp_policy_params(cfp_policy* p);    /* [param_count]                 */
+float* cfp_policy_state(cfp_policy* p);     /* live h_state [layers][n][256] */
+uint8_t* cfp_policy_rec(cfp_policy* p);     /* record scratch [n][996]       */
+float* cfp_policy_h_enc(cfp_policy* p);     /* [n][256]                      */
+float* cfp_policy_h3(cfp_policy* p);        /* [n][256]                      */
+float* cfp_policy_logits(cfp_policy* p);    /* fused head out [n][44]        */
+void* cfp_policy_stream(cfp_policy* p);     /* the object's own stream       */
+
+/* cu_encode_step (craftax_full.cu:11931), record half onward: consumes
+ * n 996-byte records (rec_row; NULL = the object's scratch) and writes
+ * h_enc[n][256] = b_enc + W_enc^T x.  The reference runs k_expand_obs +
+ * cublasSgemm + k_add_bias; here the byte->fp32 expansion is the GEMM's
+ * operand load and the bias its epilogue, one kernel.  The state->record
+ * half of cu_encode_step is cfp_record_obs below. */
+int cfp_encode_step(cfp_policy* p, const uint8_t* d_rec_row, int n, void* stream);
+
+/* cu_gru_chain (craftax_full.cu:11978): x0[n][256] -> `layers` MinGRU layers
+ * -> h3[n][256].  state[layers][n][256] is read and overwritten; envs with
+ * terminals[e] != 0 see a zero state; r_state_t (nullable) receives the
+ * post-zero state inputs [layers][n][256].  `chunk` envs per launch
+ * (0 = one launch; the reference fixes 16384, craftax_full.cu:11976). */
+int cfp_gru_chain(cfp_policy* p, const float* d_x0, float* d_state,
+                  const float* d_terminals, float* d_r_state_t, float* d_h3,
+                  int n, int chunk, void* stream);
+
+/* Fused head GEMM of cu_rollout_step (craftax_full.cu:12040-12045) plus the
+ * bias adds of k_value_sample (craftax_full.cu:9726-9730):
+ * av[e][a] = b_a[a] + W_a[a].h3[e] for a < 43, av[e][43] = b_v + W_v.h3[e]. */
+int cfp_head(cfp_policy* p, const float* d_h3, float* d_av, int n, void* stream);
+
+/* Policy half of cu_rollout_step (craftax_full.cu:12022-12048) in one launch
+ * per chunk: records -> encoder -> MinGRU x layers -> heads.  Updates d_state
+ * (NULL = the object's live state) in place, writes d_av[n][44] (NULL = the
+ * object's logits buffer); d_r_state_t, d_h_enc, d_h3 are optional outputs
+ * (NULL = not written).  `chunk` as in cfp_gru_chain. */
+int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
+                       const float* d_terminals, float* d_state,
+                       float* d_r_state_t, float* d_h_enc, float* d_h3,
+                       float* d_av, int n, int chunk, void* stream);
+
+/* ---- the dense-math seam (craftax_full.cu:11604-11666) ------------------- */
+/* cu_gemm_fwd (:11604): y[cols][m] = x[cols][k] . W[m][k]^T. */
+int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
+                 float* d_y, void* stream);
+/* cu_gemm_enc_fwd (:11616): h[cols][256] = xobs[cols][843] . W_enc[843][256]. */
+int cfp_gemm_enc_fwd(int cols, const float* d_W_enc, const float* d_xobs,
+                     float* d_h, void* stream);
+/* cu_gemm_dh (:11629): dh[cols][256] = dpre[cols][m3] . W[m3][256]. */
+int cfp_gemm_dh(int m3, int cols, const float* d_W, const float* d_dpre,
+                float* d_dh, void* stream);
+/* cu_gemm_dw (:11642): dW[rows][256] += dpre[cols][rows]^T . x[cols][256]. */
+int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
+                float* d_dW, void* stream);
+/* cu_gemv_dwv (:11655): dWv[256] += x[cols][256]^T . dv[cols]. */
+int cfp_gemv_dwv(const float* d_x, const float* d_dv, float* d_dWv, int cols,
+                 void* stream);
+
+/* k_expand_obs (craftax_full.cu:10028): records -> fp32 features
+ * xobs[count][843].  Sample w maps to record (t0 + w/mb)*n + env_start + w%mb,
+ * the trainer's window addressing; for a plain batch pass t0=0, mb=n=count,
+ * env_start=0. */
+int cfp_expand_obs(const uint8_t* d_r_obs, float* d_xobs, int t0, int count,
+                   int mb, int n, int env_start, void* stream);
+/* k_add_bias (craftax_full.cu:10056): h[cols][256] += b[256]. */
+int cfp_add_bias(float* d_h, const float* d_b, int cols, void* stream);
+/* Unfused k_mingru_epi_fwd (craftax_full.cu:9350): pre[cols][768], x[cols][256],
+ * state[cols][256] in/out, h_out[cols][256], r_state_store nullable. */
+int cfp_mingru_epi_fwd(const float* d_pre, const float* d_x, float* d_state,
+                       float* d_h_out, float* d_r_state_store,
+                       const float* d_prev_terminals, int cols, void* stream);
+
+/* ---- state -> record (k_record_obs, craftax_full.cu:9284; C spec
+ *      craftax_encode_compact_observation, craftax_full.c:2830) ------------ */
+#define CFP_MOB_SLOTS 14 /* melee 3, passive 3, ranged 2, mob-proj 3, player-proj 3 */
+/* The fields of CraftaxState the encoder reads (craftax_full.c:2205-2220,
+ * 2646-2703, 2721-2844), one struct per env.  Mob slots are the entries at
+ * level jax_index(player_level, 9), in class order. */
+typedef struct cfp_env_scalars {
+    int32_t player_position[2];
+    int32_t player_level;
+    int32_t player_direction;            /* 1..4 */
+    float player_health;
+    int32_t player_food, player_drink, player_energy, player_mana;
+    int32_t player_xp, player_dexterity, player_strength, player_intelligence;
+    int32_t is_sleeping, is_resting;
+    int32_t wood, stone, coal, iron, diamond, sapphire, ruby, sapling, torches,
+        arrows, books, pickaxe, sword, bow;
+    int32_t potions[6];
+    int32_t armour[4];
+    int32_t sword_enchantment, bow_enchantment;
+    int32_t armour_enchantments[4];
+    float light_level;
+    int32_t learned_spells[2];
+    int32_t monsters_killed_level;       /* monsters_killed[player_level] */
+    int32_t boss_timesteps_to_spawn_this_round;
+    int32_t mob_type_id[CFP_MOB_SLOTS];
+    int32_t mob_mask[CFP_MOB_SLOTS];
+    int32_t mob_position[CFP_MOB_SLOTS][2];
+} cfp_env_scalars;
+
+/* Writes n records.  map/item_map/light_map: u8 planes of 48x48; plane for
+ * (env, level) starts at base + env*env_stride + level*level_stride (bytes);
+ * level_stride = 0 when only the current level's plane is supplied. */
+int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
+                   const uint8_t* d_item_map, const uint8_t* d_light_map,
+                   size_t env_stride, size_t level_stride, uint8_t* d_rec_row,
+                   int n, void* stream);
+
+/* ---- synthetic inputs for parity tests and bench (no reference
+ *      counterpart; counter-based so host and device agree bit for bit) ---- */
+/* Records: 792 map bytes, each 0 with prob 0.4 else U{0..40}... see synth.hip;
+ * tail floats U[0,1) with 24-bit mantissas.  index = env + n*step. */
+int cfp_synth_records(uint8_t* d_rec, int n, uint64_t seed, uint64_t step,
+                      void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CFP_H_ */

@@ -1,0 +1,157 @@
+"""Shared helpers for the parity tests: seeded inputs, the numpy fp64 policy
+evaluation used to cross-check the C oracle, tolerances, and the smoke check.
+
+Tolerance (from the target statement): logits / values / hidden states within
+1e-4 relative error of an fp64 evaluation of the same fp32 weights for the fp32
+path (2e-2 for bf16 inputs).  "Relative" is taken per tensor against its RMS
+magnitude: |got - ref| <= tol * (|ref| + rms(ref)), so entries that cancel to
+near zero are judged against the tensor's scale rather than their own.
+"""
+import numpy as np
+
+HIDDEN, GRU, OBS, OBS_MAP, OBS_TAIL = 256, 768, 843, 792, 51
+REC_BYTES, ACTIONS, AV = 996, 43, 44
+TOL_FP32 = 1e-4
+TOL_BF16 = 2e-2
+
+_M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
+
+
+def mix64(seed, stream, index):
+    """Counter-based generator shared with the device (csrc/cfp_api.hip mix64)."""
+    with np.errstate(over="ignore"):
+        idx = np.asarray(index, dtype=np.uint64)
+        z = (np.uint64(seed) + np.uint64(stream) * np.uint64(0xD1B54A32D192ED03)
+             + (idx + np.uint64(1)) * np.uint64(0x9E3779B97F4A7C15))
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def unit24(z):
+    return (z >> np.uint64(40)).astype(np.float32) * np.float32(1.0 / 16777216.0)
+
+
+def synth_records_host(n, seed, step):
+    """Bit-identical host twin of cfp_synth_records: [n][996] uint8."""
+    z = mix64(seed, step, np.arange(n * 249, dtype=np.uint64)).reshape(n, 249)
+    out = np.empty((n, 249), dtype=np.uint32)
+    zm = z[:, :198]
+    w = ((zm & np.uint64(0xffff)) % np.uint64(41)).astype(np.uint32)
+    w |= (((zm >> np.uint64(16)) & np.uint64(0xffff)) % np.uint64(41)).astype(np.uint32) << 8
+    w |= (((zm >> np.uint64(32)) & np.uint64(0xffff)) % np.uint64(41)).astype(np.uint32) << 16
+    w |= (((zm >> np.uint64(48)) & np.uint64(0xffff)) % np.uint64(41)).astype(np.uint32) << 24
+    out[:, :198] = w
+    out[:, 198:] = unit24(z[:, 198:]).view(np.uint32)
+    return out.view(np.uint8).reshape(n, REC_BYTES)
+
+
+def expand_records(rec):
+    """k_expand_obs semantics (craftax_full.cu:10028): bytes -> fp32 features."""
+    rec = np.ascontiguousarray(rec).reshape(-1, REC_BYTES)
+    x = np.empty((rec.shape[0], OBS), dtype=np.float32)
+    x[:, :OBS_MAP] = rec[:, :OBS_MAP].astype(np.float32)
+    x[:, OBS_MAP:] = np.ascontiguousarray(rec[:, OBS_MAP:]).view(np.float32)
+    return x
+
+
+def random_params(layers, seed, scale=1.0):
+    """Xavier-uniform-ish random weights in the flat arena layout."""
+    rng = np.random.default_rng(seed)
+    def u(shape, bound):
+        return rng.uniform(-bound, bound, size=shape).astype(np.float32)
+    parts = [
+        u((OBS * HIDDEN,), scale * np.sqrt(6.0 / (OBS + HIDDEN))),
+        u((HIDDEN,), 1.0 / np.sqrt(OBS)),
+        u((layers * GRU * HIDDEN,), scale * np.sqrt(6.0 / (HIDDEN + GRU))),
+        u((ACTIONS * HIDDEN,), scale * np.sqrt(6.0 / (HIDDEN + ACTIONS))),
+        u((ACTIONS,), 1.0 / np.sqrt(HIDDEN)),
+        u((HIDDEN,), scale * np.sqrt(6.0 / (HIDDEN + 1))),
+        u((1,), 1.0 / np.sqrt(HIDDEN)),
+    ]
+    return np.concatenate(parts)
+
+
+def split_params(params, layers):
+    o = {}
+    off = 0
+    for name, shape in (("W_enc", (OBS, HIDDEN)), ("b_enc", (HIDDEN,)),
+                        ("W_gru", (layers, GRU, HIDDEN)), ("W_a", (ACTIONS, HIDDEN)),
+                        ("b_a", (ACTIONS,)), ("W_v", (HIDDEN,)), ("b_v", (1,))):
+        cnt = int(np.prod(shape))
+        o[name] = np.asarray(params[off:off + cnt]).reshape(shape)
+        off += cnt
+    assert off == len(params)
+    return o
+
+
+def sigmoid64(z):
+    return 1.0 / (1.0 + np.exp(-z))
+
+
+def numpy_forward_f64(params, layers, x, state, terminals):
+    """Independent fp64 evaluation with library matmuls (A.2 of the forward spec:
+    craftax_full.cu:9778-9854).  x [n][843], state [L][n][256] -> dict of fp64
+    arrays; state is not modified."""
+    w = {k: v.astype(np.float64) for k, v in split_params(params, layers).items()}
+    h = x.astype(np.float64) @ w["W_enc"] + w["b_enc"]
+    out = {"h_enc": h.copy()}
+    new_state = np.empty((layers,) + h.shape, dtype=np.float64)
+    r_state = np.empty_like(new_state)
+    dz = (np.asarray(terminals) != 0)[:, None]
+    for l in range(layers):
+        st = np.where(dz, 0.0, state[l].astype(np.float64))
+        r_state[l] = st
+        z = h @ w["W_gru"][l].T
+        zh, zg, zp = z[:, :HIDDEN], z[:, HIDDEN:2 * HIDDEN], z[:, 2 * HIDDEN:]
+        gh = np.where(zh >= 0.0, zh + 0.5, sigmoid64(zh))
+        o = st + sigmoid64(zg) * (gh - st)
+        p = sigmoid64(zp)
+        h = p * o + (1.0 - p) * h
+        new_state[l] = o
+    out["h3"] = h
+    out["state"] = new_state
+    out["r_state"] = r_state
+    out["logits"] = h @ w["W_a"].T + w["b_a"]
+    out["values"] = h @ w["W_v"] + w["b_v"][0]
+    return out
+
+
+def rel_err(got, ref):
+    """max over entries of |got-ref| / (|ref| + rms(ref))."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    rms = np.sqrt(np.mean(ref * ref)) + 1e-30
+    return float(np.max(np.abs(got - ref) / (np.abs(ref) + rms)))
+
+
+def assert_close(got, ref, tol, what):
+    e = rel_err(got, ref)
+    assert np.all(np.isfinite(np.asarray(got))), f"{what}: non-finite values"
+    assert e <= tol, f"{what}: relative error {e:.3e} exceeds {tol:.1e}"
+    return e
+
+
+def smoke_forward(pkg):
+    """One small fused forward on cuda:0 against the CPU oracle."""
+    import torch
+    import oracle_bind
+    n, layers = 64, 3
+    params = random_params(layers, 11)
+    pol = pkg.Policy(n, layers, seed=1)
+    pol.set_params(params)
+    rec_h = synth_records_host(n, 5, 0)
+    rng = np.random.default_rng(3)
+    state_h = (0.5 * rng.standard_normal((layers, n, HIDDEN))).astype(np.float32)
+    term_h = (rng.random(n) < 0.25).astype(np.float32)
+    rec = torch.from_numpy(rec_h).cuda()
+    state = torch.from_numpy(state_h.copy()).cuda()
+    term = torch.from_numpy(term_h).cuda()
+    av = pol.forward(rec, term, state)
+    torch.cuda.synchronize()
+    ref = oracle_bind.forward_f64(params, layers, expand_records(rec_h), state_h, term_h)
+    av_h = av.cpu().numpy()
+    assert_close(av_h[:, :ACTIONS], ref["logits"], TOL_FP32, "smoke logits")
+    assert_close(av_h[:, ACTIONS], ref["values"], TOL_FP32, "smoke values")
+    assert_close(state.cpu().numpy(), ref["state"], TOL_FP32, "smoke state")
+    pol.close()
