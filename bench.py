@@ -1,0 +1,162 @@
+#!/usr/bin/env python3
+"""Benchmark of the batched policy forward on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--envs N] [--no-cpu]
+
+One step = one pass of the fused policy forward (996-byte records -> encoder
+-> MinGRU x3 -> actor/value heads) over one batch of synthetic records that is
+already resident in HBM, hidden state carried from step to step.  The default
+workload is the baseline's third config: 262 144 envs, h256x3, one unchunked
+launch per step; the 16 x 16 384 chunked schedule is timed beside it.
+
+Prints ONE JSON line (metric = env-steps/s) with two extra objects:
+  roofline     algorithmic FLOPs per launch / measured launch time vs the
+               MI355X fp32 MFMA peak (HIP events on the launch stream)
+  cpu_baseline the CPU oracle's scalar fp32 forward timed on this host's cores
+               on a bounded sample of the same workload
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+FLOP_PER_ENV_STEP = 2 * 843 * 256 + 3 * 2 * 768 * 256 + 2 * 44 * 256   # 1 633 792
+BYTES_PER_ENV_STEP = 996 + 4 + 3 * 256 * 4 * 2 + 44 * 4                # 7 320
+PEAK_FP32_MFMA_TFLOPS = 157.3
+LAYERS = 3
+# HBM bytes per launch at 262 144 envs from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/policy_forward_262144_pmc.txt), scaled by the copy-kernel factor
+# stated in DESIGN.md; None until measured for another size.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--envs", type=int, default=262144)
+    ap.add_argument("--ring", type=int, default=16,
+                    help="distinct pre-generated record batches cycled through")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    return ap.parse_args()
+
+
+def time_steps(pol, recs, term, state, av, steps, chunk, torch):
+    """Time `steps` forwards with HIP events on the launch stream; returns
+    (wall seconds for all steps, mean per-step device milliseconds)."""
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+          for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        ev[i][0].record()
+        pol.forward(recs[i % len(recs)], term, state, av=av, chunk=chunk)
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = sum(a.elapsed_time(b) for a, b in ev) / steps
+    return wall, dev_ms
+
+
+def cpu_baseline(params, seed):
+    """CPU oracle (scalar fp32 port of the reference's k_policy_ref_l3) on a
+    bounded sample: 32 768 envs x 12 steps, state carried, all host threads the
+    box grants (at most 16)."""
+    import numpy as np
+    import oracle_bind as ob
+    from parity_util import HIDDEN, synth_records_host
+    threads = max(1, min(16, ob.cfo().cfo_max_threads(), os.cpu_count() or 1))
+    n, steps = 32768, 12
+    state = np.zeros((LAYERS, n, HIDDEN), np.float32)
+    term = np.zeros(n, np.float32)
+    recs = [synth_records_host(n, seed, s) for s in range(2)]
+    ob.forward_f32(params, LAYERS, recs[0][:1024], state[:, :1024].copy(), term[:1024], threads)
+    t0 = time.perf_counter()
+    for s in range(steps):
+        ob.forward_f32(params, LAYERS, recs[s % 2], state, term, threads)
+    dt = time.perf_counter() - t0
+    out = {"value": n * steps / dt, "unit": "env-steps/s", "cores": threads, "kind": "port",
+           "sample": f"{n} envs x {steps} steps of the same forward (oracle/policy_ref.c "
+                     f"cfo_forward_f32, OpenMP, {dt:.1f} s)",
+           "gflops": FLOP_PER_ENV_STEP * n * steps / dt / 1e9}
+    if ob.have_ref():
+        # the reference's own CPU env (random actions), for orientation only: a
+        # different path (env step, not policy forward)
+        sps1 = ob.ref().cfref_bench(1024, 300, 1, 0)
+        spsN = ob.ref().cfref_bench(8192, 60, threads, 0)
+        out["reference_env_sps"] = {"1024_envs_1_thread": sps1,
+                                    f"8192_envs_{threads}_threads": spsN}
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py: this build runs on one GPU only (--gpus {args.gpus} was asked "
+              "for); envs are independent, so N GPUs would each run this same kernel on "
+              "n/N envs with no exchange", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    n, steps, warmup = args.envs, args.steps, args.warmup
+    seed = 1234
+    pol = pkg.Policy(n, LAYERS, seed=1)          # weights: Xavier-uniform from seed 1
+    params = pol.get_params()
+    ring = max(1, min(args.ring, steps))
+    recs = [pkg.policy.synth_records(n, seed, s) for s in range(ring)]
+    term = (torch.rand(n, device="cuda") < 0.0034).float()   # the real env's terminal rate
+    av = torch.empty(n, 44, device="cuda")
+    state = pol.state
+    torch.cuda.synchronize()
+
+    results = {}
+    for name, chunk in (("unchunked", 0), ("chunked_16x16384", 16384 if n > 16384 else 0)):
+        state.zero_()
+        for i in range(warmup):
+            pol.forward(recs[i % ring], term, state, av=av, chunk=chunk)
+        wall, dev_ms = time_steps(pol, recs, term, state, av, steps, chunk, torch)
+        results[name] = {"ms_per_step": wall / steps * 1e3, "device_ms_per_step": dev_ms,
+                         "env_steps_per_s": n * steps / wall}
+    assert torch.isfinite(av).all(), "non-finite policy outputs"
+
+    best = results["unchunked"]
+    launch_s = best["device_ms_per_step"] * 1e-3            # one launch per step
+    achieved = FLOP_PER_ENV_STEP * n / launch_s / 1e12
+    line = {
+        "metric": "policy-forward env-steps/sec @262k envs h256x3; % fp32 MFMA peak",
+        "value": best["env_steps_per_s"], "unit": "env-steps/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": best["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"policy forward h256x3, {n} envs, one unchunked launch per "
+                               f"step, {steps} consecutive steps carrying hidden state, "
+                               "synthetic 996-byte records resident in HBM",
+                   "envs": n, "layers": LAYERS, "hidden": 256, "chunk": 0,
+                   "record_batches_in_hbm": ring},
+        "pct_fp32_mfma_peak": 100.0 * achieved / PEAK_FP32_MFMA_TFLOPS,
+        "chunked_16x16384": results["chunked_16x16384"],
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(n),
+                     "kernel": "k_policy_forward",
+                     "flops_per_launch": FLOP_PER_ENV_STEP * n,
+                     "algorithmic_hbm_bytes_per_launch": BYTES_PER_ENV_STEP * n,
+                     "launch_ms": best["device_ms_per_step"]},
+    }
+    pol.close()
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(params, seed)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -82,7 +82,11 @@ class Policy:
             lib().cfp_policy_destroy(self._h)
             self._h = C.c_void_p()
 
-    __del__ = close
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:   # interpreter shutdown: module globals may be gone
+            pass
 
     # -- parameters ----------------------------------------------------
     def set_params(self, host_params):

@@ -1,0 +1,160 @@
+/*
+ * CPU restatement of the policy forward.  TEST INFRASTRUCTURE ONLY (see cfo.h).
+ *
+ * Follows craftax_full.cu:
+ *   k_policy_ref_l3                         :9778-9854  (the scalar spec)
+ *   cf_nn_sigmoid / cf_nn_mingru_g          :9133-9138
+ *   k_mingru_epi_fwd (state zeroing, order) :9350-9395
+ *   parameter arena layout                  :9094-9102
+ */
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#include "cfo.h"
+
+enum { H = CFP_HIDDEN, G = CFP_GRU, F = CFP_OBS, FM = CFP_OBS_MAP, A = CFP_ACTIONS };
+
+int cfo_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+static double sigmoid64(double x) { return 1.0 / (1.0 + exp(-x)); }
+static double mingru_g64(double x) { return x >= 0.0 ? x + 0.5 : sigmoid64(x); }
+
+void cfo_forward_f64(const float* params, int layers, int n, const float* x,
+                     const double* state_in, const float* prev_terminals,
+                     double* h_enc, double* r_state, double* state_out,
+                     double* h3, double* logits, double* values) {
+    const float* W_enc = params + CFP_OFF_W_ENC;
+    const float* b_enc = params + CFP_OFF_B_ENC;
+    const float* W_gru = params + CFP_OFF_W_GRU;
+    const float* W_a = params + CFP_OFF_W_A(layers);
+    const float* b_a = params + CFP_OFF_B_A(layers);
+    const float* W_v = params + CFP_OFF_W_V(layers);
+    const float* b_v = params + CFP_OFF_B_V(layers);
+    const size_t hn = (size_t)H * n;
+
+#pragma omp parallel for schedule(static)
+    for (int e = 0; e < n; e++) {
+        double h[H], h2[H];
+        const float* xe = x + (size_t)e * F;
+        for (int k = 0; k < H; k++) h[k] = (double)b_enc[k];
+        for (int f = 0; f < F; f++) {
+            const double xf = (double)xe[f];
+            if (xf == 0.0) continue;
+            const float* w = W_enc + (size_t)f * H;
+            for (int k = 0; k < H; k++) h[k] += xf * (double)w[k];
+        }
+        if (h_enc) memcpy(h_enc + (size_t)e * H, h, sizeof(h));
+        const int dz = prev_terminals && prev_terminals[e] != 0.0f;
+        for (int l = 0; l < layers; l++) {
+            const float* Wl = W_gru + (size_t)l * G * H;
+            const size_t so = (size_t)l * hn + (size_t)e * H;
+            for (int k = 0; k < H; k++) {
+                const double st = dz ? 0.0 : state_in[so + k];
+                if (r_state) r_state[so + k] = st;
+                double zh = 0.0, zg = 0.0, zp = 0.0;
+                const float* wh = Wl + (size_t)k * H;
+                const float* wg = Wl + (size_t)(H + k) * H;
+                const float* wp = Wl + (size_t)(2 * H + k) * H;
+                for (int j = 0; j < H; j++) {
+                    zh += (double)wh[j] * h[j];
+                    zg += (double)wg[j] * h[j];
+                    zp += (double)wp[j] * h[j];
+                }
+                const double out = st + sigmoid64(zg) * (mingru_g64(zh) - st);
+                const double p = sigmoid64(zp);
+                h2[k] = p * out + (1.0 - p) * h[k];
+                if (state_out) state_out[so + k] = out;
+            }
+            memcpy(h, h2, sizeof(h));
+        }
+        if (h3) memcpy(h3 + (size_t)e * H, h, sizeof(h));
+        if (logits)
+            for (int a = 0; a < A; a++) {
+                double z = (double)b_a[a];
+                for (int j = 0; j < H; j++) z += (double)W_a[a * H + j] * h[j];
+                logits[(size_t)e * A + a] = z;
+            }
+        if (values) {
+            double v = (double)b_v[0];
+            for (int j = 0; j < H; j++) v += (double)W_v[j] * h[j];
+            values[e] = v;
+        }
+    }
+}
+
+static float sigmoid32(float x) { return 1.0f / (1.0f + expf(-x)); }
+static float mingru_g32(float x) { return x >= 0.0f ? x + 0.5f : sigmoid32(x); }
+
+void cfo_forward_f32(const float* params, int layers, int n, const uint8_t* rec,
+                     float* state, const float* prev_terminals, float* av,
+                     int threads) {
+    const float* W_enc = params + CFP_OFF_W_ENC;
+    const float* b_enc = params + CFP_OFF_B_ENC;
+    const float* W_gru = params + CFP_OFF_W_GRU;
+    const float* W_a = params + CFP_OFF_W_A(layers);
+    const float* b_a = params + CFP_OFF_B_A(layers);
+    const float* W_v = params + CFP_OFF_W_V(layers);
+    const float* b_v = params + CFP_OFF_B_V(layers);
+    const size_t hn = (size_t)H * n;
+#ifdef _OPENMP
+    if (threads <= 0) threads = omp_get_max_threads();
+#else
+    threads = 1;
+#endif
+
+#pragma omp parallel for schedule(static) num_threads(threads)
+    for (int e = 0; e < n; e++) {
+        float h[H], h2[H];
+        const uint8_t* r = rec + (size_t)e * CFP_REC_BYTES;
+        for (int k = 0; k < H; k++) h[k] = b_enc[k];
+        for (int f = 0; f < F; f++) {
+            float xf;
+            if (f < FM) xf = (float)r[f];
+            else memcpy(&xf, r + FM + 4 * (f - FM), sizeof(float));
+            if (xf == 0.0f) continue;
+            const float* w = W_enc + (size_t)f * H;
+            for (int k = 0; k < H; k++) h[k] = fmaf(xf, w[k], h[k]);
+        }
+        const int dz = prev_terminals && prev_terminals[e] != 0.0f;
+        for (int l = 0; l < layers; l++) {
+            const float* Wl = W_gru + (size_t)l * G * H;
+            float* st_l = state + (size_t)l * hn + (size_t)e * H;
+            for (int k = 0; k < H; k++) {
+                const float st = dz ? 0.0f : st_l[k];
+                float zh = 0.0f, zg = 0.0f, zp = 0.0f;
+                const float* wh = Wl + (size_t)k * H;
+                const float* wg = Wl + (size_t)(H + k) * H;
+                const float* wp = Wl + (size_t)(2 * H + k) * H;
+                for (int j = 0; j < H; j++) {
+                    zh = fmaf(wh[j], h[j], zh);
+                    zg = fmaf(wg[j], h[j], zg);
+                    zp = fmaf(wp[j], h[j], zp);
+                }
+                const float out = st + sigmoid32(zg) * (mingru_g32(zh) - st);
+                const float p = sigmoid32(zp);
+                h2[k] = p * out + (1.0f - p) * h[k];
+                st_l[k] = out;
+            }
+            memcpy(h, h2, sizeof(h));
+        }
+        float* ave = av + (size_t)e * CFP_AV;
+        for (int a = 0; a < A; a++) {
+            float z = b_a[a];
+            for (int j = 0; j < H; j++) z = fmaf(W_a[a * H + j], h[j], z);
+            ave[a] = z;
+        }
+        float v = b_v[0];
+        for (int j = 0; j < H; j++) v = fmaf(W_v[j], h[j], v);
+        ave[A] = v;
+    }
+}

@@ -1,0 +1,60 @@
+"""The C-ABI library loads and exports exactly what include/cfp.h declares; no
+compute is launched here (runs without a GPU)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "cfp.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cfp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported(pkg):
+    lib = C.CDLL(pkg._lib.LIB_PATH)
+    names = _declared()
+    assert len(names) >= 25
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in cfp.h but not exported"
+
+
+def test_binding_covers_every_declaration(pkg):
+    assert sorted(pkg._lib.PROTOTYPES) == _declared()
+
+
+def test_env_scalars_layout_matches_binding():
+    import oracle_bind as ob
+    text = open(os.path.join(ROOT, "include", "cfp.h")).read()
+    body = text[text.index("typedef struct cfp_env_scalars {"):text.index("} cfp_env_scalars;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    n_i32 = 0
+    for stmt in body.split("{", 1)[1].split(";"):
+        m = re.match(r"\s*(int32_t|float)\s+(.*)", stmt.strip(), flags=re.S)
+        if not m:
+            continue
+        for decl in m.group(2).split(","):
+            cnt = 1
+            for d in re.findall(r"\[(\w+)\]", decl):
+                cnt *= int(d) if d.isdigit() else {"CFP_MOB_SLOTS": 14}[d]
+            n_i32 += cnt
+    assert n_i32 * 4 == ob.SCALARS_BYTES == 424
+
+
+def test_argument_validation_needs_no_gpu(pkg):
+    """Bad arguments are rejected with a message before any HIP call, like the
+    reference's exit(1) paths (craftax_full.cu:11820-11825)."""
+    lib = pkg.lib()
+    h = C.c_void_p()
+    assert lib.cfp_policy_create(C.byref(h), 100, 3, 1) != 0          # not a multiple of 32
+    assert b"multiple of 32" in lib.cfp_last_error()
+    assert lib.cfp_policy_create(C.byref(h), 64, 4, 1) != 0           # layers out of range
+    assert b"layers" in lib.cfp_last_error()
+    assert lib.cfp_policy_create(None, 64, 3, 1) != 0
+    assert lib.cfp_gemm_fwd(0, 1, 1, None, None, None, None) != 0
+    assert lib.cfp_encode_step(None, None, 32, None) != 0
+    assert lib.cfp_abi_version() >= 1

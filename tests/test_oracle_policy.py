@@ -1,0 +1,252 @@
+"""Pins the CPU oracle's policy forward / PPO backward (oracle/policy_ref.c,
+oracle/policy_bwd_ref.c) against an independent numpy fp64 evaluation, closed
+forms, brute force and finite differences."""
+import numpy as np
+import pytest
+
+import oracle_bind as ob
+from parity_util import (ACTIONS, GRU, HIDDEN, OBS, expand_records, numpy_forward_f64,
+                         random_params, rel_err, split_params, synth_records_host)
+
+L = 3
+
+
+def _inputs(n, seed, term_p=0.3):
+    rng = np.random.default_rng(seed)
+    rec = synth_records_host(n, seed, 0)
+    x = expand_records(rec)
+    state = (0.5 * rng.standard_normal((L, n, HIDDEN))).astype(np.float32)
+    term = (rng.random(n) < term_p).astype(np.float32)
+    return rec, x, state, term
+
+
+def test_c_oracle_matches_numpy_fp64():
+    params = random_params(L, 1)
+    rec, x, state, term = _inputs(48, 2)
+    a = ob.forward_f64(params, L, x, state, term)
+    b = numpy_forward_f64(params, L, x, state, term)
+    for k in ("h_enc", "r_state", "state", "h3", "logits", "values"):
+        assert rel_err(a[k], b[k]) < 1e-12, k
+
+
+def test_zero_gate_weights_closed_form():
+    """W_gru = 0 => zh=zg=zp=0 => out = 0.5 st + 0.25, h' = 0.5 out + 0.5 h."""
+    params = random_params(L, 3)
+    sp = split_params(params, L)
+    sp["W_gru"][...] = 0.0
+    rec, x, state, term = _inputs(16, 4, term_p=0.0)
+    r = ob.forward_f64(params, L, x, state, None)
+    h = x.astype(np.float64) @ sp["W_enc"].astype(np.float64) + sp["b_enc"]
+    for l in range(L):
+        out = 0.5 * state[l].astype(np.float64) + 0.25
+        assert np.allclose(r["state"][l], out, rtol=0, atol=1e-14)
+        h = 0.5 * out + 0.5 * h
+    assert np.allclose(r["h3"], h, rtol=1e-13, atol=1e-13)
+
+
+def test_terminal_zeroes_state_and_zero_features_give_bias():
+    params = random_params(L, 5)
+    sp = split_params(params, L)
+    rec, x, state, _ = _inputs(8, 6)
+    term = np.array([1, 0, 1, 0, 0, 0, 0, 1], np.float32)
+    r = ob.forward_f64(params, L, x, state, term)
+    assert not r["r_state"][:, term != 0].any()
+    assert np.array_equal(r["r_state"][:, term == 0], state[:, term == 0].astype(np.float64))
+    z = ob.forward_f64(params, L, np.zeros_like(x), state, term)
+    assert np.allclose(z["h_enc"], np.broadcast_to(sp["b_enc"].astype(np.float64), (8, HIDDEN)))
+    # zeroed state == explicit zero state
+    st0 = state.copy(); st0[:, term != 0] = 0
+    r0 = ob.forward_f64(params, L, x, st0, None)
+    assert np.array_equal(r0["logits"], r["logits"])
+
+
+def test_gate_saturation_limits():
+    """p -> 1 gives h' = out, p -> 0 gives h' = x; zg -> +inf gives out = g(zh)."""
+    params = random_params(1, 7)
+    sp = split_params(params, 1)
+    sp["W_enc"][...] = 0.0; sp["b_enc"][...] = 1.0       # h = 1 for every unit
+    W = sp["W_gru"][0]; W[...] = 0.0
+    W[2 * HIDDEN:, :] = 1.0                               # zp = +256 -> p = 1
+    x = np.zeros((4, OBS), np.float32)
+    state = np.full((1, 4, HIDDEN), 0.3, np.float32)
+    r = ob.forward_f64(params, 1, x, state, None)
+    assert np.allclose(r["h3"], r["state"][0])
+    W[2 * HIDDEN:, :] = -1.0                              # p = 0
+    r = ob.forward_f64(params, 1, x, state, None)
+    assert np.allclose(r["h3"], 1.0, atol=1e-100)
+    W[HIDDEN:2 * HIDDEN, :] = 1.0; W[:HIDDEN, :] = 0.01   # sg = 1, zh = 2.56
+    r = ob.forward_f64(params, 1, x, state, None)
+    assert np.allclose(r["state"][0], 2.56 + 0.5, rtol=1e-6)
+    W[:HIDDEN, :] = -0.01                                  # zh = -2.56 -> sigmoid
+    r = ob.forward_f64(params, 1, x, state, None)
+    assert np.allclose(r["state"][0], 1 / (1 + np.exp(2.56)), rtol=1e-6)
+
+
+def test_fp32_port_tracks_fp64_and_carries_state():
+    params = random_params(L, 8)
+    n, T = 24, 6
+    rng = np.random.default_rng(9)
+    st32 = np.zeros((L, n, HIDDEN), np.float32)
+    st64 = np.zeros((L, n, HIDDEN), np.float64)
+    for t in range(T):
+        rec = synth_records_host(n, 10, t)
+        term = (rng.random(n) < 0.2).astype(np.float32) if t else np.zeros(n, np.float32)
+        av = ob.forward_f32(params, L, rec, st32, term, threads=2)
+        r = ob.forward_f64(params, L, expand_records(rec), st64, term)
+        st64 = r["state"]
+        assert rel_err(av[:, :ACTIONS], r["logits"]) < 1e-4
+        assert rel_err(av[:, ACTIONS], r["values"]) < 1e-4
+        assert rel_err(st32, st64) < 1e-4
+
+
+def test_multi_step_carry_brute_force():
+    """n=4, T=8 in plain numpy loops over time, random terminals."""
+    params = random_params(L, 11)
+    n, T = 4, 8
+    rng = np.random.default_rng(12)
+    st_o = np.zeros((L, n, HIDDEN)); st_n = np.zeros((L, n, HIDDEN))
+    for t in range(T):
+        x = expand_records(synth_records_host(n, 13, t))
+        term = (rng.random(n) < 0.4).astype(np.float32)
+        a = ob.forward_f64(params, L, x, st_o, term)
+        b = numpy_forward_f64(params, L, x, st_n, term)
+        st_o, st_n = a["state"], b["state"]
+        assert rel_err(a["logits"], b["logits"]) < 1e-12
+    assert rel_err(st_o, st_n) < 1e-12
+
+
+# ---- PPO update ------------------------------------------------------------------
+def _rollout(params, n, T, seed, done_p=0.1, layers=L):
+    """Synthetic stored rollout whose r_state is what the oracle forward itself
+    would have recorded (zero initial state, zeroed after a done)."""
+    rng = np.random.default_rng(seed)
+    r_obs = np.stack([synth_records_host(n, seed, t) for t in range(T)])
+    r_done = (rng.random((T, n)) < done_p).astype(np.uint8)
+    r_state = np.zeros((T, layers, n, HIDDEN), np.float32)
+    st = np.zeros((layers, n, HIDDEN))
+    for t in range(T):
+        term = r_done[t - 1].astype(np.float32) if t else np.zeros(n, np.float32)
+        r = ob.forward_f64(params, layers, expand_records(r_obs[t]), st, term)
+        r_state[t] = r["r_state"]
+        st = r["r_state"].astype(np.float32).astype(np.float64) * 0 + r["state"]
+        # the stored record is fp32; keep the live carry consistent with it
+        st = np.where(np.isfinite(st), st, 0.0)
+    r_act = rng.integers(0, ACTIONS, (T, n)).astype(np.int32)
+    r_logprob = np.full((T, n), -np.log(ACTIONS), np.float32) + 0.1 * rng.standard_normal((T, n)).astype(np.float32)
+    adv = rng.standard_normal((T, n)).astype(np.float32)
+    ret = rng.standard_normal((T, n)).astype(np.float32)
+    return dict(r_obs=r_obs, r_state=r_state, r_act=r_act, r_logprob=r_logprob, adv=adv,
+                ret=ret, r_done=r_done)
+
+
+def _consistent_rollout(params, n, T, seed, done_p=0.1):
+    """As _rollout, but the stored fp32 state is also what the live recurrence
+    carries (state rounded to fp32 each step), so loss (live) == recompute (stored)."""
+    rng = np.random.default_rng(seed)
+    ro = _rollout(params, n, T, seed, done_p)
+    st = np.zeros((L, n, HIDDEN), np.float32)
+    for t in range(T):
+        term = ro["r_done"][t - 1].astype(np.float32) if t else np.zeros(n, np.float32)
+        r = ob.forward_f64(params, L, expand_records(ro["r_obs"][t]), st, term)
+        ro["r_state"][t] = r["r_state"].astype(np.float32)
+        st = r["state"].astype(np.float32)
+    return ro
+
+
+def test_backward_matches_finite_differences():
+    """The reference's own gradcheck method (craftax_full.cu:13854-13907): central
+    differences of the loss on the largest-|g| and random parameters; fail if
+    diff > 2e-4 and rel > 3e-2.  In fp64 the agreement is far tighter (1e-5
+    relative with a 1e-5 step; the synthetic features are large, so the loss has
+    strong curvature and a 1e-3 step is already 0.25 % off)."""
+    params = random_params(L, 21)
+    n, T = 6, 5
+    ro = _consistent_rollout(params, n, T, 22, done_p=0.15)
+    batch, keep = ob.make_batch(T, n, 0, n, L, T, **ro)
+    g, l3 = ob.ppo_backward_f64(params, batch)
+    loss, l3b = ob.ppo_loss_f64(params, batch)
+    assert np.allclose(l3, l3b, rtol=1e-6), "recompute and live replay disagree on the loss"
+    rng = np.random.default_rng(23)
+    o = {k: v for k, v in zip(("W_enc", "b_enc", "W_gru", "W_a", "b_a", "W_v", "b_v"),
+                              np.cumsum([0, OBS * HIDDEN, HIDDEN, L * GRU * HIDDEN,
+                                         ACTIONS * HIDDEN, ACTIONS, HIDDEN]))}
+    probes = list(np.argsort(-np.abs(g))[:8]) + list(rng.integers(0, params.size, 24))
+    probes += [o["b_enc"] + 3, o["W_gru"] + 5, o["W_gru"] + GRU * HIDDEN + 77,
+               o["W_gru"] + 2 * GRU * HIDDEN + 600 * HIDDEN + 9, o["b_a"] + 2, o["W_v"] + 1,
+               o["b_v"]]
+    worst = 0.0
+    for i in probes:
+        eps = 1e-5 * max(1.0, abs(float(params[i])))   # curvature is large: see docstring
+        pp = params.copy(); pp[i] += eps
+        pm = params.copy(); pm[i] -= eps
+        # fp32 params: use the actually representable step
+        h = (float(pp[i]) - float(pm[i]))
+        fd = (ob.ppo_loss_f64(pp, batch)[0] - ob.ppo_loss_f64(pm, batch)[0]) / h
+        diff = abs(fd - g[i]); rel = diff / max(abs(fd), abs(g[i]), 1e-12)
+        worst = max(worst, min(diff / 2e-6, rel / 1e-5))
+        assert not (diff > 2e-6 and rel > 1e-5), (int(i), fd, g[i])
+    assert worst < 1.0
+
+
+def test_backward_truncation_and_done_semantics():
+    params = random_params(L, 31)
+    n, T = 4, 6
+    ro = _consistent_rollout(params, n, T, 32, done_p=0.0)
+    full, k1 = ob.make_batch(T, n, 0, n, L, T, **ro)
+    split, k2 = ob.make_batch(T, n, 0, n, L, 2, **ro)      # bptt_split = 3
+    g_full, _ = ob.ppo_backward_f64(params, full)
+    g_split, _ = ob.ppo_backward_f64(params, split)
+    assert not np.allclose(g_full, g_split)                 # dcarry cut changes grads
+    # all dones set: every step's dcarry is blocked => equals seg_len = 1
+    ro1 = dict(ro); ro1["r_done"] = np.ones_like(ro["r_done"])
+    a, k3 = ob.make_batch(T, n, 0, n, L, T, **ro1)
+    b, k4 = ob.make_batch(T, n, 0, n, L, 1, **ro)
+    ga, _ = ob.ppo_backward_f64(params, a)
+    gb, _ = ob.ppo_backward_f64(params, b)
+    assert np.allclose(ga, gb, rtol=1e-12, atol=1e-15)
+    # heads get gradient only from their own step: unaffected by truncation
+    oa = OBS * HIDDEN + HIDDEN + L * GRU * HIDDEN
+    assert np.allclose(g_full[oa:], g_split[oa:], rtol=1e-12, atol=1e-15)
+
+
+def test_zero_advantage_gives_entropy_and_value_gradient_only():
+    params = random_params(L, 41)
+    n, T = 4, 3
+    ro = _consistent_rollout(params, n, T, 42)
+    ro["adv"] = np.full((T, n), 0.7, np.float32)            # constant => normalised A = 0
+    b, k = ob.make_batch(T, n, 0, n, L, T, **ro)
+    g, l3 = ob.ppo_backward_f64(params, b)
+    assert abs(l3[0]) < 1e-6                                # policy loss term vanishes
+    b2, k2 = ob.make_batch(T, n, 0, n, L, T, **ro, vf=0.0, ent=0.0)
+    g2, _ = ob.ppo_backward_f64(params, b2)
+    assert np.abs(g2).max() < 1e-7
+    assert np.abs(g).max() > 1e-6
+
+
+def test_gae_and_adam_closed_forms():
+    T, n = 5, 3
+    rng = np.random.default_rng(51)
+    values = rng.standard_normal((T, n)).astype(np.float32)
+    rewards = rng.standard_normal((T, n)).astype(np.float32)
+    dones = (rng.random((T, n)) < 0.3).astype(np.uint8)
+    vboot = rng.standard_normal(n).astype(np.float32)
+    adv = np.zeros((T, n)); ret = np.zeros((T, n))
+    ob.cfo().cfo_gae_f64(values.ctypes.data, rewards.ctypes.data, dones.ctypes.data,
+                         vboot.ctypes.data, adv.ctypes.data, ret.ctypes.data, n, T, 0.99, 0.95)
+    # textbook: A_t = sum_k (gamma*lam)^k * prod(nonterm) * delta_{t+k}
+    for e in range(n):
+        for t in range(T):
+            acc, w = 0.0, 1.0
+            for k in range(t, T):
+                vn = float(vboot[e] if k == T - 1 else values[k + 1, e])
+                nt = 0.0 if dones[k, e] else 1.0
+                acc += w * (float(rewards[k, e]) + 0.99 * vn * nt - float(values[k, e]))
+                w *= 0.99 * 0.95 * nt
+            assert abs(acc - adv[t, e]) < 1e-12
+            assert abs(acc + float(values[t, e]) - ret[t, e]) < 1e-12
+    # Adam, first step from zero moments: update = lr * sign(g) (up to eps)
+    p = np.array([1.0, -2.0, 3.0]); g = np.array([0.5, -0.25, 0.0])
+    m = np.zeros(3); v = np.zeros(3)
+    ob.cfo().cfo_adam_f64(p.ctypes.data, g.ctypes.data, m.ctypes.data, v.ctypes.data, 3, 1,
+                          3e-4, 0.9, 0.999, 1e-8)
+    assert np.allclose(p, [1.0 - 3e-4, -2.0 + 3e-4, 3.0], atol=1e-9)
