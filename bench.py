@@ -44,6 +44,9 @@ def parse():
     ap.add_argument("--ring", type=int, default=16,
                     help="distinct pre-generated record batches cycled through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
+                    help="only run a plain device copy of this many MiB four times "
+                         "(calibrates the FETCH_SIZE / WRITE_SIZE counters) and exit")
     return ap.parse_args()
 
 
@@ -107,6 +110,14 @@ def main():
     pkg = ge.load_package()
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.copy_probe:
+        src = torch.full((args.copy_probe << 20,), 7, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_probe_bytes": src.numel(), "copies": 4}))
+        return
     n, steps, warmup = args.envs, args.steps, args.warmup
     seed = 1234
     pol = pkg.Policy(n, LAYERS, seed=1)          # weights: Xavier-uniform from seed 1

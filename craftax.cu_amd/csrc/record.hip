@@ -139,7 +139,10 @@ __global__ __launch_bounds__(256) void k_record_obs(
         const float xi = (float)iv;
         float v = 0.0f;
         switch (ts.kind) {
-            case T_SQRT10: v = __fsqrt_rn(xi) * 0.1f; break;
+            // IEEE sqrt: HIP's __fsqrt_rn is the approximate native sqrt unless
+            // OCML_BASIC_ROUNDED_OPERATIONS is defined; the fp64 root rounded
+            // to fp32 is the correctly rounded fp32 root (53 >= 2*24 + 2).
+            case T_SQRT10: v = (float)sqrt((double)xi) * 0.1f; break;
             case T_HALF: v = xi * 0.5f; break;
             case T_QUARTER: v = xi * 0.25f; break;
             case T_INT: v = xi; break;

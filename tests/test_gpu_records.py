@@ -29,6 +29,28 @@ def test_record_obs_matches_reference_vectors(pkg, cuda, golden, key):
     assert bad.size == 0, f"{bad.size} of {n} records differ, first {bad[:5]}"
 
 
+def test_record_tail_brute_force(pkg, cuda, golden):
+    """Every inventory value 0..99 through the device tail (IEEE sqrtf * 0.1f)."""
+    import torch
+    sc = np.zeros((100, ob.SCALARS_BYTES), np.uint8)
+    s32, f32 = sc.view(np.int32), sc.view(np.float32)
+    off = {f[0]: getattr(ob.EnvScalars, f[0]).offset // 4 for f in ob.EnvScalars._fields_}
+    for v in range(100):
+        for nme in ("wood", "stone", "coal", "iron", "diamond", "sapphire", "ruby", "sapling",
+                    "torches", "arrows", "player_food", "player_drink", "player_energy",
+                    "player_mana", "player_xp", "player_dexterity", "player_strength",
+                    "player_intelligence"):
+            s32[v, off[nme]] = v
+        s32[v, off["potions"]:off["potions"] + 6] = v
+        f32[v, off["player_health"]] = np.float32(v * 0.09)
+        s32[v, off["player_direction"]] = 1
+    planes = torch.zeros(100 * 3 * P, dtype=torch.uint8, device=cuda)
+    rec = pkg.policy.record_obs(_t(sc, cuda), planes, planes[P:], planes[2 * P:], 100, 3 * P, 0)
+    torch.cuda.synchronize()
+    got = np.ascontiguousarray(rec.cpu().numpy()[:, 792:]).view(np.uint32)
+    assert np.array_equal(got, golden["tail_probe"].view(np.uint32))
+
+
 def test_record_obs_full_level_planes(pkg, cuda, golden):
     """Same vectors laid out as the real env holds them: [env][9 levels][48][48],
     level_stride = 2304, so raw-level and clamped-level indexing are exercised."""
