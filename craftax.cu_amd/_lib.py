@@ -49,8 +49,34 @@ PROTOTYPES = {
     "cfp_mingru_epi_fwd": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int, vp]),
     "cfp_record_obs": (C.c_int, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp,
                                  C.c_int, vp]),
+    "cfp_ppo_defaults": (C.c_int, [vp]),
+    "cfp_train_create": (C.c_int, [C.POINTER(vp), vp, C.c_int, vp]),
+    "cfp_train_destroy": (None, [vp]),
+    "cfp_train_buffer": (vp, [vp, C.c_int]),
+    "cfp_train_window": (C.c_int, [vp]),
+    "cfp_train_minibatch": (C.c_int, [vp]),
+    "cfp_train_record_step": (C.c_int, [vp, C.c_int, vp, vp, vp]),
+    "cfp_train_gae": (C.c_int, [vp]*2),
+    "cfp_train_adv_stats": (C.c_int, [vp]*2),
+    "cfp_train_backward": (C.c_int, [vp, C.c_int, C.c_int, vp]),
+    "cfp_train_zero_loss": (C.c_int, [vp]*2),
+    "cfp_train_adam": (C.c_int, [vp]*2),
+    "cfp_train_loss": (C.c_int, [vp, vp, vp]),
     "cfp_synth_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),
 }
+
+
+class PpoConfig(C.Structure):
+    """cfp_ppo_config of include/cfp.h."""
+    _fields_ = [("lr", C.c_float), ("gamma", C.c_float), ("lam", C.c_float),
+                ("clip", C.c_float), ("ent", C.c_float), ("vf", C.c_float),
+                ("epochs", C.c_int), ("minibatches", C.c_int), ("bptt_split", C.c_int),
+                ("bwd_win", C.c_int)]
+
+
+BUF = {name: i for i, name in enumerate(
+    ["r_obs", "r_state", "r_act", "r_logprob", "r_value", "r_reward", "r_done", "adv",
+     "ret", "v_boot", "stats", "loss_acc", "grads", "adam_m", "adam_v", "lr", "ent"])}
 
 
 class CfpError(RuntimeError):

@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "cfp_common.h"
+#include "cfp_internal.h"
 
 namespace cfp {
 
@@ -37,21 +38,6 @@ __host__ __device__ inline float unit24(uint64_t z) {
 
 }  // namespace cfp
 
-struct cfp_policy {
-    int n = 0;
-    int layers = 0;
-    size_t param_count = 0;
-    float* params = nullptr;
-    float* we_pk = nullptr;
-    float* wg_pk = nullptr;
-    float* wav_pk = nullptr;
-    float* h_state = nullptr;
-    uint8_t* rec = nullptr;
-    float* h_enc = nullptr;
-    float* h3 = nullptr;
-    float* logits = nullptr;
-    hipStream_t stream = nullptr;
-};
 
 using namespace cfp;
 

@@ -1,0 +1,20 @@
+// Library-internal definition of the policy object (opaque in include/cfp.h).
+#pragma once
+
+#include "cfp_common.h"
+
+struct cfp_policy {
+    int n = 0;
+    int layers = 0;
+    size_t param_count = 0;
+    float* params = nullptr;
+    float* we_pk = nullptr;
+    float* wg_pk = nullptr;
+    float* wav_pk = nullptr;
+    float* h_state = nullptr;
+    uint8_t* rec = nullptr;
+    float* h_enc = nullptr;
+    float* h3 = nullptr;
+    float* logits = nullptr;
+    hipStream_t stream = nullptr;
+};

@@ -163,6 +163,76 @@ class Policy:
         return av
 
 
+class Trainer:
+    """cfp_trainer handle (CuTrain, craftax_full.cu:12688): rollout slabs, windowed
+    recompute backward, GAE, Adam."""
+
+    def __init__(self, policy, T, **cfg):
+        self.policy = policy
+        self.cfg = _lib.PpoConfig()
+        _check(lib().cfp_ppo_defaults(C.byref(self.cfg)))
+        for k, v in cfg.items():
+            assert hasattr(self.cfg, k), k
+            setattr(self.cfg, k, v)
+        self._h = C.c_void_p()
+        _check(lib().cfp_train_create(C.byref(self._h), policy._h, T, C.byref(self.cfg)))
+        self.T, self.n, self.layers = T, policy.n, policy.layers
+        self.mb = lib().cfp_train_minibatch(self._h)
+        self.window = lib().cfp_train_window(self._h)
+
+    def close(self):
+        if getattr(self, "_h", None) and self._h.value:
+            lib().cfp_train_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def buf(self, name):
+        T, n, L = self.T, self.n, self.layers
+        shapes = {
+            "r_obs": ((T, n, REC_BYTES), "|u1"), "r_state": ((T, L, n, HIDDEN), "<f4"),
+            "r_act": ((T, n), "<i4"), "r_logprob": ((T, n), "<f4"),
+            "r_value": ((T, n), "<f4"), "r_reward": ((T, n), "<f4"),
+            "r_done": ((T, n), "|u1"), "adv": ((T, n), "<f4"), "ret": ((T, n), "<f4"),
+            "v_boot": ((n,), "<f4"), "stats": ((2,), "<f8"), "loss_acc": ((3,), "<f8"),
+            "grads": ((self.policy.param_count,), "<f4"),
+            "adam_m": ((self.policy.param_count,), "<f4"),
+            "adam_v": ((self.policy.param_count,), "<f4"), "lr": ((1,), "<f4"),
+            "ent": ((1,), "<f4"),
+        }
+        shape, ts = shapes[name]
+        return _wrap(lib().cfp_train_buffer(self._h, _lib.BUF[name]), shape, ts)
+
+    def record_step(self, t, rec, terminals):
+        _check(lib().cfp_train_record_step(self._h, t, _ptr(rec), _ptr(terminals), _stream()))
+
+    def gae(self):
+        _check(lib().cfp_train_gae(self._h, _stream()))
+
+    def adv_stats(self):
+        _check(lib().cfp_train_adv_stats(self._h, _stream()))
+
+    def backward(self, env_start=0, env_count=None):
+        _check(lib().cfp_train_backward(self._h, env_start,
+                                        self.mb if env_count is None else env_count,
+                                        _stream()))
+
+    def zero_loss(self):
+        _check(lib().cfp_train_zero_loss(self._h, _stream()))
+
+    def adam(self):
+        _check(lib().cfp_train_adam(self._h, _stream()))
+
+    def loss(self):
+        out = np.zeros(4)
+        _check(lib().cfp_train_loss(self._h, out.ctypes.data_as(C.c_void_p), _stream()))
+        return out
+
+
 class _DevBuf:
     """Borrowed device memory exposed through __cuda_array_interface__."""
 

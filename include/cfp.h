@@ -191,6 +191,67 @@ int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
                    size_t env_stride, size_t level_stride, uint8_t* d_rec_row,
                    int n, void* stream);
 
+/* ---- PPO update: replaces CuTrain (craftax_full.cu:12688-12761) ----------- */
+typedef struct cfp_trainer cfp_trainer;
+
+/* CuPPOConfig + cu_ppo_defaults (craftax_full.cu:12637-12655).  bwd_win is the
+ * reference's CF_BWD_WIN (steps per recompute window, :12670); 0 = automatic:
+ * the whole horizon up to 262 144 window columns. */
+typedef struct cfp_ppo_config {
+    float lr, gamma, lam, clip, ent, vf;
+    int epochs;
+    int minibatches;   /* contiguous env-range slices per epoch          */
+    int bptt_split;    /* BPTT segments per env in backward (1 = exact)  */
+    int bwd_win;
+} cfp_ppo_config;
+int cfp_ppo_defaults(cfp_ppo_config* cfg);
+
+/* cu_train_init (craftax_full.cu:12763): allocates the rollout slabs
+ * r_obs[T][n][996], r_state[T][layers][n][256], r_act/r_logprob/r_value/
+ * r_reward/adv/ret [T][n], r_done u8 [T][n], the grads arena (params layout),
+ * Adam moments and the window workspace.  Same argument checks as the
+ * reference: minibatches divides n, bptt_split divides T, n/minibatches is a
+ * multiple of 32. */
+int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_config* cfg);
+/* cu_train_free (craftax_full.cu:12929). */
+void cfp_train_destroy(cfp_trainer* tr);
+
+enum cfp_train_buf {
+    CFP_BUF_R_OBS = 0, CFP_BUF_R_STATE, CFP_BUF_R_ACT, CFP_BUF_R_LOGPROB,
+    CFP_BUF_R_VALUE, CFP_BUF_R_REWARD, CFP_BUF_R_DONE, CFP_BUF_ADV, CFP_BUF_RET,
+    CFP_BUF_V_BOOT, CFP_BUF_STATS /* double[2] */, CFP_BUF_LOSS_ACC /* double[3] */,
+    CFP_BUF_GRADS, CFP_BUF_ADAM_M, CFP_BUF_ADAM_V, CFP_BUF_LR /* float */,
+    CFP_BUF_ENT /* float */
+};
+/* Borrowed device pointer to one of the trainer's buffers (NULL if unknown). */
+void* cfp_train_buffer(cfp_trainer* tr, int which);
+int cfp_train_window(const cfp_trainer* tr);
+int cfp_train_minibatch(const cfp_trainer* tr);
+
+/* Policy half of one cu_train_collect step (craftax_full.cu:12987-12995): runs
+ * the fused forward on the policy's live state for step t, storing the record
+ * row into r_obs[t], the post-zero state inputs into r_state[t] and the value
+ * into r_value[t]; logits stay in the policy's logits buffer.  Sampling and the
+ * env step are the caller's. */
+int cfp_train_record_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
+                          const float* d_terminals, void* stream);
+/* k_gae + k_adv_stats of cu_train_collect (craftax_full.cu:13007-13011). */
+int cfp_train_gae(cfp_trainer* tr, void* stream);
+/* k_adv_stats alone (when adv was filled by the caller). */
+int cfp_train_adv_stats(cfp_trainer* tr, void* stream);
+/* cu_train_backward (craftax_full.cu:13168): accumulates the gradients of the
+ * minibatch [env_start, env_start+env_count) into the grads arena and the raw
+ * loss sums (pg, v, ent) into loss_acc. */
+int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stream);
+int cfp_train_zero_loss(cfp_trainer* tr, void* stream);
+/* cu_train_adam (craftax_full.cu:13337): Adam step from the grads arena (which
+ * it zeroes), bumps the step counter, rebuilds the weight mirrors. */
+int cfp_train_adam(cfp_trainer* tr, void* stream);
+/* cu_train_loss (craftax_full.cu:13414): full-batch PPO loss of the stored
+ * rollout with live recurrence inside BPTT segments; host_loss4 = raw sums
+ * (pg, v, ent) and the total (pg + vf*v - ent*H) / (n*T).  Synchronises. */
+int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream);
+
 /* ---- synthetic inputs for parity tests and bench (no reference
  *      counterpart; counter-based so host and device agree bit for bit) ---- */
 /* Records: 792 map bytes, each 0 with prob 0.4 else U{0..40}... see synth.hip;
