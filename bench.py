@@ -32,7 +32,7 @@ LAYERS = 3
 # HBM bytes per launch at 262 144 envs from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/policy_forward_262144_pmc.txt), scaled by the copy-kernel factor
 # stated in DESIGN.md; None until measured for another size.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {262144: 1957465984}
 
 
 def parse():
@@ -44,6 +44,8 @@ def parse():
     ap.add_argument("--ring", type=int, default=16,
                     help="distinct pre-generated record batches cycled through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--schedule", choices=("both", "unchunked", "chunked"), default="both",
+                    help="which launch schedule(s) to time; profiles use one at a time")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MiB",
                     help="only run a plain device copy of this many MiB four times "
                          "(calibrates the FETCH_SIZE / WRITE_SIZE counters) and exit")
@@ -130,7 +132,12 @@ def main():
     torch.cuda.synchronize()
 
     results = {}
-    for name, chunk in (("unchunked", 0), ("chunked_16x16384", 16384 if n > 16384 else 0)):
+    schedules = [("unchunked", 0), ("chunked_16x16384", 16384 if n > 16384 else 0)]
+    if args.schedule == "unchunked":
+        schedules = schedules[:1]
+    elif args.schedule == "chunked":
+        schedules = schedules[1:]
+    for name, chunk in schedules:
         state.zero_()
         for i in range(warmup):
             pol.forward(recs[i % ring], term, state, av=av, chunk=chunk)
@@ -139,9 +146,10 @@ def main():
                          "env_steps_per_s": n * steps / wall}
     assert torch.isfinite(av).all(), "non-finite policy outputs"
 
-    best = results["unchunked"]
-    launch_s = best["device_ms_per_step"] * 1e-3            # one launch per step
-    achieved = FLOP_PER_ENV_STEP * n / launch_s / 1e12
+    best = results.get("unchunked") or results["chunked_16x16384"]
+    launches = 1 if "unchunked" in results else max(1, n // 16384)
+    launch_s = best["device_ms_per_step"] * 1e-3 / launches
+    achieved = FLOP_PER_ENV_STEP * (n // launches) / launch_s / 1e12
     line = {
         "metric": "policy-forward env-steps/sec @262k envs h256x3; % fp32 MFMA peak",
         "value": best["env_steps_per_s"], "unit": "env-steps/s", "n_gpus": 1,
@@ -154,14 +162,15 @@ def main():
                    "envs": n, "layers": LAYERS, "hidden": 256, "chunk": 0,
                    "record_batches_in_hbm": ring},
         "pct_fp32_mfma_peak": 100.0 * achieved / PEAK_FP32_MFMA_TFLOPS,
-        "chunked_16x16384": results["chunked_16x16384"],
+        "chunked_16x16384": results.get("chunked_16x16384"),
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(n),
+                     "traffic": (MEASURED_TRAFFIC_BYTES[n] // launches
+                                 if n in MEASURED_TRAFFIC_BYTES else None),
                      "kernel": "k_policy_forward",
-                     "flops_per_launch": FLOP_PER_ENV_STEP * n,
-                     "algorithmic_hbm_bytes_per_launch": BYTES_PER_ENV_STEP * n,
-                     "launch_ms": best["device_ms_per_step"]},
+                     "flops_per_launch": FLOP_PER_ENV_STEP * n // launches,
+                     "algorithmic_hbm_bytes_per_launch": BYTES_PER_ENV_STEP * n // launches,
+                     "launch_ms": launch_s * 1e3},
     }
     pol.close()
     if not args.no_cpu:
