@@ -19,6 +19,8 @@ PROTOTYPES = {
     "cfp_last_error": (C.c_char_p, []),
     "cfp_abi_version": (C.c_int, []),
     "cfp_policy_create": (C.c_int, [C.POINTER(vp), C.c_int, C.c_int, C.c_uint64]),
+    "cfp_policy_create_classic": (C.c_int, [C.POINTER(vp), C.c_int, C.c_int, C.c_uint64]),
+    "cfp_policy_variant": (C.c_int, [vp]),
     "cfp_policy_destroy": (None, [vp]),
     "cfp_policy_num_envs": (C.c_int, [vp]),
     "cfp_policy_layers": (C.c_int, [vp]),
@@ -62,6 +64,7 @@ PROTOTYPES = {
     "cfp_train_zero_loss": (C.c_int, [vp]*2),
     "cfp_train_adam": (C.c_int, [vp]*2),
     "cfp_train_loss": (C.c_int, [vp, vp, vp]),
+    "cfp_synth_classic_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),
     "cfp_synth_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),
 }
 

@@ -63,22 +63,24 @@ static void policy_release(cfp_policy* p) {
 
 // Xavier-uniform weights, U(+-1/sqrt(fan_in)) biases; segment order is the
 // arena order (craftax_full.cu:11832-11840).
-static void init_params_host(std::vector<float>& w, int layers, uint64_t seed) {
+static void init_params_host(std::vector<float>& w, int layers, int variant,
+                             uint64_t seed) {
     struct Seg { size_t off, count; float bound; };
-    const float xe = sqrtf(6.0f / (float)(CFP_OBS + CFP_HIDDEN));
+    const Arena ar = arena_of(variant, layers);
+    const float xe = sqrtf(6.0f / (float)(ar.obs + CFP_HIDDEN));
     const float xg = sqrtf(6.0f / (float)(CFP_HIDDEN + CFP_GRU));
-    const float xa = sqrtf(6.0f / (float)(CFP_HIDDEN + CFP_ACTIONS));
+    const float xa = sqrtf(6.0f / (float)(CFP_HIDDEN + ar.actions));
     const float xv = sqrtf(6.0f / (float)(CFP_HIDDEN + 1));
-    const float be = 1.0f / sqrtf((float)CFP_OBS);
+    const float be = 1.0f / sqrtf((float)ar.obs);
     const float bh = 1.0f / sqrtf((float)CFP_HIDDEN);
     const Seg segs[7] = {
-        {CFP_OFF_W_ENC, (size_t)CFP_OBS * CFP_HIDDEN, xe},
-        {CFP_OFF_B_ENC, CFP_HIDDEN, be},
-        {CFP_OFF_W_GRU, (size_t)layers * CFP_GRU * CFP_HIDDEN, xg},
-        {(size_t)CFP_OFF_W_A(layers), (size_t)CFP_ACTIONS * CFP_HIDDEN, xa},
-        {(size_t)CFP_OFF_B_A(layers), CFP_ACTIONS, bh},
-        {(size_t)CFP_OFF_W_V(layers), CFP_HIDDEN, xv},
-        {(size_t)CFP_OFF_B_V(layers), 1, bh},
+        {ar.w_enc, (size_t)ar.obs * CFP_HIDDEN, xe},
+        {ar.b_enc, CFP_HIDDEN, be},
+        {ar.w_gru, (size_t)layers * CFP_GRU * CFP_HIDDEN, xg},
+        {ar.w_a, (size_t)ar.actions * CFP_HIDDEN, xa},
+        {ar.b_a, (size_t)ar.actions, bh},
+        {ar.w_v, CFP_HIDDEN, xv},
+        {ar.b_v, 1, bh},
     };
     for (int s = 0; s < 7; s++)
         for (size_t i = 0; i < segs[s].count; i++) {
@@ -87,8 +89,20 @@ static void init_params_host(std::vector<float>& w, int layers, uint64_t seed) {
         }
 }
 
-int cfp_policy_create(cfp_policy** out, int num_envs, int layers,
-                      uint64_t seed) {
+static int policy_create(cfp_policy** out, int num_envs, int layers, uint64_t seed,
+                         int variant);
+
+int cfp_policy_create(cfp_policy** out, int num_envs, int layers, uint64_t seed) {
+    return policy_create(out, num_envs, layers, seed, 0);
+}
+int cfp_policy_create_classic(cfp_policy** out, int num_envs, int layers,
+                              uint64_t seed) {
+    return policy_create(out, num_envs, layers, seed, 1);
+}
+int cfp_policy_variant(const cfp_policy* p) { return p ? p->variant : -1; }
+
+static int policy_create(cfp_policy** out, int num_envs, int layers, uint64_t seed,
+                         int variant) {
     CFP_REQUIRE(out != nullptr, "cfp_policy_create: out is NULL");
     *out = nullptr;
     CFP_REQUIRE(num_envs > 0 && num_envs % 32 == 0,
@@ -99,7 +113,9 @@ int cfp_policy_create(cfp_policy** out, int num_envs, int layers,
     cfp_policy* p = new cfp_policy();
     p->n = num_envs;
     p->layers = layers;
-    p->param_count = (size_t)CFP_PARAM_COUNT(layers);
+    p->variant = variant;
+    p->param_count = arena_of(variant, layers).count;
+    const size_t rec_bytes = variant ? CFP_CLASSIC_REC_BYTES : CFP_REC_BYTES;
     const size_t hn = (size_t)CFP_HIDDEN * num_envs;
 #define CFP_ALLOC(ptr, bytes)                                                 \
     do {                                                                      \
@@ -117,7 +133,7 @@ int cfp_policy_create(cfp_policy** out, int num_envs, int layers,
               ((size_t)layers * kGruPackFloats + 4 * 6 * 64 * 4) * sizeof(float));
     CFP_ALLOC(p->wav_pk, kAvPackFloats * sizeof(float));
     CFP_ALLOC(p->h_state, (size_t)layers * hn * sizeof(float));
-    CFP_ALLOC(p->rec, (size_t)num_envs * CFP_REC_BYTES);
+    CFP_ALLOC(p->rec, (size_t)num_envs * rec_bytes);
     CFP_ALLOC(p->h_enc, hn * sizeof(float));
     CFP_ALLOC(p->h3, hn * sizeof(float));
     CFP_ALLOC(p->logits, (size_t)CFP_AV * num_envs * sizeof(float));
@@ -129,14 +145,14 @@ int cfp_policy_create(cfp_policy** out, int num_envs, int layers,
         return 1;
     }
     e = hipMemset(p->h_state, 0, (size_t)layers * hn * sizeof(float));
-    if (e == hipSuccess) e = hipMemset(p->rec, 0, (size_t)num_envs * CFP_REC_BYTES);
+    if (e == hipSuccess) e = hipMemset(p->rec, 0, (size_t)num_envs * rec_bytes);
     if (e != hipSuccess) {
         set_error("hipMemset failed: %s", hipGetErrorString(e));
         policy_release(p);
         return 1;
     }
     std::vector<float> w(p->param_count);
-    init_params_host(w, layers, seed);
+    init_params_host(w, layers, variant, seed);
     if (cfp_policy_set_params(p, w.data(), w.size()) != 0) {
         policy_release(p);
         return 1;
@@ -179,7 +195,7 @@ int cfp_policy_get_params(const cfp_policy* p, float* host_params,
 
 int cfp_policy_refresh_weights(cfp_policy* p, void* stream) {
     CFP_REQUIRE(p, "cfp_policy_refresh_weights: NULL policy");
-    return launch_pack_weights(p->params, p->layers, p->we_pk, p->wg_pk,
+    return launch_pack_weights(p->params, p->layers, p->variant, p->we_pk, p->wg_pk,
                                p->wav_pk, (hipStream_t)stream);
 }
 
@@ -192,12 +208,16 @@ float* cfp_policy_logits(cfp_policy* p) { return p->logits; }
 void* cfp_policy_stream(cfp_policy* p) { return (void*)p->stream; }
 
 static void fill_weights(const cfp_policy* p, FwdArgs& a) {
+    const Arena ar = arena_of(p->variant, p->layers);
     a.we_pk = reinterpret_cast<const f4*>(p->we_pk);
-    a.b_enc = p->params + CFP_OFF_B_ENC;
+    a.w_enc = p->params + ar.w_enc;
+    a.b_enc = p->params + ar.b_enc;
     a.wg_pk = reinterpret_cast<const f4*>(p->wg_pk);
     a.wav_pk = reinterpret_cast<const f4*>(p->wav_pk);
-    a.b_a = p->params + CFP_OFF_B_A(p->layers);
-    a.b_v = p->params + CFP_OFF_B_V(p->layers);
+    a.b_a = p->params + ar.b_a;
+    a.b_v = p->params + ar.b_v;
+    a.variant = p->variant;
+    a.actions = ar.actions;
 }
 
 // Launch over [0, n) in chunks; every per-env pointer is advanced by the
@@ -212,14 +232,15 @@ static int run_chunked(FwdArgs a, int n, int chunk, hipStream_t st) {
         FwdArgs c = a;
         c.n = n - e0 < chunk ? n - e0 : chunk;
         const size_t off = (size_t)e0;
-        if (a.rec) c.rec = a.rec + off * CFP_REC_BYTES;
+        if (a.rec)
+            c.rec = a.rec + off * (a.variant ? CFP_CLASSIC_REC_BYTES : CFP_REC_BYTES);
         if (a.x0) c.x0 = a.x0 + off * CFP_HIDDEN;
         if (a.state) c.state = a.state + off * CFP_HIDDEN;
         if (a.terminals) c.terminals = a.terminals + off;
         if (a.r_state) c.r_state = a.r_state + off * CFP_HIDDEN;
         if (a.h_enc_out) c.h_enc_out = a.h_enc_out + off * CFP_HIDDEN;
         if (a.h3_out) c.h3_out = a.h3_out + off * CFP_HIDDEN;
-        if (a.av_out) c.av_out = a.av_out + off * CFP_AV;
+        if (a.av_out) c.av_out = a.av_out + off * (a.actions + 1);
         if (launch_forward(c, st) != 0) return 1;
     }
     return 0;
@@ -322,6 +343,40 @@ __global__ void k_synth_records(uint32_t* __restrict__ rec, size_t total_dw,
     rec[i] = w;
 }
 }  // namespace cfp
+
+namespace cfp {
+// One thread per classic record (148 bytes), 8 draws of 64 bits cover the 63
+// mob nibbles; every byte is a pure function of (seed, step, env, position).
+__global__ void k_synth_classic(uint8_t* __restrict__ rec, int n, uint64_t seed,
+                                uint64_t step) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    uint8_t* o = rec + (size_t)e * CFP_CLASSIC_REC_BYTES;
+    for (int c = 0; c < 63; c++) {
+        const uint64_t z = mix64(seed, step, (uint64_t)e * 160 + c);
+        o[c] = (uint8_t)((z & 0xffff) % 17u);
+        const uint32_t r = (uint32_t)(z >> 32);
+        o[63 + c] = (r % 50u) == 0 ? (uint8_t)(1u + ((r >> 8) % 15u)) : 0;   // ~2 % of cells
+    }
+    for (int j = 0; j < 16; j++)
+        o[126 + j] = (uint8_t)((mix64(seed, step, (uint64_t)e * 160 + 64 + j) & 0xffff) % 10u);
+    const uint64_t z = mix64(seed, step, (uint64_t)e * 160 + 80);
+    o[142] = (uint8_t)(1u + (uint32_t)(z & 0xffff) % 4u);
+    o[143] = (uint8_t)((z >> 16) & 1u);
+    const uint32_t lb = __float_as_uint(unit24(mix64(seed, step, (uint64_t)e * 160 + 81)));
+    o[144] = (uint8_t)lb; o[145] = (uint8_t)(lb >> 8);
+    o[146] = (uint8_t)(lb >> 16); o[147] = (uint8_t)(lb >> 24);
+}
+}  // namespace cfp
+
+extern "C" int cfp_synth_classic_records(uint8_t* d_rec, int n, uint64_t seed,
+                                         uint64_t step, void* stream) {
+    CFP_REQUIRE(d_rec && n > 0, "cfp_synth_classic_records: bad argument");
+    hipLaunchKernelGGL(cfp::k_synth_classic, dim3((n + 255) / 256), dim3(256), 0,
+                       (hipStream_t)stream, d_rec, n, seed, step);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
 
 extern "C" int cfp_synth_records(uint8_t* d_rec, int n, uint64_t seed,
                                  uint64_t step, void* stream) {

@@ -71,10 +71,33 @@ struct FwdArgs {
     int n;                   // envs in this launch (multiple of 32)
     int layers;              // MinGRU layers to run (0 = encoder only)
     int do_head;
+    int variant;             // 0 full game (996-byte records), 1 classic (148-byte)
+    int actions;             // 43 or 17; av rows = actions + 1
+    const float* w_enc;      // classic: unpacked W_enc [1345][256] for the gather
 };
 int launch_forward(const FwdArgs& a, hipStream_t st);
 
-int launch_pack_weights(const float* params, int layers, float* we_pk,
+int launch_pack_weights(const float* params, int layers, int variant, float* we_pk,
                         float* wg_pk, float* wav_pk, hipStream_t st);
+
+// per-variant arena geometry
+struct Arena {
+    int obs, actions;
+    size_t w_enc, b_enc, w_gru, w_a, b_a, w_v, b_v, count;
+};
+inline Arena arena_of(int variant, int layers) {
+    Arena a;
+    a.obs = variant ? CFP_CLASSIC_OBS : CFP_OBS;
+    a.actions = variant ? CFP_CLASSIC_ACTIONS : CFP_ACTIONS;
+    a.w_enc = 0;
+    a.b_enc = (size_t)a.obs * CFP_HIDDEN;
+    a.w_gru = a.b_enc + CFP_HIDDEN;
+    a.w_a = a.w_gru + (size_t)layers * CFP_GRU * CFP_HIDDEN;
+    a.b_a = a.w_a + (size_t)a.actions * CFP_HIDDEN;
+    a.w_v = a.b_a + a.actions;
+    a.b_v = a.w_v + CFP_HIDDEN;
+    a.count = a.b_v + 1;
+    return a;
+}
 
 }  // namespace cfp

@@ -6,6 +6,7 @@
 struct cfp_policy {
     int n = 0;
     int layers = 0;
+    int variant = 0;   // 0 full game, 1 classic
     size_t param_count = 0;
     float* params = nullptr;
     float* we_pk = nullptr;

@@ -69,11 +69,56 @@ __device__ __forceinline__ void copy_tile_out(const float* lds, float* dst,
         d4[i] = xs4[(i >> 6) * XS4 + (i & 63)];
 }
 
+// Classic-game encoder (encode_obs_kernel, craftax_classic.cu:1714-1751): the
+// observation is one-hot per view cell, so h0 is b_enc plus a sum of W_enc
+// rows selected by the record bytes, in feature order.  Thread k owns hidden
+// unit k and walks the tile's 32 envs; the record bytes are LDS broadcasts and
+// every W_enc row read is one coalesced 1 KiB line set from L2.
+__device__ __forceinline__ void classic_encode_tile(const FwdArgs& a, uint8_t* crec,
+                                                    float* lds, size_t e0, int tid) {
+    constexpr int CELLS = 63, CH = 21, NBLK = 17;
+    constexpr int TILE_V4 = kTileEnvs * CFP_CLASSIC_REC_BYTES / 16;   // 296
+    const u4* src = reinterpret_cast<const u4*>(a.rec + e0 * CFP_CLASSIC_REC_BYTES);
+    u4* dst = reinterpret_cast<u4*>(crec);
+    for (int i = tid; i < TILE_V4; i += kFwdThreads) dst[i] = src[i];
+    __syncthreads();
+    const float* W = a.w_enc + tid;
+    const float bias = a.b_enc[tid];
+    for (int e = 0; e < kTileEnvs; e++) {
+        const uint8_t* o = crec + e * CFP_CLASSIC_REC_BYTES;
+        float hv = bias;
+        for (int cell = 0; cell < CELLS; cell++) {
+            hv += W[(size_t)(cell * CH + (int8_t)o[cell]) * CFP_HIDDEN];
+            const uint32_t m = o[CELLS + cell];
+            if (m) {
+                const float* wm = W + (size_t)(cell * CH + NBLK) * CFP_HIDDEN;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (m & (1u << j)) hv += wm[(size_t)j * CFP_HIDDEN];
+            }
+        }
+        int f = CELLS * CH;
+#pragma unroll
+        for (int j = 0; j < 16; j++, f++)
+            hv = fmaf((float)(int8_t)o[2 * CELLS + j] / 10.0f, W[(size_t)f * CFP_HIDDEN], hv);
+        const int dir = (int8_t)o[2 * CELLS + 16];
+#pragma unroll
+        for (int d = 1; d <= 4; d++, f++)
+            hv = fmaf(dir == d ? 1.0f : 0.0f, W[(size_t)f * CFP_HIDDEN], hv);
+        const float sleeping = o[2 * CELLS + 17] ? 1.0f : 0.0f;
+        const float light = *reinterpret_cast<const float*>(o + 2 * CELLS + 18);
+        hv = fmaf(light, W[(size_t)f * CFP_HIDDEN], hv); f++;
+        hv = fmaf(sleeping, W[(size_t)f * CFP_HIDDEN], hv);
+        lds[e * XS + tid] = hv;
+    }
+}
+
 }  // namespace
 
 __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     __shared__ float term_s[kTileEnvs];
+    __shared__ __attribute__((aligned(16))) uint8_t crec[kTileEnvs * CFP_CLASSIC_REC_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -85,7 +130,11 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward(FwdArgs a) {
     if (tid < kTileEnvs)
         term_s[tid] = a.terminals ? a.terminals[e0 + tid] : 0.0f;
 
-    if (a.rec) {
+    if (a.rec && a.variant == 1) {
+        classic_encode_tile(a, crec, lds, e0, tid);
+        __syncthreads();
+        if (a.h_enc_out) copy_tile_out(lds, a.h_enc_out + e0 * CFP_HIDDEN, tid);
+    } else if (a.rec) {
         // ---- stage the tile's records: contiguous 16-byte loads, rows
         // re-strided to an odd dword count so that 32 envs reading the same
         // feature hit 32 different LDS banks.
@@ -324,14 +373,14 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward(FwdArgs a) {
         __syncthreads();
         if (kh == 0) {
             const int arow = nt * 32 + l32;
-            if (arow < CFP_AV) {
-                const float bias =
-                    arow < CFP_ACTIONS ? a.b_a[arow] : a.b_v[0];
-                float* av_base = a.av_out + e0 * CFP_AV;
-                const int aoff = (4 * half) * CFP_AV + arow;
+            const int avs = a.actions + 1;     // 44, or 18 for the classic game
+            if (arow < avs) {
+                const float bias = arow < a.actions ? a.b_a[arow] : a.b_v[0];
+                float* av_base = a.av_out + e0 * avs;
+                const int aoff = (4 * half) * avs + arow;
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    (av_base + acc_row(r) * CFP_AV)[aoff] =
+                    (av_base + acc_row(r) * avs)[aoff] =
                         acc[r] + red[r * 64] + bias;
             }
         }
@@ -350,6 +399,9 @@ int launch_forward(const FwdArgs& a, hipStream_t st) {
     CFP_REQUIRE(a.x0 == nullptr ||
                     (reinterpret_cast<uintptr_t>(a.x0) & 15u) == 0,
                 "layer-0 input must be 16-byte aligned");
+    CFP_REQUIRE(a.variant == 0 || a.rec == nullptr || a.w_enc != nullptr,
+                "classic forward needs the unpacked W_enc");
+    CFP_REQUIRE(a.actions > 0 && a.actions < kAvPad, "bad action count %d", a.actions);
     CFP_REQUIRE(a.layers >= 0 && a.layers <= CFP_MAX_LAYERS,
                 "layers must be in 0..%d", CFP_MAX_LAYERS);
     CFP_REQUIRE(a.layers == 0 || a.state != nullptr,
@@ -394,29 +446,32 @@ __global__ void k_pack_gru(const float* __restrict__ W_gru,
 
 __global__ void k_pack_av(const float* __restrict__ W_a,
                           const float* __restrict__ W_v,
-                          float* __restrict__ out) {
+                          float* __restrict__ out, int actions) {
     int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int)kAvPackFloats) return;
     int j = idx & 3, lane = (idx >> 2) & 63, nt = (idx >> 8) & 1, kb = idx >> 9;
     int arow = nt * 32 + (lane & 31);
     int k = kKBlock * kb + 4 * (lane >> 5) + j;
     float v = 0.0f;
-    if (arow < CFP_ACTIONS) v = W_a[arow * CFP_HIDDEN + k];
-    else if (arow == CFP_ACTIONS) v = W_v[k];
+    if (arow < actions) v = W_a[arow * CFP_HIDDEN + k];
+    else if (arow == actions) v = W_v[k];
     out[idx] = v;
 }
 
-int launch_pack_weights(const float* params, int layers, float* we_pk,
+int launch_pack_weights(const float* params, int layers, int variant, float* we_pk,
                         float* wg_pk, float* wav_pk, hipStream_t st) {
-    const int enc_total = (kKbEnc + 2) * 2048;
-    hipLaunchKernelGGL(k_pack_enc, dim3((enc_total + 255) / 256), dim3(256), 0,
-                       st, params + CFP_OFF_W_ENC, we_pk, enc_total);
+    const Arena ar = arena_of(variant, layers);
+    if (variant == 0) {   // the classic encoder gathers from the unpacked W_enc
+        const int enc_total = (kKbEnc + 2) * 2048;
+        hipLaunchKernelGGL(k_pack_enc, dim3((enc_total + 255) / 256), dim3(256), 0,
+                           st, params + ar.w_enc, we_pk, enc_total);
+    }
     const int gru_total = layers * (int)kGruPackFloats + 4 * 6 * 64 * 4;
     hipLaunchKernelGGL(k_pack_gru, dim3((gru_total + 255) / 256), dim3(256), 0,
-                       st, params + CFP_OFF_W_GRU, wg_pk, layers, gru_total);
+                       st, params + ar.w_gru, wg_pk, layers, gru_total);
     hipLaunchKernelGGL(k_pack_av, dim3(((int)kAvPackFloats + 255) / 256),
-                       dim3(256), 0, st, params + CFP_OFF_W_A(layers),
-                       params + CFP_OFF_W_V(layers), wav_pk);
+                       dim3(256), 0, st, params + ar.w_a, params + ar.w_v, wav_pk,
+                       ar.actions);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }

@@ -397,6 +397,7 @@ int cfp_ppo_defaults(cfp_ppo_config* cfg) {
 int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_config* cfg) {
     CFP_REQUIRE(out && p && cfg, "cfp_train_create: NULL argument");
     *out = nullptr;
+    CFP_REQUIRE(p->variant == 0, "the trainer covers the full-game policy only");
     CFP_REQUIRE(T > 0, "horizon must be positive (got %d)", T);
     CFP_REQUIRE(cfg->minibatches >= 1 && p->n % cfg->minibatches == 0,
                 "minibatches must divide num_envs (%d %% %d != 0)", p->n,

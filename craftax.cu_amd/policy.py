@@ -14,6 +14,7 @@ from . import _lib
 
 HIDDEN, GRU, OBS, OBS_MAP, OBS_TAIL = 256, 768, 843, 792, 51
 REC_BYTES, ACTIONS, AV = 996, 43, 44
+CLASSIC_OBS, CLASSIC_REC_BYTES, CLASSIC_ACTIONS, CLASSIC_AV = 1345, 148, 17, 18
 
 _cfp = None
 
@@ -70,11 +71,18 @@ def split_params(params, layers):
 class Policy:
     """cfp_policy handle (CuPolicy, craftax_full.cu:11758)."""
 
-    def __init__(self, num_envs, layers=3, seed=1):
+    def __init__(self, num_envs, layers=3, seed=1, variant="full"):
+        """variant "full": 996-byte records, 43 actions; "classic": 148-byte records,
+        17 actions, gathered-column encoder (Rollout, main_classic.cu:326)."""
         self._h = C.c_void_p()
-        _check(lib().cfp_policy_create(C.byref(self._h), num_envs, layers, seed))
+        assert variant in ("full", "classic")
+        create = lib().cfp_policy_create if variant == "full" else lib().cfp_policy_create_classic
+        _check(create(C.byref(self._h), num_envs, layers, seed))
         self.n = num_envs
         self.layers = layers
+        self.variant = variant
+        self.rec_bytes = REC_BYTES if variant == "full" else CLASSIC_REC_BYTES
+        self.av_width = AV if variant == "full" else CLASSIC_AV
         self.param_count = lib().cfp_policy_param_count(self._h)
 
     def close(self):
@@ -122,7 +130,7 @@ class Policy:
 
     @property
     def rec(self):
-        return _wrap(lib().cfp_policy_rec(self._h), (self.n, REC_BYTES), "|u1")
+        return _wrap(lib().cfp_policy_rec(self._h), (self.n, self.rec_bytes), "|u1")
 
     @property
     def h_enc(self):
@@ -134,7 +142,7 @@ class Policy:
 
     @property
     def logits(self):
-        return _wrap(lib().cfp_policy_logits(self._h), (self.n, AV), "<f4")
+        return _wrap(lib().cfp_policy_logits(self._h), (self.n, self.av_width), "<f4")
 
     def gru_chain(self, x0, state, terminals, r_state_t=None, h3=None, chunk=0):
         n = x0.shape[0]
@@ -147,7 +155,7 @@ class Policy:
     def head(self, h3, av=None):
         n = h3.shape[0]
         if av is None:
-            av = torch.empty((n, AV), dtype=torch.float32, device=h3.device)
+            av = torch.empty((n, self.av_width), dtype=torch.float32, device=h3.device)
         _check(lib().cfp_head(self._h, _ptr(h3), _ptr(av), n, _stream()))
         return av
 
@@ -156,7 +164,7 @@ class Policy:
         """Policy half of rollout_step: records -> logits/value, state updated in place."""
         n = rec.shape[0]
         if av is None:
-            av = torch.empty((n, AV), dtype=torch.float32, device=rec.device)
+            av = torch.empty((n, self.av_width), dtype=torch.float32, device=rec.device)
         _check(lib().cfp_policy_forward(self._h, _ptr(rec), _ptr(terminals), _ptr(state),
                                         _ptr(r_state_t), _ptr(h_enc), _ptr(h3),
                                         _ptr(av), n, chunk, _stream()))
@@ -323,6 +331,13 @@ def record_obs(scalars_u8, maps, item_maps, light_maps, n, env_stride, level_str
     _check(lib().cfp_record_obs(_ptr(scalars_u8), _ptr(maps), _ptr(item_maps),
                                 _ptr(light_maps), env_stride, level_stride, _ptr(rec),
                                 n, _stream()))
+    return rec
+
+
+def synth_classic_records(n, seed, step, rec=None, device="cuda"):
+    if rec is None:
+        rec = torch.empty((n, CLASSIC_REC_BYTES), dtype=torch.uint8, device=device)
+    _check(lib().cfp_synth_classic_records(_ptr(rec), n, seed, step, _stream()))
     return rec
 
 

@@ -51,6 +51,17 @@ extern "C" {
 #define CFP_OFF_B_V(layers) (CFP_OFF_W_V(layers) + CFP_HIDDEN)
 #define CFP_PARAM_COUNT(layers) (CFP_OFF_B_V(layers) + 1)
 
+/* Classic-game policy (craftax_classic.cu:38-59, 1522-1533): 1345-dim one-hot
+ * observation carried as a 148-byte record, actor 17 / value 1, same MinGRU stack.
+ * Its params arena has the same segment order with 1345 / 17 in place of 843 / 43. */
+#define CFP_CLASSIC_OBS 1345
+#define CFP_CLASSIC_REC_BYTES 148
+#define CFP_CLASSIC_ACTIONS 17
+#define CFP_CLASSIC_AV (CFP_CLASSIC_ACTIONS + 1)
+#define CFP_CLASSIC_PARAM_COUNT(layers)                                           \
+    (CFP_CLASSIC_OBS * CFP_HIDDEN + CFP_HIDDEN + (layers) * CFP_GRU * CFP_HIDDEN + \
+     CFP_CLASSIC_ACTIONS * CFP_HIDDEN + CFP_CLASSIC_ACTIONS + CFP_HIDDEN + 1)
+
 const char* cfp_last_error(void);
 /* Library/ABI version, bumped when a signature changes. */
 int cfp_abi_version(void);
@@ -65,6 +76,15 @@ typedef struct cfp_policy cfp_policy;
  * U(+-1/sqrt(fan_in)) from cuRAND Philox, which is not reproducible off CUDA)
  * and builds the MFMA-ordered weight mirrors.  layers in 1..3. */
 int cfp_policy_create(cfp_policy** out, int num_envs, int layers, uint64_t seed);
+/* Classic-game variant: the Rollout object of main_classic.cu:326.  Every
+ * forward entry point below then takes 148-byte records (layout
+ * craftax_classic.cu:50-59: 63 block ids, 63 mob bitmasks, 12 inventory, 4
+ * intrinsics, direction, sleeping, light fp32) and writes av[n][18]
+ * (17 logits + value); the encoder is the gathered-column sum of
+ * encode_obs_kernel (craftax_classic.cu:1714-1751) instead of a GEMM. */
+int cfp_policy_create_classic(cfp_policy** out, int num_envs, int layers, uint64_t seed);
+/* 0 = full game (843 features, 43 actions), 1 = classic. */
+int cfp_policy_variant(const cfp_policy* p);
 /* cu_policy_free (craftax_full.cu:11907). */
 void cfp_policy_destroy(cfp_policy* p);
 
@@ -258,6 +278,11 @@ int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream);
  * tail floats U[0,1) with 24-bit mantissas.  index = env + n*step. */
 int cfp_synth_records(uint8_t* d_rec, int n, uint64_t seed, uint64_t step,
                       void* stream);
+
+/* Classic records: block ids U{0..16}, mob bitmask nonzero for ~2 % of cells,
+ * 16 scalars U{0..9}, direction U{1..4}, sleeping Bernoulli(1/2), light U[0,1). */
+int cfp_synth_classic_records(uint8_t* d_rec, int n, uint64_t seed, uint64_t step,
+                              void* stream);
 
 #ifdef __cplusplus
 }

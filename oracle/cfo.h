@@ -56,6 +56,17 @@ void cfo_forward_f64(const float* params, int layers, int n,
                      double* state_out, double* h3 /*[n][256]*/,
                      double* logits /*[n][43]*/, double* values /*[n]*/);
 
+/* Classic-game policy (config 5): record expansion of encode_obs_kernel
+ * (craftax_classic.cu:1714-1751) and the same forward with 1345 features /
+ * 17 actions; logits [n][17].  Pinned like cfo_forward_f64 (numpy fp64
+ * cross-check, one-hot closed form). */
+void cfo_classic_expand(const uint8_t* rec /*[148]*/, float* x /*[1345]*/);
+void cfo_classic_forward_f64(const float* params, int layers, int n,
+                             const float* x /*[n][1345]*/, const double* state_in,
+                             const float* prev_terminals, double* h_enc,
+                             double* r_state, double* state_out, double* h3,
+                             double* logits /*[n][17]*/, double* values);
+
 /* Scalar fp32 forward following k_policy_ref_l3 literally (fmaf chains in
  * ascending feature order, exact-zero features skipped), from records, state
  * updated in place; OpenMP over envs with `threads` threads (<=0: default).

@@ -16,7 +16,7 @@
 
 #include "cfo.h"
 
-enum { H = CFP_HIDDEN, G = CFP_GRU, F = CFP_OBS, FM = CFP_OBS_MAP, A = CFP_ACTIONS };
+enum { H = CFP_HIDDEN, G = CFP_GRU, FM = CFP_OBS_MAP };
 
 int cfo_max_threads(void) {
 #ifdef _OPENMP
@@ -29,17 +29,21 @@ int cfo_max_threads(void) {
 static double sigmoid64(double x) { return 1.0 / (1.0 + exp(-x)); }
 static double mingru_g64(double x) { return x >= 0.0 ? x + 0.5 : sigmoid64(x); }
 
-void cfo_forward_f64(const float* params, int layers, int n, const float* x,
-                     const double* state_in, const float* prev_terminals,
-                     double* h_enc, double* r_state, double* state_out,
-                     double* h3, double* logits, double* values) {
-    const float* W_enc = params + CFP_OFF_W_ENC;
-    const float* b_enc = params + CFP_OFF_B_ENC;
-    const float* W_gru = params + CFP_OFF_W_GRU;
-    const float* W_a = params + CFP_OFF_W_A(layers);
-    const float* b_a = params + CFP_OFF_B_A(layers);
-    const float* W_v = params + CFP_OFF_W_V(layers);
-    const float* b_v = params + CFP_OFF_B_V(layers);
+/* Shared by the full-game (F = 843, A = 43) and classic-game (F = 1345, A = 17)
+ * policies: the arena has the same segment order for both
+ * (craftax_full.cu:9094-9102, craftax_classic.cu:1526-1533). */
+static void forward_f64_impl(const float* params, int layers, int n, int F, int A,
+                             const float* x, const double* state_in,
+                             const float* prev_terminals, double* h_enc,
+                             double* r_state, double* state_out, double* h3,
+                             double* logits, double* values) {
+    const float* W_enc = params;
+    const float* b_enc = W_enc + (size_t)F * H;
+    const float* W_gru = b_enc + H;
+    const float* W_a = W_gru + (size_t)layers * G * H;
+    const float* b_a = W_a + (size_t)A * H;
+    const float* W_v = b_a + A;
+    const float* b_v = W_v + H;
     const size_t hn = (size_t)H * n;
 
 #pragma omp parallel for schedule(static)
@@ -92,12 +96,51 @@ void cfo_forward_f64(const float* params, int layers, int n, const float* x,
     }
 }
 
+void cfo_forward_f64(const float* params, int layers, int n, const float* x,
+                     const double* state_in, const float* prev_terminals,
+                     double* h_enc, double* r_state, double* state_out,
+                     double* h3, double* logits, double* values) {
+    forward_f64_impl(params, layers, n, CFP_OBS, CFP_ACTIONS, x, state_in, prev_terminals,
+                     h_enc, r_state, state_out, h3, logits, values);
+}
+
+/* Classic game.  Record -> 1345 features as encode_obs_kernel reads them
+ * (craftax_classic.cu:1714-1751; layout :50-59): per view cell a block one-hot
+ * (21 channels: 17 block types + 4 mob bits), 12 inventory + 4 intrinsics as
+ * (float)v / 10, direction one-hot, light, sleeping. */
+void cfo_classic_expand(const uint8_t* rec, float* x) {
+    memset(x, 0, sizeof(float) * CFP_CLASSIC_OBS);
+    for (int cell = 0; cell < 63; cell++) {
+        x[cell * 21 + (int8_t)rec[cell]] = 1.0f;
+        const uint8_t m = rec[63 + cell];
+        for (int j = 0; j < 4; j++)
+            if (m & (1 << j)) x[cell * 21 + 17 + j] = 1.0f;
+    }
+    int f = 63 * 21;
+    for (int j = 0; j < 16; j++) x[f++] = (float)(int8_t)rec[126 + j] / 10.0f;
+    const int dir = (int8_t)rec[142];
+    for (int d = 1; d <= 4; d++) x[f++] = dir == d ? 1.0f : 0.0f;
+    float light;
+    memcpy(&light, rec + 144, sizeof(float));
+    x[f++] = light;
+    x[f++] = rec[143] ? 1.0f : 0.0f;
+}
+
+void cfo_classic_forward_f64(const float* params, int layers, int n, const float* x,
+                             const double* state_in, const float* prev_terminals,
+                             double* h_enc, double* r_state, double* state_out,
+                             double* h3, double* logits, double* values) {
+    forward_f64_impl(params, layers, n, CFP_CLASSIC_OBS, CFP_CLASSIC_ACTIONS, x, state_in,
+                     prev_terminals, h_enc, r_state, state_out, h3, logits, values);
+}
+
 static float sigmoid32(float x) { return 1.0f / (1.0f + expf(-x)); }
 static float mingru_g32(float x) { return x >= 0.0f ? x + 0.5f : sigmoid32(x); }
 
 void cfo_forward_f32(const float* params, int layers, int n, const uint8_t* rec,
                      float* state, const float* prev_terminals, float* av,
                      int threads) {
+    enum { F = CFP_OBS, A = CFP_ACTIONS };
     const float* W_enc = params + CFP_OFF_W_ENC;
     const float* b_enc = params + CFP_OFF_B_ENC;
     const float* W_gru = params + CFP_OFF_W_GRU;

@@ -71,6 +71,8 @@ def cfo():
                                                  C.c_size_t, vp]
         lib.cfo_expand_record.argtypes = [vp, vp]
         lib.cfo_forward_f64.argtypes = [vp, C.c_int, C.c_int] + [vp] * 9
+        lib.cfo_classic_expand.argtypes = [vp, vp]
+        lib.cfo_classic_forward_f64.argtypes = [vp, C.c_int, C.c_int] + [vp] * 9
         lib.cfo_forward_f32.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int]
         lib.cfo_max_threads.restype = C.c_int
         lib.cfo_ppo_loss_f64.restype = C.c_double
@@ -150,6 +152,32 @@ def forward_f64(params, layers, x, state, terminals):
     cfo().cfo_forward_f64(_p(params), layers, n, _p(x), _p(st_in), _p(term),
                           _p(out["h_enc"]), _p(out["r_state"]), _p(out["state"]),
                           _p(out["h3"]), _p(out["logits"]), _p(out["values"]))
+    return out
+
+
+def classic_expand(rec):
+    rec = np.ascontiguousarray(rec, dtype=np.uint8).reshape(-1, 148)
+    x = np.empty((rec.shape[0], 1345), dtype=np.float32)
+    for i in range(rec.shape[0]):
+        cfo().cfo_classic_expand(_p(rec[i]), _p(x[i]))
+    return x
+
+
+def classic_forward_f64(params, layers, x, state, terminals):
+    """fp64 oracle forward of the classic-game policy; x [n][1345]."""
+    params = np.ascontiguousarray(params, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    n = x.shape[0]
+    st_in = np.ascontiguousarray(state, dtype=np.float64)
+    term = None if terminals is None else np.ascontiguousarray(terminals, dtype=np.float32)
+    out = {
+        "h_enc": np.empty((n, HIDDEN)), "r_state": np.empty((layers, n, HIDDEN)),
+        "state": np.empty((layers, n, HIDDEN)), "h3": np.empty((n, HIDDEN)),
+        "logits": np.empty((n, 17)), "values": np.empty(n),
+    }
+    cfo().cfo_classic_forward_f64(_p(params), layers, n, _p(x), _p(st_in), _p(term),
+                                  _p(out["h_enc"]), _p(out["r_state"]), _p(out["state"]),
+                                  _p(out["h3"]), _p(out["logits"]), _p(out["values"]))
     return out
 
 

@@ -46,6 +46,26 @@ def synth_records_host(n, seed, step):
     return out.view(np.uint8).reshape(n, REC_BYTES)
 
 
+def synth_classic_records_host(n, seed, step):
+    """Bit-identical host twin of cfp_synth_classic_records: [n][148] uint8."""
+    e = np.arange(n, dtype=np.uint64)[:, None] * np.uint64(160)
+    out = np.zeros((n, 148), dtype=np.uint8)
+    z = mix64(seed, step, e + np.arange(63, dtype=np.uint64)[None, :])
+    out[:, :63] = ((z & np.uint64(0xffff)) % np.uint64(17)).astype(np.uint8)
+    r = (z >> np.uint64(32)).astype(np.uint64)
+    mob = np.where(r % np.uint64(50) == 0, np.uint64(1) + ((r >> np.uint64(8)) % np.uint64(15)),
+                   np.uint64(0))
+    out[:, 63:126] = mob.astype(np.uint8)
+    z = mix64(seed, step, e + np.uint64(64) + np.arange(16, dtype=np.uint64)[None, :])
+    out[:, 126:142] = ((z & np.uint64(0xffff)) % np.uint64(10)).astype(np.uint8)
+    z = mix64(seed, step, e[:, 0] + np.uint64(80))
+    out[:, 142] = (np.uint64(1) + (z & np.uint64(0xffff)) % np.uint64(4)).astype(np.uint8)
+    out[:, 143] = ((z >> np.uint64(16)) & np.uint64(1)).astype(np.uint8)
+    light = unit24(mix64(seed, step, e[:, 0] + np.uint64(81)))
+    out[:, 144:148] = light.view(np.uint8).reshape(n, 4)
+    return out
+
+
 def expand_records(rec):
     """k_expand_obs semantics (craftax_full.cu:10028): bytes -> fp32 features."""
     rec = np.ascontiguousarray(rec).reshape(-1, REC_BYTES)
@@ -55,29 +75,31 @@ def expand_records(rec):
     return x
 
 
-def random_params(layers, seed, scale=1.0):
+def random_params(layers, seed, scale=1.0, obs=None, actions=None):
     """Xavier-uniform-ish random weights in the flat arena layout."""
+    OBS_, ACTIONS_ = (obs or OBS), (actions or ACTIONS)
     rng = np.random.default_rng(seed)
     def u(shape, bound):
         return rng.uniform(-bound, bound, size=shape).astype(np.float32)
     parts = [
-        u((OBS * HIDDEN,), scale * np.sqrt(6.0 / (OBS + HIDDEN))),
-        u((HIDDEN,), 1.0 / np.sqrt(OBS)),
+        u((OBS_ * HIDDEN,), scale * np.sqrt(6.0 / (OBS_ + HIDDEN))),
+        u((HIDDEN,), 1.0 / np.sqrt(OBS_)),
         u((layers * GRU * HIDDEN,), scale * np.sqrt(6.0 / (HIDDEN + GRU))),
-        u((ACTIONS * HIDDEN,), scale * np.sqrt(6.0 / (HIDDEN + ACTIONS))),
-        u((ACTIONS,), 1.0 / np.sqrt(HIDDEN)),
+        u((ACTIONS_ * HIDDEN,), scale * np.sqrt(6.0 / (HIDDEN + ACTIONS_))),
+        u((ACTIONS_,), 1.0 / np.sqrt(HIDDEN)),
         u((HIDDEN,), scale * np.sqrt(6.0 / (HIDDEN + 1))),
         u((1,), 1.0 / np.sqrt(HIDDEN)),
     ]
     return np.concatenate(parts)
 
 
-def split_params(params, layers):
+def split_params(params, layers, obs=None, actions=None):
+    OBS_, ACTIONS_ = (obs or OBS), (actions or ACTIONS)
     o = {}
     off = 0
-    for name, shape in (("W_enc", (OBS, HIDDEN)), ("b_enc", (HIDDEN,)),
-                        ("W_gru", (layers, GRU, HIDDEN)), ("W_a", (ACTIONS, HIDDEN)),
-                        ("b_a", (ACTIONS,)), ("W_v", (HIDDEN,)), ("b_v", (1,))):
+    for name, shape in (("W_enc", (OBS_, HIDDEN)), ("b_enc", (HIDDEN,)),
+                        ("W_gru", (layers, GRU, HIDDEN)), ("W_a", (ACTIONS_, HIDDEN)),
+                        ("b_a", (ACTIONS_,)), ("W_v", (HIDDEN,)), ("b_v", (1,))):
         cnt = int(np.prod(shape))
         o[name] = np.asarray(params[off:off + cnt]).reshape(shape)
         off += cnt
@@ -89,11 +111,12 @@ def sigmoid64(z):
     return 1.0 / (1.0 + np.exp(-z))
 
 
-def numpy_forward_f64(params, layers, x, state, terminals):
+def numpy_forward_f64(params, layers, x, state, terminals, obs=None, actions=None):
     """Independent fp64 evaluation with library matmuls (A.2 of the forward spec:
     craftax_full.cu:9778-9854).  x [n][843], state [L][n][256] -> dict of fp64
     arrays; state is not modified."""
-    w = {k: v.astype(np.float64) for k, v in split_params(params, layers).items()}
+    w = {k: v.astype(np.float64)
+         for k, v in split_params(params, layers, obs, actions).items()}
     h = x.astype(np.float64) @ w["W_enc"] + w["b_enc"]
     out = {"h_enc": h.copy()}
     new_state = np.empty((layers,) + h.shape, dtype=np.float64)

@@ -250,3 +250,38 @@ def test_gae_and_adam_closed_forms():
     ob.cfo().cfo_adam_f64(p.ctypes.data, g.ctypes.data, m.ctypes.data, v.ctypes.data, 3, 1,
                           3e-4, 0.9, 0.999, 1e-8)
     assert np.allclose(p, [1.0 - 3e-4, -2.0 + 3e-4, 3.0], atol=1e-9)
+
+
+# ---- classic-game policy (config 5) ---------------------------------------------------
+def test_classic_expand_and_forward_oracle():
+    from parity_util import synth_classic_records_host
+    n = 24
+    rec = synth_classic_records_host(n, 3, 1)
+    assert rec[:, :63].max() <= 16 and rec[:, 126:142].max() <= 9
+    assert set(np.unique(rec[:, 142])) <= {1, 2, 3, 4} and (rec[:, 63:126] != 0).any()
+    x = ob.classic_expand(rec)
+    # one-hot closed form: every cell has exactly one block channel set
+    cells = x[:, :63 * 21].reshape(n, 63, 21)
+    assert np.array_equal(cells[:, :, :17].sum(axis=2), np.ones((n, 63), np.float32))
+    assert np.array_equal(cells[:, :, :17].argmax(axis=2), rec[:, :63])
+    bits = (rec[:, 63:126, None] >> np.arange(4)) & 1
+    assert np.array_equal(cells[:, :, 17:], bits.astype(np.float32))
+    assert np.array_equal(x[:, 1323:1339], rec[:, 126:142].astype(np.float32) / np.float32(10.0))
+    assert np.array_equal(x[:, 1339:1343].argmax(axis=1) + 1, rec[:, 142])
+    assert np.array_equal(x[:, 1343].view(np.uint32), np.ascontiguousarray(rec[:, 144:148]).view(np.uint32)[:, 0])
+    assert np.array_equal(x[:, 1344], rec[:, 143].astype(np.float32))
+    params = random_params(L, 61, obs=1345, actions=17)
+    rng = np.random.default_rng(62)
+    state = (0.5 * rng.standard_normal((L, n, HIDDEN))).astype(np.float32)
+    term = (rng.random(n) < 0.3).astype(np.float32)
+    a = ob.classic_forward_f64(params, L, x, state, term)
+    b = numpy_forward_f64(params, L, x, state, term, obs=1345, actions=17)
+    for k in ("h_enc", "state", "h3", "logits", "values"):
+        assert rel_err(a[k], b[k]) < 1e-12, k
+    # gathered-column form of the encoder == dense form
+    sp = split_params(params, L, 1345, 17)
+    e = 5
+    h = sp["b_enc"].astype(np.float64).copy()
+    for f in np.nonzero(x[e])[0]:
+        h += float(x[e, f]) * sp["W_enc"][f].astype(np.float64)
+    assert np.allclose(h, a["h_enc"][e], rtol=1e-13, atol=1e-13)
