@@ -128,7 +128,7 @@ static int policy_create(cfp_policy** out, int num_envs, int layers, uint64_t se
         }                                                                     \
     } while (0)
     CFP_ALLOC(p->params, p->param_count * sizeof(float));
-    CFP_ALLOC(p->we_pk, (size_t)(kKbEnc + 2) * 2048 * sizeof(float));
+    CFP_ALLOC(p->we_pk, (size_t)(kKbEnc + kEncPadBlocks) * 2048 * sizeof(float));
     CFP_ALLOC(p->wg_pk,
               ((size_t)layers * kGruPackFloats + 4 * 6 * 64 * 4) * sizeof(float));
     CFP_ALLOC(p->wav_pk, kAvPackFloats * sizeof(float));

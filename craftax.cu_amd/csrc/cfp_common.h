@@ -25,6 +25,7 @@ constexpr int kKbEnc = kObsPad / kKBlock;          // 106
 constexpr int kKbMap = CFP_OBS_MAP / kKBlock;      // 99: map bytes end on a block edge
 constexpr int kKbHid = CFP_HIDDEN / kKBlock;       // 32
 constexpr int kAvPad = 64;                         // head rows padded 44 -> 64
+constexpr int kEncPadBlocks = 4;                   // encoder mirror: prefetch overrun
 
 // MFMA-ordered weight mirror sizes, in floats.
 constexpr size_t kEncPackFloats = (size_t)kObsPad * CFP_HIDDEN;

@@ -1,5 +1,5 @@
 // Fused policy forward for gfx950: 996-byte records -> Linear(843->256)
-// -> MinGRU x L -> actor(43)/value(1), one workgroup per tile of 32 envs.
+// -> MinGRU x L -> actor(43)/value(1), tiles of 32 envs.
 //
 // Replaces, in one launch, the reference's per-step chain
 //   k_expand_obs + cublasSgemm + k_add_bias       (craftax_full.cu:11954-11962)
@@ -9,22 +9,34 @@
 // pre-activations ever exist in HBM: the activations of a tile stay in LDS
 // from the record bytes to the logits.
 //
-// Data flow of one workgroup (256 threads = 4 waves, wave w owns hidden units
-// [64w, 64w+64)):
-//   records (31 872 contiguous bytes) -> LDS, rows re-strided to 255 dwords
-//   encoder: C[env][unit] += x[env][f] * W_enc[f][unit] on 32x32x2 fp32 MFMA,
-//            x taken from the LDS bytes (v_cvt_f32_ubyteN) / tail floats,
-//            W_enc fragments streamed from the MFMA-ordered mirror in L2
-//   h = C + b_enc -> LDS x tile [32][260] fp32 (aliases the record bytes)
-//   per layer: 6 accumulators (zh, zg, zp for 2 unit tiles) over K = 256,
-//            gate/blend epilogue in registers, state streamed from/to HBM
-//            with non-temporal accesses, h' written back into the x tile
-//   heads:   2 row tiles x 2 K halves over the 4 waves, reduced through LDS.
+// Schedule.  One persistent workgroup (4 waves, one per SIMD, up to 512
+// registers each) per CU walks PAIRS of 32-env tiles X, Y.  The gate/blend
+// epilogue of one tile is woven, element by element, between the MFMAs of the
+// other tile's next gate GEMM, so no wave ever sits in a pure vector phase:
+//   ENC(X+Y) | bias | K(X,0) | K(Y,0)+epi(X,0) | K(X,1)+epi(Y,0) | ...
+//   ... | K(Y,L-1)+epi(X,L-1) | epi(Y,L-1) | HEAD(X) HEAD(Y) | reduce, store
+// ("|" = workgroup barrier).  `sched_group_barrier` pins the issue order inside
+// a K block (1 MFMA : 2 VALU, one weight load per four MFMAs).  Measured on
+// MI355X, every non-MFMA instruction of the issuing wave costs the matrix pipe
+// about its own issue time (a 16-byte global load ~40 cycles, wherever it
+// hits), so the design minimises instructions per MFMA rather than latency:
+// 6 weight loads + 1 LDS read + ~35 epilogue instructions per 24 MFMAs.
 //
-// MFMA operand convention (v_mfma_f32_32x32x2_f32): A = activations
-// (row = env), B = weights (column = unit), so accumulator register r of lane
-// l holds env 8*(r/4) + 4*(l/32) + r%4, unit l%32: a half-wave touches 32
-// consecutive units of one env, i.e. one full 128-byte line of state.
+// Within the workgroup, wave w owns hidden units [64w, 64w+64).  MFMA operand
+// convention (v_mfma_f32_32x32x2_f32): A = activations (row = env), B = weights
+// (column = unit), so accumulator register r of lane l holds env
+// 8*(r/4) + 4*(l/32) + r%4, unit l%32: a half-wave touches 32 consecutive units
+// of one env, i.e. one full 128-byte line of state.
+//   encoder: x from the LDS record bytes (v_cvt_f32_ubyteN) / tail floats,
+//            W_enc fragments streamed once per pair from the MFMA-ordered
+//            mirror in L2 and used for both tiles (4 accumulators), two K
+//            blocks per step, weights three steps deep in registers
+//   layer:   6 accumulators (zh, zg, zp for 2 unit tiles) over K = 256, weights
+//            three K blocks deep; the first two blocks and the 32 state values
+//            of the NEXT phase are requested before the barrier that ends the
+//            current one; state and r_state leave through non-temporal stores
+//            next to each epilogue element; h' goes back into the x tile
+//   heads:   2 row tiles x 2 K halves over the 4 waves, reduced through LDS.
 #include "cfp_common.h"
 
 namespace cfp {
@@ -37,6 +49,9 @@ constexpr int RS = 255;   // dwords per record row in LDS: 249 data + 6 zero
 constexpr int REC_DW = CFP_REC_BYTES / 4;             // 249
 constexpr int TILE_REC_V4 = kTileEnvs * REC_DW / 4;   // 1992 16-byte chunks
 constexpr int LDS_FLOATS = kTileEnvs * XS;            // 8320 >= 32*255
+constexpr int kRedFloats = 2 * 16 * 64;               // head K-half partials
+constexpr int kEncPairs = kKbEnc / 2;                 // 53 steps of two K blocks
+constexpr int kMapPairs = kKbMap / 2;                 // 49 all-map steps (blocks 0..97)
 
 __device__ __forceinline__ float sigmoid_fast(float z) {
     return __builtin_amdgcn_rcpf(1.0f + __expf(-z));
@@ -69,78 +84,23 @@ __device__ __forceinline__ void copy_tile_out(const float* lds, float* dst,
         d4[i] = xs4[(i >> 6) * XS4 + (i & 63)];
 }
 
-// Classic-game encoder (encode_obs_kernel, craftax_classic.cu:1714-1751): the
-// observation is one-hot per view cell, so h0 is b_enc plus a sum of W_enc
-// rows selected by the record bytes, in feature order.  Thread k owns hidden
-// unit k and walks the tile's 32 envs; the record bytes are LDS broadcasts and
-// every W_enc row read is one coalesced 1 KiB line set from L2.
-__device__ __forceinline__ void classic_encode_tile(const FwdArgs& a, uint8_t* crec,
-                                                    float* lds, size_t e0, int tid) {
-    constexpr int CELLS = 63, CH = 21, NBLK = 17;
-    constexpr int TILE_V4 = kTileEnvs * CFP_CLASSIC_REC_BYTES / 16;   // 296
-    const u4* src = reinterpret_cast<const u4*>(a.rec + e0 * CFP_CLASSIC_REC_BYTES);
-    u4* dst = reinterpret_cast<u4*>(crec);
-    for (int i = tid; i < TILE_V4; i += kFwdThreads) dst[i] = src[i];
-    __syncthreads();
-    const float* W = a.w_enc + tid;
-    const float bias = a.b_enc[tid];
-    for (int e = 0; e < kTileEnvs; e++) {
-        const uint8_t* o = crec + e * CFP_CLASSIC_REC_BYTES;
-        float hv = bias;
-        for (int cell = 0; cell < CELLS; cell++) {
-            hv += W[(size_t)(cell * CH + (int8_t)o[cell]) * CFP_HIDDEN];
-            const uint32_t m = o[CELLS + cell];
-            if (m) {
-                const float* wm = W + (size_t)(cell * CH + NBLK) * CFP_HIDDEN;
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (m & (1u << j)) hv += wm[(size_t)j * CFP_HIDDEN];
-            }
-        }
-        int f = CELLS * CH;
-#pragma unroll
-        for (int j = 0; j < 16; j++, f++)
-            hv = fmaf((float)(int8_t)o[2 * CELLS + j] / 10.0f, W[(size_t)f * CFP_HIDDEN], hv);
-        const int dir = (int8_t)o[2 * CELLS + 16];
-#pragma unroll
-        for (int d = 1; d <= 4; d++, f++)
-            hv = fmaf(dir == d ? 1.0f : 0.0f, W[(size_t)f * CFP_HIDDEN], hv);
-        const float sleeping = o[2 * CELLS + 17] ? 1.0f : 0.0f;
-        const float light = *reinterpret_cast<const float*>(o + 2 * CELLS + 18);
-        hv = fmaf(light, W[(size_t)f * CFP_HIDDEN], hv); f++;
-        hv = fmaf(sleeping, W[(size_t)f * CFP_HIDDEN], hv);
-        lds[e * XS + tid] = hv;
-    }
-}
-
-}  // namespace
-
-__global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward(FwdArgs a) {
-    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
-    __shared__ float term_s[kTileEnvs];
-    __shared__ __attribute__((aligned(16))) uint8_t crec[kTileEnvs * CFP_CLASSIC_REC_BYTES];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int l32 = lane & 31;
-    const int half = lane >> 5;
-    const size_t e0 = (size_t)blockIdx.x * kTileEnvs;
-
+// Stage one tile's inputs into LDS: the records (full game: contiguous 16-byte
+// loads, rows re-strided to an odd dword count so that 32 envs reading the same
+// feature hit 32 different banks; classic: a plain copy) or the given layer-0
+// input, plus the terminal flags.
+template <int VARIANT>
+__device__ __forceinline__ void stage_tile(const FwdArgs& a, size_t e0, float* lds,
+                                           uint8_t* crec, float* term_s, int tid) {
     if (tid < kTileEnvs)
         term_s[tid] = a.terminals ? a.terminals[e0 + tid] : 0.0f;
-
-    if (a.rec && a.variant == 1) {
-        classic_encode_tile(a, crec, lds, e0, tid);
-        __syncthreads();
-        if (a.h_enc_out) copy_tile_out(lds, a.h_enc_out + e0 * CFP_HIDDEN, tid);
-    } else if (a.rec) {
-        // ---- stage the tile's records: contiguous 16-byte loads, rows
-        // re-strided to an odd dword count so that 32 envs reading the same
-        // feature hit 32 different LDS banks.
+    if (VARIANT == 1 && a.rec) {
+        constexpr int TILE_V4 = kTileEnvs * CFP_CLASSIC_REC_BYTES / 16;   // 296
+        const u4* src = reinterpret_cast<const u4*>(a.rec + e0 * CFP_CLASSIC_REC_BYTES);
+        u4* dst = reinterpret_cast<u4*>(crec);
+        for (int i = tid; i < TILE_V4; i += kFwdThreads) dst[i] = src[i];
+    } else if (VARIANT == 0 && a.rec) {
         uint32_t* rs = reinterpret_cast<uint32_t*>(lds);
-        const u4* src =
-            reinterpret_cast<const u4*>(a.rec + e0 * CFP_REC_BYTES);
+        const u4* src = reinterpret_cast<const u4*>(a.rec + e0 * CFP_REC_BYTES);
         for (int i = tid; i < TILE_REC_V4; i += kFwdThreads) {
             u4 v = __builtin_nontemporal_load(src + i);
             const uint32_t w[4] = {v.x, v.y, v.z, v.w};
@@ -157,234 +117,498 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward(FwdArgs a) {
             int c = tid - row * (RS - REC_DW);
             rs[row * RS + REC_DW + c] = 0u;   // features 843..847 read as 0.0f
         }
-        __syncthreads();
-
-        // ---- encoder GEMM: K = 848 in 106 blocks of 8; 3 rotating weight
-        // buffers, prefetch distance 2 blocks (the mirror is padded by 2).
-        f16v acc0 = zero16(), acc1 = zero16();
-        const f4* wp = a.we_pk + (size_t)(wave * 2) * 64 + lane;
-        constexpr int KB_STRIDE = 4 * 2 * 64;   // f4 per K block
-        const uint32_t* rrow = rs + l32 * RS;
-        f4 bq[3][2];
-        uint32_t wq[3];
-#pragma unroll
-        for (int s = 0; s < 2; s++) {
-            bq[s][0] = wp[(size_t)s * KB_STRIDE];
-            bq[s][1] = wp[(size_t)s * KB_STRIDE + 64];
-        }
-        wq[0] = rrow[half];
-        // The scheduling barriers pin the prefetches ahead of the MFMA block
-        // that hides them; without them the compiler sinks each load to just
-        // before its use and the L2 latency lands on the matrix pipe.
-#pragma unroll 1
-        for (int kb0 = 0; kb0 < kKbMap; kb0 += 3) {
-#pragma unroll
-            for (int s = 0; s < 3; s++) {
-                const int kb = kb0 + s;
-                const int sp = (s + 2) % 3;
-                bq[sp][0] = wp[(size_t)(kb + 2) * KB_STRIDE];
-                bq[sp][1] = wp[(size_t)(kb + 2) * KB_STRIDE + 64];
-                wq[(s + 1) % 3] = rrow[2 * (kb + 1) + half];
-                __builtin_amdgcn_sched_barrier(0);
-                const uint32_t w = wq[s];
-                const float x0 = (float)(w & 0xffu);
-                const float x1 = (float)((w >> 8) & 0xffu);
-                const float x2 = (float)((w >> 16) & 0xffu);
-                const float x3 = (float)(w >> 24);
-                acc0 = mfma(x0, bq[s][0].x, acc0);
-                acc1 = mfma(x0, bq[s][1].x, acc1);
-                acc0 = mfma(x1, bq[s][0].y, acc0);
-                acc1 = mfma(x1, bq[s][1].y, acc1);
-                acc0 = mfma(x2, bq[s][0].z, acc0);
-                acc1 = mfma(x2, bq[s][1].z, acc1);
-                acc0 = mfma(x3, bq[s][0].w, acc0);
-                acc1 = mfma(x3, bq[s][1].w, acc1);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        // tail floats: blocks 99..105 (buffer index stays kb % 3; 99 % 3 == 0)
-        const float* frow = reinterpret_cast<const float*>(rrow) +
-                            (CFP_OBS_MAP / 4) + 4 * half;
-#pragma unroll
-        for (int kt = 0; kt < kKbEnc - kKbMap; kt++) {
-            const int kb = kKbMap + kt;
-            const int s = kt % 3;
-            const int sp = (kt + 2) % 3;
-            bq[sp][0] = wp[(size_t)(kb + 2) * KB_STRIDE];
-            bq[sp][1] = wp[(size_t)(kb + 2) * KB_STRIDE + 64];
-            const float x0 = frow[8 * kt + 0];
-            const float x1 = frow[8 * kt + 1];
-            const float x2 = frow[8 * kt + 2];
-            const float x3 = frow[8 * kt + 3];
-            acc0 = mfma(x0, bq[s][0].x, acc0);
-            acc1 = mfma(x0, bq[s][1].x, acc1);
-            acc0 = mfma(x1, bq[s][0].y, acc0);
-            acc1 = mfma(x1, bq[s][1].y, acc1);
-            acc0 = mfma(x2, bq[s][0].z, acc0);
-            acc1 = mfma(x2, bq[s][1].z, acc1);
-            acc0 = mfma(x3, bq[s][0].w, acc0);
-            acc1 = mfma(x3, bq[s][1].w, acc1);
-        }
-        __syncthreads();   // every wave is done with the record bytes
-
-        // ---- bias epilogue -> x tile (aliases the record bytes)
-#pragma unroll
-        for (int ut = 0; ut < 2; ut++) {
-            const float bias = a.b_enc[wave * 64 + ut * 32 + l32];
-            float* xrow = lds + (4 * half) * XS + wave * 64 + ut * 32 + l32;
-            const f16v& acc = ut ? acc1 : acc0;
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                xrow[acc_row(r) * XS] = acc[r] + bias;
-        }
-        __syncthreads();
-        if (a.h_enc_out) copy_tile_out(lds, a.h_enc_out + e0 * CFP_HIDDEN, tid);
     } else {
-        // layer-0 input given in HBM: stage [32][256] fp32 into the x tile
         const f4* src = reinterpret_cast<const f4*>(a.x0 + e0 * CFP_HIDDEN);
         f4* xs4 = reinterpret_cast<f4*>(lds);
-        for (int i = tid; i < kTileEnvs * CFP_HIDDEN / 4; i += kFwdThreads) {
-            int row = i >> 6, c4 = i & 63;
-            xs4[row * XS4 + c4] = src[i];
-        }
-        __syncthreads();
+        for (int i = tid; i < kTileEnvs * CFP_HIDDEN / 4; i += kFwdThreads)
+            xs4[(i >> 6) * XS4 + (i & 63)] = src[i];
     }
+}
 
-    const f4* xs4 = reinterpret_cast<const f4*>(lds);
-    const int arow4 = l32 * XS4 + half;   // + 2*kb
+// Classic-game encoder (encode_obs_kernel, craftax_classic.cu:1714-1751): the
+// observation is one-hot per view cell, so h0 is b_enc plus a sum of W_enc
+// rows selected by the record bytes, in feature order.  Thread k owns hidden
+// unit k and walks the tile's 32 envs; the record bytes are LDS broadcasts and
+// every W_enc row read is one coalesced 1 KiB line set from L2.
+__device__ __forceinline__ void classic_encode_tile(const FwdArgs& a, const uint8_t* crec,
+                                                    float* lds, int tid) {
+    constexpr int CELLS = 63, CH = 21, NBLK = 17;
+    const float* W = a.w_enc;            // uniform base, [tid] applied at each load
+    const unsigned k = (unsigned)tid;
+    const float bias = a.b_enc[tid];
+    for (int e = 0; e < kTileEnvs; e++) {
+        const uint8_t* o = crec + e * CFP_CLASSIC_REC_BYTES;
+        float hv = bias;
+        for (int cell = 0; cell < CELLS; cell++) {
+            hv += (W + (size_t)(cell * CH + (int8_t)o[cell]) * CFP_HIDDEN)[k];
+            const uint32_t m = o[CELLS + cell];
+            if (m) {
+                const float* wm = W + (size_t)(cell * CH + NBLK) * CFP_HIDDEN;
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    if (m & (1u << j)) hv += (wm + (size_t)j * CFP_HIDDEN)[k];
+            }
+        }
+        int f = CELLS * CH;
+#pragma unroll
+        for (int j = 0; j < 16; j++, f++)
+            hv = fmaf((float)(int8_t)o[2 * CELLS + j] / 10.0f, (W + (size_t)f * CFP_HIDDEN)[k], hv);
+        const int dir = (int8_t)o[2 * CELLS + 16];
+#pragma unroll
+        for (int d = 1; d <= 4; d++, f++)
+            hv = fmaf(dir == d ? 1.0f : 0.0f, (W + (size_t)f * CFP_HIDDEN)[k], hv);
+        const float sleeping = o[2 * CELLS + 17] ? 1.0f : 0.0f;
+        const float light = *reinterpret_cast<const float*>(o + 2 * CELLS + 18);
+        hv = fmaf(light, (W + (size_t)f * CFP_HIDDEN)[k], hv); f++;
+        hv = fmaf(sleeping, (W + (size_t)f * CFP_HIDDEN)[k], hv);
+        lds[e * XS + tid] = hv;
+    }
+}
 
-    // ---- MinGRU layers --------------------------------------------------
-    for (int l = 0; l < a.layers; l++) {
-        constexpr int KB_STRIDE = 4 * 6 * 64;   // f4 per K block
-        const f4* wp = a.wg_pk + (size_t)l * (kGruPackFloats / 4) +
-                       (size_t)(wave * 6) * 64 + lane;
-        f16v acc[6];
+// Lane-constant context of one wave.
+struct Lane {
+    unsigned lane_u;   // 0..63
+    int half;          // lane / 32
+    int l32;           // lane % 32
+    int wave;          // 0..3, scalar
+    int arow4;         // f4 index of this lane's A fragment in an x tile, + 2*kb
+    unsigned loff;     // lane offset (floats) into a [32][256] state tile row set
+};
+
+// ---- encoder GEMM of both tiles of a pair: K = 848 as 53 steps of two 8-wide K
+// blocks.  The weight fragments of a step feed both tiles (4 accumulators), so
+// the mirror is streamed once per pair.  Weights sit three steps deep in
+// registers; the step loop is unrolled by three so that the ring needs no moves
+// (a register rotation would make every iteration wait for ALL loads in flight).
+struct EncB { f4 b[4]; };   // (block 0|1) x (unit tile 0|1)
+
+__device__ __forceinline__ EncB enc_load_b(const f4* wp, int step, unsigned lane_u) {
+    constexpr int KB_STRIDE = 4 * 2 * 64;   // f4 per K block
+    EncB r;
+    const f4* p = wp + (size_t)(2 * step) * KB_STRIDE;
+    r.b[0] = (p)[lane_u];
+    r.b[1] = (p + 64)[lane_u];
+    r.b[2] = (p + KB_STRIDE)[lane_u];
+    r.b[3] = (p + KB_STRIDE + 64)[lane_u];
+    return r;
+}
+
+__device__ __forceinline__ void enc_mma(f16v (&acc)[4], const float (&x)[8],
+                                        const float (&y)[8], const EncB& w) {
 #pragma unroll
-        for (int t = 0; t < 6; t++) acc[t] = zero16();
-        f4 bA[6], bB[6], aA, aB;
+    for (int q = 0; q < 2; q++)
 #pragma unroll
-        for (int t = 0; t < 6; t++) bA[t] = wp[t * 64];
-        aA = xs4[arow4];
+        for (int j = 0; j < 4; j++) {
+            acc[0] = mfma(x[4 * q + j], w.b[2 * q][j], acc[0]);
+            acc[1] = mfma(x[4 * q + j], w.b[2 * q + 1][j], acc[1]);
+            acc[2] = mfma(y[4 * q + j], w.b[2 * q][j], acc[2]);
+            acc[3] = mfma(y[4 * q + j], w.b[2 * q + 1][j], acc[3]);
+        }
+}
+
+__device__ __forceinline__ void bytes_to_f(uint32_t w, float* x) {
+    x[0] = (float)(w & 0xffu);
+    x[1] = (float)((w >> 8) & 0xffu);
+    x[2] = (float)((w >> 16) & 0xffu);
+    x[3] = (float)(w >> 24);
+}
+
+struct EncBytes { uint32_t x0, x1, y0, y1; };
+
+__device__ __forceinline__ EncBytes enc_bytes(const uint32_t* rx, const uint32_t* ry,
+                                              int step, int half) {
+    EncBytes r;
+    r.x0 = rx[4 * step + half];
+    r.x1 = rx[4 * step + 2 + half];
+    r.y0 = ry[4 * step + half];
+    r.y1 = ry[4 * step + 2 + half];
+    return r;
+}
+
+// One all-map step: request the weights of step p+2 and the bytes of step p+1,
+// then the 32 MFMAs of step p.
+__device__ __forceinline__ void enc_map_step(f16v (&acc)[4], const f4* wp, const uint32_t* rx,
+                                             const uint32_t* ry, int p, const EncB& use,
+                                             EncB& fill, EncBytes& cur, const Lane& L) {
+    fill = enc_load_b(wp, p + 2, L.lane_u);
+    const EncBytes nxt = enc_bytes(rx, ry, p + 1, L.half);
+    float x[8], y[8];
+    bytes_to_f(cur.x0, x);
+    bytes_to_f(cur.x1, x + 4);
+    bytes_to_f(cur.y0, y);
+    bytes_to_f(cur.y1, y + 4);
+    enc_mma(acc, x, y, use);
+    // one weight load per eight MFMAs, the LDS reads and conversions in between
+#pragma unroll
+    for (int q = 0; q < 32; q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (q % 8 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (q % 8 == 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (q < 16) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    cur = nxt;
+}
+
+// Steps 49..52: map block 98 + tail block 0, then tail blocks 1..6 (fp32 features).
+template <int P>
+__device__ __forceinline__ void enc_tail_step(f16v (&acc)[4], const f4* wp, const float* fx,
+                                              const float* fy, const EncB& use, EncB& fill,
+                                              const EncBytes& cur, const Lane& L) {
+    if (P + 2 < kEncPairs) fill = enc_load_b(wp, P + 2, L.lane_u);
+    float x[8], y[8];
+    if (P == kMapPairs) {
+        bytes_to_f(cur.x0, x);
+        bytes_to_f(cur.y0, y);
+#pragma unroll
+        for (int j = 0; j < 4; j++) { x[4 + j] = fx[j]; y[4 + j] = fy[j]; }
+    } else {
+        constexpr int kt = 2 * (P - kMapPairs) - 1;   // first tail block of the step
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            x[j] = fx[8 * kt + j];
+            x[4 + j] = fx[8 * (kt + 1) + j];
+            y[j] = fy[8 * kt + j];
+            y[4 + j] = fy[8 * (kt + 1) + j];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    enc_mma(acc, x, y, use);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void encoder_gemm(const FwdArgs& a, const float* ldsX,
+                                             const float* ldsY, const Lane& L,
+                                             f16v (&acc)[4]) {
+    static_assert(kMapPairs == 49 && kEncPairs == 53, "step schedule below assumes 49 + 4");
+    const uint32_t* rx = reinterpret_cast<const uint32_t*>(ldsX) + L.l32 * RS;
+    const uint32_t* ry = reinterpret_cast<const uint32_t*>(ldsY) + L.l32 * RS;
+    const float* fx = reinterpret_cast<const float*>(rx) + (CFP_OBS_MAP / 4) + 4 * L.half;
+    const float* fy = reinterpret_cast<const float*>(ry) + (CFP_OBS_MAP / 4) + 4 * L.half;
+    const f4* wp = a.we_pk + (size_t)(L.wave * 2) * 64;
+    EncB b0 = enc_load_b(wp, 0, L.lane_u), b1 = enc_load_b(wp, 1, L.lane_u), b2;
+    EncBytes cur = enc_bytes(rx, ry, 0, L.half);
 #pragma unroll 1
-        for (int kb = 0; kb < kKbHid; kb += 2) {
+    for (int p = 0; p < 48; p += 3) {
+        enc_map_step(acc, wp, rx, ry, p, b0, b2, cur, L);
+        enc_map_step(acc, wp, rx, ry, p + 1, b1, b0, cur, L);
+        enc_map_step(acc, wp, rx, ry, p + 2, b2, b1, cur, L);
+    }
+    // step 48 is the last all-map step; its "next bytes" are map block 98 plus
+    // the first tail dword, which step 49 re-reads as a float
+    enc_map_step(acc, wp, rx, ry, 48, b0, b2, cur, L);
+    enc_tail_step<49>(acc, wp, fx, fy, b1, b0, cur, L);
+    enc_tail_step<50>(acc, wp, fx, fy, b2, b1, cur, L);
+    enc_tail_step<51>(acc, wp, fx, fy, b0, b2, cur, L);
+    enc_tail_step<52>(acc, wp, fx, fy, b1, b0, cur, L);
+}
+
+// ---- MinGRU phases ---------------------------------------------------------------
+// Written-to-nowhere tile: state / r_state addresses of a pair's missing second
+// tile point here, so the hot loop needs no predication.
+__device__ float g_void_tile[kTileEnvs * CFP_HIDDEN];
+
+// State addressing of one (tile, layer) for the epilogue: element e = 0..31 of a
+// lane is unit tile e/16, accumulator register e%16.
+struct StateIO {
+    float* st_base;    // state tile + wave*64 (uniform)
+    float* rs_base;    // r_state tile likewise (ignored unless HAS_RS)
+    unsigned tmask;    // bit r: env row of accumulator register r had a terminal
+};
+
+__device__ __forceinline__ constexpr int st_off(int e) {
+    return acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32;
+}
+
+// Request the 32 state values the next epilogue will consume.
+__device__ __forceinline__ void state_load(const StateIO& io, float (&st)[32], const Lane& L) {
 #pragma unroll
-            for (int t = 0; t < 6; t++)
-                bB[t] = wp[(size_t)(kb + 1) * KB_STRIDE + t * 64];
-            aB = xs4[arow4 + 2 * (kb + 1)];
-            __builtin_amdgcn_sched_barrier(0);
+    for (int e = 0; e < 32; e++)
+        st[e] = __builtin_nontemporal_load((io.st_base + st_off(e)) + L.loff);
+}
+
+using WRing = f4[3][6];
+
+// First two K blocks of a layer's weights into ring slots 0 and 1.
+__device__ __forceinline__ void ring_preload(WRing& bq, const f4* wp, const Lane& L) {
+    constexpr int KB_STRIDE = 4 * 6 * 64;
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int t = 0; t < 6; t++)
+            bq[b][t] = (wp + (size_t)b * KB_STRIDE + t * 64)[L.lane_u];
+}
+
+// DO_K: accN[6] += x_K . W_l^T for the tile whose x tile is `xs4K`; the ring
+//       holds K blocks 0 and 1 on entry, block kb+2 is requested while block kb
+//       is multiplied (two blocks = 3072 matrix-pipe cycles of latency cover).
+// DO_E: the gate/blend epilogue of the OTHER tile from accO[6], one element next
+//       to each K block: element kb's ~35 vector instructions, its two LDS
+//       accesses and its state / r_state stores issue in the shadow of the 24
+//       MFMAs.  The block is branch-free (a branch would split it and leave the
+//       epilogue behind the MFMAs).  The state values were requested before the
+//       phase (st[32]); in-loop state loads would sit in front of the weight
+//       loads in the in-order return queue with their HBM latency.
+template <bool DO_K, bool DO_E, bool HAS_RS>
+__device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6], WRing& bq,
+                                          const f4* xs4K, const f4* wp, float* xsE,
+                                          const StateIO& io, const float (&st)[32],
+                                          const Lane& L) {
+    constexpr int KB_STRIDE = 4 * 6 * 64;   // f4 per K block
+    f4 aq[2];
+    if (DO_K) aq[0] = xs4K[L.arow4];
+#pragma unroll
+    for (int kb = 0; kb < kKbHid; kb++) {
+        const int cb = kb & 1, nb = cb ^ 1;
+        if (DO_K) {
+            if (kb + 2 < kKbHid) {
+#pragma unroll
+                for (int t = 0; t < 6; t++)
+                    bq[(kb + 2) % 3][t] = (wp + (size_t)(kb + 2) * KB_STRIDE + t * 64)[L.lane_u];
+            }
+            if (kb + 1 < kKbHid) aq[nb] = xs4K[L.arow4 + 2 * (kb + 1)];
+        }
+        if (DO_K) {
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int t = 0; t < 6; t++)
-                    acc[t] = mfma(aA[j], bA[t][j], acc[t]);
-            __builtin_amdgcn_sched_barrier(0);
-            // kb + 2 == 32 prefetches the next layer's first weight block (or
-            // the zero pad behind the last layer); the x index is clamped.
-#pragma unroll
-            for (int t = 0; t < 6; t++)
-                bA[t] = wp[(size_t)(kb + 2) * KB_STRIDE + t * 64];
-            aA = xs4[arow4 + 2 * (kb + 2 < kKbHid ? kb + 2 : kKbHid - 1)];
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-#pragma unroll
-                for (int t = 0; t < 6; t++)
-                    acc[t] = mfma(aB[j], bB[t][j], acc[t]);
-            __builtin_amdgcn_sched_barrier(0);
+                    accN[t] = mfma(aq[cb][j], bq[kb % 3][t][j], accN[t]);
         }
-
-        // State for this wave's 2 x 16 elements per lane, issued before the
-        // barrier so the HBM latency overlaps the other waves' K loops.
-        // Addresses are (uniform base + compile-time row offset)[lane offset]
-        // so they live in SGPRs plus one VGPR.
-        const int loff = (4 * half) * CFP_HIDDEN + wave * 64 + l32;
-        float* st_base =
-            a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN;
-        float st[2][16];
-#pragma unroll
-        for (int ut = 0; ut < 2; ut++)
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                st[ut][r] = __builtin_nontemporal_load(
-                    st_base + (acc_row(r) * CFP_HIDDEN + ut * 32) + loff);
-
-        __syncthreads();   // all waves finished reading the x tile
-
-#pragma unroll
-        for (int ut = 0; ut < 2; ut++)
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                if (term_s[acc_row(r) + 4 * half] != 0.0f) st[ut][r] = 0.0f;
-        if (a.r_state) {
-            float* rs_base =
-                a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN;
-#pragma unroll
-            for (int ut = 0; ut < 2; ut++)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    __builtin_nontemporal_store(
-                        st[ut][r],
-                        rs_base + (acc_row(r) * CFP_HIDDEN + ut * 32) + loff);
+        if (DO_E) {
+            const int ut = kb / 16, r = kb % 16;
+            float* xp = xsE + (acc_row(r) + 4 * L.half) * XS + L.wave * 64 + ut * 32 + L.l32;
+            const float s = (io.tmask >> r) & 1u ? 0.0f : st[kb];
+            if (HAS_RS) __builtin_nontemporal_store(s, (io.rs_base + st_off(kb)) + L.loff);
+            const float zh = accO[0 + ut][r];
+            const float zg = accO[2 + ut][r];
+            const float zp = accO[4 + ut][r];
+            const float sg = sigmoid_fast(zg);
+            float sh = sigmoid_fast(zh);
+            asm volatile("" : "+v"(sh));   // keep g(zh) a select, not a branch
+            const float gh = zh >= 0.0f ? zh + 0.5f : sh;
+            const float out = s + sg * (gh - s);
+            const float p = sigmoid_fast(zp);
+            const float xv = *xp;
+            *xp = p * out + (1.0f - p) * xv;
+            __builtin_nontemporal_store(out, (io.st_base + st_off(kb)) + L.loff);
         }
+        // Issue order of the block.  A vector memory instruction occupies the
+        // wave's issue port for about as long as one MFMA executes, so the six
+        // weight loads are spread one per four MFMAs instead of bunched (bunched,
+        // they leave the matrix pipe idle for ~5 MFMA slots per block).
+        if (DO_K) {
 #pragma unroll
-        for (int ut = 0; ut < 2; ut++) {
-            float* xrow = lds + (4 * half) * XS + wave * 64 + ut * 32 + l32;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float s = st[ut][r];
-                const float zh = acc[0 + ut][r];
-                const float zg = acc[2 + ut][r];
-                const float zp = acc[4 + ut][r];
-                const float sg = sigmoid_fast(zg);
-                const float gh = zh >= 0.0f ? zh + 0.5f : sigmoid_fast(zh);
-                const float out = s + sg * (gh - s);
-                const float p = sigmoid_fast(zp);
-                const float xv = xrow[acc_row(r) * XS];
-                xrow[acc_row(r) * XS] = p * out + (1.0f - p) * xv;
-                __builtin_nontemporal_store(
-                    out, st_base + (acc_row(r) * CFP_HIDDEN + ut * 32) + loff);
+            for (int q = 0; q < 24; q++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one MFMA
+                if (q % 4 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
+                if (q == 2) __builtin_amdgcn_sched_group_barrier(0x100, DO_E ? 2 : 1, 0);
+                if (DO_E) {
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // two VALU
+                    if (q == 21) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                    if (q == 22) __builtin_amdgcn_sched_group_barrier(0x040, HAS_RS ? 2 : 1, 0);
+                }
             }
         }
-        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
     }
-    if (a.layers > 0 && a.h3_out)
-        copy_tile_out(lds, a.h3_out + e0 * CFP_HIDDEN, tid);
+}
 
-    // ---- heads: wave = (row tile nt, K half kh) ---------------------------
-    if (a.do_head) {
-        const int nt = wave & 1;
-        const int kh = wave >> 1;
-        f16v acc = zero16();
-        const f4* wp = a.wav_pk + (size_t)nt * 64 + lane;
-#pragma unroll
-        for (int i = 0; i < kKbHid / 2; i++) {
-            const int kb = kh * (kKbHid / 2) + i;
-            const f4 b = wp[(size_t)kb * 128];
-            const f4 av = xs4[arow4 + 2 * kb];
-#pragma unroll
-            for (int j = 0; j < 4; j++) acc = mfma(av[j], b[j], acc);
-        }
-        __syncthreads();   // x tile dead; reuse LDS for the K-half reduction
-        float* red = lds + (nt * 16) * 64 + lane;
-        if (kh == 1) {
-#pragma unroll
-            for (int r = 0; r < 16; r++) red[r * 64] = acc[r];
+}  // namespace
+
+template <int VARIANT, bool HAS_RS>
+__global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
+    __shared__ __attribute__((aligned(16))) float lds_all[2][LDS_FLOATS];
+    __shared__ __attribute__((aligned(16))) float red_all[2][kRedFloats];
+    __shared__ float term_all[2][kTileEnvs];
+    __shared__ __attribute__((aligned(16))) uint8_t crec_all[2][kTileEnvs * CFP_CLASSIC_REC_BYTES];
+
+    const int tiles = a.n / kTileEnvs;
+    const int pairs = (tiles + 1) / 2;
+    const bool classic = VARIANT == 1 && a.rec;
+    const bool full_rec = VARIANT == 0 && a.rec;
+
+    for (int pair = blockIdx.x; pair < pairs; pair += gridDim.x) {
+        // Lane constants are re-derived per pair from an opaque copy of the thread
+        // index: hoisted out of this loop, the dozens of per-lane addresses they
+        // feed would stay live across every phase and spill.
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        Lane L;
+        L.lane_u = (unsigned)(tid & 63);
+        L.half = (tid & 63) >> 5;
+        L.l32 = tid & 31;
+        L.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        L.arow4 = L.l32 * XS4 + L.half;
+        L.loff = (unsigned)((4 * L.half) * CFP_HIDDEN + L.l32);
+        const int nt = L.wave & 1;   // head: row tile
+        const int kh = L.wave >> 1;  // head: K half
+        // tile X = 2*pair always exists; tile Y may be past the end (odd tile count)
+        const bool hasY = 2 * pair + 1 < tiles;
+        size_t e0[2] = {(size_t)(2 * pair) * kTileEnvs, (size_t)(2 * pair + 1) * kTileEnvs};
+
+        // ---- stage both tiles (a missing Y is a zero tile that is computed but
+        // never read from or written to the caller's buffers) --------------------
+        stage_tile<VARIANT>(a, e0[0], lds_all[0], crec_all[0], term_all[0], tid);
+        if (hasY) {
+            stage_tile<VARIANT>(a, e0[1], lds_all[1], crec_all[1], term_all[1], tid);
+        } else {
+            for (int i = tid; i < LDS_FLOATS; i += kFwdThreads) lds_all[1][i] = 0.0f;
+            if (tid < kTileEnvs) term_all[1][tid] = 0.0f;
+            for (int i = tid; i < kTileEnvs * CFP_CLASSIC_REC_BYTES; i += kFwdThreads)
+                crec_all[1][i] = 0;
         }
         __syncthreads();
-        if (kh == 0) {
-            const int arow = nt * 32 + l32;
-            const int avs = a.actions + 1;     // 44, or 18 for the classic game
-            if (arow < avs) {
-                const float bias = arow < a.actions ? a.b_a[arow] : a.b_v[0];
-                float* av_base = a.av_out + e0 * avs;
-                const int aoff = (4 * half) * avs + arow;
+
+        unsigned tmask[2] = {0u, 0u};
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    (av_base + acc_row(r) * avs)[aoff] =
-                        acc[r] + red[r * 64] + bias;
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                if (term_all[s][acc_row(r) + 4 * L.half] != 0.0f) tmask[s] |= 1u << r;
+
+        // ---- encoders ----------------------------------------------------------
+        if (classic) {
+#pragma unroll 1
+            for (int s = 0; s < 2; s++) classic_encode_tile(a, crec_all[s], lds_all[s], tid);
+        } else if (full_rec) {
+            f16v eacc[4];
+#pragma unroll
+            for (int t = 0; t < 4; t++) eacc[t] = zero16();
+            encoder_gemm(a, lds_all[0], lds_all[1], L, eacc);
+            __syncthreads();   // every wave is done with the record bytes
+#pragma unroll
+            for (int s = 0; s < 2; s++)
+#pragma unroll
+                for (int ut = 0; ut < 2; ut++) {
+                    const float bias = a.b_enc[L.wave * 64 + ut * 32 + L.l32];
+                    float* xrow = lds_all[s] + (4 * L.half) * XS + L.wave * 64 + ut * 32 + L.l32;
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        xrow[acc_row(r) * XS] = eacc[2 * s + ut][r] + bias;
+                }
+        }
+        __syncthreads();
+        if (a.rec && a.h_enc_out) {
+            copy_tile_out(lds_all[0], a.h_enc_out + e0[0] * CFP_HIDDEN, tid);
+            if (hasY) copy_tile_out(lds_all[1], a.h_enc_out + e0[1] * CFP_HIDDEN, tid);
+        }
+
+        // ---- MinGRU layers, the two tiles software-pipelined -------------------------
+        // phase q = 0 .. 2L:  K(tile q&1, layer q/2)  woven with  epi(tile (q-1)&1, layer (q-1)/2)
+        // Before the barrier that ends phase q, the first two weight blocks and
+        // the state of phase q+1 are requested, in that order.
+        if (a.layers > 0) {
+            f16v accO[6], accN[6];
+            float st[32];
+            WRing bq;
+            const size_t wl = kGruPackFloats / 4;   // f4 per layer of the mirror
+            const f4* wp0 = a.wg_pk + (size_t)(L.wave * 6) * 64;
+            auto state_io = [&](int q) {
+                const int s = (q - 1) & 1, l = (q - 1) >> 1;
+                StateIO c;
+                if (s == 0 || hasY) {
+                    const size_t off = (size_t)l * a.layer_stride + e0[s] * CFP_HIDDEN + L.wave * 64;
+                    c.st_base = a.state + off;
+                    c.rs_base = HAS_RS ? a.r_state + off : nullptr;
+                } else {
+                    c.st_base = g_void_tile + L.wave * 64;
+                    c.rs_base = g_void_tile + L.wave * 64;
+                }
+                c.tmask = tmask[s];
+                return c;
+            };
+            const int Q = 2 * a.layers;
+#pragma unroll
+            for (int t = 0; t < 6; t++) accO[t] = zero16();
+            ring_preload(bq, wp0, L);
+            StateIO io = state_io(1);
+            gru_phase<true, false, HAS_RS>(accO, accO, bq, reinterpret_cast<const f4*>(lds_all[0]),
+                                           wp0, nullptr, io, st, L);
+            ring_preload(bq, wp0, L);
+            state_load(io, st, L);
+            __syncthreads();
+#pragma unroll 1
+            for (int q = 1; q < Q; q++) {
+#pragma unroll
+                for (int t = 0; t < 6; t++) accN[t] = zero16();
+                gru_phase<true, true, HAS_RS>(accN, accO, bq,
+                                              reinterpret_cast<const f4*>(lds_all[q & 1]),
+                                              wp0 + (size_t)(q >> 1) * wl, lds_all[(q - 1) & 1],
+                                              io, st, L);
+                if (q + 1 < Q) ring_preload(bq, wp0 + (size_t)((q + 1) >> 1) * wl, L);
+                io = state_io(q + 1);
+                state_load(io, st, L);
+                __syncthreads();
+#pragma unroll
+                for (int t = 0; t < 6; t++) accO[t] = accN[t];
+            }
+            gru_phase<false, true, HAS_RS>(accN, accO, bq, nullptr, nullptr, lds_all[(Q - 1) & 1],
+                                           io, st, L);
+            __syncthreads();
+            if (a.h3_out) {
+                copy_tile_out(lds_all[0], a.h3_out + e0[0] * CFP_HIDDEN, tid);
+                if (hasY) copy_tile_out(lds_all[1], a.h3_out + e0[1] * CFP_HIDDEN, tid);
             }
         }
+
+        // ---- heads: wave = (row tile nt, K half kh), both tiles -----------------------
+        if (a.do_head) {
+            f16v hacc[2];
+            const f4* wp = a.wav_pk + (size_t)nt * 64;
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                hacc[s] = zero16();
+                const f4* xs4 = reinterpret_cast<const f4*>(lds_all[s]);
+#pragma unroll
+                for (int i = 0; i < kKbHid / 2; i++) {
+                    const int kb = kh * (kKbHid / 2) + i;
+                    const f4 b = (wp + (size_t)kb * 128)[L.lane_u];
+                    const f4 av = xs4[L.arow4 + 2 * kb];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) hacc[s] = mfma(av[j], b[j], hacc[s]);
+                }
+                if (kh == 1) {
+                    float* red = red_all[s] + (nt * 16) * 64 + L.lane_u;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) red[r * 64] = hacc[s][r];
+                }
+            }
+            __syncthreads();
+            if (kh == 0) {
+                const int arow = nt * 32 + L.l32;
+                const int avs = a.actions + 1;     // 44, or 18 for the classic game
+                if (arow < avs) {
+                    const float bias = arow < a.actions ? a.b_a[arow] : a.b_v[0];
+#pragma unroll
+                    for (int s = 0; s < 2; s++) {
+                        if (s == 1 && !hasY) continue;
+                        const float* red = red_all[s] + (nt * 16) * 64 + L.lane_u;
+                        float* av_base = a.av_out + e0[s] * avs;
+                        const int aoff = (4 * L.half) * avs + arow;
+#pragma unroll
+                        for (int r = 0; r < 16; r++)
+                            (av_base + acc_row(r) * avs)[aoff] = hacc[s][r] + red[r * 64] + bias;
+                    }
+                }
+            }
+        }
+        __syncthreads();   // LDS tiles and partials are free for the next pair
     }
+}
+
+static int num_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+            v > 0)
+            cus = v;
+        else
+            cus = 256;
+    }
+    return cus;
 }
 
 int launch_forward(const FwdArgs& a, hipStream_t st) {
@@ -408,8 +632,17 @@ int launch_forward(const FwdArgs& a, hipStream_t st) {
                 "MinGRU layers need a state buffer");
     CFP_REQUIRE(!a.do_head || a.av_out != nullptr,
                 "head requested without an output buffer");
-    hipLaunchKernelGGL(k_policy_forward, dim3(a.n / kTileEnvs),
-                       dim3(kFwdThreads), 0, st, a);
+    // persistent: one workgroup per CU, each walking tile pairs round-robin
+    const int pairs = (a.n / kTileEnvs + 1) / 2;
+    const int grid = pairs < num_cus() ? pairs : num_cus();
+    const dim3 g(grid), b(kFwdThreads);
+    if (a.variant == 1) {
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<1, true>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward<1, false>), g, b, 0, st, a);
+    } else {
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<0, true>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward<0, false>), g, b, 0, st, a);
+    }
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -462,7 +695,7 @@ int launch_pack_weights(const float* params, int layers, int variant, float* we_
                         float* wg_pk, float* wav_pk, hipStream_t st) {
     const Arena ar = arena_of(variant, layers);
     if (variant == 0) {   // the classic encoder gathers from the unpacked W_enc
-        const int enc_total = (kKbEnc + 2) * 2048;
+        const int enc_total = (kKbEnc + kEncPadBlocks) * 2048;
         hipLaunchKernelGGL(k_pack_enc, dim3((enc_total + 255) / 256), dim3(256), 0,
                            st, params + ar.w_enc, we_pk, enc_total);
     }
