@@ -146,6 +146,23 @@ def main():
                          "env_steps_per_s": n * steps / wall}
     assert torch.isfinite(av).all(), "non-finite policy outputs"
 
+    # bf16-input / fp32-accumulate variant of the same step (reported beside the fp32
+    # figure, never as `value`): bound by vector work and HBM, so it carries an HBM
+    # fraction instead of an MFMA one
+    bf16 = None
+    if args.schedule == "both":
+        pol.set_gemm_bf16(True)
+        state.zero_()
+        for i in range(warmup):
+            pol.forward(recs[i % ring], term, state, av=av)
+        wall, dev_ms = time_steps(pol, recs, term, state, av, steps, 0, torch)
+        pol.set_gemm_bf16(False)
+        assert torch.isfinite(av).all(), "non-finite bf16 policy outputs"
+        bf16 = {"ms_per_step": wall / steps * 1e3, "device_ms_per_step": dev_ms,
+                "env_steps_per_s": n * steps / wall, "kernel": "k_policy_forward_bf16",
+                "hbm_frac": BYTES_PER_ENV_STEP * n / (dev_ms * 1e-3) / 8e12,
+                "tflops": FLOP_PER_ENV_STEP * n / (dev_ms * 1e-3) / 1e12}
+
     best = results.get("unchunked") or results["chunked_16x16384"]
     launches = 1 if "unchunked" in results else max(1, n // 16384)
     launch_s = best["device_ms_per_step"] * 1e-3 / launches
@@ -163,6 +180,7 @@ def main():
                    "record_batches_in_hbm": ring},
         "pct_fp32_mfma_peak": 100.0 * achieved / PEAK_FP32_MFMA_TFLOPS,
         "chunked_16x16384": results.get("chunked_16x16384"),
+        "bf16_in_fp32_acc_unchunked": bf16,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
                      "traffic": (MEASURED_TRAFFIC_BYTES[n] // launches

@@ -53,6 +53,9 @@ static void policy_release(cfp_policy* p) {
     (void)hipFree(p->we_pk);
     (void)hipFree(p->wg_pk);
     (void)hipFree(p->wav_pk);
+    (void)hipFree(p->we_bf);
+    (void)hipFree(p->wg_bf);
+    (void)hipFree(p->wav_bf);
     (void)hipFree(p->h_state);
     (void)hipFree(p->rec);
     (void)hipFree(p->h_enc);
@@ -132,6 +135,9 @@ static int policy_create(cfp_policy** out, int num_envs, int layers, uint64_t se
     CFP_ALLOC(p->wg_pk,
               ((size_t)layers * kGruPackFloats + 4 * 6 * 64 * 4) * sizeof(float));
     CFP_ALLOC(p->wav_pk, kAvPackFloats * sizeof(float));
+    CFP_ALLOC(p->we_bf, kEncPackFloats * sizeof(uint16_t));
+    CFP_ALLOC(p->wg_bf, (size_t)layers * kGruPackFloats * sizeof(uint16_t));
+    CFP_ALLOC(p->wav_bf, kAvPackFloats * sizeof(uint16_t));
     CFP_ALLOC(p->h_state, (size_t)layers * hn * sizeof(float));
     CFP_ALLOC(p->rec, (size_t)num_envs * rec_bytes);
     CFP_ALLOC(p->h_enc, hn * sizeof(float));
@@ -195,9 +201,19 @@ int cfp_policy_get_params(const cfp_policy* p, float* host_params,
 
 int cfp_policy_refresh_weights(cfp_policy* p, void* stream) {
     CFP_REQUIRE(p, "cfp_policy_refresh_weights: NULL policy");
-    return launch_pack_weights(p->params, p->layers, p->variant, p->we_pk, p->wg_pk,
-                               p->wav_pk, (hipStream_t)stream);
+    if (launch_pack_weights(p->params, p->layers, p->variant, p->we_pk, p->wg_pk, p->wav_pk,
+                            (hipStream_t)stream) != 0)
+        return 1;
+    return launch_pack_weights_bf16(p->params, p->layers, p->variant, p->we_bf, p->wg_bf,
+                                    p->wav_bf, (hipStream_t)stream);
 }
+
+int cfp_policy_set_gemm_bf16(cfp_policy* p, int on) {
+    CFP_REQUIRE(p, "cfp_policy_set_gemm_bf16: NULL policy");
+    p->gemm_bf16 = on ? 1 : 0;
+    return 0;
+}
+int cfp_policy_gemm_bf16(const cfp_policy* p) { return p ? p->gemm_bf16 : -1; }
 
 float* cfp_policy_params(cfp_policy* p) { return p->params; }
 float* cfp_policy_state(cfp_policy* p) { return p->h_state; }
@@ -218,6 +234,10 @@ static void fill_weights(const cfp_policy* p, FwdArgs& a) {
     a.b_v = p->params + ar.b_v;
     a.variant = p->variant;
     a.actions = ar.actions;
+    a.we_bf = reinterpret_cast<const u4*>(p->we_bf);
+    a.wg_bf = reinterpret_cast<const u4*>(p->wg_bf);
+    a.wav_bf = reinterpret_cast<const u4*>(p->wav_bf);
+    a.bf16 = p->gemm_bf16;
 }
 
 // Launch over [0, n) in chunks; every per-env pointer is advanced by the

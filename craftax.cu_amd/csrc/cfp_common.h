@@ -75,8 +75,15 @@ struct FwdArgs {
     int variant;             // 0 full game (996-byte records), 1 classic (148-byte)
     int actions;             // 43 or 17; av rows = actions + 1
     const float* w_enc;      // classic: unpacked W_enc [1345][256] for the gather
+    const u4* we_bf;         // bf16 mirrors, used when bf16 != 0
+    const u4* wg_bf;
+    const u4* wav_bf;
+    int bf16;                // bf16-input / fp32-accumulate kernel
 };
 int launch_forward(const FwdArgs& a, hipStream_t st);
+int launch_forward_bf16(const FwdArgs& a, hipStream_t st);   // called by launch_forward
+int launch_pack_weights_bf16(const float* params, int layers, int variant, uint16_t* we_bf,
+                             uint16_t* wg_bf, uint16_t* wav_bf, hipStream_t st);
 
 int launch_pack_weights(const float* params, int layers, int variant, float* we_pk,
                         float* wg_pk, float* wav_pk, hipStream_t st);

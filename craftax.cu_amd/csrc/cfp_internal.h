@@ -12,6 +12,10 @@ struct cfp_policy {
     float* we_pk = nullptr;
     float* wg_pk = nullptr;
     float* wav_pk = nullptr;
+    uint16_t* we_bf = nullptr;    // bf16 mirrors (MFMA 32x32x16 order)
+    uint16_t* wg_bf = nullptr;
+    uint16_t* wav_bf = nullptr;
+    int gemm_bf16 = 0;            // forward entry points run the bf16-input kernel
     float* h_state = nullptr;
     uint8_t* rec = nullptr;
     float* h_enc = nullptr;

@@ -1,0 +1,317 @@
+// bf16-input / fp32-accumulate variant of the fused policy forward for gfx950.
+//
+// Same interface and data flow as the fp32 kernel (records -> encoder -> MinGRU
+// x L -> heads, one 32-env tile per workgroup, activations resident in LDS);
+// the three GEMMs run on v_mfma_f32_32x32x16_bf16 with weights read from bf16
+// mirrors and activations rounded to bf16 (round-to-nearest-even) as they are
+// loaded into the A operand.  Everything else stays fp32: accumulators, biases,
+// the gate/blend epilogue, the recurrent state and every output.  This is the
+// counterpart of the reference's CF_GEMM_BF16 mode (craftax_full.cu:11306-11316,
+// bf16 GEMM wrappers :11688-11756), without its bf16 storage of activations.
+//
+// At bf16 MFMA rates the matrix pipe is no longer the bound (a layer's gate GEMM
+// is 96 MFMAs of 32 cycles per wave); the kernel is bound by the epilogue's
+// vector instructions and the weight loads, so it runs two workgroups per CU
+// (one tile each, no cross-tile software pipeline) and lets the hardware
+// overlap one workgroup's epilogue with the other's GEMM.
+//
+// Operand layout of v_mfma_f32_32x32x16_bf16: lane l supplies row (A) / column
+// (B) l%32 and the eight consecutive k = 8*(l/32) .. 8*(l/32)+7 of the 16-wide K
+// block; the accumulator layout is that of the fp32 32x32 MFMA.
+#include "policy_tile.h"
+
+namespace cfp {
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f8 __attribute__((ext_vector_type(8)));
+
+constexpr int kKb16Enc = kObsPad / 16;        // 53 K blocks of 16
+constexpr int kKb16Map = CFP_OBS_MAP / 16;    // 49 all-map blocks; block 49 is half map, half tail
+constexpr int kKb16Hid = CFP_HIDDEN / 16;     // 16
+
+__device__ __forceinline__ f16v mfma16(const u4& a, const u4& b, f16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f16v zero16() {
+    f16v z;
+#pragma unroll
+    for (int i = 0; i < 16; i++) z[i] = 0.0f;
+    return z;
+}
+
+// eight fp32 -> eight bf16, round to nearest even
+__device__ __forceinline__ u4 to_bf16x8(const f4& lo, const f4& hi) {
+    f8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    return __builtin_bit_cast(u4, __builtin_convertvector(v, bf16x8));
+}
+
+// Two record bytes -> two bf16 (0..255 are exact in bf16: the upper half of the
+// fp32 encoding).
+__device__ __forceinline__ uint32_t bytes_to_bf16x2(uint32_t w, int i) {
+    const float lo = (float)((w >> (16 * i)) & 0xffu);
+    const float hi = (float)((w >> (16 * i + 8)) & 0xffu);
+    return (__float_as_uint(hi) & 0xffff0000u) | (__float_as_uint(lo) >> 16);
+}
+
+__device__ __forceinline__ u4 bytes_to_bf16x8(uint32_t w0, uint32_t w1) {
+    u4 r;
+    r.x = bytes_to_bf16x2(w0, 0);
+    r.y = bytes_to_bf16x2(w0, 1);
+    r.z = bytes_to_bf16x2(w1, 0);
+    r.w = bytes_to_bf16x2(w1, 1);
+    return r;
+}
+
+__device__ __forceinline__ u4 floats_to_bf16x8(const float* p) {
+    f4 lo = {p[0], p[1], p[2], p[3]}, hi = {p[4], p[5], p[6], p[7]};
+    return to_bf16x8(lo, hi);
+}
+
+// A fragment of K block kb from an fp32 x tile: x[row][16kb + 8g .. +7]
+__device__ __forceinline__ u4 a_frag(const f4* xs4, int l32, int g, int kb) {
+    const f4* p = xs4 + l32 * XS4 + 4 * kb + 2 * g;
+    return to_bf16x8(p[0], p[1]);
+}
+
+}  // namespace
+
+template <int VARIANT, bool HAS_RS>
+__global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs a) {
+    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
+    __shared__ float term_s[kTileEnvs];
+    __shared__ __attribute__((aligned(16))) uint8_t crec[VARIANT == 1 ? kTileEnvs * CFP_CLASSIC_REC_BYTES : 16];
+
+    const int tid = threadIdx.x;
+    const unsigned lane_u = (unsigned)(tid & 63);
+    const int g = (tid & 63) >> 5;       // k group of the A/B operand, env-row group of the accumulator
+    const int l32 = tid & 31;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const unsigned loff = (unsigned)((4 * g) * CFP_HIDDEN + l32);
+    const size_t e0 = (size_t)blockIdx.x * kTileEnvs;
+    const f4* xs4 = reinterpret_cast<const f4*>(lds);
+
+    stage_tile<VARIANT>(a, e0, lds, crec, term_s, tid);
+    __syncthreads();
+
+    unsigned tmask = 0u;
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+        if (term_s[acc_row(r) + 4 * g] != 0.0f) tmask |= 1u << r;
+
+    // ---- encoder ---------------------------------------------------------------
+    if (VARIANT == 1 && a.rec) {
+        classic_encode_tile(a, crec, lds, tid);
+    } else if (VARIANT == 0 && a.rec) {
+        f16v acc[2] = {zero16(), zero16()};
+        const uint32_t* rrow = reinterpret_cast<const uint32_t*>(lds) + l32 * RS;
+        const float* frow = reinterpret_cast<const float*>(rrow) + CFP_OBS_MAP / 4;
+        const u4* wp = a.we_bf + (size_t)(wave * 2) * 64;
+        constexpr int KB_STRIDE = 4 * 2 * 64;   // u4 per K block
+        u4 b0 = wp[lane_u], b1 = (wp + 64)[lane_u];
+        uint32_t w0 = rrow[2 * g], w1 = rrow[2 * g + 1];
+#pragma unroll 1
+        for (int kb = 0; kb < kKb16Map; kb++) {
+            // block kb+1: weights, and bytes (for kb = 48 the g = 1 half reads tail
+            // bits, which block 49 below replaces by the float path)
+            const u4 n0 = (wp + (size_t)(kb + 1) * KB_STRIDE)[lane_u];
+            const u4 n1 = (wp + (size_t)(kb + 1) * KB_STRIDE + 64)[lane_u];
+            const uint32_t m0 = rrow[4 * (kb + 1) + 2 * g];
+            const uint32_t m1 = rrow[4 * (kb + 1) + 2 * g + 1];
+            const u4 av = bytes_to_bf16x8(w0, w1);
+            acc[0] = mfma16(av, b0, acc[0]);
+            acc[1] = mfma16(av, b1, acc[1]);
+            b0 = n0; b1 = n1; w0 = m0; w1 = m1;
+        }
+        // block 49: features 784..791 are map bytes (g = 0), 792..799 tail floats (g = 1)
+        {
+            const u4 n0 = (wp + (size_t)(kKb16Map + 1) * KB_STRIDE)[lane_u];
+            const u4 n1 = (wp + (size_t)(kKb16Map + 1) * KB_STRIDE + 64)[lane_u];
+            const u4 ab = bytes_to_bf16x8(w0, w1);
+            const u4 af = floats_to_bf16x8(frow);
+            const u4 av = g ? af : ab;
+            acc[0] = mfma16(av, b0, acc[0]);
+            acc[1] = mfma16(av, b1, acc[1]);
+            b0 = n0; b1 = n1;
+        }
+        // blocks 50..52: tail floats 8 + 16(kb-50) + 8g .. ; features 843..847 read as 0
+#pragma unroll
+        for (int kb = kKb16Map + 1; kb < kKb16Enc; kb++) {
+            u4 n0 = b0, n1 = b1;
+            if (kb + 1 < kKb16Enc) {
+                n0 = (wp + (size_t)(kb + 1) * KB_STRIDE)[lane_u];
+                n1 = (wp + (size_t)(kb + 1) * KB_STRIDE + 64)[lane_u];
+            }
+            const u4 av = floats_to_bf16x8(frow + 16 * kb - CFP_OBS_MAP + 8 * g);
+            acc[0] = mfma16(av, b0, acc[0]);
+            acc[1] = mfma16(av, b1, acc[1]);
+            b0 = n0; b1 = n1;
+        }
+        __syncthreads();   // every wave is done with the record bytes
+#pragma unroll
+        for (int ut = 0; ut < 2; ut++) {
+            const float bias = a.b_enc[wave * 64 + ut * 32 + l32];
+            float* xrow = lds + (4 * g) * XS + wave * 64 + ut * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) xrow[acc_row(r) * XS] = acc[ut][r] + bias;
+        }
+    }
+    __syncthreads();
+    if (a.rec && a.h_enc_out) copy_tile_out(lds, a.h_enc_out + e0 * CFP_HIDDEN, tid);
+
+    // ---- MinGRU layers ------------------------------------------------------------
+    constexpr int KB_STRIDE = 4 * 6 * 64;   // u4 per K block of the gate mirror
+#pragma unroll 1
+    for (int l = 0; l < a.layers; l++) {
+        float* st_base = a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64;
+        float st[32];
+#pragma unroll
+        for (int e = 0; e < 32; e++)
+            st[e] = __builtin_nontemporal_load(
+                (st_base + (acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32)) + loff);
+
+        f16v acc[6];
+#pragma unroll
+        for (int t = 0; t < 6; t++) acc[t] = zero16();
+        const u4* wp = a.wg_bf + ((size_t)l * kKb16Hid * 4 + wave) * 6 * 64;
+        u4 bq[2][6];
+#pragma unroll
+        for (int t = 0; t < 6; t++) bq[0][t] = (wp + t * 64)[lane_u];
+#pragma unroll
+        for (int kb = 0; kb < kKb16Hid; kb++) {
+            if (kb + 1 < kKb16Hid) {
+#pragma unroll
+                for (int t = 0; t < 6; t++)
+                    bq[(kb + 1) & 1][t] = (wp + (size_t)(kb + 1) * KB_STRIDE + t * 64)[lane_u];
+            }
+            const u4 av = a_frag(xs4, l32, g, kb);
+#pragma unroll
+            for (int t = 0; t < 6; t++) acc[t] = mfma16(av, bq[kb & 1][t], acc[t]);
+        }
+        __syncthreads();   // every wave has read the layer input
+
+        float* rs_base = HAS_RS ? a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64
+                                : nullptr;
+#pragma unroll
+        for (int e = 0; e < 32; e++) {
+            const int ut = e / 16, r = e % 16;
+            const int soff = acc_row(r) * CFP_HIDDEN + ut * 32;
+            float* xp = lds + (acc_row(r) + 4 * g) * XS + wave * 64 + ut * 32 + l32;
+            const float s = (tmask >> r) & 1u ? 0.0f : st[e];
+            if (HAS_RS) __builtin_nontemporal_store(s, (rs_base + soff) + loff);
+            const float zh = acc[0 + ut][r];
+            const float zg = acc[2 + ut][r];
+            const float zp = acc[4 + ut][r];
+            const float sg = sigmoid_fast(zg);
+            const float sh = sigmoid_fast(zh);
+            const float gh = zh >= 0.0f ? zh + 0.5f : sh;
+            const float out = s + sg * (gh - s);
+            const float p = sigmoid_fast(zp);
+            const float xv = *xp;
+            *xp = p * out + (1.0f - p) * xv;
+            __builtin_nontemporal_store(out, (st_base + soff) + loff);
+        }
+        __syncthreads();
+    }
+    if (a.layers > 0 && a.h3_out) copy_tile_out(lds, a.h3_out + e0 * CFP_HIDDEN, tid);
+
+    // ---- heads: waves 0 and 1 take one 32-row tile each over the full K -------
+    if (a.do_head && wave < 2) {
+        f16v hacc = zero16();
+        const u4* wp = a.wav_bf + (size_t)wave * 64;
+#pragma unroll
+        for (int kb = 0; kb < kKb16Hid; kb++) {
+            const u4 b = (wp + (size_t)kb * 128)[lane_u];
+            const u4 av = a_frag(xs4, l32, g, kb);
+            hacc = mfma16(av, b, hacc);
+        }
+        const int arow = wave * 32 + l32;
+        const int avs = a.actions + 1;     // 44, or 18 for the classic game
+        if (arow < avs) {
+            const float bias = arow < a.actions ? a.b_a[arow] : a.b_v[0];
+            float* av_base = a.av_out + e0 * avs;
+            const int aoff = (4 * g) * avs + arow;
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                (av_base + acc_row(r) * avs)[aoff] = hacc[r] + bias;
+        }
+    }
+}
+
+int launch_forward_bf16(const FwdArgs& a, hipStream_t st) {
+    CFP_REQUIRE(a.we_bf && a.wg_bf && a.wav_bf, "bf16 forward without bf16 weight mirrors");
+    const dim3 g(a.n / kTileEnvs), b(kFwdThreads);
+    if (a.variant == 1) {
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<1, true>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward_bf16<1, false>), g, b, 0, st, a);
+    } else {
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<0, true>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward_bf16<0, false>), g, b, 0, st, a);
+    }
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+// ---- bf16 MFMA-ordered weight mirrors ---------------------------------------------
+// One 16-byte element (eight bf16) per lane and K block: lane l carries
+// k = 16*kb + 8*(l/32) + j of column l%32 of its 32-wide tile.
+__global__ void k_pack_enc_bf16(const float* __restrict__ W_enc, __bf16* __restrict__ out,
+                                int total) {
+    int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int j = idx & 7, lane = (idx >> 3) & 63, ut = (idx >> 9) & 1, wave = (idx >> 10) & 3,
+        kb = idx >> 12;
+    int unit = wave * 64 + ut * 32 + (lane & 31);
+    int f = 16 * kb + 8 * (lane >> 5) + j;
+    out[idx] = (__bf16)(f < CFP_OBS ? W_enc[(size_t)f * CFP_HIDDEN + unit] : 0.0f);
+}
+
+__global__ void k_pack_gru_bf16(const float* __restrict__ W_gru, __bf16* __restrict__ out,
+                                int total) {
+    int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int layer = idx / (int)kGruPackFloats;
+    int i = idx - layer * (int)kGruPackFloats;
+    int j = i & 7, lane = (i >> 3) & 63, q = i >> 9;
+    int t = q % 6, wave = (q / 6) & 3, kb = q / 24;
+    int gate = t >> 1, ut = t & 1;
+    int row = gate * CFP_HIDDEN + wave * 64 + ut * 32 + (lane & 31);
+    int k = 16 * kb + 8 * (lane >> 5) + j;
+    out[idx] = (__bf16)W_gru[(size_t)layer * kGruPackFloats + (size_t)row * CFP_HIDDEN + k];
+}
+
+__global__ void k_pack_av_bf16(const float* __restrict__ W_a, const float* __restrict__ W_v,
+                               __bf16* __restrict__ out, int actions) {
+    int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int)kAvPackFloats) return;
+    int j = idx & 7, lane = (idx >> 3) & 63, nt = (idx >> 9) & 1, kb = idx >> 10;
+    int arow = nt * 32 + (lane & 31);
+    int k = 16 * kb + 8 * (lane >> 5) + j;
+    float v = 0.0f;
+    if (arow < actions) v = W_a[arow * CFP_HIDDEN + k];
+    else if (arow == actions) v = W_v[k];
+    out[idx] = (__bf16)v;
+}
+
+int launch_pack_weights_bf16(const float* params, int layers, int variant, uint16_t* we_bf,
+                             uint16_t* wg_bf, uint16_t* wav_bf, hipStream_t st) {
+    const Arena ar = arena_of(variant, layers);
+    if (variant == 0) {   // the classic encoder gathers from the unpacked fp32 W_enc
+        const int enc_total = (int)kEncPackFloats;
+        hipLaunchKernelGGL(k_pack_enc_bf16, dim3((enc_total + 255) / 256), dim3(256), 0, st,
+                           params + ar.w_enc, reinterpret_cast<__bf16*>(we_bf), enc_total);
+    }
+    const int gru_total = layers * (int)kGruPackFloats;
+    hipLaunchKernelGGL(k_pack_gru_bf16, dim3((gru_total + 255) / 256), dim3(256), 0, st,
+                       params + ar.w_gru, reinterpret_cast<__bf16*>(wg_bf), gru_total);
+    hipLaunchKernelGGL(k_pack_av_bf16, dim3(((int)kAvPackFloats + 255) / 256), dim3(256), 0, st,
+                       params + ar.w_a, params + ar.w_v, reinterpret_cast<__bf16*>(wav_bf),
+                       ar.actions);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+}  // namespace cfp

@@ -109,6 +109,15 @@ class Policy:
     def refresh_weights(self):
         _check(lib().cfp_policy_refresh_weights(self._h, _stream()))
 
+    def set_gemm_bf16(self, on=True):
+        """Run the forward entry points with bf16 GEMM inputs and fp32 accumulation
+        (the reference's CF_GEMM_BF16 mode, craftax_full.cu:11306-11316)."""
+        _check(lib().cfp_policy_set_gemm_bf16(self._h, 1 if on else 0))
+
+    @property
+    def gemm_bf16(self):
+        return bool(lib().cfp_policy_gemm_bf16(self._h))
+
     # -- forward entry points ------------------------------------------------
     def encode_step(self, rec=None, n=None):
         """records [n][996] u8 (None = the object's scratch) -> the object's h_enc."""

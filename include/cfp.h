@@ -102,6 +102,14 @@ int cfp_policy_get_params(const cfp_policy* p, float* host_params, size_t count)
  * (craftax_full.cu:11805-11817) after init / Adam. */
 int cfp_policy_refresh_weights(cfp_policy* p, void* stream);
 
+/* bf16-input / fp32-accumulate GEMMs for the forward entry points of this policy
+ * (encoder, gate and head GEMMs on bf16 MFMA; state, epilogue and outputs stay
+ * fp32).  Replaces the reference's process-wide CF_GEMM_BF16 switch
+ * (craftax_full.cu:11306-11316, bf16 wrappers :11688-11756) by a per-object
+ * flag; off by default.  Accuracy: 2e-2 relative to an fp64 evaluation. */
+int cfp_policy_set_gemm_bf16(cfp_policy* p, int on);
+int cfp_policy_gemm_bf16(const cfp_policy* p);
+
 /* Borrowed device pointers owned by the policy object. */
 float* cfp_policy_params(cfp_policy* p);    /* [param_count]                 */
 float* cfp_policy_state(cfp_policy* p);     /* live h_state [layers][n][256] */

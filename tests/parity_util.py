@@ -6,6 +6,14 @@ Tolerance (from the target statement): logits / values / hidden states within
 path (2e-2 for bf16 inputs).  "Relative" is taken per tensor against its RMS
 magnitude: |got - ref| <= tol * (|ref| + rms(ref)), so entries that cancel to
 near zero are judged against the tensor's scale rather than their own.
+
+bf16 inputs: rounding both GEMM operands to 8 significant bits perturbs every
+pre-activation by ~0.2 % of its RMS, and three recurrent layers with unit-slope
+gates carry that through, so single entries of h3 / state move by up to tens of
+percent of the RMS whatever the implementation (numpy_forward_bf16_f64 shows the
+same).  The bf16 path is therefore held to (a) 2e-2 in the relative Frobenius
+norm against the fp64 oracle and (b) the per-entry metric above, at 2e-3, against
+the fp64 evaluation of the SAME bf16-rounded operands.
 """
 import numpy as np
 
@@ -138,6 +146,52 @@ def numpy_forward_f64(params, layers, x, state, terminals, obs=None, actions=Non
     out["logits"] = h @ w["W_a"].T + w["b_a"]
     out["values"] = h @ w["W_v"] + w["b_v"][0]
     return out
+
+
+def bf16_round(a):
+    """Round to the nearest bf16 (ties to even); result as fp64."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + np.uint64(0x7FFF) + ((u >> np.uint64(16)) & np.uint64(1))) & np.uint64(0xFFFF0000)
+    return u.astype(np.uint32).view(np.float32).reshape(np.shape(a)).astype(np.float64)
+
+
+def numpy_forward_bf16_f64(params, layers, x, state, terminals, obs=None, actions=None,
+                           quantize_encoder=True):
+    """fp64 evaluation of the bf16-input forward: both operands of the encoder, gate
+    and head GEMMs are rounded to bf16 (the activations from their fp32 value),
+    products and sums are exact/fp64, everything else as numpy_forward_f64."""
+    w = {k: v.astype(np.float64)
+         for k, v in split_params(params, layers, obs, actions).items()}
+    q = bf16_round
+    f32 = lambda a: a.astype(np.float32)
+    if quantize_encoder:
+        h = q(x) @ q(w["W_enc"]) + w["b_enc"]
+    else:
+        h = x.astype(np.float64) @ w["W_enc"] + w["b_enc"]
+    out = {"h_enc": h.copy()}
+    new_state = np.empty((layers,) + h.shape, dtype=np.float64)
+    dz = (np.asarray(terminals) != 0)[:, None]
+    for l in range(layers):
+        st = np.where(dz, 0.0, state[l].astype(np.float64))
+        z = q(f32(h)) @ q(w["W_gru"][l]).T
+        zh, zg, zp = z[:, :HIDDEN], z[:, HIDDEN:2 * HIDDEN], z[:, 2 * HIDDEN:]
+        gh = np.where(zh >= 0.0, zh + 0.5, sigmoid64(zh))
+        o = st + sigmoid64(zg) * (gh - st)
+        p = sigmoid64(zp)
+        h = p * o + (1.0 - p) * h
+        new_state[l] = o
+    out["h3"] = h
+    out["state"] = new_state
+    out["logits"] = q(f32(h)) @ q(w["W_a"]).T + w["b_a"]
+    out["values"] = q(f32(h)) @ q(w["W_v"]) + w["b_v"][0]
+    return out
+
+
+def fro_err(got, ref):
+    """Relative Frobenius error ||got - ref|| / ||ref||."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    return float(np.sqrt(np.sum((got - ref) ** 2)) / (np.sqrt(np.sum(ref * ref)) + 1e-30))
 
 
 def rel_err(got, ref):
