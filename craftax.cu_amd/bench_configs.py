@@ -1,0 +1,121 @@
+"""Timings of the secondary workloads on one MI355X, one JSON line each:
+
+  forward_65536   policy forward, 65 536 envs, h256x3, one step from records
+                  (fp32 and bf16-input kernels)
+  ppo_update      PPO update, 4096 envs x 64 steps = 262 144 samples, one
+                  minibatch = all envs: windowed recompute backward + Adam
+  classic_1m      classic-game policy forward, 1 048 576 envs, 148-byte records
+
+Usage:  python craftax.cu_amd/bench_configs.py [--reps 10] [--only NAME]
+The headline workload (262 144 envs) is bench.py at the repository root."""
+import argparse
+import json
+import os
+import sys
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+PEAK_FP32 = 157.3                    # TFLOP/s, fp32 MFMA
+FWD_FLOP = 1633792                   # per env-step: encoder + 3 gate GEMMs + head
+UPD_FLOP = 4469248                   # per sample: recompute forward + backward
+CLASSIC_FLOP = 1179648 + 9216        # gate GEMMs + 18-row head (gather encoder not counted)
+
+
+def _time(torch, fn, reps, warm=2):
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def forward_65536(pkg, torch, reps):
+    n = 65536
+    pol = pkg.Policy(n, 3, seed=1)
+    rec = pkg.policy.synth_records(n, 1234, 0)
+    term = torch.zeros(n, device="cuda")
+    av = torch.empty(n, 44, device="cuda")
+    out = {"workload": "forward_65536", "envs": n}
+    for name, on in (("fp32", False), ("bf16_in", True)):
+        pol.set_gemm_bf16(on)
+        ms = _time(torch, lambda: pol.forward(rec, term, pol.state, av=av), reps)
+        out[name] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
+                     "tflops": FWD_FLOP * n / ms / 1e9,
+                     "frac_fp32_mfma_peak": FWD_FLOP * n / ms / 1e9 / PEAK_FP32}
+    pol.close()
+    return out
+
+
+def ppo_update(pkg, torch, reps):
+    n, T = 4096, 64
+    pol = pkg.Policy(n, 3, seed=1)
+    tr = pkg.Trainer(pol, T)
+    pol.state.zero_()
+    term = torch.zeros(n, device="cuda")
+    for t in range(T):
+        tr.record_step(t, pkg.policy.synth_records(n, 1234, t), term)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    tr.buf("r_act").copy_(torch.randint(0, 43, (T, n), device="cuda", generator=g, dtype=torch.int32))
+    tr.buf("r_logprob").fill_(-3.7612)          # -log 43: a uniform behaviour policy
+    tr.buf("adv").copy_(torch.randn(T, n, device="cuda", generator=g))
+    tr.buf("ret").copy_(torch.randn(T, n, device="cuda", generator=g))
+    tr.buf("r_done").zero_()
+    tr.adv_stats()
+
+    def step():
+        tr.backward(0, n)
+        tr.adam()
+    ms = _time(torch, step, reps, warm=1)
+    ms_bwd = _time(torch, lambda: tr.backward(0, n), reps, warm=1)
+    tr.adam()
+    samples = n * T
+    out = {"workload": "ppo_update", "envs": n, "T": T, "samples": samples,
+           "window": tr.window, "ms_per_update": ms, "ms_backward": ms_bwd,
+           "samples_per_s": samples / ms * 1e3,
+           "tflops": UPD_FLOP * samples / ms / 1e9,
+           "frac_fp32_mfma_peak": UPD_FLOP * samples / ms / 1e9 / PEAK_FP32}
+    assert torch.isfinite(pol.params).all()
+    tr.close()
+    pol.close()
+    return out
+
+
+def classic_1m(pkg, torch, reps):
+    n = 1 << 20
+    pol = pkg.Policy(n, 3, seed=1, variant="classic")
+    rec = pkg.policy.synth_classic_records(n, 1234, 0)
+    term = torch.zeros(n, device="cuda")
+    av = torch.empty(n, 18, device="cuda")
+    out = {"workload": "classic_1m", "envs": n}
+    for name, on in (("fp32", False), ("bf16_in", True)):
+        pol.set_gemm_bf16(on)
+        ms = _time(torch, lambda: pol.forward(rec, term, pol.state, av=av), reps)
+        out[name] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
+                     "mfma_tflops": CLASSIC_FLOP * n / ms / 1e9,
+                     "frac_fp32_mfma_peak": CLASSIC_FLOP * n / ms / 1e9 / PEAK_FP32}
+    pol.close()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=10)
+    ap.add_argument("--only", default=None)
+    args = ap.parse_args()
+    import torch
+    import __graft_entry__ as ge
+    pkg = ge.load_package()
+    assert torch.cuda.is_available(), "bench_configs.py needs a GPU"
+    for fn in (forward_65536, ppo_update, classic_1m):
+        if args.only and fn.__name__ != args.only:
+            continue
+        print(json.dumps(fn(pkg, torch, args.reps)), flush=True)
+
+
+if __name__ == "__main__":
+    main()

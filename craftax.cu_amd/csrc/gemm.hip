@@ -7,20 +7,33 @@
 // One kernel covers all four shapes: C[i][j] (+)= sum_k A(i,k) * B(k,j) with
 // element strides for both operands, so "transposes" are just strides.
 //   workgroup tile 128 x 128 x 32, 4 waves as 2 x 2, each wave 64 x 64
-//   (2 x 2 accumulators of v_mfma_f32_32x32x2_f32); operands are staged
-//   through LDS as [row][k] with a 36-float row stride so that a lane's
-//   16-byte fragment read (k = 4*(lane/32)+j of an 8-wide K block) is
-//   conflict free.  Edges are zero-filled, so M, N, K are arbitrary.
+//   (2 x 2 accumulators of v_mfma_f32_32x32x2_f32).
+//   An operand whose K dimension is the unit-stride one in memory sits in LDS as
+//   [row][k] (36-float rows) and a lane's fragment for an 8-wide K block
+//   (k = 8b + 4*(lane/32) + j) is one 16-byte read; an operand whose row
+//   dimension is unit-stride sits as [k][row] (132-float rows) and the fragment
+//   is four 4-byte reads (two ds_read2).  Either way global loads and LDS
+//   writes are 16 bytes per lane and coalesced -- nothing is transposed on
+//   the way in.  The next K tile is fetched into registers while the current
+//   one is multiplied.  Edges are zero-filled, so M, N, K are arbitrary;
+//   operands whose base or leading dimension is not 16-byte aligned take a
+//   scalar-load path of the same kernel.
+//   Workgroup ids are remapped so that consecutive tiles (which share an A
+//   tile) run on the same XCD and meet in its L2.
 // dW = dpre^T x has K = window columns (>= 16k) and a small output, so K is
-// split over grid.z into a workspace and summed in a fixed order by a second
+// split over grid.y into a workspace and summed in a fixed order by a second
 // kernel: run-to-run bitwise stable, unlike float atomics.
 #include "cfp_common.h"
 
 namespace cfp {
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 32, LDT = BK + 4;
+constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int LDK = BK + 4;    // [row][k] layout: floats per row
+constexpr int LDR = BM + 4;    // [k][row] layout: floats per k
+constexpr int OPER_FLOATS = BM * LDK > BK * LDR ? BM * LDK : BK * LDR;
 constexpr int GEMM_THREADS = 256;
+constexpr int kXcds = 8;
 
 struct GemmArgs {
     const float* A; long sa_i, sa_k;   // A(i,k) = A[i*sa_i + k*sa_k]
@@ -29,55 +42,84 @@ struct GemmArgs {
     long c_split;
     int M, N, K;
     int k_per_split;                   // multiple of BK
+    int mt, nt;                        // tile counts
 };
 
-// Stage a [128 rows][32 k] operand tile into LDS [row][k].  `kfast` says k is
-// the unit-stride dimension in memory; lanes walk the unit-stride dimension so
-// every wave-wide load covers whole 128-byte segments.
-template <bool KFAST>
-__device__ __forceinline__ void stage(float* lds, const float* src, long s_row,
-                                      long s_k, int row0, int nrows, int k0,
-                                      int kend, int tid) {
-    if (KFAST) {
-        const int kk = tid & 31;
-        const int r0 = tid >> 5;
-        const int k = k0 + kk;
-        const bool kin = k < kend;
+// Fetch this thread's share (4 x 16 bytes) of a [128 rows][32 k] operand tile.
+// KFAST: k is unit-stride in memory; thread covers (row = v/8, k = 4*(v%8)..+3).
+// else : row is unit-stride;        thread covers (k = v/32, row = 4*(v%32)..+3).
+// VEC loads 16 bytes at once (the host checked alignment and that reading up to
+// the next multiple of four along the unit-stride dimension stays inside the
+// leading dimension); elements past the extent are zeroed either way.
+template <bool KFAST, bool VEC>
+__device__ __forceinline__ void fetch(f4 (&r)[4], const float* src, long s_row, long s_k,
+                                      int row0, int nrows, int k0, int kend, int tid) {
 #pragma unroll
-        for (int it = 0; it < BM / 8; it++) {
-            const int r = r0 + 8 * it;
-            const int row = row0 + r;
-            float v = 0.0f;
-            if (kin && row < nrows) v = src[(long)row * s_row + (long)k * s_k];
-            lds[r * LDT + kk] = v;
-        }
-    } else {
-        const int r = tid & 127;
-        const int kq = tid >> 7;
-        const int row = row0 + r;
-        const bool rin = row < nrows;
+    for (int it = 0; it < 4; it++) {
+        const int v = tid + GEMM_THREADS * it;
+        int row, k;
+        if (KFAST) { row = row0 + (v >> 3); k = k0 + 4 * (v & 7); }
+        else { k = k0 + (v >> 5); row = row0 + 4 * (v & 31); }
+        f4 val = {0.0f, 0.0f, 0.0f, 0.0f};
+        const int lim = KFAST ? kend - k : nrows - row;   // valid elements along the fast dim
+        const bool in = KFAST ? row < nrows : k < kend;
+        if (in && lim > 0) {
+            const float* p = src + (long)row * s_row + (long)k * s_k;
+            if (VEC) {
+                val = *reinterpret_cast<const f4*>(p);
+                if (lim < 4) {
 #pragma unroll
-        for (int it = 0; it < BK / 2; it++) {
-            const int kk = kq + 2 * it;
-            const int k = k0 + kk;
-            float v = 0.0f;
-            if (rin && k < kend) v = src[(long)row * s_row + (long)k * s_k];
-            lds[r * LDT + kk] = v;
+                    for (int c = 1; c < 4; c++)
+                        if (c >= lim) val[c] = 0.0f;
+                }
+            } else {
+                const long step = KFAST ? s_k : s_row;
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    if (c < lim) val[c] = p[c * step];
+            }
         }
+        r[it] = val;
     }
 }
 
-template <bool A_KFAST, bool B_KFAST, bool ACCUM>
+template <bool KFAST>
+__device__ __forceinline__ void stash(float* lds, const f4 (&r)[4], int tid) {
+    f4* l4 = reinterpret_cast<f4*>(lds);
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int v = tid + GEMM_THREADS * it;
+        if (KFAST) l4[(v >> 3) * (LDK / 4) + (v & 7)] = r[it];
+        else l4[(v >> 5) * (LDR / 4) + (v & 31)] = r[it];
+    }
+}
+
+// fragment of K block kb for the 32 rows starting at rb: k = 8*kb + 4*half + j
+template <bool KFAST>
+__device__ __forceinline__ f4 frag(const float* lds, int rb, int l32, int half, int kb) {
+    if (KFAST)
+        return reinterpret_cast<const f4*>(lds)[(rb + l32) * (LDK / 4) + 2 * kb + half];
+    const float* p = lds + (8 * kb + 4 * half) * LDR + rb + l32;
+    f4 r = {p[0], p[LDR], p[2 * LDR], p[3 * LDR]};
+    return r;
+}
+
+template <bool A_KFAST, bool B_KFAST, bool ACCUM, bool VEC_A, bool VEC_B>
 __global__ __launch_bounds__(GEMM_THREADS) void k_gemm(GemmArgs g) {
-    __shared__ __attribute__((aligned(16))) float As[BM * LDT];
-    __shared__ __attribute__((aligned(16))) float Bs[BN * LDT];
+    __shared__ __attribute__((aligned(16))) float As[OPER_FLOATS];
+    __shared__ __attribute__((aligned(16))) float Bs[OPER_FLOATS];
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
-    const int i0 = blockIdx.x * BM;
-    const int j0 = blockIdx.y * BN;
-    const int kbeg = blockIdx.z * g.k_per_split;
+    // XCD-aware tile id: hardware deals workgroups to the XCDs round-robin
+    const int total = g.mt * g.nt;
+    const int chunk = (total + kXcds - 1) / kXcds;
+    const int tile = (int)(blockIdx.x % kXcds) * chunk + (int)(blockIdx.x / kXcds);
+    if (tile >= total) return;
+    const int i0 = (tile / g.nt) * BM;
+    const int j0 = (tile % g.nt) * BN;
+    const int kbeg = blockIdx.y * g.k_per_split;
     const int kend = min(g.K, kbeg + g.k_per_split);
 
     f16v acc[2][2];
@@ -88,21 +130,25 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm(GemmArgs g) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
 
-    const f4* As4 = reinterpret_cast<const f4*>(As);
-    const f4* Bs4 = reinterpret_cast<const f4*>(Bs);
+    f4 ra[4], rb[4];
+    fetch<A_KFAST, VEC_A>(ra, g.A, g.sa_i, g.sa_k, i0, g.M, kbeg, kend, tid);
+    fetch<B_KFAST, VEC_B>(rb, g.B, g.sb_j, g.sb_k, j0, g.N, kbeg, kend, tid);
     for (int k0 = kbeg; k0 < kend; k0 += BK) {
-        stage<A_KFAST>(As, g.A, g.sa_i, g.sa_k, i0, g.M, k0, kend, tid);
-        stage<B_KFAST>(Bs, g.B, g.sb_j, g.sb_k, j0, g.N, k0, kend, tid);
+        __syncthreads();   // the previous tile has been read
+        stash<A_KFAST>(As, ra, tid);
+        stash<B_KFAST>(Bs, rb, tid);
         __syncthreads();
+        if (k0 + BK < kend) {
+            fetch<A_KFAST, VEC_A>(ra, g.A, g.sa_i, g.sa_k, i0, g.M, k0 + BK, kend, tid);
+            fetch<B_KFAST, VEC_B>(rb, g.B, g.sb_j, g.sb_k, j0, g.N, k0 + BK, kend, tid);
+        }
 #pragma unroll
         for (int kb = 0; kb < BK / 8; kb++) {
             f4 af[2], bf[2];
 #pragma unroll
-            for (int a = 0; a < 2; a++)
-                af[a] = As4[(wm * 64 + a * 32 + l32) * (LDT / 4) + 2 * kb + half];
+            for (int a = 0; a < 2; a++) af[a] = frag<A_KFAST>(As, wm * 64 + a * 32, l32, half, kb);
 #pragma unroll
-            for (int b = 0; b < 2; b++)
-                bf[b] = Bs4[(wn * 64 + b * 32 + l32) * (LDT / 4) + 2 * kb + half];
+            for (int b = 0; b < 2; b++) bf[b] = frag<B_KFAST>(Bs, wn * 64 + b * 32, l32, half, kb);
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
@@ -112,10 +158,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm(GemmArgs g) {
                         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(
                             af[a][j], bf[b][j], acc[a][b], 0, 0, 0);
         }
-        __syncthreads();
     }
 
-    float* C = g.C + (long)blockIdx.z * g.c_split;
+    float* C = g.C + (long)blockIdx.y * g.c_split;
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -145,36 +190,59 @@ __global__ void k_splitk_reduce(float* __restrict__ dst,
     dst[i] += s;
 }
 
-// dWv[k] += sum_c x[c][k] * dv[c]: one workgroup per 64 units, 4 waves stride
-// the columns, fixed-order LDS reduction.
-__global__ __launch_bounds__(256) void k_gemv_dwv(const float* __restrict__ x,
-                                                  const float* __restrict__ dv,
-                                                  float* __restrict__ dWv,
-                                                  int cols) {
-    __shared__ float red[4][64];
-    const int k = blockIdx.x * 64 + (threadIdx.x & 63);
-    const int w = threadIdx.x >> 6;
-    float s = 0.0f;
-    for (int c = w; c < cols; c += 4)
-        s = fmaf(x[(size_t)c * CFP_HIDDEN + k], dv[c], s);
-    red[w][threadIdx.x & 63] = s;
-    __syncthreads();
-    if (w == 0)
-        dWv[k] += (red[0][threadIdx.x] + red[1][threadIdx.x]) +
-                  (red[2][threadIdx.x] + red[3][threadIdx.x]);
+// dWv[k] += sum_c x[c][k] * dv[c].  Stage 1: workgroup z owns a contiguous slice
+// of columns, thread k walks it (each column is one coalesced 1 KiB row of x)
+// and leaves part[z][k]; stage 2 is k_splitk_reduce, slices in ascending order,
+// so the sum is run-to-run bitwise stable.
+constexpr int kGemvSlices = 1024;
+__global__ __launch_bounds__(256) void k_gemv_dwv_partial(const float* __restrict__ x,
+                                                          const float* __restrict__ dv,
+                                                          float* __restrict__ part, int cols,
+                                                          int cols_per_slice) {
+    const int c0 = blockIdx.x * cols_per_slice;
+    const int c1 = min(cols, c0 + cols_per_slice);
+    const int k = threadIdx.x;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    int c = c0;
+    for (; c + 4 <= c1; c += 4) {
+        s0 = fmaf(x[(size_t)c * CFP_HIDDEN + k], dv[c], s0);
+        s1 = fmaf(x[(size_t)(c + 1) * CFP_HIDDEN + k], dv[c + 1], s1);
+        s2 = fmaf(x[(size_t)(c + 2) * CFP_HIDDEN + k], dv[c + 2], s2);
+        s3 = fmaf(x[(size_t)(c + 3) * CFP_HIDDEN + k], dv[c + 3], s3);
+    }
+    for (; c < c1; c++) s0 = fmaf(x[(size_t)c * CFP_HIDDEN + k], dv[c], s0);
+    part[(size_t)blockIdx.x * CFP_HIDDEN + k] = (s0 + s1) + (s2 + s3);
+}
+
+// 16-byte loads need an aligned base, a leading dimension that is a multiple
+// of four floats and room to read up to the next multiple of four along the
+// unit-stride dimension.
+static bool vec_ok(const float* p, long ld, int fast_extent) {
+    return (reinterpret_cast<uintptr_t>(p) & 15u) == 0 && ld % 4 == 0 &&
+           ld >= (long)((fast_extent + 3) / 4 * 4);
+}
+
+template <bool A_KFAST, bool B_KFAST, bool ACCUM>
+int launch_gemm(const GemmArgs& g, dim3 grid, bool va, bool vb, hipStream_t st) {
+    const dim3 blk(GEMM_THREADS);
+    if (va && vb) hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, ACCUM, true, true>), grid, blk, 0, st, g);
+    else if (va) hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, ACCUM, true, false>), grid, blk, 0, st, g);
+    else if (vb) hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, ACCUM, false, true>), grid, blk, 0, st, g);
+    else hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, ACCUM, false, false>), grid, blk, 0, st, g);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
 }
 
 template <bool A_KFAST, bool B_KFAST>
 int run_gemm(GemmArgs g, int splits, bool accum, hipStream_t st) {
-    dim3 grid((g.M + BM - 1) / BM, (g.N + BN - 1) / BN, splits);
-    if (accum)
-        hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, true>), grid,
-                           dim3(GEMM_THREADS), 0, st, g);
-    else
-        hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, false>), grid,
-                           dim3(GEMM_THREADS), 0, st, g);
-    CFP_HIP_TRY(hipGetLastError());
-    return 0;
+    g.mt = (g.M + BM - 1) / BM;
+    g.nt = (g.N + BN - 1) / BN;
+    const int total = g.mt * g.nt;
+    const dim3 grid((total + kXcds - 1) / kXcds * kXcds, splits);
+    const bool va = A_KFAST ? vec_ok(g.A, g.sa_i, g.K) : vec_ok(g.A, g.sa_k, g.M);
+    const bool vb = B_KFAST ? vec_ok(g.B, g.sb_j, g.K) : vec_ok(g.B, g.sb_k, g.N);
+    if (accum) return launch_gemm<A_KFAST, B_KFAST, true>(g, grid, va, vb, st);
+    return launch_gemm<A_KFAST, B_KFAST, false>(g, grid, va, vb, st);
 }
 
 // Split-K workspace for cfp_gemm_dw: allocated once per process on first use
@@ -183,6 +251,7 @@ int run_gemm(GemmArgs g, int splits, bool accum, hipStream_t st) {
 constexpr int kMaxSplits = 64;
 constexpr size_t kDwWorkFloats = (size_t)kMaxSplits * CFP_OBS * CFP_HIDDEN;
 float* g_dw_work = nullptr;
+float* g_gemv_work = nullptr;   // [kGemvSlices][256], same life cycle
 
 }  // namespace
 }  // namespace cfp
@@ -269,8 +338,17 @@ int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
 int cfp_gemv_dwv(const float* d_x, const float* d_dv, float* d_dWv, int cols,
                  void* stream) {
     CFP_REQUIRE(cols > 0 && d_x && d_dv && d_dWv, "cfp_gemv_dwv: bad argument");
-    hipLaunchKernelGGL(k_gemv_dwv, dim3(CFP_HIDDEN / 64), dim3(256), 0,
-                       (hipStream_t)stream, d_x, d_dv, d_dWv, cols);
+    hipStream_t st = (hipStream_t)stream;
+    if (!g_gemv_work)
+        CFP_HIP_TRY(hipMalloc((void**)&g_gemv_work,
+                              (size_t)kGemvSlices * CFP_HIDDEN * sizeof(float)));
+    int per = (cols + kGemvSlices - 1) / kGemvSlices;
+    if (per < 32) per = 32;
+    const int slices = (cols + per - 1) / per;
+    hipLaunchKernelGGL(k_gemv_dwv_partial, dim3(slices), dim3(256), 0, st, d_x, d_dv,
+                       g_gemv_work, cols, per);
+    hipLaunchKernelGGL(k_splitk_reduce, dim3(1), dim3(256), 0, st, d_dWv, g_gemv_work,
+                       (long)CFP_HIDDEN, (long)CFP_HIDDEN, slices);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }

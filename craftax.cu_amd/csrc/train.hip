@@ -376,7 +376,7 @@ struct cfp_trainer {
     float* av_tmp = nullptr;   // [n][44]
 };
 
-static constexpr int kColsumSlices = 64;
+static constexpr int kColsumSlices = 1024;
 
 extern "C" {
 
