@@ -88,6 +88,16 @@ int launch_pack_weights_bf16(const float* params, int layers, int variant, uint1
 int launch_pack_weights(const float* params, int layers, int variant, float* we_pk,
                         float* wg_pk, float* wav_pk, hipStream_t st);
 
+// Library-internal forms of the dense-math seam with explicit leading dimensions
+// (the trainer keeps its feature matrix 848 floats wide so that rows stay
+// 16-byte aligned); the C ABI entry points call these with the tight widths.
+int launch_expand_obs(const uint8_t* r_obs, float* xobs, int t0, int count, int mb, int n,
+                      int env_start, int ld, hipStream_t st);
+int gemm_enc_fwd_ld(int cols, const float* W_enc, const float* xobs, int ldx, float* h,
+                    hipStream_t st);
+int gemm_dw_ld(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
+               hipStream_t st);
+
 // per-variant arena geometry
 struct Arena {
     int obs, actions;

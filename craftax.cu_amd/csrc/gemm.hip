@@ -194,7 +194,7 @@ __global__ void k_splitk_reduce(float* __restrict__ dst,
 // of columns, thread k walks it (each column is one coalesced 1 KiB row of x)
 // and leaves part[z][k]; stage 2 is k_splitk_reduce, slices in ascending order,
 // so the sum is run-to-run bitwise stable.
-constexpr int kGemvSlices = 1024;
+constexpr int kGemvSlices = 256;
 __global__ __launch_bounds__(256) void k_gemv_dwv_partial(const float* __restrict__ x,
                                                           const float* __restrict__ dv,
                                                           float* __restrict__ part, int cols,
@@ -258,52 +258,26 @@ float* g_gemv_work = nullptr;   // [kGemvSlices][256], same life cycle
 
 using namespace cfp;
 
-extern "C" {
+namespace cfp {
 
-int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
-                 float* d_y, void* stream) {
-    CFP_REQUIRE(m > 0 && cols > 0 && k > 0 && d_W && d_x && d_y,
-                "cfp_gemm_fwd: bad argument");
-    GemmArgs g{};
-    g.A = d_x; g.sa_i = k; g.sa_k = 1;
-    g.B = d_W; g.sb_k = 1; g.sb_j = k;
-    g.C = d_y; g.ldc = m; g.c_split = 0;
-    g.M = cols; g.N = m; g.K = k;
-    g.k_per_split = (k + BK - 1) / BK * BK;
-    return run_gemm<true, true>(g, 1, false, (hipStream_t)stream);
-}
-
-int cfp_gemm_enc_fwd(int cols, const float* d_W_enc, const float* d_xobs,
-                     float* d_h, void* stream) {
-    CFP_REQUIRE(cols > 0 && d_W_enc && d_xobs && d_h,
+int gemm_enc_fwd_ld(int cols, const float* d_W_enc, const float* d_xobs, int ldx, float* d_h,
+                    hipStream_t st) {
+    CFP_REQUIRE(cols > 0 && d_W_enc && d_xobs && d_h && ldx >= CFP_OBS,
                 "cfp_gemm_enc_fwd: bad argument");
     GemmArgs g{};
-    g.A = d_xobs; g.sa_i = CFP_OBS; g.sa_k = 1;
+    g.A = d_xobs; g.sa_i = ldx; g.sa_k = 1;
     g.B = d_W_enc; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
     g.C = d_h; g.ldc = CFP_HIDDEN; g.c_split = 0;
     g.M = cols; g.N = CFP_HIDDEN; g.K = CFP_OBS;
     g.k_per_split = (CFP_OBS + BK - 1) / BK * BK;
-    return run_gemm<true, false>(g, 1, false, (hipStream_t)stream);
+    return run_gemm<true, false>(g, 1, false, st);
 }
 
-int cfp_gemm_dh(int m3, int cols, const float* d_W, const float* d_dpre,
-                float* d_dh, void* stream) {
-    CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh,
-                "cfp_gemm_dh: bad argument");
-    GemmArgs g{};
-    g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
-    g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
-    g.C = d_dh; g.ldc = CFP_HIDDEN; g.c_split = 0;
-    g.M = cols; g.N = CFP_HIDDEN; g.K = m3;
-    g.k_per_split = (m3 + BK - 1) / BK * BK;
-    return run_gemm<true, false>(g, 1, false, (hipStream_t)stream);
-}
-
-int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
-                float* d_dW, void* stream) {
-    CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW,
+int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld_dpre,
+               float* d_dW, hipStream_t st) {
+    CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW &&
+                    ld_dpre >= rows,
                 "cfp_gemm_dw: bad argument (rows must be in 1..%d)", CFP_OBS);
-    hipStream_t st = (hipStream_t)stream;
     // enough workgroups to fill 256 CUs: tiles(M) * tiles(N=2) * splits
     const int tiles = ((rows + BM - 1) / BM) * (CFP_HIDDEN / BN);
     int splits = (1024 + tiles - 1) / tiles;
@@ -314,7 +288,7 @@ int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
     const int k_per_split = ((kblocks + splits - 1) / splits) * BK;
     splits = (cols + k_per_split - 1) / k_per_split;
     GemmArgs g{};
-    g.A = d_dpre; g.sa_i = 1; g.sa_k = rows;
+    g.A = d_dpre; g.sa_i = 1; g.sa_k = ld_dpre;
     g.B = d_x; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
     g.ldc = CFP_HIDDEN;
     g.M = rows; g.N = CFP_HIDDEN; g.K = cols;
@@ -333,6 +307,46 @@ int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
                        dim3(256), 0, st, d_dW, g_dw_work, count, count, splits);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
+}
+
+}  // namespace cfp
+
+extern "C" {
+
+int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
+                 float* d_y, void* stream) {
+    CFP_REQUIRE(m > 0 && cols > 0 && k > 0 && d_W && d_x && d_y,
+                "cfp_gemm_fwd: bad argument");
+    GemmArgs g{};
+    g.A = d_x; g.sa_i = k; g.sa_k = 1;
+    g.B = d_W; g.sb_k = 1; g.sb_j = k;
+    g.C = d_y; g.ldc = m; g.c_split = 0;
+    g.M = cols; g.N = m; g.K = k;
+    g.k_per_split = (k + BK - 1) / BK * BK;
+    return run_gemm<true, true>(g, 1, false, (hipStream_t)stream);
+}
+
+int cfp_gemm_enc_fwd(int cols, const float* d_W_enc, const float* d_xobs,
+                     float* d_h, void* stream) {
+    return gemm_enc_fwd_ld(cols, d_W_enc, d_xobs, CFP_OBS, d_h, (hipStream_t)stream);
+}
+
+int cfp_gemm_dh(int m3, int cols, const float* d_W, const float* d_dpre,
+                float* d_dh, void* stream) {
+    CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh,
+                "cfp_gemm_dh: bad argument");
+    GemmArgs g{};
+    g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
+    g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
+    g.C = d_dh; g.ldc = CFP_HIDDEN; g.c_split = 0;
+    g.M = cols; g.N = CFP_HIDDEN; g.K = m3;
+    g.k_per_split = (m3 + BK - 1) / BK * BK;
+    return run_gemm<true, false>(g, 1, false, (hipStream_t)stream);
+}
+
+int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
+                float* d_dW, void* stream) {
+    return gemm_dw_ld(rows, cols, d_x, d_dpre, rows, d_dW, (hipStream_t)stream);
 }
 
 int cfp_gemv_dwv(const float* d_x, const float* d_dv, float* d_dWv, int cols,

@@ -167,11 +167,12 @@ __global__ __launch_bounds__(256) void k_record_obs(
 
 __global__ void k_expand_obs(const uint8_t* __restrict__ r_obs,
                              float* __restrict__ xobs, int t0, size_t total,
-                             int mb, int n, int env_start) {
+                             int mb, int n, int env_start, int ld) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
-    const int f = (int)(idx % CFP_OBS);
-    const size_t w = idx / CFP_OBS;
+    const int f = (int)(idx % (size_t)ld);
+    const size_t w = idx / (size_t)ld;
+    if (f >= CFP_OBS) { xobs[idx] = 0.0f; return; }   // padding of a widened row
     const size_t t = (size_t)t0 + w / (size_t)mb;
     const size_t el = w % (size_t)mb;
     const uint8_t* rec = r_obs + (t * (size_t)n + env_start + el) * CFP_REC_BYTES;
@@ -224,6 +225,17 @@ __global__ void k_mingru_epi_fwd(const float* __restrict__ pre,
 
 using namespace cfp;
 
+namespace cfp {
+int launch_expand_obs(const uint8_t* r_obs, float* xobs, int t0, int count, int mb, int n,
+                      int env_start, int ld, hipStream_t st) {
+    const size_t total = (size_t)count * ld;
+    hipLaunchKernelGGL(k_expand_obs, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       r_obs, xobs, t0, total, mb, n, env_start, ld);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+}  // namespace cfp
+
 extern "C" {
 
 int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
@@ -251,12 +263,8 @@ int cfp_expand_obs(const uint8_t* d_r_obs, float* d_xobs, int t0, int count,
                 "cfp_expand_obs: bad argument");
     CFP_REQUIRE((reinterpret_cast<uintptr_t>(d_r_obs) & 3u) == 0,
                 "records must be 4-byte aligned");
-    const size_t total = (size_t)count * CFP_OBS;
-    hipLaunchKernelGGL(k_expand_obs, dim3((unsigned)((total + 255) / 256)),
-                       dim3(256), 0, (hipStream_t)stream, d_r_obs, d_xobs, t0,
-                       total, mb, n, env_start);
-    CFP_HIP_TRY(hipGetLastError());
-    return 0;
+    return launch_expand_obs(d_r_obs, d_xobs, t0, count, mb, n, env_start, CFP_OBS,
+                             (hipStream_t)stream);
 }
 
 int cfp_add_bias(float* d_h, const float* d_b, int cols, void* stream) {

@@ -134,14 +134,26 @@ __global__ __launch_bounds__(128) void k_head_bwd_win(
     if (threadIdx.x < 3) block_loss[3 * blockIdx.x + threadIdx.x] = s_l[threadIdx.x][0];
 }
 
-// loss_acc[q] += sum_b block_loss[3b+q], ascending b, one thread per q.
-__global__ void k_loss_fold(const double* __restrict__ block_loss, int blocks,
-                            double* __restrict__ loss_acc) {
-    const int q = threadIdx.x;
-    if (q >= 3) return;
-    double s = 0.0;
-    for (int b = 0; b < blocks; b++) s += block_loss[3 * b + q];
-    loss_acc[q] += s;
+// loss_acc[q] += sum_b block_loss[3b+q].  Fixed order: thread (q, c) of 3 x 64 sums
+// the blocks of chunk c in ascending order, then thread (q, 0) adds the 64 chunk
+// sums in ascending order.
+__global__ __launch_bounds__(256) void k_loss_fold(const double* __restrict__ block_loss,
+                                                   int blocks, double* __restrict__ loss_acc) {
+    __shared__ double red[3][64];
+    const int q = threadIdx.x >> 6, c = threadIdx.x & 63;
+    if (q < 3) {
+        const int per = (blocks + 63) / 64;
+        const int b1 = min(blocks, (c + 1) * per);
+        double s = 0.0;
+        for (int b = c * per; b < b1; b++) s += block_loss[3 * b + q];
+        red[q][c] = s;
+    }
+    __syncthreads();
+    if (q < 3 && c == 0) {
+        double s = 0.0;
+        for (int i = 0; i < 64; i++) s += red[q][i];
+        loss_acc[q] += s;
+    }
 }
 
 __global__ void k_add_dv_wv(float* __restrict__ dh, const float* __restrict__ dv,
@@ -169,13 +181,27 @@ __global__ __launch_bounds__(256) void k_colsum_partial(
     for (int c = c0; c < c1; c++) s += src[(size_t)c * rows + r];
     part[(size_t)blockIdx.x * rows + r] = s;
 }
-__global__ void k_colsum_fold(const float* __restrict__ part, float* __restrict__ out,
-                              int rows, int slices) {
-    const int r = blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= rows) return;
+// Fixed order: thread (row, c) of 4 x 64 sums the slices of chunk c in ascending
+// order, thread (row, 0) then adds the 64 chunk sums in ascending order.
+__global__ __launch_bounds__(256) void k_colsum_fold(const float* __restrict__ part,
+                                                     float* __restrict__ out, int rows,
+                                                     int slices) {
+    __shared__ float red[4][64];
+    const int rl = threadIdx.x >> 6, c = threadIdx.x & 63;
+    const int r = blockIdx.x * 4 + rl;
+    const int per = (slices + 63) / 64;
     float s = 0.0f;
-    for (int z = 0; z < slices; z++) s += part[(size_t)z * rows + r];
-    out[r] += s;
+    if (r < rows) {
+        const int z1 = min(slices, (c + 1) * per);
+        for (int z = c * per; z < z1; z++) s += part[(size_t)z * rows + r];
+    }
+    red[rl][c] = s;
+    __syncthreads();
+    if (c == 0 && r < rows) {
+        float t = 0.0f;
+        for (int i = 0; i < 64; i++) t += red[rl][i];
+        out[r] += t;
+    }
 }
 
 // Reverse MinGRU over one window: thread per (unit, env), t descending, live
@@ -450,7 +476,7 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     TA(adam_ctr, sizeof(uint64_t));
     TA(d_lr, sizeof(float));
     TA(d_ent, sizeof(float));
-    TA(xobs, cc * CFP_OBS * sizeof(float));
+    TA(xobs, cc * kObsPad * sizeof(float));   // rows widened 843 -> 848: 16-byte aligned
     for (int l = 0; l <= tr->L; l++) TA(x[l], cc * H * sizeof(float));
     for (int l = 0; l < tr->L; l++) TA(preb[l], cc * G * sizeof(float));
     for (int l = 0; l < tr->L; l++) TA(dcarry[l], (size_t)mb * H * sizeof(float));
@@ -551,7 +577,7 @@ static int colsum_into(cfp_trainer* tr, const float* src, float* out, int rows, 
     slices = (cols + per - 1) / per;
     hipLaunchKernelGGL(k_colsum_partial, dim3(slices, (rows + 255) / 256), dim3(256), 0,
                        st, src, tr->colsum_part, rows, cols, per);
-    hipLaunchKernelGGL(k_colsum_fold, dim3((rows + 255) / 256), dim3(256), 0, st,
+    hipLaunchKernelGGL(k_colsum_fold, dim3((rows + 3) / 4), dim3(256), 0, st,
                        tr->colsum_part, out, rows, slices);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
@@ -586,8 +612,9 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         const int cols = Tw * mb;
         const size_t hc = (size_t)H * cols;
         // ---- forward recompute of the window into tight columns
-        if (cfp_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, stream)) return 1;
-        if (cfp_gemm_enc_fwd(cols, W_enc, tr->xobs, tr->x[0], stream)) return 1;
+        if (launch_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, kObsPad, st))
+            return 1;
+        if (gemm_enc_fwd_ld(cols, W_enc, tr->xobs, kObsPad, tr->x[0], st)) return 1;
         if (cfp_add_bias(tr->x[0], b_enc, cols, stream)) return 1;
         for (int l = 0; l < L; l++) {
             if (cfp_gemm_fwd(G, cols, H, W_gru + (size_t)l * G * H, tr->x[l], tr->preb[l],
@@ -605,7 +632,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
                            tr->adv + env_start, tr->ret + env_start, tr->stats, tr->dlogits,
                            tr->dvalue, tr->block_loss, t0, cols, mb, n, n, T, tr->cfg.clip,
                            tr->cfg.vf, tr->d_ent);
-        hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(64), 0, st, tr->block_loss, hb,
+        hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(256), 0, st, tr->block_loss, hb,
                            tr->loss_acc);
         if (cfp_gemm_dh(A, cols, W_a, tr->dlogits, tr->dh3b, stream)) return 1;
         hipLaunchKernelGGL(k_add_dv_wv, dim3(grid1(hc)), dim3(256), 0, st, tr->dh3b,
@@ -633,7 +660,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         // ---- encoder: dh_enc = dhG + highway; db_enc; dW_enc += xobs^T dh_enc
         hipLaunchKernelGGL(k_vadd, dim3(grid1(hc)), dim3(256), 0, st, tr->dhG, tr->dhX, hc);
         if (colsum_into(tr, tr->dhG, g + CFP_OFF_B_ENC, H, cols, st)) return 1;
-        if (cfp_gemm_dw(CFP_OBS, cols, tr->dhG, tr->xobs, g + CFP_OFF_W_ENC, stream)) return 1;
+        if (gemm_dw_ld(CFP_OBS, cols, tr->dhG, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, st)) return 1;
     }
     CFP_HIP_TRY(hipGetLastError());
     return 0;
@@ -683,7 +710,7 @@ int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream) {
         hipLaunchKernelGGL(k_loss_accum, dim3(hb), dim3(128), 0, st, tr->av_tmp, tr->r_act,
                            tr->r_logprob, tr->adv, tr->ret, tr->stats, tr->block_loss, t, n,
                            T, tr->cfg.clip);
-        hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(64), 0, st, tr->block_loss, hb,
+        hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(256), 0, st, tr->block_loss, hb,
                            tr->loss_acc);
     }
     CFP_HIP_TRY(hipGetLastError());
