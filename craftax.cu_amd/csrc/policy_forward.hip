@@ -44,6 +44,8 @@ namespace cfp {
 namespace {
 
 constexpr int kRedFloats = 2 * 16 * 64;               // head K-half partials
+// classic encoder tables: [21 chunks][64 envs][4] gather words + [64 envs][24] scalars
+constexpr int kClassicTabDwords = 21 * 64 * 4 + 64 * 24;
 constexpr int kEncPairs = kKbEnc / 2;                 // 53 steps of two K blocks
 constexpr int kMapPairs = kKbMap / 2;                 // 49 all-map steps (blocks 0..97)
 __device__ __forceinline__ f16v mfma(float a, float b, f16v c) {
@@ -185,6 +187,160 @@ __device__ __forceinline__ void encoder_gemm(const FwdArgs& a, const float* ldsX
     enc_tail_step<52>(acc, wp, fx, fy, b1, b0, cur, L);
 }
 
+// ---- classic-game encoder for a pair of tiles (64 envs) ----------------------------
+// encode_obs_kernel (craftax_classic.cu:1714-1751): the observation is one-hot per
+// view cell, so h0 = b_enc + the sum of the W_enc rows the record selects.  Thread
+// k owns hidden unit k and keeps the 64 envs' sums in registers.  W_enc (1.38 MB)
+// is walked once per pair in chunks of three cells (63 rows, 63 KiB) staged in
+// the LDS that later holds the x tiles, the next chunk travelling through
+// registers meanwhile; every gather is then one conflict-free LDS read of a row
+// that all lanes share.  `tab[chunk][env]` holds the byte offsets of the three
+// block rows inside the chunk and the cells' mob bits; row reads run several envs
+// ahead of their adds.  Mob bits are rare and take a wave-uniform branch.
+// Summation order per env: bias, then per chunk the three block rows followed by
+// that chunk's mob rows (cell, bit ascending), then the 22 scalar features.
+__device__ __forceinline__ void classic_encode_pair(const FwdArgs& a, const uint8_t* crecX,
+                                                    const uint8_t* crecY, float* wbuf,
+                                                    uint32_t* tab, float* xsX, float* xsY,
+                                                    int tid) {
+    constexpr int CELLS = 63, CH = 21, NBLK = 17, CHUNK_CELLS = 3;
+    constexpr int CHUNKS = CELLS / CHUNK_CELLS;                 // 21
+    constexpr int CHUNK_V4 = CHUNK_CELLS * CH * CFP_HIDDEN / 4;  // 4032 16-byte pieces
+    constexpr int PF = (CHUNK_V4 + kFwdThreads - 1) / kFwdThreads;   // 16 per thread
+    constexpr int NSCAL = CFP_CLASSIC_OBS - CELLS * CH;         // 22 scalar features
+    constexpr int ENVS = 2 * kTileEnvs;
+    static_assert(CHUNK_CELLS * CH * CFP_HIDDEN <= 2 * LDS_FLOATS, "chunk must fit the x tiles");
+    constexpr int SVS = 24;                                     // floats per env row of `sv`
+    static_assert(CHUNKS * ENVS * 4 + ENVS * SVS <= kClassicTabDwords, "table storage");
+    // the 22 scalar features of every env as fp32, 16-byte aligned rows
+    float* sv = reinterpret_cast<float*>(tab + CHUNKS * ENVS * 4);
+
+    // tab[chunk][env] = {byte offset of the block row of cell 0, 1, 2 inside the
+    // chunk buffer, the three cells' mob bits (4 each)}
+    for (int i = tid; i < CHUNKS * ENVS; i += kFwdThreads) {
+        const int c = i / ENVS, e = i - c * ENVS;
+        const uint8_t* o = (e < kTileEnvs ? crecX : crecY) + (e % kTileEnvs) * CFP_CLASSIC_REC_BYTES;
+        u4 w;
+        uint32_t m = 0;
+        uint32_t off[CHUNK_CELLS];
+#pragma unroll
+        for (int q = 0; q < CHUNK_CELLS; q++) {
+            const int cell = c * CHUNK_CELLS + q;
+            off[q] = (uint32_t)(q * CH + (int8_t)o[cell]) * (CFP_HIDDEN * 4);
+            m |= (o[CELLS + cell] & 15u) << (4 * q);
+        }
+        w.x = off[0]; w.y = off[1]; w.z = off[2]; w.w = m;
+        reinterpret_cast<u4*>(tab)[i] = w;
+    }
+    for (int i = tid; i < ENVS * SVS; i += kFwdThreads) {
+        const int e = i / SVS, f = i - e * SVS;
+        const uint8_t* o = (e < kTileEnvs ? crecX : crecY) +
+                           (e % kTileEnvs) * CFP_CLASSIC_REC_BYTES + 2 * CELLS;
+        float v = 0.0f;
+        if (f < 16) v = (float)(int8_t)o[f] / 10.0f;                  // inventory, intrinsics
+        else if (f < 20) v = (int8_t)o[16] == f - 15 ? 1.0f : 0.0f;   // direction 1..4
+        else if (f == 20) v = *reinterpret_cast<const float*>(o + 18);   // light
+        else if (f == 21) v = o[17] ? 1.0f : 0.0f;                    // sleeping
+        sv[i] = v;
+    }
+    float acc[ENVS];
+    const float bias = a.b_enc[tid];
+#pragma unroll
+    for (int e = 0; e < ENVS; e++) acc[e] = bias;
+
+    const f4* W4 = reinterpret_cast<const f4*>(a.w_enc);
+    f4* wbuf4 = reinterpret_cast<f4*>(wbuf);
+    const float* wk = wbuf + tid;
+    f4 pf[PF];
+#pragma unroll
+    for (int i = 0; i < PF; i++) {
+        const int v = tid + kFwdThreads * i;
+        pf[i] = v < CHUNK_V4 ? W4[v] : f4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+#pragma unroll 1
+    for (int c = 0; c <= CHUNKS; c++) {
+        __syncthreads();   // the previous chunk (and the tables) complete / consumed
+#pragma unroll
+        for (int i = 0; i < PF; i++) {
+            const int v = tid + kFwdThreads * i;
+            if (v < CHUNK_V4) wbuf4[v] = pf[i];
+        }
+        __syncthreads();
+        if (c < CHUNKS) {
+            // next: cells 3(c+1).., or for c+1 == CHUNKS the 22 scalar-feature rows
+            const size_t base = (size_t)(c + 1) * CHUNK_V4;
+            const int limit = c + 1 < CHUNKS ? CHUNK_V4 : NSCAL * CFP_HIDDEN / 4;
+#pragma unroll
+            for (int i = 0; i < PF; i++) {
+                const int v = tid + kFwdThreads * i;
+                if (v < limit) pf[i] = W4[base + v];
+            }
+            // Software pipeline over the envs: while env e is added, the three row
+            // reads of envs e+1 .. e+3 and the table words of env e+4 are in flight
+            // (the LDS counter tracks fifteen operations).
+            const u4* t4 = reinterpret_cast<const u4*>(tab) + c * ENVS;
+            const char* wkb = reinterpret_cast<const char*>(wk);
+            constexpr int DEPTH = 4;
+            u4 wq[DEPTH + 1];
+            float r[DEPTH][CHUNK_CELLS];
+            uint32_t mm[DEPTH];
+            auto issue = [&](int slot, const u4& w) {
+                r[slot][0] = *reinterpret_cast<const float*>(wkb + w.x);
+                r[slot][1] = *reinterpret_cast<const float*>(wkb + w.y);
+                r[slot][2] = *reinterpret_cast<const float*>(wkb + w.z);
+                mm[slot] = w.w;
+            };
+#pragma unroll
+            for (int e = 0; e < DEPTH; e++) wq[e] = t4[e];
+#pragma unroll
+            for (int e = 0; e < DEPTH - 1; e++) issue(e, wq[e]);
+#pragma unroll
+            for (int e = 0; e < ENVS; e++) {
+                if (e + DEPTH < ENVS) wq[(e + DEPTH) % (DEPTH + 1)] = t4[e + DEPTH];
+                if (e + DEPTH - 1 < ENVS)
+                    issue((e + DEPTH - 1) % DEPTH, wq[(e + DEPTH - 1) % (DEPTH + 1)]);
+                __builtin_amdgcn_sched_barrier(0);
+                acc[e] += r[e % DEPTH][0];
+                acc[e] += r[e % DEPTH][1];
+                acc[e] += r[e % DEPTH][2];
+                // rare: mob bits of this env's three cells (wave-uniform branch)
+                const uint32_t m = __builtin_amdgcn_readfirstlane(mm[e % DEPTH]);
+                if (m) {
+#pragma unroll
+                    for (int q = 0; q < CHUNK_CELLS; q++)
+#pragma unroll
+                        for (int j = 0; j < 4; j++)
+                            if (m & (1u << (4 * q + j)))
+                                acc[e] += wk[(q * CH + NBLK + j) * CFP_HIDDEN];
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            // 16 inventory / intrinsic scalars, direction one-hot, light, sleeping
+            float wv[NSCAL];
+#pragma unroll
+            for (int f = 0; f < NSCAL; f++) wv[f] = wk[f * CFP_HIDDEN];
+#pragma unroll
+            for (int e = 0; e < ENVS; e++) {
+                const f4* r4 = reinterpret_cast<const f4*>(sv + e * SVS);
+                float hv = acc[e];
+#pragma unroll
+                for (int f4i = 0; f4i < (NSCAL + 3) / 4; f4i++) {
+                    const f4 x = r4[f4i];
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (4 * f4i + j < NSCAL) hv = fmaf(x[j], wv[4 * f4i + j], hv);
+                }
+                acc[e] = hv;
+            }
+        }
+    }
+    __syncthreads();   // the weight chunk buffer becomes the x tiles
+#pragma unroll
+    for (int e = 0; e < ENVS; e++)
+        (e < kTileEnvs ? xsX : xsY)[(e % kTileEnvs) * XS + tid] = acc[e];
+}
+
 // ---- MinGRU phases ---------------------------------------------------------------
 // Written-to-nowhere tile: state / r_state addresses of a pair's missing second
 // tile point here, so the hot loop needs no predication.
@@ -304,6 +460,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float red_all[2][kRedFloats];
     __shared__ float term_all[2][kTileEnvs];
     __shared__ __attribute__((aligned(16))) uint8_t crec_all[2][kTileEnvs * CFP_CLASSIC_REC_BYTES];
+    __shared__ __attribute__((aligned(16))) uint32_t ctab[VARIANT == 1 ? kClassicTabDwords : 4];
 
     const int tiles = a.n / kTileEnvs;
     const int pairs = (tiles + 1) / 2;
@@ -351,8 +508,9 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
 
         // ---- encoders ----------------------------------------------------------
         if (classic) {
-#pragma unroll 1
-            for (int s = 0; s < 2; s++) classic_encode_tile(a, crec_all[s], lds_all[s], tid);
+            classic_encode_pair(a, crec_all[0], crec_all[1], &lds_all[0][0],
+                                ctab, lds_all[0],
+                                lds_all[1], tid);
         } else if (full_rec) {
             f16v eacc[4];
 #pragma unroll
