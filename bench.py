@@ -30,9 +30,10 @@ BYTES_PER_ENV_STEP = 996 + 4 + 3 * 256 * 4 * 2 + 44 * 4                # 7 320
 PEAK_FP32_MFMA_TFLOPS = 157.3
 LAYERS = 3
 # HBM bytes per launch at 262 144 envs from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/policy_forward_262144_pmc.txt), scaled by the copy-kernel factor
-# stated in DESIGN.md; None until measured for another size.
-MEASURED_TRAFFIC_BYTES = {262144: 1957465984}
+# (profiles/policy_forward_262144_pmc.txt), scaled by the factors the same counters
+# show for a plain 1 GiB copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0); None until
+# measured for another size.
+MEASURED_TRAFFIC_BYTES = {262144: 2052732928}
 
 
 def parse():
