@@ -36,13 +36,6 @@ __device__ __forceinline__ f16v mfma16(const u4& a, const u4& b, f16v c) {
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-__device__ __forceinline__ f16v zero16() {
-    f16v z;
-#pragma unroll
-    for (int i = 0; i < 16; i++) z[i] = 0.0f;
-    return z;
-}
-
 // eight fp32 -> eight bf16, round to nearest even
 __device__ __forceinline__ u4 to_bf16x8(const f4& lo, const f4& hi) {
     f8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};

@@ -126,5 +126,146 @@ struct Lane {
     unsigned loff;     // lane offset (floats) into a [32][256] state tile row set
 };
 
+constexpr int kEncPairs = kKbEnc / 2;                 // 53 steps of two K blocks
+constexpr int kMapPairs = kKbMap / 2;                 // 49 all-map steps (blocks 0..97)
+__device__ __forceinline__ f16v mfma(float a, float b, f16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f16v zero16() {
+    f16v z;
+#pragma unroll
+    for (int i = 0; i < 16; i++) z[i] = 0.0f;
+    return z;
+}
+
+// ---- encoder GEMM of both tiles of a pair: K = 848 as 53 steps of two 8-wide K
+// blocks.  The weight fragments of a step feed both tiles (4 accumulators), so
+// the mirror is streamed once per pair.  Weights sit three steps deep in
+// registers; the step loop is unrolled by three so that the ring needs no moves
+// (a register rotation would make every iteration wait for ALL loads in flight).
+struct EncB { f4 b[4]; };   // (block 0|1) x (unit tile 0|1)
+
+__device__ __forceinline__ EncB enc_load_b(const f4* wp, int step, unsigned lane_u) {
+    constexpr int KB_STRIDE = 4 * 2 * 64;   // f4 per K block
+    EncB r;
+    const f4* p = wp + (size_t)(2 * step) * KB_STRIDE;
+    r.b[0] = (p)[lane_u];
+    r.b[1] = (p + 64)[lane_u];
+    r.b[2] = (p + KB_STRIDE)[lane_u];
+    r.b[3] = (p + KB_STRIDE + 64)[lane_u];
+    return r;
+}
+
+__device__ __forceinline__ void enc_mma(f16v (&acc)[4], const float (&x)[8],
+                                        const float (&y)[8], const EncB& w) {
+#pragma unroll
+    for (int q = 0; q < 2; q++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc[0] = mfma(x[4 * q + j], w.b[2 * q][j], acc[0]);
+            acc[1] = mfma(x[4 * q + j], w.b[2 * q + 1][j], acc[1]);
+            acc[2] = mfma(y[4 * q + j], w.b[2 * q][j], acc[2]);
+            acc[3] = mfma(y[4 * q + j], w.b[2 * q + 1][j], acc[3]);
+        }
+}
+
+__device__ __forceinline__ void bytes_to_f(uint32_t w, float* x) {
+    x[0] = (float)(w & 0xffu);
+    x[1] = (float)((w >> 8) & 0xffu);
+    x[2] = (float)((w >> 16) & 0xffu);
+    x[3] = (float)(w >> 24);
+}
+
+struct EncBytes { uint32_t x0, x1, y0, y1; };
+
+__device__ __forceinline__ EncBytes enc_bytes(const uint32_t* rx, const uint32_t* ry,
+                                              int step, int half) {
+    EncBytes r;
+    r.x0 = rx[4 * step + half];
+    r.x1 = rx[4 * step + 2 + half];
+    r.y0 = ry[4 * step + half];
+    r.y1 = ry[4 * step + 2 + half];
+    return r;
+}
+
+// One all-map step: request the weights of step p+2 and the bytes of step p+1,
+// then the 32 MFMAs of step p.
+__device__ __forceinline__ void enc_map_step(f16v (&acc)[4], const f4* wp, const uint32_t* rx,
+                                             const uint32_t* ry, int p, const EncB& use,
+                                             EncB& fill, EncBytes& cur, const Lane& L) {
+    fill = enc_load_b(wp, p + 2, L.lane_u);
+    const EncBytes nxt = enc_bytes(rx, ry, p + 1, L.half);
+    float x[8], y[8];
+    bytes_to_f(cur.x0, x);
+    bytes_to_f(cur.x1, x + 4);
+    bytes_to_f(cur.y0, y);
+    bytes_to_f(cur.y1, y + 4);
+    enc_mma(acc, x, y, use);
+    // one weight load per eight MFMAs, the LDS reads and conversions in between
+#pragma unroll
+    for (int q = 0; q < 32; q++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (q % 8 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        if (q % 8 == 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        if (q < 16) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    cur = nxt;
+}
+
+// Steps 49..52: map block 98 + tail block 0, then tail blocks 1..6 (fp32 features).
+template <int P>
+__device__ __forceinline__ void enc_tail_step(f16v (&acc)[4], const f4* wp, const float* fx,
+                                              const float* fy, const EncB& use, EncB& fill,
+                                              const EncBytes& cur, const Lane& L) {
+    if (P + 2 < kEncPairs) fill = enc_load_b(wp, P + 2, L.lane_u);
+    float x[8], y[8];
+    if (P == kMapPairs) {
+        bytes_to_f(cur.x0, x);
+        bytes_to_f(cur.y0, y);
+#pragma unroll
+        for (int j = 0; j < 4; j++) { x[4 + j] = fx[j]; y[4 + j] = fy[j]; }
+    } else {
+        constexpr int kt = 2 * (P - kMapPairs) - 1;   // first tail block of the step
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            x[j] = fx[8 * kt + j];
+            x[4 + j] = fx[8 * (kt + 1) + j];
+            y[j] = fy[8 * kt + j];
+            y[4 + j] = fy[8 * (kt + 1) + j];
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    enc_mma(acc, x, y, use);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+__device__ __forceinline__ void encoder_gemm(const FwdArgs& a, const float* ldsX,
+                                             const float* ldsY, const Lane& L,
+                                             f16v (&acc)[4]) {
+    static_assert(kMapPairs == 49 && kEncPairs == 53, "step schedule below assumes 49 + 4");
+    const uint32_t* rx = reinterpret_cast<const uint32_t*>(ldsX) + L.l32 * RS;
+    const uint32_t* ry = reinterpret_cast<const uint32_t*>(ldsY) + L.l32 * RS;
+    const float* fx = reinterpret_cast<const float*>(rx) + (CFP_OBS_MAP / 4) + 4 * L.half;
+    const float* fy = reinterpret_cast<const float*>(ry) + (CFP_OBS_MAP / 4) + 4 * L.half;
+    const f4* wp = a.we_pk + (size_t)(L.wave * 2) * 64;
+    EncB b0 = enc_load_b(wp, 0, L.lane_u), b1 = enc_load_b(wp, 1, L.lane_u), b2;
+    EncBytes cur = enc_bytes(rx, ry, 0, L.half);
+#pragma unroll 1
+    for (int p = 0; p < 48; p += 3) {
+        enc_map_step(acc, wp, rx, ry, p, b0, b2, cur, L);
+        enc_map_step(acc, wp, rx, ry, p + 1, b1, b0, cur, L);
+        enc_map_step(acc, wp, rx, ry, p + 2, b2, b1, cur, L);
+    }
+    // step 48 is the last all-map step; its "next bytes" are map block 98 plus
+    // the first tail dword, which step 49 re-reads as a float
+    enc_map_step(acc, wp, rx, ry, 48, b0, b2, cur, L);
+    enc_tail_step<49>(acc, wp, fx, fy, b1, b0, cur, L);
+    enc_tail_step<50>(acc, wp, fx, fy, b2, b1, cur, L);
+    enc_tail_step<51>(acc, wp, fx, fy, b0, b2, cur, L);
+    enc_tail_step<52>(acc, wp, fx, fy, b1, b0, cur, L);
+}
+
 }  // namespace
 }  // namespace cfp
