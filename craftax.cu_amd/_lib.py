@@ -60,6 +60,10 @@ PROTOTYPES = {
     "cfp_train_window": (C.c_int, [vp]),
     "cfp_train_minibatch": (C.c_int, [vp]),
     "cfp_train_record_step": (C.c_int, [vp, C.c_int, vp, vp, vp]),
+    "cfp_rollout_step": (C.c_int, [vp, C.c_int, vp, vp, C.c_uint64, vp, vp]),
+    "cfp_train_bootstrap": (C.c_int, [vp, vp, vp, vp]),
+    "cfp_value_sample": (C.c_int, [vp, C.c_int, C.c_int, vp, vp, vp, vp, C.c_uint64, vp, vp]),
+    "cfp_record_rd": (C.c_int, [vp, vp, vp, vp, C.c_int, vp]),
     "cfp_train_gae": (C.c_int, [vp]*2),
     "cfp_train_adv_stats": (C.c_int, [vp]*2),
     "cfp_train_backward": (C.c_int, [vp, C.c_int, C.c_int, vp]),
@@ -81,7 +85,7 @@ class PpoConfig(C.Structure):
 
 BUF = {name: i for i, name in enumerate(
     ["r_obs", "r_state", "r_act", "r_logprob", "r_value", "r_reward", "r_done", "adv",
-     "ret", "v_boot", "stats", "loss_acc", "grads", "adam_m", "adam_v", "lr", "ent"])}
+     "ret", "v_boot", "stats", "loss_acc", "grads", "adam_m", "adam_v", "lr", "ent", "step_ctr"])}
 
 
 class CfpError(RuntimeError):

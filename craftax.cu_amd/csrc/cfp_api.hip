@@ -22,20 +22,6 @@ void set_error(const char* fmt, ...) {
     va_end(ap);
 }
 
-// Counter-based generator shared with the host-side test utilities:
-// value(seed, stream, index) is a splitmix64 finalizer of a linear counter.
-__host__ __device__ inline uint64_t mix64(uint64_t seed, uint64_t stream,
-                                          uint64_t index) {
-    uint64_t z = seed + stream * 0xD1B54A32D192ED03ULL +
-                 (index + 1) * 0x9E3779B97F4A7C15ULL;
-    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
-    z = (z ^ (z >> 27)) * 0x94D049BB133111EBULL;
-    return z ^ (z >> 31);
-}
-__host__ __device__ inline float unit24(uint64_t z) {
-    return (float)(z >> 40) * (1.0f / 16777216.0f);
-}
-
 }  // namespace cfp
 
 

@@ -1,0 +1,88 @@
+// Rollout-side kernels of the policy path: categorical sampling from the fused
+// head's outputs and reward/done extraction into the rollout slabs.
+//
+// Reference: k_value_sample (craftax_full.cu:9714-9741) with
+// cf_nn_sample_action (:9147-9165), k_record_rd (:9758-9767).  The reference
+// draws its uniform from cuRAND Philox (seed ^ 0xA5A5..., subsequence = env,
+// offset = device step counter); that stream cannot be reproduced without CUDA,
+// so the uniform here comes from this library's own counter generator with the
+// same three inputs: unit24(mix64(seed ^ 0xA5A5A5A5A5A5A5A5, step, env)).  Given
+// the uniform, the action and its log-probability follow the reference's
+// arithmetic exactly (max-shifted expf, ascending cumulative sum, first index
+// with target <= cum, last action as the fall-through).
+#include "cfp_common.h"
+
+namespace cfp {
+namespace {
+
+constexpr int kMaxActions = 64;
+
+__global__ void k_value_sample(const float* __restrict__ av, int avs, int actions,
+                               float* __restrict__ env_actions, int32_t* __restrict__ act,
+                               float* __restrict__ logprobs, float* __restrict__ values, int n,
+                               uint64_t seed, const uint64_t* __restrict__ step_ctr) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    const float* lp = av + (size_t)e * avs;
+    if (values) values[e] = lp[actions];
+    float m = lp[0];
+    for (int a = 1; a < actions; a++) m = fmaxf(m, lp[a]);
+    float p[kMaxActions], total = 0.0f;
+    for (int a = 0; a < actions; a++) {
+        p[a] = expf(lp[a] - m);
+        total += p[a];
+    }
+    const uint64_t step = step_ctr ? *step_ctr : 0;
+    const float u = unit24(mix64(seed ^ 0xA5A5A5A5A5A5A5A5ULL, step, (uint64_t)e));
+    const float target = u * total;
+    float cum = 0.0f;
+    int action = actions - 1;
+    for (int a = 0; a < actions; a++) {
+        cum += p[a];
+        if (target <= cum) { action = a; break; }
+    }
+    if (env_actions) env_actions[e] = (float)action;
+    act[e] = action;
+    logprobs[e] = lp[action] - m - logf(total);
+}
+
+__global__ void k_record_rd(const float* __restrict__ rewards, const float* __restrict__ terminals,
+                            float* __restrict__ r_reward_row, uint8_t* __restrict__ r_done_row,
+                            int n) {
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= n) return;
+    r_reward_row[e] = rewards[e];
+    r_done_row[e] = terminals[e] != 0.0f ? 1 : 0;
+}
+
+}  // namespace
+}  // namespace cfp
+
+using namespace cfp;
+
+extern "C" {
+
+int cfp_value_sample(const float* d_av, int n, int actions, float* d_env_actions,
+                     int32_t* d_actions, float* d_logprobs, float* d_values, uint64_t seed,
+                     const uint64_t* d_step_ctr, void* stream) {
+    CFP_REQUIRE(d_av && d_actions && d_logprobs && n > 0, "cfp_value_sample: bad argument");
+    CFP_REQUIRE(actions > 0 && actions <= kMaxActions, "cfp_value_sample: actions must be in 1..%d",
+                kMaxActions);
+    hipLaunchKernelGGL(k_value_sample, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       d_av, actions + 1, actions, d_env_actions, d_actions, d_logprobs, d_values,
+                       n, seed, d_step_ctr);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int cfp_record_rd(const float* d_rewards, const float* d_terminals, float* d_r_reward_row,
+                  uint8_t* d_r_done_row, int n, void* stream) {
+    CFP_REQUIRE(d_rewards && d_terminals && d_r_reward_row && d_r_done_row && n > 0,
+                "cfp_record_rd: bad argument");
+    hipLaunchKernelGGL(k_record_rd, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       d_rewards, d_terminals, d_r_reward_row, d_r_done_row, n);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+}  // extern "C"

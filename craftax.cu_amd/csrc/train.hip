@@ -390,6 +390,8 @@ struct cfp_trainer {
     double *stats = nullptr, *loss_acc = nullptr, *block_loss = nullptr, *stats_part = nullptr;
     float *grads = nullptr, *adam_m = nullptr, *adam_v = nullptr;
     uint64_t* adam_ctr = nullptr;
+    uint64_t* step_ctr = nullptr;   // rollout steps taken (the sampler's offset), device side
+    float* boot_state = nullptr;    // [L][n][256] copy of the live state for the bootstrap value
     float *d_lr = nullptr, *d_ent = nullptr;
     // window workspace
     float* xobs = nullptr; float* x[CFP_MAX_LAYERS + 1] = {}; float* preb[CFP_MAX_LAYERS] = {};
@@ -474,6 +476,8 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     TA(adam_m, pc * sizeof(float));
     TA(adam_v, pc * sizeof(float));
     TA(adam_ctr, sizeof(uint64_t));
+    TA(step_ctr, sizeof(uint64_t));
+    TA(boot_state, (size_t)tr->L * hn * sizeof(float));
     TA(d_lr, sizeof(float));
     TA(d_ent, sizeof(float));
     TA(xobs, cc * kObsPad * sizeof(float));   // rows widened 843 -> 848: 16-byte aligned
@@ -522,6 +526,7 @@ void* cfp_train_buffer(cfp_trainer* tr, int which) {
         case CFP_BUF_ADAM_V: return tr->adam_v;
         case CFP_BUF_LR: return tr->d_lr;
         case CFP_BUF_ENT: return tr->d_ent;
+        case CFP_BUF_STEP_CTR: return tr->step_ctr;
         default: return nullptr;
     }
 }
@@ -545,6 +550,45 @@ int cfp_train_record_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
         return 1;
     hipLaunchKernelGGL(k_take_value, dim3(grid1(n)), dim3(256), 0, st, tr->p->logits,
                        tr->r_value + (size_t)t * n, tr->n);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int cfp_rollout_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
+                     const float* d_prev_terminals, uint64_t seed, float* d_env_actions,
+                     void* stream) {
+    CFP_REQUIRE(tr && d_rec_row, "cfp_rollout_step: NULL argument");
+    CFP_REQUIRE(t >= 0 && t < tr->T, "step %d outside the horizon %d", t, tr->T);
+    hipStream_t st = (hipStream_t)stream;
+    const size_t n = tr->n, hn = (size_t)H * n, o = (size_t)t * n;
+    uint8_t* row = tr->r_obs + o * CFP_REC_BYTES;
+    if (d_rec_row != row)
+        CFP_HIP_TRY(hipMemcpyAsync(row, d_rec_row, n * CFP_REC_BYTES, hipMemcpyDeviceToDevice,
+                                   st));
+    if (cfp_policy_forward(tr->p, row, d_prev_terminals, nullptr, tr->r_state + o * tr->L * H,
+                           nullptr, nullptr, nullptr, tr->n, 0, stream) != 0)
+        return 1;
+    if (cfp_value_sample(tr->p->logits, tr->n, A, d_env_actions, tr->r_act + o, tr->r_logprob + o,
+                         tr->r_value + o, seed, tr->step_ctr, stream) != 0)
+        return 1;
+    hipLaunchKernelGGL(k_bump_ctr, dim3(1), dim3(1), 0, st, tr->step_ctr);
+    CFP_HIP_TRY(hipGetLastError());
+    (void)hn;
+    return 0;
+}
+
+int cfp_train_bootstrap(cfp_trainer* tr, const uint8_t* d_rec_row, const float* d_terminals,
+                        void* stream) {
+    CFP_REQUIRE(tr && d_rec_row, "cfp_train_bootstrap: NULL argument");
+    hipStream_t st = (hipStream_t)stream;
+    const size_t n = tr->n, hn = (size_t)H * n;
+    CFP_HIP_TRY(hipMemcpyAsync(tr->boot_state, tr->p->h_state, (size_t)tr->L * hn * sizeof(float),
+                               hipMemcpyDeviceToDevice, st));
+    if (cfp_policy_forward(tr->p, d_rec_row, d_terminals, tr->boot_state, nullptr, nullptr,
+                           nullptr, tr->av_tmp, tr->n, 0, stream) != 0)
+        return 1;
+    hipLaunchKernelGGL(k_take_value, dim3(grid1(n)), dim3(256), 0, st, tr->av_tmp, tr->v_boot,
+                       tr->n);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }

@@ -219,13 +219,22 @@ class Trainer:
             "grads": ((self.policy.param_count,), "<f4"),
             "adam_m": ((self.policy.param_count,), "<f4"),
             "adam_v": ((self.policy.param_count,), "<f4"), "lr": ((1,), "<f4"),
-            "ent": ((1,), "<f4"),
+            "ent": ((1,), "<f4"), "step_ctr": ((1,), "<i8"),
         }
         shape, ts = shapes[name]
         return _wrap(lib().cfp_train_buffer(self._h, _lib.BUF[name]), shape, ts)
 
     def record_step(self, t, rec, terminals):
         _check(lib().cfp_train_record_step(self._h, t, _ptr(rec), _ptr(terminals), _stream()))
+
+    def rollout_step(self, t, rec, prev_terminals, seed, env_actions=None):
+        """Policy half of cu_rollout_step: forward + sample into the slab rows of step t."""
+        _check(lib().cfp_rollout_step(self._h, t, _ptr(rec), _ptr(prev_terminals), seed,
+                                      _ptr(env_actions), _stream()))
+
+    def bootstrap(self, rec, terminals):
+        """V(s_T) on a copy of the live state -> v_boot."""
+        _check(lib().cfp_train_bootstrap(self._h, _ptr(rec), _ptr(terminals), _stream()))
 
     def gae(self):
         _check(lib().cfp_train_gae(self._h, _stream()))
@@ -341,6 +350,22 @@ def record_obs(scalars_u8, maps, item_maps, light_maps, n, env_stride, level_str
                                 _ptr(light_maps), env_stride, level_stride, _ptr(rec),
                                 n, _stream()))
     return rec
+
+
+def value_sample(av, seed, step_ctr=None, env_actions=None):
+    """k_value_sample (:9714): av [n][A+1] -> (actions i32[n], logprobs f32[n], values f32[n])."""
+    n, w = av.shape
+    act = torch.empty(n, dtype=torch.int32, device=av.device)
+    lp = torch.empty(n, dtype=torch.float32, device=av.device)
+    val = torch.empty(n, dtype=torch.float32, device=av.device)
+    _check(lib().cfp_value_sample(_ptr(av), n, w - 1, _ptr(env_actions), _ptr(act), _ptr(lp),
+                                  _ptr(val), seed, _ptr(step_ctr), _stream()))
+    return act, lp, val
+
+
+def record_rd(rewards, terminals, r_reward_row, r_done_row):
+    _check(lib().cfp_record_rd(_ptr(rewards), _ptr(terminals), _ptr(r_reward_row),
+                               _ptr(r_done_row), rewards.shape[0], _stream()))
 
 
 def synth_classic_records(n, seed, step, rec=None, device="cuda"):

@@ -219,6 +219,23 @@ int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
                    size_t env_stride, size_t level_stride, uint8_t* d_rec_row,
                    int n, void* stream);
 
+/* k_value_sample (craftax_full.cu:9714-9741) on the fused head's output
+ * av[n][actions+1] (biases already added): values[e] = av[e][actions] (d_values
+ * may be NULL), action ~ softmax(av[e][0..actions)) by inversion of the cumulative
+ * sum (cf_nn_sample_action :9147-9165), logprob = log softmax at the action; the
+ * action also goes to d_env_actions[e] as a float when that is not NULL (the
+ * reference's env action slot).  The uniform is
+ * unit24(mix64(seed ^ 0xA5A5A5A5A5A5A5A5, *d_step_ctr or 0, e)) -- this library's
+ * counter generator in place of the reference's cuRAND Philox stream, which
+ * cannot be reproduced without CUDA. */
+int cfp_value_sample(const float* d_av, int n, int actions, float* d_env_actions,
+                     int32_t* d_actions, float* d_logprobs, float* d_values, uint64_t seed,
+                     const uint64_t* d_step_ctr, void* stream);
+/* k_record_rd (craftax_full.cu:9758-9767): this step's rewards and terminals into
+ * the rollout slab rows. */
+int cfp_record_rd(const float* d_rewards, const float* d_terminals, float* d_r_reward_row,
+                  uint8_t* d_r_done_row, int n, void* stream);
+
 /* ---- PPO update: replaces CuTrain (craftax_full.cu:12688-12761) ----------- */
 typedef struct cfp_trainer cfp_trainer;
 
@@ -249,7 +266,7 @@ enum cfp_train_buf {
     CFP_BUF_R_VALUE, CFP_BUF_R_REWARD, CFP_BUF_R_DONE, CFP_BUF_ADV, CFP_BUF_RET,
     CFP_BUF_V_BOOT, CFP_BUF_STATS /* double[2] */, CFP_BUF_LOSS_ACC /* double[3] */,
     CFP_BUF_GRADS, CFP_BUF_ADAM_M, CFP_BUF_ADAM_V, CFP_BUF_LR /* float */,
-    CFP_BUF_ENT /* float */
+    CFP_BUF_ENT /* float */, CFP_BUF_STEP_CTR /* uint64: rollout steps taken */
 };
 /* Borrowed device pointer to one of the trainer's buffers (NULL if unknown). */
 void* cfp_train_buffer(cfp_trainer* tr, int which);
@@ -263,6 +280,20 @@ int cfp_train_minibatch(const cfp_trainer* tr);
  * env step are the caller's. */
 int cfp_train_record_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
                           const float* d_terminals, void* stream);
+/* Policy half of cu_rollout_step (craftax_full.cu:12022-12044): as
+ * cfp_train_record_step, then samples an action per env from the logits
+ * (cfp_value_sample with the trainer's device step counter as the sampler
+ * offset) into r_act[t] / r_logprob[t] / r_value[t] and, when d_env_actions is
+ * not NULL, into the env's float action slots; the step counter is then bumped
+ * on the device (k_bump_ctr :9770), so a captured graph replays with fresh draws. */
+int cfp_rollout_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
+                     const float* d_prev_terminals, uint64_t seed, float* d_env_actions,
+                     void* stream);
+/* Bootstrap value of cu_train_collect (craftax_full.cu:12996-13006): V(s_T) from
+ * the post-rollout records on a COPY of the policy's live state (which is left
+ * untouched), into v_boot. */
+int cfp_train_bootstrap(cfp_trainer* tr, const uint8_t* d_rec_row, const float* d_terminals,
+                        void* stream);
 /* k_gae + k_adv_stats of cu_train_collect (craftax_full.cu:13007-13011). */
 int cfp_train_gae(cfp_trainer* tr, void* stream);
 /* k_adv_stats alone (when adv was filled by the caller). */

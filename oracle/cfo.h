@@ -16,6 +16,8 @@
  *   cfo_backward_f64        pinned: central finite differences of cfo_loss_f64
  *                           (the reference's own gradcheck method,
  *                           craftax_full.cu:13854-13907) and closed forms
+ *   cfo_sample_action       pinned: closed forms (equal logits, dominant logit,
+ *                           normalisation of exp(logprob))
  *   The reference's cuRAND Philox streams (weight init, action sampling) are
  *   "parity unpinned": they cannot be reproduced without CUDA and are not
  *   restated here.
@@ -75,6 +77,12 @@ void cfo_forward_f32(const float* params, int layers, int n,
                      const uint8_t* rec /*[n][996]*/, float* state /*[L][n][256]*/,
                      const float* prev_terminals, float* av /*[n][44]*/,
                      int threads);
+
+/* cf_nn_sample_action (craftax_full.cu:9147-9165) for a given uniform u; pinned
+ * by closed forms (equal logits -> floor(u*A), dominant logit, exp(logprob) sums
+ * to one) -- the reference's Philox uniform itself is not restated. */
+int cfo_sample_action(const float* logits, int actions, float u, float* logprob);
+float cfo_sample_margin(const float* logits, int actions, float u);
 
 int cfo_max_threads(void);
 

@@ -201,3 +201,46 @@ void cfo_forward_f32(const float* params, int layers, int n, const uint8_t* rec,
         ave[A] = v;
     }
 }
+
+/* cf_nn_sample_action (craftax_full.cu:9147-9165): max-shifted expf, ascending
+ * cumulative sum, first action with u*total <= cum, last action as the
+ * fall-through; logprob = log softmax at the action.  fp32 like the reference. */
+int cfo_sample_action(const float* logits, int actions, float u, float* logprob) {
+    float m = logits[0];
+    for (int a = 1; a < actions; a++) m = fmaxf(m, logits[a]);
+    float p[64], total = 0.0f;
+    for (int a = 0; a < actions; a++) {
+        p[a] = expf(logits[a] - m);
+        total += p[a];
+    }
+    const float target = u * total;
+    float cum = 0.0f;
+    int action = actions - 1;
+    for (int a = 0; a < actions; a++) {
+        cum += p[a];
+        if (target <= cum) { action = a; break; }
+    }
+    if (logprob) *logprob = logits[action] - m - logf(total);
+    return action;
+}
+
+/* Distance of u*total from the nearest cumulative-sum boundary, relative to
+ * total: draws this close to a boundary may legitimately land on either side
+ * when expf differs by an ulp between implementations. */
+float cfo_sample_margin(const float* logits, int actions, float u) {
+    float m = logits[0];
+    for (int a = 1; a < actions; a++) m = fmaxf(m, logits[a]);
+    float p[64], total = 0.0f;
+    for (int a = 0; a < actions; a++) {
+        p[a] = expf(logits[a] - m);
+        total += p[a];
+    }
+    const float target = u * total;
+    float cum = 0.0f, best = 1e30f;
+    for (int a = 0; a < actions; a++) {
+        cum += p[a];
+        const float d = fabsf(target - cum);
+        if (d < best) best = d;
+    }
+    return best / total;
+}

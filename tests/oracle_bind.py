@@ -72,6 +72,10 @@ def cfo():
         lib.cfo_expand_record.argtypes = [vp, vp]
         lib.cfo_forward_f64.argtypes = [vp, C.c_int, C.c_int] + [vp] * 9
         lib.cfo_classic_expand.argtypes = [vp, vp]
+        lib.cfo_sample_action.argtypes = [vp, C.c_int, C.c_float, vp]
+        lib.cfo_sample_action.restype = C.c_int
+        lib.cfo_sample_margin.argtypes = [vp, C.c_int, C.c_float]
+        lib.cfo_sample_margin.restype = C.c_float
         lib.cfo_classic_forward_f64.argtypes = [vp, C.c_int, C.c_int] + [vp] * 9
         lib.cfo_forward_f32.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int]
         lib.cfo_max_threads.restype = C.c_int
@@ -262,3 +266,21 @@ class RefEnv:
 
     def close(self):
         ref().cfref_free()
+
+
+def sample_actions(logits, u):
+    """cfo_sample_action row by row: logits [n][A] f32, u [n] f32 ->
+    (actions i32[n], logprobs f32[n], margins f32[n])."""
+    logits = np.ascontiguousarray(logits, dtype=np.float32)
+    u = np.ascontiguousarray(u, dtype=np.float32)
+    n, A = logits.shape
+    act = np.empty(n, dtype=np.int32)
+    lp = np.empty(n, dtype=np.float32)
+    mg = np.empty(n, dtype=np.float32)
+    one = C.c_float()
+    lib = cfo()
+    for i in range(n):
+        act[i] = lib.cfo_sample_action(_p(logits[i]), A, float(u[i]), C.byref(one))
+        lp[i] = one.value
+        mg[i] = lib.cfo_sample_margin(_p(logits[i]), A, float(u[i]))
+    return act, lp, mg

@@ -1,0 +1,144 @@
+"""GPU tests of the rollout-side entry points through the C ABI: categorical
+sampling (cfp_value_sample), reward/done recording (cfp_record_rd), the policy
+half of a rollout step (cfp_rollout_step) and the bootstrap value
+(cfp_train_bootstrap).
+
+The uniform behind each draw is this library's counter generator (the reference's
+cuRAND Philox stream cannot be reproduced without CUDA: parity unpinned); given
+the uniform, actions and log-probabilities follow cf_nn_sample_action
+(craftax_full.cu:9147-9165) and are checked against its C restatement.  Actions
+must agree except where u*total lies within 1e-6 (relative) of a cumulative-sum
+boundary, where a one-ulp difference between device and host expf may tip the
+comparison; log-probabilities within 1e-5 absolute."""
+import numpy as np
+import pytest
+
+import oracle_bind as ob
+from parity_util import ACTIONS, HIDDEN, mix64, random_params, synth_records_host, unit24
+
+pytestmark = pytest.mark.gpu
+L = 3
+SALT = np.uint64(0xA5A5A5A5A5A5A5A5)
+
+
+def _t(a, cuda):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).to(cuda)
+
+
+def _uniforms(seed, step, n):
+    return unit24(mix64(np.uint64(seed) ^ SALT, step, np.arange(n, dtype=np.uint64)))
+
+
+def _check_draws(av_h, act, lp, val, seed, step):
+    n = av_h.shape[0]
+    A = av_h.shape[1] - 1
+    u = _uniforms(seed, step, n)
+    ref_act, ref_lp, margin = ob.sample_actions(av_h[:, :A], u)
+    bad = act != ref_act
+    assert np.all(margin[bad] < 1e-6), f"{bad.sum()} draws differ away from a boundary"
+    assert bad.mean() < 1e-3
+    ok = ~bad
+    assert np.max(np.abs(lp[ok] - ref_lp[ok])) < 1e-5
+    assert np.array_equal(val, av_h[:, A])
+
+
+@pytest.mark.parametrize("n,A,scale", [(4096, 43, 1.0), (1000, 43, 6.0), (2048, 17, 2.0)])
+def test_value_sample_matches_restatement(pkg, cuda, n, A, scale):
+    import torch
+    rng = np.random.default_rng(n + A)
+    av_h = (scale * rng.standard_normal((n, A + 1))).astype(np.float32)
+    ctr = torch.tensor([7], dtype=torch.int64, device=cuda)
+    env_act = torch.zeros(n, device=cuda)
+    act, lp, val = pkg.policy.value_sample(_t(av_h, cuda), 1234, step_ctr=ctr, env_actions=env_act)
+    torch.cuda.synchronize()
+    act_h = act.cpu().numpy()
+    _check_draws(av_h, act_h, lp.cpu().numpy(), val.cpu().numpy(), 1234, 7)
+    assert np.array_equal(env_act.cpu().numpy(), act_h.astype(np.float32))
+    # same inputs -> same draws; another step -> other draws; no counter -> step 0
+    act2, _, _ = pkg.policy.value_sample(_t(av_h, cuda), 1234, step_ctr=ctr)
+    ctr.fill_(8)
+    act3, _, _ = pkg.policy.value_sample(_t(av_h, cuda), 1234, step_ctr=ctr)
+    act0, lp0, val0 = pkg.policy.value_sample(_t(av_h, cuda), 1234)
+    torch.cuda.synchronize()
+    assert torch.equal(act, act2) and not torch.equal(act, act3)
+    _check_draws(av_h, act0.cpu().numpy(), lp0.cpu().numpy(), val0.cpu().numpy(), 1234, 0)
+
+
+def test_value_sample_distribution(pkg, cuda):
+    """One logit vector replicated over 2^20 envs: empirical action frequencies
+    match softmax within five binomial standard deviations (pins that the
+    uniforms are uniform and the inversion unbiased)."""
+    import torch
+    n, A = 1 << 20, 43
+    rng = np.random.default_rng(3)
+    logits = (1.5 * rng.standard_normal(A)).astype(np.float32)
+    av = torch.empty(n, A + 1, device=cuda)
+    av[:, :A] = _t(logits, cuda)
+    av[:, A] = 0.25
+    act, lp, val = pkg.policy.value_sample(av, 99)
+    torch.cuda.synchronize()
+    p = np.exp(logits.astype(np.float64) - logits.max())
+    p /= p.sum()
+    freq = np.bincount(act.cpu().numpy(), minlength=A) / n
+    sd = np.sqrt(p * (1 - p) / n)
+    assert np.all(np.abs(freq - p) < 5 * sd + 1e-9)
+    assert torch.all(val == 0.25)
+
+
+def test_record_rd(pkg, cuda):
+    import torch
+    n = 1000
+    rng = np.random.default_rng(1)
+    rew = rng.standard_normal(n).astype(np.float32)
+    term = (rng.random(n) < 0.3).astype(np.float32) * rng.choice([1.0, 2.0], n).astype(np.float32)
+    r_rew = torch.full((n,), -7.0, device=cuda)
+    r_done = torch.full((n,), 9, dtype=torch.uint8, device=cuda)
+    pkg.policy.record_rd(_t(rew, cuda), _t(term, cuda), r_rew, r_done)
+    torch.cuda.synchronize()
+    assert np.array_equal(r_rew.cpu().numpy(), rew)
+    assert np.array_equal(r_done.cpu().numpy(), (term != 0).astype(np.uint8))
+
+
+def test_rollout_step_and_bootstrap(pkg, cuda):
+    """cfp_rollout_step == forward on the live state + sampling with the device step
+    counter, written into the slab rows; cfp_train_bootstrap values the next
+    records on a copy of the live state."""
+    import torch
+    n, T, seed = 256, 4, 4321
+    params = random_params(L, 21, scale=0.5)
+    pol = pkg.Policy(n, L, seed=1)
+    pol.set_params(params)
+    twin = pkg.Policy(n, L, seed=1)      # same weights, driven by hand
+    twin.set_params(params)
+    tr = pkg.Trainer(pol, T)
+    rng = np.random.default_rng(22)
+    pol.state.zero_()
+    twin_state = torch.zeros(L, n, HIDDEN, device=cuda)
+    env_act = torch.zeros(n, device=cuda)
+    for t in range(T):
+        rec = _t(synth_records_host(n, 5, t), cuda)
+        term = _t((rng.random(n) < 0.2).astype(np.float32) if t else np.zeros(n, np.float32), cuda)
+        r_state_ref = torch.zeros(L, n, HIDDEN, device=cuda)
+        av = twin.forward(rec, term, twin_state, r_state_t=r_state_ref).clone()
+        tr.rollout_step(t, rec, term, seed, env_actions=env_act)
+        torch.cuda.synchronize()
+        assert int(tr.buf("step_ctr").cpu()[0]) == t + 1
+        assert torch.equal(pol.state, twin_state)
+        assert torch.equal(tr.buf("r_state")[t], r_state_ref)
+        assert torch.equal(tr.buf("r_obs")[t], rec)
+        act = tr.buf("r_act")[t].cpu().numpy()
+        _check_draws(av.cpu().numpy(), act, tr.buf("r_logprob")[t].cpu().numpy(),
+                     tr.buf("r_value")[t].cpu().numpy(), seed, t)
+        assert np.array_equal(env_act.cpu().numpy(), act.astype(np.float32))
+    # bootstrap: value of the next records, live state untouched
+    rec = _t(synth_records_host(n, 5, T), cuda)
+    term = _t((rng.random(n) < 0.2).astype(np.float32), cuda)
+    live_before = pol.state.clone()
+    tr.bootstrap(rec, term)
+    st_copy = twin_state.clone()
+    av = twin.forward(rec, term, st_copy)
+    torch.cuda.synchronize()
+    assert torch.equal(pol.state, live_before)
+    assert torch.equal(tr.buf("v_boot"), av[:, ACTIONS])
+    tr.close(); pol.close(); twin.close()

@@ -285,3 +285,37 @@ def test_classic_expand_and_forward_oracle():
     for f in np.nonzero(x[e])[0]:
         h += float(x[e, f]) * sp["W_enc"][f].astype(np.float64)
     assert np.allclose(h, a["h_enc"][e], rtol=1e-13, atol=1e-13)
+
+
+# ---- cfo_sample_action (cf_nn_sample_action, craftax_full.cu:9147-9165) -----------
+def test_sample_action_closed_forms():
+    """Pins the sampling restatement without the reference's RNG: with equal
+    logits the cumulative sum is a staircase of equal steps, so the action is
+    ceil(u*A) - 1 (0 for u = 0); a dominant logit takes every u > 0; the
+    log-probability is log softmax; exp(logprob) over all actions sums to one."""
+    A = 43
+    u = np.array([0.0, 1e-7, 0.01, 0.2, 0.5, 0.999, 0.9999999], dtype=np.float32)
+    eq = np.zeros((len(u), A), dtype=np.float32)
+    act, lp, _ = ob.sample_actions(eq, u)
+    expect = np.maximum(np.ceil(u.astype(np.float64) * A) - 1, 0).astype(np.int32)
+    assert np.array_equal(act, expect)
+    assert np.allclose(lp, -np.log(A), atol=1e-6)
+    dom = np.full((len(u), A), -30.0, dtype=np.float32)
+    dom[:, 17] = 5.0
+    act, lp, _ = ob.sample_actions(dom, u)
+    # u = 0 gives target 0 <= p[0] for any positive p[0]: action 0 by construction
+    assert act[0] == 0 and np.all(act[(u > 0) & (u < 0.999999)] == 17)
+    assert np.allclose(lp[act == 17], 0.0, atol=1e-6)
+    rng = np.random.default_rng(5)
+    logits = rng.standard_normal((1, A)).astype(np.float32) * 3
+    # walk u over the unit interval: every action is hit in order, and the
+    # log-probabilities reported along the way form a normalised distribution
+    grid = (np.arange(20000, dtype=np.float32) + 0.5) / 20000
+    acts, lps, _ = ob.sample_actions(np.repeat(logits, len(grid), 0), grid)
+    assert np.all(np.diff(acts) >= 0)
+    ref_lp = logits[0] - logits[0].max() - np.log(np.sum(np.exp(logits[0].astype(np.float64) - logits[0].max())))
+    seen = np.unique(acts)
+    assert np.allclose([lps[acts == a][0] for a in seen], ref_lp[seen], atol=2e-6)
+    # frequencies on the grid equal the softmax probabilities to the grid resolution
+    freq = np.bincount(acts, minlength=A) / len(grid)
+    assert np.max(np.abs(freq - np.exp(ref_lp))) < 2.0 / len(grid) + 1e-6
