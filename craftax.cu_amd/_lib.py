@@ -28,6 +28,8 @@ PROTOTYPES = {
     "cfp_policy_set_params": (C.c_int, [vp, vp, C.c_size_t]),
     "cfp_policy_get_params": (C.c_int, [vp, vp, C.c_size_t]),
     "cfp_policy_refresh_weights": (C.c_int, [vp, vp]),
+    "cfp_save_weights": (C.c_int, [vp, C.c_char_p]),
+    "cfp_load_weights": (C.c_int, [vp, C.c_char_p]),
     "cfp_policy_set_gemm_bf16": (C.c_int, [vp, C.c_int]),
     "cfp_policy_gemm_bf16": (C.c_int, [vp]),
     "cfp_policy_params": (vp, [vp]),

@@ -185,6 +185,44 @@ int cfp_policy_get_params(const cfp_policy* p, float* host_params,
     return 0;
 }
 
+// CFW1 files (craftax_full.cu:12244-12293): uint32 {magic "CFW1", hidden, layers,
+// param count} followed by the fp32 params arena.
+static constexpr uint32_t kCkptMagic = 0x31574643u;
+
+int cfp_save_weights(const cfp_policy* p, const char* path) {
+    CFP_REQUIRE(p && path, "cfp_save_weights: NULL argument");
+    std::vector<float> h(p->param_count);
+    CFP_HIP_TRY(hipMemcpy(h.data(), p->params, h.size() * sizeof(float), hipMemcpyDeviceToHost));
+    FILE* f = fopen(path, "wb");
+    CFP_REQUIRE(f, "cannot write %s", path);
+    const uint32_t hdr[4] = {kCkptMagic, CFP_HIDDEN, (uint32_t)p->layers,
+                             (uint32_t)p->param_count};
+    const bool ok = fwrite(hdr, sizeof(hdr), 1, f) == 1 &&
+                    fwrite(h.data(), sizeof(float), h.size(), f) == h.size();
+    const bool closed = fclose(f) == 0;
+    CFP_REQUIRE(ok && closed, "short write to %s", path);
+    return 0;
+}
+
+int cfp_load_weights(cfp_policy* p, const char* path) {
+    CFP_REQUIRE(p && path, "cfp_load_weights: NULL argument");
+    FILE* f = fopen(path, "rb");
+    CFP_REQUIRE(f, "cannot read %s", path);
+    uint32_t hdr[4];
+    if (fread(hdr, sizeof(hdr), 1, f) != 1 || hdr[0] != kCkptMagic || hdr[1] != CFP_HIDDEN ||
+        hdr[2] != (uint32_t)p->layers || hdr[3] != (uint32_t)p->param_count) {
+        fclose(f);
+        set_error("%s: bad header (want h%dx%d, %zu params)", path, CFP_HIDDEN, p->layers,
+                  p->param_count);
+        return 1;
+    }
+    std::vector<float> h(p->param_count);
+    const size_t got = fread(h.data(), sizeof(float), h.size(), f);
+    fclose(f);
+    CFP_REQUIRE(got == h.size(), "%s: truncated", path);
+    return cfp_policy_set_params(p, h.data(), h.size());   // also refreshes the mirrors
+}
+
 int cfp_policy_refresh_weights(cfp_policy* p, void* stream) {
     CFP_REQUIRE(p, "cfp_policy_refresh_weights: NULL policy");
     if (launch_pack_weights(p->params, p->layers, p->variant, p->we_pk, p->wg_pk, p->wav_pk,

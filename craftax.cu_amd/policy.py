@@ -109,6 +109,13 @@ class Policy:
     def refresh_weights(self):
         _check(lib().cfp_policy_refresh_weights(self._h, _stream()))
 
+    def save_weights(self, path):
+        """CFW1 checkpoint (cu_save_weights, craftax_full.cu:12248)."""
+        _check(lib().cfp_save_weights(self._h, str(path).encode()))
+
+    def load_weights(self, path):
+        _check(lib().cfp_load_weights(self._h, str(path).encode()))
+
     def set_gemm_bf16(self, on=True):
         """Run the forward entry points with bf16 GEMM inputs and fp32 accumulation
         (the reference's CF_GEMM_BF16 mode, craftax_full.cu:11306-11316)."""

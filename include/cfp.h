@@ -102,6 +102,13 @@ int cfp_policy_get_params(const cfp_policy* p, float* host_params, size_t count)
  * (craftax_full.cu:11805-11817) after init / Adam. */
 int cfp_policy_refresh_weights(cfp_policy* p, void* stream);
 
+/* cu_save_weights / cu_load_weights (craftax_full.cu:12248, :12264): the "CFW1"
+ * file -- uint32 {0x31574643, hidden = 256, layers, param count} then the fp32
+ * params arena.  Loading checks the header against the policy (error, params
+ * untouched, on mismatch or truncation) and refreshes the weight mirrors. */
+int cfp_save_weights(const cfp_policy* p, const char* path);
+int cfp_load_weights(cfp_policy* p, const char* path);
+
 /* bf16-input / fp32-accumulate GEMMs for the forward entry points of this policy
  * (encoder, gate and head GEMMs on bf16 MFMA; state, epilogue and outputs stay
  * fp32).  Replaces the reference's process-wide CF_GEMM_BF16 switch

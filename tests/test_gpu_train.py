@@ -216,3 +216,74 @@ def test_config4_shape_properties(pkg, cuda):
         assert_close(g_halves[sl].cpu().numpy(), g_full[sl].cpu().numpy(), TOL_FP32,
                      f"linearity d{name}")
     tr.close(); pol.close()
+
+
+def test_update_iteration_replays_from_a_graph(pkg, cuda):
+    """backward + Adam captured once (after the lazily allocated GEMM workspaces
+    exist) and replayed: every replay, with eager work and synchronisations in
+    between, must leave the same parameters as the same number of eager updates
+    on an identical twin (the step counter and lr live in device memory)."""
+    import torch
+    n, T = 64, 6
+    twins = [_collect(pkg, cuda, n, T, 123, 0.1) for _ in range(2)]
+    (_, pol_e, tr_e, _), (_, pol_g, tr_g, _) = twins
+
+    def update(tr):
+        tr.zero_loss()
+        tr.backward(0, n)
+        tr.adam()
+
+    update(tr_e)                      # warm-up: allocates the split-K / gemv workspaces
+    update(tr_g)
+    torch.cuda.synchronize()
+    assert torch.equal(pol_e.params, pol_g.params)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        update(tr_g)
+    for i in range(3):
+        update(tr_e)
+        graph.replay()
+        torch.cuda.synchronize()
+        junk = torch.randn(1 << 16, device=cuda).sum().item()   # eager work between replays
+        assert np.isfinite(junk)
+        assert torch.equal(pol_e.params, pol_g.params), f"replay {i}"
+        assert torch.equal(tr_e.buf("adam_v"), tr_g.buf("adam_v"))
+    # the forward weights follow the replayed updates (mirrors refreshed inside the graph)
+    rec = _t(synth_records_host(n, 9, 0), cuda)
+    term = torch.zeros(n, device=cuda)
+    sa = torch.zeros(L, n, HIDDEN, device=cuda); sb = torch.zeros(L, n, HIDDEN, device=cuda)
+    assert torch.equal(pol_e.forward(rec, term, sa), pol_g.forward(rec, term, sb))
+    for _, pol, tr, _ in twins:
+        tr.close(); pol.close()
+
+
+def test_checkpoint_roundtrip(pkg, cuda, tmp_path):
+    """CFW1 file: header words, byte-exact params, mirrors refreshed on load, and the
+    reference's rejections (wrong shape, truncated file)."""
+    import torch
+    n = 32
+    a = pkg.Policy(n, L, seed=11)
+    path = tmp_path / "w.cfw"
+    a.save_weights(path)
+    raw = np.fromfile(path, dtype=np.uint32)
+    assert raw[0] == 0x31574643 and raw[1] == 256 and raw[2] == L and raw[3] == a.param_count
+    assert np.array_equal(raw[4:].view(np.float32), a.get_params())
+    b = pkg.Policy(n, L, seed=12)
+    b.load_weights(path)
+    assert np.array_equal(b.get_params(), a.get_params())
+    rec = pkg.policy.synth_records(n, 3, 0)
+    term = torch.zeros(n, device=cuda)
+    sa = torch.zeros(L, n, HIDDEN, device=cuda); sb = torch.zeros(L, n, HIDDEN, device=cuda)
+    assert torch.equal(a.forward(rec, term, sa), b.forward(rec, term, sb))
+    c = pkg.Policy(n, 2, seed=1)
+    before = c.get_params()
+    with pytest.raises(pkg._lib.CfpError):
+        c.load_weights(path)                       # layer count differs
+    assert np.array_equal(c.get_params(), before)
+    raw[: 4 + 100].tofile(tmp_path / "short.cfw")
+    with pytest.raises(pkg._lib.CfpError):
+        b.load_weights(tmp_path / "short.cfw")
+    with pytest.raises(pkg._lib.CfpError):
+        b.load_weights(tmp_path / "missing.cfw")
+    for p in (a, b, c):
+        p.close()
