@@ -44,6 +44,8 @@ PROTOTYPES = {
     "cfp_head": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "cfp_policy_forward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int,
                                      C.c_int, vp]),
+    "cfp_set_gemm_bf16": (C.c_int, [C.c_int]),
+    "cfp_get_gemm_bf16": (C.c_int, []),
     "cfp_gemm_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
     "cfp_gemm_enc_fwd": (C.c_int, [C.c_int, vp, vp, vp, vp]),
     "cfp_gemm_dh": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),

@@ -79,6 +79,13 @@ def ppo_update(pkg, torch, reps):
            "samples_per_s": samples / ms * 1e3,
            "tflops": UPD_FLOP * samples / ms / 1e9,
            "frac_fp32_mfma_peak": UPD_FLOP * samples / ms / 1e9 / PEAK_FP32}
+    pkg.policy.set_gemm_bf16(True)       # same update with bf16 GEMM inputs
+    try:
+        ms16 = _time(torch, step, reps, warm=1)
+    finally:
+        pkg.policy.set_gemm_bf16(False)
+    out["bf16_in"] = {"ms_per_update": ms16, "samples_per_s": samples / ms16 * 1e3,
+                      "tflops": UPD_FLOP * samples / ms16 / 1e9}
     assert torch.isfinite(pol.params).all()
     tr.close()
     pol.close()

@@ -179,6 +179,111 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm(GemmArgs g) {
         }
 }
 
+// ---- bf16-input / fp32-accumulate form of the same GEMM ----------------------------
+// (the reference's CF_GEMM_BF16 wrappers, craftax_full.cu:11688-11756).  Operands
+// stay fp32 in memory; they are rounded to bf16 (nearest even) on their way into
+// LDS, where both sit as [row][k] with 80-byte rows so that a lane's fragment for
+// v_mfma_f32_32x32x16_bf16 (eight consecutive k of one row) is one 16-byte read.
+// An operand whose K dimension is unit-stride arrives as four consecutive k
+// (one 8-byte LDS write); one whose row dimension is unit-stride arrives as four
+// rows of one k and is transposed by four 2-byte writes.  At bf16 rates the
+// kernel is bound by this staging and by HBM, not by the matrix pipe.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+constexpr int LDB = 40;   // bf16 per LDS row: 32 k + 8 pad
+
+template <bool KFAST>
+__device__ __forceinline__ void stash_bf16(__bf16* lds, const f4 (&r)[4], int tid) {
+#pragma unroll
+    for (int it = 0; it < 4; it++) {
+        const int v = tid + GEMM_THREADS * it;
+        const bf16x4 h = __builtin_convertvector(r[it], bf16x4);
+        if (KFAST) {
+            *reinterpret_cast<bf16x4*>(lds + (v >> 3) * LDB + 4 * (v & 7)) = h;
+        } else {
+            __bf16* q = lds + (4 * (v & 31)) * LDB + (v >> 5);
+#pragma unroll
+            for (int c = 0; c < 4; c++) q[c * LDB] = h[c];
+        }
+    }
+}
+
+template <bool A_KFAST, bool B_KFAST, bool ACCUM, bool VEC_A, bool VEC_B>
+__global__ __launch_bounds__(GEMM_THREADS) void k_gemm_bf16(GemmArgs g) {
+    __shared__ __attribute__((aligned(16))) __bf16 As[BM * LDB];
+    __shared__ __attribute__((aligned(16))) __bf16 Bs[BN * LDB];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int total = g.mt * g.nt;
+    const int chunk = (total + kXcds - 1) / kXcds;
+    const int tile = (int)(blockIdx.x % kXcds) * chunk + (int)(blockIdx.x / kXcds);
+    if (tile >= total) return;
+    const int i0 = (tile / g.nt) * BM;
+    const int j0 = (tile % g.nt) * BN;
+    const int kbeg = blockIdx.y * g.k_per_split;
+    const int kend = min(g.K, kbeg + g.k_per_split);
+
+    f16v acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[a][b][r] = 0.0f;
+
+    f4 ra[4], rb[4];
+    fetch<A_KFAST, VEC_A>(ra, g.A, g.sa_i, g.sa_k, i0, g.M, kbeg, kend, tid);
+    fetch<B_KFAST, VEC_B>(rb, g.B, g.sb_j, g.sb_k, j0, g.N, kbeg, kend, tid);
+    for (int k0 = kbeg; k0 < kend; k0 += BK) {
+        __syncthreads();
+        stash_bf16<A_KFAST>(As, ra, tid);
+        stash_bf16<B_KFAST>(Bs, rb, tid);
+        __syncthreads();
+        if (k0 + BK < kend) {
+            fetch<A_KFAST, VEC_A>(ra, g.A, g.sa_i, g.sa_k, i0, g.M, k0 + BK, kend, tid);
+            fetch<B_KFAST, VEC_B>(rb, g.B, g.sb_j, g.sb_k, j0, g.N, k0 + BK, kend, tid);
+        }
+#pragma unroll
+        for (int kb = 0; kb < BK / 16; kb++) {
+            bf16x8 af[2], bf[2];
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+                af[a] = *reinterpret_cast<const bf16x8*>(As + (wm * 64 + a * 32 + l32) * LDB +
+                                                          16 * kb + 8 * half);
+#pragma unroll
+            for (int b = 0; b < 2; b++)
+                bf[b] = *reinterpret_cast<const bf16x8*>(Bs + (wn * 64 + b * 32 + l32) * LDB +
+                                                          16 * kb + 8 * half);
+#pragma unroll
+            for (int a = 0; a < 2; a++)
+#pragma unroll
+                for (int b = 0; b < 2; b++)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[a], bf[b], acc[a][b],
+                                                                        0, 0, 0);
+        }
+    }
+
+    float* C = g.C + (long)blockIdx.y * g.c_split;
+#pragma unroll
+    for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const int j = j0 + wn * 64 + b * 32 + l32;
+            if (j >= g.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int i = i0 + wm * 64 + a * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (i < g.M) {
+                    float* c = C + (long)i * g.ldc + j;
+                    if (ACCUM) *c += acc[a][b][r];
+                    else *c = acc[a][b][r];
+                }
+            }
+        }
+}
+
 // dst[i] += sum_z part[z*stride + i], z ascending.
 __global__ void k_splitk_reduce(float* __restrict__ dst,
                                 const float* __restrict__ part, long count,
@@ -222,9 +327,21 @@ static bool vec_ok(const float* p, long ld, int fast_extent) {
            ld >= (long)((fast_extent + 3) / 4 * 4);
 }
 
+// Process-wide switch of the seam's GEMMs to bf16 inputs, like the reference's
+// g_gemm_bf16 (craftax_full.cu:11306-11316).
+int g_gemm_bf16 = 0;
+
 template <bool A_KFAST, bool B_KFAST, bool ACCUM>
 int launch_gemm(const GemmArgs& g, dim3 grid, bool va, bool vb, hipStream_t st) {
     const dim3 blk(GEMM_THREADS);
+    if (g_gemm_bf16) {
+        if (va && vb) hipLaunchKernelGGL((k_gemm_bf16<A_KFAST, B_KFAST, ACCUM, true, true>), grid, blk, 0, st, g);
+        else if (va) hipLaunchKernelGGL((k_gemm_bf16<A_KFAST, B_KFAST, ACCUM, true, false>), grid, blk, 0, st, g);
+        else if (vb) hipLaunchKernelGGL((k_gemm_bf16<A_KFAST, B_KFAST, ACCUM, false, true>), grid, blk, 0, st, g);
+        else hipLaunchKernelGGL((k_gemm_bf16<A_KFAST, B_KFAST, ACCUM, false, false>), grid, blk, 0, st, g);
+        CFP_HIP_TRY(hipGetLastError());
+        return 0;
+    }
     if (va && vb) hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, ACCUM, true, true>), grid, blk, 0, st, g);
     else if (va) hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, ACCUM, true, false>), grid, blk, 0, st, g);
     else if (vb) hipLaunchKernelGGL((k_gemm<A_KFAST, B_KFAST, ACCUM, false, true>), grid, blk, 0, st, g);
@@ -312,6 +429,12 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
 }  // namespace cfp
 
 extern "C" {
+
+int cfp_set_gemm_bf16(int on) {
+    g_gemm_bf16 = on ? 1 : 0;
+    return 0;
+}
+int cfp_get_gemm_bf16(void) { return g_gemm_bf16; }
 
 int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
                  float* d_y, void* stream) {

@@ -280,6 +280,12 @@ def _wrap(ptr, shape, typestr):
 
 
 # -- the dense-math seam -------------------------------------------------------
+def set_gemm_bf16(on=True):
+    """Process-wide: bf16 inputs / fp32 accumulation for cfp_gemm_* and the PPO update
+    (the reference's CF_GEMM_BF16, craftax_full.cu:11306-11316)."""
+    _check(lib().cfp_set_gemm_bf16(1 if on else 0))
+
+
 def gemm_fwd(W, x, y=None):
     """y[cols][m] = x[cols][k] . W[m][k]^T (cu_gemm_fwd :11604)."""
     m, k = W.shape

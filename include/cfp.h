@@ -159,6 +159,15 @@ int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
                        float* d_av, int n, int chunk, void* stream);
 
 /* ---- the dense-math seam (craftax_full.cu:11604-11666) ------------------- */
+/* bf16 inputs with fp32 accumulation for every GEMM of this seam (cfp_gemm_fwd /
+ * enc_fwd / dh / dw, hence the whole PPO update): the reference's process-wide
+ * CF_GEMM_BF16 / g_gemm_bf16 switch (craftax_full.cu:11306-11316, wrappers
+ * :11688-11756).  Operands stay fp32 in memory and are rounded to bf16 on the way
+ * into the kernel; results stay fp32 (the reference also emits bf16 C for the gate
+ * and dh GEMMs; this library does not).  Off by default. */
+int cfp_set_gemm_bf16(int on);
+int cfp_get_gemm_bf16(void);
+
 /* cu_gemm_fwd (:11604): y[cols][m] = x[cols][k] . W[m][k]^T. */
 int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
                  float* d_y, void* stream);

@@ -91,3 +91,68 @@ def test_unfused_epilogue_and_bias(pkg, cuda):
     pkg.policy.add_bias(hb, b)
     torch.cuda.synchronize()
     assert torch.equal(hb, x + b)
+
+
+# ---- bf16-input / fp32-accumulate seam (cfp_set_gemm_bf16) ---------------------------
+@pytest.fixture
+def bf16_gemms(pkg):
+    pkg.policy.set_gemm_bf16(True)
+    yield
+    pkg.policy.set_gemm_bf16(False)
+
+
+def _grid(t):
+    """fp32 tensor rounded to the bf16 grid (so that the kernel's own rounding is exact)."""
+    import torch
+    return t.to(torch.bfloat16).to(torch.float32)
+
+
+@pytest.mark.parametrize("exact", [True, False])
+def test_bf16_gemms(pkg, cuda, bf16_gemms, exact):
+    """All four GEMM shapes with bf16 inputs.  exact=True: operands already on the
+    bf16 grid, every product is exact and the result must match fp64 to fp32
+    summation accuracy (pins fragment layout and the LDS transposition of both
+    operand orientations, vector and scalar load paths, edge tiles, split-K);
+    exact=False: arbitrary fp32 operands, 2e-2 relative to fp64 and 1e-4 against
+    fp64 on the bf16-rounded operands (the rounding is to nearest even)."""
+    import torch
+    from parity_util import TOL_BF16
+
+    def check(got, a, b, what, base=None):
+        ref = a.double() @ b.double()
+        ref_q = _grid(a).double() @ _grid(b).double()
+        if base is not None:
+            ref, ref_q = ref + base, ref_q + base
+        assert_close(got.cpu().numpy(), ref_q.cpu().numpy(), 1e-4, what + " vs bf16-rounded fp64")
+        if not exact:
+            assert_close(got.cpu().numpy(), ref.cpu().numpy(), TOL_BF16, what + " vs fp64")
+
+    prep = _grid if exact else (lambda t: t)
+    for m, cols, k in [(768, 500, 256), (44, 96, 256), (100, 33, 77), (768, 16384, 256)]:
+        W, x = prep(_r((m, k), cuda, 1, 0.1)), prep(_r((cols, k), cuda, 2))
+        check(pkg.policy.gemm_fwd(W, x), x, W.T, f"bf16 gemm_fwd {m}x{cols}x{k}")
+    for cols in (1, 100, 4096):
+        W, x = prep(_r((OBS, HIDDEN), cuda, 3, 0.05)), prep(_r((cols, OBS), cuda, 4, 5.0))
+        check(pkg.policy.gemm_enc_fwd(W, x), x, W, f"bf16 gemm_enc_fwd {cols}")
+    for m3, cols in [(768, 777), (43, 130), (768, 8192)]:
+        W, d = prep(_r((m3, HIDDEN), cuda, 5, 0.1)), prep(_r((cols, m3), cuda, 6))
+        check(pkg.policy.gemm_dh(W, d), d, W, f"bf16 gemm_dh {m3}x{cols}")
+    for rows, cols in [(768, 5000), (43, 300), (843, 2048), (768, 31), (768, 65536)]:
+        x, d = prep(_r((cols, HIDDEN), cuda, 7)), prep(_r((cols, rows), cuda, 8))
+        dW = torch.full((rows, HIDDEN), 0.5, device=cuda)
+        pkg.policy.gemm_dw(x, d, dW)
+        check(dW, d.T, x, f"bf16 gemm_dw {rows}x{cols}", base=0.5)
+    torch.cuda.synchronize()
+
+
+def test_bf16_switch_is_off_by_default_and_reversible(pkg, cuda):
+    import torch
+    W, x = _r((768, 256), cuda, 1, 0.1), _r((300, 256), cuda, 2)
+    assert pkg.lib().cfp_get_gemm_bf16() == 0
+    y0 = pkg.policy.gemm_fwd(W, x)
+    pkg.policy.set_gemm_bf16(True)
+    y1 = pkg.policy.gemm_fwd(W, x)
+    pkg.policy.set_gemm_bf16(False)
+    y2 = pkg.policy.gemm_fwd(W, x)
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y2) and not torch.equal(y0, y1)

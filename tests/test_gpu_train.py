@@ -287,3 +287,50 @@ def test_checkpoint_roundtrip(pkg, cuda, tmp_path):
         b.load_weights(tmp_path / "missing.cfw")
     for p in (a, b, c):
         p.close()
+
+
+def test_backward_with_bf16_gemms(pkg, cuda):
+    """The update with bf16 GEMM inputs (cfp_set_gemm_bf16) against the fp64 oracle,
+    every gradient segment in the relative Frobenius norm (the per-entry metric
+    does not apply to bf16 inputs, see parity_util).  The clipped surrogate is
+    discontinuous in the logits where the probability ratio crosses 1 +- clip, so
+    the behaviour log-probabilities are set to the current policy's own (plus 0.02
+    of noise): every sample then sits well inside the clip range and the loss is
+    smooth under the 1e-2-sized logit perturbation bf16 inputs cause."""
+    import torch
+    from parity_util import TOL_BF16, fro_err, expand_records
+    n, T = 64, 8
+    params, pol, tr, host = _collect(pkg, cuda, n, T, 150, 0.1)
+    rng = np.random.default_rng(151)
+    for t in range(T):
+        ref = ob.forward_f64(params, L, expand_records(host["r_obs"][t]), host["r_state"][t], None)
+        z = ref["logits"] - ref["logits"].max(axis=1, keepdims=True)
+        logp = z - np.log(np.exp(z).sum(axis=1, keepdims=True))
+        host["r_logprob"][t] = (logp[np.arange(n), host["r_act"][t]]
+                                + 0.02 * rng.standard_normal(n)).astype(np.float32)
+    tr.buf("r_logprob").copy_(_t(host["r_logprob"], cuda))
+    batch, keep = ob.make_batch(T, n, 0, n, L, T, **host)
+    g_ref, l3_ref = ob.ppo_backward_f64(params, batch)
+    grads = {}
+    for mode in (False, True):
+        pkg.policy.set_gemm_bf16(mode)
+        try:
+            tr.buf("grads").zero_()
+            tr.zero_loss()
+            tr.backward(0, n)
+            torch.cuda.synchronize()
+        finally:
+            pkg.policy.set_gemm_bf16(False)
+        grads[mode] = tr.buf("grads").cpu().numpy().copy()
+        l3 = tr.buf("loss_acc").cpu().numpy()
+        # the pg sum nearly cancels (ratios ~ 1, zero-mean advantages): absolute floor
+        tol = 1e-2 if mode else 1e-4
+        assert np.allclose(l3, l3_ref, rtol=tol, atol=tol * np.abs(l3_ref).max()), (mode, l3, l3_ref)
+    worst = 0.0
+    for name, sl in _segments(L):
+        assert_close(grads[False][sl], g_ref[sl], TOL_FP32, f"fp32 d{name} (same batch)")
+        e = fro_err(grads[True][sl], g_ref[sl])
+        assert e <= TOL_BF16, f"bf16 d{name}: relative Frobenius error {e:.3e}"
+        worst = max(worst, e)
+    assert worst > 1e-4, "the bf16 GEMMs did not run"
+    tr.close(); pol.close()
