@@ -327,6 +327,15 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     const bool classic = VARIANT == 1 && a.rec;
     const bool full_rec = VARIANT == 0 && a.rec;
 
+    // Full-game records travel one pair ahead through registers: requested while
+    // the previous pair runs its last epilogue, written into LDS at the pair's start.
+    RecRegs pre[2];
+    if (full_rec && (int)blockIdx.x < pairs) {
+        const int tid0 = threadIdx.x;
+        rec_fetch(a, (size_t)(2 * blockIdx.x) * kTileEnvs, pre[0], tid0);
+        if (2 * (int)blockIdx.x + 1 < tiles)
+            rec_fetch(a, (size_t)(2 * blockIdx.x + 1) * kTileEnvs, pre[1], tid0);
+    }
     for (int pair = blockIdx.x; pair < pairs; pair += gridDim.x) {
         // Lane constants are re-derived per pair from an opaque copy of the thread
         // index: hoisted out of this loop, the dozens of per-lane addresses they
@@ -348,9 +357,11 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
 
         // ---- stage both tiles (a missing Y is a zero tile that is computed but
         // never read from or written to the caller's buffers) --------------------
-        stage_tile<VARIANT>(a, e0[0], lds_all[0], crec_all[0], term_all[0], tid);
+        if (full_rec) rec_scatter(pre[0], lds_all[0], term_all[0], tid);
+        else stage_tile<VARIANT>(a, e0[0], lds_all[0], crec_all[0], term_all[0], tid);
         if (hasY) {
-            stage_tile<VARIANT>(a, e0[1], lds_all[1], crec_all[1], term_all[1], tid);
+            if (full_rec) rec_scatter(pre[1], lds_all[1], term_all[1], tid);
+            else stage_tile<VARIANT>(a, e0[1], lds_all[1], crec_all[1], term_all[1], tid);
         } else {
             for (int i = tid; i < LDS_FLOATS; i += kFwdThreads) lds_all[1][i] = 0.0f;
             if (tid < kTileEnvs) term_all[1][tid] = 0.0f;
@@ -393,6 +404,16 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             copy_tile_out(lds_all[0], a.h_enc_out + e0[0] * CFP_HIDDEN, tid);
             if (hasY) copy_tile_out(lds_all[1], a.h_enc_out + e0[1] * CFP_HIDDEN, tid);
         }
+
+        // next pair's records -> registers (no-op past the last pair of this workgroup)
+        auto fetch_next = [&]() {
+            const int np = pair + (int)gridDim.x;
+            if (np < pairs) {
+                rec_fetch(a, (size_t)(2 * np) * kTileEnvs, pre[0], tid);
+                if (2 * np + 1 < tiles) rec_fetch(a, (size_t)(2 * np + 1) * kTileEnvs, pre[1], tid);
+            }
+        };
+        if (full_rec && a.layers == 0) fetch_next();
 
         // ---- MinGRU layers, the two tiles software-pipelined -------------------------
         // phase q = 0 .. 2L:  K(tile q&1, layer q/2)  woven with  epi(tile (q-1)&1, layer (q-1)/2)
@@ -443,6 +464,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
 #pragma unroll
                 for (int t = 0; t < 6; t++) accO[t] = accN[t];
             }
+            if (full_rec) fetch_next();
             gru_phase<false, true, HAS_RS>(accN, accO, bq, nullptr, nullptr, lds_all[(Q - 1) & 1],
                                            io, st, L);
             __syncthreads();

@@ -76,6 +76,51 @@ __device__ __forceinline__ void stage_tile(const FwdArgs& a, size_t e0, float* l
     }
 }
 
+// Full-game record staging split in two so that the HBM latency of the next
+// pair's records can be spent under the current pair's last phases: rec_fetch
+// requests a tile's 31 872 bytes (8 x 16 bytes per thread) into registers,
+// rec_scatter writes them into the LDS rows (stride RS dwords) later.
+constexpr int kRecV4PerThread = (TILE_REC_V4 + kFwdThreads - 1) / kFwdThreads;   // 8
+
+struct RecRegs {
+    u4 v[kRecV4PerThread];
+    float term;   // terminal flag of env `tid` of the tile (threads 0..31)
+};
+
+__device__ __forceinline__ void rec_fetch(const FwdArgs& a, size_t e0, RecRegs& r, int tid) {
+    const u4* src = reinterpret_cast<const u4*>(a.rec + e0 * CFP_REC_BYTES);
+#pragma unroll
+    for (int j = 0; j < kRecV4PerThread; j++) {
+        const int i = tid + kFwdThreads * j;
+        if (i < TILE_REC_V4) r.v[j] = __builtin_nontemporal_load(src + i);
+    }
+    r.term = (tid < kTileEnvs && a.terminals) ? a.terminals[e0 + tid] : 0.0f;
+}
+
+__device__ __forceinline__ void rec_scatter(const RecRegs& r, float* lds, float* term_s, int tid) {
+    uint32_t* rs = reinterpret_cast<uint32_t*>(lds);
+#pragma unroll
+    for (int j = 0; j < kRecV4PerThread; j++) {
+        const int i = tid + kFwdThreads * j;
+        if (i < TILE_REC_V4) {
+            const uint32_t w[4] = {r.v[j].x, r.v[j].y, r.v[j].z, r.v[j].w};
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const int d = 4 * i + c;
+                const int row = d / REC_DW;
+                const int col = d - row * REC_DW;
+                rs[row * RS + col] = w[c];
+            }
+        }
+    }
+    if (tid < kTileEnvs * (RS - REC_DW)) {
+        const int row = tid / (RS - REC_DW);
+        const int c = tid - row * (RS - REC_DW);
+        rs[row * RS + REC_DW + c] = 0u;   // features 843..847 read as 0.0f
+    }
+    if (tid < kTileEnvs) term_s[tid] = r.term;
+}
+
 // Classic-game encoder (encode_obs_kernel, craftax_classic.cu:1714-1751): the
 // observation is one-hot per view cell, so h0 is b_enc plus a sum of W_enc
 // rows selected by the record bytes, in feature order.  Thread k owns hidden
