@@ -247,7 +247,11 @@ float* cfp_policy_h3(cfp_policy* p) { return p->h3; }
 float* cfp_policy_logits(cfp_policy* p) { return p->logits; }
 void* cfp_policy_stream(cfp_policy* p) { return (void*)p->stream; }
 
-static void fill_weights(const cfp_policy* p, FwdArgs& a) {
+static void fill_weights(const cfp_policy* p, FwdArgs& a) { cfp::fill_forward_weights(p, a); }
+
+}  // extern "C"
+
+void cfp::fill_forward_weights(const cfp_policy* p, FwdArgs& a) {
     const Arena ar = arena_of(p->variant, p->layers);
     a.we_pk = reinterpret_cast<const f4*>(p->we_pk);
     a.w_enc = p->params + ar.w_enc;
@@ -263,6 +267,8 @@ static void fill_weights(const cfp_policy* p, FwdArgs& a) {
     a.wav_bf = reinterpret_cast<const u4*>(p->wav_bf);
     a.bf16 = p->gemm_bf16;
 }
+
+extern "C" {
 
 // Launch over [0, n) in chunks; every per-env pointer is advanced by the
 // chunk start, the layer stride of state / r_state stays that of the full n.

@@ -92,6 +92,16 @@ struct FwdArgs {
     const u4* wg_bf;
     const u4* wav_bf;
     int bf16;                // bf16-input / fp32-accumulate kernel
+    // Window recompute of the PPO update (fp32 full game only): "env" c of this
+    // launch is window column c = (t0 + c / mb, env_start + c % mb); `rec` is the
+    // r_obs slab, `state` the r_state slab [T][layers][n_all][256] whose stored
+    // post-zero state is the layer's state input (nothing is written back);
+    // every layer's gate pre-activations and output are written out for the
+    // reverse pass.  tr_x[0] is filled through h_enc_out.
+    int train;
+    int tr_t0, tr_mb, tr_n_all, tr_env_start;
+    float* tr_pre[CFP_MAX_LAYERS];   // [cols][768]: zh | zg | zp
+    float* tr_x[CFP_MAX_LAYERS + 1]; // [cols][256]: tr_x[l+1] = output of layer l
 };
 int launch_forward(const FwdArgs& a, hipStream_t st);
 int launch_forward_bf16(const FwdArgs& a, hipStream_t st);   // called by launch_forward

@@ -23,3 +23,8 @@ struct cfp_policy {
     float* logits = nullptr;
     hipStream_t stream = nullptr;
 };
+
+namespace cfp {
+// weight pointers, variant and action count of a policy into launch arguments
+void fill_forward_weights(const cfp_policy* p, FwdArgs& a);
+}  // namespace cfp

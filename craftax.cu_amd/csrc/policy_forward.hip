@@ -205,14 +205,21 @@ __device__ __forceinline__ void classic_encode_pair(const FwdArgs& a, const uint
 // Written-to-nowhere tile: state / r_state addresses of a pair's missing second
 // tile point here, so the hot loop needs no predication.
 __device__ float g_void_tile[kTileEnvs * CFP_HIDDEN];
+__device__ float g_void_pre[kTileEnvs * CFP_GRU];
 
 // State addressing of one (tile, layer) for the epilogue: element e = 0..31 of a
 // lane is unit tile e/16, accumulator register e%16.
 struct StateIO {
     float* st_base;    // state tile + wave*64 (uniform)
-    float* rs_base;    // r_state tile likewise (ignored unless HAS_RS)
+    float* rs_base;    // MODE 1: r_state tile likewise; MODE 2: next layer's input tile
+    float* pre_base;   // MODE 2: gate pre-activation tile [32][768] + wave*64
     unsigned tmask;    // bit r: env row of accumulator register r had a terminal
 };
+
+// Kernel modes: 0 = inference, 1 = inference that also records the post-zero state
+// (r_state), 2 = window recompute of the PPO update (state read from the stored
+// slab and not written back; pre-activations and layer outputs written out).
+constexpr int kModePlain = 0, kModeRecord = 1, kModeTrain = 2;
 
 __device__ __forceinline__ constexpr int st_off(int e) {
     return acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32;
@@ -247,7 +254,7 @@ __device__ __forceinline__ void ring_preload(WRing& bq, const f4* wp, const Lane
 //       epilogue behind the MFMAs).  The state values were requested before the
 //       phase (st[32]); in-loop state loads would sit in front of the weight
 //       loads in the in-order return queue with their HBM latency.
-template <bool DO_K, bool DO_E, bool HAS_RS>
+template <bool DO_K, bool DO_E, int MODE>
 __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6], WRing& bq,
                                           const f4* xs4K, const f4* wp, float* xsE,
                                           const StateIO& io, const float (&st)[32],
@@ -276,11 +283,18 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
         if (DO_E) {
             const int ut = kb / 16, r = kb % 16;
             float* xp = xsE + (acc_row(r) + 4 * L.half) * XS + L.wave * 64 + ut * 32 + L.l32;
-            const float s = (io.tmask >> r) & 1u ? 0.0f : st[kb];
-            if (HAS_RS) __builtin_nontemporal_store(s, (io.rs_base + st_off(kb)) + L.loff);
+            const float s = (MODE != kModeTrain && ((io.tmask >> r) & 1u)) ? 0.0f : st[kb];
+            if (MODE == kModeRecord)
+                __builtin_nontemporal_store(s, (io.rs_base + st_off(kb)) + L.loff);
             const float zh = accO[0 + ut][r];
             const float zg = accO[2 + ut][r];
             const float zp = accO[4 + ut][r];
+            if (MODE == kModeTrain) {
+                float* pp = io.pre_base + (acc_row(r) * CFP_GRU + ut * 32);
+                __builtin_nontemporal_store(zh, pp + L.loff3);
+                __builtin_nontemporal_store(zg, (pp + CFP_HIDDEN) + L.loff3);
+                __builtin_nontemporal_store(zp, (pp + 2 * CFP_HIDDEN) + L.loff3);
+            }
             const float sg = sigmoid_fast(zg);
             float sh = sigmoid_fast(zh);
             asm volatile("" : "+v"(sh));   // keep g(zh) a select, not a branch
@@ -288,8 +302,12 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
             const float out = s + sg * (gh - s);
             const float p = sigmoid_fast(zp);
             const float xv = *xp;
-            *xp = p * out + (1.0f - p) * xv;
-            __builtin_nontemporal_store(out, (io.st_base + st_off(kb)) + L.loff);
+            const float hn = p * out + (1.0f - p) * xv;
+            *xp = hn;
+            if (MODE == kModeTrain)
+                __builtin_nontemporal_store(hn, (io.rs_base + st_off(kb)) + L.loff);
+            else
+                __builtin_nontemporal_store(out, (io.st_base + st_off(kb)) + L.loff);
         }
         // Issue order of the block.  A vector memory instruction occupies the
         // wave's issue port for about as long as one MFMA executes, so the six
@@ -304,7 +322,9 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
                 if (DO_E) {
                     __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // two VALU
                     if (q == 21) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-                    if (q == 22) __builtin_amdgcn_sched_group_barrier(0x040, HAS_RS ? 2 : 1, 0);
+                    if (q == 22)
+                        __builtin_amdgcn_sched_group_barrier(
+                            0x040, MODE == kModeTrain ? 4 : (MODE == kModeRecord ? 2 : 1), 0);
                 }
             }
         }
@@ -314,7 +334,7 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
 
 }  // namespace
 
-template <int VARIANT, bool HAS_RS>
+template <int VARIANT, int MODE>
 __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds_all[2][LDS_FLOATS];
     __shared__ __attribute__((aligned(16))) float red_all[2][kRedFloats];
@@ -330,11 +350,25 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     // Full-game records travel one pair ahead through registers: requested while
     // the previous pair runs its last epilogue, written into LDS at the pair's start.
     RecRegs pre[2];
+    // tile -> its records / terminal flags.  Window recompute: tile = 32 columns of
+    // one step t (the minibatch is a multiple of 32 envs), records in the slab row.
+    auto slab_env = [&](size_t c0) {   // first env of the tile as an index into [T][n_all]
+        const size_t tr = c0 / (size_t)a.tr_mb;
+        return ((size_t)a.tr_t0 + tr) * a.tr_n_all + a.tr_env_start + (c0 - tr * a.tr_mb);
+    };
+    auto rec_of = [&](int tile) {
+        const size_t c0 = (size_t)tile * kTileEnvs;
+        return a.rec + (MODE == kModeTrain ? slab_env(c0) : c0) * CFP_REC_BYTES;
+    };
+    auto term_of = [&](int tile) -> const float* {
+        return (MODE != kModeTrain && a.terminals) ? a.terminals + (size_t)tile * kTileEnvs
+                                                   : nullptr;
+    };
     if (full_rec && (int)blockIdx.x < pairs) {
         const int tid0 = threadIdx.x;
-        rec_fetch(a, (size_t)(2 * blockIdx.x) * kTileEnvs, pre[0], tid0);
+        rec_fetch(rec_of(2 * blockIdx.x), term_of(2 * blockIdx.x), pre[0], tid0);
         if (2 * (int)blockIdx.x + 1 < tiles)
-            rec_fetch(a, (size_t)(2 * blockIdx.x + 1) * kTileEnvs, pre[1], tid0);
+            rec_fetch(rec_of(2 * blockIdx.x + 1), term_of(2 * blockIdx.x + 1), pre[1], tid0);
     }
     for (int pair = blockIdx.x; pair < pairs; pair += gridDim.x) {
         // Lane constants are re-derived per pair from an opaque copy of the thread
@@ -349,6 +383,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
         L.wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         L.arow4 = L.l32 * XS4 + L.half;
         L.loff = (unsigned)((4 * L.half) * CFP_HIDDEN + L.l32);
+        L.loff3 = (unsigned)((4 * L.half) * CFP_GRU + L.l32);
         const int nt = L.wave & 1;   // head: row tile
         const int kh = L.wave >> 1;  // head: K half
         // tile X = 2*pair always exists; tile Y may be past the end (odd tile count)
@@ -409,8 +444,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
         auto fetch_next = [&]() {
             const int np = pair + (int)gridDim.x;
             if (np < pairs) {
-                rec_fetch(a, (size_t)(2 * np) * kTileEnvs, pre[0], tid);
-                if (2 * np + 1 < tiles) rec_fetch(a, (size_t)(2 * np + 1) * kTileEnvs, pre[1], tid);
+                rec_fetch(rec_of(2 * np), term_of(2 * np), pre[0], tid);
+                if (2 * np + 1 < tiles) rec_fetch(rec_of(2 * np + 1), term_of(2 * np + 1), pre[1], tid);
             }
         };
         if (full_rec && a.layers == 0) fetch_next();
@@ -428,10 +463,23 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             auto state_io = [&](int q) {
                 const int s = (q - 1) & 1, l = (q - 1) >> 1;
                 StateIO c;
-                if (s == 0 || hasY) {
+                c.pre_base = nullptr;
+                if (MODE == kModeTrain) {
+                    // stored state of (t, layer l, env) -> this layer's pre / output tiles
+                    const size_t se = slab_env(e0[s]);
+                    const size_t tt = se / a.tr_n_all, ee = se - tt * a.tr_n_all;
+                    c.st_base = a.state + ((tt * a.layers + l) * a.tr_n_all + ee) * CFP_HIDDEN +
+                                L.wave * 64;
+                    c.rs_base = a.tr_x[l + 1] + e0[s] * CFP_HIDDEN + L.wave * 64;
+                    c.pre_base = a.tr_pre[l] + e0[s] * CFP_GRU + L.wave * 64;
+                    if (s == 1 && !hasY) {
+                        c.st_base = c.rs_base = g_void_tile + L.wave * 64;
+                        c.pre_base = g_void_pre + L.wave * 64;
+                    }
+                } else if (s == 0 || hasY) {
                     const size_t off = (size_t)l * a.layer_stride + e0[s] * CFP_HIDDEN + L.wave * 64;
                     c.st_base = a.state + off;
-                    c.rs_base = HAS_RS ? a.r_state + off : nullptr;
+                    c.rs_base = MODE == kModeRecord ? a.r_state + off : nullptr;
                 } else {
                     c.st_base = g_void_tile + L.wave * 64;
                     c.rs_base = g_void_tile + L.wave * 64;
@@ -444,7 +492,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             for (int t = 0; t < 6; t++) accO[t] = zero16();
             ring_preload(bq, wp0, L);
             StateIO io = state_io(1);
-            gru_phase<true, false, HAS_RS>(accO, accO, bq, reinterpret_cast<const f4*>(lds_all[0]),
+            gru_phase<true, false, MODE>(accO, accO, bq, reinterpret_cast<const f4*>(lds_all[0]),
                                            wp0, nullptr, io, st, L);
             ring_preload(bq, wp0, L);
             state_load(io, st, L);
@@ -453,7 +501,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             for (int q = 1; q < Q; q++) {
 #pragma unroll
                 for (int t = 0; t < 6; t++) accN[t] = zero16();
-                gru_phase<true, true, HAS_RS>(accN, accO, bq,
+                gru_phase<true, true, MODE>(accN, accO, bq,
                                               reinterpret_cast<const f4*>(lds_all[q & 1]),
                                               wp0 + (size_t)(q >> 1) * wl, lds_all[(q - 1) & 1],
                                               io, st, L);
@@ -465,7 +513,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
                 for (int t = 0; t < 6; t++) accO[t] = accN[t];
             }
             if (full_rec) fetch_next();
-            gru_phase<false, true, HAS_RS>(accN, accO, bq, nullptr, nullptr, lds_all[(Q - 1) & 1],
+            gru_phase<false, true, MODE>(accN, accO, bq, nullptr, nullptr, lds_all[(Q - 1) & 1],
                                            io, st, L);
             __syncthreads();
             if (a.h3_out) {
@@ -559,12 +607,17 @@ int launch_forward(const FwdArgs& a, hipStream_t st) {
     const int pairs = (a.n / kTileEnvs + 1) / 2;
     const int grid = pairs < num_cus() ? pairs : num_cus();
     const dim3 g(grid), b(kFwdThreads);
-    if (a.variant == 1) {
-        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<1, true>), g, b, 0, st, a);
-        else hipLaunchKernelGGL((k_policy_forward<1, false>), g, b, 0, st, a);
+    if (a.train) {
+        CFP_REQUIRE(a.variant == 0 && a.rec && a.state && a.layers > 0 && !a.r_state &&
+                        a.tr_mb > 0 && a.tr_mb % kTileEnvs == 0 && a.h_enc_out == a.tr_x[0],
+                    "window recompute: bad arguments");
+        hipLaunchKernelGGL((k_policy_forward<0, kModeTrain>), g, b, 0, st, a);
+    } else if (a.variant == 1) {
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<1, kModeRecord>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward<1, kModePlain>), g, b, 0, st, a);
     } else {
-        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<0, true>), g, b, 0, st, a);
-        else hipLaunchKernelGGL((k_policy_forward<0, false>), g, b, 0, st, a);
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<0, kModeRecord>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward<0, kModePlain>), g, b, 0, st, a);
     }
     CFP_HIP_TRY(hipGetLastError());
     return 0;

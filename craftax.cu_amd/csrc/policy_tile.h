@@ -87,14 +87,15 @@ struct RecRegs {
     float term;   // terminal flag of env `tid` of the tile (threads 0..31)
 };
 
-__device__ __forceinline__ void rec_fetch(const FwdArgs& a, size_t e0, RecRegs& r, int tid) {
-    const u4* src = reinterpret_cast<const u4*>(a.rec + e0 * CFP_REC_BYTES);
+__device__ __forceinline__ void rec_fetch(const uint8_t* rec_tile, const float* term_tile,
+                                          RecRegs& r, int tid) {
+    const u4* src = reinterpret_cast<const u4*>(rec_tile);
 #pragma unroll
     for (int j = 0; j < kRecV4PerThread; j++) {
         const int i = tid + kFwdThreads * j;
         if (i < TILE_REC_V4) r.v[j] = __builtin_nontemporal_load(src + i);
     }
-    r.term = (tid < kTileEnvs && a.terminals) ? a.terminals[e0 + tid] : 0.0f;
+    r.term = (tid < kTileEnvs && term_tile) ? term_tile[tid] : 0.0f;
 }
 
 __device__ __forceinline__ void rec_scatter(const RecRegs& r, float* lds, float* term_s, int tid) {
@@ -169,6 +170,7 @@ struct Lane {
     int wave;          // 0..3, scalar
     int arow4;         // f4 index of this lane's A fragment in an x tile, + 2*kb
     unsigned loff;     // lane offset (floats) into a [32][256] state tile row set
+    unsigned loff3;    // likewise into a [32][768] pre-activation tile
 };
 
 constexpr int kEncPairs = kKbEnc / 2;                 // 53 steps of two K blocks

@@ -68,7 +68,8 @@ __global__ __launch_bounds__(128) void k_head_bwd_win(
     const float* __restrict__ ret, const double* __restrict__ adv_stats,
     float* __restrict__ dlogits, float* __restrict__ dvalue,
     double* __restrict__ block_loss, int t0, int cols, int mb, int n, int n_all,
-    int T_all, float clip_eps, float vf_coef, const float* __restrict__ ent_coef_p) {
+    int T_all, float clip_eps, float vf_coef, const float* __restrict__ ent_coef_p,
+    int logits_ld) {   // b_a == nullptr: the logits already carry their bias
     __shared__ double s_l[3][128];
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     double l_pg = 0.0, l_v = 0.0, l_e = 0.0;
@@ -83,11 +84,11 @@ __global__ __launch_bounds__(128) void k_head_bwd_win(
         const double var = adv_stats[1] * inv_count - m * m;
         const float adv_inv_std = 1.0f / ((float)sqrt(var > 0.0 ? var : 0.0) + 1e-8f);
         const float inv_batch = 1.0f / (float)(T_all * mb);
-        const float* lp = logits + (size_t)c * A;
+        const float* lp = logits + (size_t)c * logits_ld;
         float lg[A], pi[A];
         float mx = -1e30f;
 #pragma unroll
-        for (int a = 0; a < A; a++) { lg[a] = lp[a] + b_a[a]; mx = fmaxf(mx, lg[a]); }
+        for (int a = 0; a < A; a++) { lg[a] = lp[a] + (b_a ? b_a[a] : 0.0f); mx = fmaxf(mx, lg[a]); }
         float total = 0.0f;
 #pragma unroll
         for (int a = 0; a < A; a++) { pi[a] = expf(lg[a] - mx); total += pi[a]; }
@@ -484,7 +485,7 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     for (int l = 0; l <= tr->L; l++) TA(x[l], cc * H * sizeof(float));
     for (int l = 0; l < tr->L; l++) TA(preb[l], cc * G * sizeof(float));
     for (int l = 0; l < tr->L; l++) TA(dcarry[l], (size_t)mb * H * sizeof(float));
-    TA(logitsb, cc * A * sizeof(float));
+    TA(logitsb, cc * (A + 1) * sizeof(float));   // [cols][44] from the fused recompute, [cols][43] unfused
     TA(dlogits, cc * A * sizeof(float));
     TA(dvalue, cc * sizeof(float));
     TA(dh3b, cc * H * sizeof(float));
@@ -655,27 +656,51 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         const int Tw = t_end - t0;
         const int cols = Tw * mb;
         const size_t hc = (size_t)H * cols;
-        // ---- forward recompute of the window into tight columns
-        if (launch_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, kObsPad, st))
-            return 1;
-        if (gemm_enc_fwd_ld(cols, W_enc, tr->xobs, kObsPad, tr->x[0], st)) return 1;
-        if (cfp_add_bias(tr->x[0], b_enc, cols, stream)) return 1;
-        for (int l = 0; l < L; l++) {
-            if (cfp_gemm_fwd(G, cols, H, W_gru + (size_t)l * G * H, tr->x[l], tr->preb[l],
-                             stream))
+        // ---- forward recompute of the window into tight columns: one launch of the
+        // fused forward kernel in its window mode (stored state in, pre-activations
+        // and layer outputs out); with bf16 GEMM inputs the unfused chain below
+        const bool fused = cfp_get_gemm_bf16() == 0;
+        if (fused) {
+            FwdArgs fa{};
+            fill_forward_weights(p, fa);
+            fa.bf16 = 0;
+            fa.rec = tr->r_obs;
+            fa.state = tr->r_state;
+            fa.h_enc_out = tr->x[0];
+            fa.av_out = tr->logitsb;
+            fa.n = cols;
+            fa.layers = L;
+            fa.do_head = 1;
+            fa.train = 1;
+            fa.tr_t0 = t0; fa.tr_mb = mb; fa.tr_n_all = n; fa.tr_env_start = env_start;
+            for (int l = 0; l < L; l++) fa.tr_pre[l] = tr->preb[l];
+            for (int l = 0; l <= L; l++) fa.tr_x[l] = tr->x[l];
+            if (launch_forward(fa, st)) return 1;
+            // the dW_enc GEMM of the reverse pass still reads the fp32 feature matrix
+            if (launch_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, kObsPad, st))
                 return 1;
-            hipLaunchKernelGGL(k_mingru_epi_replay_win, dim3(grid1(hc)), dim3(256), 0, st,
-                               tr->preb[l], tr->x[l], tr->r_state, tr->x[l + 1], t0, hc,
-                               mb, n, env_start, l, L);
+        } else {
+            if (launch_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, kObsPad, st))
+                return 1;
+            if (gemm_enc_fwd_ld(cols, W_enc, tr->xobs, kObsPad, tr->x[0], st)) return 1;
+            if (cfp_add_bias(tr->x[0], b_enc, cols, stream)) return 1;
+            for (int l = 0; l < L; l++) {
+                if (cfp_gemm_fwd(G, cols, H, W_gru + (size_t)l * G * H, tr->x[l], tr->preb[l],
+                                 stream))
+                    return 1;
+                hipLaunchKernelGGL(k_mingru_epi_replay_win, dim3(grid1(hc)), dim3(256), 0, st,
+                                   tr->preb[l], tr->x[l], tr->r_state, tr->x[l + 1], t0, hc,
+                                   mb, n, env_start, l, L);
+            }
+            if (cfp_gemm_fwd(A, cols, H, W_a, tr->x[L], tr->logitsb, stream)) return 1;
         }
-        if (cfp_gemm_fwd(A, cols, H, W_a, tr->x[L], tr->logitsb, stream)) return 1;
         // ---- head gradients
         const int hb = (cols + 127) / 128;
         hipLaunchKernelGGL(k_head_bwd_win, dim3(hb), dim3(128), 0, st, tr->logitsb, tr->x[L],
-                           b_a, W_v, b_v, tr->r_act + env_start, tr->r_logprob + env_start,
+                           fused ? nullptr : b_a, W_v, b_v, tr->r_act + env_start, tr->r_logprob + env_start,
                            tr->adv + env_start, tr->ret + env_start, tr->stats, tr->dlogits,
                            tr->dvalue, tr->block_loss, t0, cols, mb, n, n, T, tr->cfg.clip,
-                           tr->cfg.vf, tr->d_ent);
+                           tr->cfg.vf, tr->d_ent, fused ? A + 1 : A);
         hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(256), 0, st, tr->block_loss, hb,
                            tr->loss_acc);
         if (cfp_gemm_dh(A, cols, W_a, tr->dlogits, tr->dh3b, stream)) return 1;
