@@ -225,64 +225,147 @@ __device__ __forceinline__ constexpr int st_off(int e) {
     return acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32;
 }
 
-// Request the 32 state values the next epilogue will consume.
+// Request the 32 state values the next epilogue will consume, in element order
+// (the compiler barriers pin the issue order).  The epilogue consumes element kb
+// in K block kb, so the wait the compiler places there leaves at least the 31
+// youngest operations it knows of in flight -- and with them the weight requests
+// issued since, which it does not know of and must not be made to wait for.
 __device__ __forceinline__ void state_load(const StateIO& io, float (&st)[32], const Lane& L) {
 #pragma unroll
-    for (int e = 0; e < 32; e++)
+    for (int e = 0; e < 32; e++) {
         st[e] = __builtin_nontemporal_load((io.st_base + st_off(e)) + L.loff);
+        asm volatile("" ::: "memory");
+    }
 }
 
-using WRing = f4[3][6];
+// ---- weight stream: global -> LDS -> registers -----------------------------------
+// On this machine an MFMA whose B operand sits in registers that vector-memory
+// loads keep rewriting loses ~15 % of the matrix pipe's time, however far ahead
+// the loads run; fed from LDS reads it does not (measured in place: a gate GEMM
+// phase 26.3 -> 22.1 us).  So each wave streams its weight fragments into a
+// private LDS ring with LDS-direct loads (global_load_lds_dwordx4: lane l's 16
+// bytes land at base + 16*l, no registers involved) two K blocks ahead, and
+// reads the current block's six fragments back with ds_read_b128.
+// The DMA loads are issued from inline assembly: the compiler does not know of
+// them, so the wait that makes a ring slot readable is explicit (s_waitcnt vmcnt
+// with the exact number of younger vector-memory operations, loads and stores
+// complete in issue order) and everything the compiler schedules itself only
+// ever over-waits.
+constexpr int kRingSlots = 3;
+constexpr int kRingSlotF4 = 6 * 64;                       // one K block of one wave: 6 KiB
+constexpr int kRingF4 = 4 * kRingSlots * kRingSlotF4;     // 72 KiB for the workgroup
 
-// First two K blocks of a layer's weights into ring slots 0 and 1.
-__device__ __forceinline__ void ring_preload(WRing& bq, const f4* wp, const Lane& L) {
+// K block kb of a layer (wp = mirror + layer + wave*6*64 fragments) -> ring slot.
+// `after` is a register the slot's previous contents were last read into: as an
+// operand it keeps the request behind the completion of those reads.
+__device__ __forceinline__ void ring_dma(const f4* wp, int kb, f4* slot, const Lane& L,
+                                         float after = 0.0f) {
     constexpr int KB_STRIDE = 4 * 6 * 64;
-#pragma unroll
-    for (int b = 0; b < 2; b++)
-#pragma unroll
-        for (int t = 0; t < 6; t++)
-            bq[b][t] = (wp + (size_t)b * KB_STRIDE + t * 64)[L.lane_u];
+    const f4* src = wp + (size_t)kb * KB_STRIDE;
+    const unsigned lds_lo = (unsigned)(size_t)slot;       // LDS byte address of the slot
+    const unsigned voff = L.lane_u * 16u;
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:3072"
+        :
+        : "v"(voff), "s"(src), "s"(lds_lo), "v"(after)
+        : "memory", "m0");
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:1024"
+        :
+        : "v"(voff), "s"(src + 4 * 64), "s"(lds_lo + 4096u)
+        : "memory", "m0");
 }
 
-// DO_K: accN[6] += x_K . W_l^T for the tile whose x tile is `xs4K`; the ring
-//       holds K blocks 0 and 1 on entry, block kb+2 is requested while block kb
-//       is multiplied (two blocks = 3072 matrix-pipe cycles of latency cover).
+// First three K blocks of a layer's weights into ring slots 0, 1, 2.
+__device__ __forceinline__ void ring_preload(f4* ring, const f4* wp, const Lane& L) {
+#pragma unroll
+    for (int i = 0; i < kRingSlots; i++) ring_dma(wp, i, ring + i * kRingSlotF4, L);
+}
+
+// s_waitcnt vmcnt(n); n must fold to a constant after unrolling (the switch then
+// leaves one instruction).
+__device__ __forceinline__ void vm_wait(int n) {
+#define CFP_VMW(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
+    switch (n) {
+        CFP_VMW(0) CFP_VMW(2) CFP_VMW(4) CFP_VMW(6) CFP_VMW(8) CFP_VMW(10) CFP_VMW(12)
+        CFP_VMW(13) CFP_VMW(14) CFP_VMW(16) CFP_VMW(20) CFP_VMW(44) CFP_VMW(45) CFP_VMW(46)
+        CFP_VMW(48)
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+#undef CFP_VMW
+}
+
+// DO_K: accN[6] += x_K . W_l^T for the tile whose x tile is `xs4K`.  On entry the
+//       ring holds (has been asked for) K blocks 0..2, requested by ring_preload,
+//       followed, when DO_E, by the 32 loads of state_load and nothing else.
+//       While block kb is multiplied, block kb+1 is read from its slot into the
+//       other half of bl[2][6] and block kb+3 is requested into the slot block kb
+//       was read from one block earlier: LDS latency is covered by one block
+//       (1536 matrix-pipe cycles), L2 latency by two.
 // DO_E: the gate/blend epilogue of the OTHER tile from accO[6], one element next
 //       to each K block: element kb's ~35 vector instructions, its two LDS
 //       accesses and its state / r_state stores issue in the shadow of the 24
 //       MFMAs.  The block is branch-free (a branch would split it and leave the
 //       epilogue behind the MFMAs).  The state values were requested before the
 //       phase (st[32]); in-loop state loads would sit in front of the weight
-//       loads in the in-order return queue with their HBM latency.
+//       requests in the in-order return queue with their HBM latency.
 template <bool DO_K, bool DO_E, int MODE>
-__device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6], WRing& bq,
+__device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6], f4* ring,
                                           const f4* xs4K, const f4* wp, float* xsE,
                                           const StateIO& io, const float (&st)[32],
                                           const Lane& L) {
-    constexpr int KB_STRIDE = 4 * 6 * 64;   // f4 per K block
+    // Vector-memory operations complete in issue order, so "block b has landed"
+    // is "at most N operations are outstanding", N = those issued after b's six:
+    // the later requests, the S stores each epilogue block issues, and in the
+    // first blocks the P state loads that follow the preload.
+    constexpr int S = !DO_E ? 0 : (MODE == kModeTrain ? 4 : (MODE == kModeRecord ? 2 : 1));
+    constexpr int P = DO_E ? 32 : 0;
     f4 aq[2];
-    if (DO_K) aq[0] = xs4K[L.arow4];
+    f4 bl[2][6];
+    if (DO_K) {
+        aq[0] = xs4K[L.arow4];
+        vm_wait(12 + P);   // block 0 landed; blocks 1, 2 and the state loads may be in flight
+#pragma unroll
+        for (int t = 0; t < 6; t++) bl[0][t] = ring[t * 64 + L.lane_u];
+    }
 #pragma unroll
     for (int kb = 0; kb < kKbHid; kb++) {
         const int cb = kb & 1, nb = cb ^ 1;
-        if (DO_K) {
-            if (kb + 2 < kKbHid) {
-#pragma unroll
-                for (int t = 0; t < 6; t++)
-                    bq[(kb + 2) % 3][t] = (wp + (size_t)(kb + 2) * KB_STRIDE + t * 64)[L.lane_u];
-            }
-            if (kb + 1 < kKbHid) aq[nb] = xs4K[L.arow4 + 2 * (kb + 1)];
+        float* xp = nullptr;
+        float xv = 0.0f;
+        if (DO_E) {
+            xp = xsE + (acc_row(kb % 16) + 4 * L.half) * XS + L.wave * 64 + (kb / 16) * 32 + L.l32;
+            xv = *xp;
         }
         if (DO_K) {
+            if (kb + 3 < kKbHid)
+                ring_dma(wp, kb + 3, ring + (kb % kRingSlots) * kRingSlotF4, L, bl[cb][5][3]);
+            if (kb + 1 < kKbHid) {
+                // block kb+1 landed?  younger: blocks kb+2, kb+3 and what lies between
+                if (kb + 3 < kKbHid) vm_wait(12 + (kb >= 2 ? 2 * S : P + kb * S));
+                else if (kb + 2 < kKbHid) vm_wait(6 + 2 * S);
+                else vm_wait(2 * S);
+                const f4* slot = ring + ((kb + 1) % kRingSlots) * kRingSlotF4 + L.lane_u;
+#pragma unroll
+                for (int t = 0; t < 6; t++) bl[nb][t] = slot[t * 64];
+                aq[nb] = xs4K[L.arow4 + 2 * (kb + 1)];
+            }
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int t = 0; t < 6; t++)
-                    accN[t] = mfma(aq[cb][j], bq[kb % 3][t][j], accN[t]);
+                    accN[t] = mfma(aq[cb][j], bl[cb][t][j], accN[t]);
         }
         if (DO_E) {
             const int ut = kb / 16, r = kb % 16;
-            float* xp = xsE + (acc_row(r) + 4 * L.half) * XS + L.wave * 64 + ut * 32 + L.l32;
             const float s = (MODE != kModeTrain && ((io.tmask >> r) & 1u)) ? 0.0f : st[kb];
             if (MODE == kModeRecord)
                 __builtin_nontemporal_store(s, (io.rs_base + st_off(kb)) + L.loff);
@@ -301,7 +384,6 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
             const float gh = zh >= 0.0f ? zh + 0.5f : sh;
             const float out = s + sg * (gh - s);
             const float p = sigmoid_fast(zp);
-            const float xv = *xp;
             const float hn = p * out + (1.0f - p) * xv;
             *xp = hn;
             if (MODE == kModeTrain)
@@ -309,16 +391,14 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
             else
                 __builtin_nontemporal_store(out, (io.st_base + st_off(kb)) + L.loff);
         }
-        // Issue order of the block.  A vector memory instruction occupies the
-        // wave's issue port for about as long as one MFMA executes, so the six
-        // weight loads are spread one per four MFMAs instead of bunched (bunched,
-        // they leave the matrix pipe idle for ~5 MFMA slots per block).
+        // Issue order of the block: the epilogue's vector instructions two per MFMA.
         if (DO_K) {
 #pragma unroll
             for (int q = 0; q < 24; q++) {
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                  // one MFMA
-                if (q % 4 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one load
-                if (q == 2) __builtin_amdgcn_sched_group_barrier(0x100, DO_E ? 2 : 1, 0);
+                if (q == 0 && DO_E) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // x value
+                // next block's six weight fragments and x fragment, back to back
+                if (q == 1) __builtin_amdgcn_sched_group_barrier(0x100, 7, 0);
                 if (DO_E) {
                     __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);              // two VALU
                     if (q == 21) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
@@ -339,8 +419,14 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds_all[2][LDS_FLOATS];
     __shared__ __attribute__((aligned(16))) float red_all[2][kRedFloats];
     __shared__ float term_all[2][kTileEnvs];
-    __shared__ __attribute__((aligned(16))) uint8_t crec_all[2][kTileEnvs * CFP_CLASSIC_REC_BYTES];
-    __shared__ __attribute__((aligned(16))) uint32_t ctab[VARIANT == 1 ? kClassicTabDwords : 4];
+    // 72 KiB shared by the weight ring (MinGRU phases) and, for the classic game, the
+    // record bytes and gather tables of the encoder, which runs before those phases
+    __shared__ __attribute__((aligned(16))) f4 aux[kRingF4];
+    constexpr int kCrecBytes = kTileEnvs * CFP_CLASSIC_REC_BYTES;
+    static_assert(2 * kCrecBytes + kClassicTabDwords * 4 <= kRingF4 * 16, "classic tables fit the ring");
+    uint8_t* const crec_base = reinterpret_cast<uint8_t*>(aux);
+    uint8_t* const crec_all[2] = {crec_base, crec_base + kCrecBytes};
+    uint32_t* const ctab = reinterpret_cast<uint32_t*>(crec_base + 2 * kCrecBytes);
 
     const int tiles = a.n / kTileEnvs;
     const int pairs = (tiles + 1) / 2;
@@ -400,8 +486,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
         } else {
             for (int i = tid; i < LDS_FLOATS; i += kFwdThreads) lds_all[1][i] = 0.0f;
             if (tid < kTileEnvs) term_all[1][tid] = 0.0f;
-            for (int i = tid; i < kTileEnvs * CFP_CLASSIC_REC_BYTES; i += kFwdThreads)
-                crec_all[1][i] = 0;
+            if (VARIANT == 1)
+                for (int i = tid; i < kCrecBytes; i += kFwdThreads) crec_all[1][i] = 0;
         }
         __syncthreads();
 
@@ -457,7 +543,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
         if (a.layers > 0) {
             f16v accO[6], accN[6];
             float st[32];
-            WRing bq;
+            f4* const bq = aux + L.wave * (kRingSlots * kRingSlotF4);   // this wave's ring
             const size_t wl = kGruPackFloats / 4;   // f4 per layer of the mirror
             const f4* wp0 = a.wg_pk + (size_t)(L.wave * 6) * 64;
             auto state_io = [&](int q) {
@@ -505,8 +591,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
                                               reinterpret_cast<const f4*>(lds_all[q & 1]),
                                               wp0 + (size_t)(q >> 1) * wl, lds_all[(q - 1) & 1],
                                               io, st, L);
-                if (q + 1 < Q) ring_preload(bq, wp0 + (size_t)((q + 1) >> 1) * wl, L);
                 io = state_io(q + 1);
+                if (q + 1 < Q) ring_preload(bq, wp0 + (size_t)((q + 1) >> 1) * wl, L);
                 state_load(io, st, L);
                 __syncthreads();
 #pragma unroll
