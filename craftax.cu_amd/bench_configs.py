@@ -5,6 +5,9 @@
   ppo_update      PPO update, 4096 envs x 64 steps = 262 144 samples, one
                   minibatch = all envs: windowed recompute backward + Adam
   classic_1m      classic-game policy forward, 1 048 576 envs, 148-byte records
+  record_kernels  the HBM-bound byte kernels at 65 536 envs: state -> 996-byte
+                  records (fuzzed reference states of tests/golden, tiled) and
+                  records -> fp32 features
 
 Usage:  python craftax.cu_amd/bench_configs.py [--reps 10] [--only NAME]
 The headline workload (262 144 envs) is bench.py at the repository root."""
@@ -109,6 +112,32 @@ def classic_1m(pkg, torch, reps):
     return out
 
 
+def record_kernels(pkg, torch, reps):
+    import numpy as np
+    n = 65536
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    g = np.load(os.path.join(root, "tests", "golden", "record_fixtures.npz"))
+    sc, pl = g["fuzz_scalars"], g["fuzz_planes"]          # [384][S], [384][3][2304]
+    idx = np.arange(n) % sc.shape[0]
+    scalars = torch.from_numpy(np.ascontiguousarray(sc[idx])).cuda()
+    planes = torch.from_numpy(np.ascontiguousarray(pl[idx])).cuda().view(-1)
+    plane = pl.shape[2]
+    rec = torch.empty(n, 996, dtype=torch.uint8, device="cuda")
+    xobs = torch.empty(n, 843, device="cuda")
+    P = pkg.policy
+    ms_r = _time(torch, lambda: P.record_obs(scalars, planes, planes[plane:], planes[2 * plane:],
+                                             n, 3 * plane, 0, rec=rec), reps)
+    ms_x = _time(torch, lambda: P.expand_obs(rec, n, xobs=xobs), reps)
+    # algorithmic bytes per env: scalars + 99 cells x 3 plane bytes gathered + 996 written;
+    # 996 read + 843 x 4 written
+    b_r, b_x = sc.shape[1] + 99 * 3 + 996, 996 + 843 * 4
+    return {"workload": "record_kernels", "envs": n,
+            "record_obs": {"ms": ms_r, "envs_per_s": n / ms_r * 1e3, "bytes_per_env": b_r,
+                           "gb_per_s": b_r * n / ms_r / 1e6, "frac_hbm_peak": b_r * n / ms_r / 1e6 / 8000},
+            "expand_obs": {"ms": ms_x, "envs_per_s": n / ms_x * 1e3, "bytes_per_env": b_x,
+                           "gb_per_s": b_x * n / ms_x / 1e6, "frac_hbm_peak": b_x * n / ms_x / 1e6 / 8000}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=10)
@@ -118,7 +147,7 @@ def main():
     import __graft_entry__ as ge
     pkg = ge.load_package()
     assert torch.cuda.is_available(), "bench_configs.py needs a GPU"
-    for fn in (forward_65536, ppo_update, classic_1m):
+    for fn in (forward_65536, ppo_update, classic_1m, record_kernels):
         if args.only and fn.__name__ != args.only:
             continue
         print(json.dumps(fn(pkg, torch, args.reps)), flush=True)

@@ -16,11 +16,14 @@
 //   ENC(X+Y) | bias | K(X,0) | K(Y,0)+epi(X,0) | K(X,1)+epi(Y,0) | ...
 //   ... | K(Y,L-1)+epi(X,L-1) | epi(Y,L-1) | HEAD(X) HEAD(Y) | reduce, store
 // ("|" = workgroup barrier).  `sched_group_barrier` pins the issue order inside
-// a K block (1 MFMA : 2 VALU, one weight load per four MFMAs).  Measured on
-// MI355X, every non-MFMA instruction of the issuing wave costs the matrix pipe
-// about its own issue time (a 16-byte global load ~40 cycles, wherever it
-// hits), so the design minimises instructions per MFMA rather than latency:
-// 6 weight loads + 1 LDS read + ~35 epilogue instructions per 24 MFMAs.
+// a K block (1 MFMA : 2 VALU).  Measured on MI355X with v_mfma_f32_32x32x2_f32
+// (64 cycles in the matrix pipe), one wave per SIMD: every vector or LDS
+// instruction the MFMA-issuing wave issues in between delays its next MFMA by
+// about 8.5 cycles (12.5 for a transcendental), a 16-byte global load into
+// registers by 40-60.  So the design minimises instructions per MFMA rather than
+// latency: per 24 MFMAs, 6 LDS-direct weight requests (no registers written),
+// 7 LDS reads and ~25 epilogue instructions.  The shader clock under this load
+// is 2.06-2.13 GHz, not the 2.4 GHz behind the 157.3 TFLOP/s peak.
 //
 // Within the workgroup, wave w owns hidden units [64w, 64w+64).  MFMA operand
 // convention (v_mfma_f32_32x32x2_f32): A = activations (row = env), B = weights
@@ -31,11 +34,13 @@
 //            W_enc fragments streamed once per pair from the MFMA-ordered
 //            mirror in L2 and used for both tiles (4 accumulators), two K
 //            blocks per step, weights three steps deep in registers
-//   layer:   6 accumulators (zh, zg, zp for 2 unit tiles) over K = 256, weights
-//            three K blocks deep; the first two blocks and the 32 state values
-//            of the NEXT phase are requested before the barrier that ends the
-//            current one; state and r_state leave through non-temporal stores
-//            next to each epilogue element; h' goes back into the x tile
+//   layer:   6 accumulators (zh, zg, zp for 2 unit tiles) over K = 256; weights
+//            go L2 -> per-wave LDS ring (LDS-direct loads, three K blocks ahead)
+//            -> registers (one block ahead); the first three blocks and the 32
+//            state values of the NEXT phase are requested before the barrier
+//            that ends the current one; state and r_state leave through
+//            non-temporal stores next to each epilogue element; h' goes back
+//            into the x tile
 //   heads:   2 row tiles x 2 K halves over the 4 waves, reduced through LDS.
 #include "policy_tile.h"
 
@@ -239,18 +244,19 @@ __device__ __forceinline__ void state_load(const StateIO& io, float (&st)[32], c
 }
 
 // ---- weight stream: global -> LDS -> registers -----------------------------------
-// On this machine an MFMA whose B operand sits in registers that vector-memory
-// loads keep rewriting loses ~15 % of the matrix pipe's time, however far ahead
-// the loads run; fed from LDS reads it does not (measured in place: a gate GEMM
-// phase 26.3 -> 22.1 us).  So each wave streams its weight fragments into a
-// private LDS ring with LDS-direct loads (global_load_lds_dwordx4: lane l's 16
-// bytes land at base + 16*l, no registers involved) two K blocks ahead, and
-// reads the current block's six fragments back with ds_read_b128.
-// The DMA loads are issued from inline assembly: the compiler does not know of
-// them, so the wait that makes a ring slot readable is explicit (s_waitcnt vmcnt
-// with the exact number of younger vector-memory operations, loads and stores
-// complete in issue order) and everything the compiler schedules itself only
-// ever over-waits.
+// A 16-byte global load into registers costs the MFMA-issuing wave 40-60 cycles
+// of matrix-pipe time on this machine wherever it hits; an LDS-direct load
+// (global_load_lds_dwordx4: lane l's 16 bytes land at M0 base + 16*l, no
+// registers involved) plus the LDS read that fetches the fragment cost about
+// half of that together (a gate GEMM phase: 54.6k -> 51.0k cycles, of 49.2k
+// ideal).  So each wave streams its weight fragments into a private LDS ring,
+// three K blocks ahead, and reads the next block's six fragments back with
+// ds_read_b128 while the current block multiplies.
+// The LDS-direct loads are issued from inline assembly: the compiler does not
+// know of them, so the wait that makes a ring slot readable is explicit
+// (s_waitcnt vmcnt with the exact number of younger vector-memory operations;
+// loads and stores complete in issue order) and every wait the compiler places
+// for its own loads only ever over-waits.
 constexpr int kRingSlots = 3;
 constexpr int kRingSlotF4 = 6 * 64;                       // one K block of one wave: 6 KiB
 constexpr int kRingF4 = 4 * kRingSlots * kRingSlotF4;     // 72 KiB for the workgroup

@@ -186,6 +186,71 @@ __global__ void k_expand_obs(const uint8_t* __restrict__ r_obs,
     xobs[idx] = x;
 }
 
+// Four features per thread, for rows whose width is a multiple of four floats
+// and 16-byte aligned: one dword of the record in (four map bytes, or one to four
+// tail floats), one 16-byte store out.  792 = 4 * 198, so a group never straddles
+// the map / tail boundary.
+__global__ void k_expand_obs_v4(const uint8_t* __restrict__ r_obs, f4* __restrict__ xobs4,
+                                int t0, size_t total4, int mb, int n, int env_start, int ld4) {
+    static_assert(CFP_OBS_MAP % 4 == 0, "map bytes end on a dword");
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total4) return;
+    const unsigned w = (unsigned)(idx / (unsigned)ld4);
+    const int f = 4 * (int)(idx - (size_t)w * (unsigned)ld4);
+    const unsigned tr = w / (unsigned)mb;
+    const unsigned el = w - tr * (unsigned)mb;
+    const uint32_t* rec = reinterpret_cast<const uint32_t*>(
+        r_obs + (((size_t)t0 + tr) * (size_t)n + env_start + el) * CFP_REC_BYTES);
+    f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (f < CFP_OBS_MAP) {
+        const uint32_t b = __builtin_nontemporal_load(rec + (f >> 2));
+        v[0] = (float)(b & 0xffu);
+        v[1] = (float)((b >> 8) & 0xffu);
+        v[2] = (float)((b >> 16) & 0xffu);
+        v[3] = (float)(b >> 24);
+    } else {
+        const uint32_t* tail = rec + CFP_OBS_MAP / 4 + (f - CFP_OBS_MAP);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (f + j < CFP_OBS) v[j] = __uint_as_float(tail[j]);
+    }
+    __builtin_nontemporal_store(v, xobs4 + idx);
+}
+
+// Any row width, output base 16-byte aligned: thread i writes flat floats
+// 4i .. 4i+3 with one 16-byte store; a group may run over the end of a row
+// into the next sample.
+__global__ void k_expand_obs_flat4(const uint8_t* __restrict__ r_obs, float* __restrict__ xobs,
+                                   int t0, size_t total, int mb, int n, int env_start, int ld) {
+    const size_t i0 = 4 * ((size_t)blockIdx.x * blockDim.x + threadIdx.x);
+    if (i0 >= total) return;
+    unsigned w = (unsigned)(i0 / (unsigned)ld);
+    int f = (int)(i0 - (size_t)w * (unsigned)ld);
+    auto rec_of = [&](unsigned ww) {
+        const unsigned tr = ww / (unsigned)mb;
+        const unsigned el = ww - tr * (unsigned)mb;
+        return r_obs + (((size_t)t0 + tr) * (size_t)n + env_start + el) * CFP_REC_BYTES;
+    };
+    const uint8_t* rec = rec_of(w);
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float x = 0.0f;                                   // padding of a widened row
+        if (i0 + j >= total) {
+        } else if (f < CFP_OBS_MAP) x = (float)rec[f];
+        else if (f < CFP_OBS)
+            x = __uint_as_float(reinterpret_cast<const uint32_t*>(rec + CFP_OBS_MAP)[f - CFP_OBS_MAP]);
+        v[j] = x;
+        if (++f == ld) { f = 0; rec = rec_of(++w); }      // past the last sample: not read
+    }
+    if (i0 + 4 <= total) {
+        const f4 o = {v[0], v[1], v[2], v[3]};
+        __builtin_nontemporal_store(o, reinterpret_cast<f4*>(xobs + i0));
+    } else {
+        for (int j = 0; i0 + j < total; j++) xobs[i0 + j] = v[j];
+    }
+}
+
 __global__ void k_add_bias(float* __restrict__ h, const float* __restrict__ b,
                            size_t total) {
     size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -228,7 +293,22 @@ using namespace cfp;
 namespace cfp {
 int launch_expand_obs(const uint8_t* r_obs, float* xobs, int t0, int count, int mb, int n,
                       int env_start, int ld, hipStream_t st) {
+    if (ld % 4 == 0 && (reinterpret_cast<uintptr_t>(xobs) & 15u) == 0) {
+        const size_t total4 = (size_t)count * (ld / 4);
+        hipLaunchKernelGGL(k_expand_obs_v4, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0,
+                           st, r_obs, reinterpret_cast<f4*>(xobs), t0, total4, mb, n, env_start,
+                           ld / 4);
+        CFP_HIP_TRY(hipGetLastError());
+        return 0;
+    }
     const size_t total = (size_t)count * ld;
+    if (ld >= 4 && (reinterpret_cast<uintptr_t>(xobs) & 15u) == 0) {
+        const size_t groups = (total + 3) / 4;
+        hipLaunchKernelGGL(k_expand_obs_flat4, dim3((unsigned)((groups + 255) / 256)), dim3(256),
+                           0, st, r_obs, xobs, t0, total, mb, n, env_start, ld);
+        CFP_HIP_TRY(hipGetLastError());
+        return 0;
+    }
     hipLaunchKernelGGL(k_expand_obs, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                        r_obs, xobs, t0, total, mb, n, env_start, ld);
     CFP_HIP_TRY(hipGetLastError());

@@ -94,6 +94,15 @@ def test_expand_obs_bit_exact(pkg, cuda):
     x = pkg.policy.expand_obs(_t(rec, cuda), 320)
     torch.cuda.synchronize()
     assert np.array_equal(x.cpu().numpy().view(np.uint32), expand_records(rec).view(np.uint32))
+    # output base not 16-byte aligned (element-wise kernel) and a ragged float count
+    big = torch.zeros(321 * 843 + 1, device=cuda)
+    rec321 = np.concatenate([rec, rec[:1]])
+    pkg.policy.expand_obs(_t(rec321, cuda), 321, xobs=big[1:].view(321, 843))
+    x2 = pkg.policy.expand_obs(_t(rec321, cuda), 321)
+    torch.cuda.synchronize()
+    want321 = expand_records(rec321).view(np.uint32)
+    assert np.array_equal(big[1:].view(321, 843).cpu().numpy().view(np.uint32), want321)
+    assert np.array_equal(x2.cpu().numpy().view(np.uint32), want321)
     # trainer window addressing: t0, mb, n, env_start
     slab = rng.integers(0, 256, (4, 8, 996), dtype=np.uint8)
     x = pkg.policy.expand_obs(_t(slab, cuda), count=2 * 3, t0=1, mb=3, n=8, env_start=2)
