@@ -37,6 +37,7 @@ static void policy_release(cfp_policy* p) {
     if (p->stream) (void)hipStreamDestroy(p->stream);
     (void)hipFree(p->params);
     (void)hipFree(p->we_pk);
+    (void)hipFree(p->we_s3);
     (void)hipFree(p->wg_pk);
     (void)hipFree(p->wav_pk);
     (void)hipFree(p->we_bf);
@@ -118,6 +119,7 @@ static int policy_create(cfp_policy** out, int num_envs, int layers, uint64_t se
     } while (0)
     CFP_ALLOC(p->params, p->param_count * sizeof(float));
     CFP_ALLOC(p->we_pk, (size_t)(kKbEnc + kEncPadBlocks) * 2048 * sizeof(float));
+    CFP_ALLOC(p->we_s3, kEncSplitBf16 * sizeof(uint16_t));
     CFP_ALLOC(p->wg_pk,
               ((size_t)layers * kGruPackFloats + 4 * 6 * 64 * 4) * sizeof(float));
     CFP_ALLOC(p->wav_pk, kAvPackFloats * sizeof(float));
@@ -228,6 +230,8 @@ int cfp_policy_refresh_weights(cfp_policy* p, void* stream) {
     if (launch_pack_weights(p->params, p->layers, p->variant, p->we_pk, p->wg_pk, p->wav_pk,
                             (hipStream_t)stream) != 0)
         return 1;
+    if (launch_pack_enc_split(p->params, p->layers, p->variant, p->we_s3, (hipStream_t)stream) != 0)
+        return 1;
     return launch_pack_weights_bf16(p->params, p->layers, p->variant, p->we_bf, p->wg_bf,
                                     p->wav_bf, (hipStream_t)stream);
 }
@@ -254,6 +258,7 @@ static void fill_weights(const cfp_policy* p, FwdArgs& a) { cfp::fill_forward_we
 void cfp::fill_forward_weights(const cfp_policy* p, FwdArgs& a) {
     const Arena ar = arena_of(p->variant, p->layers);
     a.we_pk = reinterpret_cast<const f4*>(p->we_pk);
+    a.we_s3 = reinterpret_cast<const u4*>(p->we_s3);
     a.w_enc = p->params + ar.w_enc;
     a.b_enc = p->params + ar.b_enc;
     a.wg_pk = reinterpret_cast<const f4*>(p->wg_pk);

@@ -29,6 +29,8 @@ constexpr int kEncPadBlocks = 4;                   // encoder mirror: prefetch o
 
 // MFMA-ordered weight mirror sizes, in floats.
 constexpr size_t kEncPackFloats = (size_t)kObsPad * CFP_HIDDEN;
+constexpr int kKb16Split = (CFP_OBS_MAP + 15) / 16;                   // 50 K blocks of 16 map bytes
+constexpr size_t kEncSplitBf16 = (size_t)kKb16Split * 4 * 6 * 64 * 8;  // bf16 elements of the split mirror
 constexpr size_t kGruPackFloats = (size_t)CFP_GRU * CFP_HIDDEN;   // per layer
 constexpr size_t kAvPackFloats = (size_t)kAvPad * CFP_HIDDEN;
 
@@ -70,6 +72,7 @@ struct FwdArgs {
     const uint8_t* rec;      // [n][996] or null (then x0 is the layer-0 input)
     const float* x0;         // [n][256] or null
     const f4* we_pk;         // packed encoder weights
+    const u4* we_s3;         // map rows of W_enc as three bf16 terms (hi, mid, lo) per weight
     const float* b_enc;
     const f4* wg_pk;         // packed gate weights, layers back to back
     const f4* wav_pk;        // packed head weights
@@ -108,6 +111,8 @@ int launch_forward_bf16(const FwdArgs& a, hipStream_t st);   // called by launch
 int launch_pack_weights_bf16(const float* params, int layers, int variant, uint16_t* we_bf,
                              uint16_t* wg_bf, uint16_t* wav_bf, hipStream_t st);
 
+int launch_pack_enc_split(const float* params, int layers, int variant, uint16_t* we_s3,
+                          hipStream_t st);
 int launch_pack_weights(const float* params, int layers, int variant, float* we_pk,
                         float* wg_pk, float* wav_pk, hipStream_t st);
 

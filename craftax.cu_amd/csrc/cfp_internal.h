@@ -10,6 +10,7 @@ struct cfp_policy {
     size_t param_count = 0;
     float* params = nullptr;
     float* we_pk = nullptr;
+    uint16_t* we_s3 = nullptr;    // map rows of W_enc split in three bf16 terms
     float* wg_pk = nullptr;
     float* wav_pk = nullptr;
     uint16_t* we_bf = nullptr;    // bf16 mirrors (MFMA 32x32x16 order)

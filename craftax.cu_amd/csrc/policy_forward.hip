@@ -513,7 +513,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             f16v eacc[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) eacc[t] = zero16();
-            encoder_gemm(a, lds_all[0], lds_all[1], L, eacc);
+            encoder_gemm_split(a, lds_all[0], lds_all[1], L, eacc);
             __syncthreads();   // every wave is done with the record bytes
 #pragma unroll
             for (int s = 0; s < 2; s++)
@@ -757,6 +757,37 @@ __global__ void k_pack_av(const float* __restrict__ W_a,
     if (arow < actions) v = W_a[arow * CFP_HIDDEN + k];
     else if (arow == actions) v = W_v[k];
     out[idx] = v;
+}
+
+// Map rows of W_enc as three bf16 terms per weight, MFMA 32x32x16 order: one
+// 16-byte element (eight bf16) per lane, K block of 16 and term; lane l carries
+// k = 16*kb + 8*(l/32) + j of column l%32 of its 32-wide tile.  Features past the
+// map (the fp32 tail runs on the fp32 mirror) carry zeros.
+__global__ void k_pack_enc_split(const float* __restrict__ W_enc, __bf16* __restrict__ out,
+                                 int total) {
+    int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    int j = idx & 7, lane = (idx >> 3) & 63, q = idx >> 9;
+    int s = q % 3, ut = (q / 3) & 1, wave = (q / 6) & 3, kb = q / 24;
+    int unit = wave * 64 + ut * 32 + (lane & 31);
+    int f = 16 * kb + 8 * (lane >> 5) + j;
+    const float w = f < CFP_OBS_MAP ? W_enc[(size_t)f * CFP_HIDDEN + unit] : 0.0f;
+    const __bf16 hi = (__bf16)w;
+    const float r1 = w - (float)hi;
+    const __bf16 mid = (__bf16)r1;
+    const __bf16 lo = (__bf16)(r1 - (float)mid);
+    out[idx] = s == 0 ? hi : (s == 1 ? mid : lo);
+}
+
+int launch_pack_enc_split(const float* params, int layers, int variant, uint16_t* we_s3,
+                          hipStream_t st) {
+    if (variant != 0) return 0;   // the classic encoder gathers from the unpacked W_enc
+    const Arena ar = arena_of(variant, layers);
+    const int total = (int)kEncSplitBf16;
+    hipLaunchKernelGGL(k_pack_enc_split, dim3((total + 255) / 256), dim3(256), 0, st,
+                       params + ar.w_enc, reinterpret_cast<__bf16*>(we_s3), total);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
 }
 
 int launch_pack_weights(const float* params, int layers, int variant, float* we_pk,

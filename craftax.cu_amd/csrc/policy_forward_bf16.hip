@@ -24,39 +24,16 @@ namespace cfp {
 
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f8 __attribute__((ext_vector_type(8)));
 
 constexpr int kKb16Enc = kObsPad / 16;        // 53 K blocks of 16
 constexpr int kKb16Map = CFP_OBS_MAP / 16;    // 49 all-map blocks; block 49 is half map, half tail
 constexpr int kKb16Hid = CFP_HIDDEN / 16;     // 16
 
-__device__ __forceinline__ f16v mfma16(const u4& a, const u4& b, f16v c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
 // eight fp32 -> eight bf16, round to nearest even
 __device__ __forceinline__ u4 to_bf16x8(const f4& lo, const f4& hi) {
     f8 v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     return __builtin_bit_cast(u4, __builtin_convertvector(v, bf16x8));
-}
-
-// Two record bytes -> two bf16 (0..255 are exact in bf16: the upper half of the
-// fp32 encoding).
-__device__ __forceinline__ uint32_t bytes_to_bf16x2(uint32_t w, int i) {
-    const float lo = (float)((w >> (16 * i)) & 0xffu);
-    const float hi = (float)((w >> (16 * i + 8)) & 0xffu);
-    return (__float_as_uint(hi) & 0xffff0000u) | (__float_as_uint(lo) >> 16);
-}
-
-__device__ __forceinline__ u4 bytes_to_bf16x8(uint32_t w0, uint32_t w1) {
-    u4 r;
-    r.x = bytes_to_bf16x2(w0, 0);
-    r.y = bytes_to_bf16x2(w0, 1);
-    r.z = bytes_to_bf16x2(w1, 0);
-    r.w = bytes_to_bf16x2(w1, 1);
-    return r;
 }
 
 __device__ __forceinline__ u4 floats_to_bf16x8(const float* p) {

@@ -186,6 +186,138 @@ __device__ __forceinline__ f16v zero16() {
     return z;
 }
 
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ f16v mfma16(const u4& a, const u4& b, f16v c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// Two record bytes -> two bf16 (0..255 are exact in bf16: the upper half of the
+// fp32 encoding).
+__device__ __forceinline__ uint32_t bytes_to_bf16x2(uint32_t w, int i) {
+    const float lo = (float)((w >> (16 * i)) & 0xffu);
+    const float hi = (float)((w >> (16 * i + 8)) & 0xffu);
+    return (__float_as_uint(hi) & 0xffff0000u) | (__float_as_uint(lo) >> 16);
+}
+
+__device__ __forceinline__ u4 bytes_to_bf16x8(uint32_t w0, uint32_t w1) {
+    u4 r;
+    r.x = bytes_to_bf16x2(w0, 0);
+    r.y = bytes_to_bf16x2(w0, 1);
+    r.z = bytes_to_bf16x2(w1, 0);
+    r.w = bytes_to_bf16x2(w1, 1);
+    return r;
+}
+
+// ---- encoder GEMM of both tiles of a pair, map bytes on the bf16 matrix pipe -------
+// 792 of the 843 features are record bytes, exact in bf16.  An fp32 weight is
+// exactly the sum of three bf16 numbers (hi = bf16(w), mid = bf16(w - hi),
+// lo = w - hi - mid: 3 x 8 significant bits), so byte x weight is the sum of three
+// bf16 x bf16 products, each exact in the fp32 the MFMA accumulates in: the same
+// arithmetic as an fp32 FMA chain up to the order of the roundings, at
+// 3 x 32 cycles of v_mfma_f32_32x32x16_bf16 per 16 features instead of 8 x 64 of
+// v_mfma_f32_32x32x2_f32.  K = 792 as 50 blocks of 16 (the upper half of block 49
+// is fed zeros); the 51 fp32 tail features follow on the fp32 MFMA (7 K blocks of
+// 8 from the fp32 mirror).  Weights three blocks deep in registers; the block loop
+// is unrolled by three so that the ring needs no moves.
+struct EncS { u4 b[6]; };   // (unit tile 0|1) x (hi, mid, lo)
+struct EncDw { uint32_t x0, x1, y0, y1; };
+
+__device__ __forceinline__ EncS encs_load(const u4* wp, int kb, unsigned lane_u) {
+    constexpr int KB_STRIDE = 4 * 6 * 64;   // u4 per K block
+    const u4* p = wp + (size_t)kb * KB_STRIDE;
+    EncS r;
+#pragma unroll
+    for (int i = 0; i < 6; i++) r.b[i] = (p + i * 64)[lane_u];
+    return r;
+}
+
+__device__ __forceinline__ EncDw encs_bytes(const uint32_t* rx, const uint32_t* ry, int kb,
+                                            int half) {
+    EncDw r;
+    r.x0 = rx[4 * kb + 2 * half];
+    r.x1 = rx[4 * kb + 2 * half + 1];
+    r.y0 = ry[4 * kb + 2 * half];
+    r.y1 = ry[4 * kb + 2 * half + 1];
+    return r;
+}
+
+__device__ __forceinline__ void encs_mma(f16v (&acc)[4], const u4& ax, const u4& ay,
+                                         const EncS& w) {
+#pragma unroll
+    for (int s = 0; s < 3; s++)
+#pragma unroll
+        for (int ut = 0; ut < 2; ut++) {
+            acc[ut] = mfma16(ax, w.b[3 * ut + s], acc[ut]);
+            acc[2 + ut] = mfma16(ay, w.b[3 * ut + s], acc[2 + ut]);
+        }
+}
+
+// Block kb: request the weights of block kb+2 and the bytes of block kb+1, then
+// the 12 MFMAs of block kb.
+__device__ __forceinline__ void encs_step(f16v (&acc)[4], const u4* wp, const uint32_t* rx,
+                                          const uint32_t* ry, int kb, const EncS& use, EncS& fill,
+                                          EncDw& cur, const Lane& L) {
+    fill = encs_load(wp, kb + 2, L.lane_u);
+    const EncDw nxt = encs_bytes(rx, ry, kb + 1, L.half);
+    const u4 ax = bytes_to_bf16x8(cur.x0, cur.x1);
+    const u4 ay = bytes_to_bf16x8(cur.y0, cur.y1);
+    encs_mma(acc, ax, ay, use);
+    cur = nxt;
+}
+
+__device__ __forceinline__ void encoder_gemm_split(const FwdArgs& a, const float* ldsX,
+                                                   const float* ldsY, const Lane& L,
+                                                   f16v (&acc)[4]) {
+    static_assert(kKb16Split == 50 && CFP_OBS_MAP == 16 * 49 + 8, "block schedule below");
+    const uint32_t* rx = reinterpret_cast<const uint32_t*>(ldsX) + L.l32 * RS;
+    const uint32_t* ry = reinterpret_cast<const uint32_t*>(ldsY) + L.l32 * RS;
+    const u4* wp = a.we_s3 + (size_t)(L.wave * 6) * 64;
+    EncS b0 = encs_load(wp, 0, L.lane_u), b1 = encs_load(wp, 1, L.lane_u), b2;
+    EncDw cur = encs_bytes(rx, ry, 0, L.half);
+#pragma unroll 1
+    for (int kb = 0; kb < 48; kb += 3) {
+        encs_step(acc, wp, rx, ry, kb, b0, b2, cur, L);
+        encs_step(acc, wp, rx, ry, kb + 1, b1, b0, cur, L);
+        encs_step(acc, wp, rx, ry, kb + 2, b2, b1, cur, L);
+    }
+    // the fp32 tail's weights, requested ahead of the last two map blocks
+    const f4* wq = a.we_pk + (size_t)(L.wave * 2) * 64;
+    constexpr int KB8_STRIDE = 4 * 2 * 64;
+    f4 tb0[7], tb1[7];
+#pragma unroll
+    for (int t = 0; t < 7; t++) {
+        const f4* p = wq + (size_t)(kKbMap + t) * KB8_STRIDE;
+        tb0[t] = p[L.lane_u];
+        tb1[t] = (p + 64)[L.lane_u];
+    }
+    {   // block 48, then block 49 whose upper eight features are past the map
+        const EncDw nxt = encs_bytes(rx, ry, 49, L.half);
+        encs_mma(acc, bytes_to_bf16x8(cur.x0, cur.x1), bytes_to_bf16x8(cur.y0, cur.y1), b0);
+        u4 ax = bytes_to_bf16x8(nxt.x0, nxt.x1), ay = bytes_to_bf16x8(nxt.y0, nxt.y1);
+        if (L.half) {
+            ax = u4{0u, 0u, 0u, 0u};
+            ay = u4{0u, 0u, 0u, 0u};
+        }
+        encs_mma(acc, ax, ay, b1);
+    }
+    // tail floats 8t + 4*half + j of the record (51 valid, then zeros) on the fp32 MFMA
+    const float* fx = reinterpret_cast<const float*>(rx) + (CFP_OBS_MAP / 4) + 4 * L.half;
+    const float* fy = reinterpret_cast<const float*>(ry) + (CFP_OBS_MAP / 4) + 4 * L.half;
+#pragma unroll
+    for (int t = 0; t < 7; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float x = fx[8 * t + j], y = fy[8 * t + j];
+            acc[0] = mfma(x, tb0[t][j], acc[0]);
+            acc[1] = mfma(x, tb1[t][j], acc[1]);
+            acc[2] = mfma(y, tb0[t][j], acc[2]);
+            acc[3] = mfma(y, tb1[t][j], acc[3]);
+        }
+    }
+}
+
 // ---- encoder GEMM of both tiles of a pair: K = 848 as 53 steps of two 8-wide K
 // blocks.  The weight fragments of a step feed both tiles (4 accumulators), so
 // the mirror is streamed once per pair.  Weights sit three steps deep in
