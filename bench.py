@@ -10,8 +10,12 @@ workload is the baseline's third config: 262 144 envs, h256x3, one unchunked
 launch per step; the 16 x 16 384 chunked schedule is timed beside it.
 
 Prints ONE JSON line (metric = env-steps/s) with two extra objects:
-  roofline     algorithmic FLOPs per launch / measured launch time vs the
-               MI355X fp32 MFMA peak (HIP events on the launch stream)
+  roofline     algorithmic FLOPs per launch / measured launch time (HIP events on
+               the launch stream) vs the matrix-pipe bound of the kernel's
+               instruction mix: fp32 MFMA (157.3 TFLOP/s) for all but the
+               encoder's byte-valued features, which issue as three bf16 MFMAs
+               per product (2.5 PFLOP/s); the fraction of the plain fp32 MFMA
+               peak is reported beside it
   cpu_baseline the CPU oracle's scalar fp32 forward timed on this host's cores
                on a bounded sample of the same workload
 """
@@ -28,12 +32,24 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 FLOP_PER_ENV_STEP = 2 * 843 * 256 + 3 * 2 * 768 * 256 + 2 * 44 * 256   # 1 633 792
 BYTES_PER_ENV_STEP = 996 + 4 + 3 * 256 * 4 * 2 + 44 * 4                # 7 320
 PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_BF16_MFMA_TFLOPS = 2500.0
+# Which matrix pipe the FLOPs issue on.  The encoder's 792 byte-valued features
+# are exact in bf16 and each fp32 weight is exactly three bf16 terms, so their
+# products run as three bf16 MFMAs (fp32 accumulate); everything else (51 fp32
+# tail features, gate GEMMs, heads) is fp32 MFMA.
+FLOP_BF16_PIPE_ALGO = 2 * 792 * 256                 # per env-step, algorithmic
+FLOP_BF16_PIPE_ISSUED = 3 * FLOP_BF16_PIPE_ALGO     # three terms per weight
+FLOP_FP32_PIPE = FLOP_PER_ENV_STEP - FLOP_BF16_PIPE_ALGO
+# matrix-pipe time bound per env-step and the effective peak of this mix
+T_BOUND_PER_ENV_STEP = (FLOP_FP32_PIPE / (PEAK_FP32_MFMA_TFLOPS * 1e12) +
+                        FLOP_BF16_PIPE_ISSUED / (PEAK_BF16_MFMA_TFLOPS * 1e12))
+PEAK_MIX_TFLOPS = FLOP_PER_ENV_STEP / T_BOUND_PER_ENV_STEP / 1e12   # 196.9
 LAYERS = 3
 # HBM bytes per launch at 262 144 envs from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/policy_forward_262144_pmc.txt), scaled by the factors the same counters
 # show for a plain 1 GiB copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0); None until
 # measured for another size.
-MEASURED_TRAFFIC_BYTES = {262144: 2052732928}
+MEASURED_TRAFFIC_BYTES = {262144: 2223613338}
 
 
 def parse():
@@ -182,8 +198,13 @@ def main():
         "pct_fp32_mfma_peak": 100.0 * achieved / PEAK_FP32_MFMA_TFLOPS,
         "chunked_16x16384": results.get("chunked_16x16384"),
         "bf16_in_fp32_acc_unchunked": bf16,
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+        # peak = algorithmic FLOPs / matrix-pipe time bound of the kernel's instruction
+        # mix (fp32 pipe at 157.3, the encoder's byte features on the bf16 pipe at 2500)
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MIX_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_MIX_TFLOPS,
+                     "frac_of_fp32_mfma_peak": achieved / PEAK_FP32_MFMA_TFLOPS,
+                     "fp32_pipe_flops_per_launch": FLOP_FP32_PIPE * n // launches,
+                     "bf16_pipe_issued_flops_per_launch": FLOP_BF16_PIPE_ISSUED * n // launches,
                      "traffic": (MEASURED_TRAFFIC_BYTES[n] // launches
                                  if n in MEASURED_TRAFFIC_BYTES else None),
                      "kernel": "k_policy_forward",

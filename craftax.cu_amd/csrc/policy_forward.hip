@@ -309,6 +309,75 @@ __device__ __forceinline__ void vm_wait(int n) {
 #undef CFP_VMW
 }
 
+// ---- encoder GEMM of both tiles of a pair, weights through the ring ---------------
+// The three-term bf16 weight fragments (policy_tile.h, "map bytes on the bf16 matrix
+// pipe") are streamed like the gate weights: K block kb+3 requested into the ring
+// and block kb+1 read back while block kb multiplies.  Its 16-byte elements and its
+// 6 KiB per wave and block are those of the gate mirror, so ring_dma serves both.
+__device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const float* ldsX,
+                                                        const float* ldsY, f4* ring,
+                                                        const Lane& L, f16v (&acc)[4]) {
+    static_assert(kKb16Split == 50 && CFP_OBS_MAP == 16 * 49 + 8, "block schedule below");
+    const uint32_t* rx = reinterpret_cast<const uint32_t*>(ldsX) + L.l32 * RS;
+    const uint32_t* ry = reinterpret_cast<const uint32_t*>(ldsY) + L.l32 * RS;
+    // the fp32 tail's weights first: older than every ring request, used last
+    const f4* wq = a.we_pk + (size_t)(L.wave * 2) * 64;
+    constexpr int KB8_STRIDE = 4 * 2 * 64;
+    f4 tb0[7], tb1[7];
+#pragma unroll
+    for (int t = 0; t < 7; t++) {
+        const f4* p = wq + (size_t)(kKbMap + t) * KB8_STRIDE;
+        tb0[t] = p[L.lane_u];
+        tb1[t] = (p + 64)[L.lane_u];
+    }
+    asm volatile("" ::: "memory");
+    const f4* wp = reinterpret_cast<const f4*>(a.we_s3) + (size_t)(L.wave * 6) * 64;
+    ring_preload(ring, wp, L);
+    EncDw cur = encs_bytes(rx, ry, 0, L.half);
+    EncS bl[2];
+    vm_wait(12);
+#pragma unroll
+    for (int i = 0; i < 6; i++)
+        bl[0].b[i] = __builtin_bit_cast(u4, ring[i * 64 + L.lane_u]);
+#pragma unroll
+    for (int kb = 0; kb < kKb16Split; kb++) {
+        const int cb = kb & 1, nb = cb ^ 1;
+        if (kb + 3 < kKb16Split)
+            ring_dma(wp, kb + 3, ring + (kb % kRingSlots) * kRingSlotF4, L,
+                     __uint_as_float(bl[cb].b[5].w));
+        EncDw nxt = cur;
+        if (kb + 1 < kKb16Split) {
+            vm_wait(kb + 3 < kKb16Split ? 12 : (kb + 2 < kKb16Split ? 6 : 0));
+            const f4* slot = ring + ((kb + 1) % kRingSlots) * kRingSlotF4 + L.lane_u;
+#pragma unroll
+            for (int i = 0; i < 6; i++) bl[nb].b[i] = __builtin_bit_cast(u4, slot[i * 64]);
+            nxt = encs_bytes(rx, ry, kb + 1, L.half);
+        }
+        u4 ax = bytes_to_bf16x8(cur.x0, cur.x1), ay = bytes_to_bf16x8(cur.y0, cur.y1);
+        if (kb == kKb16Split - 1 && L.half) {   // features 792..799 are not map bytes
+            ax = u4{0u, 0u, 0u, 0u};
+            ay = u4{0u, 0u, 0u, 0u};
+        }
+        encs_mma(acc, ax, ay, bl[cb]);
+        cur = nxt;
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // tail floats 8t + 4*half + j of the record (51 valid, then zeros) on the fp32 MFMA
+    const float* fx = reinterpret_cast<const float*>(rx) + (CFP_OBS_MAP / 4) + 4 * L.half;
+    const float* fy = reinterpret_cast<const float*>(ry) + (CFP_OBS_MAP / 4) + 4 * L.half;
+#pragma unroll
+    for (int t = 0; t < 7; t++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float x = fx[8 * t + j], y = fy[8 * t + j];
+            acc[0] = mfma(x, tb0[t][j], acc[0]);
+            acc[1] = mfma(x, tb1[t][j], acc[1]);
+            acc[2] = mfma(y, tb0[t][j], acc[2]);
+            acc[3] = mfma(y, tb1[t][j], acc[3]);
+        }
+    }
+}
+
 // DO_K: accN[6] += x_K . W_l^T for the tile whose x tile is `xs4K`.  On entry the
 //       ring holds (has been asked for) K blocks 0..2, requested by ring_preload,
 //       followed, when DO_E, by the 32 loads of state_load and nothing else.
@@ -513,7 +582,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             f16v eacc[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) eacc[t] = zero16();
-            encoder_gemm_split(a, lds_all[0], lds_all[1], L, eacc);
+            encoder_gemm_split_ring(a, lds_all[0], lds_all[1],
+                                    aux + L.wave * (kRingSlots * kRingSlotF4), L, eacc);
             __syncthreads();   // every wave is done with the record bytes
 #pragma unroll
             for (int s = 0; s < 2; s++)

@@ -219,19 +219,9 @@ __device__ __forceinline__ u4 bytes_to_bf16x8(uint32_t w0, uint32_t w1) {
 // 3 x 32 cycles of v_mfma_f32_32x32x16_bf16 per 16 features instead of 8 x 64 of
 // v_mfma_f32_32x32x2_f32.  K = 792 as 50 blocks of 16 (the upper half of block 49
 // is fed zeros); the 51 fp32 tail features follow on the fp32 MFMA (7 K blocks of
-// 8 from the fp32 mirror).  Weights three blocks deep in registers; the block loop
-// is unrolled by three so that the ring needs no moves.
+// 8 from the fp32 mirror).
 struct EncS { u4 b[6]; };   // (unit tile 0|1) x (hi, mid, lo)
 struct EncDw { uint32_t x0, x1, y0, y1; };
-
-__device__ __forceinline__ EncS encs_load(const u4* wp, int kb, unsigned lane_u) {
-    constexpr int KB_STRIDE = 4 * 6 * 64;   // u4 per K block
-    const u4* p = wp + (size_t)kb * KB_STRIDE;
-    EncS r;
-#pragma unroll
-    for (int i = 0; i < 6; i++) r.b[i] = (p + i * 64)[lane_u];
-    return r;
-}
 
 __device__ __forceinline__ EncDw encs_bytes(const uint32_t* rx, const uint32_t* ry, int kb,
                                             int half) {
@@ -252,198 +242,6 @@ __device__ __forceinline__ void encs_mma(f16v (&acc)[4], const u4& ax, const u4&
             acc[ut] = mfma16(ax, w.b[3 * ut + s], acc[ut]);
             acc[2 + ut] = mfma16(ay, w.b[3 * ut + s], acc[2 + ut]);
         }
-}
-
-// Block kb: request the weights of block kb+2 and the bytes of block kb+1, then
-// the 12 MFMAs of block kb.
-__device__ __forceinline__ void encs_step(f16v (&acc)[4], const u4* wp, const uint32_t* rx,
-                                          const uint32_t* ry, int kb, const EncS& use, EncS& fill,
-                                          EncDw& cur, const Lane& L) {
-    fill = encs_load(wp, kb + 2, L.lane_u);
-    const EncDw nxt = encs_bytes(rx, ry, kb + 1, L.half);
-    const u4 ax = bytes_to_bf16x8(cur.x0, cur.x1);
-    const u4 ay = bytes_to_bf16x8(cur.y0, cur.y1);
-    encs_mma(acc, ax, ay, use);
-    cur = nxt;
-}
-
-__device__ __forceinline__ void encoder_gemm_split(const FwdArgs& a, const float* ldsX,
-                                                   const float* ldsY, const Lane& L,
-                                                   f16v (&acc)[4]) {
-    static_assert(kKb16Split == 50 && CFP_OBS_MAP == 16 * 49 + 8, "block schedule below");
-    const uint32_t* rx = reinterpret_cast<const uint32_t*>(ldsX) + L.l32 * RS;
-    const uint32_t* ry = reinterpret_cast<const uint32_t*>(ldsY) + L.l32 * RS;
-    const u4* wp = a.we_s3 + (size_t)(L.wave * 6) * 64;
-    EncS b0 = encs_load(wp, 0, L.lane_u), b1 = encs_load(wp, 1, L.lane_u), b2;
-    EncDw cur = encs_bytes(rx, ry, 0, L.half);
-#pragma unroll 1
-    for (int kb = 0; kb < 48; kb += 3) {
-        encs_step(acc, wp, rx, ry, kb, b0, b2, cur, L);
-        encs_step(acc, wp, rx, ry, kb + 1, b1, b0, cur, L);
-        encs_step(acc, wp, rx, ry, kb + 2, b2, b1, cur, L);
-    }
-    // the fp32 tail's weights, requested ahead of the last two map blocks
-    const f4* wq = a.we_pk + (size_t)(L.wave * 2) * 64;
-    constexpr int KB8_STRIDE = 4 * 2 * 64;
-    f4 tb0[7], tb1[7];
-#pragma unroll
-    for (int t = 0; t < 7; t++) {
-        const f4* p = wq + (size_t)(kKbMap + t) * KB8_STRIDE;
-        tb0[t] = p[L.lane_u];
-        tb1[t] = (p + 64)[L.lane_u];
-    }
-    {   // block 48, then block 49 whose upper eight features are past the map
-        const EncDw nxt = encs_bytes(rx, ry, 49, L.half);
-        encs_mma(acc, bytes_to_bf16x8(cur.x0, cur.x1), bytes_to_bf16x8(cur.y0, cur.y1), b0);
-        u4 ax = bytes_to_bf16x8(nxt.x0, nxt.x1), ay = bytes_to_bf16x8(nxt.y0, nxt.y1);
-        if (L.half) {
-            ax = u4{0u, 0u, 0u, 0u};
-            ay = u4{0u, 0u, 0u, 0u};
-        }
-        encs_mma(acc, ax, ay, b1);
-    }
-    // tail floats 8t + 4*half + j of the record (51 valid, then zeros) on the fp32 MFMA
-    const float* fx = reinterpret_cast<const float*>(rx) + (CFP_OBS_MAP / 4) + 4 * L.half;
-    const float* fy = reinterpret_cast<const float*>(ry) + (CFP_OBS_MAP / 4) + 4 * L.half;
-#pragma unroll
-    for (int t = 0; t < 7; t++) {
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const float x = fx[8 * t + j], y = fy[8 * t + j];
-            acc[0] = mfma(x, tb0[t][j], acc[0]);
-            acc[1] = mfma(x, tb1[t][j], acc[1]);
-            acc[2] = mfma(y, tb0[t][j], acc[2]);
-            acc[3] = mfma(y, tb1[t][j], acc[3]);
-        }
-    }
-}
-
-// ---- encoder GEMM of both tiles of a pair: K = 848 as 53 steps of two 8-wide K
-// blocks.  The weight fragments of a step feed both tiles (4 accumulators), so
-// the mirror is streamed once per pair.  Weights sit three steps deep in
-// registers; the step loop is unrolled by three so that the ring needs no moves
-// (a register rotation would make every iteration wait for ALL loads in flight).
-struct EncB { f4 b[4]; };   // (block 0|1) x (unit tile 0|1)
-
-__device__ __forceinline__ EncB enc_load_b(const f4* wp, int step, unsigned lane_u) {
-    constexpr int KB_STRIDE = 4 * 2 * 64;   // f4 per K block
-    EncB r;
-    const f4* p = wp + (size_t)(2 * step) * KB_STRIDE;
-    r.b[0] = (p)[lane_u];
-    r.b[1] = (p + 64)[lane_u];
-    r.b[2] = (p + KB_STRIDE)[lane_u];
-    r.b[3] = (p + KB_STRIDE + 64)[lane_u];
-    return r;
-}
-
-__device__ __forceinline__ void enc_mma(f16v (&acc)[4], const float (&x)[8],
-                                        const float (&y)[8], const EncB& w) {
-#pragma unroll
-    for (int q = 0; q < 2; q++)
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            acc[0] = mfma(x[4 * q + j], w.b[2 * q][j], acc[0]);
-            acc[1] = mfma(x[4 * q + j], w.b[2 * q + 1][j], acc[1]);
-            acc[2] = mfma(y[4 * q + j], w.b[2 * q][j], acc[2]);
-            acc[3] = mfma(y[4 * q + j], w.b[2 * q + 1][j], acc[3]);
-        }
-}
-
-__device__ __forceinline__ void bytes_to_f(uint32_t w, float* x) {
-    x[0] = (float)(w & 0xffu);
-    x[1] = (float)((w >> 8) & 0xffu);
-    x[2] = (float)((w >> 16) & 0xffu);
-    x[3] = (float)(w >> 24);
-}
-
-struct EncBytes { uint32_t x0, x1, y0, y1; };
-
-__device__ __forceinline__ EncBytes enc_bytes(const uint32_t* rx, const uint32_t* ry,
-                                              int step, int half) {
-    EncBytes r;
-    r.x0 = rx[4 * step + half];
-    r.x1 = rx[4 * step + 2 + half];
-    r.y0 = ry[4 * step + half];
-    r.y1 = ry[4 * step + 2 + half];
-    return r;
-}
-
-// One all-map step: request the weights of step p+2 and the bytes of step p+1,
-// then the 32 MFMAs of step p.
-__device__ __forceinline__ void enc_map_step(f16v (&acc)[4], const f4* wp, const uint32_t* rx,
-                                             const uint32_t* ry, int p, const EncB& use,
-                                             EncB& fill, EncBytes& cur, const Lane& L) {
-    fill = enc_load_b(wp, p + 2, L.lane_u);
-    const EncBytes nxt = enc_bytes(rx, ry, p + 1, L.half);
-    float x[8], y[8];
-    bytes_to_f(cur.x0, x);
-    bytes_to_f(cur.x1, x + 4);
-    bytes_to_f(cur.y0, y);
-    bytes_to_f(cur.y1, y + 4);
-    enc_mma(acc, x, y, use);
-    // one weight load per eight MFMAs, the LDS reads and conversions in between
-#pragma unroll
-    for (int q = 0; q < 32; q++) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (q % 8 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        if (q % 8 == 4) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        if (q < 16) __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    cur = nxt;
-}
-
-// Steps 49..52: map block 98 + tail block 0, then tail blocks 1..6 (fp32 features).
-template <int P>
-__device__ __forceinline__ void enc_tail_step(f16v (&acc)[4], const f4* wp, const float* fx,
-                                              const float* fy, const EncB& use, EncB& fill,
-                                              const EncBytes& cur, const Lane& L) {
-    if (P + 2 < kEncPairs) fill = enc_load_b(wp, P + 2, L.lane_u);
-    float x[8], y[8];
-    if (P == kMapPairs) {
-        bytes_to_f(cur.x0, x);
-        bytes_to_f(cur.y0, y);
-#pragma unroll
-        for (int j = 0; j < 4; j++) { x[4 + j] = fx[j]; y[4 + j] = fy[j]; }
-    } else {
-        constexpr int kt = 2 * (P - kMapPairs) - 1;   // first tail block of the step
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            x[j] = fx[8 * kt + j];
-            x[4 + j] = fx[8 * (kt + 1) + j];
-            y[j] = fy[8 * kt + j];
-            y[4 + j] = fy[8 * (kt + 1) + j];
-        }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    enc_mma(acc, x, y, use);
-    __builtin_amdgcn_sched_barrier(0);
-}
-
-__device__ __forceinline__ void encoder_gemm(const FwdArgs& a, const float* ldsX,
-                                             const float* ldsY, const Lane& L,
-                                             f16v (&acc)[4]) {
-    static_assert(kMapPairs == 49 && kEncPairs == 53, "step schedule below assumes 49 + 4");
-    const uint32_t* rx = reinterpret_cast<const uint32_t*>(ldsX) + L.l32 * RS;
-    const uint32_t* ry = reinterpret_cast<const uint32_t*>(ldsY) + L.l32 * RS;
-    const float* fx = reinterpret_cast<const float*>(rx) + (CFP_OBS_MAP / 4) + 4 * L.half;
-    const float* fy = reinterpret_cast<const float*>(ry) + (CFP_OBS_MAP / 4) + 4 * L.half;
-    const f4* wp = a.we_pk + (size_t)(L.wave * 2) * 64;
-    EncB b0 = enc_load_b(wp, 0, L.lane_u), b1 = enc_load_b(wp, 1, L.lane_u), b2;
-    EncBytes cur = enc_bytes(rx, ry, 0, L.half);
-#pragma unroll 1
-    for (int p = 0; p < 48; p += 3) {
-        enc_map_step(acc, wp, rx, ry, p, b0, b2, cur, L);
-        enc_map_step(acc, wp, rx, ry, p + 1, b1, b0, cur, L);
-        enc_map_step(acc, wp, rx, ry, p + 2, b2, b1, cur, L);
-    }
-    // step 48 is the last all-map step; its "next bytes" are map block 98 plus
-    // the first tail dword, which step 49 re-reads as a float
-    enc_map_step(acc, wp, rx, ry, 48, b0, b2, cur, L);
-    enc_tail_step<49>(acc, wp, fx, fy, b1, b0, cur, L);
-    enc_tail_step<50>(acc, wp, fx, fy, b2, b1, cur, L);
-    enc_tail_step<51>(acc, wp, fx, fy, b0, b2, cur, L);
-    enc_tail_step<52>(acc, wp, fx, fy, b1, b0, cur, L);
 }
 
 }  // namespace

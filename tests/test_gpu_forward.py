@@ -56,6 +56,50 @@ def test_fused_forward_matches_oracle(pkg, cuda, n, layers, term_p):
     pol.close()
 
 
+def test_encoder_weight_split_is_exact(pkg, cuda):
+    """The encoder multiplies the byte-valued features on the bf16 matrix pipe
+    against a three-term bf16 split of each fp32 weight.  Weights whose three
+    terms are all non-zero (1 + m*2^-10 + 2^-20), one 16-feature K block of ones
+    per env and nothing else make every product and every partial sum exactly
+    representable in fp32, so h_enc must equal the fp64 result (rounded once, when
+    the bias is added) bit for bit: a
+    dropped or misplaced term, block or unit column shows as a 2^-16 (or larger)
+    difference.  The 51 fp32 tail features get the same treatment on their own
+    envs (values 0.5, weights with 24 significant bits)."""
+    import torch
+    from parity_util import OBS, split_params
+    n = 128
+    params = np.zeros_like(random_params(L, 1))
+    o = split_params(params, L)                      # views into params
+    u = np.arange(HIDDEN)
+    f = np.arange(OBS)[:, None]
+    o["W_enc"][:] = (1.0 + (1 + (u[None, :] + f) % 4) * 2.0 ** -10 + 2.0 ** -20).astype(np.float32)
+    o["W_enc"][792:] = (1.0 + 2.0 ** -12 + 2.0 ** -23) * (1 + (u[None, :] % 3))
+    o["b_enc"][:] = (u % 7).astype(np.float32)
+    assert np.array_equal(o["W_enc"].astype(np.float64),
+                          np.float64(o["W_enc"]))     # fp32 values, exactly
+    rec = np.zeros((n, 996), np.uint8)
+    tail = np.zeros((n, 51), np.float32)
+    for e in range(n):
+        if e < 100:                                   # map K blocks 0..49, twice (ones, then threes)
+            kb = e % 50
+            rec[e, 16 * kb:min(16 * kb + 16, 792)] = 1 if e < 50 else 3
+        else:                                         # tail features in groups of 4
+            j = min((e - 100) * 2, 47)
+            tail[e, j:j + 4] = 0.5
+    rec[:, 792:] = tail.view(np.uint8).reshape(n, 204)
+    pol = pkg.Policy(n, L, seed=1)
+    pol.set_params(params)
+    h = pol.encode_step(_t(rec, cuda)).cpu().numpy()
+    x64 = expand_records(rec).astype(np.float64)
+    dot = x64 @ o["W_enc"].astype(np.float64)
+    assert np.array_equal(dot.astype(np.float32).astype(np.float64), dot)   # sums representable
+    want = (dot + o["b_enc"].astype(np.float64)).astype(np.float32)         # one rounding: + bias
+    bad = np.nonzero(h != want)
+    assert bad[0].size == 0, f"{bad[0].size} entries differ, first env {bad[0][:4]} unit {bad[1][:4]}"
+    pol.close()
+
+
 def test_split_entry_points_match_fused_and_oracle(pkg, cuda):
     """cfp_encode_step + cfp_gru_chain + cfp_head == cfp_policy_forward == oracle."""
     import torch
