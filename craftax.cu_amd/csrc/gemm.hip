@@ -18,8 +18,7 @@
 //   one is multiplied.  Edges are zero-filled, so M, N, K are arbitrary;
 //   operands whose base or leading dimension is not 16-byte aligned take a
 //   scalar-load path of the same kernel.
-//   Workgroup ids are remapped so that consecutive tiles (which share an A
-//   tile) run on the same XCD and meet in its L2.
+//   Workgroup ids are remapped to the XCDs (tile_of_block below).
 // dW = dpre^T x has K = window columns (>= 16k) and a small output, so K is
 // split over grid.y into a workspace and summed in a fixed order by a second
 // kernel: run-to-run bitwise stable, unlike float atomics.
@@ -42,8 +41,32 @@ struct GemmArgs {
     long c_split;
     int M, N, K;
     int k_per_split;                   // multiple of BK
+    int splits;                        // K splits (1 = none)
     int mt, nt;                        // tile counts
 };
+
+// Workgroup -> (output tile, K split).  The hardware deals workgroups to the eight
+// XCDs round-robin, each XCD with its own L2.
+//   no split: consecutive tiles (which share an A tile) go to the same XCD;
+//   split K : every XCD takes whole splits -- all output tiles of the splits
+//             s = xcd (mod 8), one split after the other -- so the A and B slices
+//             of a split are fetched from HBM once and shared through that L2 by
+//             the tiles that need them, and all eight XCDs are busy however few
+//             output tiles there are.
+__device__ __forceinline__ bool tile_of_block(const GemmArgs& g, int& tile, int& split) {
+    const int total = g.mt * g.nt;
+    const int xcd = (int)(blockIdx.x % kXcds), q = (int)(blockIdx.x / kXcds);
+    if (g.splits == 1) {
+        const int chunk = (total + kXcds - 1) / kXcds;
+        tile = xcd * chunk + q;
+        split = 0;
+        return tile < total;
+    }
+    const int sl = q / total;
+    tile = q - sl * total;
+    split = sl * kXcds + xcd;
+    return split < g.splits;
+}
 
 // Fetch this thread's share (4 x 16 bytes) of a [128 rows][32 k] operand tile.
 // KFAST: k is unit-stride in memory; thread covers (row = v/8, k = 4*(v%8)..+3).
@@ -113,13 +136,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm(GemmArgs g) {
     const int l32 = lane & 31, half = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
     // XCD-aware tile id: hardware deals workgroups to the XCDs round-robin
-    const int total = g.mt * g.nt;
-    const int chunk = (total + kXcds - 1) / kXcds;
-    const int tile = (int)(blockIdx.x % kXcds) * chunk + (int)(blockIdx.x / kXcds);
-    if (tile >= total) return;
+    int tile, split;
+    if (!tile_of_block(g, tile, split)) return;
     const int i0 = (tile / g.nt) * BM;
     const int j0 = (tile % g.nt) * BN;
-    const int kbeg = blockIdx.y * g.k_per_split;
+    const int kbeg = split * g.k_per_split;
     const int kend = min(g.K, kbeg + g.k_per_split);
 
     f16v acc[2][2];
@@ -160,7 +181,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm(GemmArgs g) {
         }
     }
 
-    float* C = g.C + (long)blockIdx.y * g.c_split;
+    float* C = g.C + (long)split * g.c_split;
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -216,13 +237,11 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm_bf16(GemmArgs g) {
     const int lane = tid & 63, wave = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
     const int wm = wave >> 1, wn = wave & 1;
-    const int total = g.mt * g.nt;
-    const int chunk = (total + kXcds - 1) / kXcds;
-    const int tile = (int)(blockIdx.x % kXcds) * chunk + (int)(blockIdx.x / kXcds);
-    if (tile >= total) return;
+    int tile, split;
+    if (!tile_of_block(g, tile, split)) return;
     const int i0 = (tile / g.nt) * BM;
     const int j0 = (tile % g.nt) * BN;
-    const int kbeg = blockIdx.y * g.k_per_split;
+    const int kbeg = split * g.k_per_split;
     const int kend = min(g.K, kbeg + g.k_per_split);
 
     f16v acc[2][2];
@@ -265,7 +284,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm_bf16(GemmArgs g) {
         }
     }
 
-    float* C = g.C + (long)blockIdx.y * g.c_split;
+    float* C = g.C + (long)split * g.c_split;
 #pragma unroll
     for (int a = 0; a < 2; a++)
 #pragma unroll
@@ -355,7 +374,9 @@ int run_gemm(GemmArgs g, int splits, bool accum, hipStream_t st) {
     g.mt = (g.M + BM - 1) / BM;
     g.nt = (g.N + BN - 1) / BN;
     const int total = g.mt * g.nt;
-    const dim3 grid((total + kXcds - 1) / kXcds * kXcds, splits);
+    g.splits = splits;
+    const dim3 grid(splits == 1 ? (total + kXcds - 1) / kXcds * kXcds
+                                : kXcds * total * ((splits + kXcds - 1) / kXcds));
     const bool va = A_KFAST ? vec_ok(g.A, g.sa_i, g.K) : vec_ok(g.A, g.sa_k, g.M);
     const bool vb = B_KFAST ? vec_ok(g.B, g.sb_j, g.K) : vec_ok(g.B, g.sb_k, g.N);
     if (accum) return launch_gemm<A_KFAST, B_KFAST, true>(g, grid, va, vb, st);
@@ -400,7 +421,10 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
     int splits = (1024 + tiles - 1) / tiles;
     const int kblocks = (cols + BK - 1) / BK;
     if (splits > kblocks) splits = kblocks;
-    if (splits > kMaxSplits) splits = kMaxSplits;
+    // the workspace holds kMaxSplits slices of the largest dW; a smaller one may use more
+    int max_splits = (int)(kDwWorkFloats / ((size_t)rows * CFP_HIDDEN));
+    if (max_splits > 8 * kMaxSplits) max_splits = 8 * kMaxSplits;
+    if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
     const int k_per_split = ((kblocks + splits - 1) / splits) * BK;
     splits = (cols + k_per_split - 1) / k_per_split;
