@@ -263,7 +263,9 @@ constexpr int kRingF4 = 4 * kRingSlots * kRingSlotF4;     // 72 KiB for the work
 
 // K block kb of a layer (wp = mirror + layer + wave*6*64 fragments) -> ring slot.
 // `after` is a register the slot's previous contents were last read into: as an
-// operand it keeps the request behind the completion of those reads.
+// operand it keeps the request behind the completion of those reads.  M0 (the LDS
+// base of an LDS-direct load) is reserved: the compiler neither allocates it nor,
+// in this file, uses it for anything else.
 __device__ __forceinline__ void ring_dma(const f4* wp, int kb, f4* slot, const Lane& L,
                                          float after = 0.0f) {
     constexpr int KB_STRIDE = 4 * 6 * 64;
@@ -279,7 +281,7 @@ __device__ __forceinline__ void ring_dma(const f4* wp, int kb, f4* slot, const L
         "global_load_lds_dwordx4 %0, %1 offset:3072"
         :
         : "v"(voff), "s"(src), "s"(lds_lo), "v"(after)
-        : "memory", "m0");
+        : "memory");
     asm volatile(
         "s_mov_b32 m0, %2\n\t"
         "s_nop 0\n\t"
@@ -287,7 +289,7 @@ __device__ __forceinline__ void ring_dma(const f4* wp, int kb, f4* slot, const L
         "global_load_lds_dwordx4 %0, %1 offset:1024"
         :
         : "v"(voff), "s"(src + 4 * 64), "s"(lds_lo + 4096u)
-        : "memory", "m0");
+        : "memory");
 }
 
 // First three K blocks of a layer's weights into ring slots 0, 1, 2.
@@ -686,21 +688,30 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
 
         // ---- heads: wave = (row tile nt, K half kh), both tiles -----------------------
         if (a.do_head) {
-            f16v hacc[2];
+            // both tiles share each weight fragment; their MFMAs alternate, so no MFMA
+            // waits for the one before it on the same accumulator
+            f16v hacc[2] = {zero16(), zero16()};
             const f4* wp = a.wav_pk + (size_t)nt * 64;
+            const f4* xsX = reinterpret_cast<const f4*>(lds_all[0]);
+            const f4* xsY = reinterpret_cast<const f4*>(lds_all[1]);
+            f4 hb[kKbHid / 2];
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                hacc[s] = zero16();
-                const f4* xs4 = reinterpret_cast<const f4*>(lds_all[s]);
+            for (int i = 0; i < kKbHid / 2; i++)
+                hb[i] = (wp + (size_t)(kh * (kKbHid / 2) + i) * 128)[L.lane_u];
 #pragma unroll
-                for (int i = 0; i < kKbHid / 2; i++) {
-                    const int kb = kh * (kKbHid / 2) + i;
-                    const f4 b = (wp + (size_t)kb * 128)[L.lane_u];
-                    const f4 av = xs4[L.arow4 + 2 * kb];
+            for (int i = 0; i < kKbHid / 2; i++) {
+                const int kb = kh * (kKbHid / 2) + i;
+                const f4 ax = xsX[L.arow4 + 2 * kb];
+                const f4 ay = xsY[L.arow4 + 2 * kb];
 #pragma unroll
-                    for (int j = 0; j < 4; j++) hacc[s] = mfma(av[j], b[j], hacc[s]);
+                for (int j = 0; j < 4; j++) {
+                    hacc[0] = mfma(ax[j], hb[i][j], hacc[0]);
+                    hacc[1] = mfma(ay[j], hb[i][j], hacc[1]);
                 }
-                if (kh == 1) {
+            }
+            if (kh == 1) {
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
                     float* red = red_all[s] + (nt * 16) * 64 + L.lane_u;
 #pragma unroll
                     for (int r = 0; r < 16; r++) red[r * 64] = hacc[s][r];
