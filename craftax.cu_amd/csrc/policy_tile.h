@@ -198,7 +198,8 @@ __device__ __forceinline__ f16v mfma16(const u4& a, const u4& b, f16v c) {
 __device__ __forceinline__ uint32_t bytes_to_bf16x2(uint32_t w, int i) {
     const float lo = (float)((w >> (16 * i)) & 0xffu);
     const float hi = (float)((w >> (16 * i + 8)) & 0xffu);
-    return (__float_as_uint(hi) & 0xffff0000u) | (__float_as_uint(lo) >> 16);
+    // upper halves of hi and lo in one byte permute: {hi[3], hi[2], lo[3], lo[2]}
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
 }
 
 __device__ __forceinline__ u4 bytes_to_bf16x8(uint32_t w0, uint32_t w1) {
