@@ -7,7 +7,7 @@
 // (9 rows x 11 cols, row-major) x 8 bytes {block, item+1, visible, melee+1,
 // passive+1, ranged+1, mob-projectile+1, player-projectile+1}, then 51 raw
 // little-endian fp32 scalars.  All of it is integer/byte work bound by HBM
-// gathers; one wavefront encodes one env, a lane per view cell.
+// gathers; one wavefront encodes one env.
 #include "cfp_common.h"
 
 namespace cfp {
@@ -75,60 +75,67 @@ __constant__ TailSpec kTail[CFP_OBS_TAIL] = {
 __constant__ uint8_t kSlotClass[CFP_MOB_SLOTS] = {0, 0, 0, 1, 1, 1, 2, 2,
                                                   3, 3, 3, 4, 4, 4};
 
+// One wavefront per env, the record assembled in LDS and written out as 249
+// coalesced dwords: lanes walk the 99 view cells (block, item, visible), lanes
+// 0..13 each judge one mob slot and drop its byte into its cell, lanes 0..50
+// compute the tail.  LDS operations of a wave execute in program order, so the
+// byte of a mob lands after the dword of its cell without a barrier.
 __global__ __launch_bounds__(256) void k_record_obs(
     const cfp_env_scalars* __restrict__ scalars,
     const uint8_t* __restrict__ map, const uint8_t* __restrict__ item_map,
     const uint8_t* __restrict__ light_map, size_t env_stride,
     size_t level_stride, uint8_t* __restrict__ rec_row, int n) {
+    __shared__ uint32_t stage_all[4][CFP_REC_BYTES / 4 + 3];
     const int lane = threadIdx.x & 63;
-    const int env = __builtin_amdgcn_readfirstlane(
-        (int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
+    const int wv = threadIdx.x >> 6;
+    const int env = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + wv));
     if (env >= n) return;
+    uint32_t* stage = stage_all[wv];
     const cfp_env_scalars* s = scalars + env;
     const int pr = s->player_position[0], pc = s->player_position[1];
     const int level = s->player_level;
     const int mlevel = jax_index(level, 9);
     const size_t cell_plane = (size_t)env * env_stride + (size_t)level * level_stride;
     const size_t mob_plane = (size_t)env * env_stride + (size_t)mlevel * level_stride;
-    const uint8_t* light_m = light_map + mob_plane;
 
-    // Mob list: slot s contributes (cell, channel, value) when it passes the
-    // predicates of craftax_encode_mobs{3,2}_compact (craftax_full.c:2747-2825);
-    // evaluated identically by every lane, ascending slot order = last wins.
-    int mob_cell[CFP_MOB_SLOTS];
-    int mob_val[CFP_MOB_SLOTS];
-#pragma unroll
-    for (int m = 0; m < CFP_MOB_SLOTS; m++) {
-        const int type = s->mob_type_id[m];
-        const int mr = s->mob_position[m][0], mc = s->mob_position[m][1];
-        const int lr = mr - pr + ROWS / 2, lc = mc - pc + COLS / 2;
-        bool ok = type >= 0 && type < 8 && s->mob_mask[m] != 0 && lr >= 0 &&
-                  lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
-                  mc >= 0 && mc < MAP;
-        if (ok) ok = light_m[mr * MAP + mc] > 12;
-        mob_cell[m] = ok ? lr * COLS + lc : -1;
-        mob_val[m] = type + 1;
-    }
-
-    uint32_t* out = reinterpret_cast<uint32_t*>(rec_row + (size_t)env * CFP_REC_BYTES);
     for (int cell = lane; cell < CELLS; cell += 64) {
         const int row = cell / COLS, col = cell - row * COLS;
         const int wr = pr - ROWS / 2 + row, wc = pc - COLS / 2 + col;
-        uint32_t lo = 0, hi = 0;
+        uint32_t lo = 0;
         if (wr >= 0 && wr < MAP && wc >= 0 && wc < MAP) {
+            // all three planes requested at once (one memory round trip, not two)
             const size_t o = cell_plane + (size_t)(wr * MAP + wc);
-            if (light_map[o] > 12)
-                lo = (uint32_t)map[o] | ((uint32_t)(uint8_t)(item_map[o] + 1) << 8) |
-                     (1u << 16);
+            const uint32_t lv = light_map[o], bv = map[o], iv = item_map[o];
+            if (lv > 12) lo = bv | ((uint32_t)(uint8_t)(iv + 1) << 8) | (1u << 16);
         }
-        uint32_t ch[5] = {0, 0, 0, 0, 0};
+        stage[2 * cell] = lo;
+        stage[2 * cell + 1] = 0u;
+    }
+
+    // Mob slot m = lane contributes (cell, channel 3 + class, type + 1) when it passes
+    // the predicates of craftax_encode_mobs{3,2}_compact (craftax_full.c:2747-2825).
+    // Within a class the last slot on a cell wins: a slot stands back when one of the
+    // (at most two) later slots of its class sits on the same cell.
+    {
+        const int m = lane < CFP_MOB_SLOTS ? lane : CFP_MOB_SLOTS - 1;
+        const int type = s->mob_type_id[m];
+        const int mr = s->mob_position[m][0], mc = s->mob_position[m][1];
+        const int lr = mr - pr + ROWS / 2, lc = mc - pc + COLS / 2;
+        bool ok = lane < CFP_MOB_SLOTS && type >= 0 && type < 8 && s->mob_mask[m] != 0 &&
+                  lr >= 0 && lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
+                  mc >= 0 && mc < MAP;
+        if (ok) ok = light_map[mob_plane + (size_t)(mr * MAP + mc)] > 12;
+        const int cell = ok ? lr * COLS + lc : -1;
+        const int cls = kSlotClass[m];
+        bool over = false;
 #pragma unroll
-        for (int m = 0; m < CFP_MOB_SLOTS; m++)
-            if (mob_cell[m] == cell) ch[kSlotClass[m]] = (uint32_t)(uint8_t)mob_val[m];
-        lo |= ch[0] << 24;
-        hi = ch[1] | (ch[2] << 8) | (ch[3] << 16) | (ch[4] << 24);
-        out[2 * cell] = lo;
-        out[2 * cell + 1] = hi;
+        for (int d = 1; d <= 2; d++) {
+            const int oc = __shfl_down(cell, d, 64);
+            const int ocls = __shfl_down(cls, d, 64);
+            over = over || (lane + d < CFP_MOB_SLOTS && ocls == cls && oc == cell);
+        }
+        if (ok && !over)
+            reinterpret_cast<uint8_t*>(stage)[cell * 8 + 3 + cls] = (uint8_t)(type + 1);
     }
 
     if (lane < CFP_OBS_TAIL) {
@@ -161,8 +168,12 @@ __global__ __launch_bounds__(256) void k_record_obs(
                 v = (!any && s->boss_timesteps_to_spawn_this_round <= 0) ? 1.0f : 0.0f;
             } break;
         }
-        out[CFP_OBS_MAP / 4 + lane] = __float_as_uint(v);
+        stage[CFP_OBS_MAP / 4 + lane] = __float_as_uint(v);
     }
+
+    __builtin_amdgcn_wave_barrier();
+    uint32_t* out = reinterpret_cast<uint32_t*>(rec_row + (size_t)env * CFP_REC_BYTES);
+    for (int d = lane; d < CFP_REC_BYTES / 4; d += 64) out[d] = stage[d];
 }
 
 __global__ void k_expand_obs(const uint8_t* __restrict__ r_obs,

@@ -83,6 +83,44 @@ def test_record_obs_ragged_count_and_oracle(pkg, cuda, golden):
     assert (got[37:] == 0xEE).all()            # nothing written past n
 
 
+def test_record_obs_mob_collisions_last_slot_wins(pkg, cuda, golden):
+    """Several live mobs of one class on one lit cell: the highest slot's type is the
+    one recorded (craftax_encode_mobs3_compact writes in ascending slot order).  Built
+    from a fuzzed reference state; compared with the oracle and checked directly."""
+    import torch
+    sc = golden["fuzz_scalars"][:64].copy()
+    pl = golden["fuzz_planes"][:64].copy()
+    pl[:, 2] = 255                                     # every cell lit
+    s32 = sc.view(np.int32)
+    off = {f[0]: getattr(ob.EnvScalars, f[0]).offset // 4 for f in ob.EnvScalars._fields_}
+    groups = ((0, 3), (3, 3), (6, 2), (8, 3), (11, 3))  # first slot, slots of each class
+    for e in range(64):
+        s32[e, off["player_position"]:off["player_position"] + 2] = (20, 20)
+        s32[e, off["mob_mask"]:off["mob_mask"] + 14] = 0
+        first, cnt = groups[e % 5]
+        for j in range(cnt):
+            m = first + j
+            if (e // 5) % 2 == 1 and j == 1:
+                continue                               # a gap: slots first and first+2 collide
+            s32[e, off["mob_mask"] + m] = 1
+            s32[e, off["mob_type_id"] + m] = (e + 3 * j) % 8
+            s32[e, off["mob_position"] + 2 * m:off["mob_position"] + 2 * m + 2] = (21, 19)
+    want = ob.encode_compact(sc, pl[:, 0], pl[:, 1], pl[:, 2])
+    planes = _t(pl, cuda).view(-1)
+    rec = pkg.policy.record_obs(_t(sc, cuda), planes, planes[P:], planes[2 * P:], 64, 3 * P, 0)
+    torch.cuda.synchronize()
+    got = rec.cpu().numpy()
+    assert np.array_equal(got, want)
+    cell = (21 - 20 + 4) * 11 + (19 - 20 + 5)          # view cell of map (21, 19)
+    for e in range(64):
+        first, cnt = groups[e % 5]
+        gap = (e // 5) % 2 == 1
+        last_j = 0 if (gap and cnt == 2) else cnt - 1
+        last_type = (e + 3 * last_j) % 8
+        ch = 3 + e % 5
+        assert got[e, cell * 8 + ch] == last_type + 1, (e, got[e, cell * 8:cell * 8 + 8])
+
+
 def test_expand_obs_bit_exact(pkg, cuda):
     import torch
     rec = np.zeros((320, 996), np.uint8)
