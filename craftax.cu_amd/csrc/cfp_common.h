@@ -30,7 +30,8 @@ constexpr int kEncPadBlocks = 4;                   // encoder mirror: prefetch o
 // MFMA-ordered weight mirror sizes, in floats.
 constexpr size_t kEncPackFloats = (size_t)kObsPad * CFP_HIDDEN;
 constexpr int kKb16Split = (CFP_OBS_MAP + 15) / 16;                   // 50 K blocks of 16 map bytes
-constexpr size_t kEncSplitBf16 = (size_t)kKb16Split * 4 * 6 * 64 * 8;  // bf16 elements of the split mirror
+// bf16 elements of the split mirror: 50 blocks (full game) or 83 (classic, 1323 cell features)
+constexpr size_t kEncSplitBf16 = (size_t)83 * 4 * 6 * 64 * 8;
 constexpr size_t kGruPackFloats = (size_t)CFP_GRU * CFP_HIDDEN;   // per layer
 constexpr size_t kAvPackFloats = (size_t)kAvPad * CFP_HIDDEN;
 

@@ -49,163 +49,6 @@ namespace cfp {
 namespace {
 
 constexpr int kRedFloats = 2 * 16 * 64;               // head K-half partials
-// classic encoder tables: [21 chunks][64 envs][4] gather words + [64 envs][24] scalars
-constexpr int kClassicTabDwords = 21 * 64 * 4 + 64 * 24;
-
-// ---- classic-game encoder for a pair of tiles (64 envs) ----------------------------
-// encode_obs_kernel (craftax_classic.cu:1714-1751): the observation is one-hot per
-// view cell, so h0 = b_enc + the sum of the W_enc rows the record selects.  Thread
-// k owns hidden unit k and keeps the 64 envs' sums in registers.  W_enc (1.38 MB)
-// is walked once per pair in chunks of three cells (63 rows, 63 KiB) staged in
-// the LDS that later holds the x tiles, the next chunk travelling through
-// registers meanwhile; every gather is then one conflict-free LDS read of a row
-// that all lanes share.  `tab[chunk][env]` holds the byte offsets of the three
-// block rows inside the chunk and the cells' mob bits; row reads run several envs
-// ahead of their adds.  Mob bits are rare and take a wave-uniform branch.
-// Summation order per env: bias, then per chunk the three block rows followed by
-// that chunk's mob rows (cell, bit ascending), then the 22 scalar features.
-__device__ __forceinline__ void classic_encode_pair(const FwdArgs& a, const uint8_t* crecX,
-                                                    const uint8_t* crecY, float* wbuf,
-                                                    uint32_t* tab, float* xsX, float* xsY,
-                                                    int tid) {
-    constexpr int CELLS = 63, CH = 21, NBLK = 17, CHUNK_CELLS = 3;
-    constexpr int CHUNKS = CELLS / CHUNK_CELLS;                 // 21
-    constexpr int CHUNK_V4 = CHUNK_CELLS * CH * CFP_HIDDEN / 4;  // 4032 16-byte pieces
-    constexpr int PF = (CHUNK_V4 + kFwdThreads - 1) / kFwdThreads;   // 16 per thread
-    constexpr int NSCAL = CFP_CLASSIC_OBS - CELLS * CH;         // 22 scalar features
-    constexpr int ENVS = 2 * kTileEnvs;
-    static_assert(CHUNK_CELLS * CH * CFP_HIDDEN <= 2 * LDS_FLOATS, "chunk must fit the x tiles");
-    constexpr int SVS = 24;                                     // floats per env row of `sv`
-    static_assert(CHUNKS * ENVS * 4 + ENVS * SVS <= kClassicTabDwords, "table storage");
-    // the 22 scalar features of every env as fp32, 16-byte aligned rows
-    float* sv = reinterpret_cast<float*>(tab + CHUNKS * ENVS * 4);
-
-    // tab[chunk][env] = {byte offset of the block row of cell 0, 1, 2 inside the
-    // chunk buffer, the three cells' mob bits (4 each)}
-    for (int i = tid; i < CHUNKS * ENVS; i += kFwdThreads) {
-        const int c = i / ENVS, e = i - c * ENVS;
-        const uint8_t* o = (e < kTileEnvs ? crecX : crecY) + (e % kTileEnvs) * CFP_CLASSIC_REC_BYTES;
-        u4 w;
-        uint32_t m = 0;
-        uint32_t off[CHUNK_CELLS];
-#pragma unroll
-        for (int q = 0; q < CHUNK_CELLS; q++) {
-            const int cell = c * CHUNK_CELLS + q;
-            off[q] = (uint32_t)(q * CH + (int8_t)o[cell]) * (CFP_HIDDEN * 4);
-            m |= (o[CELLS + cell] & 15u) << (4 * q);
-        }
-        w.x = off[0]; w.y = off[1]; w.z = off[2]; w.w = m;
-        reinterpret_cast<u4*>(tab)[i] = w;
-    }
-    for (int i = tid; i < ENVS * SVS; i += kFwdThreads) {
-        const int e = i / SVS, f = i - e * SVS;
-        const uint8_t* o = (e < kTileEnvs ? crecX : crecY) +
-                           (e % kTileEnvs) * CFP_CLASSIC_REC_BYTES + 2 * CELLS;
-        float v = 0.0f;
-        if (f < 16) v = (float)(int8_t)o[f] / 10.0f;                  // inventory, intrinsics
-        else if (f < 20) v = (int8_t)o[16] == f - 15 ? 1.0f : 0.0f;   // direction 1..4
-        else if (f == 20) v = *reinterpret_cast<const float*>(o + 18);   // light
-        else if (f == 21) v = o[17] ? 1.0f : 0.0f;                    // sleeping
-        sv[i] = v;
-    }
-    float acc[ENVS];
-    const float bias = a.b_enc[tid];
-#pragma unroll
-    for (int e = 0; e < ENVS; e++) acc[e] = bias;
-
-    const f4* W4 = reinterpret_cast<const f4*>(a.w_enc);
-    f4* wbuf4 = reinterpret_cast<f4*>(wbuf);
-    const float* wk = wbuf + tid;
-    f4 pf[PF];
-#pragma unroll
-    for (int i = 0; i < PF; i++) {
-        const int v = tid + kFwdThreads * i;
-        pf[i] = v < CHUNK_V4 ? W4[v] : f4{0.0f, 0.0f, 0.0f, 0.0f};
-    }
-#pragma unroll 1
-    for (int c = 0; c <= CHUNKS; c++) {
-        __syncthreads();   // the previous chunk (and the tables) complete / consumed
-#pragma unroll
-        for (int i = 0; i < PF; i++) {
-            const int v = tid + kFwdThreads * i;
-            if (v < CHUNK_V4) wbuf4[v] = pf[i];
-        }
-        __syncthreads();
-        if (c < CHUNKS) {
-            // next: cells 3(c+1).., or for c+1 == CHUNKS the 22 scalar-feature rows
-            const size_t base = (size_t)(c + 1) * CHUNK_V4;
-            const int limit = c + 1 < CHUNKS ? CHUNK_V4 : NSCAL * CFP_HIDDEN / 4;
-#pragma unroll
-            for (int i = 0; i < PF; i++) {
-                const int v = tid + kFwdThreads * i;
-                if (v < limit) pf[i] = W4[base + v];
-            }
-            // Software pipeline over the envs: while env e is added, the three row
-            // reads of envs e+1 .. e+3 and the table words of env e+4 are in flight
-            // (the LDS counter tracks fifteen operations).
-            const u4* t4 = reinterpret_cast<const u4*>(tab) + c * ENVS;
-            const char* wkb = reinterpret_cast<const char*>(wk);
-            constexpr int DEPTH = 4;
-            u4 wq[DEPTH + 1];
-            float r[DEPTH][CHUNK_CELLS];
-            uint32_t mm[DEPTH];
-            auto issue = [&](int slot, const u4& w) {
-                r[slot][0] = *reinterpret_cast<const float*>(wkb + w.x);
-                r[slot][1] = *reinterpret_cast<const float*>(wkb + w.y);
-                r[slot][2] = *reinterpret_cast<const float*>(wkb + w.z);
-                mm[slot] = w.w;
-            };
-#pragma unroll
-            for (int e = 0; e < DEPTH; e++) wq[e] = t4[e];
-#pragma unroll
-            for (int e = 0; e < DEPTH - 1; e++) issue(e, wq[e]);
-#pragma unroll
-            for (int e = 0; e < ENVS; e++) {
-                if (e + DEPTH < ENVS) wq[(e + DEPTH) % (DEPTH + 1)] = t4[e + DEPTH];
-                if (e + DEPTH - 1 < ENVS)
-                    issue((e + DEPTH - 1) % DEPTH, wq[(e + DEPTH - 1) % (DEPTH + 1)]);
-                __builtin_amdgcn_sched_barrier(0);
-                acc[e] += r[e % DEPTH][0];
-                acc[e] += r[e % DEPTH][1];
-                acc[e] += r[e % DEPTH][2];
-                // rare: mob bits of this env's three cells (wave-uniform branch)
-                const uint32_t m = __builtin_amdgcn_readfirstlane(mm[e % DEPTH]);
-                if (m) {
-#pragma unroll
-                    for (int q = 0; q < CHUNK_CELLS; q++)
-#pragma unroll
-                        for (int j = 0; j < 4; j++)
-                            if (m & (1u << (4 * q + j)))
-                                acc[e] += wk[(q * CH + NBLK + j) * CFP_HIDDEN];
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
-            // 16 inventory / intrinsic scalars, direction one-hot, light, sleeping
-            float wv[NSCAL];
-#pragma unroll
-            for (int f = 0; f < NSCAL; f++) wv[f] = wk[f * CFP_HIDDEN];
-#pragma unroll
-            for (int e = 0; e < ENVS; e++) {
-                const f4* r4 = reinterpret_cast<const f4*>(sv + e * SVS);
-                float hv = acc[e];
-#pragma unroll
-                for (int f4i = 0; f4i < (NSCAL + 3) / 4; f4i++) {
-                    const f4 x = r4[f4i];
-#pragma unroll
-                    for (int j = 0; j < 4; j++)
-                        if (4 * f4i + j < NSCAL) hv = fmaf(x[j], wv[4 * f4i + j], hv);
-                }
-                acc[e] = hv;
-            }
-        }
-    }
-    __syncthreads();   // the weight chunk buffer becomes the x tiles
-#pragma unroll
-    for (int e = 0; e < ENVS; e++)
-        (e < kTileEnvs ? xsX : xsY)[(e % kTileEnvs) * XS + tid] = acc[e];
-}
-
 // ---- MinGRU phases ---------------------------------------------------------------
 // Written-to-nowhere tile: state / r_state addresses of a pair's missing second
 // tile point here, so the hot loop needs no predication.
@@ -380,6 +223,139 @@ __device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const 
     }
 }
 
+// ---- classic-game encoder for a pair of tiles (64 envs) ----------------------------
+// encode_obs_kernel (craftax_classic.cu:1714-1751): h0 = b_enc + W_enc^T x with
+// x = 63 view cells x (one-hot of 17 block ids + 4 mob bits) followed by 22 scalar
+// features.  The 1323 cell features are 0/1, exact in bf16, so they run like the
+// full game's byte features: three bf16 MFMAs per product against the three-term
+// split of the fp32 weights, weights streamed through the ring.  The A operand
+// needs no arithmetic: the pair's 64 x 1323 feature bits are packed once into
+// LDS (cell c = 21 bits at bit 21c), a lane's eight features of a K block are one
+// byte of that, and a 256-entry LDS table turns the byte into eight bf16 0/1.
+// The 22 scalar features (inventory and intrinsics / 10, direction one-hot, light,
+// sleeping) follow on the fp32 MFMA (3 K blocks of 8).  Block ids must be 0..16.
+constexpr int kClsCells = 63, kClsCh = 21;
+constexpr int kClsBits = kClsCells * kClsCh;                 // 1323
+constexpr int kClsKb16 = (kClsBits + 15) / 16;               // 83
+constexpr int kClsBitRow = 44;                               // dwords per env (42 used)
+constexpr int kClsSv = 24;                                   // scalar features per env, padded
+constexpr int kClsTailKb = kClsSv / 8;                       // 3 fp32 K blocks
+constexpr int kClsEnvs = 2 * kTileEnvs;
+// byte layout inside the (not yet used) x tiles
+constexpr int kClsOffRecY = kTileEnvs * CFP_CLASSIC_REC_BYTES;
+constexpr int kClsOffBits = 2 * kClsOffRecY;
+constexpr int kClsOffLut = kClsOffBits + kClsEnvs * kClsBitRow * 4;
+constexpr int kClsOffSv = kClsOffLut + 256 * 16;
+static_assert(kClsOffSv + kClsEnvs * kClsSv * 4 <= 2 * LDS_FLOATS * 4, "classic tables fit the x tiles");
+static_assert(kClsOffBits % 16 == 0 && kClsOffLut % 16 == 0 && kClsOffSv % 16 == 0, "alignment");
+
+// Bit rows, byte -> 8 x bf16 table and scalar rows from the two tiles' records
+// (all 256 threads; ends with a barrier).
+__device__ __forceinline__ void classic_prepare(uint8_t* base, int tid) {
+    uint32_t* bits = reinterpret_cast<uint32_t*>(base + kClsOffBits);
+    u4* lut = reinterpret_cast<u4*>(base + kClsOffLut);
+    float* sv = reinterpret_cast<float*>(base + kClsOffSv);
+    for (int i = tid; i < kClsEnvs * kClsBitRow; i += kFwdThreads) bits[i] = 0u;
+    {
+        u4 v;
+        uint32_t d[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            d[i] = (((unsigned)tid >> (2 * i)) & 1u) * 0x3F80u |
+                   (((unsigned)tid >> (2 * i + 1)) & 1u) * 0x3F800000u;
+        v.x = d[0]; v.y = d[1]; v.z = d[2]; v.w = d[3];
+        lut[tid] = v;
+    }
+    for (int i = tid; i < kClsEnvs * kClsSv; i += kFwdThreads) {
+        const int e = i / kClsSv, f = i - e * kClsSv;
+        const uint8_t* o = base + e * CFP_CLASSIC_REC_BYTES + 2 * kClsCells;
+        float v = 0.0f;
+        if (f < 16) v = (float)(int8_t)o[f] / 10.0f;                  // inventory, intrinsics
+        else if (f < 20) v = (int8_t)o[16] == f - 15 ? 1.0f : 0.0f;   // direction 1..4
+        else if (f == 20) v = *reinterpret_cast<const float*>(o + 18);   // light
+        else if (f == 21) v = o[17] ? 1.0f : 0.0f;                    // sleeping
+        sv[i] = v;
+    }
+    __syncthreads();   // rows are zero before the bits go in
+    for (int i = tid; i < kClsEnvs * kClsCells; i += kFwdThreads) {
+        const int e = i / kClsCells, cell = i - e * kClsCells;
+        const uint8_t* o = base + e * CFP_CLASSIC_REC_BYTES;
+        const uint32_t v = (1u << (o[cell] & 31u)) & 0x1FFFFu | ((o[kClsCells + cell] & 15u) << 17);
+        const int bit = kClsCh * cell, dw = bit >> 5, sh = bit & 31;
+        uint32_t* row = bits + e * kClsBitRow;
+        atomicOr(row + dw, v << sh);
+        if (sh > 32 - kClsCh) atomicOr(row + dw + 1, v >> (32 - sh));
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ void classic_encoder_gemm(const FwdArgs& a, const uint8_t* base,
+                                                     f4* ring, const Lane& L, f16v (&acc)[4]) {
+    const uint8_t* bx = base + kClsOffBits + L.l32 * (kClsBitRow * 4) + L.half;
+    const uint8_t* by = bx + kTileEnvs * (kClsBitRow * 4);
+    const u4* lut = reinterpret_cast<const u4*>(base + kClsOffLut);
+    // the scalar features' weights first: older than every ring request, used last
+    const f4* wq = a.we_pk + (size_t)(L.wave * 2) * 64;
+    constexpr int KB8_STRIDE = 4 * 2 * 64;
+    f4 tb0[kClsTailKb], tb1[kClsTailKb];
+#pragma unroll
+    for (int t = 0; t < kClsTailKb; t++) {
+        const f4* p = wq + (size_t)t * KB8_STRIDE;
+        tb0[t] = p[L.lane_u];
+        tb1[t] = (p + 64)[L.lane_u];
+    }
+    asm volatile("" ::: "memory");
+    const f4* wp = reinterpret_cast<const f4*>(a.we_s3) + (size_t)(L.wave * 6) * 64;
+    ring_preload(ring, wp, L);
+    // eight features of K block kb for this lane = byte 2*kb + half of the env's row
+    uint32_t mx = bx[0], my = by[0];
+    u4 ax = lut[mx], ay = lut[my];
+    mx = bx[2];
+    my = by[2];
+    EncS bl[2];
+    vm_wait(12);
+#pragma unroll
+    for (int i = 0; i < 6; i++) bl[0].b[i] = __builtin_bit_cast(u4, ring[i * 64 + L.lane_u]);
+#pragma unroll
+    for (int kb = 0; kb < kClsKb16; kb++) {
+        const int cb = kb & 1, nb = cb ^ 1;
+        if (kb + 3 < kClsKb16)
+            ring_dma(wp, kb + 3, ring + (kb % kRingSlots) * kRingSlotF4, L,
+                     __uint_as_float(bl[cb].b[5].w));
+        u4 nx = ax, ny = ay;
+        if (kb + 1 < kClsKb16) {
+            vm_wait(kb + 3 < kClsKb16 ? 12 : (kb + 2 < kClsKb16 ? 6 : 0));
+            const f4* slot = ring + ((kb + 1) % kRingSlots) * kRingSlotF4 + L.lane_u;
+#pragma unroll
+            for (int i = 0; i < 6; i++) bl[nb].b[i] = __builtin_bit_cast(u4, slot[i * 64]);
+            nx = lut[mx];          // block kb+1
+            ny = lut[my];
+            if (kb + 2 < kClsKb16) {
+                mx = bx[2 * (kb + 2)];
+                my = by[2 * (kb + 2)];
+            }
+        }
+        encs_mma(acc, ax, ay, bl[cb]);
+        ax = nx;
+        ay = ny;
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    const float* fx = reinterpret_cast<const float*>(base + kClsOffSv) + L.l32 * kClsSv + 4 * L.half;
+    const float* fy = fx + kTileEnvs * kClsSv;
+#pragma unroll
+    for (int t = 0; t < kClsTailKb; t++) {
+        const f4 x = *reinterpret_cast<const f4*>(fx + 8 * t);
+        const f4 y = *reinterpret_cast<const f4*>(fy + 8 * t);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc[0] = mfma(x[j], tb0[t][j], acc[0]);
+            acc[1] = mfma(x[j], tb1[t][j], acc[1]);
+            acc[2] = mfma(y[j], tb0[t][j], acc[2]);
+            acc[3] = mfma(y[j], tb1[t][j], acc[3]);
+        }
+    }
+}
+
 // DO_K: accN[6] += x_K . W_l^T for the tile whose x tile is `xs4K`.  On entry the
 //       ring holds (has been asked for) K blocks 0..2, requested by ring_preload,
 //       followed, when DO_E, by the 32 loads of state_load and nothing else.
@@ -496,14 +472,14 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds_all[2][LDS_FLOATS];
     __shared__ __attribute__((aligned(16))) float red_all[2][kRedFloats];
     __shared__ float term_all[2][kTileEnvs];
-    // 72 KiB shared by the weight ring (MinGRU phases) and, for the classic game, the
-    // record bytes and gather tables of the encoder, which runs before those phases
+    // the per-wave weight rings (encoder and MinGRU phases), 72 KiB
     __shared__ __attribute__((aligned(16))) f4 aux[kRingF4];
+    // classic game: record bytes and the encoder's tables sit in the x tiles until the
+    // encoder's result replaces them
     constexpr int kCrecBytes = kTileEnvs * CFP_CLASSIC_REC_BYTES;
-    static_assert(2 * kCrecBytes + kClassicTabDwords * 4 <= kRingF4 * 16, "classic tables fit the ring");
-    uint8_t* const crec_base = reinterpret_cast<uint8_t*>(aux);
-    uint8_t* const crec_all[2] = {crec_base, crec_base + kCrecBytes};
-    uint32_t* const ctab = reinterpret_cast<uint32_t*>(crec_base + 2 * kCrecBytes);
+    static_assert(kCrecBytes == kClsOffRecY, "record layout of the classic tables");
+    uint8_t* const cbase = reinterpret_cast<uint8_t*>(&lds_all[0][0]);
+    uint8_t* const crec_all[2] = {cbase, cbase + kClsOffRecY};
 
     const int tiles = a.n / kTileEnvs;
     const int pairs = (tiles + 1) / 2;
@@ -576,17 +552,18 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
                 if (term_all[s][acc_row(r) + 4 * L.half] != 0.0f) tmask[s] |= 1u << r;
 
         // ---- encoders ----------------------------------------------------------
-        if (classic) {
-            classic_encode_pair(a, crec_all[0], crec_all[1], &lds_all[0][0],
-                                ctab, lds_all[0],
-                                lds_all[1], tid);
-        } else if (full_rec) {
+        if (classic || full_rec) {
             f16v eacc[4];
 #pragma unroll
             for (int t = 0; t < 4; t++) eacc[t] = zero16();
-            encoder_gemm_split_ring(a, lds_all[0], lds_all[1],
-                                    aux + L.wave * (kRingSlots * kRingSlotF4), L, eacc);
-            __syncthreads();   // every wave is done with the record bytes
+            f4* const ring = aux + L.wave * (kRingSlots * kRingSlotF4);
+            if (classic) {
+                classic_prepare(cbase, tid);
+                classic_encoder_gemm(a, cbase, ring, L, eacc);
+            } else {
+                encoder_gemm_split_ring(a, lds_all[0], lds_all[1], ring, L, eacc);
+            }
+            __syncthreads();   // every wave is done with the record bytes / tables
 #pragma unroll
             for (int s = 0; s < 2; s++)
 #pragma unroll
@@ -845,14 +822,14 @@ __global__ void k_pack_av(const float* __restrict__ W_a,
 // k = 16*kb + 8*(l/32) + j of column l%32 of its 32-wide tile.  Features past the
 // map (the fp32 tail runs on the fp32 mirror) carry zeros.
 __global__ void k_pack_enc_split(const float* __restrict__ W_enc, __bf16* __restrict__ out,
-                                 int total) {
+                                 int total, int nfeat) {
     int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     int j = idx & 7, lane = (idx >> 3) & 63, q = idx >> 9;
     int s = q % 3, ut = (q / 3) & 1, wave = (q / 6) & 3, kb = q / 24;
     int unit = wave * 64 + ut * 32 + (lane & 31);
     int f = 16 * kb + 8 * (lane >> 5) + j;
-    const float w = f < CFP_OBS_MAP ? W_enc[(size_t)f * CFP_HIDDEN + unit] : 0.0f;
+    const float w = f < nfeat ? W_enc[(size_t)f * CFP_HIDDEN + unit] : 0.0f;
     const __bf16 hi = (__bf16)w;
     const float r1 = w - (float)hi;
     const __bf16 mid = (__bf16)r1;
@@ -862,22 +839,39 @@ __global__ void k_pack_enc_split(const float* __restrict__ W_enc, __bf16* __rest
 
 int launch_pack_enc_split(const float* params, int layers, int variant, uint16_t* we_s3,
                           hipStream_t st) {
-    if (variant != 0) return 0;   // the classic encoder gathers from the unpacked W_enc
     const Arena ar = arena_of(variant, layers);
-    const int total = (int)kEncSplitBf16;
+    // full game: the 792 map bytes; classic: the 1323 cell features
+    const int nfeat = variant == 0 ? CFP_OBS_MAP : kClsBits;
+    const int total = (variant == 0 ? kKb16Split : kClsKb16) * 4 * 6 * 64 * 8;
     hipLaunchKernelGGL(k_pack_enc_split, dim3((total + 255) / 256), dim3(256), 0, st,
-                       params + ar.w_enc, reinterpret_cast<__bf16*>(we_s3), total);
+                       params + ar.w_enc, reinterpret_cast<__bf16*>(we_s3), total, nfeat);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
+}
+
+// Classic game: the 22 scalar features' rows of W_enc (features 1323..1344, padded to
+// 24) as three fp32 K blocks in the order of k_pack_enc.
+__global__ void k_pack_enc_classic_tail(const float* __restrict__ W_enc,
+                                        float* __restrict__ out) {
+    int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= kClsTailKb * 2048) return;
+    int j = idx & 3, lane = (idx >> 2) & 63, ut = (idx >> 8) & 1,
+        wave = (idx >> 9) & 3, kb = idx >> 11;
+    int unit = wave * 64 + ut * 32 + (lane & 31);
+    int f = kClsBits + kKBlock * kb + 4 * (lane >> 5) + j;
+    out[idx] = f < CFP_CLASSIC_OBS ? W_enc[(size_t)f * CFP_HIDDEN + unit] : 0.0f;
 }
 
 int launch_pack_weights(const float* params, int layers, int variant, float* we_pk,
                         float* wg_pk, float* wav_pk, hipStream_t st) {
     const Arena ar = arena_of(variant, layers);
-    if (variant == 0) {   // the classic encoder gathers from the unpacked W_enc
+    if (variant == 0) {
         const int enc_total = (kKbEnc + kEncPadBlocks) * 2048;
         hipLaunchKernelGGL(k_pack_enc, dim3((enc_total + 255) / 256), dim3(256), 0,
                            st, params + ar.w_enc, we_pk, enc_total);
+    } else {
+        hipLaunchKernelGGL(k_pack_enc_classic_tail, dim3((kClsTailKb * 2048 + 255) / 256),
+                           dim3(256), 0, st, params + ar.w_enc, we_pk);
     }
     const int gru_total = layers * (int)kGruPackFloats + 4 * 6 * 64 * 4;
     hipLaunchKernelGGL(k_pack_gru, dim3((gru_total + 255) / 256), dim3(256), 0,
