@@ -22,18 +22,22 @@
 // about 8.5 cycles (12.5 for a transcendental), a 16-byte global load into
 // registers by 40-60.  So the design minimises instructions per MFMA rather than
 // latency: per 24 MFMAs, 6 LDS-direct weight requests (no registers written),
-// 7 LDS reads and ~25 epilogue instructions.  The shader clock under this load
-// is 2.06-2.13 GHz, not the 2.4 GHz behind the 157.3 TFLOP/s peak.
+// 7 LDS reads and ~25 epilogue instructions.  (The same instructions issued by a
+// second wave on the SIMD cost the MFMA wave about as much: a two-group variant of
+// this schedule measured no faster.)  The shader clock under this load is
+// 1.9-2.1 GHz, not the 2.4 GHz behind the 157.3 TFLOP/s peak.
 //
 // Within the workgroup, wave w owns hidden units [64w, 64w+64).  MFMA operand
 // convention (v_mfma_f32_32x32x2_f32): A = activations (row = env), B = weights
 // (column = unit), so accumulator register r of lane l holds env
 // 8*(r/4) + 4*(l/32) + r%4, unit l%32: a half-wave touches 32 consecutive units
 // of one env, i.e. one full 128-byte line of state.
-//   encoder: x from the LDS record bytes (v_cvt_f32_ubyteN) / tail floats,
-//            W_enc fragments streamed once per pair from the MFMA-ordered
-//            mirror in L2 and used for both tiles (4 accumulators), two K
-//            blocks per step, weights three steps deep in registers
+//   encoder: the byte-valued features (full game: 792 map bytes; classic game:
+//            1323 cell bits) are exact in bf16 and run as three bf16 MFMAs per
+//            product against an exact three-term bf16 split of the fp32 weights,
+//            fp32 accumulate (policy_tile.h); the remaining fp32 features follow
+//            on the fp32 MFMA.  Weight fragments stream through the same ring as
+//            the gate weights and feed both tiles (4 accumulators)
 //   layer:   6 accumulators (zh, zg, zp for 2 unit tiles) over K = 256; weights
 //            go L2 -> per-wave LDS ring (LDS-direct loads, three K blocks ahead)
 //            -> registers (one block ahead); the first three blocks and the 32
@@ -41,7 +45,8 @@
 //            that ends the current one; state and r_state leave through
 //            non-temporal stores next to each epilogue element; h' goes back
 //            into the x tile
-//   heads:   2 row tiles x 2 K halves over the 4 waves, reduced through LDS.
+//   heads:   2 row tiles x 2 K halves over the 4 waves, each weight fragment used for
+//            both tiles, partial sums reduced through LDS.
 #include "policy_tile.h"
 
 namespace cfp {
