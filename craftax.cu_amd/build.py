@@ -18,6 +18,23 @@ def hipcc_path():
     raise RuntimeError("hipcc not found (looked at $HIPCC, PATH, /opt/rocm/bin)")
 
 
+def check_no_scratch(remarks):
+    """The fused fp32 forward kernel waits for its LDS-direct weight loads with
+    explicit `s_waitcnt vmcnt(N)`, N = the number of younger vector-memory
+    operations it issues itself.  A register spill is such an operation too, one
+    the source cannot count, so a build whose forward kernel uses scratch memory
+    is rejected."""
+    name, bad = None, []
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+        elif "ScratchSize [bytes/lane]:" in line and name and "k_policy_forwardI" in name:
+            if int(line.split("ScratchSize [bytes/lane]:")[1].split()[0]) != 0:
+                bad.append(name)
+    if bad:
+        raise RuntimeError("k_policy_forward spills registers to scratch memory in: " + ", ".join(bad))
+
+
 def build(verbose=False):
     """Compile every HIP source into one shared library; always recompiles."""
     cmd = [
@@ -25,15 +42,17 @@ def build(verbose=False):
         "-shared", "-Wall", "-Wno-unused-function",
         # packed fp32 VALU ops are kept off for gfx950 device code
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-Rpass-analysis=kernel-resource-usage",
         "-o", OUT,
     ] + [os.path.join(CSRC, s) for s in SOURCES]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
+    noise = ("is not a recognized feature for this target", "[-Rpass-analysis=kernel-resource-usage]")
+    err = "\n".join(l for l in res.stderr.splitlines() if not any(n in l for n in noise))
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
+    check_no_scratch(res.stderr)
     if verbose and err.strip():
         print(err, file=sys.stderr)
     return OUT

@@ -58,3 +58,20 @@ def test_argument_validation_needs_no_gpu(pkg):
     assert lib.cfp_gemm_fwd(0, 1, 1, None, None, None, None) != 0
     assert lib.cfp_encode_step(None, None, 32, None) != 0
     assert lib.cfp_abi_version() >= 1
+
+
+def test_build_rejects_a_spilling_forward_kernel():
+    """The forward kernel counts its own vector-memory operations for explicit
+    s_waitcnt; the build refuses a compile whose k_policy_forward uses scratch."""
+    import importlib.util
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "craftax.cu_amd", "build.py")
+    spec = importlib.util.spec_from_file_location("cfp_build", path)
+    b = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(b)
+    fn = "remark: f.hip:1:1: Function Name: _ZN3cfp16k_policy_forwardILi0ELi0EEEvNS_7FwdArgsE [-R]\n"
+    other = "remark: f.hip:1:1: Function Name: _ZN3cfp6k_gemmILb0EEEvNS_8GemmArgsE [-R]\n"
+    b.check_no_scratch(fn + "remark:     ScratchSize [bytes/lane]: 0 [-R]\n" +
+                       other + "remark:     ScratchSize [bytes/lane]: 64 [-R]\n")
+    with pytest.raises(RuntimeError, match="scratch"):
+        b.check_no_scratch(fn + "remark:     ScratchSize [bytes/lane]: 24 [-R]\n")
