@@ -124,6 +124,8 @@ int launch_expand_obs(const uint8_t* r_obs, float* xobs, int t0, int count, int 
                       int env_start, int ld, hipStream_t st);
 int gemm_enc_fwd_ld(int cols, const float* W_enc, const float* xobs, int ldx, float* h,
                     hipStream_t st);
+int gemm_dh_acc(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
+                hipStream_t st);
 int gemm_dw_ld(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
                hipStream_t st);
 

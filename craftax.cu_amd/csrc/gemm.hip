@@ -411,6 +411,19 @@ int gemm_enc_fwd_ld(int cols, const float* d_W_enc, const float* d_xobs, int ldx
     return run_gemm<true, false>(g, 1, false, st);
 }
 
+// cu_gemm_dh with an accumulate switch: dh[cols][256] (+)= dpre[cols][m3] . W[m3][256]
+int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* d_dh,
+                bool accumulate, hipStream_t st) {
+    CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh: bad argument");
+    GemmArgs g{};
+    g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
+    g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
+    g.C = d_dh; g.ldc = CFP_HIDDEN; g.c_split = 0;
+    g.M = cols; g.N = CFP_HIDDEN; g.K = m3;
+    g.k_per_split = (m3 + BK - 1) / BK * BK;
+    return run_gemm<true, false>(g, 1, accumulate, st);
+}
+
 int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld_dpre,
                float* d_dW, hipStream_t st) {
     CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW &&
@@ -480,15 +493,7 @@ int cfp_gemm_enc_fwd(int cols, const float* d_W_enc, const float* d_xobs,
 
 int cfp_gemm_dh(int m3, int cols, const float* d_W, const float* d_dpre,
                 float* d_dh, void* stream) {
-    CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh,
-                "cfp_gemm_dh: bad argument");
-    GemmArgs g{};
-    g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
-    g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
-    g.C = d_dh; g.ldc = CFP_HIDDEN; g.c_split = 0;
-    g.M = cols; g.N = CFP_HIDDEN; g.K = m3;
-    g.k_per_split = (m3 + BK - 1) / BK * BK;
-    return run_gemm<true, false>(g, 1, false, (hipStream_t)stream);
+    return gemm_dh_acc(m3, cols, d_W, d_dpre, d_dh, false, (hipStream_t)stream);
 }
 
 int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,

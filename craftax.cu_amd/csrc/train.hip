@@ -2,8 +2,9 @@
 // Adam.  Host-side mirror of the reference's CuTrain layer
 // (craftax_full.cu:12637-13480); kernels follow
 //   k_mingru_epi_replay_win :9460   k_head_bwd_win      :9603
-//   k_mingru_window_bwd     :9510   k_add_dv_wv         :10224
-//   k_colsum / 256 / small  :10442  k_vadd              :10069
+//   k_mingru_window_bwd     :9510   k_colsum / 256 / small  :10442
+//   (k_add_dv_wv :10224 is folded into the top layer's reverse kernel, k_vadd
+//    :10069 into the layer-0 dh GEMM, which accumulates onto the highway term)
 //   k_gae :10617  k_adv_stats :10638  k_adam :10668  k_loss_accum :10508
 // The GEMMs go through the fp32 MFMA seam in gemm.hip.  All reductions are
 // done in a fixed order (no float atomics), so a backward pass is bitwise
@@ -157,18 +158,6 @@ __global__ __launch_bounds__(256) void k_loss_fold(const double* __restrict__ bl
     }
 }
 
-__global__ void k_add_dv_wv(float* __restrict__ dh, const float* __restrict__ dv,
-                            const float* __restrict__ W_v, size_t total) {
-    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    dh[idx] += dv[idx / H] * W_v[idx & (H - 1)];
-}
-
-__global__ void k_vadd(float* __restrict__ a, const float* __restrict__ b, size_t total) {
-    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx < total) a[idx] += b[idx];
-}
-
 // out[r] += sum_c src[c*rows + r]: partial sums over `slices` column ranges
 // (grid.x), then folded in slice order by k_colsum_fold.
 __global__ __launch_bounds__(256) void k_colsum_partial(
@@ -212,12 +201,14 @@ __global__ void k_mingru_window_bwd(
     const float* __restrict__ dhGEMM, const float* __restrict__ dhExtra,
     const float* __restrict__ r_state, const uint8_t* __restrict__ r_done,
     float* __restrict__ dhExtraOut, float* __restrict__ dcarry, int t0, int Tw,
-    int mb, int n, int env_start, int layer, int layers, int T_all, int seg_len) {
+    int mb, int n, int env_start, int layer, int layers, int T_all, int seg_len,
+    const float* __restrict__ dv, const float* __restrict__ W_v) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)H * mb) return;
     const int k = (int)(idx & (H - 1));
     const size_t el = idx / H;
     float dc = dcarry[idx];
+    const float wv_k = dv ? W_v[k] : 0.0f;
     for (int tr = Tw - 1; tr >= 0; tr--) {
         const int t = t0 + tr;
         if (t == T_all - 1 || ((t + 1) % seg_len) == 0) dc = 0.0f;
@@ -226,6 +217,7 @@ __global__ void k_mingru_window_bwd(
         const size_t o3 = w * G + k;
         const float zh = pre[o3], zg = pre[o3 + H], zp = pre[o3 + 2 * H];
         float dhout = dhGEMM[o];
+        if (dv) dhout += dv[w] * wv_k;   // top layer: the value head's share (k_add_dv_wv)
         if (dhExtra) dhout += dhExtra[o];
         const size_t rs = (((size_t)t * layers + layer) * (size_t)n + env_start + el) * H + k;
         const float s_in = r_state[rs];
@@ -703,9 +695,9 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
                            tr->cfg.vf, tr->d_ent, fused ? A + 1 : A);
         hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(256), 0, st, tr->block_loss, hb,
                            tr->loss_acc);
+        // dh3 = W_a^T dlogits here; the value head's dv * W_v is added where the top
+        // layer's reverse kernel reads dh3 (the reference's k_add_dv_wv pass, :10224)
         if (cfp_gemm_dh(A, cols, W_a, tr->dlogits, tr->dh3b, stream)) return 1;
-        hipLaunchKernelGGL(k_add_dv_wv, dim3(grid1(hc)), dim3(256), 0, st, tr->dh3b,
-                           tr->dvalue, W_v, hc);
         if (cfp_gemm_dw(A, cols, tr->x[L], tr->dlogits, g + CFP_OFF_W_A(L), stream)) return 1;
         if (cfp_gemv_dwv(tr->x[L], tr->dvalue, g + CFP_OFF_W_V(L), cols, stream)) return 1;
         if (colsum_into(tr, tr->dlogits, g + CFP_OFF_B_A(L), A, cols, st)) return 1;
@@ -717,19 +709,20 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             hipLaunchKernelGGL(k_mingru_window_bwd, dim3(grid1((size_t)H * mb)), dim3(256),
                                0, st, tr->preb[l], tr->x[l], dh_gemm, dh_extra, tr->r_state,
                                tr->r_done, tr->dhX, tr->dcarry[l], t0, Tw, mb, n, env_start,
-                               l, L, T, seg);
+                               l, L, T, seg, l == L - 1 ? tr->dvalue : nullptr, W_v);
             if (cfp_gemm_dw(G, cols, tr->x[l], tr->preb[l],
                             g + CFP_OFF_W_GRU + (size_t)l * G * H, stream))
                 return 1;
-            if (cfp_gemm_dh(G, cols, W_gru + (size_t)l * G * H, tr->preb[l], tr->dhG, stream))
+            // layer 0: dh_enc = W_0^T dpre + highway, accumulated onto the highway term
+            if (gemm_dh_acc(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
+                            l == 0 ? tr->dhX : tr->dhG, l == 0, st))
                 return 1;
             dh_gemm = tr->dhG;
             dh_extra = tr->dhX;
         }
-        // ---- encoder: dh_enc = dhG + highway; db_enc; dW_enc += xobs^T dh_enc
-        hipLaunchKernelGGL(k_vadd, dim3(grid1(hc)), dim3(256), 0, st, tr->dhG, tr->dhX, hc);
-        if (colsum_into(tr, tr->dhG, g + CFP_OFF_B_ENC, H, cols, st)) return 1;
-        if (gemm_dw_ld(CFP_OBS, cols, tr->dhG, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, st)) return 1;
+        // ---- encoder: db_enc; dW_enc += xobs^T dh_enc (dh_enc sits in dhX)
+        if (colsum_into(tr, tr->dhX, g + CFP_OFF_B_ENC, H, cols, st)) return 1;
+        if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, st)) return 1;
     }
     CFP_HIP_TRY(hipGetLastError());
     return 0;
