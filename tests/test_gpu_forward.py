@@ -255,6 +255,39 @@ def test_full_size_properties(pkg, cuda):
     small.close(); pol.close()
 
 
+def test_forward_is_bitwise_reproducible_under_memory_pressure(pkg, cuda):
+    """The kernel waits for its LDS-direct weight loads by counting its own vector
+    memory operations; a miscount would read a ring slot before it has landed, and
+    what it reads then depends on timing.  Same inputs, three runs -- one alone, two
+    racing a large device copy on another stream -- must agree bit for bit, for the
+    plain, the r_state-recording and the classic kernels."""
+    import torch
+    n = 65536
+    side = torch.cuda.Stream()
+    big = torch.empty(1 << 28, dtype=torch.uint8, device=cuda)
+    for variant in ("full", "classic"):
+        pol = pkg.Policy(n, L, seed=5, variant=variant)
+        rec = (pkg.policy.synth_classic_records(n, 3, 1) if variant == "classic"
+               else pkg.policy.synth_records(n, 3, 1))
+        term = (torch.rand(n, device=cuda) < 0.1).float()
+        st0 = torch.randn(L, n, HIDDEN, device=cuda) * 0.5
+        outs = []
+        for run in range(3):
+            st = st0.clone()
+            rs = torch.zeros_like(st0) if run != 1 else None
+            torch.cuda.synchronize()
+            if run:
+                with torch.cuda.stream(side):
+                    for _ in range(4):
+                        big[: 1 << 27].copy_(big[1 << 27:])
+            av = pol.forward(rec, term, st, r_state_t=rs).clone()
+            torch.cuda.synchronize()
+            outs.append((av, st))
+        for av, st in outs[1:]:
+            assert torch.equal(av, outs[0][0]) and torch.equal(st, outs[0][1]), variant
+        pol.close()
+
+
 def test_error_paths_on_device(pkg, cuda):
     import torch
     pol = pkg.Policy(64, L, seed=1)
