@@ -129,6 +129,18 @@ int gemm_dh_acc(int m3, int cols, const float* W, const float* dpre, float* dh, 
 int gemm_dw_ld(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
                hipStream_t st);
 
+// split-K workspace of the dW GEMMs (allocated on first use) and the fixed-order fold
+// dst[i] += sum_z part[z*stride + i]
+int dw_workspace(float** work, size_t* floats);
+int launch_splitk_reduce(float* dst, const float* part, long count, long stride, int splits,
+                         hipStream_t st);
+// dW_enc[843][256] += features^T dh over the window columns, read from the records
+// (bf16 MFMA on the map bytes); needs envs per minibatch % 8 == 0.  tail_scratch:
+// cols * 76 floats.
+bool dw_enc_records_ok(int mb);
+int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
+                   int cols, int mb, int n_all, int env_start, hipStream_t st);
+
 // per-variant arena geometry
 struct Arena {
     int obs, actions;

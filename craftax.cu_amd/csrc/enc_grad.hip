@@ -1,0 +1,243 @@
+// Encoder weight gradient of the PPO update, taken straight from the recorded
+// observation records:  dW_enc[f][u] += sum_c feature_f(c) * dh_enc[c][u]  over the
+// window columns c.  The reference expands the records into a dense fp32 feature
+// matrix (k_expand_obs, craftax_full.cu:10022-10031) and calls
+// cu_gemm_dw(CF_NN_OBS, cols, dh, xobs) on it (craftax_full.cu:13324).
+//
+// Here the 768 leading map bytes never become floats in memory.  A byte is exact in
+// bf16, and an fp32 gradient is exactly the sum of three bf16 numbers (8 + 8 + 8
+// significand bits), so byte * gradient is three bf16 MFMA products accumulated in
+// fp32: the same sum of exact fp32 products that the fp32 MFMA adds up, at 3/16 of its
+// cost, and the operand read per column is 768 bytes instead of 3 KiB.
+//   grid      : 3 feature groups (256 map bytes each) x S splits of the columns; the
+//               three groups of a split run on one XCD so that dh is fetched from HBM
+//               once and shared through that L2
+//   workgroup : 8 waves; wave w owns units 32w..32w+31 and all 8 row blocks of the
+//               group: 8 accumulators of v_mfma_f32_32x32x16_bf16
+//   K loop    : 64 columns per iteration (4 MFMA K steps of 16).  The record side is
+//               shared through LDS: each wave fetches the dwords of one (K step,
+//               128-byte span) -- 4 features x 8 columns per lane -- turns them into
+//               four ready MFMA fragments (feature 4i+c of the span is row i of
+//               fragment c) and all waves read them back, one 16-byte read per
+//               fragment.  The gradient side is private to the wave: 8 loads of 4
+//               bytes per lane and K step (each a coalesced 128-byte row piece),
+//               split into hi/mid/lo by masking.
+//   output    : partial sums per split, folded in ascending split order by
+//               k_splitk_reduce (run-to-run bitwise stable).
+// The last map bytes (768..791) and the 51 fp32 features go through the fp32 GEMM as
+// a 75-row operand (k_expand_obs_tail + gemm_dw_ld).
+#include "policy_tile.h"
+
+namespace cfp {
+namespace {
+
+constexpr int kEgThreads = 512;
+constexpr int kEgGroups = 3;               // feature groups of 256 map bytes
+constexpr int kEgBlocks = 8;               // 32-row MFMA blocks per group
+constexpr int kEgIterCols = 64;            // columns per iteration
+constexpr int kEgFeat = kEgGroups * 256;   // 768 features on the bf16 path
+constexpr int kEgTail = CFP_OBS - kEgFeat; // 75 features on the fp32 path
+constexpr int kEgTailLd = 76;
+constexpr int kEgXcds = 8;
+constexpr int kRecDw = CFP_REC_BYTES / 4;  // 249
+
+// bf16 pair {byte c of a (low half), byte c of b (high half)}
+template <int C>
+__device__ __forceinline__ uint32_t byte_pair_bf16(uint32_t a, uint32_t b) {
+    const float lo = (float)((a >> (8 * C)) & 0xffu);
+    const float hi = (float)((b >> (8 * C)) & 0xffu);
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+}
+template <int C>
+__device__ __forceinline__ u4 byte_frag(const uint32_t (&d)[8]) {
+    u4 f;
+    f.x = byte_pair_bf16<C>(d[0], d[1]);
+    f.y = byte_pair_bf16<C>(d[2], d[3]);
+    f.z = byte_pair_bf16<C>(d[4], d[5]);
+    f.w = byte_pair_bf16<C>(d[6], d[7]);
+    return f;
+}
+
+// v = hi + mid + lo exactly, each with at most 8 significant bits; packed as bf16
+// pairs (element 2p in the low half).
+__device__ __forceinline__ void split3(const float (&v)[8], u4& hi, u4& mid, u4& lo) {
+    uint32_t h[4], m[4], l[4];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const float v0 = v[2 * p], v1 = v[2 * p + 1];
+        const float r0 = v0 - __uint_as_float(__float_as_uint(v0) & 0xffff0000u);
+        const float r1 = v1 - __uint_as_float(__float_as_uint(v1) & 0xffff0000u);
+        const float l0 = r0 - __uint_as_float(__float_as_uint(r0) & 0xffff0000u);
+        const float l1 = r1 - __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
+        h[p] = __builtin_amdgcn_perm(__float_as_uint(v1), __float_as_uint(v0), 0x07060302u);
+        m[p] = __builtin_amdgcn_perm(__float_as_uint(r1), __float_as_uint(r0), 0x07060302u);
+        l[p] = __builtin_amdgcn_perm(__float_as_uint(l1), __float_as_uint(l0), 0x07060302u);
+    }
+    hi = u4{h[0], h[1], h[2], h[3]};
+    mid = u4{m[0], m[1], m[2], m[3]};
+    lo = u4{l[0], l[1], l[2], l[3]};
+}
+
+__global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
+    const uint8_t* __restrict__ r_obs, const float* __restrict__ dh, float* __restrict__ part,
+    int t0, int cols, int mb, int n_all, int env_start, int iters_per_split, int n_wg) {
+    __shared__ u4 stage[2][4][kEgBlocks][64];   // 64 KiB: [buffer][K step][fragment][lane]
+    const int xcd = (int)(blockIdx.x % kEgXcds), q = (int)(blockIdx.x / kEgXcds);
+    const int lin = xcd * (int)(gridDim.x / kEgXcds) + q;
+    if (lin >= n_wg) return;
+    const int split = lin / kEgGroups, gi = lin - split * kEgGroups;
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int total_iters = (cols + kEgIterCols - 1) / kEgIterCols;
+    const int it0 = split * iters_per_split;
+    const int it1 = min(total_iters, it0 + iters_per_split);
+    const int pks = w >> 1, psb = w & 1;   // the (K step, 128-byte span) this wave stages
+
+    // columns cg..cg+7 of a lane share their time step: minibatches are multiples of 8 envs
+    auto rec_load = [&](int it, uint32_t (&d)[8]) {
+        const int cg = it * kEgIterCols + pks * 16 + 8 * g;
+        if (cg < cols) {
+            const unsigned trw = (unsigned)cg / (unsigned)mb;
+            const unsigned el = (unsigned)cg - trw * (unsigned)mb;
+            const uint32_t* p = reinterpret_cast<const uint32_t*>(
+                r_obs + (((size_t)t0 + trw) * (size_t)n_all + env_start + el) * CFP_REC_BYTES +
+                gi * 256 + psb * 128 + 4 * n);
+#pragma unroll
+            for (int j = 0; j < 8; j++) d[j] = __builtin_nontemporal_load(p + j * kRecDw);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) d[j] = 0u;
+        }
+    };
+    auto rec_store = [&](int buf, const uint32_t (&d)[8]) {
+        stage[buf][pks][psb * 4 + 0][lane] = byte_frag<0>(d);
+        stage[buf][pks][psb * 4 + 1][lane] = byte_frag<1>(d);
+        stage[buf][pks][psb * 4 + 2][lane] = byte_frag<2>(d);
+        stage[buf][pks][psb * 4 + 3][lane] = byte_frag<3>(d);
+    };
+    auto dh_load = [&](int it, int ks, float (&v)[8]) {
+        const int cg = it * kEgIterCols + ks * 16 + 8 * g;
+        if (cg < cols) {
+            const float* p = dh + (size_t)cg * CFP_HIDDEN + 32 * w + n;
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = p[j * CFP_HIDDEN];
+        } else {
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = 0.0f;
+        }
+    };
+
+    f16v acc[kEgBlocks];
+#pragma unroll
+    for (int b = 0; b < kEgBlocks; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
+
+    uint32_t d[8];
+    float raw[4][8];   // gradient rows are requested two K steps ahead of their use
+    if (it0 < it1) {
+        rec_load(it0, d);
+        rec_store(0, d);
+        dh_load(it0, 0, raw[0]);
+        dh_load(it0, 1, raw[1]);
+    }
+    __syncthreads();
+    for (int it = it0; it < it1; it++) {
+        const int buf = (it - it0) & 1;
+        const bool more = it + 1 < it1;
+        if (more) rec_load(it + 1, d);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            if (ks < 2) dh_load(it, ks + 2, raw[ks + 2]);
+            else if (more) dh_load(it + 1, ks - 2, raw[ks - 2]);
+            u4 bh, bm, bl;
+            split3(raw[ks], bh, bm, bl);
+#pragma unroll
+            for (int b = 0; b < kEgBlocks; b += 2) {
+                const u4 a0 = stage[buf][ks][b][lane];
+                const u4 a1 = stage[buf][ks][b + 1][lane];
+                acc[b] = mfma16(a0, bh, acc[b]);
+                acc[b + 1] = mfma16(a1, bh, acc[b + 1]);
+                acc[b] = mfma16(a0, bm, acc[b]);
+                acc[b + 1] = mfma16(a1, bm, acc[b + 1]);
+                acc[b] = mfma16(a0, bl, acc[b]);
+                acc[b + 1] = mfma16(a1, bl, acc[b + 1]);
+            }
+        }
+        if (more) rec_store(buf ^ 1, d);
+        __syncthreads();
+    }
+    // accumulator register r of fragment c of span sb: feature sb*128 + 4*row + c
+    float* o = part + ((size_t)split * kEgFeat + gi * 256) * CFP_HIDDEN + 32 * w + n;
+#pragma unroll
+    for (int b = 0; b < kEgBlocks; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int row = acc_row(r) + 4 * g;
+            o[(size_t)((b >> 2) * 128 + 4 * row + (b & 3)) * CFP_HIDDEN] = acc[b][r];
+        }
+}
+
+// Features 768..842 of the window columns as an fp32 matrix [cols][76]: 24 map bytes,
+// then the record's 51 floats; thread = one 16-byte piece.
+__global__ void k_expand_obs_tail(const uint8_t* __restrict__ r_obs, f4* __restrict__ out,
+                                  int t0, size_t total4, int mb, int n_all, int env_start) {
+    static_assert((CFP_OBS_MAP - kEgFeat) % 4 == 0 && kEgTailLd % 4 == 0, "whole dwords");
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total4) return;
+    constexpr int LD4 = kEgTailLd / 4, MAP4 = (CFP_OBS_MAP - kEgFeat) / 4;   // 19, 6
+    const unsigned c = (unsigned)(idx / LD4);
+    const int q = (int)(idx - (size_t)c * LD4);
+    const unsigned trw = c / (unsigned)mb, el = c - trw * (unsigned)mb;
+    const uint32_t* rec = reinterpret_cast<const uint32_t*>(
+        r_obs + (((size_t)t0 + trw) * (size_t)n_all + env_start + el) * CFP_REC_BYTES);
+    f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (q < MAP4) {
+        const uint32_t b = rec[kEgFeat / 4 + q];
+        v[0] = (float)(b & 0xffu);
+        v[1] = (float)((b >> 8) & 0xffu);
+        v[2] = (float)((b >> 16) & 0xffu);
+        v[3] = (float)(b >> 24);
+    } else {
+        const int f = 4 * (q - MAP4);
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (f + j < CFP_OBS - CFP_OBS_MAP) v[j] = __uint_as_float(rec[CFP_OBS_MAP / 4 + f + j]);
+    }
+    out[idx] = v;
+}
+
+}  // namespace
+
+bool dw_enc_records_ok(int mb) { return mb > 0 && mb % 8 == 0; }
+
+int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
+                   int cols, int mb, int n_all, int env_start, hipStream_t st) {
+    CFP_REQUIRE(r_obs && dh && dW && tail_scratch && cols > 0 && dw_enc_records_ok(mb) &&
+                    cols % 8 == 0,
+                "dw_enc_records: columns and envs per minibatch must be multiples of 8");
+    float* work = nullptr;
+    size_t work_floats = 0;
+    if (dw_workspace(&work, &work_floats)) return 1;
+    const int total_iters = (cols + kEgIterCols - 1) / kEgIterCols;
+    // one workgroup per CU: 85 splits x 3 groups
+    int splits = 256 / kEgGroups;
+    const int cap = (int)(work_floats / ((size_t)kEgFeat * CFP_HIDDEN));
+    if (splits > cap) splits = cap;
+    if (splits > total_iters) splits = total_iters;
+    const int ips = (total_iters + splits - 1) / splits;
+    splits = (total_iters + ips - 1) / ips;
+    const int n_wg = splits * kEgGroups;
+    const int grid = (n_wg + kEgXcds - 1) / kEgXcds * kEgXcds;
+    hipLaunchKernelGGL(k_dw_enc_bytes, dim3(grid), dim3(kEgThreads), 0, st, r_obs, dh, work, t0,
+                       cols, mb, n_all, env_start, ips, n_wg);
+    const long count = (long)kEgFeat * CFP_HIDDEN;
+    if (launch_splitk_reduce(dW, work, count, count, splits, st)) return 1;
+    const size_t total4 = (size_t)cols * (kEgTailLd / 4);
+    hipLaunchKernelGGL(k_expand_obs_tail, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, st,
+                       r_obs, reinterpret_cast<f4*>(tail_scratch), t0, total4, mb, n_all,
+                       env_start);
+    CFP_HIP_TRY(hipGetLastError());
+    return gemm_dw_ld(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, st);
+}
+
+}  // namespace cfp

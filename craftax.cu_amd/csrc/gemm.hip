@@ -303,15 +303,35 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_gemm_bf16(GemmArgs g) {
         }
 }
 
-// dst[i] += sum_z part[z*stride + i], z ascending.
-__global__ void k_splitk_reduce(float* __restrict__ dst,
-                                const float* __restrict__ part, long count,
-                                long stride, int splits) {
-    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= count) return;
-    float s = 0.0f;
-    for (int z = 0; z < splits; z++) s += part[(long)z * stride + i];
-    dst[i] += s;
+// dst[i] += sum_z part[z*stride + i] in a fixed order: the splits are dealt to four
+// thread groups (contiguous quarters), each walks its quarter with four independent
+// running sums (z = 0, 1, 2, 3 mod 4), and the sixteen sums are folded in one fixed
+// tree -- enough loads in flight to run at memory speed, run-to-run bitwise stable.
+constexpr int kReduceOut = 64;   // outputs per workgroup of 256 threads
+__global__ __launch_bounds__(256) void k_splitk_reduce(float* __restrict__ dst,
+                                                       const float* __restrict__ part,
+                                                       long count, long stride, int splits) {
+    __shared__ float fold[4][kReduceOut];
+    const int o = threadIdx.x & (kReduceOut - 1), zg = threadIdx.x / kReduceOut;
+    const long i = (long)blockIdx.x * kReduceOut + o;
+    const int per = (splits + 3) / 4;
+    const int z0 = zg * per, z1 = min(splits, z0 + per);
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    if (i < count) {
+        const float* p = part + i;
+        int z = z0;
+        for (; z + 4 <= z1; z += 4) {
+            s0 += p[(long)z * stride];
+            s1 += p[(long)(z + 1) * stride];
+            s2 += p[(long)(z + 2) * stride];
+            s3 += p[(long)(z + 3) * stride];
+        }
+        for (; z < z1; z++) s0 += p[(long)z * stride];
+    }
+    fold[zg][o] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (zg == 0 && i < count)
+        dst[i] += (fold[0][o] + fold[1][o]) + (fold[2][o] + fold[3][o]);
 }
 
 // dWv[k] += sum_c x[c][k] * dv[c].  Stage 1: workgroup z owns a contiguous slice
@@ -424,6 +444,24 @@ int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* 
     return run_gemm<true, false>(g, 1, accumulate, st);
 }
 
+// The split-K workspace, allocated on first use; shared by everything that runs its
+// partial sums and their fold back to back on one stream.
+int dw_workspace(float** work, size_t* floats) {
+    if (!g_dw_work)
+        CFP_HIP_TRY(hipMalloc((void**)&g_dw_work, kDwWorkFloats * sizeof(float)));
+    *work = g_dw_work;
+    *floats = kDwWorkFloats;
+    return 0;
+}
+
+int launch_splitk_reduce(float* dst, const float* part, long count, long stride, int splits,
+                         hipStream_t st) {
+    hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)((count + kReduceOut - 1) / kReduceOut)),
+                       dim3(256), 0, st, dst, part, count, stride, splits);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld_dpre,
                float* d_dW, hipStream_t st) {
     CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW &&
@@ -451,16 +489,13 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
         g.C = d_dW; g.c_split = 0;
         return run_gemm<false, false>(g, 1, true, st);
     }
-    if (!g_dw_work)
-        CFP_HIP_TRY(hipMalloc((void**)&g_dw_work, kDwWorkFloats * sizeof(float)));
+    size_t work_floats = 0;
+    if (dw_workspace(&g_dw_work, &work_floats)) return 1;
     g.C = g_dw_work;
     g.c_split = (long)rows * CFP_HIDDEN;
     if (run_gemm<false, false>(g, splits, false, st) != 0) return 1;
     const long count = (long)rows * CFP_HIDDEN;
-    hipLaunchKernelGGL(k_splitk_reduce, dim3((unsigned)((count + 255) / 256)),
-                       dim3(256), 0, st, d_dW, g_dw_work, count, count, splits);
-    CFP_HIP_TRY(hipGetLastError());
-    return 0;
+    return launch_splitk_reduce(d_dW, g_dw_work, count, count, splits, st);
 }
 
 }  // namespace cfp
@@ -513,10 +548,8 @@ int cfp_gemv_dwv(const float* d_x, const float* d_dv, float* d_dWv, int cols,
     const int slices = (cols + per - 1) / per;
     hipLaunchKernelGGL(k_gemv_dwv_partial, dim3(slices), dim3(256), 0, st, d_x, d_dv,
                        g_gemv_work, cols, per);
-    hipLaunchKernelGGL(k_splitk_reduce, dim3(1), dim3(256), 0, st, d_dWv, g_gemv_work,
-                       (long)CFP_HIDDEN, (long)CFP_HIDDEN, slices);
-    CFP_HIP_TRY(hipGetLastError());
-    return 0;
+    return launch_splitk_reduce(d_dWv, g_gemv_work, (long)CFP_HIDDEN, (long)CFP_HIDDEN, slices,
+                                st);
 }
 
 }  // extern "C"

@@ -668,8 +668,10 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             for (int l = 0; l < L; l++) fa.tr_pre[l] = tr->preb[l];
             for (int l = 0; l <= L; l++) fa.tr_x[l] = tr->x[l];
             if (launch_forward(fa, st)) return 1;
-            // the dW_enc GEMM of the reverse pass still reads the fp32 feature matrix
-            if (launch_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, kObsPad, st))
+            // without the record-fed dW_enc kernel the reverse pass reads the fp32
+            // feature matrix
+            if (!dw_enc_records_ok(mb) &&
+                launch_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, kObsPad, st))
                 return 1;
         } else {
             if (launch_expand_obs(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, kObsPad, st))
@@ -722,7 +724,15 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         }
         // ---- encoder: db_enc; dW_enc += xobs^T dh_enc (dh_enc sits in dhX)
         if (colsum_into(tr, tr->dhX, g + CFP_OFF_B_ENC, H, cols, st)) return 1;
-        if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, st)) return 1;
+        if (dw_enc_records_ok(mb)) {
+            // map bytes straight from the records; xobs is free by now and takes the
+            // 76-float rows of the fp32 remainder
+            if (dw_enc_records(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
+                               env_start, st))
+                return 1;
+        } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, st)) {
+            return 1;
+        }
     }
     CFP_HIP_TRY(hipGetLastError());
     return 0;
