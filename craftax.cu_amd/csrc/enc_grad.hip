@@ -92,38 +92,37 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
     const int it1 = min(total_iters, it0 + iters_per_split);
     const int pks = w >> 1, psb = w & 1;   // the (K step, 128-byte span) this wave stages
 
-    // columns cg..cg+7 of a lane share their time step: minibatches are multiples of 8 envs
+    // columns cg..cg+7 of a lane share their time step: minibatches are multiples of 8
+    // envs.  The loop body is branch free: loads past the last column are redirected
+    // to the last 8 columns, and the record side of such columns is zeroed, which
+    // makes their products zero whatever the gradient side holds.
     auto rec_load = [&](int it, uint32_t (&d)[8]) {
         const int cg = it * kEgIterCols + pks * 16 + 8 * g;
-        if (cg < cols) {
-            const unsigned trw = (unsigned)cg / (unsigned)mb;
-            const unsigned el = (unsigned)cg - trw * (unsigned)mb;
-            const uint32_t* p = reinterpret_cast<const uint32_t*>(
-                r_obs + (((size_t)t0 + trw) * (size_t)n_all + env_start + el) * CFP_REC_BYTES +
-                gi * 256 + psb * 128 + 4 * n);
+        const int cc = min(cg, cols - 8);
+        const unsigned trw = (unsigned)cc / (unsigned)mb;
+        const unsigned el = (unsigned)cc - trw * (unsigned)mb;
+        const uint32_t* p = reinterpret_cast<const uint32_t*>(
+            r_obs + (((size_t)t0 + trw) * (size_t)n_all + env_start + el) * CFP_REC_BYTES +
+            gi * 256 + psb * 128 + 4 * n);
 #pragma unroll
-            for (int j = 0; j < 8; j++) d[j] = __builtin_nontemporal_load(p + j * kRecDw);
-        } else {
+        for (int j = 0; j < 8; j++) d[j] = __builtin_nontemporal_load(p + j * kRecDw);
+    };
+    auto rec_store = [&](int it, int buf, const uint32_t (&d)[8]) {
+        const bool in = it * kEgIterCols + pks * 16 + 8 * g < cols;
+        uint32_t e[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) d[j] = 0u;
-        }
+        for (int j = 0; j < 8; j++) e[j] = in ? d[j] : 0u;
+        stage[buf][pks][psb * 4 + 0][lane] = byte_frag<0>(e);
+        stage[buf][pks][psb * 4 + 1][lane] = byte_frag<1>(e);
+        stage[buf][pks][psb * 4 + 2][lane] = byte_frag<2>(e);
+        stage[buf][pks][psb * 4 + 3][lane] = byte_frag<3>(e);
     };
-    auto rec_store = [&](int buf, const uint32_t (&d)[8]) {
-        stage[buf][pks][psb * 4 + 0][lane] = byte_frag<0>(d);
-        stage[buf][pks][psb * 4 + 1][lane] = byte_frag<1>(d);
-        stage[buf][pks][psb * 4 + 2][lane] = byte_frag<2>(d);
-        stage[buf][pks][psb * 4 + 3][lane] = byte_frag<3>(d);
-    };
+    const float* dh_lane = dh + 32 * w + n;
     auto dh_load = [&](int it, int ks, float (&v)[8]) {
-        const int cg = it * kEgIterCols + ks * 16 + 8 * g;
-        if (cg < cols) {
-            const float* p = dh + (size_t)cg * CFP_HIDDEN + 32 * w + n;
+        const int cc = min(it * kEgIterCols + ks * 16 + 8 * g, cols - 8);
+        const float* p = dh_lane + (size_t)cc * CFP_HIDDEN;
 #pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = p[j * CFP_HIDDEN];
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = 0.0f;
-        }
+        for (int j = 0; j < 8; j++) v[j] = p[j * CFP_HIDDEN];
     };
 
     f16v acc[kEgBlocks];
@@ -132,39 +131,62 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
 
-    uint32_t d[8];
-    float raw[4][8];   // gradient rows are requested two K steps ahead of their use
     if (it0 < it1) {
+        // Software pipeline.  Gradient rows are requested three K steps ahead of their
+        // MFMAs and split one K step ahead; record fragments come out of LDS one pair
+        // ahead; the next iteration's records are requested at the top of the
+        // iteration and staged into the other buffer during its last K step.  The
+        // barrier sits after this wave's last read of the current buffer has
+        // returned, so a buffer is never written while another wave still reads it.
+        uint32_t d[8];
+        float raw[4][8];
         rec_load(it0, d);
-        rec_store(0, d);
+        rec_store(it0, 0, d);
         dh_load(it0, 0, raw[0]);
         dh_load(it0, 1, raw[1]);
-    }
-    __syncthreads();
-    for (int it = it0; it < it1; it++) {
-        const int buf = (it - it0) & 1;
-        const bool more = it + 1 < it1;
-        if (more) rec_load(it + 1, d);
+        dh_load(it0, 2, raw[2]);
+        __syncthreads();
+        u4 a[2][2];
+        a[0][0] = stage[0][0][0][lane];
+        a[0][1] = stage[0][0][1][lane];
+        u4 bh, bm, bl;
+        split3(raw[0], bh, bm, bl);
+        for (int it = it0; it < it1; it++) {
+            const int buf = (it - it0) & 1;
+            const int itn = min(it + 1, it1 - 1);
+            rec_load(itn, d);
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            if (ks < 2) dh_load(it, ks + 2, raw[ks + 2]);
-            else if (more) dh_load(it + 1, ks - 2, raw[ks - 2]);
-            u4 bh, bm, bl;
-            split3(raw[ks], bh, bm, bl);
+            for (int ks = 0; ks < 4; ks++) {
+                if (ks < 1) dh_load(it, ks + 3, raw[ks + 3]);
+                else dh_load(itn, ks - 1, raw[ks - 1]);
+                u4 nh, nm, nl;
+                split3(raw[(ks + 1) & 3], nh, nm, nl);
 #pragma unroll
-            for (int b = 0; b < kEgBlocks; b += 2) {
-                const u4 a0 = stage[buf][ks][b][lane];
-                const u4 a1 = stage[buf][ks][b + 1][lane];
-                acc[b] = mfma16(a0, bh, acc[b]);
-                acc[b + 1] = mfma16(a1, bh, acc[b + 1]);
-                acc[b] = mfma16(a0, bm, acc[b]);
-                acc[b + 1] = mfma16(a1, bm, acc[b + 1]);
-                acc[b] = mfma16(a0, bl, acc[b]);
-                acc[b + 1] = mfma16(a1, bl, acc[b + 1]);
+                for (int pr = 0; pr < 4; pr++) {
+                    const int cur = pr & 1, nxt = cur ^ 1;
+                    if (pr < 3) {
+                        a[nxt][0] = stage[buf][ks][2 * pr + 2][lane];
+                        a[nxt][1] = stage[buf][ks][2 * pr + 3][lane];
+                    } else if (ks < 3) {
+                        a[nxt][0] = stage[buf][ks + 1][0][lane];
+                        a[nxt][1] = stage[buf][ks + 1][1][lane];
+                    } else {
+                        rec_store(itn, buf ^ 1, d);
+                        __syncthreads();
+                        a[nxt][0] = stage[buf ^ 1][0][0][lane];
+                        a[nxt][1] = stage[buf ^ 1][0][1][lane];
+                    }
+                    const int b = 2 * pr;
+                    acc[b] = mfma16(a[cur][0], bh, acc[b]);
+                    acc[b + 1] = mfma16(a[cur][1], bh, acc[b + 1]);
+                    acc[b] = mfma16(a[cur][0], bm, acc[b]);
+                    acc[b + 1] = mfma16(a[cur][1], bm, acc[b + 1]);
+                    acc[b] = mfma16(a[cur][0], bl, acc[b]);
+                    acc[b + 1] = mfma16(a[cur][1], bl, acc[b + 1]);
+                }
+                bh = nh; bm = nm; bl = nl;
             }
         }
-        if (more) rec_store(buf ^ 1, d);
-        __syncthreads();
     }
     // accumulator register r of fragment c of span sb: feature sb*128 + 4*row + c
     float* o = part + ((size_t)split * kEgFeat + gi * 256) * CFP_HIDDEN + 32 * w + n;
