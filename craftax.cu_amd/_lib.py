@@ -46,6 +46,8 @@ PROTOTYPES = {
                                      C.c_int, vp]),
     "cfp_set_gemm_bf16": (C.c_int, [C.c_int]),
     "cfp_get_gemm_bf16": (C.c_int, []),
+    "cfp_set_gemm_split": (C.c_int, [C.c_int]),
+    "cfp_get_gemm_split": (C.c_int, []),
     "cfp_gemm_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
     "cfp_gemm_enc_fwd": (C.c_int, [C.c_int, vp, vp, vp, vp]),
     "cfp_gemm_dh": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),

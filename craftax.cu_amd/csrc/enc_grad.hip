@@ -58,26 +58,6 @@ __device__ __forceinline__ u4 byte_frag(const uint32_t (&d)[8]) {
     return f;
 }
 
-// v = hi + mid + lo exactly, each with at most 8 significant bits; packed as bf16
-// pairs (element 2p in the low half).
-__device__ __forceinline__ void split3(const float (&v)[8], u4& hi, u4& mid, u4& lo) {
-    uint32_t h[4], m[4], l[4];
-#pragma unroll
-    for (int p = 0; p < 4; p++) {
-        const float v0 = v[2 * p], v1 = v[2 * p + 1];
-        const float r0 = v0 - __uint_as_float(__float_as_uint(v0) & 0xffff0000u);
-        const float r1 = v1 - __uint_as_float(__float_as_uint(v1) & 0xffff0000u);
-        const float l0 = r0 - __uint_as_float(__float_as_uint(r0) & 0xffff0000u);
-        const float l1 = r1 - __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
-        h[p] = __builtin_amdgcn_perm(__float_as_uint(v1), __float_as_uint(v0), 0x07060302u);
-        m[p] = __builtin_amdgcn_perm(__float_as_uint(r1), __float_as_uint(r0), 0x07060302u);
-        l[p] = __builtin_amdgcn_perm(__float_as_uint(l1), __float_as_uint(l0), 0x07060302u);
-    }
-    hi = u4{h[0], h[1], h[2], h[3]};
-    mid = u4{m[0], m[1], m[2], m[3]};
-    lo = u4{l[0], l[1], l[2], l[3]};
-}
-
 __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
     const uint8_t* __restrict__ r_obs, const float* __restrict__ dh, float* __restrict__ part,
     int t0, int cols, int mb, int n_all, int env_start, int iters_per_split, int n_wg) {

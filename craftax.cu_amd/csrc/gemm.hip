@@ -369,6 +369,8 @@ static bool vec_ok(const float* p, long ld, int fast_extent) {
 // Process-wide switch of the seam's GEMMs to bf16 inputs, like the reference's
 // g_gemm_bf16 (craftax_full.cu:11306-11316).
 int g_gemm_bf16 = 0;
+// fp32 operands split into bf16 triples for the update's shapes (gemm_x9.hip)
+int g_gemm_split = 1;
 
 template <bool A_KFAST, bool B_KFAST, bool ACCUM>
 int launch_gemm(const GemmArgs& g, dim3 grid, bool va, bool vb, hipStream_t st) {
@@ -467,6 +469,8 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
     CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW &&
                     ld_dpre >= rows,
                 "cfp_gemm_dw: bad argument (rows must be in 1..%d)", CFP_OBS);
+    if (!g_gemm_bf16 && g_gemm_split && gemm_dw_x9_ok(rows, cols))
+        return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, st);
     // enough workgroups to fill 256 CUs: tiles(M) * tiles(N=2) * splits
     const int tiles = ((rows + BM - 1) / BM) * (CFP_HIDDEN / BN);
     int splits = (2048 + tiles - 1) / tiles;   // measured: 128 splits of the gate dW beat 64 by 3 %
@@ -507,6 +511,11 @@ int cfp_set_gemm_bf16(int on) {
     return 0;
 }
 int cfp_get_gemm_bf16(void) { return g_gemm_bf16; }
+int cfp_set_gemm_split(int on) {
+    g_gemm_split = on ? 1 : 0;
+    return 0;
+}
+int cfp_get_gemm_split(void) { return g_gemm_split; }
 
 int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
                  float* d_y, void* stream) {

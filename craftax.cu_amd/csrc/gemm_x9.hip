@@ -1,0 +1,182 @@
+// fp32 GEMMs of the PPO update on the bf16 matrix pipe.
+//
+// An fp32 number is exactly hi + mid + lo with three bf16 numbers (8 + 8 + 8 significand
+// bits, split3), so a product a*b is exactly the sum of the nine products of their
+// parts, each of which is exact in fp32 (8 x 8 bits).  Nine v_mfma_f32_32x32x16_bf16
+// with fp32 accumulation therefore add up the same exact products as the fp32 MFMA --
+// with one accumulator rounding per 16 products instead of per 2 -- and take 9/16 of
+// its pipe time.  The reference runs these GEMMs as cublasSgemm behind cu_gemm_dw
+// and cu_gemm_dh (craftax_full.cu:11642-11666).
+//
+// k_dw_x9: dW[rows][256] += sum_c dpre[c][row] * x[c][unit], K = window columns.
+//   grid      : (rows / 128) row groups x S splits of the columns; the groups of a
+//               split sit on one XCD and share x through its L2
+//   workgroup : 8 waves; wave w owns units 32w..32w+31 and the group's four 32-row
+//               blocks (4 accumulators)
+//   K loop    : 64 columns per iteration (4 K steps of 16).  dpre side through LDS:
+//               every wave fetches two (K step, row block) pieces -- 8 columns per
+//               lane, each load a coalesced 128-byte row piece -- splits them and
+//               stores three ready MFMA fragments each.  x side private to the wave,
+//               split in registers.  Same software pipeline as the record-fed
+//               encoder kernel.
+//   output    : per-split partial sums, folded in a fixed order.
+#include "policy_tile.h"
+
+namespace cfp {
+namespace {
+
+constexpr int kX9Threads = 512;
+constexpr int kX9Blocks = 4;               // 32-row blocks per row group
+constexpr int kX9GroupRows = 32 * kX9Blocks;
+constexpr int kX9IterCols = 64;
+constexpr int kX9Xcds = 8;
+
+__global__ __launch_bounds__(kX9Threads) void k_dw_x9(
+    const float* __restrict__ dpre, int ldp, int rows, const float* __restrict__ x,
+    float* __restrict__ part, int cols, int iters_per_split, int n_wg, int groups) {
+    // [buffer][K step][3 * row block + part][lane]: 96 KiB
+    __shared__ u4 stage[2][4][3 * kX9Blocks][64];
+    const int xcd = (int)(blockIdx.x % kX9Xcds), q = (int)(blockIdx.x / kX9Xcds);
+    const int lin = xcd * (int)(gridDim.x / kX9Xcds) + q;
+    if (lin >= n_wg) return;
+    const int split = lin / groups, gi = lin - split * groups;
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int total_iters = (cols + kX9IterCols - 1) / kX9IterCols;
+    const int it0 = split * iters_per_split;
+    const int it1 = min(total_iters, it0 + iters_per_split);
+    // this wave stages row block pb of K steps pk and pk + 2
+    const int pk = w >> 2, pb = w & 3;
+
+    // Branch-free body: loads past the last column go to the last 8 columns and the
+    // dpre side of such columns is zeroed (cols % 8 == 0, so 8-column groups are all
+    // in or all out).
+    const float* dp_lane = dpre + gi * kX9GroupRows + 32 * pb + n;
+    auto dp_load = [&](int it, int ks, float (&v)[8]) {
+        const int cc = min(it * kX9IterCols + ks * 16 + 8 * g, cols - 8);
+        const float* p = dp_lane + (size_t)cc * ldp;
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = p[(size_t)j * ldp];
+    };
+    auto dp_store = [&](int it, int ks, int buf, const float (&v)[8]) {
+        const bool in = it * kX9IterCols + ks * 16 + 8 * g < cols;
+        float e[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) e[j] = in ? v[j] : 0.0f;
+        u4 h, m, l;
+        split3(e, h, m, l);
+        stage[buf][ks][3 * pb + 0][lane] = h;
+        stage[buf][ks][3 * pb + 1][lane] = m;
+        stage[buf][ks][3 * pb + 2][lane] = l;
+    };
+    const float* x_lane = x + 32 * w + n;
+    auto x_load = [&](int it, int ks, float (&v)[8]) {
+        const int cc = min(it * kX9IterCols + ks * 16 + 8 * g, cols - 8);
+        const float* p = x_lane + (size_t)cc * CFP_HIDDEN;
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = p[j * CFP_HIDDEN];
+    };
+    auto frag_load = [&](int buf, int ks, int pair, u4 (&a)[6]) {
+#pragma unroll
+        for (int i = 0; i < 6; i++) a[i] = stage[buf][ks][6 * pair + i][lane];
+    };
+
+    f16v acc[kX9Blocks];
+#pragma unroll
+    for (int b = 0; b < kX9Blocks; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
+
+    if (it0 < it1) {
+        float d0[8], d1[8];
+        float raw[4][8];
+        dp_load(it0, pk, d0);
+        dp_load(it0, pk + 2, d1);
+        x_load(it0, 0, raw[0]);
+        x_load(it0, 1, raw[1]);
+        x_load(it0, 2, raw[2]);
+        dp_store(it0, pk, 0, d0);
+        dp_store(it0, pk + 2, 0, d1);
+        __syncthreads();
+        u4 a[2][6];
+        frag_load(0, 0, 0, a[0]);
+        u4 bs[3];
+        split3(raw[0], bs[0], bs[1], bs[2]);
+        for (int it = it0; it < it1; it++) {
+            const int buf = (it - it0) & 1;
+            const int itn = min(it + 1, it1 - 1);
+            dp_load(itn, pk, d0);
+            dp_load(itn, pk + 2, d1);
+#pragma unroll
+            for (int ks = 0; ks < 4; ks++) {
+                if (ks < 1) x_load(it, ks + 3, raw[ks + 3]);
+                else x_load(itn, ks - 1, raw[ks - 1]);
+                u4 ns[3];
+                split3(raw[(ks + 1) & 3], ns[0], ns[1], ns[2]);
+#pragma unroll
+                for (int pr = 0; pr < 2; pr++) {
+                    const int cur = pr, nxt = pr ^ 1;
+                    if (pr < 1) {
+                        frag_load(buf, ks, 1, a[nxt]);
+                    } else if (ks < 3) {
+                        frag_load(buf, ks + 1, 0, a[nxt]);
+                    } else {
+                        // this wave's last read of the current buffer is in flight or
+                        // done; the barrier's wait covers it
+                        dp_store(itn, pk, buf ^ 1, d0);
+                        dp_store(itn, pk + 2, buf ^ 1, d1);
+                        __syncthreads();
+                        frag_load(buf ^ 1, 0, 0, a[nxt]);
+                    }
+                    const int b = 2 * pr;
+#pragma unroll
+                    for (int i = 0; i < 3; i++)
+#pragma unroll
+                        for (int j = 0; j < 3; j++) {
+                            acc[b] = mfma16(a[cur][i], bs[j], acc[b]);
+                            acc[b + 1] = mfma16(a[cur][3 + i], bs[j], acc[b + 1]);
+                        }
+                }
+                bs[0] = ns[0]; bs[1] = ns[1]; bs[2] = ns[2];
+            }
+        }
+    }
+    float* o = part + ((size_t)split * rows + gi * kX9GroupRows) * CFP_HIDDEN + 32 * w + n;
+#pragma unroll
+    for (int b = 0; b < kX9Blocks; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++)
+            o[(size_t)(32 * b + acc_row(r) + 4 * g) * CFP_HIDDEN] = acc[b][r];
+}
+
+}  // namespace
+
+bool gemm_dw_x9_ok(int rows, int cols) {
+    return rows > 0 && rows % kX9GroupRows == 0 && cols >= 8 && cols % 8 == 0;
+}
+
+int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
+               hipStream_t st) {
+    CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows,
+                "gemm_dw_x9: rows must be a multiple of %d and columns of 8", kX9GroupRows);
+    float* work = nullptr;
+    size_t work_floats = 0;
+    if (dw_workspace(&work, &work_floats)) return 1;
+    const int groups = rows / kX9GroupRows;
+    const int total_iters = (cols + kX9IterCols - 1) / kX9IterCols;
+    int splits = 256 / groups;   // one workgroup per CU
+    const int cap = (int)(work_floats / ((size_t)rows * CFP_HIDDEN));
+    if (splits > cap) splits = cap;
+    if (splits > total_iters) splits = total_iters;
+    if (splits < 1) splits = 1;
+    const int ips = (total_iters + splits - 1) / splits;
+    splits = (total_iters + ips - 1) / ips;
+    const int n_wg = splits * groups;
+    const int grid = (n_wg + kX9Xcds - 1) / kX9Xcds * kX9Xcds;
+    hipLaunchKernelGGL(k_dw_x9, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x, work,
+                       cols, ips, n_wg, groups);
+    CFP_HIP_TRY(hipGetLastError());
+    const long count = (long)rows * CFP_HIDDEN;
+    return launch_splitk_reduce(dW, work, count, count, splits, st);
+}
+
+}  // namespace cfp

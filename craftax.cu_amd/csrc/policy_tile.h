@@ -193,6 +193,26 @@ __device__ __forceinline__ f16v mfma16(const u4& a, const u4& b, f16v c) {
                                                    __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// v = hi + mid + lo exactly, each with at most 8 significant bits; packed as bf16
+// pairs (element 2p in the low half).
+__device__ __forceinline__ void split3(const float (&v)[8], u4& hi, u4& mid, u4& lo) {
+    uint32_t h[4], m[4], l[4];
+#pragma unroll
+    for (int p = 0; p < 4; p++) {
+        const float v0 = v[2 * p], v1 = v[2 * p + 1];
+        const float r0 = v0 - __uint_as_float(__float_as_uint(v0) & 0xffff0000u);
+        const float r1 = v1 - __uint_as_float(__float_as_uint(v1) & 0xffff0000u);
+        const float l0 = r0 - __uint_as_float(__float_as_uint(r0) & 0xffff0000u);
+        const float l1 = r1 - __uint_as_float(__float_as_uint(r1) & 0xffff0000u);
+        h[p] = __builtin_amdgcn_perm(__float_as_uint(v1), __float_as_uint(v0), 0x07060302u);
+        m[p] = __builtin_amdgcn_perm(__float_as_uint(r1), __float_as_uint(r0), 0x07060302u);
+        l[p] = __builtin_amdgcn_perm(__float_as_uint(l1), __float_as_uint(l0), 0x07060302u);
+    }
+    hi = u4{h[0], h[1], h[2], h[3]};
+    mid = u4{m[0], m[1], m[2], m[3]};
+    lo = u4{l[0], l[1], l[2], l[3]};
+}
+
 // Two record bytes -> two bf16 (0..255 are exact in bf16: the upper half of the
 // fp32 encoding).
 __device__ __forceinline__ uint32_t bytes_to_bf16x2(uint32_t w, int i) {

@@ -286,6 +286,12 @@ def set_gemm_bf16(on=True):
     _check(lib().cfp_set_gemm_bf16(1 if on else 0))
 
 
+def set_gemm_split(on=True):
+    """Process-wide: fp32 GEMMs of the update's shapes as nine exact bf16 partial
+    products per product (on by default); off = fp32 MFMA everywhere."""
+    _check(lib().cfp_set_gemm_split(1 if on else 0))
+
+
 def gemm_fwd(W, x, y=None):
     """y[cols][m] = x[cols][k] . W[m][k]^T (cu_gemm_fwd :11604)."""
     m, k = W.shape

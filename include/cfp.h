@@ -167,6 +167,14 @@ int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
  * and dh GEMMs; this library does not).  Off by default. */
 int cfp_set_gemm_bf16(int on);
 int cfp_get_gemm_bf16(void);
+/* fp32 GEMMs on the bf16 matrix pipe: every fp32 operand is split exactly into three
+ * bf16 numbers and each product becomes the nine exact partial products, accumulated
+ * in fp32 (same products as cublasSgemm adds up behind cu_gemm_dw / cu_gemm_dh,
+ * craftax_full.cu:11642-11666, in 9/16 of the fp32 pipe time).  Used by cfp_gemm_dw and
+ * cfp_gemm_dh for the shapes of the PPO update when bf16 inputs are off; other shapes
+ * take the fp32 MFMA kernel.  On by default; off = fp32 MFMA everywhere. */
+int cfp_set_gemm_split(int on);
+int cfp_get_gemm_split(void);
 
 /* cu_gemm_fwd (:11604): y[cols][m] = x[cols][k] . W[m][k]^T. */
 int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,

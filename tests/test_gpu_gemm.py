@@ -58,6 +58,28 @@ def test_gemm_dw_accumulates(pkg, cuda, rows, cols):
     assert torch.equal(dW, dW2)
 
 
+@pytest.mark.parametrize("rows,cols", [(768, 4096), (768, 1000), (128, 8)])
+def test_gemm_dw_split_is_as_accurate_as_fp32_mfma(pkg, cuda, rows, cols):
+    """fp32 operands as bf16 triples, nine partial products each: the error against
+    fp64 must stay at the level of the fp32 MFMA kernel's.  A missing partial product
+    would show as a relative error of 2^-16 (hi*lo) or 2^-8 (hi*mid), far above it."""
+    import torch
+    x, d = _r((cols, HIDDEN), cuda, 21), _r((cols, rows), cuda, 22)
+    want = (d.double().T @ x.double())
+    scale = (d.double().abs().T @ x.double().abs())
+    errs = {}
+    assert pkg.policy.lib().cfp_get_gemm_split() == 1
+    for on in (True, False):
+        pkg.policy.set_gemm_split(on)
+        dW = torch.zeros(rows, HIDDEN, device=cuda)
+        pkg.policy.gemm_dw(x, d, dW)
+        torch.cuda.synchronize()
+        errs[on] = ((dW.double() - want).abs() / scale).max().item()
+    pkg.policy.set_gemm_split(True)
+    assert errs[True] <= 3.0 * errs[False] + 1e-7, errs
+    assert errs[True] < 2e-6, errs
+
+
 def test_gemv_dwv(pkg, cuda):
     import torch
     x, dv = _r((5000, HIDDEN), cuda, 9), _r((5000,), cuda, 10)
