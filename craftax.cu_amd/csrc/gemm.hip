@@ -437,6 +437,8 @@ int gemm_enc_fwd_ld(int cols, const float* d_W_enc, const float* d_xobs, int ldx
 int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* d_dh,
                 bool accumulate, hipStream_t st) {
     CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh: bad argument");
+    if (!g_gemm_bf16 && g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre))
+        return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, st);
     GemmArgs g{};
     g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
     g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;

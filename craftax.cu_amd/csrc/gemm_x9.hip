@@ -148,7 +148,148 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
             o[(size_t)(32 * b + acc_row(r) + 4 * g) * CFP_HIDDEN] = acc[b][r];
 }
 
+// k_dh_x9: dh[c][u] (+)= sum_k dpre[c][k] * W[k][u] for 256 units, K = m3 (multiple of 16).
+//   workgroup : 256 columns; wave w owns columns 32w..32w+31 of them and all 256 units
+//               (8 accumulators).  Its dpre fragment of a K step is 32 contiguous
+//               bytes per lane, split in registers one step ahead.
+//   W         : split once into an MFMA-ordered mirror (k_pack_w_x9: [K step][unit tile]
+//               [part][lane] 16-byte fragments); every step the eight waves copy its 24
+//               fragments into LDS (3 each) and all read them back, two at a time, one
+//               group of 6 MFMAs ahead of their use.  One barrier per step, placed
+//               before the step's last group so that the next step's first fragments
+//               are on their way while it runs.
+constexpr int kDhThreads = 512;
+constexpr int kDhTileCols = 256;
+constexpr int kDhFrags = 24;   // 8 unit tiles x 3 parts per K step
+
+__global__ void k_pack_w_x9(const float* __restrict__ W, u4* __restrict__ out, int total) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total) return;
+    const int lane = idx & 63, f = (idx >> 6) % kDhFrags, s = idx / (64 * kDhFrags);
+    const int t = f / 3, part = f - 3 * t, n = lane & 31, g = lane >> 5;
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = W[(size_t)(16 * s + 8 * g + j) * CFP_HIDDEN + 32 * t + n];
+    u4 h, m, l;
+    split3(v, h, m, l);
+    out[idx] = part == 0 ? h : (part == 1 ? m : l);
+}
+
+__global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ dpre, int m3,
+                                                      const u4* __restrict__ wm,
+                                                      float* __restrict__ dh, int cols,
+                                                      int accumulate) {
+    __shared__ u4 stage[2][kDhFrags][64];   // 48 KiB
+    const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
+    const int steps = m3 / 16;
+    const int cb = (int)blockIdx.x * kDhTileCols + 32 * w;
+    const bool live = cb < cols;               // cols % 32 == 0: blocks are whole
+    const int cbc = live ? cb : cols - 32;     // idle waves still stage W and meet the barriers
+    const float* a_lane = dpre + (size_t)(cbc + n) * m3 + 8 * g;
+    auto a_load = [&](int s, float (&v)[8]) {
+        const f4* p = reinterpret_cast<const f4*>(a_lane + 16 * s);
+        const f4 x0 = p[0], x1 = p[1];
+#pragma unroll
+        for (int j = 0; j < 4; j++) { v[j] = x0[j]; v[4 + j] = x1[j]; }
+    };
+    const u4* w_lane = wm + (size_t)3 * w * 64 + lane;
+    auto w_load = [&](int s, u4 (&b)[3]) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) b[i] = w_lane[((size_t)s * kDhFrags + i) * 64];
+    };
+    auto w_store = [&](int buf, const u4 (&b)[3]) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) stage[buf][3 * w + i][lane] = b[i];
+    };
+    // group q of a step: unit tiles 2*(q/3), 2*(q/3)+1, part q%3 of W
+    auto frag_load = [&](int buf, int q, u4 (&b)[2]) {
+        const int tp = q / 3, j = q - 3 * tp;
+        b[0] = stage[buf][6 * tp + j][lane];
+        b[1] = stage[buf][6 * tp + 3 + j][lane];
+    };
+
+    f16v acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.0f;
+
+    float raw[2][8];
+    u4 wb[3];
+    const int last = steps - 1;
+    w_load(0, wb);
+    a_load(0, raw[0]);
+    a_load(min(1, last), raw[1]);
+    w_store(0, wb);
+    w_load(min(1, last), wb);
+    u4 as[3];
+    split3(raw[0], as[0], as[1], as[2]);
+    __syncthreads();
+    u4 b[2][2];
+    frag_load(0, 0, b[0]);
+    for (int s = 0; s < steps; s++) {
+        const int buf = s & 1;
+        // raw[s & 1] held step s (already split): refill it two steps ahead
+        if (s & 1) a_load(min(s + 2, last), raw[1]);
+        else a_load(min(s + 2, last), raw[0]);
+        u4 ns[3];
+        if (s & 1) split3(raw[0], ns[0], ns[1], ns[2]);
+        else split3(raw[1], ns[0], ns[1], ns[2]);
+#pragma unroll
+        for (int q = 0; q < 12; q++) {
+            const int cur = q & 1, nxt = cur ^ 1;
+            if (q < 11) {
+                frag_load(buf, q + 1, b[nxt]);
+            } else {
+                // next step's W parts: everyone is past its reads of the other buffer
+                // (they precede the previous barrier)
+                w_store(buf ^ 1, wb);
+                __syncthreads();
+                w_load(min(s + 2, last), wb);
+                frag_load(buf ^ 1, 0, b[nxt]);
+            }
+            const int t = 2 * (q / 3);
+#pragma unroll
+            for (int i = 0; i < 3; i++) {
+                acc[t] = mfma16(as[i], b[cur][0], acc[t]);
+                acc[t + 1] = mfma16(as[i], b[cur][1], acc[t + 1]);
+            }
+        }
+        as[0] = ns[0]; as[1] = ns[1]; as[2] = ns[2];
+    }
+    if (!live) return;
+#pragma unroll
+    for (int t = 0; t < 8; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            float* o = dh + (size_t)(cb + acc_row(r) + 4 * g) * CFP_HIDDEN + 32 * t + n;
+            *o = accumulate ? *o + acc[t][r] : acc[t][r];
+        }
+}
+
+u4* g_w_x9 = nullptr;   // W mirror of the call in flight: one stream at a time
+constexpr int kDhMaxK = CFP_GRU;
+
 }  // namespace
+
+bool gemm_dh_x9_ok(int m3, int cols, const float* dpre) {
+    return m3 >= 16 && m3 % 16 == 0 && m3 <= kDhMaxK && cols >= 32 && cols % 32 == 0 &&
+           (reinterpret_cast<uintptr_t>(dpre) & 15u) == 0;
+}
+
+int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
+               hipStream_t st) {
+    CFP_REQUIRE(gemm_dh_x9_ok(m3, cols, dpre) && W && dh,
+                "gemm_dh_x9: K must be a multiple of 16 up to %d and columns of 32", kDhMaxK);
+    if (!g_w_x9)
+        CFP_HIP_TRY(hipMalloc((void**)&g_w_x9, (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4)));
+    const int total = (m3 / 16) * kDhFrags * 64;
+    hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, W, g_w_x9, total);
+    hipLaunchKernelGGL(k_dh_x9, dim3((cols + kDhTileCols - 1) / kDhTileCols), dim3(kDhThreads), 0,
+                       st, dpre, m3, g_w_x9, dh, cols, accumulate ? 1 : 0);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
 
 bool gemm_dw_x9_ok(int rows, int cols) {
     return rows > 0 && rows % kX9GroupRows == 0 && cols >= 8 && cols % 8 == 0;

@@ -80,6 +80,26 @@ def test_gemm_dw_split_is_as_accurate_as_fp32_mfma(pkg, cuda, rows, cols):
     assert errs[True] < 2e-6, errs
 
 
+@pytest.mark.parametrize("m3,cols", [(768, 8192), (768, 32), (768, 4000 * 32), (48, 288)])
+def test_gemm_dh_split_is_as_accurate_as_fp32_mfma(pkg, cuda, m3, cols):
+    """Same bar for dh = dpre . W on bf16 triples (W split into an MFMA-ordered mirror,
+    dpre in registers).  The accumulating form (layer 0 of the update, onto the highway
+    term) has no entry point of its own and is covered by the trainer's parity tests."""
+    import torch
+    W, d = _r((m3, HIDDEN), cuda, 23, 0.1), _r((cols, m3), cuda, 24)
+    want = d.double() @ W.double()
+    scale = d.double().abs() @ W.double().abs()
+    errs = {}
+    for on in (True, False):
+        pkg.policy.set_gemm_split(on)
+        out = pkg.policy.gemm_dh(W, d)
+        torch.cuda.synchronize()
+        errs[on] = ((out.double() - want).abs() / scale).max().item()
+    pkg.policy.set_gemm_split(True)
+    assert errs[True] <= 3.0 * errs[False] + 1e-7, errs
+    assert errs[True] < 2e-6, errs
+
+
 def test_gemv_dwv(pkg, cuda):
     import torch
     x, dv = _r((5000, HIDDEN), cuda, 9), _r((5000,), cuda, 10)
