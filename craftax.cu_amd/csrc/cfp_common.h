@@ -142,7 +142,7 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
                    int cols, int mb, int n_all, int env_start, hipStream_t st);
 
 // dW[rows][256] += dpre^T x with both fp32 operands split into bf16 triples
-// (rows % 128 == 0, cols % 8 == 0)
+// (cols % 8 == 0)
 bool gemm_dw_x9_ok(int rows, int cols);
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
                hipStream_t st);

@@ -9,7 +9,7 @@
 // and cu_gemm_dh (craftax_full.cu:11642-11666).
 //
 // k_dw_x9: dW[rows][256] += sum_c dpre[c][row] * x[c][unit], K = window columns.
-//   grid      : (rows / 128) row groups x S splits of the columns; the groups of a
+//   grid      : ceil(rows / 128) row groups x S splits of the columns; the groups of a
 //               split sit on one XCD and share x through its L2
 //   workgroup : 8 waves; wave w owns units 32w..32w+31 and the group's four 32-row
 //               blocks (4 accumulators)
@@ -50,7 +50,8 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
     // Branch-free body: loads past the last column go to the last 8 columns and the
     // dpre side of such columns is zeroed (cols % 8 == 0, so 8-column groups are all
     // in or all out).
-    const float* dp_lane = dpre + gi * kX9GroupRows + 32 * pb + n;
+    // rows past the last one read the last row; their results are not stored
+    const float* dp_lane = dpre + min(gi * kX9GroupRows + 32 * pb + n, rows - 1);
     auto dp_load = [&](int it, int ks, float (&v)[8]) {
         const int cc = min(it * kX9IterCols + ks * 16 + 8 * g, cols - 8);
         const float* p = dp_lane + (size_t)cc * ldp;
@@ -144,8 +145,10 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
 #pragma unroll
     for (int b = 0; b < kX9Blocks; b++)
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-            o[(size_t)(32 * b + acc_row(r) + 4 * g) * CFP_HIDDEN] = acc[b][r];
+        for (int r = 0; r < 16; r++) {
+            const int row = 32 * b + acc_row(r) + 4 * g;
+            if (gi * kX9GroupRows + row < rows) o[(size_t)row * CFP_HIDDEN] = acc[b][r];
+        }
 }
 
 // k_dh_x9: dh[c][u] (+)= sum_k dpre[c][k] * W[k][u] for 256 units, K = m3 (multiple of 16).
@@ -208,11 +211,15 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
         b[1] = stage[buf][6 * tp + 3 + j][lane];
     };
 
+    // accumulating form: the accumulators start from dh, all 128 loads in flight at
+    // once under the prologue's own loads, and the epilogue is stores only
+    float* o_lane = dh + (size_t)(cbc + 4 * g) * CFP_HIDDEN + n;
     f16v acc[8];
 #pragma unroll
     for (int t = 0; t < 8; t++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[t][r] = 0.0f;
+        for (int r = 0; r < 16; r++)
+            acc[t][r] = accumulate ? o_lane[(size_t)acc_row(r) * CFP_HIDDEN + 32 * t] : 0.0f;
 
     float raw[2][8];
     u4 wb[3];
@@ -261,10 +268,8 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
 #pragma unroll
     for (int t = 0; t < 8; t++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            float* o = dh + (size_t)(cb + acc_row(r) + 4 * g) * CFP_HIDDEN + 32 * t + n;
-            *o = accumulate ? *o + acc[t][r] : acc[t][r];
-        }
+        for (int r = 0; r < 16; r++)
+            o_lane[(size_t)acc_row(r) * CFP_HIDDEN + 32 * t] = acc[t][r];
 }
 
 u4* g_w_x9 = nullptr;   // W mirror of the call in flight: one stream at a time
@@ -292,17 +297,17 @@ int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, b
 }
 
 bool gemm_dw_x9_ok(int rows, int cols) {
-    return rows > 0 && rows % kX9GroupRows == 0 && cols >= 8 && cols % 8 == 0;
+    return rows > 0 && cols >= 8 && cols % 8 == 0;
 }
 
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
                hipStream_t st) {
     CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows,
-                "gemm_dw_x9: rows must be a multiple of %d and columns of 8", kX9GroupRows);
+                "gemm_dw_x9: columns must be a multiple of 8");
     float* work = nullptr;
     size_t work_floats = 0;
     if (dw_workspace(&work, &work_floats)) return 1;
-    const int groups = rows / kX9GroupRows;
+    const int groups = (rows + kX9GroupRows - 1) / kX9GroupRows;
     const int total_iters = (cols + kX9IterCols - 1) / kX9IterCols;
     int splits = 256 / groups;   // one workgroup per CU
     const int cap = (int)(work_floats / ((size_t)rows * CFP_HIDDEN));

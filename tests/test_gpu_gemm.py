@@ -58,7 +58,8 @@ def test_gemm_dw_accumulates(pkg, cuda, rows, cols):
     assert torch.equal(dW, dW2)
 
 
-@pytest.mark.parametrize("rows,cols", [(768, 4096), (768, 1000), (128, 8)])
+@pytest.mark.parametrize("rows,cols", [(768, 4096), (768, 1000), (128, 8), (75, 2048), (43, 520),
+                                       (843, 264)])
 def test_gemm_dw_split_is_as_accurate_as_fp32_mfma(pkg, cuda, rows, cols):
     """fp32 operands as bf16 triples, nine partial products each: the error against
     fp64 must stay at the level of the fp32 MFMA kernel's.  A missing partial product
