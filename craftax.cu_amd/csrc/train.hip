@@ -159,17 +159,40 @@ __global__ __launch_bounds__(256) void k_loss_fold(const double* __restrict__ bl
 }
 
 // out[r] += sum_c src[c*rows + r]: partial sums over `slices` column ranges
-// (grid.x), then folded in slice order by k_colsum_fold.
+// (grid.x), then folded in slice order by k_colsum_fold.  A workgroup covers RB rows
+// with CL = 256 / RB threads each; a thread walks every CL-th column of the slice with
+// four independent running sums (loads in flight instead of one dependent chain) and
+// the CL sums of a row are added in thread order: a fixed order throughout.
+template <int RB>
 __global__ __launch_bounds__(256) void k_colsum_partial(
     const float* __restrict__ src, float* __restrict__ part, int rows, int cols,
     int cols_per_slice) {
-    const int r = blockIdx.y * 256 + threadIdx.x;
-    if (r >= rows) return;
+    constexpr int CL = 256 / RB;
+    __shared__ float red[CL][RB];
+    const int rl = threadIdx.x % RB, cl = threadIdx.x / RB;
+    const int r = blockIdx.y * RB + rl;
     const int c0 = blockIdx.x * cols_per_slice;
     const int c1 = min(cols, c0 + cols_per_slice);
-    float s = 0.0f;
-    for (int c = c0; c < c1; c++) s += src[(size_t)c * rows + r];
-    part[(size_t)blockIdx.x * rows + r] = s;
+    float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+    if (r < rows) {
+        const float* p = src + r;
+        int c = c0 + cl;
+        for (; c + 3 * CL < c1; c += 4 * CL) {
+            s0 += p[(size_t)c * rows];
+            s1 += p[(size_t)(c + CL) * rows];
+            s2 += p[(size_t)(c + 2 * CL) * rows];
+            s3 += p[(size_t)(c + 3 * CL) * rows];
+        }
+        for (; c < c1; c += CL) s0 += p[(size_t)c * rows];
+    }
+    red[cl][rl] = (s0 + s1) + (s2 + s3);
+    __syncthreads();
+    if (cl == 0 && r < rows) {
+        float t = red[0][rl];
+#pragma unroll
+        for (int i = 1; i < CL; i++) t += red[i][rl];
+        part[(size_t)blockIdx.x * rows + r] = t;
+    }
 }
 // Fixed order: thread (row, c) of 4 x 64 sums the slices of chunk c in ascending
 // order, thread (row, 0) then adds the 64 chunk sums in ascending order.
@@ -612,8 +635,12 @@ static int colsum_into(cfp_trainer* tr, const float* src, float* out, int rows, 
     if (slices > cols) slices = cols;
     const int per = (cols + slices - 1) / slices;
     slices = (cols + per - 1) / per;
-    hipLaunchKernelGGL(k_colsum_partial, dim3(slices, (rows + 255) / 256), dim3(256), 0,
-                       st, src, tr->colsum_part, rows, cols, per);
+    if (rows <= 64)
+        hipLaunchKernelGGL(k_colsum_partial<64>, dim3(slices, 1), dim3(256), 0, st, src,
+                           tr->colsum_part, rows, cols, per);
+    else
+        hipLaunchKernelGGL(k_colsum_partial<256>, dim3(slices, (rows + 255) / 256), dim3(256), 0,
+                           st, src, tr->colsum_part, rows, cols, per);
     hipLaunchKernelGGL(k_colsum_fold, dim3((rows + 3) / 4), dim3(256), 0, st,
                        tr->colsum_part, out, rows, slices);
     CFP_HIP_TRY(hipGetLastError());
