@@ -82,6 +82,15 @@ def ppo_update(pkg, torch, reps):
            "samples_per_s": samples / ms * 1e3,
            "tflops": UPD_FLOP * samples / ms / 1e9,
            "frac_fp32_mfma_peak": UPD_FLOP * samples / ms / 1e9 / PEAK_FP32}
+    # same update with the GEMMs as fp32 MFMA (mode 0) and as six partial products (mode 2)
+    for mode, key in ((0, "fp32_mfma_gemms"), (2, "split6_gemms")):
+        pkg.policy.set_gemm_split(mode)
+        try:
+            ms_m = _time(torch, step, reps, warm=1)
+        finally:
+            pkg.policy.set_gemm_split(1)
+        out[key] = {"ms_per_update": ms_m, "samples_per_s": samples / ms_m * 1e3,
+                    "tflops": UPD_FLOP * samples / ms_m / 1e9}
     pkg.policy.set_gemm_bf16(True)       # same update with bf16 GEMM inputs
     try:
         ms16 = _time(torch, step, reps, warm=1)

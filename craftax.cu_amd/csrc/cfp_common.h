@@ -145,13 +145,13 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
 // (cols % 8 == 0)
 bool gemm_dw_x9_ok(int rows, int cols);
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               hipStream_t st);
+               int terms, hipStream_t st);
 
 // dh[cols][256] (+)= dpre[cols][m3] . W[m3][256], same splitting (m3 % 16 == 0,
 // cols % 32 == 0, dpre 16-byte aligned)
 bool gemm_dh_x9_ok(int m3, int cols, const float* dpre);
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               hipStream_t st);
+               int terms, hipStream_t st);
 
 // per-variant arena geometry
 struct Arena {

@@ -438,7 +438,7 @@ int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* 
                 bool accumulate, hipStream_t st) {
     CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh: bad argument");
     if (!g_gemm_bf16 && g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre))
-        return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, st);
+        return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, g_gemm_split == 2 ? 6 : 9, st);
     GemmArgs g{};
     g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
     g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
@@ -472,7 +472,7 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
                     ld_dpre >= rows,
                 "cfp_gemm_dw: bad argument (rows must be in 1..%d)", CFP_OBS);
     if (!g_gemm_bf16 && g_gemm_split && gemm_dw_x9_ok(rows, cols))
-        return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, st);
+        return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, g_gemm_split == 2 ? 6 : 9, st);
     // enough workgroups to fill 256 CUs: tiles(M) * tiles(N=2) * splits
     const int tiles = ((rows + BM - 1) / BM) * (CFP_HIDDEN / BN);
     int splits = (2048 + tiles - 1) / tiles;   // measured: 128 splits of the gate dW beat 64 by 3 %
@@ -513,8 +513,9 @@ int cfp_set_gemm_bf16(int on) {
     return 0;
 }
 int cfp_get_gemm_bf16(void) { return g_gemm_bf16; }
-int cfp_set_gemm_split(int on) {
-    g_gemm_split = on ? 1 : 0;
+int cfp_set_gemm_split(int mode) {
+    CFP_REQUIRE(mode >= 0 && mode <= 2, "cfp_set_gemm_split: mode must be 0, 1 or 2 (got %d)", mode);
+    g_gemm_split = mode;
     return 0;
 }
 int cfp_get_gemm_split(void) { return g_gemm_split; }

@@ -7,6 +7,9 @@
 // with one accumulator rounding per 16 products instead of per 2 -- and take 9/16 of
 // its pipe time.  The reference runs these GEMMs as cublasSgemm behind cu_gemm_dw
 // and cu_gemm_dh (craftax_full.cu:11642-11666).
+// TERMS = 6 leaves out mid*lo, lo*mid and lo*lo: at most 2^-23 of |a*b| per product
+// (2^-25 on average, always towards zero since the parts are truncations), i.e. below
+// one fp32 rounding of the product, for two thirds of the MFMAs.  Opt-in.
 //
 // k_dw_x9: dW[rows][256] += sum_c dpre[c][row] * x[c][unit], K = window columns.
 //   grid      : ceil(rows / 128) row groups x S splits of the columns; the groups of a
@@ -31,6 +34,7 @@ constexpr int kX9GroupRows = 32 * kX9Blocks;
 constexpr int kX9IterCols = 64;
 constexpr int kX9Xcds = 8;
 
+template <int TERMS>
 __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
     const float* __restrict__ dpre, int ldp, int rows, const float* __restrict__ x,
     float* __restrict__ part, int cols, int iters_per_split, int n_wg, int groups) {
@@ -133,6 +137,7 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
                     for (int i = 0; i < 3; i++)
 #pragma unroll
                         for (int j = 0; j < 3; j++) {
+                            if (TERMS == 6 && i + j > 2) continue;
                             acc[b] = mfma16(a[cur][i], bs[j], acc[b]);
                             acc[b + 1] = mfma16(a[cur][3 + i], bs[j], acc[b + 1]);
                         }
@@ -178,6 +183,7 @@ __global__ void k_pack_w_x9(const float* __restrict__ W, u4* __restrict__ out, i
     out[idx] = part == 0 ? h : (part == 1 ? m : l);
 }
 
+template <int TERMS>
 __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ dpre, int m3,
                                                       const u4* __restrict__ wm,
                                                       float* __restrict__ dh, int cols,
@@ -258,6 +264,7 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             const int t = 2 * (q / 3);
 #pragma unroll
             for (int i = 0; i < 3; i++) {
+                if (TERMS == 6 && i + q % 3 > 2) continue;
                 acc[t] = mfma16(as[i], b[cur][0], acc[t]);
                 acc[t + 1] = mfma16(as[i], b[cur][1], acc[t + 1]);
             }
@@ -283,15 +290,20 @@ bool gemm_dh_x9_ok(int m3, int cols, const float* dpre) {
 }
 
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               hipStream_t st) {
+               int terms, hipStream_t st) {
     CFP_REQUIRE(gemm_dh_x9_ok(m3, cols, dpre) && W && dh,
                 "gemm_dh_x9: K must be a multiple of 16 up to %d and columns of 32", kDhMaxK);
     if (!g_w_x9)
         CFP_HIP_TRY(hipMalloc((void**)&g_w_x9, (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4)));
     const int total = (m3 / 16) * kDhFrags * 64;
     hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, W, g_w_x9, total);
-    hipLaunchKernelGGL(k_dh_x9, dim3((cols + kDhTileCols - 1) / kDhTileCols), dim3(kDhThreads), 0,
-                       st, dpre, m3, g_w_x9, dh, cols, accumulate ? 1 : 0);
+    const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
+    if (terms == 6)
+        hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, dpre, m3, g_w_x9, dh, cols,
+                           accumulate ? 1 : 0);
+    else
+        hipLaunchKernelGGL(k_dh_x9<9>, grid, dim3(kDhThreads), 0, st, dpre, m3, g_w_x9, dh, cols,
+                           accumulate ? 1 : 0);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -301,7 +313,7 @@ bool gemm_dw_x9_ok(int rows, int cols) {
 }
 
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               hipStream_t st) {
+               int terms, hipStream_t st) {
     CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows,
                 "gemm_dw_x9: columns must be a multiple of 8");
     float* work = nullptr;
@@ -318,8 +330,12 @@ int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpr
     splits = (total_iters + ips - 1) / ips;
     const int n_wg = splits * groups;
     const int grid = (n_wg + kX9Xcds - 1) / kX9Xcds * kX9Xcds;
-    hipLaunchKernelGGL(k_dw_x9, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x, work,
-                       cols, ips, n_wg, groups);
+    if (terms == 6)
+        hipLaunchKernelGGL(k_dw_x9<6>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
+                           work, cols, ips, n_wg, groups);
+    else
+        hipLaunchKernelGGL(k_dw_x9<9>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
+                           work, cols, ips, n_wg, groups);
     CFP_HIP_TRY(hipGetLastError());
     const long count = (long)rows * CFP_HIDDEN;
     return launch_splitk_reduce(dW, work, count, count, splits, st);

@@ -286,10 +286,11 @@ def set_gemm_bf16(on=True):
     _check(lib().cfp_set_gemm_bf16(1 if on else 0))
 
 
-def set_gemm_split(on=True):
-    """Process-wide: fp32 GEMMs of the update's shapes as nine exact bf16 partial
-    products per product (on by default); off = fp32 MFMA everywhere."""
-    _check(lib().cfp_set_gemm_split(1 if on else 0))
+def set_gemm_split(mode=1):
+    """Process-wide: fp32 GEMMs of the update's shapes on the bf16 pipe.  1 (default):
+    nine exact bf16 partial products per product; 2: the six largest; 0: fp32 MFMA
+    everywhere."""
+    _check(lib().cfp_set_gemm_split(int(mode)))
 
 
 def gemm_fwd(W, x, y=None):

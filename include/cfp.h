@@ -172,8 +172,10 @@ int cfp_get_gemm_bf16(void);
  * in fp32 (same products as cublasSgemm adds up behind cu_gemm_dw / cu_gemm_dh,
  * craftax_full.cu:11642-11666, in 9/16 of the fp32 pipe time).  Used by cfp_gemm_dw and
  * cfp_gemm_dh for the shapes of the PPO update when bf16 inputs are off; other shapes
- * take the fp32 MFMA kernel.  On by default; off = fp32 MFMA everywhere. */
-int cfp_set_gemm_split(int on);
+ * take the fp32 MFMA kernel.  mode 1 (default): all nine partial products; mode 2: the
+ * six largest (mid*lo, lo*mid, lo*lo left out: at most 2^-23 of |a*b| per product,
+ * below one fp32 rounding of it; opt-in); mode 0: fp32 MFMA everywhere. */
+int cfp_set_gemm_split(int mode);
 int cfp_get_gemm_split(void);
 
 /* cu_gemm_fwd (:11604): y[cols][m] = x[cols][k] . W[m][k]^T. */

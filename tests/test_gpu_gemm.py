@@ -58,6 +58,21 @@ def test_gemm_dw_accumulates(pkg, cuda, rows, cols):
     assert torch.equal(dW, dW2)
 
 
+def _check_split_errors(errs):
+    """errs[mode] = max |got - fp64| / sum_k |a_k b_k|.  Mode 1 (nine exact partial
+    products) must sit at the fp32 MFMA kernel's level (mode 0); mode 2 (six) may add
+    its documented 2^-23 per product on top."""
+    assert errs[1] <= 3.0 * errs[0] + 1e-7, errs
+    assert errs[1] < 2e-6, errs
+    assert errs[2] <= 3.0 * errs[0] + 1e-7 + 2.0 ** -23, errs
+
+
+def test_gemm_split_mode_is_checked(pkg, cuda):
+    with pytest.raises(pkg._lib.CfpError, match="mode must be 0, 1 or 2"):
+        pkg.policy.set_gemm_split(3)
+    assert pkg.policy.lib().cfp_get_gemm_split() == 1
+
+
 @pytest.mark.parametrize("rows,cols", [(768, 4096), (768, 1000), (128, 8), (75, 2048), (43, 520),
                                        (843, 264)])
 def test_gemm_dw_split_is_as_accurate_as_fp32_mfma(pkg, cuda, rows, cols):
@@ -70,15 +85,14 @@ def test_gemm_dw_split_is_as_accurate_as_fp32_mfma(pkg, cuda, rows, cols):
     scale = (d.double().abs().T @ x.double().abs())
     errs = {}
     assert pkg.policy.lib().cfp_get_gemm_split() == 1
-    for on in (True, False):
-        pkg.policy.set_gemm_split(on)
+    for mode in (1, 2, 0):
+        pkg.policy.set_gemm_split(mode)
         dW = torch.zeros(rows, HIDDEN, device=cuda)
         pkg.policy.gemm_dw(x, d, dW)
         torch.cuda.synchronize()
-        errs[on] = ((dW.double() - want).abs() / scale).max().item()
-    pkg.policy.set_gemm_split(True)
-    assert errs[True] <= 3.0 * errs[False] + 1e-7, errs
-    assert errs[True] < 2e-6, errs
+        errs[mode] = ((dW.double() - want).abs() / scale).max().item()
+    pkg.policy.set_gemm_split(1)
+    _check_split_errors(errs)
 
 
 @pytest.mark.parametrize("m3,cols", [(768, 8192), (768, 32), (768, 4000 * 32), (48, 288)])
@@ -91,14 +105,13 @@ def test_gemm_dh_split_is_as_accurate_as_fp32_mfma(pkg, cuda, m3, cols):
     want = d.double() @ W.double()
     scale = d.double().abs() @ W.double().abs()
     errs = {}
-    for on in (True, False):
-        pkg.policy.set_gemm_split(on)
+    for mode in (1, 2, 0):
+        pkg.policy.set_gemm_split(mode)
         out = pkg.policy.gemm_dh(W, d)
         torch.cuda.synchronize()
-        errs[on] = ((out.double() - want).abs() / scale).max().item()
-    pkg.policy.set_gemm_split(True)
-    assert errs[True] <= 3.0 * errs[False] + 1e-7, errs
-    assert errs[True] < 2e-6, errs
+        errs[mode] = ((out.double() - want).abs() / scale).max().item()
+    pkg.policy.set_gemm_split(1)
+    _check_split_errors(errs)
 
 
 def test_gemv_dwv(pkg, cuda):
