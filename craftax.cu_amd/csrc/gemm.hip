@@ -371,6 +371,8 @@ static bool vec_ok(const float* p, long ld, int fast_extent) {
 int g_gemm_bf16 = 0;
 // fp32 operands split into bf16 triples for the update's shapes (gemm_x9.hip)
 int g_gemm_split = 1;
+// partial products per product on those kernels: bf16 inputs -> 1 (rounded operands)
+inline int split_terms() { return g_gemm_bf16 ? 1 : (g_gemm_split == 2 ? 6 : 9); }
 
 template <bool A_KFAST, bool B_KFAST, bool ACCUM>
 int launch_gemm(const GemmArgs& g, dim3 grid, bool va, bool vb, hipStream_t st) {
@@ -437,8 +439,8 @@ int gemm_enc_fwd_ld(int cols, const float* d_W_enc, const float* d_xobs, int ldx
 int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* d_dh,
                 bool accumulate, hipStream_t st) {
     CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh: bad argument");
-    if (!g_gemm_bf16 && g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre))
-        return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, g_gemm_split == 2 ? 6 : 9, st);
+    if (g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre))
+        return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, split_terms(), st);
     GemmArgs g{};
     g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
     g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
@@ -471,8 +473,8 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
     CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW &&
                     ld_dpre >= rows,
                 "cfp_gemm_dw: bad argument (rows must be in 1..%d)", CFP_OBS);
-    if (!g_gemm_bf16 && g_gemm_split && gemm_dw_x9_ok(rows, cols))
-        return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, g_gemm_split == 2 ? 6 : 9, st);
+    if (g_gemm_split && gemm_dw_x9_ok(rows, cols))
+        return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, split_terms(), st);
     // enough workgroups to fill 256 CUs: tiles(M) * tiles(N=2) * splits
     const int tiles = ((rows + BM - 1) / BM) * (CFP_HIDDEN / BN);
     int splits = (2048 + tiles - 1) / tiles;   // measured: 128 splits of the gate dW beat 64 by 3 %

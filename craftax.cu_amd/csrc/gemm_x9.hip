@@ -10,6 +10,8 @@
 // TERMS = 6 leaves out mid*lo, lo*mid and lo*lo: at most 2^-23 of |a*b| per product
 // (2^-25 on average, always towards zero since the parts are truncations), i.e. below
 // one fp32 rounding of the product, for two thirds of the MFMAs.  Opt-in.
+// TERMS = 1 is the seam's bf16-input mode (operands rounded to nearest even, one
+// product) on the same kernels: same loads and pipeline, a ninth of the MFMAs.
 //
 // k_dw_x9: dW[rows][256] += sum_c dpre[c][row] * x[c][unit], K = window columns.
 //   grid      : ceil(rows / 128) row groups x S splits of the columns; the groups of a
@@ -27,6 +29,23 @@
 
 namespace cfp {
 namespace {
+
+// The operand parts a kernel multiplies: TERMS = 9 or 6 -> the exact triple; TERMS = 1 ->
+// the operand rounded to bf16 (the bf16-input mode of the seam), one product.
+template <int TERMS>
+__device__ __forceinline__ void parts_of(const float (&v)[8], u4 (&p)[3]) {
+    if (TERMS == 1) {
+        p[0] = round_bf16x8(v);
+        p[1] = p[0];
+        p[2] = p[0];
+    } else {
+        split3(v, p[0], p[1], p[2]);
+    }
+}
+template <int TERMS>
+__device__ __forceinline__ constexpr bool term_used(int i, int j) {
+    return TERMS == 9 || (TERMS == 6 && i + j <= 2) || (TERMS == 1 && i == 0 && j == 0);
+}
 
 constexpr int kX9Threads = 512;
 constexpr int kX9Blocks = 4;               // 32-row blocks per row group
@@ -67,11 +86,13 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
         float e[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) e[j] = in ? v[j] : 0.0f;
-        u4 h, m, l;
-        split3(e, h, m, l);
-        stage[buf][ks][3 * pb + 0][lane] = h;
-        stage[buf][ks][3 * pb + 1][lane] = m;
-        stage[buf][ks][3 * pb + 2][lane] = l;
+        u4 p[3];
+        parts_of<TERMS>(e, p);
+        stage[buf][ks][3 * pb + 0][lane] = p[0];
+        if (TERMS > 1) {
+            stage[buf][ks][3 * pb + 1][lane] = p[1];
+            stage[buf][ks][3 * pb + 2][lane] = p[2];
+        }
     };
     const float* x_lane = x + 32 * w + n;
     auto x_load = [&](int it, int ks, float (&v)[8]) {
@@ -105,7 +126,7 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
         u4 a[2][6];
         frag_load(0, 0, 0, a[0]);
         u4 bs[3];
-        split3(raw[0], bs[0], bs[1], bs[2]);
+        parts_of<TERMS>(raw[0], bs);
         for (int it = it0; it < it1; it++) {
             const int buf = (it - it0) & 1;
             const int itn = min(it + 1, it1 - 1);
@@ -116,7 +137,7 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
                 if (ks < 1) x_load(it, ks + 3, raw[ks + 3]);
                 else x_load(itn, ks - 1, raw[ks - 1]);
                 u4 ns[3];
-                split3(raw[(ks + 1) & 3], ns[0], ns[1], ns[2]);
+                parts_of<TERMS>(raw[(ks + 1) & 3], ns);
 #pragma unroll
                 for (int pr = 0; pr < 2; pr++) {
                     const int cur = pr, nxt = pr ^ 1;
@@ -137,7 +158,7 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
                     for (int i = 0; i < 3; i++)
 #pragma unroll
                         for (int j = 0; j < 3; j++) {
-                            if (TERMS == 6 && i + j > 2) continue;
+                            if (!term_used<TERMS>(i, j)) continue;
                             acc[b] = mfma16(a[cur][i], bs[j], acc[b]);
                             acc[b + 1] = mfma16(a[cur][3 + i], bs[j], acc[b + 1]);
                         }
@@ -170,7 +191,8 @@ constexpr int kDhThreads = 512;
 constexpr int kDhTileCols = 256;
 constexpr int kDhFrags = 24;   // 8 unit tiles x 3 parts per K step
 
-__global__ void k_pack_w_x9(const float* __restrict__ W, u4* __restrict__ out, int total) {
+__global__ void k_pack_w_x9(const float* __restrict__ W, u4* __restrict__ out, int total,
+                            int rounded) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int lane = idx & 63, f = (idx >> 6) % kDhFrags, s = idx / (64 * kDhFrags);
@@ -180,6 +202,7 @@ __global__ void k_pack_w_x9(const float* __restrict__ W, u4* __restrict__ out, i
     for (int j = 0; j < 8; j++) v[j] = W[(size_t)(16 * s + 8 * g + j) * CFP_HIDDEN + 32 * t + n];
     u4 h, m, l;
     split3(v, h, m, l);
+    if (rounded) h = round_bf16x8(v);   // bf16-input mode: part 0 is the rounded operand
     out[idx] = part == 0 ? h : (part == 1 ? m : l);
 }
 
@@ -236,7 +259,7 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     w_store(0, wb);
     w_load(min(1, last), wb);
     u4 as[3];
-    split3(raw[0], as[0], as[1], as[2]);
+    parts_of<TERMS>(raw[0], as);
     __syncthreads();
     u4 b[2][2];
     frag_load(0, 0, b[0]);
@@ -246,8 +269,8 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
         if (s & 1) a_load(min(s + 2, last), raw[1]);
         else a_load(min(s + 2, last), raw[0]);
         u4 ns[3];
-        if (s & 1) split3(raw[0], ns[0], ns[1], ns[2]);
-        else split3(raw[1], ns[0], ns[1], ns[2]);
+        if (s & 1) parts_of<TERMS>(raw[0], ns);
+        else parts_of<TERMS>(raw[1], ns);
 #pragma unroll
         for (int q = 0; q < 12; q++) {
             const int cur = q & 1, nxt = cur ^ 1;
@@ -264,7 +287,7 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             const int t = 2 * (q / 3);
 #pragma unroll
             for (int i = 0; i < 3; i++) {
-                if (TERMS == 6 && i + q % 3 > 2) continue;
+                if (!term_used<TERMS>(i, q % 3)) continue;
                 acc[t] = mfma16(as[i], b[cur][0], acc[t]);
                 acc[t + 1] = mfma16(as[i], b[cur][1], acc[t + 1]);
             }
@@ -296,9 +319,13 @@ int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, b
     if (!g_w_x9)
         CFP_HIP_TRY(hipMalloc((void**)&g_w_x9, (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4)));
     const int total = (m3 / 16) * kDhFrags * 64;
-    hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, W, g_w_x9, total);
+    hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, W, g_w_x9, total,
+                       terms == 1 ? 1 : 0);
     const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
-    if (terms == 6)
+    if (terms == 1)
+        hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, dpre, m3, g_w_x9, dh, cols,
+                           accumulate ? 1 : 0);
+    else if (terms == 6)
         hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, dpre, m3, g_w_x9, dh, cols,
                            accumulate ? 1 : 0);
     else
@@ -330,7 +357,10 @@ int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpr
     splits = (total_iters + ips - 1) / ips;
     const int n_wg = splits * groups;
     const int grid = (n_wg + kX9Xcds - 1) / kX9Xcds * kX9Xcds;
-    if (terms == 6)
+    if (terms == 1)
+        hipLaunchKernelGGL(k_dw_x9<1>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
+                           work, cols, ips, n_wg, groups);
+    else if (terms == 6)
         hipLaunchKernelGGL(k_dw_x9<6>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
                            work, cols, ips, n_wg, groups);
     else

@@ -213,6 +213,16 @@ __device__ __forceinline__ void split3(const float (&v)[8], u4& hi, u4& mid, u4&
     lo = u4{l[0], l[1], l[2], l[3]};
 }
 
+// Eight fp32 -> eight bf16, round to nearest even.
+__device__ __forceinline__ u4 round_bf16x8(const float (&v)[8]) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
+    const f4 a = {v[0], v[1], v[2], v[3]}, b = {v[4], v[5], v[6], v[7]};
+    const u2_t lo = __builtin_bit_cast(u2_t, __builtin_convertvector(a, bf16x4_t));
+    const u2_t hi = __builtin_bit_cast(u2_t, __builtin_convertvector(b, bf16x4_t));
+    return u4{lo.x, lo.y, hi.x, hi.y};
+}
+
 // Two record bytes -> two bf16 (0..255 are exact in bf16: the upper half of the
 // fp32 encoding).
 __device__ __forceinline__ uint32_t bytes_to_bf16x2(uint32_t w, int i) {

@@ -174,7 +174,9 @@ int cfp_get_gemm_bf16(void);
  * cfp_gemm_dh for the shapes of the PPO update when bf16 inputs are off; other shapes
  * take the fp32 MFMA kernel.  mode 1 (default): all nine partial products; mode 2: the
  * six largest (mid*lo, lo*mid, lo*lo left out: at most 2^-23 of |a*b| per product,
- * below one fp32 rounding of it; opt-in); mode 0: fp32 MFMA everywhere. */
+ * below one fp32 rounding of it; opt-in); mode 0: fp32 MFMA everywhere (and, with bf16
+ * inputs on, the generic bf16 kernel).  With cfp_set_gemm_bf16(1) and mode 1 or 2 the same
+ * kernels run with both operands rounded to bf16 and one product. */
 int cfp_set_gemm_split(int mode);
 int cfp_get_gemm_split(void);
 
