@@ -49,7 +49,11 @@ __device__ __forceinline__ u4 a_frag(const f4* xs4, int l32, int g, int kb) {
 
 }  // namespace
 
-template <int VARIANT, bool HAS_RS>
+// TRAIN: window recompute of the PPO update, as in the fp32 kernel: tile = 32 columns of
+// one step of the slabs (records in r_obs, the stored post-zero state of every layer
+// as the state input), every layer's gate pre-activations and output written out,
+// nothing written back to the state.
+template <int VARIANT, bool HAS_RS, bool TRAIN>
 __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     __shared__ float term_s[kTileEnvs];
@@ -61,10 +65,17 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
     const int l32 = tid & 31;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned loff = (unsigned)((4 * g) * CFP_HIDDEN + l32);
+    const unsigned loff3 = (unsigned)((4 * g) * CFP_GRU + l32);
     const size_t e0 = (size_t)blockIdx.x * kTileEnvs;
     const f4* xs4 = reinterpret_cast<const f4*>(lds);
+    // first env of the tile as an index into the [T][n_all] slabs
+    size_t se = e0;
+    if (TRAIN) {
+        const size_t tr = e0 / (size_t)a.tr_mb;
+        se = ((size_t)a.tr_t0 + tr) * a.tr_n_all + a.tr_env_start + (e0 - tr * a.tr_mb);
+    }
 
-    stage_tile<VARIANT>(a, e0, lds, crec, term_s, tid);
+    stage_tile<VARIANT>(a, se, lds, crec, term_s, tid);
     __syncthreads();
 
     unsigned tmask = 0u;
@@ -137,6 +148,10 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
 #pragma unroll 1
     for (int l = 0; l < a.layers; l++) {
         float* st_base = a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64;
+        if (TRAIN) {
+            const size_t tt = se / a.tr_n_all, ee = se - tt * a.tr_n_all;
+            st_base = a.state + ((tt * a.layers + l) * a.tr_n_all + ee) * CFP_HIDDEN + wave * 64;
+        }
         float st[32];
 #pragma unroll
         for (int e = 0; e < 32; e++)
@@ -165,24 +180,34 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
 
         float* rs_base = HAS_RS ? a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64
                                 : nullptr;
+        float* out_base = TRAIN ? a.tr_x[l + 1] + e0 * CFP_HIDDEN + wave * 64 : nullptr;
+        float* pre_base = TRAIN ? a.tr_pre[l] + e0 * CFP_GRU + wave * 64 : nullptr;
 #pragma unroll
         for (int e = 0; e < 32; e++) {
             const int ut = e / 16, r = e % 16;
             const int soff = acc_row(r) * CFP_HIDDEN + ut * 32;
             float* xp = lds + (acc_row(r) + 4 * g) * XS + wave * 64 + ut * 32 + l32;
-            const float s = (tmask >> r) & 1u ? 0.0f : st[e];
+            const float s = (!TRAIN && ((tmask >> r) & 1u)) ? 0.0f : st[e];
             if (HAS_RS) __builtin_nontemporal_store(s, (rs_base + soff) + loff);
             const float zh = acc[0 + ut][r];
             const float zg = acc[2 + ut][r];
             const float zp = acc[4 + ut][r];
+            if (TRAIN) {
+                float* pp = pre_base + (acc_row(r) * CFP_GRU + ut * 32);
+                __builtin_nontemporal_store(zh, pp + loff3);
+                __builtin_nontemporal_store(zg, (pp + CFP_HIDDEN) + loff3);
+                __builtin_nontemporal_store(zp, (pp + 2 * CFP_HIDDEN) + loff3);
+            }
             const float sg = sigmoid_fast(zg);
             const float sh = sigmoid_fast(zh);
             const float gh = zh >= 0.0f ? zh + 0.5f : sh;
             const float out = s + sg * (gh - s);
             const float p = sigmoid_fast(zp);
             const float xv = *xp;
-            *xp = p * out + (1.0f - p) * xv;
-            __builtin_nontemporal_store(out, (st_base + soff) + loff);
+            const float hn = p * out + (1.0f - p) * xv;
+            *xp = hn;
+            if (TRAIN) __builtin_nontemporal_store(hn, (out_base + soff) + loff);
+            else __builtin_nontemporal_store(out, (st_base + soff) + loff);
         }
         __syncthreads();
     }
@@ -214,12 +239,18 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
 int launch_forward_bf16(const FwdArgs& a, hipStream_t st) {
     CFP_REQUIRE(a.we_bf && a.wg_bf && a.wav_bf, "bf16 forward without bf16 weight mirrors");
     const dim3 g(a.n / kTileEnvs), b(kFwdThreads);
-    if (a.variant == 1) {
-        if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<1, true>), g, b, 0, st, a);
-        else hipLaunchKernelGGL((k_policy_forward_bf16<1, false>), g, b, 0, st, a);
+    if (a.train) {
+        CFP_REQUIRE(a.variant == 0 && a.rec && a.state && a.layers > 0 && !a.r_state &&
+                        !a.terminals && a.tr_mb > 0 && a.tr_mb % kTileEnvs == 0 &&
+                        a.h_enc_out == a.tr_x[0],
+                    "window recompute: bad arguments");
+        hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true>), g, b, 0, st, a);
+    } else if (a.variant == 1) {
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<1, true, false>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward_bf16<1, false, false>), g, b, 0, st, a);
     } else {
-        if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<0, true>), g, b, 0, st, a);
-        else hipLaunchKernelGGL((k_policy_forward_bf16<0, false>), g, b, 0, st, a);
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<0, true, false>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward_bf16<0, false, false>), g, b, 0, st, a);
     }
     CFP_HIP_TRY(hipGetLastError());
     return 0;

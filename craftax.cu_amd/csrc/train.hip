@@ -676,13 +676,14 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         const int cols = Tw * mb;
         const size_t hc = (size_t)H * cols;
         // ---- forward recompute of the window into tight columns: one launch of the
-        // fused forward kernel in its window mode (stored state in, pre-activations
-        // and layer outputs out); with bf16 GEMM inputs the unfused chain below
-        const bool fused = cfp_get_gemm_bf16() == 0;
+        // fused forward kernel (fp32, or the bf16-input one) in its window mode: stored
+        // state in, pre-activations and layer outputs out.  The unfused chain below is
+        // what bf16 inputs run with the split kernels switched off.
+        const bool fused = cfp_get_gemm_bf16() == 0 || cfp_get_gemm_split() != 0;
         if (fused) {
             FwdArgs fa{};
             fill_forward_weights(p, fa);
-            fa.bf16 = 0;
+            fa.bf16 = cfp_get_gemm_bf16();
             fa.rec = tr->r_obs;
             fa.state = tr->r_state;
             fa.h_enc_out = tr->x[0];
