@@ -70,7 +70,7 @@ __global__ __launch_bounds__(128) void k_head_bwd_win(
     float* __restrict__ dlogits, float* __restrict__ dvalue,
     double* __restrict__ block_loss, int t0, int cols, int mb, int n, int n_all,
     int T_all, float clip_eps, float vf_coef, const float* __restrict__ ent_coef_p,
-    int logits_ld) {   // b_a == nullptr: the logits already carry their bias
+    int logits_ld) {   // b_a == nullptr: rows of the fused forward, 43 logits + value, biases included
     __shared__ double s_l[3][128];
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     double l_pg = 0.0, l_v = 0.0, l_e = 0.0;
@@ -109,10 +109,15 @@ __global__ __launch_bounds__(128) void k_head_bwd_win(
         float Hent = 0.0f;
 #pragma unroll
         for (int a = 0; a < A; a++) Hent -= pi[a] * (lg[a] - lse);
-        float v = b_v[0];
-        const float* hc = h3 + (size_t)c * H;
+        float v;
+        if (b_a) {
+            v = b_v[0];
+            const float* hc = h3 + (size_t)c * H;
 #pragma unroll 4
-        for (int j = 0; j < H; j++) v = fmaf(W_v[j], hc[j], v);
+            for (int j = 0; j < H; j++) v = fmaf(W_v[j], hc[j], v);
+        } else {
+            v = lp[A];   // the fused forward leaves the value (bias included) behind the logits
+        }
         const float dret = v - ret[o];
         dvalue[c] = inv_batch * vf_coef * dret;
         float* dq = dlogits + (size_t)c * A;
