@@ -145,7 +145,11 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
 // (cols % 8 == 0)
 bool gemm_dw_x9_ok(int rows, int cols);
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               int terms, hipStream_t st);
+               int terms, hipStream_t st, int rows_first = 0, float* dW_rest = nullptr);
+// dW_a[rows_a][256] += and dW_b[rows_b][256] += from adjacent columns of one dpre matrix
+// (one pass over x on the split kernels, two passes otherwise)
+int gemm_dw_two(int rows_a, int rows_b, int cols, const float* x, const float* dpre, int ld_dpre,
+                float* dW_a, float* dW_b, hipStream_t st);
 
 // dh[cols][256] (+)= dpre[cols][m3] . W[m3][256], same splitting (m3 % 16 == 0,
 // cols % 32 == 0, dpre 16-byte aligned)

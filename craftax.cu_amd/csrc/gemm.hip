@@ -506,6 +506,17 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
     return launch_splitk_reduce(d_dW, g_dw_work, count, count, splits, st);
 }
 
+int gemm_dw_two(int rows_a, int rows_b, int cols, const float* d_x, const float* d_dpre,
+                int ld_dpre, float* d_dW_a, float* d_dW_b, hipStream_t st) {
+    CFP_REQUIRE(rows_a > 0 && rows_b > 0 && ld_dpre >= rows_a + rows_b && d_dW_a && d_dW_b,
+                "gemm_dw_two: bad argument");
+    if (g_gemm_split && gemm_dw_x9_ok(rows_a + rows_b, cols))
+        return gemm_dw_x9(rows_a + rows_b, cols, d_x, d_dpre, ld_dpre, d_dW_a, split_terms(), st,
+                          rows_a, d_dW_b);
+    if (gemm_dw_ld(rows_a, cols, d_x, d_dpre, ld_dpre, d_dW_a, st)) return 1;
+    return gemm_dw_ld(rows_b, cols, d_x, d_dpre + rows_a, ld_dpre, d_dW_b, st);
+}
+
 }  // namespace cfp
 
 extern "C" {

@@ -340,8 +340,9 @@ bool gemm_dw_x9_ok(int rows, int cols) {
 }
 
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               int terms, hipStream_t st) {
-    CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows,
+               int terms, hipStream_t st, int rows_first, float* dW_rest) {
+    CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows &&
+                    (!dW_rest || (rows_first > 0 && rows_first < rows)),
                 "gemm_dw_x9: columns must be a multiple of 8");
     float* work = nullptr;
     size_t work_floats = 0;
@@ -367,8 +368,13 @@ int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpr
         hipLaunchKernelGGL(k_dw_x9<9>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
                            work, cols, ips, n_wg, groups);
     CFP_HIP_TRY(hipGetLastError());
+    // rows [0, rows_first) are added onto dW, the others (if any) onto dW_rest
     const long count = (long)rows * CFP_HIDDEN;
-    return launch_splitk_reduce(dW, work, count, count, splits, st);
+    const long first = dW_rest ? (long)rows_first * CFP_HIDDEN : count;
+    if (launch_splitk_reduce(dW, work, first, count, splits, st)) return 1;
+    if (first < count)
+        return launch_splitk_reduce(dW_rest, work + first, count - first, count, splits, st);
+    return 0;
 }
 
 }  // namespace cfp

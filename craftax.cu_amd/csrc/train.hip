@@ -61,13 +61,27 @@ __global__ void k_mingru_epi_replay_win(const float* __restrict__ pre,
 
 // PPO head gradients for one window column per thread; loss terms are reduced
 // per block in a fixed order and written to block_loss[3*blockIdx] (double).
+// The head's gradient rows are 48 floats wide: [43 dlogits | dvalue | 0 0 0 0], and the
+// head weights are mirrored as one [48][256] matrix [W_a ; W_v ; 0].  dh3 = rows . mirror
+// then carries the value head's share (the reference's k_add_dv_wv pass,
+// craftax_full.cu:10224), K = 48 suits the 16-wide MFMA steps, and one dW GEMM over 44
+// rows yields dW_a and dW_v together (cu_gemv_dwv, :11655, needs no pass of its own).
+constexpr int kHeadLd = 48;
+__global__ void k_head_mirror(const float* __restrict__ W_a, const float* __restrict__ W_v,
+                              float* __restrict__ out) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= kHeadLd * H) return;
+    const int r = idx / H, k = idx - r * H;
+    out[idx] = r < A ? W_a[idx] : (r == A ? W_v[k] : 0.0f);
+}
+
 __global__ __launch_bounds__(128) void k_head_bwd_win(
     const float* __restrict__ logits, const float* __restrict__ h3,
     const float* __restrict__ b_a, const float* __restrict__ W_v,
     const float* __restrict__ b_v, const int32_t* __restrict__ r_act,
     const float* __restrict__ r_logprob, const float* __restrict__ adv,
     const float* __restrict__ ret, const double* __restrict__ adv_stats,
-    float* __restrict__ dlogits, float* __restrict__ dvalue,
+    float* __restrict__ dlogits,
     double* __restrict__ block_loss, int t0, int cols, int mb, int n, int n_all,
     int T_all, float clip_eps, float vf_coef, const float* __restrict__ ent_coef_p,
     int logits_ld) {   // b_a == nullptr: rows of the fused forward, 43 logits + value, biases included
@@ -119,14 +133,17 @@ __global__ __launch_bounds__(128) void k_head_bwd_win(
             v = lp[A];   // the fused forward leaves the value (bias included) behind the logits
         }
         const float dret = v - ret[o];
-        dvalue[c] = inv_batch * vf_coef * dret;
-        float* dq = dlogits + (size_t)c * A;
+        // one 48-float row per column: 43 logit gradients, the value gradient, zeros
+        float* dq = dlogits + (size_t)c * kHeadLd;
 #pragma unroll
         for (int a = 0; a < A; a++) {
             float d = dlogp * ((a == act ? 1.0f : 0.0f) - pi[a]);
             d += ent_coef * pi[a] * ((lg[a] - lse) + Hent);
             dq[a] = d * inv_batch;
         }
+        dq[A] = inv_batch * vf_coef * dret;
+#pragma unroll
+        for (int a = A + 1; a < kHeadLd; a++) dq[a] = 0.0f;
         l_pg = (double)(-fminf(u1, u2));
         l_v = (double)(0.5f * dret * dret);
         l_e = (double)Hent;
@@ -163,14 +180,14 @@ __global__ __launch_bounds__(256) void k_loss_fold(const double* __restrict__ bl
     }
 }
 
-// out[r] += sum_c src[c*rows + r]: partial sums over `slices` column ranges
+// out[r] += sum_c src[c*ld + r]: partial sums over `slices` column ranges
 // (grid.x), then folded in slice order by k_colsum_fold.  A workgroup covers RB rows
 // with CL = 256 / RB threads each; a thread walks every CL-th column of the slice with
 // four independent running sums (loads in flight instead of one dependent chain) and
 // the CL sums of a row are added in thread order: a fixed order throughout.
 template <int RB>
 __global__ __launch_bounds__(256) void k_colsum_partial(
-    const float* __restrict__ src, float* __restrict__ part, int rows, int cols,
+    const float* __restrict__ src, int ld, float* __restrict__ part, int rows, int cols,
     int cols_per_slice) {
     constexpr int CL = 256 / RB;
     __shared__ float red[CL][RB];
@@ -183,12 +200,12 @@ __global__ __launch_bounds__(256) void k_colsum_partial(
         const float* p = src + r;
         int c = c0 + cl;
         for (; c + 3 * CL < c1; c += 4 * CL) {
-            s0 += p[(size_t)c * rows];
-            s1 += p[(size_t)(c + CL) * rows];
-            s2 += p[(size_t)(c + 2 * CL) * rows];
-            s3 += p[(size_t)(c + 3 * CL) * rows];
+            s0 += p[(size_t)c * ld];
+            s1 += p[(size_t)(c + CL) * ld];
+            s2 += p[(size_t)(c + 2 * CL) * ld];
+            s3 += p[(size_t)(c + 3 * CL) * ld];
         }
-        for (; c < c1; c += CL) s0 += p[(size_t)c * rows];
+        for (; c < c1; c += CL) s0 += p[(size_t)c * ld];
     }
     red[cl][rl] = (s0 + s1) + (s2 + s3);
     __syncthreads();
@@ -229,14 +246,12 @@ __global__ void k_mingru_window_bwd(
     const float* __restrict__ dhGEMM, const float* __restrict__ dhExtra,
     const float* __restrict__ r_state, const uint8_t* __restrict__ r_done,
     float* __restrict__ dhExtraOut, float* __restrict__ dcarry, int t0, int Tw,
-    int mb, int n, int env_start, int layer, int layers, int T_all, int seg_len,
-    const float* __restrict__ dv, const float* __restrict__ W_v) {
+    int mb, int n, int env_start, int layer, int layers, int T_all, int seg_len) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)H * mb) return;
     const int k = (int)(idx & (H - 1));
     const size_t el = idx / H;
     float dc = dcarry[idx];
-    const float wv_k = dv ? W_v[k] : 0.0f;
     for (int tr = Tw - 1; tr >= 0; tr--) {
         const int t = t0 + tr;
         if (t == T_all - 1 || ((t + 1) % seg_len) == 0) dc = 0.0f;
@@ -245,7 +260,6 @@ __global__ void k_mingru_window_bwd(
         const size_t o3 = w * G + k;
         const float zh = pre[o3], zg = pre[o3 + H], zp = pre[o3 + 2 * H];
         float dhout = dhGEMM[o];
-        if (dv) dhout += dv[w] * wv_k;   // top layer: the value head's share (k_add_dv_wv)
         if (dhExtra) dhout += dhExtra[o];
         const size_t rs = (((size_t)t * layers + layer) * (size_t)n + env_start + el) * H + k;
         const float s_in = r_state[rs];
@@ -416,7 +430,7 @@ struct cfp_trainer {
     float *d_lr = nullptr, *d_ent = nullptr;
     // window workspace
     float* xobs = nullptr; float* x[CFP_MAX_LAYERS + 1] = {}; float* preb[CFP_MAX_LAYERS] = {};
-    float *logitsb = nullptr, *dlogits = nullptr, *dvalue = nullptr;
+    float *logitsb = nullptr, *dlogits = nullptr, *w_head = nullptr;
     float *dh3b = nullptr, *dhG = nullptr, *dhX = nullptr;
     float* dcarry[CFP_MAX_LAYERS] = {};
     float* colsum_part = nullptr;
@@ -506,8 +520,8 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     for (int l = 0; l < tr->L; l++) TA(preb[l], cc * G * sizeof(float));
     for (int l = 0; l < tr->L; l++) TA(dcarry[l], (size_t)mb * H * sizeof(float));
     TA(logitsb, cc * (A + 1) * sizeof(float));   // [cols][44] from the fused recompute, [cols][43] unfused
-    TA(dlogits, cc * A * sizeof(float));
-    TA(dvalue, cc * sizeof(float));
+    TA(dlogits, cc * kHeadLd * sizeof(float));
+    TA(w_head, (size_t)kHeadLd * H * sizeof(float));
     TA(dh3b, cc * H * sizeof(float));
     TA(dhG, cc * H * sizeof(float));
     TA(dhX, cc * H * sizeof(float));
@@ -634,18 +648,18 @@ int cfp_train_adv_stats(cfp_trainer* tr, void* stream) {
     return 0;
 }
 
-static int colsum_into(cfp_trainer* tr, const float* src, float* out, int rows, int cols,
-                       hipStream_t st) {
+static int colsum_into(cfp_trainer* tr, const float* src, int ld, float* out, int rows,
+                       int cols, hipStream_t st) {
     int slices = kColsumSlices;
     if (slices > cols) slices = cols;
     const int per = (cols + slices - 1) / slices;
     slices = (cols + per - 1) / per;
     if (rows <= 64)
-        hipLaunchKernelGGL(k_colsum_partial<64>, dim3(slices, 1), dim3(256), 0, st, src,
+        hipLaunchKernelGGL(k_colsum_partial<64>, dim3(slices, 1), dim3(256), 0, st, src, ld,
                            tr->colsum_part, rows, cols, per);
     else
         hipLaunchKernelGGL(k_colsum_partial<256>, dim3(slices, (rows + 255) / 256), dim3(256), 0,
-                           st, src, tr->colsum_part, rows, cols, per);
+                           st, src, ld, tr->colsum_part, rows, cols, per);
     hipLaunchKernelGGL(k_colsum_fold, dim3((rows + 3) / 4), dim3(256), 0, st,
                        tr->colsum_part, out, rows, slices);
     CFP_HIP_TRY(hipGetLastError());
@@ -674,6 +688,9 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
     for (int l = 0; l < L; l++)
         hipLaunchKernelGGL(k_fill, dim3(grid1((size_t)H * mb)), dim3(256), 0, st,
                            tr->dcarry[l], (size_t)H * mb, 0.0f);
+
+    hipLaunchKernelGGL(k_head_mirror, dim3((kHeadLd * H + 255) / 256), dim3(256), 0, st, W_a, W_v,
+                       tr->w_head);
 
     for (int t_end = T; t_end > 0; t_end -= tr->win) {
         const int t0 = t_end - tr->win > 0 ? t_end - tr->win : 0;
@@ -726,17 +743,17 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         hipLaunchKernelGGL(k_head_bwd_win, dim3(hb), dim3(128), 0, st, tr->logitsb, tr->x[L],
                            fused ? nullptr : b_a, W_v, b_v, tr->r_act + env_start, tr->r_logprob + env_start,
                            tr->adv + env_start, tr->ret + env_start, tr->stats, tr->dlogits,
-                           tr->dvalue, tr->block_loss, t0, cols, mb, n, n, T, tr->cfg.clip,
+                           tr->block_loss, t0, cols, mb, n, n, T, tr->cfg.clip,
                            tr->cfg.vf, tr->d_ent, fused ? A + 1 : A);
         hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(256), 0, st, tr->block_loss, hb,
                            tr->loss_acc);
-        // dh3 = W_a^T dlogits here; the value head's dv * W_v is added where the top
-        // layer's reverse kernel reads dh3 (the reference's k_add_dv_wv pass, :10224)
-        if (cfp_gemm_dh(A, cols, W_a, tr->dlogits, tr->dh3b, stream)) return 1;
-        if (cfp_gemm_dw(A, cols, tr->x[L], tr->dlogits, g + CFP_OFF_W_A(L), stream)) return 1;
-        if (cfp_gemv_dwv(tr->x[L], tr->dvalue, g + CFP_OFF_W_V(L), cols, stream)) return 1;
-        if (colsum_into(tr, tr->dlogits, g + CFP_OFF_B_A(L), A, cols, st)) return 1;
-        if (colsum_into(tr, tr->dvalue, g + CFP_OFF_B_V(L), 1, cols, st)) return 1;
+        // dh3 = [dlogits | dvalue] . [W_a ; W_v]; dW_a and dW_v from one GEMM; bias sums
+        if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, st)) return 1;
+        if (gemm_dw_two(A, 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L),
+                        g + CFP_OFF_W_V(L), st))
+            return 1;
+        if (colsum_into(tr, tr->dlogits, kHeadLd, g + CFP_OFF_B_A(L), A, cols, st)) return 1;
+        if (colsum_into(tr, tr->dlogits + A, kHeadLd, g + CFP_OFF_B_V(L), 1, cols, st)) return 1;
         // ---- reverse MinGRU layers
         const float* dh_gemm = tr->dh3b;
         const float* dh_extra = nullptr;
@@ -744,7 +761,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             hipLaunchKernelGGL(k_mingru_window_bwd, dim3(grid1((size_t)H * mb)), dim3(256),
                                0, st, tr->preb[l], tr->x[l], dh_gemm, dh_extra, tr->r_state,
                                tr->r_done, tr->dhX, tr->dcarry[l], t0, Tw, mb, n, env_start,
-                               l, L, T, seg, l == L - 1 ? tr->dvalue : nullptr, W_v);
+                               l, L, T, seg);
             if (cfp_gemm_dw(G, cols, tr->x[l], tr->preb[l],
                             g + CFP_OFF_W_GRU + (size_t)l * G * H, stream))
                 return 1;
@@ -756,7 +773,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             dh_extra = tr->dhX;
         }
         // ---- encoder: db_enc; dW_enc += xobs^T dh_enc (dh_enc sits in dhX)
-        if (colsum_into(tr, tr->dhX, g + CFP_OFF_B_ENC, H, cols, st)) return 1;
+        if (colsum_into(tr, tr->dhX, H, g + CFP_OFF_B_ENC, H, cols, st)) return 1;
         if (dw_enc_records_ok(mb)) {
             // map bytes straight from the records; xobs is free by now and takes the
             // 76-float rows of the fp32 remainder
