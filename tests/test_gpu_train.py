@@ -311,9 +311,13 @@ def test_backward_with_bf16_gemms(pkg, cuda):
     tr.buf("r_logprob").copy_(_t(host["r_logprob"], cuda))
     batch, keep = ob.make_batch(T, n, 0, n, L, T, **host)
     g_ref, l3_ref = ob.ppo_backward_f64(params, batch)
+    # (bf16 inputs, split mode): fp32 on the split kernels with nine / six partial products
+    # and on the fp32 MFMA kernel; bf16 inputs on the split kernels with the fused bf16
+    # window recompute, and on the generic bf16 kernel with the unfused chain
     grads = {}
-    for mode in (False, True):
-        pkg.policy.set_gemm_bf16(mode)
+    for mode in ((False, 1), (False, 2), (False, 0), (True, 1), (True, 0)):
+        pkg.policy.set_gemm_bf16(mode[0])
+        pkg.policy.set_gemm_split(mode[1])
         try:
             tr.buf("grads").zero_()
             tr.zero_loss()
@@ -321,16 +325,21 @@ def test_backward_with_bf16_gemms(pkg, cuda):
             torch.cuda.synchronize()
         finally:
             pkg.policy.set_gemm_bf16(False)
+            pkg.policy.set_gemm_split(1)
         grads[mode] = tr.buf("grads").cpu().numpy().copy()
         l3 = tr.buf("loss_acc").cpu().numpy()
         # the pg sum nearly cancels (ratios ~ 1, zero-mean advantages): absolute floor
-        tol = 1e-2 if mode else 1e-4
+        tol = 1e-2 if mode[0] else 1e-4
         assert np.allclose(l3, l3_ref, rtol=tol, atol=tol * np.abs(l3_ref).max()), (mode, l3, l3_ref)
-    worst = 0.0
     for name, sl in _segments(L):
-        assert_close(grads[False][sl], g_ref[sl], TOL_FP32, f"fp32 d{name} (same batch)")
-        e = fro_err(grads[True][sl], g_ref[sl])
-        assert e <= TOL_BF16, f"bf16 d{name}: relative Frobenius error {e:.3e}"
-        worst = max(worst, e)
-    assert worst > 1e-4, "the bf16 GEMMs did not run"
+        for split in (1, 2, 0):
+            assert_close(grads[(False, split)][sl], g_ref[sl], TOL_FP32,
+                         f"fp32 d{name}, split mode {split} (same batch)")
+    for split in (1, 0):
+        worst = 0.0
+        for name, sl in _segments(L):
+            e = fro_err(grads[(True, split)][sl], g_ref[sl])
+            assert e <= TOL_BF16, f"bf16 d{name}, split mode {split}: relative Frobenius error {e:.3e}"
+            worst = max(worst, e)
+        assert worst > 1e-4, "the bf16 GEMMs did not run"
     tr.close(); pol.close()
