@@ -157,6 +157,12 @@ bool gemm_dh_x9_ok(int m3, int cols, const float* dpre);
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
                int terms, hipStream_t st);
 
+// y[cols][m] = x[cols][k] . W[m][k]^T on the same kernel (m % 256 == 0, k % 16 == 0,
+// cols % 32 == 0, x 16-byte aligned)
+bool gemm_fwd_x9_ok(int m, int cols, int k, const float* x);
+int gemm_fwd_x9(int m, int cols, int k, const float* W, const float* x, float* y, int terms,
+                hipStream_t st);
+
 // per-variant arena geometry
 struct Arena {
     int obs, actions;

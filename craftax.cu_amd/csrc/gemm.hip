@@ -537,6 +537,8 @@ int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
                  float* d_y, void* stream) {
     CFP_REQUIRE(m > 0 && cols > 0 && k > 0 && d_W && d_x && d_y,
                 "cfp_gemm_fwd: bad argument");
+    if (g_gemm_split && gemm_fwd_x9_ok(m, cols, k, d_x))
+        return gemm_fwd_x9(m, cols, k, d_W, d_x, d_y, split_terms(), (hipStream_t)stream);
     GemmArgs g{};
     g.A = d_x; g.sa_i = k; g.sa_k = 1;
     g.B = d_W; g.sb_k = 1; g.sb_j = k;

@@ -177,7 +177,8 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
         }
 }
 
-// k_dh_x9: dh[c][u] (+)= sum_k dpre[c][k] * W[k][u] for 256 units, K = m3 (multiple of 16).
+// k_dh_x9: dh[c][u] (+)= sum_k dpre[c][k] * W[k][u] for 256 units, K = m3 (multiple of 16);
+// also the gate-forward shape y = x . W^T, 256 output rows at a time (gemm_fwd_x9).
 //   workgroup : 256 columns; wave w owns columns 32w..32w+31 of them and all 256 units
 //               (8 accumulators).  Its dpre fragment of a K step is 32 contiguous
 //               bytes per lane, split in registers one step ahead.
@@ -191,15 +192,15 @@ constexpr int kDhThreads = 512;
 constexpr int kDhTileCols = 256;
 constexpr int kDhFrags = 24;   // 8 unit tiles x 3 parts per K step
 
-__global__ void k_pack_w_x9(const float* __restrict__ W, u4* __restrict__ out, int total,
-                            int rounded) {
+__global__ void k_pack_w_x9(const float* __restrict__ W, long sk, long su,
+                            u4* __restrict__ out, int total, int rounded) {   // W(k, u) = W[k*sk + u*su]
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int lane = idx & 63, f = (idx >> 6) % kDhFrags, s = idx / (64 * kDhFrags);
     const int t = f / 3, part = f - 3 * t, n = lane & 31, g = lane >> 5;
     float v[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) v[j] = W[(size_t)(16 * s + 8 * g + j) * CFP_HIDDEN + 32 * t + n];
+    for (int j = 0; j < 8; j++) v[j] = W[(long)(16 * s + 8 * g + j) * sk + (long)(32 * t + n) * su];
     u4 h, m, l;
     split3(v, h, m, l);
     if (rounded) h = round_bf16x8(v);   // bf16-input mode: part 0 is the rounded operand
@@ -209,7 +210,7 @@ __global__ void k_pack_w_x9(const float* __restrict__ W, u4* __restrict__ out, i
 template <int TERMS>
 __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ dpre, int m3,
                                                       const u4* __restrict__ wm,
-                                                      float* __restrict__ dh, int cols,
+                                                      float* __restrict__ dh, int ldc, int cols,
                                                       int accumulate) {
     __shared__ u4 stage[2][kDhFrags][64];   // 48 KiB
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
@@ -242,13 +243,13 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
 
     // accumulating form: the accumulators start from dh, all 128 loads in flight at
     // once under the prologue's own loads, and the epilogue is stores only
-    float* o_lane = dh + (size_t)(cbc + 4 * g) * CFP_HIDDEN + n;
+    float* o_lane = dh + (size_t)(cbc + 4 * g) * ldc + n;
     f16v acc[8];
 #pragma unroll
     for (int t = 0; t < 8; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++)
-            acc[t][r] = accumulate ? o_lane[(size_t)acc_row(r) * CFP_HIDDEN + 32 * t] : 0.0f;
+            acc[t][r] = accumulate ? o_lane[(size_t)acc_row(r) * ldc + 32 * t] : 0.0f;
 
     float raw[2][8];
     u4 wb[3];
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     for (int t = 0; t < 8; t++)
 #pragma unroll
         for (int r = 0; r < 16; r++)
-            o_lane[(size_t)acc_row(r) * CFP_HIDDEN + 32 * t] = acc[t][r];
+            o_lane[(size_t)acc_row(r) * ldc + 32 * t] = acc[t][r];
 }
 
 u4* g_w_x9 = nullptr;   // W mirror of the call in flight: one stream at a time
@@ -312,26 +313,46 @@ bool gemm_dh_x9_ok(int m3, int cols, const float* dpre) {
            (reinterpret_cast<uintptr_t>(dpre) & 15u) == 0;
 }
 
+// out[cols][ldc] (+)= A[cols][K] . B, B(k, u) = B[k*sk + u*su] for 256 units
+static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const float* A,
+                        float* out, int ldc, bool accumulate, int terms, hipStream_t st) {
+    if (!g_w_x9)
+        CFP_HIP_TRY(hipMalloc((void**)&g_w_x9, (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4)));
+    const int total = (K / 16) * kDhFrags * 64;
+    hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, B, sk, su, g_w_x9,
+                       total, terms == 1 ? 1 : 0);
+    const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
+    const int acc = accumulate ? 1 : 0;
+    if (terms == 1)
+        hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+    else if (terms == 6)
+        hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+    else
+        hipLaunchKernelGGL(k_dh_x9<9>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
                int terms, hipStream_t st) {
     CFP_REQUIRE(gemm_dh_x9_ok(m3, cols, dpre) && W && dh,
                 "gemm_dh_x9: K must be a multiple of 16 up to %d and columns of 32", kDhMaxK);
-    if (!g_w_x9)
-        CFP_HIP_TRY(hipMalloc((void**)&g_w_x9, (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4)));
-    const int total = (m3 / 16) * kDhFrags * 64;
-    hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, W, g_w_x9, total,
-                       terms == 1 ? 1 : 0);
-    const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
-    if (terms == 1)
-        hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, dpre, m3, g_w_x9, dh, cols,
-                           accumulate ? 1 : 0);
-    else if (terms == 6)
-        hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, dpre, m3, g_w_x9, dh, cols,
-                           accumulate ? 1 : 0);
-    else
-        hipLaunchKernelGGL(k_dh_x9<9>, grid, dim3(kDhThreads), 0, st, dpre, m3, g_w_x9, dh, cols,
-                           accumulate ? 1 : 0);
-    CFP_HIP_TRY(hipGetLastError());
+    return launch_dh_x9(m3, cols, W, CFP_HIDDEN, 1, dpre, dh, CFP_HIDDEN, accumulate, terms, st);
+}
+
+// y[cols][m] = x[cols][k] . W[m][k]^T in slices of 256 output rows of W
+bool gemm_fwd_x9_ok(int m, int cols, int k, const float* x) {
+    return m >= CFP_HIDDEN && m % CFP_HIDDEN == 0 && gemm_dh_x9_ok(k, cols, x);
+}
+
+int gemm_fwd_x9(int m, int cols, int k, const float* W, const float* x, float* y, int terms,
+                hipStream_t st) {
+    CFP_REQUIRE(gemm_fwd_x9_ok(m, cols, k, x) && W && y,
+                "gemm_fwd_x9: m must be a multiple of 256, k of 16 up to %d, columns of 32", kDhMaxK);
+    for (int j = 0; j < m / CFP_HIDDEN; j++)
+        if (launch_dh_x9(k, cols, W + (size_t)j * CFP_HIDDEN * k, 1, k, x, y + j * CFP_HIDDEN, m,
+                         false, terms, st))
+            return 1;
     return 0;
 }
 

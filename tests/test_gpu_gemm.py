@@ -114,6 +114,23 @@ def test_gemm_dh_split_is_as_accurate_as_fp32_mfma(pkg, cuda, m3, cols):
     _check_split_errors(errs)
 
 
+@pytest.mark.parametrize("m,cols,k", [(768, 8192, 256), (256, 64, 32), (768, 32000, 256)])
+def test_gemm_fwd_split_is_as_accurate_as_fp32_mfma(pkg, cuda, m, cols, k):
+    """The gate-forward shape y = x . W^T on the dh kernel, 256 rows of W at a time."""
+    import torch
+    W, x = _r((m, k), cuda, 26, 0.1), _r((cols, k), cuda, 27)
+    want = x.double() @ W.double().T
+    scale = x.double().abs() @ W.double().abs().T
+    errs = {}
+    for mode in (1, 2, 0):
+        pkg.policy.set_gemm_split(mode)
+        out = pkg.policy.gemm_fwd(W, x)
+        torch.cuda.synchronize()
+        errs[mode] = ((out.double() - want).abs() / scale).max().item()
+    pkg.policy.set_gemm_split(1)
+    _check_split_errors(errs)
+
+
 def test_gemv_dwv(pkg, cuda):
     import torch
     x, dv = _r((5000, HIDDEN), cuda, 9), _r((5000,), cuda, 10)
