@@ -258,12 +258,14 @@ __global__ void k_mingru_window_bwd(
         const size_t w = (size_t)tr * mb + el;
         const size_t o = w * H + k;
         const size_t o3 = w * G + k;
-        const float zh = pre[o3], zg = pre[o3 + H], zp = pre[o3 + 2 * H];
-        float dhout = dhGEMM[o];
-        if (dhExtra) dhout += dhExtra[o];
+        const float zh = __builtin_nontemporal_load(pre + o3);
+        const float zg = __builtin_nontemporal_load(pre + o3 + H);
+        const float zp = __builtin_nontemporal_load(pre + o3 + 2 * H);
+        float dhout = __builtin_nontemporal_load(dhGEMM + o);
+        if (dhExtra) dhout += __builtin_nontemporal_load(dhExtra + o);
         const size_t rs = (((size_t)t * layers + layer) * (size_t)n + env_start + el) * H + k;
-        const float s_in = r_state[rs];
-        const float xv = x[o];
+        const float s_in = __builtin_nontemporal_load(r_state + rs);
+        const float xv = __builtin_nontemporal_load(x + o);
         const bool done_t = r_done[(size_t)t * n + env_start + el] != 0;
         const float sg = sigm(zg);
         const float gh = gfun(zh);
