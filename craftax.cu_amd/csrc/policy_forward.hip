@@ -472,7 +472,11 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
 
 }  // namespace
 
-template <int VARIANT, int MODE>
+// SINGLE: one tile per workgroup instead of a pair, for batches of at most one tile per
+// CU (a rollout of a few thousand envs): twice as many CUs work, and a layer is its K
+// phase followed by its epilogue instead of the two tiles' interleave.  Encoder and
+// heads still run their two-tile code with an all-zero second tile.
+template <int VARIANT, int MODE, bool SINGLE>
 __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds_all[2][LDS_FLOATS];
     __shared__ __attribute__((aligned(16))) float red_all[2][kRedFloats];
@@ -487,7 +491,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     uint8_t* const crec_all[2] = {cbase, cbase + kClsOffRecY};
 
     const int tiles = a.n / kTileEnvs;
-    const int pairs = (tiles + 1) / 2;
+    constexpr int TS = SINGLE ? 1 : 2;   // tiles per unit of work ("pair")
+    const int pairs = (tiles + TS - 1) / TS;
     const bool classic = VARIANT == 1 && a.rec;
     const bool full_rec = VARIANT == 0 && a.rec;
 
@@ -510,8 +515,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     };
     if (full_rec && (int)blockIdx.x < pairs) {
         const int tid0 = threadIdx.x;
-        rec_fetch(rec_of(2 * blockIdx.x), term_of(2 * blockIdx.x), pre[0], tid0);
-        if (2 * (int)blockIdx.x + 1 < tiles)
+        rec_fetch(rec_of(TS * blockIdx.x), term_of(TS * blockIdx.x), pre[0], tid0);
+        if (!SINGLE && 2 * (int)blockIdx.x + 1 < tiles)
             rec_fetch(rec_of(2 * blockIdx.x + 1), term_of(2 * blockIdx.x + 1), pre[1], tid0);
     }
     for (int pair = blockIdx.x; pair < pairs; pair += gridDim.x) {
@@ -531,8 +536,8 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
         const int nt = L.wave & 1;   // head: row tile
         const int kh = L.wave >> 1;  // head: K half
         // tile X = 2*pair always exists; tile Y may be past the end (odd tile count)
-        const bool hasY = 2 * pair + 1 < tiles;
-        size_t e0[2] = {(size_t)(2 * pair) * kTileEnvs, (size_t)(2 * pair + 1) * kTileEnvs};
+        const bool hasY = !SINGLE && 2 * pair + 1 < tiles;
+        size_t e0[2] = {(size_t)(TS * pair) * kTileEnvs, (size_t)(TS * pair + 1) * kTileEnvs};
 
         // ---- stage both tiles (a missing Y is a zero tile that is computed but
         // never read from or written to the caller's buffers) --------------------
@@ -590,8 +595,9 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
         auto fetch_next = [&]() {
             const int np = pair + (int)gridDim.x;
             if (np < pairs) {
-                rec_fetch(rec_of(2 * np), term_of(2 * np), pre[0], tid);
-                if (2 * np + 1 < tiles) rec_fetch(rec_of(2 * np + 1), term_of(2 * np + 1), pre[1], tid);
+                rec_fetch(rec_of(TS * np), term_of(TS * np), pre[0], tid);
+                if (!SINGLE && 2 * np + 1 < tiles)
+                    rec_fetch(rec_of(2 * np + 1), term_of(2 * np + 1), pre[1], tid);
             }
         };
         if (full_rec && a.layers == 0) fetch_next();
@@ -634,6 +640,26 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
                 return c;
             };
             const int Q = 2 * a.layers;
+            if (SINGLE) {
+                // one tile: K phase, then its epilogue, layer by layer.  The state is
+                // requested before the weights, so it has landed when block 0 has.
+                if (full_rec) fetch_next();
+#pragma unroll 1
+                for (int l = 0; l < a.layers; l++) {
+                    const StateIO io1 = state_io(2 * l + 1);
+                    state_load(io1, st, L);
+                    ring_preload(bq, wp0 + (size_t)l * wl, L);
+#pragma unroll
+                    for (int t = 0; t < 6; t++) accO[t] = zero16();
+                    gru_phase<true, false, MODE>(accO, accO, bq,
+                                                 reinterpret_cast<const f4*>(lds_all[0]),
+                                                 wp0 + (size_t)l * wl, nullptr, io1, st, L);
+                    __syncthreads();   // every wave has read the layer input
+                    gru_phase<false, true, MODE>(accN, accO, bq, nullptr, nullptr, lds_all[0], io1,
+                                                 st, L);
+                    __syncthreads();
+                }
+            } else {
 #pragma unroll
             for (int t = 0; t < 6; t++) accO[t] = zero16();
             ring_preload(bq, wp0, L);
@@ -662,6 +688,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             gru_phase<false, true, MODE>(accN, accO, bq, nullptr, nullptr, lds_all[(Q - 1) & 1],
                                            io, st, L);
             __syncthreads();
+            }
             if (a.h3_out) {
                 copy_tile_out(lds_all[0], a.h3_out + e0[0] * CFP_HIDDEN, tid);
                 if (hasY) copy_tile_out(lds_all[1], a.h3_out + e0[1] * CFP_HIDDEN, tid);
@@ -758,21 +785,28 @@ int launch_forward(const FwdArgs& a, hipStream_t st) {
     CFP_REQUIRE(!a.do_head || a.av_out != nullptr,
                 "head requested without an output buffer");
     if (a.bf16) return launch_forward_bf16(a, st);
-    // persistent: one workgroup per CU, each walking tile pairs round-robin
-    const int pairs = (a.n / kTileEnvs + 1) / 2;
+    // persistent: one workgroup per CU, each walking tile pairs round-robin; a full-game
+    // batch of at most one tile per CU runs one tile per workgroup instead
+    const int tiles = a.n / kTileEnvs;
+    const int pairs = (tiles + 1) / 2;
     const int grid = pairs < num_cus() ? pairs : num_cus();
     const dim3 g(grid), b(kFwdThreads);
+    const bool single = a.variant == 0 && !a.train && tiles <= num_cus() && tiles > 1;
     if (a.train) {
         CFP_REQUIRE(a.variant == 0 && a.rec && a.state && a.layers > 0 && !a.r_state &&
                         a.tr_mb > 0 && a.tr_mb % kTileEnvs == 0 && a.h_enc_out == a.tr_x[0],
                     "window recompute: bad arguments");
-        hipLaunchKernelGGL((k_policy_forward<0, kModeTrain>), g, b, 0, st, a);
+        hipLaunchKernelGGL((k_policy_forward<0, kModeTrain, false>), g, b, 0, st, a);
     } else if (a.variant == 1) {
-        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<1, kModeRecord>), g, b, 0, st, a);
-        else hipLaunchKernelGGL((k_policy_forward<1, kModePlain>), g, b, 0, st, a);
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<1, kModeRecord, false>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward<1, kModePlain, false>), g, b, 0, st, a);
+    } else if (single) {
+        const dim3 g1(tiles);
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<0, kModeRecord, true>), g1, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward<0, kModePlain, true>), g1, b, 0, st, a);
     } else {
-        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<0, kModeRecord>), g, b, 0, st, a);
-        else hipLaunchKernelGGL((k_policy_forward<0, kModePlain>), g, b, 0, st, a);
+        if (a.r_state) hipLaunchKernelGGL((k_policy_forward<0, kModeRecord, false>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward<0, kModePlain, false>), g, b, 0, st, a);
     }
     CFP_HIP_TRY(hipGetLastError());
     return 0;
