@@ -144,6 +144,31 @@ def test_chunked_equals_unchunked(pkg, cuda):
     pol.close()
 
 
+def test_one_tile_per_workgroup_schedule_matches_pairs(pkg, cuda):
+    """Batches of at most one tile per CU run one tile per workgroup (a layer's K
+    phase, then its epilogue) instead of the two-tile interleave; the arithmetic per
+    tile is the same, so the bits are.  16 384 envs in one launch take the pair
+    schedule, the same envs in chunks of 4096 the single one; plain and recording."""
+    import torch
+    n = 16384
+    pol = pkg.Policy(n, L, seed=4)
+    rec = pkg.policy.synth_records(n, 31, 2)
+    term = (torch.rand(n, device=cuda) < 0.1).float()
+    st0 = torch.randn(L, n, HIDDEN, device=cuda) * 0.5
+    for record in (False, True):
+        outs = []
+        for chunk in (0, 4096):
+            st = st0.clone()
+            rs = torch.full_like(st0, 7.0) if record else None
+            av = pol.forward(rec, term, st, r_state_t=rs, chunk=chunk).clone()
+            torch.cuda.synchronize()
+            outs.append((av, st, rs))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        if record:
+            assert torch.equal(outs[0][2], outs[1][2])
+    pol.close()
+
+
 def test_multi_step_carry_with_terminals(pkg, cuda):
     """16 consecutive steps carrying hidden state on device vs the oracle carrying
     it in fp64; state zeroed on the step after a terminal."""
