@@ -239,60 +239,14 @@ __device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const 
 // byte of that, and a 256-entry LDS table turns the byte into eight bf16 0/1.
 // The 22 scalar features (inventory and intrinsics / 10, direction one-hot, light,
 // sleeping) follow on the fp32 MFMA (3 K blocks of 8).  Block ids must be 0..16.
-constexpr int kClsCells = 63, kClsCh = 21;
-constexpr int kClsBits = kClsCells * kClsCh;                 // 1323
-constexpr int kClsKb16 = (kClsBits + 15) / 16;               // 83
-constexpr int kClsBitRow = 44;                               // dwords per env (42 used)
-constexpr int kClsSv = 24;                                   // scalar features per env, padded
-constexpr int kClsTailKb = kClsSv / 8;                       // 3 fp32 K blocks
 constexpr int kClsEnvs = 2 * kTileEnvs;
 // byte layout inside the (not yet used) x tiles
 constexpr int kClsOffRecY = kTileEnvs * CFP_CLASSIC_REC_BYTES;
-constexpr int kClsOffBits = 2 * kClsOffRecY;
-constexpr int kClsOffLut = kClsOffBits + kClsEnvs * kClsBitRow * 4;
-constexpr int kClsOffSv = kClsOffLut + 256 * 16;
-static_assert(kClsOffSv + kClsEnvs * kClsSv * 4 <= 2 * LDS_FLOATS * 4, "classic tables fit the x tiles");
-static_assert(kClsOffBits % 16 == 0 && kClsOffLut % 16 == 0 && kClsOffSv % 16 == 0, "alignment");
-
-// Bit rows, byte -> 8 x bf16 table and scalar rows from the two tiles' records
-// (all 256 threads; ends with a barrier).
-__device__ __forceinline__ void classic_prepare(uint8_t* base, int tid) {
-    uint32_t* bits = reinterpret_cast<uint32_t*>(base + kClsOffBits);
-    u4* lut = reinterpret_cast<u4*>(base + kClsOffLut);
-    float* sv = reinterpret_cast<float*>(base + kClsOffSv);
-    for (int i = tid; i < kClsEnvs * kClsBitRow; i += kFwdThreads) bits[i] = 0u;
-    {
-        u4 v;
-        uint32_t d[4];
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-            d[i] = (((unsigned)tid >> (2 * i)) & 1u) * 0x3F80u |
-                   (((unsigned)tid >> (2 * i + 1)) & 1u) * 0x3F800000u;
-        v.x = d[0]; v.y = d[1]; v.z = d[2]; v.w = d[3];
-        lut[tid] = v;
-    }
-    for (int i = tid; i < kClsEnvs * kClsSv; i += kFwdThreads) {
-        const int e = i / kClsSv, f = i - e * kClsSv;
-        const uint8_t* o = base + e * CFP_CLASSIC_REC_BYTES + 2 * kClsCells;
-        float v = 0.0f;
-        if (f < 16) v = (float)(int8_t)o[f] / 10.0f;                  // inventory, intrinsics
-        else if (f < 20) v = (int8_t)o[16] == f - 15 ? 1.0f : 0.0f;   // direction 1..4
-        else if (f == 20) v = *reinterpret_cast<const float*>(o + 18);   // light
-        else if (f == 21) v = o[17] ? 1.0f : 0.0f;                    // sleeping
-        sv[i] = v;
-    }
-    __syncthreads();   // rows are zero before the bits go in
-    for (int i = tid; i < kClsEnvs * kClsCells; i += kFwdThreads) {
-        const int e = i / kClsCells, cell = i - e * kClsCells;
-        const uint8_t* o = base + e * CFP_CLASSIC_REC_BYTES;
-        const uint32_t v = (1u << (o[cell] & 31u)) & 0x1FFFFu | ((o[kClsCells + cell] & 15u) << 17);
-        const int bit = kClsCh * cell, dw = bit >> 5, sh = bit & 31;
-        uint32_t* row = bits + e * kClsBitRow;
-        atomicOr(row + dw, v << sh);
-        if (sh > 32 - kClsCh) atomicOr(row + dw + 1, v >> (32 - sh));
-    }
-    __syncthreads();
-}
+constexpr int kClsOffBits = ClsLayout<kClsEnvs>::offBits;
+constexpr int kClsOffLut = ClsLayout<kClsEnvs>::offLut;
+constexpr int kClsOffSv = ClsLayout<kClsEnvs>::offSv;
+static_assert(kClsOffBits == 2 * kClsOffRecY, "the pair's records lie back to back");
+static_assert(ClsLayout<kClsEnvs>::end <= 2 * LDS_FLOATS * 4, "classic tables fit the x tiles");
 
 __device__ __forceinline__ void classic_encoder_gemm(const FwdArgs& a, const uint8_t* base,
                                                      f4* ring, const Lane& L, f16v (&acc)[4]) {
@@ -568,7 +522,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             for (int t = 0; t < 4; t++) eacc[t] = zero16();
             f4* const ring = aux + L.wave * (kRingSlots * kRingSlotF4);
             if (classic) {
-                classic_prepare(cbase, tid);
+                classic_prepare<kClsEnvs>(cbase, tid);
                 classic_encoder_gemm(a, cbase, ring, L, eacc);
             } else {
                 encoder_gemm_split_ring(a, lds_all[0], lds_all[1], ring, L, eacc);

@@ -57,7 +57,10 @@ template <int VARIANT, bool HAS_RS, bool TRAIN>
 __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     __shared__ float term_s[kTileEnvs];
-    __shared__ __attribute__((aligned(16))) uint8_t crec[VARIANT == 1 ? kTileEnvs * CFP_CLASSIC_REC_BYTES : 16];
+    // classic game: the records and the encoder's tables sit in the x tile until the
+    // encoder's result replaces them
+    static_assert(ClsLayout<kTileEnvs>::end <= LDS_FLOATS * 4, "classic tables fit the x tile");
+    uint8_t* const crec = reinterpret_cast<uint8_t*>(lds);
 
     const int tid = threadIdx.x;
     const unsigned lane_u = (unsigned)(tid & 63);
@@ -85,7 +88,59 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
 
     // ---- encoder ---------------------------------------------------------------
     if (VARIANT == 1 && a.rec) {
-        classic_encode_tile(a, crec, lds, tid);
+        // encode_obs_kernel (craftax_classic.cu:1714-1751).  Cell features: bits -> bf16
+        // 0/1 through the table, against the hi and mid parts of the three-term split
+        // of W_enc (16 significant bits of every weight: at least what rounding the
+        // weight to bf16 keeps); the 22 scalar features on the fp32 MFMA.
+        using LY = ClsLayout<kTileEnvs>;
+        classic_prepare<kTileEnvs>(crec, tid);
+        f16v acc[2] = {zero16(), zero16()};
+        const uint8_t* brow = crec + LY::offBits + l32 * (kClsBitRow * 4) + g;
+        const u4* lut = reinterpret_cast<const u4*>(crec + LY::offLut);
+        const u4* wp = a.we_s3 + (size_t)(wave * 6) * 64;
+        constexpr int KB_STRIDE = 4 * 6 * 64;   // u4 per K block: [wave][unit tile][part][lane]
+        u4 b[2][4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) b[0][i] = (wp + ((i >> 1) * 3 + (i & 1)) * 64)[lane_u];
+        u4 av = lut[brow[0]];
+#pragma unroll 2
+        for (int kb = 0; kb < kClsKb16; kb++) {
+            const int cb = kb & 1, nb = cb ^ 1;
+            u4 an = av;
+            if (kb + 1 < kClsKb16) {
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    b[nb][i] = (wp + (size_t)(kb + 1) * KB_STRIDE + ((i >> 1) * 3 + (i & 1)) * 64)[lane_u];
+                an = lut[brow[2 * (kb + 1)]];
+            }
+            acc[0] = mfma16(av, b[cb][0], acc[0]);
+            acc[1] = mfma16(av, b[cb][2], acc[1]);
+            acc[0] = mfma16(av, b[cb][1], acc[0]);
+            acc[1] = mfma16(av, b[cb][3], acc[1]);
+            av = an;
+        }
+        const f4* wq = a.we_pk + (size_t)(wave * 2) * 64;
+        constexpr int KB8_STRIDE = 4 * 2 * 64;
+        const float* fx = reinterpret_cast<const float*>(crec + LY::offSv) + l32 * kClsSv + 4 * g;
+#pragma unroll
+        for (int t = 0; t < kClsTailKb; t++) {
+            const f4 w0 = (wq + (size_t)t * KB8_STRIDE)[lane_u];
+            const f4 w1 = (wq + (size_t)t * KB8_STRIDE + 64)[lane_u];
+            const f4 x = *reinterpret_cast<const f4*>(fx + 8 * t);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                acc[0] = mfma(x[j], w0[j], acc[0]);
+                acc[1] = mfma(x[j], w1[j], acc[1]);
+            }
+        }
+        __syncthreads();   // every wave is done with the records and tables
+#pragma unroll
+        for (int ut = 0; ut < 2; ut++) {
+            const float bias = a.b_enc[wave * 64 + ut * 32 + l32];
+            float* xrow = lds + (4 * g) * XS + wave * 64 + ut * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) xrow[acc_row(r) * XS] = acc[ut][r] + bias;
+        }
     } else if (VARIANT == 0 && a.rec) {
         f16v acc[2] = {zero16(), zero16()};
         const uint32_t* rrow = reinterpret_cast<const uint32_t*>(lds) + l32 * RS;
@@ -238,6 +293,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
 
 int launch_forward_bf16(const FwdArgs& a, hipStream_t st) {
     CFP_REQUIRE(a.we_bf && a.wg_bf && a.wav_bf, "bf16 forward without bf16 weight mirrors");
+    CFP_REQUIRE(a.variant == 0 || !a.rec || (a.we_s3 && a.we_pk),
+                "classic bf16 forward without the split encoder mirror");
     const dim3 g(a.n / kTileEnvs), b(kFwdThreads);
     if (a.train) {
         CFP_REQUIRE(a.variant == 0 && a.rec && a.state && a.layers > 0 && !a.r_state &&

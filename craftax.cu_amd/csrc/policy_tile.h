@@ -122,44 +122,69 @@ __device__ __forceinline__ void rec_scatter(const RecRegs& r, float* lds, float*
     if (tid < kTileEnvs) term_s[tid] = r.term;
 }
 
-// Classic-game encoder (encode_obs_kernel, craftax_classic.cu:1714-1751): the
-// observation is one-hot per view cell, so h0 is b_enc plus a sum of W_enc
-// rows selected by the record bytes, in feature order.  Thread k owns hidden
-// unit k and walks the tile's 32 envs; the record bytes are LDS broadcasts and
-// every W_enc row read is one coalesced 1 KiB line set from L2.
-__device__ __forceinline__ void classic_encode_tile(const FwdArgs& a, const uint8_t* crec,
-                                                    float* lds, int tid) {
-    constexpr int CELLS = 63, CH = 21, NBLK = 17;
-    const float* W = a.w_enc;            // uniform base, [tid] applied at each load
-    const unsigned k = (unsigned)tid;
-    const float bias = a.b_enc[tid];
-    for (int e = 0; e < kTileEnvs; e++) {
-        const uint8_t* o = crec + e * CFP_CLASSIC_REC_BYTES;
-        float hv = bias;
-        for (int cell = 0; cell < CELLS; cell++) {
-            hv += (W + (size_t)(cell * CH + (int8_t)o[cell]) * CFP_HIDDEN)[k];
-            const uint32_t m = o[CELLS + cell];
-            if (m) {
-                const float* wm = W + (size_t)(cell * CH + NBLK) * CFP_HIDDEN;
+
+// ---- classic-game encoder tables ---------------------------------------------------
+// The 1323 cell features (63 view cells x (one-hot of 17 block ids + 4 mob bits)) are
+// 0/1: an env's features are packed into a row of bits (cell c = 21 bits at bit 21c), a
+// lane's eight features of a 16-wide K block are one byte of that row, and a 256-entry
+// table turns the byte into eight bf16 0/1.  The 22 scalar features (inventory and
+// intrinsics / 10, direction one-hot, light, sleeping) sit beside them as floats.
+// Layout for ENVS envs inside a byte region that starts with their 148-byte records.
+constexpr int kClsCells = 63, kClsCh = 21;
+constexpr int kClsBits = kClsCells * kClsCh;                 // 1323
+constexpr int kClsKb16 = (kClsBits + 15) / 16;               // 83
+constexpr int kClsBitRow = 44;                               // dwords per env (42 used)
+constexpr int kClsSv = 24;                                   // scalar features per env, padded
+constexpr int kClsTailKb = kClsSv / 8;                       // 3 fp32 K blocks
+template <int ENVS>
+struct ClsLayout {
+    static constexpr int offBits = ENVS * CFP_CLASSIC_REC_BYTES;
+    static constexpr int offLut = offBits + ENVS * kClsBitRow * 4;
+    static constexpr int offSv = offLut + 256 * 16;
+    static constexpr int end = offSv + ENVS * kClsSv * 4;
+    static_assert(offBits % 16 == 0 && offLut % 16 == 0 && offSv % 16 == 0, "alignment");
+};
+
+// Bit rows, byte -> 8 x bf16 table and scalar rows from the records at `base`
+// (all 256 threads; ends with a barrier).  Block ids must be 0..16.
+template <int ENVS>
+__device__ __forceinline__ void classic_prepare(uint8_t* base, int tid) {
+    using LY = ClsLayout<ENVS>;
+    uint32_t* bits = reinterpret_cast<uint32_t*>(base + LY::offBits);
+    u4* lut = reinterpret_cast<u4*>(base + LY::offLut);
+    float* sv = reinterpret_cast<float*>(base + LY::offSv);
+    for (int i = tid; i < ENVS * kClsBitRow; i += kFwdThreads) bits[i] = 0u;
+    {
+        u4 v;
+        uint32_t d[4];
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    if (m & (1u << j)) hv += (wm + (size_t)j * CFP_HIDDEN)[k];
-            }
-        }
-        int f = CELLS * CH;
-#pragma unroll
-        for (int j = 0; j < 16; j++, f++)
-            hv = fmaf((float)(int8_t)o[2 * CELLS + j] / 10.0f, (W + (size_t)f * CFP_HIDDEN)[k], hv);
-        const int dir = (int8_t)o[2 * CELLS + 16];
-#pragma unroll
-        for (int d = 1; d <= 4; d++, f++)
-            hv = fmaf(dir == d ? 1.0f : 0.0f, (W + (size_t)f * CFP_HIDDEN)[k], hv);
-        const float sleeping = o[2 * CELLS + 17] ? 1.0f : 0.0f;
-        const float light = *reinterpret_cast<const float*>(o + 2 * CELLS + 18);
-        hv = fmaf(light, (W + (size_t)f * CFP_HIDDEN)[k], hv); f++;
-        hv = fmaf(sleeping, (W + (size_t)f * CFP_HIDDEN)[k], hv);
-        lds[e * XS + tid] = hv;
+        for (int i = 0; i < 4; i++)
+            d[i] = (((unsigned)tid >> (2 * i)) & 1u) * 0x3F80u |
+                   (((unsigned)tid >> (2 * i + 1)) & 1u) * 0x3F800000u;
+        v.x = d[0]; v.y = d[1]; v.z = d[2]; v.w = d[3];
+        lut[tid] = v;
     }
+    for (int i = tid; i < ENVS * kClsSv; i += kFwdThreads) {
+        const int e = i / kClsSv, f = i - e * kClsSv;
+        const uint8_t* o = base + e * CFP_CLASSIC_REC_BYTES + 2 * kClsCells;
+        float v = 0.0f;
+        if (f < 16) v = (float)(int8_t)o[f] / 10.0f;                  // inventory, intrinsics
+        else if (f < 20) v = (int8_t)o[16] == f - 15 ? 1.0f : 0.0f;   // direction 1..4
+        else if (f == 20) v = *reinterpret_cast<const float*>(o + 18);   // light
+        else if (f == 21) v = o[17] ? 1.0f : 0.0f;                    // sleeping
+        sv[i] = v;
+    }
+    __syncthreads();   // rows are zero before the bits go in
+    for (int i = tid; i < ENVS * kClsCells; i += kFwdThreads) {
+        const int e = i / kClsCells, cell = i - e * kClsCells;
+        const uint8_t* o = base + e * CFP_CLASSIC_REC_BYTES;
+        const uint32_t v = ((1u << (o[cell] & 31u)) & 0x1FFFFu) | ((o[kClsCells + cell] & 15u) << 17);
+        const int bit = kClsCh * cell, dw = bit >> 5, sh = bit & 31;
+        uint32_t* row = bits + e * kClsBitRow;
+        atomicOr(row + dw, v << sh);
+        if (sh > 32 - kClsCh) atomicOr(row + dw + 1, v >> (32 - sh));
+    }
+    __syncthreads();
 }
 
 // Lane-constant context of one wave.
