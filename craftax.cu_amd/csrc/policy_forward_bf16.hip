@@ -86,6 +86,23 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
     for (int r = 0; r < 16; r++)
         if (term_s[acc_row(r) + 4 * g] != 0.0f) tmask |= 1u << r;
 
+    float st[32], stn[32];
+    auto state_fetch = [&](const float* base, float (&v)[32]) {
+#pragma unroll
+        for (int e = 0; e < 32; e++)
+            v[e] = __builtin_nontemporal_load(
+                (base + (acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32)) + loff);
+    };
+    auto state_base = [&](int l) -> float* {
+        if (TRAIN) {
+            const size_t tt = se / a.tr_n_all, ee = se - tt * a.tr_n_all;
+            return a.state + ((tt * a.layers + l) * a.tr_n_all + ee) * CFP_HIDDEN + wave * 64;
+        }
+        return a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64;
+    };
+    // layer 0's state is requested before the encoder and lands under it
+    if (a.layers > 0) state_fetch(state_base(0), st);
+
     // ---- encoder ---------------------------------------------------------------
     if (VARIANT == 1 && a.rec) {
         // encode_obs_kernel (craftax_classic.cu:1714-1751).  Cell features: bits -> bf16
@@ -207,11 +224,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
             const size_t tt = se / a.tr_n_all, ee = se - tt * a.tr_n_all;
             st_base = a.state + ((tt * a.layers + l) * a.tr_n_all + ee) * CFP_HIDDEN + wave * 64;
         }
-        float st[32];
-#pragma unroll
-        for (int e = 0; e < 32; e++)
-            st[e] = __builtin_nontemporal_load(
-                (st_base + (acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32)) + loff);
+        // The state was requested one layer ahead (at the start of the previous layer's
+        // epilogue): vector loads return in order, so a request made here would hold
+        // the first weight fragments of the K loop behind its HBM latency.
 
         f16v acc[6];
 #pragma unroll
@@ -233,6 +248,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
         }
         __syncthreads();   // every wave has read the layer input
 
+        if (l + 1 < a.layers) state_fetch(state_base(l + 1), stn);
         float* rs_base = HAS_RS ? a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64
                                 : nullptr;
         float* out_base = TRAIN ? a.tr_x[l + 1] + e0 * CFP_HIDDEN + wave * 64 : nullptr;
@@ -264,6 +280,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
             if (TRAIN) __builtin_nontemporal_store(hn, (out_base + soff) + loff);
             else __builtin_nontemporal_store(out, (st_base + soff) + loff);
         }
+#pragma unroll
+        for (int e = 0; e < 32; e++) st[e] = stn[e];
         __syncthreads();
     }
     if (a.layers > 0 && a.h3_out) copy_tile_out(lds, a.h3_out + e0 * CFP_HIDDEN, tid);
