@@ -87,6 +87,7 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
         if (term_s[acc_row(r) + 4 * g] != 0.0f) tmask |= 1u << r;
 
     float st[32], stn[32];
+    u4 bq[2][6];
     auto state_fetch = [&](const float* base, float (&v)[32]) {
 #pragma unroll
         for (int e = 0; e < 32; e++)
@@ -232,9 +233,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
 #pragma unroll
         for (int t = 0; t < 6; t++) acc[t] = zero16();
         const u4* wp = a.wg_bf + ((size_t)l * kKb16Hid * 4 + wave) * 6 * 64;
-        u4 bq[2][6];
+        // block 0 of layers 1.. was requested before the previous epilogue, ahead of its
+        // stores and of the state requests in the in-order return queue
+        if (l == 0) {
 #pragma unroll
-        for (int t = 0; t < 6; t++) bq[0][t] = (wp + t * 64)[lane_u];
+            for (int t = 0; t < 6; t++) bq[0][t] = (wp + t * 64)[lane_u];
+        }
 #pragma unroll
         for (int kb = 0; kb < kKb16Hid; kb++) {
             if (kb + 1 < kKb16Hid) {
@@ -245,6 +249,11 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
             const u4 av = a_frag(xs4, l32, g, kb);
 #pragma unroll
             for (int t = 0; t < 6; t++) acc[t] = mfma16(av, bq[kb & 1][t], acc[t]);
+        }
+        if (l + 1 < a.layers) {
+            const u4* wn = wp + (size_t)kKb16Hid * 4 * 6 * 64;   // next layer's mirror
+#pragma unroll
+            for (int t = 0; t < 6; t++) bq[0][t] = (wn + t * 64)[lane_u];
         }
         __syncthreads();   // every wave has read the layer input
 
