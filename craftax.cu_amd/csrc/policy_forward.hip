@@ -317,7 +317,7 @@ __device__ __forceinline__ void classic_encoder_gemm(const FwdArgs& a, const uin
 
 // DO_K: accN[6] += x_K . W_l^T for the tile whose x tile is `xs4K`.  On entry the
 //       ring holds (has been asked for) K blocks 0..2, requested by ring_preload,
-//       followed, when DO_E, by the 32 loads of state_load and nothing else.
+//       followed, when DO_E (or PX = 32), by the 32 loads of state_load and nothing else.
 //       While block kb is multiplied, block kb+1 is read from its slot into the
 //       other half of bl[2][6] and block kb+3 is requested into the slot block kb
 //       was read from one block earlier: LDS latency is covered by one block
@@ -329,7 +329,7 @@ __device__ __forceinline__ void classic_encoder_gemm(const FwdArgs& a, const uin
 //       epilogue behind the MFMAs).  The state values were requested before the
 //       phase (st[32]); in-loop state loads would sit in front of the weight
 //       requests in the in-order return queue with their HBM latency.
-template <bool DO_K, bool DO_E, int MODE>
+template <bool DO_K, bool DO_E, int MODE, int PX = 0>   // PX: loads that follow the preload when !DO_E
 __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6], f4* ring,
                                           const f4* xs4K, const f4* wp, float* xsE,
                                           const StateIO& io, const float (&st)[32],
@@ -339,7 +339,7 @@ __device__ __forceinline__ void gru_phase(f16v (&accN)[6], const f16v (&accO)[6]
     // the later requests, the S stores each epilogue block issues, and in the
     // first blocks the P state loads that follow the preload.
     constexpr int S = !DO_E ? 0 : (MODE == kModeTrain ? 4 : (MODE == kModeRecord ? 2 : 1));
-    constexpr int P = DO_E ? 32 : 0;
+    constexpr int P = DO_E ? 32 : PX;
     f4 aq[2];
     f4 bl[2][6];
     if (DO_K) {
@@ -595,17 +595,17 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
             };
             const int Q = 2 * a.layers;
             if (SINGLE) {
-                // one tile: K phase, then its epilogue, layer by layer.  The state is
-                // requested before the weights, so it has landed when block 0 has.
+                // one tile: K phase, then its epilogue, layer by layer; the state is
+                // requested right behind the first weight blocks, as in the pair schedule
                 if (full_rec) fetch_next();
 #pragma unroll 1
                 for (int l = 0; l < a.layers; l++) {
                     const StateIO io1 = state_io(2 * l + 1);
-                    state_load(io1, st, L);
                     ring_preload(bq, wp0 + (size_t)l * wl, L);
+                    state_load(io1, st, L);   // behind the weights: lands under the K phase
 #pragma unroll
                     for (int t = 0; t < 6; t++) accO[t] = zero16();
-                    gru_phase<true, false, MODE>(accO, accO, bq,
+                    gru_phase<true, false, MODE, 32>(accO, accO, bq,
                                                  reinterpret_cast<const f4*>(lds_all[0]),
                                                  wp0 + (size_t)l * wl, nullptr, io1, st, L);
                     __syncthreads();   // every wave has read the layer input
