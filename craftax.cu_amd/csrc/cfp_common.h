@@ -145,7 +145,11 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
 // (cols % 8 == 0)
 bool gemm_dw_x9_ok(int rows, int cols);
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               int terms, hipStream_t st, int rows_first = 0, float* dW_rest = nullptr);
+               int terms, hipStream_t st, int rows_first = 0, float* dW_rest = nullptr,
+               float* own_work = nullptr, size_t own_work_floats = 0);
+// partial products per product the split kernels run with now (9, 6, or 1 with bf16
+// inputs); 0 when they are switched off
+int gemm_split_terms();
 // dW_a[rows_a][256] += and dW_b[rows_b][256] += from adjacent columns of one dpre matrix
 // (one pass over x on the split kernels, two passes otherwise)
 int gemm_dw_two(int rows_a, int rows_b, int cols, const float* x, const float* dpre, int ld_dpre,

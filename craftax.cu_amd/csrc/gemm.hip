@@ -506,6 +506,8 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
     return launch_splitk_reduce(d_dW, g_dw_work, count, count, splits, st);
 }
 
+int gemm_split_terms() { return g_gemm_split ? split_terms() : 0; }
+
 int gemm_dw_two(int rows_a, int rows_b, int cols, const float* d_x, const float* d_dpre,
                 int ld_dpre, float* d_dW_a, float* d_dW_b, hipStream_t st) {
     CFP_REQUIRE(rows_a > 0 && rows_b > 0 && ld_dpre >= rows_a + rows_b && d_dW_a && d_dW_b,

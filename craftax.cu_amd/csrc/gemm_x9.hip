@@ -361,20 +361,22 @@ bool gemm_dw_x9_ok(int rows, int cols) {
 }
 
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               int terms, hipStream_t st, int rows_first, float* dW_rest) {
+               int terms, hipStream_t st, int rows_first, float* dW_rest, float* own_work,
+               size_t own_work_floats) {
     CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows &&
                     (!dW_rest || (rows_first > 0 && rows_first < rows)),
                 "gemm_dw_x9: columns must be a multiple of 8");
-    float* work = nullptr;
-    size_t work_floats = 0;
-    if (dw_workspace(&work, &work_floats)) return 1;
+    // a caller that overlaps this GEMM with others brings its own split workspace
+    float* work = own_work;
+    size_t work_floats = own_work_floats;
+    if (!work && dw_workspace(&work, &work_floats)) return 1;
     const int groups = (rows + kX9GroupRows - 1) / kX9GroupRows;
     const int total_iters = (cols + kX9IterCols - 1) / kX9IterCols;
     int splits = 256 / groups;   // one workgroup per CU
     const int cap = (int)(work_floats / ((size_t)rows * CFP_HIDDEN));
     if (splits > cap) splits = cap;
     if (splits > total_iters) splits = total_iters;
-    if (splits < 1) splits = 1;
+    CFP_REQUIRE(splits >= 1, "gemm_dw_x9: split workspace too small for %d rows", rows);
     const int ips = (total_iters + splits - 1) / splits;
     splits = (total_iters + ips - 1) / ips;
     const int n_wg = splits * groups;

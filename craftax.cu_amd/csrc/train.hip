@@ -439,6 +439,13 @@ struct cfp_trainer {
     float* live = nullptr;     // [L][n][256] live state for the loss replay
     float* termf = nullptr;    // [n]
     float* av_tmp = nullptr;   // [n][44]
+    // second stream of the backward pass (the layers' dependent chain alternates between
+    // it and the caller's, see cfp_train_backward) and the dW GEMMs' own split workspaces
+    hipStream_t st2 = nullptr;
+    hipEvent_t ev_dh[CFP_MAX_LAYERS] = {};
+    hipEvent_t ev_join = nullptr;
+    float* dw_work2 = nullptr;
+    size_t dw_work2_floats = 0;
 };
 
 static constexpr int kColsumSlices = 1024;
@@ -448,6 +455,10 @@ extern "C" {
 void cfp_train_destroy(cfp_trainer* tr) {
     if (!tr) return;
     for (void* q : tr->owned) (void)hipFree(q);
+    for (hipEvent_t e : tr->ev_dh)
+        if (e) (void)hipEventDestroy(e);
+    if (tr->ev_join) (void)hipEventDestroy(tr->ev_join);
+    if (tr->st2) (void)hipStreamDestroy(tr->st2);
     delete tr;
 }
 
@@ -531,7 +542,14 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     TA(live, (size_t)tr->L * hn * sizeof(float));
     TA(termf, (size_t)tr->n * sizeof(float));
     TA(av_tmp, (size_t)tr->n * CFP_AV * sizeof(float));
+    tr->dw_work2_floats = (size_t)48 * G * H;   // per layer: 48 splits of a gate dW
+    TA(dw_work2, (size_t)tr->L * tr->dw_work2_floats * sizeof(float));
 #undef TA
+    // default priority, as every stream of this library
+    if (ok) ok = hipStreamCreateWithFlags(&tr->st2, hipStreamNonBlocking) == hipSuccess &&
+                 hipEventCreateWithFlags(&tr->ev_join, hipEventDisableTiming) == hipSuccess;
+    for (int l = 0; ok && l < tr->L; l++)
+        ok = hipEventCreateWithFlags(&tr->ev_dh[l], hipEventDisableTiming) == hipSuccess;
     if (ok) ok = hipMemcpy(tr->d_lr, &cfg->lr, 4, hipMemcpyHostToDevice) == hipSuccess &&
                  hipMemcpy(tr->d_ent, &cfg->ent, 4, hipMemcpyHostToDevice) == hipSuccess;
     if (!ok) {
@@ -757,33 +775,58 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         if (colsum_into(tr, tr->dlogits, kHeadLd, g + CFP_OFF_B_A(L), A, cols, st)) return 1;
         if (colsum_into(tr, tr->dlogits + A, kHeadLd, g + CFP_OFF_B_V(L), 1, cols, st)) return 1;
         // ---- reverse MinGRU layers
+        // With the split kernels the dependent chain  reverse(l) -> dh(l) -> reverse(l-1)
+        // hops between two streams: dW(l) is enqueued right behind dh(l) on the stream
+        // that ran it, and the next layer's chain on the other stream behind an event.
+        // dW(l) so starts first and takes its one workgroup per CU; the HBM-bound
+        // reverse kernel of the next layer then fills the wave slots that are left and
+        // runs under it.  Every dW has a split workspace of its own.
+        const int terms = gemm_split_terms();
+        const bool overlap = terms > 1 && gemm_dw_x9_ok(G, cols);
+        hipStream_t chain = st, other = tr->st2;
         const float* dh_gemm = tr->dh3b;
         const float* dh_extra = nullptr;
         for (int l = L - 1; l >= 0; l--) {
             hipLaunchKernelGGL(k_mingru_window_bwd, dim3(grid1((size_t)H * mb)), dim3(256),
-                               0, st, tr->preb[l], tr->x[l], dh_gemm, dh_extra, tr->r_state,
+                               0, chain, tr->preb[l], tr->x[l], dh_gemm, dh_extra, tr->r_state,
                                tr->r_done, tr->dhX, tr->dcarry[l], t0, Tw, mb, n, env_start,
                                l, L, T, seg);
-            if (cfp_gemm_dw(G, cols, tr->x[l], tr->preb[l],
-                            g + CFP_OFF_W_GRU + (size_t)l * G * H, stream))
+            if (!overlap &&
+                gemm_dw_ld(G, cols, tr->x[l], tr->preb[l], G, g + CFP_OFF_W_GRU + (size_t)l * G * H,
+                           chain))
                 return 1;
             // layer 0: dh_enc = W_0^T dpre + highway, accumulated onto the highway term
             if (gemm_dh_acc(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
-                            l == 0 ? tr->dhX : tr->dhG, l == 0, st))
+                            l == 0 ? tr->dhX : tr->dhG, l == 0, chain))
                 return 1;
+            if (overlap) {
+                CFP_HIP_TRY(hipEventRecord(tr->ev_dh[l], chain));
+                if (gemm_dw_x9(G, cols, tr->x[l], tr->preb[l], G,
+                               g + CFP_OFF_W_GRU + (size_t)l * G * H, terms, chain, 0, nullptr,
+                               tr->dw_work2 + (size_t)l * tr->dw_work2_floats, tr->dw_work2_floats))
+                    return 1;
+                CFP_HIP_TRY(hipStreamWaitEvent(other, tr->ev_dh[l], 0));
+                hipStream_t t = chain; chain = other; other = t;
+            }
             dh_gemm = tr->dhG;
             dh_extra = tr->dhX;
         }
         // ---- encoder: db_enc; dW_enc += xobs^T dh_enc (dh_enc sits in dhX)
-        if (colsum_into(tr, tr->dhX, H, g + CFP_OFF_B_ENC, H, cols, st)) return 1;
+        if (colsum_into(tr, tr->dhX, H, g + CFP_OFF_B_ENC, H, cols, chain)) return 1;
         if (dw_enc_records_ok(mb)) {
             // map bytes straight from the records; xobs is free by now and takes the
             // 76-float rows of the fp32 remainder
             if (dw_enc_records(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
-                               env_start, st))
+                               env_start, chain))
                 return 1;
-        } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, st)) {
+        } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, chain)) {
             return 1;
+        }
+        if (overlap) {
+            // both streams meet on the caller's: the window's buffers are free again and
+            // the gradients complete once it has passed this point
+            CFP_HIP_TRY(hipEventRecord(tr->ev_join, tr->st2));
+            CFP_HIP_TRY(hipStreamWaitEvent(st, tr->ev_join, 0));
         }
     }
     CFP_HIP_TRY(hipGetLastError());
