@@ -75,6 +75,7 @@ PROTOTYPES = {
     "cfp_train_backward": (C.c_int, [vp, C.c_int, C.c_int, vp]),
     "cfp_train_zero_loss": (C.c_int, [vp]*2),
     "cfp_train_adam": (C.c_int, [vp]*2),
+    "cfp_train_update": (C.c_int, [vp, C.c_int, vp]),
     "cfp_train_loss": (C.c_int, [vp, vp, vp]),
     "cfp_synth_classic_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),
     "cfp_synth_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),

@@ -446,6 +446,12 @@ struct cfp_trainer {
     hipEvent_t ev_join = nullptr;
     float* dw_work2 = nullptr;
     size_t dw_work2_floats = 0;
+    // cfp_train_update's captured iteration (epochs x minibatches x (backward, Adam)) and
+    // the process-wide GEMM modes it was captured under
+    hipGraph_t tgraph = nullptr;
+    hipGraphExec_t texec = nullptr;
+    int graph_split = -1, graph_bf16 = -1, graph_pol_bf16 = -1;
+    hipStream_t st_own = nullptr;   // capture stream when the caller passes the null stream
 };
 
 static constexpr int kColsumSlices = 1024;
@@ -458,7 +464,10 @@ void cfp_train_destroy(cfp_trainer* tr) {
     for (hipEvent_t e : tr->ev_dh)
         if (e) (void)hipEventDestroy(e);
     if (tr->ev_join) (void)hipEventDestroy(tr->ev_join);
+    if (tr->texec) (void)hipGraphExecDestroy(tr->texec);
+    if (tr->tgraph) (void)hipGraphDestroy(tr->tgraph);
     if (tr->st2) (void)hipStreamDestroy(tr->st2);
+    if (tr->st_own) (void)hipStreamDestroy(tr->st_own);
     delete tr;
 }
 
@@ -850,6 +859,79 @@ int cfp_train_adam(cfp_trainer* tr, void* stream) {
     hipLaunchKernelGGL(k_bump_ctr, dim3(1), dim3(1), 0, st, tr->adam_ctr);
     CFP_HIP_TRY(hipGetLastError());
     return cfp_policy_refresh_weights(tr->p, stream);
+}
+
+// cu_train_body without its collect (craftax_full.cu:13348-13366): per epoch the loss
+// sums start at zero, then every minibatch's backward is followed by its Adam step.
+static int train_body(cfp_trainer* tr, void* stream) {
+    for (int e = 0; e < tr->cfg.epochs; e++) {
+        int rc = cfp_train_zero_loss(tr, stream);
+        for (int m = 0; m < tr->cfg.minibatches && rc == 0; m++) {
+            rc = cfp_train_backward(tr, m * tr->mb, tr->mb, stream);
+            if (rc == 0) rc = cfp_train_adam(tr, stream);
+        }
+        if (rc != 0) return rc;
+    }
+    return 0;
+}
+
+int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
+    CFP_REQUIRE(tr, "cfp_train_update: NULL trainer");
+    hipStream_t st = (hipStream_t)stream;
+    if (!use_graph) {
+        const int rc = train_body(tr, st);
+        if (rc != 0) return rc;
+        CFP_HIP_TRY(hipStreamSynchronize(st));
+        return 0;
+    }
+    if (!st) {   // the null stream cannot be captured
+        if (!tr->st_own) CFP_HIP_TRY(hipStreamCreate(&tr->st_own));
+        st = tr->st_own;
+    }
+    const int split = cfp_get_gemm_split(), bf = cfp_get_gemm_bf16(),
+              pbf = cfp_policy_gemm_bf16(tr->p);
+    if (tr->texec && (split != tr->graph_split || bf != tr->graph_bf16 ||
+                      pbf != tr->graph_pol_bf16)) {
+        (void)hipGraphExecDestroy(tr->texec);
+        (void)hipGraphDestroy(tr->tgraph);
+        tr->texec = nullptr;
+        tr->tgraph = nullptr;
+    }
+    if (!tr->texec) {
+        // Warm-up as in the reference (:13379-13386): one bare backward, no Adam, so that
+        // the lazily allocated GEMM workspaces exist before the capture (an allocation
+        // inside a capture is illegal); parameters stay untouched, the gradients it
+        // left are cleared again.
+        int rc = cfp_train_backward(tr, 0, tr->mb, st);
+        if (rc != 0) return rc;
+        hipLaunchKernelGGL(k_fill, dim3(grid1(tr->p->param_count)), dim3(256), 0, st, tr->grads,
+                           tr->p->param_count, 0.0f);
+        CFP_HIP_TRY(hipGetLastError());
+        CFP_HIP_TRY(hipStreamSynchronize(st));
+        CFP_HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        rc = train_body(tr, st);
+        hipGraph_t g = nullptr;
+        const hipError_t ec = hipStreamEndCapture(st, &g);   // always leaves capture mode
+        if (rc != 0) {
+            if (g) (void)hipGraphDestroy(g);
+            return rc;
+        }
+        CFP_HIP_TRY(ec);
+        hipGraphExec_t ex = nullptr;
+        const hipError_t ei = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+        if (ei != hipSuccess) {
+            (void)hipGraphDestroy(g);
+            CFP_HIP_TRY(ei);
+        }
+        tr->tgraph = g;
+        tr->texec = ex;
+        tr->graph_split = split;
+        tr->graph_bf16 = bf;
+        tr->graph_pol_bf16 = pbf;
+    }
+    CFP_HIP_TRY(hipGraphLaunch(tr->texec, st));
+    CFP_HIP_TRY(hipStreamSynchronize(st));
+    return 0;
 }
 
 int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream) {

@@ -260,6 +260,10 @@ class Trainer:
     def adam(self):
         _check(lib().cfp_train_adam(self._h, _stream()))
 
+    def update(self, use_graph=False):
+        """cu_train_update (craftax_full.cu:13372) over the stored rollout."""
+        _check(lib().cfp_train_update(self._h, 1 if use_graph else 0, _stream()))
+
     def loss(self):
         out = np.zeros(4)
         _check(lib().cfp_train_loss(self._h, out.ctypes.data_as(C.c_void_p), _stream()))

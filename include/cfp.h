@@ -334,6 +334,22 @@ int cfp_train_zero_loss(cfp_trainer* tr, void* stream);
 /* cu_train_adam (craftax_full.cu:13337): Adam step from the grads arena (which
  * it zeroes), bumps the step counter, rebuilds the weight mirrors. */
 int cfp_train_adam(cfp_trainer* tr, void* stream);
+/* cu_train_body without its collect + cu_train_update (craftax_full.cu:13348-13406):
+ * one PPO iteration over the stored rollout (slabs, adv/ret and the advantage
+ * statistics already in place): epochs x (loss sums reset, minibatches x
+ * (cfp_train_backward of the m-th contiguous env slice, cfp_train_adam)), then a
+ * synchronisation of the stream, as in the reference.  use_graph != 0 is the
+ * reference's graph mode: the first call runs one bare backward as a warm-up
+ * (no Adam, parameters untouched; the grads arena is cleared afterwards, so it
+ * must hold nothing the caller still needs), captures the iteration once on
+ * `stream` (on a stream of the trainer's own when `stream` is NULL, which cannot
+ * be captured) and replays it; later calls only replay.  lr, the entropy
+ * coefficient and the Adam step counter live in device memory, so replays see
+ * their current values.  A change of cfp_set_gemm_split / cfp_set_gemm_bf16 /
+ * cfp_policy_set_gemm_bf16 between calls makes the next call capture again.
+ * Unlike the reference, a graph that cannot be instantiated is an error, not a
+ * silent eager run: call again with use_graph = 0. */
+int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream);
 /* cu_train_loss (craftax_full.cu:13414): full-batch PPO loss of the stored
  * rollout with live recurrence inside BPTT segments; host_loss4 = raw sums
  * (pg, v, ent) and the total (pg + vf*v - ent*H) / (n*T).  Synchronises. */

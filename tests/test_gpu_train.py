@@ -257,6 +257,61 @@ def test_update_iteration_replays_from_a_graph(pkg, cuda):
         tr.close(); pol.close()
 
 
+@pytest.mark.parametrize("on_side_stream", [False, True])
+def test_train_update_eager_and_graph_match_the_manual_loop(pkg, cuda, on_side_stream):
+    """cfp_train_update (the reference's cu_train_update without its collect): two
+    epochs of two minibatches, (a) eager and (b) captured by the library and replayed,
+    against (c) the same loop written out with backward / adam calls on identical
+    triplets.  Parameters, Adam moments and the last epoch's loss sums must agree bit
+    for bit after every iteration; between iterations lr is annealed through its
+    device scalar and eager work runs, so a replay that baked in a value or read
+    stale memory would differ."""
+    import torch
+    n, T = 64, 6
+    cfg = dict(epochs=2, minibatches=2)
+    trip = [_collect(pkg, cuda, n, T, 321, 0.1, **cfg) for _ in range(3)]
+    (_, pol_m, tr_m, _), (_, pol_e, tr_e, _), (_, pol_g, tr_g, _) = trip
+    mb = n // 2
+    assert tr_m.mb == mb
+    stream = torch.cuda.Stream() if on_side_stream else torch.cuda.current_stream()
+    with torch.cuda.stream(stream):
+        for it in range(3):
+            for tr in (tr_m, tr_e, tr_g):
+                tr.buf("lr").fill_(3e-4 * (1.0 - 0.25 * it))
+            for _ in range(cfg["epochs"]):
+                tr_m.zero_loss()
+                for m in range(cfg["minibatches"]):
+                    tr_m.backward(m * mb, mb)
+                    tr_m.adam()
+            tr_e.update(use_graph=False)
+            tr_g.update(use_graph=True)
+            torch.cuda.synchronize()
+            junk = torch.randn(1 << 16, device=cuda).sum().item()   # eager work between replays
+            assert np.isfinite(junk)
+            for name, pol, tr in (("eager", pol_e, tr_e), ("graph", pol_g, tr_g)):
+                assert torch.equal(pol.params, pol_m.params), f"{name} params, iteration {it}"
+                assert torch.equal(tr.buf("adam_m"), tr_m.buf("adam_m")), f"{name} adam_m {it}"
+                assert torch.equal(tr.buf("adam_v"), tr_m.buf("adam_v")), f"{name} adam_v {it}"
+                assert torch.equal(tr.buf("loss_acc"), tr_m.buf("loss_acc")), f"{name} loss {it}"
+                assert not tr.buf("grads").any(), f"{name}: Adam leaves the grads arena zero"
+        assert not torch.equal(pol_m.params, _t(trip[0][0], cuda))     # the updates moved them
+        # a change of the GEMM mode makes the next graph call capture again
+        pkg.policy.set_gemm_split(0)
+        try:
+            for _ in range(cfg["epochs"]):
+                tr_m.zero_loss()
+                for m in range(cfg["minibatches"]):
+                    tr_m.backward(m * mb, mb)
+                    tr_m.adam()
+            tr_g.update(use_graph=True)
+            torch.cuda.synchronize()
+            assert torch.equal(pol_g.params, pol_m.params), "re-captured under the new GEMM mode"
+        finally:
+            pkg.policy.set_gemm_split(1)
+    for _, pol, tr, _ in trip:
+        tr.close(); pol.close()
+
+
 def test_checkpoint_roundtrip(pkg, cuda, tmp_path):
     """CFW1 file: header words, byte-exact params, mirrors refreshed on load, and the
     reference's rejections (wrong shape, truncated file)."""
