@@ -7,7 +7,8 @@
   classic_1m      classic-game policy forward, 1 048 576 envs, 148-byte records
   record_kernels  the HBM-bound byte kernels at 65 536 envs: state -> 996-byte
                   records (fuzzed reference states of tests/golden, tiled) and
-                  records -> fp32 features
+                  records -> fp32 features, and the unfused MinGRU gate/blend
+                  epilogue of one layer
 
 Usage:  python craftax.cu_amd/bench_configs.py [--reps 10] [--only NAME]
 The headline workload (262 144 envs) is bench.py at the repository root."""
@@ -137,6 +138,16 @@ def record_kernels(pkg, torch, reps):
     ms_r = _time(torch, lambda: P.record_obs(scalars, planes, planes[plane:], planes[2 * plane:],
                                              n, 3 * plane, 0, rec=rec), reps)
     ms_x = _time(torch, lambda: P.expand_obs(rec, n, xobs=xobs), reps)
+    # the unfused gate/blend epilogue of one MinGRU layer (k_mingru_epi_fwd), recording form
+    pre = torch.randn(n, 768, device="cuda")
+    xin = torch.randn(n, 256, device="cuda")
+    state = torch.randn(n, 256, device="cuda") * 0.5
+    rs = torch.empty(n, 256, device="cuda")
+    hout = torch.empty(n, 256, device="cuda")
+    term = torch.zeros(n, device="cuda")
+    ms_e = _time(torch, lambda: P.mingru_epi_fwd(pre, xin, state, term, r_state_store=rs,
+                                                 h_out=hout), reps)
+    b_e = 4 + 256 * 4 * (3 + 1 + 1 + 3)     # terminal; pre(3), x, state in; h, state, r_state out
     # algorithmic bytes per env: scalars + 99 cells x 3 plane bytes gathered + 996 written;
     # 996 read + 843 x 4 written
     b_r, b_x = sc.shape[1] + 99 * 3 + 996, 996 + 843 * 4
@@ -144,7 +155,10 @@ def record_kernels(pkg, torch, reps):
             "record_obs": {"ms": ms_r, "envs_per_s": n / ms_r * 1e3, "bytes_per_env": b_r,
                            "gb_per_s": b_r * n / ms_r / 1e6, "frac_hbm_peak": b_r * n / ms_r / 1e6 / 8000},
             "expand_obs": {"ms": ms_x, "envs_per_s": n / ms_x * 1e3, "bytes_per_env": b_x,
-                           "gb_per_s": b_x * n / ms_x / 1e6, "frac_hbm_peak": b_x * n / ms_x / 1e6 / 8000}}
+                           "gb_per_s": b_x * n / ms_x / 1e6, "frac_hbm_peak": b_x * n / ms_x / 1e6 / 8000},
+            "mingru_epi_fwd": {"ms": ms_e, "envs_per_s": n / ms_e * 1e3, "bytes_per_env": b_e,
+                               "gb_per_s": b_e * n / ms_e / 1e6,
+                               "frac_hbm_peak": b_e * n / ms_e / 1e6 / 8000}}
 
 
 def main():

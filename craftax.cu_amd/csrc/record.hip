@@ -7,7 +7,7 @@
 // (9 rows x 11 cols, row-major) x 8 bytes {block, item+1, visible, melee+1,
 // passive+1, ranged+1, mob-projectile+1, player-projectile+1}, then 51 raw
 // little-endian fp32 scalars.  All of it is integer/byte work bound by HBM
-// gathers; one wavefront encodes one env.
+// gathers; sixteen lanes encode one env.
 #include "cfp_common.h"
 
 namespace cfp {
@@ -276,26 +276,38 @@ __device__ __forceinline__ float sigmoid_fast(float z) {
     return __builtin_amdgcn_rcpf(1.0f + __expf(-z));
 }
 
-__global__ void k_mingru_epi_fwd(const float* __restrict__ pre,
-                                 const float* __restrict__ x,
-                                 float* __restrict__ state,
-                                 float* __restrict__ h_out,
-                                 float* __restrict__ r_state_store,
-                                 const float* __restrict__ prev_terminals,
-                                 size_t total) {
-    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int k = (int)(idx & (CFP_HIDDEN - 1));
-    const size_t col = idx / CFP_HIDDEN;
-    float st = state[idx];
-    if (prev_terminals && prev_terminals[col] != 0.0f) st = 0.0f;
-    if (r_state_store) r_state_store[idx] = st;
-    const size_t o3 = col * CFP_GRU + k;
-    const float zh = pre[o3], zg = pre[o3 + CFP_HIDDEN], zp = pre[o3 + 2 * CFP_HIDDEN];
-    const float gh = zh >= 0.0f ? zh + 0.5f : sigmoid_fast(zh);
-    const float out = st + sigmoid_fast(zg) * (gh - st);
-    const float p = sigmoid_fast(zp);
-    h_out[idx] = p * out + (1.0f - p) * x[idx];
+// Four hidden units per thread: every operand is one 16-byte access (the three
+// gate rows of a column are 256 floats apart), all seven loads in flight before
+// the first use; pre and x are read once (streamed past the caches).
+__global__ __launch_bounds__(256) void k_mingru_epi_fwd(const f4* __restrict__ pre,
+                                                        const f4* __restrict__ x,
+                                                        f4* __restrict__ state,
+                                                        f4* __restrict__ h_out,
+                                                        f4* __restrict__ r_state_store,
+                                                        const float* __restrict__ prev_terminals,
+                                                        size_t total4) {
+    constexpr int H4 = CFP_HIDDEN / 4;
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= total4) return;
+    const int k4 = (int)(idx & (H4 - 1));
+    const size_t col = idx / H4;
+    const size_t o3 = col * (CFP_GRU / 4) + k4;
+    const f4 zh = __builtin_nontemporal_load(pre + o3);
+    const f4 zg = __builtin_nontemporal_load(pre + o3 + H4);
+    const f4 zp = __builtin_nontemporal_load(pre + o3 + 2 * H4);
+    const f4 xv = __builtin_nontemporal_load(x + idx);
+    f4 st = state[idx];
+    if (prev_terminals && prev_terminals[col] != 0.0f) st = f4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (r_state_store) __builtin_nontemporal_store(st, r_state_store + idx);
+    f4 out, h;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const float gh = zh[j] >= 0.0f ? zh[j] + 0.5f : sigmoid_fast(zh[j]);
+        out[j] = st[j] + sigmoid_fast(zg[j]) * (gh - st[j]);
+        const float p = sigmoid_fast(zp[j]);
+        h[j] = p * out[j] + (1.0f - p) * xv[j];
+    }
+    h_out[idx] = h;
     state[idx] = out;
 }
 
@@ -375,10 +387,17 @@ int cfp_mingru_epi_fwd(const float* d_pre, const float* d_x, float* d_state,
                        const float* d_prev_terminals, int cols, void* stream) {
     CFP_REQUIRE(d_pre && d_x && d_state && d_h_out && cols > 0,
                 "cfp_mingru_epi_fwd: bad argument");
-    const size_t total = (size_t)cols * CFP_HIDDEN;
-    hipLaunchKernelGGL(k_mingru_epi_fwd, dim3((unsigned)((total + 255) / 256)),
-                       dim3(256), 0, (hipStream_t)stream, d_pre, d_x, d_state,
-                       d_h_out, d_r_state_store, d_prev_terminals, total);
+    const uintptr_t all = reinterpret_cast<uintptr_t>(d_pre) | reinterpret_cast<uintptr_t>(d_x) |
+                          reinterpret_cast<uintptr_t>(d_state) |
+                          reinterpret_cast<uintptr_t>(d_h_out) |
+                          reinterpret_cast<uintptr_t>(d_r_state_store);
+    CFP_REQUIRE((all & 15u) == 0, "cfp_mingru_epi_fwd: buffers must be 16-byte aligned");
+    const size_t total4 = (size_t)cols * (CFP_HIDDEN / 4);
+    hipLaunchKernelGGL(k_mingru_epi_fwd, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0,
+                       (hipStream_t)stream, reinterpret_cast<const f4*>(d_pre),
+                       reinterpret_cast<const f4*>(d_x), reinterpret_cast<f4*>(d_state),
+                       reinterpret_cast<f4*>(d_h_out), reinterpret_cast<f4*>(d_r_state_store),
+                       d_prev_terminals, total4);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }
