@@ -87,7 +87,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
         if (term_s[acc_row(r) + 4 * g] != 0.0f) tmask |= 1u << r;
 
     float st[32], stn[32];
-    u4 bq[2][6];
+    constexpr int kGateAhead = 2;   // K blocks of gate weights in flight
+    u4 bq[kGateAhead + 1][6];
     auto state_fetch = [&](const float* base, float (&v)[32]) {
 #pragma unroll
         for (int e = 0; e < 32; e++)
@@ -165,44 +166,58 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
         const float* frow = reinterpret_cast<const float*>(rrow) + CFP_OBS_MAP / 4;
         const u4* wp = a.we_bf + (size_t)(wave * 2) * 64;
         constexpr int KB_STRIDE = 4 * 2 * 64;   // u4 per K block
-        u4 b0 = wp[lane_u], b1 = (wp + 64)[lane_u];
+        // weights of kEncAhead K blocks in flight: one block ahead the wave would sit out
+        // an L2 round trip per block of two MFMAs
+        constexpr int kEncAhead = 4;
+        static_assert(kKb16Map - 1 == 12 * kEncAhead && kKb16Enc == kKb16Map + 4, "block schedule below");
+        u4 bw[kEncAhead][2];
+#pragma unroll
+        for (int i = 0; i < kEncAhead; i++) {
+            bw[i][0] = (wp + (size_t)i * KB_STRIDE)[lane_u];
+            bw[i][1] = (wp + (size_t)i * KB_STRIDE + 64)[lane_u];
+        }
         uint32_t w0 = rrow[2 * g], w1 = rrow[2 * g + 1];
 #pragma unroll 1
-        for (int kb = 0; kb < kKb16Map; kb++) {
-            // block kb+1: weights, and bytes (for kb = 48 the g = 1 half reads tail
-            // bits, which block 49 below replaces by the float path)
-            const u4 n0 = (wp + (size_t)(kb + 1) * KB_STRIDE)[lane_u];
-            const u4 n1 = (wp + (size_t)(kb + 1) * KB_STRIDE + 64)[lane_u];
-            const uint32_t m0 = rrow[4 * (kb + 1) + 2 * g];
-            const uint32_t m1 = rrow[4 * (kb + 1) + 2 * g + 1];
+        for (int kb0 = 0; kb0 < kKb16Map - 1; kb0 += kEncAhead) {
+#pragma unroll
+            for (int i = 0; i < kEncAhead; i++) {
+                const int kb = kb0 + i;
+                const uint32_t m0 = rrow[4 * (kb + 1) + 2 * g];
+                const uint32_t m1 = rrow[4 * (kb + 1) + 2 * g + 1];
+                const u4 av = bytes_to_bf16x8(w0, w1);
+                acc[0] = mfma16(av, bw[i][0], acc[0]);
+                acc[1] = mfma16(av, bw[i][1], acc[1]);
+                bw[i][0] = (wp + (size_t)(kb + kEncAhead) * KB_STRIDE)[lane_u];     // <= block 51
+                bw[i][1] = (wp + (size_t)(kb + kEncAhead) * KB_STRIDE + 64)[lane_u];
+                w0 = m0; w1 = m1;
+            }
+        }
+        // bw[0..3] now hold blocks 48..51.  Block 48: the last all-map block
+        {
+            const uint32_t m0 = rrow[4 * kKb16Map + 2 * g];       // g = 1 reads tail bits, which
+            const uint32_t m1 = rrow[4 * kKb16Map + 2 * g + 1];   // block 49 replaces by floats
             const u4 av = bytes_to_bf16x8(w0, w1);
-            acc[0] = mfma16(av, b0, acc[0]);
-            acc[1] = mfma16(av, b1, acc[1]);
-            b0 = n0; b1 = n1; w0 = m0; w1 = m1;
+            acc[0] = mfma16(av, bw[0][0], acc[0]);
+            acc[1] = mfma16(av, bw[0][1], acc[1]);
+            bw[0][0] = (wp + (size_t)(kKb16Enc - 1) * KB_STRIDE)[lane_u];           // block 52
+            bw[0][1] = (wp + (size_t)(kKb16Enc - 1) * KB_STRIDE + 64)[lane_u];
+            w0 = m0; w1 = m1;
         }
         // block 49: features 784..791 are map bytes (g = 0), 792..799 tail floats (g = 1)
         {
-            const u4 n0 = (wp + (size_t)(kKb16Map + 1) * KB_STRIDE)[lane_u];
-            const u4 n1 = (wp + (size_t)(kKb16Map + 1) * KB_STRIDE + 64)[lane_u];
             const u4 ab = bytes_to_bf16x8(w0, w1);
             const u4 af = floats_to_bf16x8(frow);
             const u4 av = g ? af : ab;
-            acc[0] = mfma16(av, b0, acc[0]);
-            acc[1] = mfma16(av, b1, acc[1]);
-            b0 = n0; b1 = n1;
+            acc[0] = mfma16(av, bw[1][0], acc[0]);
+            acc[1] = mfma16(av, bw[1][1], acc[1]);
         }
         // blocks 50..52: tail floats 8 + 16(kb-50) + 8g .. ; features 843..847 read as 0
 #pragma unroll
         for (int kb = kKb16Map + 1; kb < kKb16Enc; kb++) {
-            u4 n0 = b0, n1 = b1;
-            if (kb + 1 < kKb16Enc) {
-                n0 = (wp + (size_t)(kb + 1) * KB_STRIDE)[lane_u];
-                n1 = (wp + (size_t)(kb + 1) * KB_STRIDE + 64)[lane_u];
-            }
+            const int slot = (kb - (kKb16Map - 1)) % kEncAhead;
             const u4 av = floats_to_bf16x8(frow + 16 * kb - CFP_OBS_MAP + 8 * g);
-            acc[0] = mfma16(av, b0, acc[0]);
-            acc[1] = mfma16(av, b1, acc[1]);
-            b0 = n0; b1 = n1;
+            acc[0] = mfma16(av, bw[slot][0], acc[0]);
+            acc[1] = mfma16(av, bw[slot][1], acc[1]);
         }
         __syncthreads();   // every wave is done with the record bytes
 #pragma unroll
@@ -233,27 +248,37 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
 #pragma unroll
         for (int t = 0; t < 6; t++) acc[t] = zero16();
         const u4* wp = a.wg_bf + ((size_t)l * kKb16Hid * 4 + wave) * 6 * 64;
-        // block 0 of layers 1.. was requested before the previous epilogue, ahead of its
-        // stores and of the state requests in the in-order return queue
+        // The weights travel kGateAhead K blocks ahead: one block ahead, every block of six
+        // MFMAs (192 cycles) sat out a whole L2 round trip (~1000 cycles under this load).
+        // The first blocks of layers 1.. were requested before the previous epilogue, ahead
+        // of its stores and of the state requests in the in-order return queue.
         if (l == 0) {
 #pragma unroll
-            for (int t = 0; t < 6; t++) bq[0][t] = (wp + t * 64)[lane_u];
+            for (int i = 0; i < kGateAhead; i++)
+#pragma unroll
+                for (int t = 0; t < 6; t++)
+                    bq[i][t] = (wp + (size_t)i * KB_STRIDE + t * 64)[lane_u];
         }
 #pragma unroll
         for (int kb = 0; kb < kKb16Hid; kb++) {
-            if (kb + 1 < kKb16Hid) {
+            if (kb + kGateAhead < kKb16Hid) {
 #pragma unroll
                 for (int t = 0; t < 6; t++)
-                    bq[(kb + 1) & 1][t] = (wp + (size_t)(kb + 1) * KB_STRIDE + t * 64)[lane_u];
+                    bq[(kb + kGateAhead) % (kGateAhead + 1)][t] =
+                        (wp + (size_t)(kb + kGateAhead) * KB_STRIDE + t * 64)[lane_u];
             }
             const u4 av = a_frag(xs4, l32, g, kb);
 #pragma unroll
-            for (int t = 0; t < 6; t++) acc[t] = mfma16(av, bq[kb & 1][t], acc[t]);
+            for (int t = 0; t < 6; t++)
+                acc[t] = mfma16(av, bq[kb % (kGateAhead + 1)][t], acc[t]);
         }
         if (l + 1 < a.layers) {
             const u4* wn = wp + (size_t)kKb16Hid * 4 * 6 * 64;   // next layer's mirror
 #pragma unroll
-            for (int t = 0; t < 6; t++) bq[0][t] = (wn + t * 64)[lane_u];
+            for (int i = 0; i < kGateAhead; i++)
+#pragma unroll
+                for (int t = 0; t < 6; t++)
+                    bq[i][t] = (wn + (size_t)i * KB_STRIDE + t * 64)[lane_u];
         }
         __syncthreads();   // every wave has read the layer input
 
@@ -281,10 +306,13 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
             const float sg = sigmoid_fast(zg);
             const float sh = sigmoid_fast(zh);
             const float gh = zh >= 0.0f ? zh + 0.5f : sh;
-            const float out = s + sg * (gh - s);
+            // explicit fused multiply-adds: left to the compiler, which product of
+            // p*out + (1-p)*x gets contracted depends on the surrounding code, and every
+            // instantiation of this kernel must produce the same bits
+            const float out = __builtin_fmaf(sg, gh - s, s);
             const float p = sigmoid_fast(zp);
             const float xv = *xp;
-            const float hn = p * out + (1.0f - p) * xv;
+            const float hn = __builtin_fmaf(p, out - xv, xv);
             *xp = hn;
             if (TRAIN) __builtin_nontemporal_store(hn, (out_base + soff) + loff);
             else __builtin_nontemporal_store(out, (st_base + soff) + loff);
