@@ -50,6 +50,35 @@ __host__ __device__ inline float unit24(uint64_t z) {
     return (float)(z >> 40) * (1.0f / 16777216.0f);
 }
 
+// Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2,
+// 3", SC'11; the generator behind curandStatePhilox4_32_10_t): ten rounds of
+//   (c0, c1, c2, c3) <- (hi(M1*c2) ^ c1 ^ k0, lo(M1*c2), hi(M0*c0) ^ c3 ^ k1, lo(M0*c0)),
+// the key bumped by the Weyl constants between rounds.
+__host__ __device__ inline void philox4x32_10(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
+    for (int r = 0; r < 10; r++) {
+        const uint64_t p0 = 0xD2511F53ull * c[0], p1 = 0xCD9E8D57ull * c[2];
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c[1] ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c[3] ^ k1;
+        c[1] = (uint32_t)p1;
+        c[3] = (uint32_t)p0;
+        c[0] = n0;
+        c[2] = n2;
+        k0 += 0x9E3779B9u;
+        k1 += 0xBB67AE85u;
+    }
+}
+// The first curand_uniform() after curand_init(seed, subsequence, offset, &state) of a
+// Philox4_32_10 state, by cuRAND's documented state layout: key = seed, the 128-bit
+// counter = subsequence * 2^64 + offset / 4, of whose four output words the draw is word
+// offset % 4; uniform = x * 2^-32 + 2^-33, in (0, 1].
+__host__ __device__ inline float philox_uniform(uint64_t seed, uint64_t subsequence,
+                                                uint64_t offset) {
+    const uint64_t blk = offset >> 2;
+    uint32_t c[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subsequence,
+                     (uint32_t)(subsequence >> 32)};
+    philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
+    return __builtin_fmaf((float)c[offset & 3], 2.3283064365386963e-10f, 1.1641532182693481e-10f);
+}
+
 #define CFP_HIP_TRY(expr)                                                     \
     do {                                                                      \
         hipError_t e_ = (expr);                                               \

@@ -3,10 +3,12 @@
 //
 // Reference: k_value_sample (craftax_full.cu:9714-9741) with
 // cf_nn_sample_action (:9147-9165), k_record_rd (:9758-9767).  The reference
-// draws its uniform from cuRAND Philox (seed ^ 0xA5A5..., subsequence = env,
-// offset = device step counter); that stream cannot be reproduced without CUDA,
-// so the uniform here comes from this library's own counter generator with the
-// same three inputs: unit24(mix64(seed ^ 0xA5A5A5A5A5A5A5A5, step, env)).  Given
+// draws its uniform from cuRAND: curand_init(seed ^ 0xA5A5..., subsequence = env,
+// offset = device step counter) of a Philox4_32_10 state, then curand_uniform.
+// Here the same draw is computed directly (philox_uniform in cfp_common.h): the
+// Philox4x32-10 block function is pinned by the published known-answer vectors;
+// the mapping of (seed, subsequence, offset) onto key and counter follows cuRAND's
+// documented state layout and could only be confirmed against a CUDA run.  Given
 // the uniform, the action and its log-probability follow the reference's
 // arithmetic exactly (max-shifted expf, ascending cumulative sum, first index
 // with target <= cum, last action as the fall-through).
@@ -33,7 +35,7 @@ __global__ void k_value_sample(const float* __restrict__ av, int avs, int action
         total += p[a];
     }
     const uint64_t step = step_ctr ? *step_ctr : 0;
-    const float u = unit24(mix64(seed ^ 0xA5A5A5A5A5A5A5A5ULL, step, (uint64_t)e));
+    const float u = philox_uniform(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)e, step);
     const float target = u * total;
     float cum = 0.0f;
     int action = actions - 1;

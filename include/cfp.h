@@ -252,10 +252,11 @@ int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
  * may be NULL), action ~ softmax(av[e][0..actions)) by inversion of the cumulative
  * sum (cf_nn_sample_action :9147-9165), logprob = log softmax at the action; the
  * action also goes to d_env_actions[e] as a float when that is not NULL (the
- * reference's env action slot).  The uniform is
- * unit24(mix64(seed ^ 0xA5A5A5A5A5A5A5A5, *d_step_ctr or 0, e)) -- this library's
- * counter generator in place of the reference's cuRAND Philox stream, which
- * cannot be reproduced without CUDA. */
+ * reference's env action slot).  The uniform is the reference's: the first
+ * curand_uniform of a Philox4_32_10 state after curand_init(seed ^
+ * 0xA5A5A5A5A5A5A5A5, subsequence e, offset *d_step_ctr or 0), computed directly
+ * (Philox4x32-10 with key = seed, counter = subsequence * 2^64 + offset / 4, word
+ * offset % 4; x * 2^-32 + 2^-33). */
 int cfp_value_sample(const float* d_av, int n, int actions, float* d_env_actions,
                      int32_t* d_actions, float* d_logprobs, float* d_values, uint64_t seed,
                      const uint64_t* d_step_ctr, void* stream);

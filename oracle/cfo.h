@@ -18,9 +18,13 @@
  *                           craftax_full.cu:13854-13907) and closed forms
  *   cfo_sample_action       pinned: closed forms (equal logits, dominant logit,
  *                           normalisation of exp(logprob))
- *   The reference's cuRAND Philox streams (weight init, action sampling) are
- *   "parity unpinned": they cannot be reproduced without CUDA and are not
- *   restated here.
+ *   cfo_philox4x32_10       pinned: the three known-answer vectors published with
+ *                           the generator (Random123 kat_vectors, philox4x32 10)
+ *   cfo_philox_uniform      "parity unpinned": how cuRAND maps (seed, subsequence,
+ *                           offset) onto Philox key / counter / output word is
+ *                           restated from its documentation; only a CUDA run could
+ *                           confirm it.  The reference's weight-init stream
+ *                           (k_nn_init_weights) is not restated.
  */
 #ifndef CFO_H_
 #define CFO_H_
@@ -80,8 +84,12 @@ void cfo_forward_f32(const float* params, int layers, int n,
 
 /* cf_nn_sample_action (craftax_full.cu:9147-9165) for a given uniform u; pinned
  * by closed forms (equal logits -> floor(u*A), dominant logit, exp(logprob) sums
- * to one) -- the reference's Philox uniform itself is not restated. */
+ * to one). */
 int cfo_sample_action(const float* logits, int actions, float u, float* logprob);
+/* Philox4x32-10 and the uniform of the reference's sampler (k_value_sample,
+ * craftax_full.cu:9732-9736: curand_init(seed ^ 0xA5A5.., env, step) + curand_uniform). */
+void cfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+float cfo_philox_uniform(uint64_t seed, uint64_t subsequence, uint64_t offset);
 float cfo_sample_margin(const float* logits, int actions, float u);
 
 int cfo_max_threads(void);

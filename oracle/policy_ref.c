@@ -224,6 +224,33 @@ int cfo_sample_action(const float* logits, int actions, float u, float* logprob)
     return action;
 }
 
+/* Philox4x32-10 block function (Salmon et al., SC'11; the generator of the
+ * reference's curandStatePhilox4_32_10_t, craftax_full.cu:9123-9131, :9732-9736). */
+void cfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+    uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+    for (int r = 0; r < 10; r++) {
+        const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+        const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+        c1 = (uint32_t)p1; c3 = (uint32_t)p0; c0 = n0; c2 = n2;
+        k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+    }
+    out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* First curand_uniform() after curand_init(seed, subsequence, offset) of a Philox
+ * state, by cuRAND's documented layout: key = seed, counter = subsequence * 2^64 +
+ * offset / 4, output word offset % 4, uniform = x * 2^-32 + 2^-33 (one fused
+ * multiply-add, as nvcc contracts it). */
+float cfo_philox_uniform(uint64_t seed, uint64_t subsequence, uint64_t offset) {
+    const uint64_t blk = offset >> 2;
+    const uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subsequence,
+                             (uint32_t)(subsequence >> 32)};
+    const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+    uint32_t out[4];
+    cfo_philox4x32_10(ctr, key, out);
+    return fmaf((float)out[offset & 3], 2.3283064365386963e-10f, 1.1641532182693481e-10f);
+}
+
 /* Distance of u*total from the nearest cumulative-sum boundary, relative to
  * total: draws this close to a boundary may legitimately land on either side
  * when expf differs by an ulp between implementations. */

@@ -76,6 +76,10 @@ def cfo():
         lib.cfo_sample_action.restype = C.c_int
         lib.cfo_sample_margin.argtypes = [vp, C.c_int, C.c_float]
         lib.cfo_sample_margin.restype = C.c_float
+        lib.cfo_philox4x32_10.argtypes = [vp, vp, vp]
+        lib.cfo_philox4x32_10.restype = None
+        lib.cfo_philox_uniform.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64]
+        lib.cfo_philox_uniform.restype = C.c_float
         lib.cfo_classic_forward_f64.argtypes = [vp, C.c_int, C.c_int] + [vp] * 9
         lib.cfo_forward_f32.argtypes = [vp, C.c_int, C.c_int, vp, vp, vp, vp, C.c_int]
         lib.cfo_max_threads.restype = C.c_int
@@ -266,6 +270,20 @@ class RefEnv:
 
     def close(self):
         ref().cfref_free()
+
+
+def philox4x32_10(ctr, key):
+    c = np.asarray(ctr, dtype=np.uint32); k = np.asarray(key, dtype=np.uint32)
+    out = np.zeros(4, dtype=np.uint32)
+    cfo().cfo_philox4x32_10(_p(c), _p(k), _p(out))
+    return out
+
+
+def philox_uniforms(seed, subsequences, offset):
+    """cfo_philox_uniform for one seed/offset over an array of subsequences."""
+    lib = cfo()
+    return np.array([lib.cfo_philox_uniform(int(seed), int(s), int(offset)) for s in subsequences],
+                    dtype=np.float32)
 
 
 def sample_actions(logits, u):

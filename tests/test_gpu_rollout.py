@@ -14,11 +14,11 @@ import numpy as np
 import pytest
 
 import oracle_bind as ob
-from parity_util import ACTIONS, HIDDEN, mix64, random_params, synth_records_host, unit24
+from parity_util import ACTIONS, HIDDEN, random_params, synth_records_host
 
 pytestmark = pytest.mark.gpu
 L = 3
-SALT = np.uint64(0xA5A5A5A5A5A5A5A5)
+SALT = 0xA5A5A5A5A5A5A5A5
 
 
 def _t(a, cuda):
@@ -27,7 +27,7 @@ def _t(a, cuda):
 
 
 def _uniforms(seed, step, n):
-    return unit24(mix64(np.uint64(seed) ^ SALT, step, np.arange(n, dtype=np.uint64)))
+    return ob.philox_uniforms(int(seed) ^ SALT, range(n), step)
 
 
 def _check_draws(av_h, act, lp, val, seed, step):

@@ -319,3 +319,38 @@ def test_sample_action_closed_forms():
     # frequencies on the grid equal the softmax probabilities to the grid resolution
     freq = np.bincount(acts, minlength=A) / len(grid)
     assert np.max(np.abs(freq - np.exp(ref_lp))) < 2.0 / len(grid) + 1e-6
+
+
+# ---- Philox4x32-10 (the reference's curandStatePhilox4_32_10_t) --------------------
+def test_philox_known_answer_vectors():
+    """The three known-answer vectors published with the generator (Random123
+    kat_vectors, "philox4x32 10": zero counter and key, all-ones, digits of pi).
+    A wrong multiplier, Weyl constant, round count or word order fails all twelve
+    words."""
+    kats = [
+        ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+        ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+        ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+         [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+    ]
+    for ctr, key, out in kats:
+        assert [int(x) for x in ob.philox4x32_10(ctr, key)] == out
+
+
+def test_philox_uniform_state_layout():
+    """cfo_philox_uniform against the block function: key = seed, counter low half =
+    offset / 4, high half = subsequence, word = offset % 4, uniform = x * 2^-32 +
+    2^-33 in (0, 1].  (That cuRAND lays its state out this way is taken from its
+    documentation: parity unpinned.)"""
+    seed, sub = 0x0123456789ABCDEF, (7 << 32) | 99
+    lib = ob.cfo()
+    for off in (0, 1, 2, 3, 4, 5, 11, (1 << 34) + 2):
+        words = ob.philox4x32_10([(off >> 2) & 0xffffffff, (off >> 2) >> 32, sub & 0xffffffff, sub >> 32],
+                                 [seed & 0xffffffff, seed >> 32])
+        x = np.float32(int(words[off & 3]))
+        expect = np.float32(np.float64(x) * 2.0 ** -32 + 2.0 ** -33)   # one rounding, like the fma
+        got = np.float32(lib.cfo_philox_uniform(seed, sub, off))
+        assert got == expect and 0.0 < got <= 1.0
+    u = ob.philox_uniforms(1234, range(20000), 5)
+    assert abs(u.mean() - 0.5) < 0.01 and abs(u.var() - 1.0 / 12.0) < 0.005
+    assert len(np.unique(u)) > 19900
