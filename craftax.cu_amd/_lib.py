@@ -26,6 +26,7 @@ PROTOTYPES = {
     "cfp_policy_layers": (C.c_int, [vp]),
     "cfp_policy_param_count": (C.c_size_t, [vp]),
     "cfp_policy_set_params": (C.c_int, [vp, vp, C.c_size_t]),
+    "cfp_policy_init_reference": (C.c_int, [vp, C.c_uint64]),
     "cfp_policy_get_params": (C.c_int, [vp, vp, C.c_size_t]),
     "cfp_policy_refresh_weights": (C.c_int, [vp, vp]),
     "cfp_save_weights": (C.c_int, [vp, C.c_char_p]),

@@ -176,6 +176,29 @@ int cfp_policy_set_params(cfp_policy* p, const float* host_params,
     return 0;
 }
 
+int cfp_policy_init_reference(cfp_policy* p, uint64_t seed) {
+    CFP_REQUIRE(p, "cfp_policy_init_reference: NULL policy");
+    const Arena ar = arena_of(p->variant, p->layers);
+    const float be = 1.0f / sqrtf((float)ar.obs);
+    const float bh = 1.0f / sqrtf((float)CFP_HIDDEN);
+    struct Seg { size_t off, count; float bound; };
+    const Seg segs[7] = {
+        {ar.w_enc, (size_t)ar.obs * CFP_HIDDEN, be},
+        {ar.b_enc, CFP_HIDDEN, be},
+        {ar.w_gru, (size_t)p->layers * CFP_GRU * CFP_HIDDEN, bh},
+        {ar.w_a, (size_t)ar.actions * CFP_HIDDEN, bh},
+        {ar.b_a, (size_t)ar.actions, bh},
+        {ar.w_v, CFP_HIDDEN, bh},
+        {ar.b_v, 1, bh},
+    };
+    std::vector<float> w(p->param_count);
+    for (int s = 0; s < 7; s++)
+        for (size_t i = 0; i < segs[s].count; i++)
+            w[segs[s].off + i] =
+                (2.0f * philox_uniform(seed, (uint64_t)s, (uint64_t)i) - 1.0f) * segs[s].bound;
+    return cfp_policy_set_params(p, w.data(), w.size());
+}
+
 int cfp_policy_get_params(const cfp_policy* p, float* host_params,
                           size_t count) {
     CFP_REQUIRE(p && host_params, "cfp_policy_get_params: NULL argument");

@@ -101,6 +101,10 @@ class Policy:
         a = np.ascontiguousarray(host_params, dtype=np.float32)
         _check(lib().cfp_policy_set_params(self._h, a.ctypes.data_as(C.c_void_p), a.size))
 
+    def init_reference(self, seed=1234):
+        """The reference's weight initialisation (cu_policy_init :11830-11845)."""
+        _check(lib().cfp_policy_init_reference(self._h, int(seed)))
+
     def get_params(self):
         a = np.empty(self.param_count, dtype=np.float32)
         _check(lib().cfp_policy_get_params(self._h, a.ctypes.data_as(C.c_void_p), a.size))

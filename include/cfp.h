@@ -97,6 +97,16 @@ size_t cfp_policy_param_count(const cfp_policy* p);
  * craftax_full.cu:12248/12264).  set_params also rebuilds the mirrors. */
 int cfp_policy_set_params(cfp_policy* p, const float* host_params, size_t count);
 int cfp_policy_get_params(const cfp_policy* p, float* host_params, size_t count);
+/* The reference's own initialisation (cu_policy_init, craftax_full.cu:11830-11845 with
+ * k_nn_init_weights :9123-9131; main_classic.cu:366-374 for the classic game): the seven
+ * arena segments s = 0..6 (W_enc, b_enc, W_gru, W_a, b_a, W_v, b_v) filled with
+ * (2u - 1) * bound, bound = 1/sqrt(obs) for the first two and 1/sqrt(256) for the
+ * rest, u = the first curand_uniform of a Philox4_32_10 state after
+ * curand_init(seed, s, i) (the reference passes seed 1234).  Replaces the
+ * Xavier-uniform weights cfp_policy_create made and refreshes the mirrors.  The
+ * Philox block function is checked against published vectors; cuRAND's mapping of
+ * (seed, subsequence, offset) onto it is taken from its documentation. */
+int cfp_policy_init_reference(cfp_policy* p, uint64_t seed);
 /* Rebuild the MFMA-ordered weight mirrors from the params arena after the
  * arena changed on device: the role of cu_params_refresh_bf16 + cu_pack_wav
  * (craftax_full.cu:11805-11817) after init / Adam. */

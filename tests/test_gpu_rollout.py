@@ -142,3 +142,41 @@ def test_rollout_step_and_bootstrap(pkg, cuda):
     assert torch.equal(pol.state, live_before)
     assert torch.equal(tr.buf("v_boot"), av[:, ACTIONS])
     tr.close(); pol.close(); twin.close()
+
+
+@pytest.mark.parametrize("classic", [False, True])
+def test_reference_weight_init(pkg, cuda, classic):
+    """cfp_policy_init_reference: segment s, element i = (2u - 1) * bound with u the
+    Philox uniform of (seed, subsequence s, offset i) -- checked against the oracle's
+    restatement at the segment boundaries and on a random sample, plus the bounds
+    and the uniform's moments per segment; the forward then runs on these weights."""
+    import torch
+    n = 64
+    pol = pkg.Policy(n, L, seed=1, variant="classic" if classic else "full")
+    before = pol.get_params()
+    pol.init_reference(1234)
+    w = pol.get_params()
+    assert not np.array_equal(w, before)
+    obs, actions = (1345, 17) if classic else (843, 43)
+    be, bh = np.float32(1.0) / np.sqrt(np.float32(obs)), np.float32(1.0) / np.sqrt(np.float32(256))
+    counts = [obs * 256, 256, L * 768 * 256, actions * 256, actions, 256, 1]
+    bounds = [be, be, bh, bh, bh, bh, bh]
+    assert sum(counts) == w.size
+    rng = np.random.default_rng(3)
+    off = 0
+    lib = ob.cfo()
+    for s, (cnt, b) in enumerate(zip(counts, bounds)):
+        seg = w[off:off + cnt]
+        assert np.all(np.abs(seg) <= b)
+        idx = np.unique(np.concatenate([[0, cnt - 1], rng.integers(0, cnt, 64)]))
+        for i in idx:
+            u = np.float32(lib.cfo_philox_uniform(1234, s, int(i)))
+            assert seg[i] == (np.float32(2.0) * u - np.float32(1.0)) * np.float32(b), (s, i)
+        if cnt >= 4096:
+            assert abs(seg.mean()) < 0.05 * b and abs(seg.var() / (b * b / 3.0) - 1.0) < 0.05
+        off += cnt
+    rec = (pkg.policy.synth_classic_records(n, 3, 0) if classic else pkg.policy.synth_records(n, 3, 0))
+    av = pol.forward(rec, torch.zeros(n, device=cuda), pol.state)
+    torch.cuda.synchronize()
+    assert torch.isfinite(av).all()
+    pol.close()
