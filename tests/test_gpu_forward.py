@@ -215,11 +215,13 @@ def test_reference_rollout_slice(pkg, cuda, golden):
 
 @pytest.mark.skipif(not ob.have_ref(), reason="oracle/_ref not built (no reference source)")
 def test_config1_live_reference_env(pkg, cuda):
-    """Config 1 plumbing on the box: the compiled reference env (1024 envs, seed 0,
-    xorshift32 % 43 actions) feeds the device policy for 200 steps; every 20th
-    step is checked one-step against the oracle from the device's own state."""
+    """Config 1 in full on the box: the compiled reference env (1024 envs, seed 0,
+    xorshift32 % 43 actions) feeds the device policy for 2000 steps, state carried and
+    zeroed after terminals; during the first 200 steps every 20th step and every step
+    with a terminal, afterwards every 50th step, is checked one-step against the
+    oracle from the device's own state."""
     import torch
-    n, T = 1024, 200
+    n, T = 1024, 2000
     env = ob.RefEnv(n, 0)
     pol = pkg.Policy(n, L, seed=1)
     params = pol.get_params()
@@ -230,7 +232,7 @@ def test_config1_live_reference_env(pkg, cuda):
             rec_h = env.records()
             term_h = env.terminals() if t else np.zeros(n, np.float32)
             n_term += int((term_h != 0).sum())
-            check = (t % 20 == 0) or (term_h != 0).any()
+            check = (t % 20 == 0 or (term_h != 0).any()) if t < 200 else t % 50 == 0
             if check:
                 st_in = state.cpu().numpy().copy()
             av = pol.forward(_t(rec_h, cuda), _t(term_h, cuda), state)
@@ -240,6 +242,7 @@ def test_config1_live_reference_env(pkg, cuda):
                 assert_close(av.cpu().numpy()[:, ACTIONS], ref["values"], TOL_FP32, f"t={t} values")
                 assert_close(state.cpu().numpy(), ref["state"], TOL_FP32, f"t={t} state")
             env.step()
+        assert n_term > 0, "no episode ended: the terminal path was not exercised"
     finally:
         env.close()
         pol.close()

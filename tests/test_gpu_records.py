@@ -155,3 +155,35 @@ def test_synth_records_device_equals_host(pkg, cuda):
         d = pkg.policy.synth_records(n, seed, step)
         torch.cuda.synchronize()
         assert np.array_equal(d.cpu().numpy(), synth_records_host(n, seed, step))
+
+
+@pytest.mark.skipif(not ob.have_ref(), reason="oracle/_ref not built (no reference source)")
+def test_record_obs_live_reference_env(pkg, cuda):
+    """State -> record on the device against the compiled reference env itself: 256 envs
+    (seed 7, the harness's xorshift32 % 43 actions) stepped 600 times; every 40th step
+    the encoder-input state of every env goes through k_record_obs and must equal the
+    996-byte record the reference wrote for that env, bit for bit.  Fresh states on
+    every run of the box, beyond the committed fixtures (mobs, darkness, deeper levels
+    and post-reset states all occur within these steps)."""
+    import torch
+    n = 256
+    env = ob.RefEnv(n, 7)
+    try:
+        checked = 0
+        for t in range(601):
+            if t % 40 == 0:
+                want = env.records()
+                views = [env.view(e) for e in range(n)]
+                sc = np.stack([v[0] for v in views])
+                pl = np.stack([v[1] for v in views]).reshape(n, 3, P)
+                base = _t(pl, cuda).view(-1)
+                rec = pkg.policy.record_obs(_t(sc, cuda), base, base[P:], base[2 * P:], n, 3 * P, 0)
+                torch.cuda.synchronize()
+                got = rec.cpu().numpy()
+                bad = np.nonzero((got != want).any(axis=1))[0]
+                assert bad.size == 0, f"step {t}: {bad.size} of {n} records differ, first {bad[:5]}"
+                checked += n
+            env.step()
+        assert checked == 16 * n
+    finally:
+        env.close()
