@@ -30,7 +30,6 @@ __device__ __forceinline__ void copy_tile_out(const float* lds, float* dst,
                                               int tid) {
     const f4* xs4 = reinterpret_cast<const f4*>(lds);
     f4* d4 = reinterpret_cast<f4*>(dst);
-#pragma unroll
     for (int i = tid; i < kTileEnvs * CFP_HIDDEN / 4; i += kFwdThreads)
         d4[i] = xs4[(i >> 6) * XS4 + (i & 63)];
 }
