@@ -4,6 +4,8 @@
                   (fp32 and bf16-input kernels)
   ppo_update      PPO update, 4096 envs x 64 steps = 262 144 samples, one
                   minibatch = all envs: windowed recompute backward + Adam
+  rollout_policy_side  forward in recording mode + sampling + reward/done rows per
+                  step at 4096 .. 262 144 envs (the policy half of cu_rollout_step)
   classic_1m      classic-game policy forward, 1 048 576 envs, 148-byte records
   record_kernels  the HBM-bound byte kernels at 65 536 envs: state -> 996-byte
                   records (fuzzed reference states of tests/golden, tiled) and
@@ -105,6 +107,38 @@ def ppo_update(pkg, torch, reps):
     return out
 
 
+def rollout_policy_side(pkg, torch, reps):
+    """The policy half of the reference's rollout step (cu_rollout_step + k_record_rd):
+    record -> fused forward on the live state with the r_obs / r_state rows written ->
+    categorical sampling (Philox) into r_act / r_logprob / r_value and the env's action
+    slots -> reward/done rows; T = 8 steps per round of slabs, state carried.  The env
+    step itself is not part of this library."""
+    out = {"workload": "rollout_policy_side", "steps_per_round": 8, "sizes": {}}
+    T = 8
+    for n in (4096, 8192, 65536, 262144):
+        pol = pkg.Policy(n, 3, seed=1)
+        tr = pkg.Trainer(pol, T)
+        # as in the reference, the records of step t are produced straight into the slab
+        # row r_obs[t] (k_record_obs writes there), so the step makes no copy of them
+        r_obs = tr.buf("r_obs")
+        recs = [pkg.policy.synth_records(n, 99, t, rec=r_obs[t]) for t in range(T)]
+        term = (torch.rand(n, device="cuda") < 0.0025).float()
+        rew = torch.rand(n, device="cuda")
+        acts = torch.empty(n, device="cuda")
+        r_rew, r_done = tr.buf("r_reward"), tr.buf("r_done")
+
+        def round_():
+            for t in range(T):
+                tr.rollout_step(t, recs[t], term, 1234, env_actions=acts)
+                pkg.policy.record_rd(rew, term, r_rew[t], r_done[t])
+        ms = _time(torch, round_, max(2, reps // 2), warm=1) / T
+        out["sizes"][str(n)] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
+                                "frac_fp32_mfma_peak": FWD_FLOP * n / ms / 1e9 / PEAK_FP32}
+        tr.close()
+        pol.close()
+    return out
+
+
 def classic_1m(pkg, torch, reps):
     n = 1 << 20
     pol = pkg.Policy(n, 3, seed=1, variant="classic")
@@ -170,7 +204,7 @@ def main():
     import __graft_entry__ as ge
     pkg = ge.load_package()
     assert torch.cuda.is_available(), "bench_configs.py needs a GPU"
-    for fn in (forward_65536, ppo_update, classic_1m, record_kernels):
+    for fn in (forward_65536, ppo_update, rollout_policy_side, classic_1m, record_kernels):
         if args.only and fn.__name__ != args.only:
             continue
         print(json.dumps(fn(pkg, torch, args.reps)), flush=True)

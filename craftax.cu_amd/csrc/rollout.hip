@@ -19,28 +19,51 @@ namespace {
 
 constexpr int kMaxActions = 64;
 
-__global__ void k_value_sample(const float* __restrict__ av, int avs, int actions,
-                               float* __restrict__ env_actions, int32_t* __restrict__ act,
-                               float* __restrict__ logprobs, float* __restrict__ values, int n,
-                               uint64_t seed, const uint64_t* __restrict__ step_ctr) {
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n) return;
-    const float* lp = av + (size_t)e * avs;
+// Sixteen lanes per env, sixteen envs per workgroup.  The workgroup's logits rows are
+// one contiguous piece of av and are staged through LDS with coalesced loads (a thread
+// walking its own 176-byte row straight from memory touches 64 different lines per
+// load instruction).  The order-independent parts -- the maximum and the
+// exponentials -- are spread over the env's lanes; the two sums, whose rounding
+// depends on their order, are then run by one lane in the reference's ascending
+// order over the exponentials in LDS, so the draw is the sequential kernel's bit for bit.
+constexpr int kSampleLanes = 16;
+constexpr int kSampleEnvs = 256 / kSampleLanes;
+
+__global__ __launch_bounds__(256) void k_value_sample(
+    const float* __restrict__ av, int avs, int actions, float* __restrict__ env_actions,
+    int32_t* __restrict__ act, float* __restrict__ logprobs, float* __restrict__ values, int n,
+    uint64_t seed, const uint64_t* __restrict__ step_ctr) {
+    __shared__ float logit[kSampleEnvs * (kMaxActions + 1)];
+    __shared__ float expo[kSampleEnvs * kMaxActions];
+    const int e0 = (int)blockIdx.x * kSampleEnvs;
+    const int nb = n - e0 < kSampleEnvs ? n - e0 : kSampleEnvs;
+    const float* src = av + (size_t)e0 * avs;
+    for (int i = threadIdx.x; i < nb * avs; i += 256) logit[i] = src[i];
+    __syncthreads();
+    const int sub = threadIdx.x % kSampleLanes, slot = threadIdx.x / kSampleLanes;
+    const bool live = slot < nb;
+    const float* lp = logit + slot * avs;
+    float* px = expo + slot * kMaxActions;
+    float m = -INFINITY;
+    if (live)
+        for (int a = sub; a < actions; a += kSampleLanes) m = fmaxf(m, lp[a]);
+#pragma unroll
+    for (int d = kSampleLanes / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, kSampleLanes));
+    if (live)
+        for (int a = sub; a < actions; a += kSampleLanes) px[a] = expf(lp[a] - m);
+    __syncthreads();
+    if (!live || sub != 0) return;
+    const int e = e0 + slot;
     if (values) values[e] = lp[actions];
-    float m = lp[0];
-    for (int a = 1; a < actions; a++) m = fmaxf(m, lp[a]);
-    float p[kMaxActions], total = 0.0f;
-    for (int a = 0; a < actions; a++) {
-        p[a] = expf(lp[a] - m);
-        total += p[a];
-    }
+    float total = 0.0f;
+    for (int a = 0; a < actions; a++) total += px[a];
     const uint64_t step = step_ctr ? *step_ctr : 0;
     const float u = philox_uniform(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)e, step);
     const float target = u * total;
     float cum = 0.0f;
     int action = actions - 1;
     for (int a = 0; a < actions; a++) {
-        cum += p[a];
+        cum += px[a];
         if (target <= cum) { action = a; break; }
     }
     if (env_actions) env_actions[e] = (float)action;
@@ -70,7 +93,8 @@ int cfp_value_sample(const float* d_av, int n, int actions, float* d_env_actions
     CFP_REQUIRE(d_av && d_actions && d_logprobs && n > 0, "cfp_value_sample: bad argument");
     CFP_REQUIRE(actions > 0 && actions <= kMaxActions, "cfp_value_sample: actions must be in 1..%d",
                 kMaxActions);
-    hipLaunchKernelGGL(k_value_sample, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+    hipLaunchKernelGGL(k_value_sample, dim3((n + kSampleEnvs - 1) / kSampleEnvs), dim3(256), 0,
+                       (hipStream_t)stream,
                        d_av, actions + 1, actions, d_env_actions, d_actions, d_logprobs, d_values,
                        n, seed, d_step_ctr);
     CFP_HIP_TRY(hipGetLastError());
