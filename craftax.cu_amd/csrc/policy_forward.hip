@@ -164,6 +164,7 @@ __device__ __forceinline__ void vm_wait(int n) {
 // pipe") are streamed like the gate weights: K block kb+3 requested into the ring
 // and block kb+1 read back while block kb multiplies.  Its 16-byte elements and its
 // 6 KiB per wave and block are those of the gate mirror, so ring_dma serves both.
+template <bool ONE>
 __device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const float* ldsX,
                                                         const float* ldsY, f4* ring,
                                                         const Lane& L, f16v (&acc)[4]) {
@@ -208,7 +209,7 @@ __device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const 
             ax = u4{0u, 0u, 0u, 0u};
             ay = u4{0u, 0u, 0u, 0u};
         }
-        encs_mma(acc, ax, ay, bl[cb]);
+        encs_mma<ONE>(acc, ax, ay, bl[cb]);
         cur = nxt;
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -222,8 +223,10 @@ __device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const 
             const float x = fx[8 * t + j], y = fy[8 * t + j];
             acc[0] = mfma(x, tb0[t][j], acc[0]);
             acc[1] = mfma(x, tb1[t][j], acc[1]);
-            acc[2] = mfma(y, tb0[t][j], acc[2]);
-            acc[3] = mfma(y, tb1[t][j], acc[3]);
+            if (!ONE) {
+                acc[2] = mfma(y, tb0[t][j], acc[2]);
+                acc[3] = mfma(y, tb1[t][j], acc[3]);
+            }
         }
     }
 }
@@ -525,11 +528,11 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
                 classic_prepare<kClsEnvs>(cbase, tid);
                 classic_encoder_gemm(a, cbase, ring, L, eacc);
             } else {
-                encoder_gemm_split_ring(a, lds_all[0], lds_all[1], ring, L, eacc);
+                encoder_gemm_split_ring<SINGLE>(a, lds_all[0], lds_all[1], ring, L, eacc);
             }
             __syncthreads();   // every wave is done with the record bytes / tables
 #pragma unroll
-            for (int s = 0; s < 2; s++)
+            for (int s = 0; s < (SINGLE ? 1 : 2); s++)
 #pragma unroll
                 for (int ut = 0; ut < 2; ut++) {
                     const float bias = a.b_enc[L.wave * 64 + ut * 32 + L.l32];
@@ -669,12 +672,12 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     hacc[0] = mfma(ax[j], hb[i][j], hacc[0]);
-                    hacc[1] = mfma(ay[j], hb[i][j], hacc[1]);
+                    if (!SINGLE) hacc[1] = mfma(ay[j], hb[i][j], hacc[1]);
                 }
             }
             if (kh == 1) {
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
+                for (int s = 0; s < (SINGLE ? 1 : 2); s++) {
                     float* red = red_all[s] + (nt * 16) * 64 + L.lane_u;
 #pragma unroll
                     for (int r = 0; r < 16; r++) red[r * 64] = hacc[s][r];

@@ -288,6 +288,8 @@ __device__ __forceinline__ EncDw encs_bytes(const uint32_t* rx, const uint32_t* 
     return r;
 }
 
+// ONE: the second tile does not exist (one tile per workgroup); its products are left out.
+template <bool ONE = false>
 __device__ __forceinline__ void encs_mma(f16v (&acc)[4], const u4& ax, const u4& ay,
                                          const EncS& w) {
 #pragma unroll
@@ -295,7 +297,7 @@ __device__ __forceinline__ void encs_mma(f16v (&acc)[4], const u4& ax, const u4&
 #pragma unroll
         for (int ut = 0; ut < 2; ut++) {
             acc[ut] = mfma16(ax, w.b[3 * ut + s], acc[ut]);
-            acc[2 + ut] = mfma16(ay, w.b[3 * ut + s], acc[2 + ut]);
+            if (!ONE) acc[2 + ut] = mfma16(ay, w.b[3 * ut + s], acc[2 + ut]);
         }
 }
 
