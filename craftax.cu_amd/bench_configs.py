@@ -134,6 +134,17 @@ def rollout_policy_side(pkg, torch, reps):
         ms = _time(torch, round_, max(2, reps // 2), warm=1) / T
         out["sizes"][str(n)] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
                                 "frac_fp32_mfma_peak": FWD_FLOP * n / ms / 1e9 / PEAK_FP32}
+        if n <= 8192:
+            # the same round captured once into a graph and replayed, as the reference does
+            # with its rollout (the device step counter keeps the draws fresh)
+            side = torch.cuda.Stream()
+            with torch.cuda.stream(side):
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=side):
+                    round_()
+                ms_g = _time(torch, graph.replay, max(2, reps // 2), warm=1) / T
+            out["sizes"][str(n)]["graph_replay_ms_per_step"] = ms_g
+            del graph
         tr.close()
         pol.close()
     return out
