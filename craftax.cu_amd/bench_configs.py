@@ -4,6 +4,8 @@
                   (fp32 and bf16-input kernels)
   ppo_update      PPO update, 4096 envs x 64 steps = 262 144 samples, one
                   minibatch = all envs: windowed recompute backward + Adam
+  ppo_update_shapes    the update iteration (cfp_train_update, eager and graph) at
+                  other horizons, env counts, minibatch and epoch settings
   rollout_policy_side  forward in recording mode + sampling + reward/done rows per
                   step at 4096 .. 262 144 envs (the policy half of cu_rollout_step)
   classic_1m      classic-game policy forward, 1 048 576 envs, 148-byte records
@@ -104,6 +106,37 @@ def ppo_update(pkg, torch, reps):
     assert torch.isfinite(pol.params).all()
     tr.close()
     pol.close()
+    return out
+
+
+def ppo_update_shapes(pkg, torch, reps):
+    """cfp_train_update (epochs x minibatches x (backward, Adam)) at other shapes than
+    config 4, eager and as the library's captured graph."""
+    out = {"workload": "ppo_update_shapes", "shapes": []}
+    for n, T, cfg in ((4096, 128, {}), (8192, 64, {}), (4096, 64, {"minibatches": 4}),
+                      (1024, 128, {"epochs": 2}), (4096, 64, {"bptt_split": 4})):
+        pol = pkg.Policy(n, 3, seed=1)
+        tr = pkg.Trainer(pol, T, **cfg)
+        pol.state.zero_()
+        term = torch.zeros(n, device="cuda")
+        for t in range(T):
+            tr.record_step(t, pkg.policy.synth_records(n, 1234, t), term)
+        g = torch.Generator(device="cuda").manual_seed(7)
+        tr.buf("r_act").copy_(torch.randint(0, 43, (T, n), device="cuda", generator=g, dtype=torch.int32))
+        tr.buf("r_logprob").fill_(-3.7612)
+        tr.buf("adv").copy_(torch.randn(T, n, device="cuda", generator=g))
+        tr.buf("ret").copy_(torch.randn(T, n, device="cuda", generator=g))
+        tr.buf("r_done").zero_()
+        tr.adv_stats()
+        row = {"envs": n, "T": T, **cfg, "window": tr.window, "minibatch": tr.mb}
+        for key, use_graph in (("eager", False), ("graph", True)):
+            ms = _time(torch, lambda: tr.update(use_graph=use_graph), max(2, reps // 3), warm=1)
+            row[key] = {"ms_per_iteration": ms,
+                        "samples_per_s": n * T * cfg.get("epochs", 1) / ms * 1e3}
+        assert torch.isfinite(pol.params).all()
+        out["shapes"].append(row)
+        tr.close()
+        pol.close()
     return out
 
 
@@ -215,7 +248,8 @@ def main():
     import __graft_entry__ as ge
     pkg = ge.load_package()
     assert torch.cuda.is_available(), "bench_configs.py needs a GPU"
-    for fn in (forward_65536, ppo_update, rollout_policy_side, classic_1m, record_kernels):
+    for fn in (forward_65536, ppo_update, ppo_update_shapes, rollout_policy_side, classic_1m,
+               record_kernels):
         if args.only and fn.__name__ != args.only:
             continue
         print(json.dumps(fn(pkg, torch, args.reps)), flush=True)
