@@ -187,3 +187,33 @@ def test_record_obs_live_reference_env(pkg, cuda):
         assert checked == 16 * n
     finally:
         env.close()
+
+
+@pytest.mark.skipif(not ob.have_ref(), reason="oracle/_ref not built (no reference source)")
+def test_record_obs_live_fuzzed_states(pkg, cuda):
+    """2048 freshly fuzzed states of the compiled reference (edge positions, every level,
+    random mobs of every class on lit and dark cells, full inventories; seeds other than
+    the committed fixtures') through k_record_obs in batches of 256, against the
+    reference's own encoder on the same state, bit for bit."""
+    import torch
+    n = 256
+    env = ob.RefEnv(n, 3)
+    try:
+        for rnd in range(8):
+            want = np.empty((n, 996), dtype=np.uint8)
+            scs, pls = [], []
+            for e in range(n):
+                env.fuzz(e, 500000 + rnd * n + e)
+                sc, pl = env.view(e)
+                scs.append(sc); pls.append(pl)
+                want[e] = env.encode(e)
+            base = _t(np.stack(pls).reshape(n, 3, P), cuda).view(-1)
+            rec = pkg.policy.record_obs(_t(np.stack(scs), cuda), base, base[P:], base[2 * P:], n, 3 * P, 0)
+            torch.cuda.synchronize()
+            got = rec.cpu().numpy()
+            bad = np.nonzero((got != want).any(axis=1))[0]
+            assert bad.size == 0, f"round {rnd}: {bad.size} records differ, first seeds {500000 + rnd * n + bad[:5]}"
+            mobs = (want[:, :792].reshape(n, 99, 8)[:, :, 3:] != 0).sum()
+            assert mobs > 0, "the fuzzed states put no mob into view"
+    finally:
+        env.close()
