@@ -71,6 +71,56 @@ __global__ __launch_bounds__(256) void k_value_sample(
     logprobs[e] = lp[action] - m - logf(total);
 }
 
+// Large batches: one thread per env, 128 envs per workgroup (every lane busy through
+// the sums; the sixteen-lane form above leaves fifteen of sixteen idle there and wins
+// only while the launch is too small to fill the machine).  Same staging, rows of an
+// odd stride so that the threads' rows start in different banks; the exponentials
+// replace the logits in the row.  Same operations in the same order: same bits.
+constexpr int kSampleRowEnvs = 128;
+
+__global__ __launch_bounds__(kSampleRowEnvs) void k_value_sample_rows(
+    const float* __restrict__ av, int avs, int actions, float* __restrict__ env_actions,
+    int32_t* __restrict__ act, float* __restrict__ logprobs, float* __restrict__ values, int n,
+    uint64_t seed, const uint64_t* __restrict__ step_ctr) {
+    __shared__ float rows[kSampleRowEnvs * (kMaxActions + 1)];
+    const int stride = avs | 1;
+    const int e0 = (int)blockIdx.x * kSampleRowEnvs;
+    const int nb = n - e0 < kSampleRowEnvs ? n - e0 : kSampleRowEnvs;
+    const float* src = av + (size_t)e0 * avs;
+    const float inv = 1.0f / (float)avs;
+    for (int i = threadIdx.x; i < nb * avs; i += kSampleRowEnvs) {
+        // i / avs through the reciprocal: (i + 0.5) / avs keeps 0.5 / avs away from every
+        // integer, far more than the rounding of this product for i < 2^14
+        const int row = (int)(((float)i + 0.5f) * inv);
+        rows[row * stride + (i - row * avs)] = src[i];
+    }
+    __syncthreads();
+    const int e = e0 + (int)threadIdx.x;
+    if (e >= n) return;
+    float* lp = rows + threadIdx.x * stride;
+    if (values) values[e] = lp[actions];
+    float m = lp[0];
+    for (int a = 1; a < actions; a++) m = fmaxf(m, lp[a]);
+    float total = 0.0f;
+    for (int a = 0; a < actions; a++) {
+        const float p = expf(lp[a] - m);
+        lp[a] = p;
+        total += p;
+    }
+    const uint64_t step = step_ctr ? *step_ctr : 0;
+    const float u = philox_uniform(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)e, step);
+    const float target = u * total;
+    float cum = 0.0f;
+    int action = actions - 1;
+    for (int a = 0; a < actions; a++) {
+        cum += lp[a];
+        if (target <= cum) { action = a; break; }
+    }
+    if (env_actions) env_actions[e] = (float)action;
+    act[e] = action;
+    logprobs[e] = av[(size_t)e * avs + action] - m - logf(total);
+}
+
 __global__ void k_record_rd(const float* __restrict__ rewards, const float* __restrict__ terminals,
                             float* __restrict__ r_reward_row, uint8_t* __restrict__ r_done_row,
                             int n) {
@@ -93,10 +143,14 @@ int cfp_value_sample(const float* d_av, int n, int actions, float* d_env_actions
     CFP_REQUIRE(d_av && d_actions && d_logprobs && n > 0, "cfp_value_sample: bad argument");
     CFP_REQUIRE(actions > 0 && actions <= kMaxActions, "cfp_value_sample: actions must be in 1..%d",
                 kMaxActions);
-    hipLaunchKernelGGL(k_value_sample, dim3((n + kSampleEnvs - 1) / kSampleEnvs), dim3(256), 0,
-                       (hipStream_t)stream,
-                       d_av, actions + 1, actions, d_env_actions, d_actions, d_logprobs, d_values,
-                       n, seed, d_step_ctr);
+    if (n >= 16384)
+        hipLaunchKernelGGL(k_value_sample_rows, dim3((n + kSampleRowEnvs - 1) / kSampleRowEnvs),
+                           dim3(kSampleRowEnvs), 0, (hipStream_t)stream, d_av, actions + 1, actions,
+                           d_env_actions, d_actions, d_logprobs, d_values, n, seed, d_step_ctr);
+    else
+        hipLaunchKernelGGL(k_value_sample, dim3((n + kSampleEnvs - 1) / kSampleEnvs), dim3(256), 0,
+                           (hipStream_t)stream, d_av, actions + 1, actions, d_env_actions,
+                           d_actions, d_logprobs, d_values, n, seed, d_step_ctr);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }

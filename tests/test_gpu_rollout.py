@@ -43,7 +43,8 @@ def _check_draws(av_h, act, lp, val, seed, step):
     assert np.array_equal(val, av_h[:, A])
 
 
-@pytest.mark.parametrize("n,A,scale", [(4096, 43, 1.0), (1000, 43, 6.0), (2048, 17, 2.0)])
+@pytest.mark.parametrize("n,A,scale", [(4096, 43, 1.0), (1000, 43, 6.0), (2048, 17, 2.0),
+                                       (16384 + 37, 43, 3.0), (20000, 17, 2.0)])
 def test_value_sample_matches_restatement(pkg, cuda, n, A, scale):
     import torch
     rng = np.random.default_rng(n + A)
@@ -63,6 +64,22 @@ def test_value_sample_matches_restatement(pkg, cuda, n, A, scale):
     torch.cuda.synchronize()
     assert torch.equal(act, act2) and not torch.equal(act, act3)
     _check_draws(av_h, act0.cpu().numpy(), lp0.cpu().numpy(), val0.cpu().numpy(), 1234, 0)
+
+
+def test_value_sample_both_kernels_agree(pkg, cuda):
+    """Batches below 16 384 envs run sixteen lanes per env, larger ones one thread per env;
+    both do the order-dependent sums in ascending order, so env e of a large launch draws
+    what env e of a small launch over the same rows draws, bit for bit."""
+    import torch
+    for A in (43, 17):
+        n = 16384 + 517
+        av = _t((2.5 * np.random.default_rng(A).standard_normal((n, A + 1))).astype(np.float32), cuda)
+        ctr = torch.tensor([11], dtype=torch.int64, device=cuda)
+        act_l, lp_l, val_l = pkg.policy.value_sample(av, 77, step_ctr=ctr)
+        act_s, lp_s, val_s = pkg.policy.value_sample(av[:4096].contiguous(), 77, step_ctr=ctr)
+        torch.cuda.synchronize()
+        assert torch.equal(act_l[:4096], act_s) and torch.equal(lp_l[:4096], lp_s)
+        assert torch.equal(val_l[:4096], val_s)
 
 
 def test_value_sample_distribution(pkg, cuda):
