@@ -112,8 +112,8 @@ constexpr int kRingF4 = 4 * kRingSlots * kRingSlotF4;     // 72 KiB for the work
 // K block kb of a layer (wp = mirror + layer + wave*6*64 fragments) -> ring slot.
 // `after` is a register the slot's previous contents were last read into: as an
 // operand it keeps the request behind the completion of those reads.  M0 (the LDS
-// base of an LDS-direct load) is reserved: the compiler neither allocates it nor,
-// in this file, uses it for anything else.
+// base of an LDS-direct load) is written by each block and declared as clobbered,
+// so the compiler keeps nothing of its own in it across a request.
 __device__ __forceinline__ void ring_dma(const f4* wp, int kb, f4* slot, const Lane& L,
                                          float after = 0.0f) {
     constexpr int KB_STRIDE = 4 * 6 * 64;
@@ -129,7 +129,7 @@ __device__ __forceinline__ void ring_dma(const f4* wp, int kb, f4* slot, const L
         "global_load_lds_dwordx4 %0, %1 offset:3072"
         :
         : "v"(voff), "s"(src), "s"(lds_lo), "v"(after)
-        : "memory");
+        : "memory", "m0");
     asm volatile(
         "s_mov_b32 m0, %2\n\t"
         "s_nop 0\n\t"
@@ -137,7 +137,7 @@ __device__ __forceinline__ void ring_dma(const f4* wp, int kb, f4* slot, const L
         "global_load_lds_dwordx4 %0, %1 offset:1024"
         :
         : "v"(voff), "s"(src + 4 * 64), "s"(lds_lo + 4096u)
-        : "memory");
+        : "memory", "m0");
 }
 
 // First three K blocks of a layer's weights into ring slots 0, 1, 2.

@@ -1,31 +1,23 @@
 // On-device PPO update: rollout slabs, windowed recompute backward, GAE,
 // Adam.  Host-side mirror of the reference's CuTrain layer
-// (craftax_full.cu:12637-13480); kernels follow
-//   k_mingru_epi_replay_win :9460   k_head_bwd_win      :9603
-//   k_mingru_window_bwd     :9510   k_colsum / 256 / small  :10442
-//   (k_add_dv_wv :10224 is folded into the top layer's reverse kernel, k_vadd
-//    :10069 into the layer-0 dh GEMM, which accumulates onto the highway term)
-//   k_gae :10617  k_adv_stats :10638  k_adam :10668  k_loss_accum :10508
-// The GEMMs go through the fp32 MFMA seam in gemm.hip.  All reductions are
-// done in a fixed order (no float atomics), so a backward pass is bitwise
-// reproducible run to run.
+// (craftax_full.cu:12637-13480).  The streaming kernels (reverse MinGRU sweep, head
+// gradients, GAE, Adam) live in ppo_kernels.hip, the GEMMs behind the seam of
+// gemm.hip / gemm_x9.hip; here: the window loop, the two-stream schedule, graph
+// capture and the column sums (the reference's k_colsum family, :10442).
+//   k_add_dv_wv :10224 is folded into the head's 48-wide gradient rows, k_vadd
+//   :10069 into the layer-0 dh GEMM, which accumulates onto the highway term.
+// All reductions are done in a fixed order (no float atomics), so a backward pass
+// is bitwise reproducible run to run.
 #include <vector>
 
 #include "cfp_common.h"
 #include "cfp_internal.h"
+#include "ppo_kernels.h"
 
 namespace cfp {
 namespace {
 
 constexpr int H = CFP_HIDDEN, G = CFP_GRU, A = CFP_ACTIONS;
-
-__device__ __forceinline__ float sigm(float z) { return 1.0f / (1.0f + expf(-z)); }
-__device__ __forceinline__ float gfun(float z) { return z >= 0.0f ? z + 0.5f : sigm(z); }
-__device__ __forceinline__ float dgfun(float z) {
-    if (z >= 0.0f) return 1.0f;
-    const float s = sigm(z);
-    return s * (1.0f - s);
-}
 
 __global__ void k_fill(float* p, size_t count, float v) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -35,149 +27,18 @@ __global__ void k_fill_f64(double* p, int count) {
     if ((int)threadIdx.x < count) p[threadIdx.x] = 0.0;
 }
 
-// Window recompute epilogue: column w = (t0 + w/mb, env_start + w%mb) reloads
-// the stored post-zero state for every step (no live carry).
-__global__ void k_mingru_epi_replay_win(const float* __restrict__ pre,
-                                        const float* __restrict__ x,
-                                        const float* __restrict__ r_state,
-                                        float* __restrict__ x_next, int t0,
-                                        size_t total, int mb, int n,
-                                        int env_start, int layer, int layers) {
-    size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int k = (int)(idx & (H - 1));
-    const size_t w = idx / H;
-    const size_t tr = w / (size_t)mb;
-    const size_t el = w - tr * (size_t)mb;
-    const size_t t = (size_t)t0 + tr;
-    const size_t rs = ((t * layers + layer) * (size_t)n + env_start + el) * H + k;
-    const float st = r_state[rs];
-    const size_t o3 = w * G + k;
-    const float zh = pre[o3], zg = pre[o3 + H], zp = pre[o3 + 2 * H];
-    const float out = st + sigm(zg) * (gfun(zh) - st);
-    const float p = sigm(zp);
-    x_next[idx] = p * out + (1.0f - p) * x[idx];
-}
-
-// PPO head gradients for one window column per thread; loss terms are reduced
-// per block in a fixed order and written to block_loss[3*blockIdx] (double).
 // The head's gradient rows are 48 floats wide: [43 dlogits | dvalue | 0 0 0 0], and the
 // head weights are mirrored as one [48][256] matrix [W_a ; W_v ; 0].  dh3 = rows . mirror
 // then carries the value head's share (the reference's k_add_dv_wv pass,
 // craftax_full.cu:10224), K = 48 suits the 16-wide MFMA steps, and one dW GEMM over 44
 // rows yields dW_a and dW_v together (cu_gemv_dwv, :11655, needs no pass of its own).
-constexpr int kHeadLd = 48;
+constexpr int kHeadLd = kHeadGradLd;
 __global__ void k_head_mirror(const float* __restrict__ W_a, const float* __restrict__ W_v,
                               float* __restrict__ out) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= kHeadLd * H) return;
     const int r = idx / H, k = idx - r * H;
     out[idx] = r < A ? W_a[idx] : (r == A ? W_v[k] : 0.0f);
-}
-
-__global__ __launch_bounds__(128) void k_head_bwd_win(
-    const float* __restrict__ logits, const float* __restrict__ h3,
-    const float* __restrict__ b_a, const float* __restrict__ W_v,
-    const float* __restrict__ b_v, const int32_t* __restrict__ r_act,
-    const float* __restrict__ r_logprob, const float* __restrict__ adv,
-    const float* __restrict__ ret, const double* __restrict__ adv_stats,
-    float* __restrict__ dlogits,
-    double* __restrict__ block_loss, int t0, int cols, int mb, int n, int n_all,
-    int T_all, float clip_eps, float vf_coef, const float* __restrict__ ent_coef_p,
-    int logits_ld) {   // b_a == nullptr: rows of the fused forward, 43 logits + value, biases included
-    __shared__ double s_l[3][128];
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    double l_pg = 0.0, l_v = 0.0, l_e = 0.0;
-    if (c < cols) {
-        const int t_rel = c / mb;
-        const int el = c - t_rel * mb;
-        const size_t o = (size_t)(t0 + t_rel) * n + el;
-        const float ent_coef = *ent_coef_p;
-        const double inv_count = 1.0 / ((double)n_all * (double)T_all);
-        const double m = adv_stats[0] * inv_count;
-        const float adv_mean = (float)m;
-        const double var = adv_stats[1] * inv_count - m * m;
-        const float adv_inv_std = 1.0f / ((float)sqrt(var > 0.0 ? var : 0.0) + 1e-8f);
-        const float inv_batch = 1.0f / (float)(T_all * mb);
-        const float* lp = logits + (size_t)c * logits_ld;
-        float lg[A], pi[A];
-        float mx = -1e30f;
-#pragma unroll
-        for (int a = 0; a < A; a++) { lg[a] = lp[a] + (b_a ? b_a[a] : 0.0f); mx = fmaxf(mx, lg[a]); }
-        float total = 0.0f;
-#pragma unroll
-        for (int a = 0; a < A; a++) { pi[a] = expf(lg[a] - mx); total += pi[a]; }
-        const float inv_total = 1.0f / total;
-#pragma unroll
-        for (int a = 0; a < A; a++) pi[a] *= inv_total;
-        const float lse = mx + logf(total);
-        const int act = r_act[o];
-        float lg_act = 0.0f;
-#pragma unroll
-        for (int a = 0; a < A; a++) lg_act = (a == act) ? lg[a] : lg_act;
-        const float ratio = expf((lg_act - lse) - r_logprob[o]);
-        const float Ad = (adv[o] - adv_mean) * adv_inv_std;
-        const float u1 = ratio * Ad;
-        const float u2 = fminf(fmaxf(ratio, 1.0f - clip_eps), 1.0f + clip_eps) * Ad;
-        const float dlogp = (u1 <= u2) ? -Ad * ratio : 0.0f;
-        float Hent = 0.0f;
-#pragma unroll
-        for (int a = 0; a < A; a++) Hent -= pi[a] * (lg[a] - lse);
-        float v;
-        if (b_a) {
-            v = b_v[0];
-            const float* hc = h3 + (size_t)c * H;
-#pragma unroll 4
-            for (int j = 0; j < H; j++) v = fmaf(W_v[j], hc[j], v);
-        } else {
-            v = lp[A];   // the fused forward leaves the value (bias included) behind the logits
-        }
-        const float dret = v - ret[o];
-        // one 48-float row per column: 43 logit gradients, the value gradient, zeros
-        float* dq = dlogits + (size_t)c * kHeadLd;
-#pragma unroll
-        for (int a = 0; a < A; a++) {
-            float d = dlogp * ((a == act ? 1.0f : 0.0f) - pi[a]);
-            d += ent_coef * pi[a] * ((lg[a] - lse) + Hent);
-            dq[a] = d * inv_batch;
-        }
-        dq[A] = inv_batch * vf_coef * dret;
-#pragma unroll
-        for (int a = A + 1; a < kHeadLd; a++) dq[a] = 0.0f;
-        l_pg = (double)(-fminf(u1, u2));
-        l_v = (double)(0.5f * dret * dret);
-        l_e = (double)Hent;
-    }
-    s_l[0][threadIdx.x] = l_pg; s_l[1][threadIdx.x] = l_v; s_l[2][threadIdx.x] = l_e;
-    __syncthreads();
-    for (int w = 64; w > 0; w >>= 1) {
-        if ((int)threadIdx.x < w)
-            for (int q = 0; q < 3; q++) s_l[q][threadIdx.x] += s_l[q][threadIdx.x + w];
-        __syncthreads();
-    }
-    if (threadIdx.x < 3) block_loss[3 * blockIdx.x + threadIdx.x] = s_l[threadIdx.x][0];
-}
-
-// loss_acc[q] += sum_b block_loss[3b+q].  Fixed order: thread (q, c) of 3 x 64 sums
-// the blocks of chunk c in ascending order, then thread (q, 0) adds the 64 chunk
-// sums in ascending order.
-__global__ __launch_bounds__(256) void k_loss_fold(const double* __restrict__ block_loss,
-                                                   int blocks, double* __restrict__ loss_acc) {
-    __shared__ double red[3][64];
-    const int q = threadIdx.x >> 6, c = threadIdx.x & 63;
-    if (q < 3) {
-        const int per = (blocks + 63) / 64;
-        const int b1 = min(blocks, (c + 1) * per);
-        double s = 0.0;
-        for (int b = c * per; b < b1; b++) s += block_loss[3 * b + q];
-        red[q][c] = s;
-    }
-    __syncthreads();
-    if (q < 3 && c == 0) {
-        double s = 0.0;
-        for (int i = 0; i < 64; i++) s += red[q][i];
-        loss_acc[q] += s;
-    }
 }
 
 // out[r] += sum_c src[c*ld + r]: partial sums over `slices` column ranges
@@ -239,116 +100,6 @@ __global__ __launch_bounds__(256) void k_colsum_fold(const float* __restrict__ p
     }
 }
 
-// Reverse MinGRU over one window: thread per (unit, env), t descending, live
-// dcarry across windows; dpre overwrites pre in place.
-__global__ void k_mingru_window_bwd(
-    float* __restrict__ pre, const float* __restrict__ x,
-    const float* __restrict__ dhGEMM, const float* __restrict__ dhExtra,
-    const float* __restrict__ r_state, const uint8_t* __restrict__ r_done,
-    float* __restrict__ dhExtraOut, float* __restrict__ dcarry, int t0, int Tw,
-    int mb, int n, int env_start, int layer, int layers, int T_all, int seg_len) {
-    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (size_t)H * mb) return;
-    const int k = (int)(idx & (H - 1));
-    const size_t el = idx / H;
-    float dc = dcarry[idx];
-    for (int tr = Tw - 1; tr >= 0; tr--) {
-        const int t = t0 + tr;
-        if (t == T_all - 1 || ((t + 1) % seg_len) == 0) dc = 0.0f;
-        const size_t w = (size_t)tr * mb + el;
-        const size_t o = w * H + k;
-        const size_t o3 = w * G + k;
-        const float zh = __builtin_nontemporal_load(pre + o3);
-        const float zg = __builtin_nontemporal_load(pre + o3 + H);
-        const float zp = __builtin_nontemporal_load(pre + o3 + 2 * H);
-        float dhout = __builtin_nontemporal_load(dhGEMM + o);
-        if (dhExtra) dhout += __builtin_nontemporal_load(dhExtra + o);
-        const size_t rs = (((size_t)t * layers + layer) * (size_t)n + env_start + el) * H + k;
-        const float s_in = __builtin_nontemporal_load(r_state + rs);
-        const float xv = __builtin_nontemporal_load(x + o);
-        const bool done_t = r_done[(size_t)t * n + env_start + el] != 0;
-        const float sg = sigm(zg);
-        const float gh = gfun(zh);
-        const float p = sigm(zp);
-        const float out_k = s_in + sg * (gh - s_in);
-        const float dout = dhout * p + (done_t ? 0.0f : dc);
-        const float dzp = dhout * (out_k - xv) * p * (1.0f - p);
-        if (dhExtraOut) dhExtraOut[o] = dhout * (1.0f - p);
-        dc = dout * (1.0f - sg);
-        const float dzg = dout * (gh - s_in) * sg * (1.0f - sg);
-        const float dzh = dout * sg * dgfun(zh);
-        pre[o3] = dzh;
-        pre[o3 + H] = dzg;
-        pre[o3 + 2 * H] = dzp;
-    }
-    dcarry[idx] = dc;
-}
-
-__global__ void k_gae(const float* __restrict__ values, const float* __restrict__ rewards,
-                      const uint8_t* __restrict__ dones, const float* __restrict__ v_boot,
-                      float* __restrict__ adv, float* __restrict__ ret, int n, int T,
-                      float gamma, float lam) {
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= n) return;
-    float Aacc = 0.0f;
-    for (int t = T - 1; t >= 0; t--) {
-        const size_t o = (size_t)t * n + e;
-        const float vnext = (t == T - 1) ? v_boot[e] : values[o + n];
-        const float nonterm = dones[o] ? 0.0f : 1.0f;
-        const float delta = rewards[o] + gamma * vnext * nonterm - values[o];
-        Aacc = delta + gamma * lam * nonterm * Aacc;
-        adv[o] = Aacc;
-        ret[o] = Aacc + values[o];
-    }
-}
-
-// (sum, sum of squares) in double; 256 blocks of partials, folded in order.
-__global__ __launch_bounds__(256) void k_adv_stats_partial(
-    const float* __restrict__ adv, size_t count, double* __restrict__ part) {
-    __shared__ double s_sum[256], s_sq[256];
-    double sum = 0.0, sq = 0.0;
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count;
-         i += (size_t)gridDim.x * blockDim.x) {
-        const double a = adv[i];
-        sum += a; sq += a * a;
-    }
-    s_sum[threadIdx.x] = sum; s_sq[threadIdx.x] = sq;
-    __syncthreads();
-    for (int w = 128; w > 0; w >>= 1) {
-        if ((int)threadIdx.x < w) {
-            s_sum[threadIdx.x] += s_sum[threadIdx.x + w];
-            s_sq[threadIdx.x] += s_sq[threadIdx.x + w];
-        }
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) { part[2 * blockIdx.x] = s_sum[0]; part[2 * blockIdx.x + 1] = s_sq[0]; }
-}
-__global__ void k_adv_stats_fold(const double* __restrict__ part, int blocks,
-                                 double* __restrict__ stats) {
-    if (threadIdx.x >= 2) return;
-    double s = 0.0;
-    for (int b = 0; b < blocks; b++) s += part[2 * b + threadIdx.x];
-    stats[threadIdx.x] = s;
-}
-
-__global__ void k_adam(float* __restrict__ params, float* __restrict__ grads,
-                       float* __restrict__ m, float* __restrict__ v,
-                       const uint64_t* __restrict__ step_ctr,
-                       const float* __restrict__ lr_ptr, float beta1, float beta2,
-                       float eps, int count) {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= count) return;
-    const float lr = *lr_ptr;
-    const int step = (int)(*step_ctr) + 1;
-    const float g = grads[i];
-    grads[i] = 0.0f;
-    const float mi = beta1 * m[i] + (1.0f - beta1) * g;
-    const float vi = beta2 * v[i] + (1.0f - beta2) * g * g;
-    m[i] = mi; v[i] = vi;
-    const float mhat = mi / (1.0f - powf(beta1, (float)step));
-    const float vhat = vi / (1.0f - powf(beta2, (float)step));
-    params[i] -= lr * mhat / (sqrtf(vhat) + eps);
-}
 __global__ void k_bump_ctr(uint64_t* ctr) { *ctr += 1; }
 
 __global__ void k_take_value(const float* __restrict__ av, float* __restrict__ value_row,
@@ -359,49 +110,6 @@ __global__ void k_take_value(const float* __restrict__ av, float* __restrict__ v
 __global__ void k_done_to_float(const uint8_t* __restrict__ d, float* __restrict__ f, int n) {
     const int e = blockIdx.x * blockDim.x + threadIdx.x;
     if (e < n) f[e] = d[e] ? 1.0f : 0.0f;
-}
-
-// Loss terms of one step from biased logits/value rows [n][44] (k_loss_accum).
-__global__ __launch_bounds__(128) void k_loss_accum(
-    const float* __restrict__ av, const int32_t* __restrict__ r_act,
-    const float* __restrict__ r_logprob, const float* __restrict__ adv,
-    const float* __restrict__ ret, const double* __restrict__ adv_stats,
-    double* __restrict__ block_loss, int t, int n, int T_all, float clip_eps) {
-    __shared__ double s_l[3][128];
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    double l_pg = 0.0, l_v = 0.0, l_e = 0.0;
-    if (e < n) {
-        const size_t o = (size_t)t * n + e;
-        const double inv_count = 1.0 / ((double)n * (double)T_all);
-        const double m = adv_stats[0] * inv_count;
-        const double var = adv_stats[1] * inv_count - m * m;
-        const float amean = (float)m;
-        const float ainv = 1.0f / ((float)sqrt(var > 0.0 ? var : 0.0) + 1e-8f);
-        const float* lg = av + (size_t)e * CFP_AV;
-        float mx = -1e30f;
-        for (int a = 0; a < A; a++) mx = fmaxf(mx, lg[a]);
-        float total = 0.0f;
-        for (int a = 0; a < A; a++) total += expf(lg[a] - mx);
-        const float lse = mx + logf(total);
-        float Hent = 0.0f;
-        for (int a = 0; a < A; a++) Hent -= (expf(lg[a] - mx) / total) * (lg[a] - lse);
-        const float Ad = (adv[o] - amean) * ainv;
-        const float ratio = expf((lg[r_act[o]] - lse) - r_logprob[o]);
-        const float u1 = ratio * Ad;
-        const float u2 = fminf(fmaxf(ratio, 1.0f - clip_eps), 1.0f + clip_eps) * Ad;
-        const float dret = lg[A] - ret[o];
-        l_pg = (double)(-fminf(u1, u2));
-        l_v = (double)(0.5f * dret * dret);
-        l_e = (double)Hent;
-    }
-    s_l[0][threadIdx.x] = l_pg; s_l[1][threadIdx.x] = l_v; s_l[2][threadIdx.x] = l_e;
-    __syncthreads();
-    for (int w = 64; w > 0; w >>= 1) {
-        if ((int)threadIdx.x < w)
-            for (int q = 0; q < 3; q++) s_l[q][threadIdx.x] += s_l[q][threadIdx.x + w];
-        __syncthreads();
-    }
-    if (threadIdx.x < 3) block_loss[3 * blockIdx.x + threadIdx.x] = s_l[threadIdx.x][0];
 }
 
 inline unsigned grid1(size_t total, int block = 256) {
@@ -527,8 +235,8 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     TA(v_boot, (size_t)tr->n * sizeof(float));
     TA(stats, 2 * sizeof(double));
     TA(loss_acc, 3 * sizeof(double));
-    TA(block_loss, 3 * sizeof(double) * ((cc > (size_t)tr->n ? cc : tr->n) / 128 + 1));
-    TA(stats_part, 2 * 256 * sizeof(double));
+    TA(block_loss, 3 * sizeof(double) * (size_t)head_blocks((int)(cc > (size_t)tr->n ? cc : tr->n)));
+    TA(stats_part, 2 * sizeof(double) * (size_t)(gae_blocks(tr->n) > kMomentBlocks ? gae_blocks(tr->n) : kMomentBlocks));
     TA(grads, pc * sizeof(float));
     TA(adam_m, pc * sizeof(float));
     TA(adam_v, pc * sizeof(float));
@@ -541,7 +249,7 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     for (int l = 0; l <= tr->L; l++) TA(x[l], cc * H * sizeof(float));
     for (int l = 0; l < tr->L; l++) TA(preb[l], cc * G * sizeof(float));
     for (int l = 0; l < tr->L; l++) TA(dcarry[l], (size_t)mb * H * sizeof(float));
-    TA(logitsb, cc * (A + 1) * sizeof(float));   // [cols][44] from the fused recompute, [cols][43] unfused
+    TA(logitsb, cc * kHeadLd * sizeof(float));   // [cols][44] from the fused recompute, [cols][48] unfused
     TA(dlogits, cc * kHeadLd * sizeof(float));
     TA(w_head, (size_t)kHeadLd * H * sizeof(float));
     TA(dh3b, cc * H * sizeof(float));
@@ -660,21 +368,15 @@ int cfp_train_bootstrap(cfp_trainer* tr, const uint8_t* d_rec_row, const float* 
 int cfp_train_gae(cfp_trainer* tr, void* stream) {
     CFP_REQUIRE(tr, "cfp_train_gae: NULL trainer");
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(k_gae, dim3(grid1(tr->n)), dim3(256), 0, st, tr->r_value,
-                       tr->r_reward, tr->r_done, tr->v_boot, tr->adv, tr->ret, tr->n,
-                       tr->T, tr->cfg.gamma, tr->cfg.lam);
-    return cfp_train_adv_stats(tr, stream);
+    // one pass: advantages, returns and the advantage moments
+    return launch_gae(tr->r_value, tr->r_reward, tr->r_done, tr->v_boot, tr->adv, tr->ret, tr->n,
+                      tr->T, tr->cfg.gamma, tr->cfg.lam, tr->stats_part, tr->stats, st);
 }
 
 int cfp_train_adv_stats(cfp_trainer* tr, void* stream) {
     CFP_REQUIRE(tr, "cfp_train_adv_stats: NULL trainer");
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(k_adv_stats_partial, dim3(256), dim3(256), 0, st, tr->adv,
-                       (size_t)tr->n * tr->T, tr->stats_part);
-    hipLaunchKernelGGL(k_adv_stats_fold, dim3(1), dim3(64), 0, st, tr->stats_part, 256,
-                       tr->stats);
-    CFP_HIP_TRY(hipGetLastError());
-    return 0;
+    return launch_adv_moments(tr->adv, (size_t)tr->n * tr->T, tr->stats_part, tr->stats, st);
 }
 
 static int colsum_into(cfp_trainer* tr, const float* src, int ld, float* out, int rows,
@@ -713,6 +415,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
     const float* W_v = p->params + CFP_OFF_W_V(L);
     const float* b_v = p->params + CFP_OFF_B_V(L);
     float* g = tr->grads;
+    const WindowMap wm_all{0, mb, n, env_start};
 
     for (int l = 0; l < L; l++)
         hipLaunchKernelGGL(k_fill, dim3(grid1((size_t)H * mb)), dim3(256), 0, st,
@@ -725,7 +428,8 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         const int t0 = t_end - tr->win > 0 ? t_end - tr->win : 0;
         const int Tw = t_end - t0;
         const int cols = Tw * mb;
-        const size_t hc = (size_t)H * cols;
+        WindowMap wm = wm_all;
+        wm.t0 = t0;
         // ---- forward recompute of the window into tight columns: one launch of the
         // fused forward kernel (fp32, or the bf16-input one) in its window mode: stored
         // state in, pre-activations and layer outputs out.  The unfused chain below is
@@ -761,21 +465,27 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
                 if (cfp_gemm_fwd(G, cols, H, W_gru + (size_t)l * G * H, tr->x[l], tr->preb[l],
                                  stream))
                     return 1;
-                hipLaunchKernelGGL(k_mingru_epi_replay_win, dim3(grid1(hc)), dim3(256), 0, st,
-                                   tr->preb[l], tr->x[l], tr->r_state, tr->x[l + 1], t0, hc,
-                                   mb, n, env_start, l, L);
+                if (launch_gru_replay(tr->preb[l], tr->x[l], tr->r_state, tr->x[l + 1], wm, cols, l,
+                                      L, st))
+                    return 1;
             }
-            if (cfp_gemm_fwd(A, cols, H, W_a, tr->x[L], tr->logitsb, stream)) return 1;
+            // 48-row head against the [W_a ; W_v ; 0] mirror: logits and value, no biases
+            if (cfp_gemm_fwd(kHeadLd, cols, H, tr->w_head, tr->x[L], tr->logitsb, stream)) return 1;
         }
         // ---- head gradients
-        const int hb = (cols + 127) / 128;
-        hipLaunchKernelGGL(k_head_bwd_win, dim3(hb), dim3(128), 0, st, tr->logitsb, tr->x[L],
-                           fused ? nullptr : b_a, W_v, b_v, tr->r_act + env_start, tr->r_logprob + env_start,
-                           tr->adv + env_start, tr->ret + env_start, tr->stats, tr->dlogits,
-                           tr->block_loss, t0, cols, mb, n, n, T, tr->cfg.clip,
-                           tr->cfg.vf, tr->d_ent, fused ? A + 1 : A);
-        hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(256), 0, st, tr->block_loss, hb,
-                           tr->loss_acc);
+        HeadArgs ha{};
+        ha.rows = tr->logitsb;
+        ha.ld = fused ? A + 1 : kHeadLd;     // the fused forward's rows carry the biases
+        ha.bias_a = fused ? nullptr : b_a;
+        ha.bias_v = fused ? nullptr : b_v;
+        ha.act = tr->r_act; ha.old_logp = tr->r_logprob; ha.adv = tr->adv; ha.ret = tr->ret;
+        ha.adv_moments = tr->stats;
+        ha.grad_rows = tr->dlogits;
+        ha.block_loss = tr->block_loss;
+        ha.w = wm; ha.cols = cols; ha.horizon = T;
+        ha.clip = tr->cfg.clip; ha.vf = tr->cfg.vf; ha.ent_coef = tr->d_ent;
+        if (launch_head(ha, st)) return 1;
+        if (launch_fold_f64(tr->block_loss, head_blocks(cols), 3, tr->loss_acc, true, st)) return 1;
         // dh3 = [dlogits | dvalue] . [W_a ; W_v]; dW_a and dW_v from one GEMM; bias sums
         if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, st)) return 1;
         if (gemm_dw_two(A, 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L),
@@ -796,10 +506,12 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         const float* dh_gemm = tr->dh3b;
         const float* dh_extra = nullptr;
         for (int l = L - 1; l >= 0; l--) {
-            hipLaunchKernelGGL(k_mingru_window_bwd, dim3(grid1((size_t)H * mb)), dim3(256),
-                               0, chain, tr->preb[l], tr->x[l], dh_gemm, dh_extra, tr->r_state,
-                               tr->r_done, tr->dhX, tr->dcarry[l], t0, Tw, mb, n, env_start,
-                               l, L, T, seg);
+            ReverseArgs ra{};
+            ra.gates = tr->preb[l]; ra.layer_in = tr->x[l];
+            ra.grad_a = dh_gemm; ra.grad_b = dh_extra; ra.highway_out = tr->dhX;
+            ra.slab_state = tr->r_state; ra.slab_done = tr->r_done; ra.carry = tr->dcarry[l];
+            ra.w = wm; ra.steps = Tw; ra.layer = l; ra.layers = L; ra.horizon = T; ra.seg = seg;
+            if (launch_gru_reverse(ra, chain)) return 1;
             if (!overlap &&
                 gemm_dw_ld(G, cols, tr->x[l], tr->preb[l], G, g + CFP_OFF_W_GRU + (size_t)l * G * H,
                            chain))
@@ -852,13 +564,13 @@ int cfp_train_zero_loss(cfp_trainer* tr, void* stream) {
 int cfp_train_adam(cfp_trainer* tr, void* stream) {
     CFP_REQUIRE(tr, "cfp_train_adam: NULL trainer");
     hipStream_t st = (hipStream_t)stream;
-    const int pc = (int)tr->p->param_count;
-    hipLaunchKernelGGL(k_adam, dim3(grid1(pc)), dim3(256), 0, st, tr->p->params, tr->grads,
-                       tr->adam_m, tr->adam_v, tr->adam_ctr, tr->d_lr, 0.9f, 0.999f, 1e-8f,
-                       pc);
+    // parameters, moments and every weight mirror of the forward kernels in one pass
+    if (launch_adam(tr->p, tr->grads, tr->adam_m, tr->adam_v, tr->adam_ctr, tr->d_lr, 0.9f, 0.999f,
+                    1e-8f, st))
+        return 1;
     hipLaunchKernelGGL(k_bump_ctr, dim3(1), dim3(1), 0, st, tr->adam_ctr);
     CFP_HIP_TRY(hipGetLastError());
-    return cfp_policy_refresh_weights(tr->p, stream);
+    return 0;
 }
 
 // cu_train_body without its collect (craftax_full.cu:13348-13366): per epoch the loss
@@ -941,7 +653,13 @@ int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream) {
     const int seg = T / tr->cfg.bptt_split;
     const size_t hn = (size_t)H * n;
     if (cfp_train_zero_loss(tr, stream)) return 1;
-    const int hb = (n + 127) / 128;
+    HeadArgs ha{};
+    ha.rows = tr->av_tmp; ha.ld = A + 1;
+    ha.act = tr->r_act; ha.old_logp = tr->r_logprob; ha.adv = tr->adv; ha.ret = tr->ret;
+    ha.adv_moments = tr->stats;
+    ha.block_loss = tr->block_loss;
+    ha.cols = n; ha.horizon = T;
+    ha.clip = tr->cfg.clip; ha.vf = tr->cfg.vf; ha.ent_coef = tr->d_ent;
     for (int t = 0; t < T; t++) {
         const bool segstart = (t % seg) == 0;
         const float* term = nullptr;
@@ -956,11 +674,9 @@ int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream) {
         if (cfp_policy_forward(tr->p, tr->r_obs + (size_t)t * n * CFP_REC_BYTES, term,
                                tr->live, nullptr, nullptr, nullptr, tr->av_tmp, n, 0, stream))
             return 1;
-        hipLaunchKernelGGL(k_loss_accum, dim3(hb), dim3(128), 0, st, tr->av_tmp, tr->r_act,
-                           tr->r_logprob, tr->adv, tr->ret, tr->stats, tr->block_loss, t, n,
-                           T, tr->cfg.clip);
-        hipLaunchKernelGGL(k_loss_fold, dim3(1), dim3(256), 0, st, tr->block_loss, hb,
-                           tr->loss_acc);
+        ha.w = WindowMap{t, n, n, 0};
+        if (launch_head(ha, st)) return 1;
+        if (launch_fold_f64(tr->block_loss, head_blocks(n), 3, tr->loss_acc, true, st)) return 1;
     }
     CFP_HIP_TRY(hipGetLastError());
     CFP_HIP_TRY(hipStreamSynchronize(st));

@@ -398,3 +398,38 @@ def test_backward_with_bf16_gemms(pkg, cuda):
             worst = max(worst, e)
         assert worst > 1e-4, "the bf16 GEMMs did not run"
     tr.close(); pol.close()
+
+
+def test_adam_writes_every_weight_mirror(pkg, cuda):
+    """cfp_train_adam rewrites the forward kernels' weight mirrors (fp32 MFMA order, the
+    three-term bf16 split of the encoder, the bf16 mirrors) in the pass that updates the
+    parameters.  After two steps with gradients on every parameter, the fp32 and the
+    bf16-input forward of the trained policy must equal, bit for bit, those of a fresh
+    policy given the same parameters through cfp_policy_set_params, whose mirrors come
+    from the pack kernels."""
+    import torch
+    n = 64
+    pol = pkg.Policy(n, L, seed=21)
+    tr = pkg.Trainer(pol, 4)
+    rng = np.random.default_rng(22)
+    before = pol.get_params()
+    for _ in range(2):
+        g = (rng.standard_normal(before.size) * 0.1).astype(np.float32)
+        tr.buf("grads").copy_(_t(g, cuda))
+        tr.adam()
+    torch.cuda.synchronize()
+    after = pol.get_params()
+    assert np.all(after != before)                      # every parameter moved
+    twin = pkg.Policy(n, L, seed=99)
+    twin.set_params(after)
+    rec = _t(synth_records_host(n, 23, 0), cuda)
+    term = torch.zeros(n, device=cuda)
+    s0 = (0.5 * rng.standard_normal((L, n, HIDDEN))).astype(np.float32)
+    for bf16 in (False, True):
+        pol.set_gemm_bf16(bf16); twin.set_gemm_bf16(bf16)
+        sa, sb = _t(s0, cuda), _t(s0, cuda)
+        av_a = pol.forward(rec, term, sa).clone()
+        av_b = twin.forward(rec, term, sb).clone()
+        assert torch.equal(av_a, av_b), f"bf16={bf16}: head rows differ"
+        assert torch.equal(sa, sb), f"bf16={bf16}: states differ"
+    tr.close(); pol.close(); twin.close()
