@@ -42,82 +42,214 @@ __device__ __forceinline__ double wave_sum(double v) {
 }
 
 // ---- reverse MinGRU sweep --------------------------------------------------------
+// The loads and stores of a step are issued from inline assembly and the wait that
+// makes a step's operands readable is an explicit s_waitcnt vmcnt(N): the compiler's own
+// wait insertion drains the whole queue (vmcnt(0)) in front of every store, which leaves
+// nothing in flight while a wavefront computes.  Vector-memory operations complete in
+// issue order, so "the set fetched three stages ago has landed" is "at most N younger
+// operations are outstanding".  Three register sets rotate through a loop unrolled by
+// three (a set is never copied: a copy would read registers whose loads are in flight).
 struct StepIn {
     f4 zh, zg, zp, ga, gb, s, x;
     unsigned done;
 };
 
+template <bool TWO_GRADS>
+__device__ __forceinline__ void sweep_fetch(StepIn& r, unsigned lane_off, const f4* gates,
+                                            const f4* ga, const f4* gb, const f4* state,
+                                            const f4* xin, const uint8_t* done) {
+    const unsigned zero = 0u;
+    if (TWO_GRADS)
+        asm volatile(
+            "global_load_dwordx4 %0, %8, %10 nt\n\t"
+            "global_load_dwordx4 %1, %8, %10 offset:1024 nt\n\t"
+            "global_load_dwordx4 %2, %8, %10 offset:2048 nt\n\t"
+            "global_load_dwordx4 %3, %8, %11 nt\n\t"
+            "global_load_dwordx4 %4, %8, %12 nt\n\t"
+            "global_load_dwordx4 %5, %8, %13 nt\n\t"
+            "global_load_dwordx4 %6, %8, %14 nt\n\t"
+            "global_load_ubyte %7, %9, %15"
+            : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.gb), "=&v"(r.s),
+              "=&v"(r.x), "=&v"(r.done)
+            : "v"(lane_off), "v"(zero), "s"(gates), "s"(ga), "s"(gb), "s"(state), "s"(xin), "s"(done)
+            : "memory");
+    else
+        asm volatile(
+            "global_load_dwordx4 %0, %7, %9 nt\n\t"
+            "global_load_dwordx4 %1, %7, %9 offset:1024 nt\n\t"
+            "global_load_dwordx4 %2, %7, %9 offset:2048 nt\n\t"
+            "global_load_dwordx4 %3, %7, %10 nt\n\t"
+            "global_load_dwordx4 %4, %7, %11 nt\n\t"
+            "global_load_dwordx4 %5, %7, %12 nt\n\t"
+            "global_load_ubyte %6, %8, %13"
+            : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.s), "=&v"(r.x),
+              "=&v"(r.done)
+            : "v"(lane_off), "v"(zero), "s"(gates), "s"(ga), "s"(state), "s"(xin), "s"(done)
+            : "memory");
+}
+
+// Every later use of the set depends on this statement's outputs, so none can be moved
+// in front of the wait.
+template <int N, bool TWO_GRADS>
+__device__ __forceinline__ void sweep_wait(StepIn& r) {
+    if (TWO_GRADS)
+        asm volatile("s_waitcnt vmcnt(%8)"
+                     : "+v"(r.zh), "+v"(r.zg), "+v"(r.zp), "+v"(r.ga), "+v"(r.gb), "+v"(r.s),
+                       "+v"(r.x), "+v"(r.done)
+                     : "n"(N));
+    else
+        asm volatile("s_waitcnt vmcnt(%7)"
+                     : "+v"(r.zh), "+v"(r.zg), "+v"(r.zp), "+v"(r.ga), "+v"(r.s), "+v"(r.x),
+                       "+v"(r.done)
+                     : "n"(N));
+}
+
+template <bool HIGHWAY>
+__device__ __forceinline__ void sweep_store(unsigned lane_off, f4* gates, f4* hw, const f4& dzh,
+                                            const f4& dzg, const f4& dzp, const f4& hwv) {
+    // the trailing s_nop keeps the next instruction clear of the store data registers
+    if (HIGHWAY)
+        asm volatile(
+            "global_store_dwordx4 %0, %1, %5 nt\n\t"
+            "global_store_dwordx4 %0, %2, %5 offset:1024 nt\n\t"
+            "global_store_dwordx4 %0, %3, %5 offset:2048 nt\n\t"
+            "global_store_dwordx4 %0, %4, %6 nt\n\t"
+            "s_nop 0"
+            :
+            : "v"(lane_off), "v"(dzh), "v"(dzg), "v"(dzp), "v"(hwv), "s"(gates), "s"(hw)
+            : "memory");
+    else
+        asm volatile(
+            "global_store_dwordx4 %0, %1, %4 nt\n\t"
+            "global_store_dwordx4 %0, %2, %4 offset:1024 nt\n\t"
+            "global_store_dwordx4 %0, %3, %4 offset:2048 nt\n\t"
+            "s_nop 0"
+            :
+            : "v"(lane_off), "v"(dzh), "v"(dzg), "v"(dzp), "s"(gates)
+            : "memory");
+}
+
+// Drain the queue; every set is an output, so nothing of any set is read before it.
+template <bool TWO_GRADS>
+__device__ __forceinline__ void sweep_drain(StepIn& p, StepIn& q, StepIn& r) {
+    if (TWO_GRADS)
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(p.zh), "+v"(p.zg), "+v"(p.zp), "+v"(p.ga), "+v"(p.gb), "+v"(p.s),
+                       "+v"(p.x), "+v"(p.done), "+v"(q.zh), "+v"(q.zg), "+v"(q.zp), "+v"(q.ga),
+                       "+v"(q.gb), "+v"(q.s), "+v"(q.x), "+v"(q.done), "+v"(r.zh), "+v"(r.zg),
+                       "+v"(r.zp), "+v"(r.ga), "+v"(r.gb), "+v"(r.s), "+v"(r.x), "+v"(r.done));
+    else
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(p.zh), "+v"(p.zg), "+v"(p.zp), "+v"(p.ga), "+v"(p.s), "+v"(p.x),
+                       "+v"(p.done), "+v"(q.zh), "+v"(q.zg), "+v"(q.zp), "+v"(q.ga), "+v"(q.s),
+                       "+v"(q.x), "+v"(q.done), "+v"(r.zh), "+v"(r.zg), "+v"(r.zp), "+v"(r.ga),
+                       "+v"(r.s), "+v"(r.x), "+v"(r.done));
+}
+
+#ifndef CFP_SWEEP_EPB
+#define CFP_SWEEP_EPB 1
+#endif
+constexpr int kSweepEnvs = CFP_SWEEP_EPB;   // envs (wavefronts) per workgroup
 template <bool TWO_GRADS, bool HIGHWAY>
-__global__ __launch_bounds__(256) void k_gru_reverse(ReverseArgs a) {
+__global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-    const int env = (int)blockIdx.x * 4 + wave;   // mb % 4 == 0: whole wavefronts only
-    const int q = threadIdx.x & 63;               // units 4q .. 4q+3
-    if (env >= a.w.mb) return;
-    const size_t col_stride = (size_t)a.w.mb;
-    f4* const gates = reinterpret_cast<f4*>(a.gates) + (size_t)env * G4 + q;
-    const size_t hq = (size_t)env * H4 + q;
-    const f4* const xin = reinterpret_cast<const f4*>(a.layer_in) + hq;
-    const f4* const ga = reinterpret_cast<const f4*>(a.grad_a) + hq;
-    const f4* const gb = TWO_GRADS ? reinterpret_cast<const f4*>(a.grad_b) + hq : nullptr;
-    f4* const hw = HIGHWAY ? reinterpret_cast<f4*>(a.highway_out) + hq : nullptr;
+    const int env = (int)blockIdx.x * kSweepEnvs + wave;   // mb % 32 == 0: whole wavefronts only
+    const unsigned lane_off = (threadIdx.x & 63u) * 16u;   // units 4q .. 4q+3 of a 1 KiB row
+    // wavefront-uniform row pointers of this env; a step back in time is one stride
+    const size_t mbz = (size_t)a.w.mb;
+    f4* const gates = reinterpret_cast<f4*>(a.gates) + (size_t)env * G4;
+    const f4* const xin = reinterpret_cast<const f4*>(a.layer_in) + (size_t)env * H4;
+    const f4* const ga = reinterpret_cast<const f4*>(a.grad_a) + (size_t)env * H4;
+    const f4* const gb = TWO_GRADS ? reinterpret_cast<const f4*>(a.grad_b) + (size_t)env * H4 : nullptr;
+    f4* const hw = HIGHWAY ? reinterpret_cast<f4*>(a.highway_out) + (size_t)env * H4 : nullptr;
     const size_t slab_env = (size_t)a.w.env_start + env;
     const size_t state_step = (size_t)a.layers * a.w.n_all * H4;
     const f4* const state = reinterpret_cast<const f4*>(a.slab_state) +
-                            (((size_t)a.w.t0 * a.layers + a.layer) * a.w.n_all + slab_env) * H4 + q;
+                            (((size_t)a.w.t0 * a.layers + a.layer) * a.w.n_all + slab_env) * H4;
     const uint8_t* const done = a.slab_done + (size_t)a.w.t0 * a.w.n_all + slab_env;
+    // Every stage fetches, so that the number of operations in flight is the same at
+    // every wait; a stage with no step left to fetch reads rows of the carry array
+    // instead (cache-resident, never used).  Three consecutive rows must exist.
+    const f4* const idle = reinterpret_cast<const f4*>(a.carry) +
+                           (size_t)(env < a.w.mb - 2 ? env : a.w.mb - 3) * H4;
 
-    auto fetch = [&](int s, StepIn& r) {
-        const size_t c = (size_t)s * col_stride;
-        r.zh = ld_stream(gates + c * G4);
-        r.zg = ld_stream(gates + c * G4 + H4);
-        r.zp = ld_stream(gates + c * G4 + 2 * H4);
-        r.ga = ld_stream(ga + c * H4);
-        if (TWO_GRADS) r.gb = ld_stream(gb + c * H4);
-        r.s = ld_stream(state + (size_t)s * state_step);
-        r.x = ld_stream(xin + c * H4);
-        r.done = done[(size_t)s * a.w.n_all];
+    auto fetch = [&](int s, StepIn& r) {   // s < 0: nothing left, an idle fetch
+        const bool real = s >= 0;
+        const size_t c = (size_t)(real ? s : 0) * mbz;
+        sweep_fetch<TWO_GRADS>(r, lane_off, real ? gates + c * G4 : idle, real ? ga + c * H4 : idle,
+                               TWO_GRADS ? (real ? gb + c * H4 : idle) : nullptr,
+                               real ? state + (size_t)s * state_step : idle,
+                               real ? xin + c * H4 : idle, done + (size_t)(real ? s : 0) * a.w.n_all);
     };
 
-    f4* const carry_p = reinterpret_cast<f4*>(a.carry) + hq;
+    f4* const carry_p = reinterpret_cast<f4*>(a.carry) + (size_t)env * H4 + (threadIdx.x & 63u);
     f4 carry = *carry_p;
+    // the recurrence is cut behind the last step of the rollout and of every BPTT
+    // segment: `phase` = (t + 1) % seg of the step about to be consumed
     const int last = a.steps - 1;
-    StepIn cur, nx1;
-    fetch(last, cur);
-    fetch(last > 0 ? last - 1 : 0, nx1);
-    StepIn nx2 = nx1;
-    for (int s = last; s >= 0; s--) {
-        if (s >= 2) fetch(s - 2, nx2);
-        const int t = a.w.t0 + s;
-        // the recurrence is cut at the end of the rollout and of every BPTT segment
-        if (t == a.horizon - 1 || (t + 1) % a.seg == 0) carry = f4{0.0f, 0.0f, 0.0f, 0.0f};
-        const float pass = cur.done ? 0.0f : 1.0f;   // a terminal step hands nothing back
+    int phase = (a.w.t0 + last + 1) % a.seg;
+
+    auto consume = [&](int s, const StepIn& in) {
+        if (a.w.t0 + s == a.horizon - 1 || phase == 0) carry = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        phase = (phase == 0 ? a.seg : phase) - 1;
+        const float pass = (in.done & 0xffu) ? 0.0f : 1.0f;   // a terminal step hands nothing back
         f4 dzh, dzg, dzp, hwv;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const float sg = sigmoid_fast(cur.zg[j]);
-            const float mix = sigmoid_fast(cur.zp[j]);
-            const float sh = sigmoid_fast(cur.zh[j]);
-            const bool lin = cur.zh[j] >= 0.0f;
-            const float cand = lin ? cur.zh[j] + 0.5f : sh;          // g(zh)
+            const float sg = sigmoid_fast(in.zg[j]);
+            const float mix = sigmoid_fast(in.zp[j]);
+            const float sh = sigmoid_fast(in.zh[j]);
+            const bool lin = in.zh[j] >= 0.0f;
+            const float cand = lin ? in.zh[j] + 0.5f : sh;           // g(zh)
             const float dcand = lin ? 1.0f : sh * (1.0f - sh);       // g'(zh)
-            const float gap = cand - cur.s[j];
-            const float h_new = cur.s[j] + sg * gap;
-            const float g_top = TWO_GRADS ? cur.ga[j] + cur.gb[j] : cur.ga[j];
+            const float gap = cand - in.s[j];
+            const float h_new = in.s[j] + sg * gap;
+            const float g_top = TWO_GRADS ? in.ga[j] + in.gb[j] : in.ga[j];
             const float g_h = g_top * mix + pass * carry[j];
-            dzp[j] = g_top * (h_new - cur.x[j]) * mix * (1.0f - mix);
+            dzp[j] = g_top * (h_new - in.x[j]) * mix * (1.0f - mix);
             hwv[j] = g_top * (1.0f - mix);
             carry[j] = g_h * (1.0f - sg);
             dzg[j] = g_h * gap * sg * (1.0f - sg);
             dzh[j] = g_h * sg * dcand;
         }
-        const size_t c = (size_t)s * col_stride;
-        st_stream(gates + c * G4, dzh);
-        st_stream(gates + c * G4 + H4, dzg);
-        st_stream(gates + c * G4 + 2 * H4, dzp);
-        if (HIGHWAY) st_stream(hw + c * H4, hwv);
-        cur = nx1;
-        nx1 = nx2;
+        const size_t c = (size_t)s * mbz;
+        sweep_store<HIGHWAY>(lane_off, gates + c * G4, HIGHWAY ? hw + c * H4 : nullptr, dzh, dzg, dzp, hwv);
+    };
+
+    // Operations per stage: NL loads then (after the step's arithmetic) NS stores.
+    // When a set is waited for, the younger operations are the two fetches behind it and
+    // the stores of the stages in between: two stages' worth in the steady state, fewer
+    // stores in the first round.  A round is straight-line code: no control flow ever
+    // merges registers whose loads are in flight.
+    constexpr int NL = TWO_GRADS ? 8 : 7, NS = HIGHWAY ? 4 : 3;
+    StepIn b0, b1, b2;
+    fetch(last, b0);
+    fetch(last - 1, b1);
+    fetch(last - 2, b2);
+#define CFP_SWEEP_ROUND(s_, N0, N1, N2)                 \
+    do {                                                \
+        sweep_wait<(N0), TWO_GRADS>(b0);                \
+        consume((s_), b0);                              \
+        fetch((s_) - 3, b0);                            \
+        sweep_wait<(N1), TWO_GRADS>(b1);                \
+        consume((s_) - 1, b1);                          \
+        fetch((s_) - 4, b1);                            \
+        sweep_wait<(N2), TWO_GRADS>(b2);                \
+        consume((s_) - 2, b2);                          \
+        fetch((s_) - 5, b2);                            \
+    } while (0)
+    int s = last;
+    if (s >= 2) {
+        CFP_SWEEP_ROUND(s, 2 * NL, 2 * NL + NS, 2 * NL + 2 * NS);
+        for (s -= 3; s >= 2; s -= 3)
+            CFP_SWEEP_ROUND(s, 2 * NL + 2 * NS, 2 * NL + 2 * NS, 2 * NL + 2 * NS);
     }
+#undef CFP_SWEEP_ROUND
+    // at most two steps are left, in b0 then b1; everything in flight lands first
+    sweep_drain<TWO_GRADS>(b0, b1, b2);
+    if (s >= 0) consume(s, b0);
+    if (s >= 1) consume(s - 1, b1);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     *carry_p = carry;
 }
 
@@ -493,9 +625,9 @@ __global__ __launch_bounds__(256) void k_adam_mirrors(AdamArgs a) {
 
 int launch_gru_reverse(const ReverseArgs& a, hipStream_t st) {
     CFP_REQUIRE(a.gates && a.layer_in && a.grad_a && a.slab_state && a.slab_done && a.carry &&
-                    a.steps > 0 && a.w.mb > 0 && a.w.mb % 4 == 0 && a.seg > 0,
+                    a.steps > 0 && a.w.mb > 0 && a.w.mb % kSweepEnvs == 0 && a.seg > 0,
                 "reverse MinGRU sweep: bad arguments");
-    const dim3 grid(a.w.mb / 4), blk(256);
+    const dim3 grid(a.w.mb / kSweepEnvs), blk(64 * kSweepEnvs);
     if (a.grad_b && a.highway_out) hipLaunchKernelGGL((k_gru_reverse<true, true>), grid, blk, 0, st, a);
     else if (a.grad_b) hipLaunchKernelGGL((k_gru_reverse<true, false>), grid, blk, 0, st, a);
     else if (a.highway_out) hipLaunchKernelGGL((k_gru_reverse<false, true>), grid, blk, 0, st, a);
