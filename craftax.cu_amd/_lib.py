@@ -51,6 +51,7 @@ PROTOTYPES = {
     "cfp_get_gemm_split": (C.c_int, []),
     "cfp_gemm_fwd": (C.c_int, [C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]),
     "cfp_gemm_enc_fwd": (C.c_int, [C.c_int, vp, vp, vp, vp]),
+    "cfp_seam_reserve": (C.c_int, []),
     "cfp_gemm_dh": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),
     "cfp_gemm_dw": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),
     "cfp_gemv_dwv": (C.c_int, [vp, vp, vp, C.c_int, vp]),

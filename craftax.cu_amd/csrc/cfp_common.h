@@ -153,14 +153,28 @@ int launch_expand_obs(const uint8_t* r_obs, float* xobs, int t0, int count, int 
                       int env_start, int ld, hipStream_t st);
 int gemm_enc_fwd_ld(int cols, const float* W_enc, const float* xobs, int ldx, float* h,
                     hipStream_t st);
-int gemm_dh_acc(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-                hipStream_t st);
-int gemm_dw_ld(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               hipStream_t st);
+// Scratch memory of the seam's kernels: the split mirror of W that k_dh_x9 reads, the
+// split-K partial sums of a dW GEMM, the slice sums of the value-head gemv.  One user
+// at a time: calls that share a SeamWork must be ordered (one stream, or events).
+// A trainer owns its own; the raw C entry points share the process-wide one.
+struct SeamWork {
+    u4* w_mirror = nullptr;
+    float* dw_part = nullptr;
+    size_t dw_part_floats = 0;
+    float* gemv_part = nullptr;
+};
+int seam_work_create(SeamWork* w);
+void seam_work_destroy(SeamWork* w);
+// process-wide workspace of the raw C entry points: made by cfp_seam_reserve() or by the
+// first call that needs it; null (error set) when the allocation fails
+const SeamWork* seam_default();
 
-// split-K workspace of the dW GEMMs (allocated on first use) and the fixed-order fold
-// dst[i] += sum_z part[z*stride + i]
-int dw_workspace(float** work, size_t* floats);
+int gemm_dh_acc(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
+                const SeamWork& sw, hipStream_t st);
+int gemm_dw_ld(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
+               const SeamWork& sw, hipStream_t st);
+
+// the fixed-order fold dst[i] += sum_z part[z*stride + i] of split-K partial sums
 int launch_splitk_reduce(float* dst, const float* part, long count, long stride, int splits,
                          hipStream_t st);
 // dW_enc[843][256] += features^T dh over the window columns, read from the records
@@ -168,33 +182,34 @@ int launch_splitk_reduce(float* dst, const float* part, long count, long stride,
 // cols * 76 floats.
 bool dw_enc_records_ok(int mb);
 int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
-                   int cols, int mb, int n_all, int env_start, hipStream_t st);
+                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st);
 
 // dW[rows][256] += dpre^T x with both fp32 operands split into bf16 triples
 // (cols % 8 == 0)
 bool gemm_dw_x9_ok(int rows, int cols);
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               int terms, hipStream_t st, int rows_first = 0, float* dW_rest = nullptr,
-               float* own_work = nullptr, size_t own_work_floats = 0);
+               int terms, const SeamWork& sw, hipStream_t st, int rows_first = 0,
+               float* dW_rest = nullptr);
 // partial products per product the split kernels run with now (9, 6, or 1 with bf16
 // inputs); 0 when they are switched off
 int gemm_split_terms();
 // dW_a[rows_a][256] += and dW_b[rows_b][256] += from adjacent columns of one dpre matrix
 // (one pass over x on the split kernels, two passes otherwise)
 int gemm_dw_two(int rows_a, int rows_b, int cols, const float* x, const float* dpre, int ld_dpre,
-                float* dW_a, float* dW_b, hipStream_t st);
+                float* dW_a, float* dW_b, const SeamWork& sw, hipStream_t st);
 
 // dh[cols][256] (+)= dpre[cols][m3] . W[m3][256], same splitting (m3 % 16 == 0,
 // cols % 32 == 0, dpre 16-byte aligned)
 bool gemm_dh_x9_ok(int m3, int cols, const float* dpre);
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               int terms, hipStream_t st);
+               int terms, u4* w_mirror, hipStream_t st);
+size_t dh_mirror_bytes();   // size of the split mirror of W (K up to 768)
 
 // y[cols][m] = x[cols][k] . W[m][k]^T on the same kernel (m % 256 == 0, k % 16 == 0,
 // cols % 32 == 0, x 16-byte aligned)
 bool gemm_fwd_x9_ok(int m, int cols, int k, const float* x);
 int gemm_fwd_x9(int m, int cols, int k, const float* W, const float* x, float* y, int terms,
-                hipStream_t st);
+                u4* w_mirror, hipStream_t st);
 
 // per-variant arena geometry
 struct Arena {

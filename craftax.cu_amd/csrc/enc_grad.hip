@@ -213,13 +213,13 @@ __global__ void k_expand_obs_tail(const uint8_t* __restrict__ r_obs, f4* __restr
 bool dw_enc_records_ok(int mb) { return mb > 0 && mb % 8 == 0; }
 
 int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
-                   int cols, int mb, int n_all, int env_start, hipStream_t st) {
+                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st) {
     CFP_REQUIRE(r_obs && dh && dW && tail_scratch && cols > 0 && dw_enc_records_ok(mb) &&
                     cols % 8 == 0,
                 "dw_enc_records: columns and envs per minibatch must be multiples of 8");
-    float* work = nullptr;
-    size_t work_floats = 0;
-    if (dw_workspace(&work, &work_floats)) return 1;
+    float* work = sw.dw_part;
+    const size_t work_floats = sw.dw_part_floats;
+    CFP_REQUIRE(work, "dw_enc_records: no split workspace");
     const int total_iters = (cols + kEgIterCols - 1) / kEgIterCols;
     // one workgroup per CU: 85 splits x 3 groups
     int splits = 256 / kEgGroups;
@@ -239,7 +239,7 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
                        r_obs, reinterpret_cast<f4*>(tail_scratch), t0, total4, mb, n_all,
                        env_start);
     CFP_HIP_TRY(hipGetLastError());
-    return gemm_dw_ld(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, st);
+    return gemm_dw_ld(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, sw, st);
 }
 
 }  // namespace cfp

@@ -22,6 +22,8 @@
 // dW = dpre^T x has K = window columns (>= 16k) and a small output, so K is
 // split over grid.y into a workspace and summed in a fixed order by a second
 // kernel: run-to-run bitwise stable, unlike float atomics.
+#include <mutex>
+
 #include "cfp_common.h"
 
 namespace cfp {
@@ -407,13 +409,15 @@ int run_gemm(GemmArgs g, int splits, bool accum, hipStream_t st) {
     return launch_gemm<A_KFAST, B_KFAST, false>(g, grid, va, vb, st);
 }
 
-// Split-K workspace for cfp_gemm_dw: allocated once per process on first use
-// (the reference pre-warms cuBLAS workspaces the same way before capturing a
-// graph, craftax_full.cu:12094-12122).
+// Split-K workspace of a dW GEMM: room for 128 splits of the largest one (843 rows).
 constexpr int kMaxSplits = 128;
 constexpr size_t kDwWorkFloats = (size_t)kMaxSplits * CFP_OBS * CFP_HIDDEN;
-float* g_dw_work = nullptr;
-float* g_gemv_work = nullptr;   // [kGemvSlices][256], same life cycle
+// The raw C entry points' shared workspace (the reference pre-warms cuBLAS's
+// workspaces before capturing a graph, craftax_full.cu:12094-12122: here
+// cfp_seam_reserve does that).
+std::mutex g_seam_mu;
+SeamWork g_seam;
+bool g_seam_ready = false;
 
 }  // namespace
 }  // namespace cfp
@@ -436,11 +440,42 @@ int gemm_enc_fwd_ld(int cols, const float* d_W_enc, const float* d_xobs, int ldx
 }
 
 // cu_gemm_dh with an accumulate switch: dh[cols][256] (+)= dpre[cols][m3] . W[m3][256]
+int seam_work_create(SeamWork* w) {
+    *w = SeamWork{};
+    hipError_t e = hipMalloc((void**)&w->w_mirror, dh_mirror_bytes());
+    if (e == hipSuccess) e = hipMalloc((void**)&w->dw_part, kDwWorkFloats * sizeof(float));
+    if (e == hipSuccess)
+        e = hipMalloc((void**)&w->gemv_part, (size_t)kGemvSlices * CFP_HIDDEN * sizeof(float));
+    if (e != hipSuccess) {
+        set_error("GEMM workspace allocation failed: %s", hipGetErrorString(e));
+        seam_work_destroy(w);
+        return 1;
+    }
+    w->dw_part_floats = kDwWorkFloats;
+    return 0;
+}
+
+void seam_work_destroy(SeamWork* w) {
+    (void)hipFree(w->w_mirror);
+    (void)hipFree(w->dw_part);
+    (void)hipFree(w->gemv_part);
+    *w = SeamWork{};
+}
+
+const SeamWork* seam_default() {
+    std::lock_guard<std::mutex> lock(g_seam_mu);
+    if (!g_seam_ready) {
+        if (seam_work_create(&g_seam)) return nullptr;
+        g_seam_ready = true;
+    }
+    return &g_seam;
+}
+
 int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* d_dh,
-                bool accumulate, hipStream_t st) {
+                bool accumulate, const SeamWork& sw, hipStream_t st) {
     CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh: bad argument");
     if (g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre))
-        return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, split_terms(), st);
+        return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, split_terms(), sw.w_mirror, st);
     GemmArgs g{};
     g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
     g.B = d_W; g.sb_k = CFP_HIDDEN; g.sb_j = 1;
@@ -448,16 +483,6 @@ int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* 
     g.M = cols; g.N = CFP_HIDDEN; g.K = m3;
     g.k_per_split = (m3 + BK - 1) / BK * BK;
     return run_gemm<true, false>(g, 1, accumulate, st);
-}
-
-// The split-K workspace, allocated on first use; shared by everything that runs its
-// partial sums and their fold back to back on one stream.
-int dw_workspace(float** work, size_t* floats) {
-    if (!g_dw_work)
-        CFP_HIP_TRY(hipMalloc((void**)&g_dw_work, kDwWorkFloats * sizeof(float)));
-    *work = g_dw_work;
-    *floats = kDwWorkFloats;
-    return 0;
 }
 
 int launch_splitk_reduce(float* dst, const float* part, long count, long stride, int splits,
@@ -469,19 +494,19 @@ int launch_splitk_reduce(float* dst, const float* part, long count, long stride,
 }
 
 int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld_dpre,
-               float* d_dW, hipStream_t st) {
+               float* d_dW, const SeamWork& sw, hipStream_t st) {
     CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW &&
                     ld_dpre >= rows,
                 "cfp_gemm_dw: bad argument (rows must be in 1..%d)", CFP_OBS);
     if (g_gemm_split && gemm_dw_x9_ok(rows, cols))
-        return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, split_terms(), st);
+        return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, split_terms(), sw, st);
     // enough workgroups to fill 256 CUs: tiles(M) * tiles(N=2) * splits
     const int tiles = ((rows + BM - 1) / BM) * (CFP_HIDDEN / BN);
     int splits = (2048 + tiles - 1) / tiles;   // measured: 128 splits of the gate dW beat 64 by 3 %
     const int kblocks = (cols + BK - 1) / BK;
     if (splits > kblocks) splits = kblocks;
     // the workspace holds kMaxSplits slices of the largest dW; a smaller one may use more
-    int max_splits = (int)(kDwWorkFloats / ((size_t)rows * CFP_HIDDEN));
+    int max_splits = (int)(sw.dw_part_floats / ((size_t)rows * CFP_HIDDEN));
     if (max_splits > 4 * kMaxSplits) max_splits = 4 * kMaxSplits;
     if (splits > max_splits) splits = max_splits;
     if (splits < 1) splits = 1;
@@ -497,31 +522,32 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
         g.C = d_dW; g.c_split = 0;
         return run_gemm<false, false>(g, 1, true, st);
     }
-    size_t work_floats = 0;
-    if (dw_workspace(&g_dw_work, &work_floats)) return 1;
-    g.C = g_dw_work;
+    CFP_REQUIRE(sw.dw_part, "cfp_gemm_dw: no split workspace");
+    g.C = sw.dw_part;
     g.c_split = (long)rows * CFP_HIDDEN;
     if (run_gemm<false, false>(g, splits, false, st) != 0) return 1;
     const long count = (long)rows * CFP_HIDDEN;
-    return launch_splitk_reduce(d_dW, g_dw_work, count, count, splits, st);
+    return launch_splitk_reduce(d_dW, sw.dw_part, count, count, splits, st);
 }
 
 int gemm_split_terms() { return g_gemm_split ? split_terms() : 0; }
 
 int gemm_dw_two(int rows_a, int rows_b, int cols, const float* d_x, const float* d_dpre,
-                int ld_dpre, float* d_dW_a, float* d_dW_b, hipStream_t st) {
+                int ld_dpre, float* d_dW_a, float* d_dW_b, const SeamWork& sw, hipStream_t st) {
     CFP_REQUIRE(rows_a > 0 && rows_b > 0 && ld_dpre >= rows_a + rows_b && d_dW_a && d_dW_b,
                 "gemm_dw_two: bad argument");
     if (g_gemm_split && gemm_dw_x9_ok(rows_a + rows_b, cols))
-        return gemm_dw_x9(rows_a + rows_b, cols, d_x, d_dpre, ld_dpre, d_dW_a, split_terms(), st,
+        return gemm_dw_x9(rows_a + rows_b, cols, d_x, d_dpre, ld_dpre, d_dW_a, split_terms(), sw, st,
                           rows_a, d_dW_b);
-    if (gemm_dw_ld(rows_a, cols, d_x, d_dpre, ld_dpre, d_dW_a, st)) return 1;
-    return gemm_dw_ld(rows_b, cols, d_x, d_dpre + rows_a, ld_dpre, d_dW_b, st);
+    if (gemm_dw_ld(rows_a, cols, d_x, d_dpre, ld_dpre, d_dW_a, sw, st)) return 1;
+    return gemm_dw_ld(rows_b, cols, d_x, d_dpre + rows_a, ld_dpre, d_dW_b, sw, st);
 }
 
 }  // namespace cfp
 
 extern "C" {
+
+int cfp_seam_reserve(void) { return seam_default() ? 0 : 1; }
 
 int cfp_set_gemm_bf16(int on) {
     g_gemm_bf16 = on ? 1 : 0;
@@ -539,8 +565,12 @@ int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
                  float* d_y, void* stream) {
     CFP_REQUIRE(m > 0 && cols > 0 && k > 0 && d_W && d_x && d_y,
                 "cfp_gemm_fwd: bad argument");
-    if (g_gemm_split && gemm_fwd_x9_ok(m, cols, k, d_x))
-        return gemm_fwd_x9(m, cols, k, d_W, d_x, d_y, split_terms(), (hipStream_t)stream);
+    if (g_gemm_split && gemm_fwd_x9_ok(m, cols, k, d_x)) {
+        const SeamWork* sw = seam_default();
+        if (!sw) return 1;
+        return gemm_fwd_x9(m, cols, k, d_W, d_x, d_y, split_terms(), sw->w_mirror,
+                           (hipStream_t)stream);
+    }
     GemmArgs g{};
     g.A = d_x; g.sa_i = k; g.sa_k = 1;
     g.B = d_W; g.sb_k = 1; g.sb_j = k;
@@ -557,21 +587,25 @@ int cfp_gemm_enc_fwd(int cols, const float* d_W_enc, const float* d_xobs,
 
 int cfp_gemm_dh(int m3, int cols, const float* d_W, const float* d_dpre,
                 float* d_dh, void* stream) {
-    return gemm_dh_acc(m3, cols, d_W, d_dpre, d_dh, false, (hipStream_t)stream);
+    const SeamWork* sw = seam_default();
+    if (!sw) return 1;
+    return gemm_dh_acc(m3, cols, d_W, d_dpre, d_dh, false, *sw, (hipStream_t)stream);
 }
 
 int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
                 float* d_dW, void* stream) {
-    return gemm_dw_ld(rows, cols, d_x, d_dpre, rows, d_dW, (hipStream_t)stream);
+    const SeamWork* sw = seam_default();
+    if (!sw) return 1;
+    return gemm_dw_ld(rows, cols, d_x, d_dpre, rows, d_dW, *sw, (hipStream_t)stream);
 }
 
 int cfp_gemv_dwv(const float* d_x, const float* d_dv, float* d_dWv, int cols,
                  void* stream) {
     CFP_REQUIRE(cols > 0 && d_x && d_dv && d_dWv, "cfp_gemv_dwv: bad argument");
     hipStream_t st = (hipStream_t)stream;
-    if (!g_gemv_work)
-        CFP_HIP_TRY(hipMalloc((void**)&g_gemv_work,
-                              (size_t)kGemvSlices * CFP_HIDDEN * sizeof(float)));
+    const SeamWork* sw = seam_default();
+    if (!sw) return 1;
+    float* const g_gemv_work = sw->gemv_part;
     int per = (cols + kGemvSlices - 1) / kGemvSlices;
     if (per < 32) per = 32;
     const int slices = (cols + per - 1) / per;

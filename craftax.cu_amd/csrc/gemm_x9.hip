@@ -303,8 +303,8 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             o_lane[(size_t)acc_row(r) * ldc + 32 * t] = acc[t][r];
 }
 
-u4* g_w_x9 = nullptr;   // W mirror of the call in flight: one stream at a time
 constexpr int kDhMaxK = CFP_GRU;
+constexpr size_t kDhMirrorBytes = (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4);   // 1.125 MiB
 
 }  // namespace
 
@@ -315,9 +315,9 @@ bool gemm_dh_x9_ok(int m3, int cols, const float* dpre) {
 
 // out[cols][ldc] (+)= A[cols][K] . B, B(k, u) = B[k*sk + u*su] for 256 units
 static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const float* A,
-                        float* out, int ldc, bool accumulate, int terms, hipStream_t st) {
-    if (!g_w_x9)
-        CFP_HIP_TRY(hipMalloc((void**)&g_w_x9, (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4)));
+                        float* out, int ldc, bool accumulate, int terms, u4* g_w_x9,
+                        hipStream_t st) {
+    CFP_REQUIRE(g_w_x9, "k_dh_x9: no mirror buffer for W");
     const int total = (K / 16) * kDhFrags * 64;
     hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, B, sk, su, g_w_x9,
                        total, terms == 1 ? 1 : 0);
@@ -333,11 +333,14 @@ static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const
     return 0;
 }
 
+size_t dh_mirror_bytes() { return kDhMirrorBytes; }
+
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               int terms, hipStream_t st) {
+               int terms, u4* w_mirror, hipStream_t st) {
     CFP_REQUIRE(gemm_dh_x9_ok(m3, cols, dpre) && W && dh,
                 "gemm_dh_x9: K must be a multiple of 16 up to %d and columns of 32", kDhMaxK);
-    return launch_dh_x9(m3, cols, W, CFP_HIDDEN, 1, dpre, dh, CFP_HIDDEN, accumulate, terms, st);
+    return launch_dh_x9(m3, cols, W, CFP_HIDDEN, 1, dpre, dh, CFP_HIDDEN, accumulate, terms, w_mirror,
+                        st);
 }
 
 // y[cols][m] = x[cols][k] . W[m][k]^T in slices of 256 output rows of W
@@ -346,12 +349,12 @@ bool gemm_fwd_x9_ok(int m, int cols, int k, const float* x) {
 }
 
 int gemm_fwd_x9(int m, int cols, int k, const float* W, const float* x, float* y, int terms,
-                hipStream_t st) {
+                u4* w_mirror, hipStream_t st) {
     CFP_REQUIRE(gemm_fwd_x9_ok(m, cols, k, x) && W && y,
                 "gemm_fwd_x9: m must be a multiple of 256, k of 16 up to %d, columns of 32", kDhMaxK);
     for (int j = 0; j < m / CFP_HIDDEN; j++)
         if (launch_dh_x9(k, cols, W + (size_t)j * CFP_HIDDEN * k, 1, k, x, y + j * CFP_HIDDEN, m,
-                         false, terms, st))
+                         false, terms, w_mirror, st))
             return 1;
     return 0;
 }
@@ -361,15 +364,14 @@ bool gemm_dw_x9_ok(int rows, int cols) {
 }
 
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               int terms, hipStream_t st, int rows_first, float* dW_rest, float* own_work,
-               size_t own_work_floats) {
+               int terms, const SeamWork& sw, hipStream_t st, int rows_first, float* dW_rest) {
     CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows &&
                     (!dW_rest || (rows_first > 0 && rows_first < rows)),
                 "gemm_dw_x9: columns must be a multiple of 8");
-    // a caller that overlaps this GEMM with others brings its own split workspace
-    float* work = own_work;
-    size_t work_floats = own_work_floats;
-    if (!work && dw_workspace(&work, &work_floats)) return 1;
+    // GEMMs that overlap each other need split workspaces of their own
+    float* work = sw.dw_part;
+    const size_t work_floats = sw.dw_part_floats;
+    CFP_REQUIRE(work, "gemm_dw_x9: no split workspace");
     const int groups = (rows + kX9GroupRows - 1) / kX9GroupRows;
     const int total_iters = (cols + kX9IterCols - 1) / kX9IterCols;
     int splits = 256 / groups;   // one workgroup per CU

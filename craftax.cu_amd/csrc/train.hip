@@ -148,10 +148,14 @@ struct cfp_trainer {
     float* termf = nullptr;    // [n]
     float* av_tmp = nullptr;   // [n][44]
     // second stream of the backward pass (the layers' dependent chain alternates between
-    // it and the caller's, see cfp_train_backward) and the dW GEMMs' own split workspaces
+    // it and the caller's, see cfp_train_backward)
     hipStream_t st2 = nullptr;
     hipEvent_t ev_dh[CFP_MAX_LAYERS] = {};
     hipEvent_t ev_join = nullptr;
+    // GEMM scratch owned by this trainer: `sw` for the chain's GEMMs, and a split
+    // workspace per layer for the gate dW GEMMs that run beside the chain
+    SeamWork sw;
+    SeamWork sw_layer[CFP_MAX_LAYERS];
     float* dw_work2 = nullptr;
     size_t dw_work2_floats = 0;
     // cfp_train_update's captured iteration (epochs x minibatches x (backward, Adam)) and
@@ -169,6 +173,7 @@ extern "C" {
 void cfp_train_destroy(cfp_trainer* tr) {
     if (!tr) return;
     for (void* q : tr->owned) (void)hipFree(q);
+    seam_work_destroy(&tr->sw);
     for (hipEvent_t e : tr->ev_dh)
         if (e) (void)hipEventDestroy(e);
     if (tr->ev_join) (void)hipEventDestroy(tr->ev_join);
@@ -262,6 +267,11 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     tr->dw_work2_floats = (size_t)48 * G * H;   // per layer: 48 splits of a gate dW
     TA(dw_work2, (size_t)tr->L * tr->dw_work2_floats * sizeof(float));
 #undef TA
+    if (ok) ok = seam_work_create(&tr->sw) == 0;
+    for (int l = 0; ok && l < tr->L; l++) {
+        tr->sw_layer[l].dw_part = tr->dw_work2 + (size_t)l * tr->dw_work2_floats;
+        tr->sw_layer[l].dw_part_floats = tr->dw_work2_floats;
+    }
     // default priority, as every stream of this library
     if (ok) ok = hipStreamCreateWithFlags(&tr->st2, hipStreamNonBlocking) == hipSuccess &&
                  hipEventCreateWithFlags(&tr->ev_join, hipEventDisableTiming) == hipSuccess;
@@ -487,9 +497,9 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         if (launch_head(ha, st)) return 1;
         if (launch_fold_f64(tr->block_loss, head_blocks(cols), 3, tr->loss_acc, true, st)) return 1;
         // dh3 = [dlogits | dvalue] . [W_a ; W_v]; dW_a and dW_v from one GEMM; bias sums
-        if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, st)) return 1;
+        if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, tr->sw, st)) return 1;
         if (gemm_dw_two(A, 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L),
-                        g + CFP_OFF_W_V(L), st))
+                        g + CFP_OFF_W_V(L), tr->sw, st))
             return 1;
         if (colsum_into(tr, tr->dlogits, kHeadLd, g + CFP_OFF_B_A(L), A, cols, st)) return 1;
         if (colsum_into(tr, tr->dlogits + A, kHeadLd, g + CFP_OFF_B_V(L), 1, cols, st)) return 1;
@@ -514,17 +524,16 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             if (launch_gru_reverse(ra, chain)) return 1;
             if (!overlap &&
                 gemm_dw_ld(G, cols, tr->x[l], tr->preb[l], G, g + CFP_OFF_W_GRU + (size_t)l * G * H,
-                           chain))
+                           tr->sw, chain))
                 return 1;
             // layer 0: dh_enc = W_0^T dpre + highway, accumulated onto the highway term
             if (gemm_dh_acc(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
-                            l == 0 ? tr->dhX : tr->dhG, l == 0, chain))
+                            l == 0 ? tr->dhX : tr->dhG, l == 0, tr->sw, chain))
                 return 1;
             if (overlap) {
                 CFP_HIP_TRY(hipEventRecord(tr->ev_dh[l], chain));
                 if (gemm_dw_x9(G, cols, tr->x[l], tr->preb[l], G,
-                               g + CFP_OFF_W_GRU + (size_t)l * G * H, terms, chain, 0, nullptr,
-                               tr->dw_work2 + (size_t)l * tr->dw_work2_floats, tr->dw_work2_floats))
+                               g + CFP_OFF_W_GRU + (size_t)l * G * H, terms, tr->sw_layer[l], chain))
                     return 1;
                 CFP_HIP_TRY(hipStreamWaitEvent(other, tr->ev_dh[l], 0));
                 hipStream_t t = chain; chain = other; other = t;
@@ -538,9 +547,10 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             // map bytes straight from the records; xobs is free by now and takes the
             // 76-float rows of the fp32 remainder
             if (dw_enc_records(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
-                               env_start, chain))
+                               env_start, tr->sw, chain))
                 return 1;
-        } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, chain)) {
+        } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, tr->sw,
+                              chain)) {
             return 1;
         }
         if (overlap) {
@@ -610,18 +620,12 @@ int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
         tr->tgraph = nullptr;
     }
     if (!tr->texec) {
-        // Warm-up as in the reference (:13379-13386): one bare backward, no Adam, so that
-        // the lazily allocated GEMM workspaces exist before the capture (an allocation
-        // inside a capture is illegal); parameters stay untouched, the gradients it
-        // left are cleared again.
-        int rc = cfp_train_backward(tr, 0, tr->mb, st);
-        if (rc != 0) return rc;
-        hipLaunchKernelGGL(k_fill, dim3(grid1(tr->p->param_count)), dim3(256), 0, st, tr->grads,
-                           tr->p->param_count, 0.0f);
-        CFP_HIP_TRY(hipGetLastError());
+        // No warm-up pass (the reference runs one, :13379-13386, to get cuBLAS's lazy
+        // workspaces allocated before the capture): every buffer the iteration touches,
+        // GEMM scratch included, was allocated by cfp_train_create.
         CFP_HIP_TRY(hipStreamSynchronize(st));
         CFP_HIP_TRY(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-        rc = train_body(tr, st);
+        const int rc = train_body(tr, st);
         hipGraph_t g = nullptr;
         const hipError_t ec = hipStreamEndCapture(st, &g);   // always leaves capture mode
         if (rc != 0) {

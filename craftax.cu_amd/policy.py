@@ -328,6 +328,10 @@ def gemm_dh(W, dpre, dh=None):
     return dh
 
 
+def seam_reserve():
+    _check(lib().cfp_seam_reserve())
+
+
 def gemm_dw(x, dpre, dW):
     """dW[rows][256] += dpre[cols][rows]^T . x[cols][256] (cu_gemm_dw :11642)."""
     cols, rows = dpre.shape

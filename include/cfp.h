@@ -6,7 +6,9 @@
  * The reference exposes no FFI for this path, so the seam kept here is the
  * call surface of its rollout/trainer layers: same argument order, same
  * tensor layouts, same "all work is enqueued on the given stream, nothing is
- * allocated inside a step" contract.
+ * allocated inside a step" contract: a policy or trainer object owns every buffer
+ * its entry points touch (allocated by its create call); the raw GEMM entry points
+ * of the dense-math seam share one process-wide workspace, see cfp_seam_reserve.
  *
  * Conventions
  *   - All pointers named d_* / documented "device" are HIP device pointers.
@@ -169,6 +171,16 @@ int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
                        float* d_av, int n, int chunk, void* stream);
 
 /* ---- the dense-math seam (craftax_full.cu:11604-11666) ------------------- */
+/* Workspace of the raw entry points below (cfp_gemm_fwd / dh / dw, cfp_gemv_dwv):
+ * 1.1 MB for the split mirror of W, 110 MB of split-K partial sums, 256 KB of gemv
+ * slices, allocated once per process -- by this call, or by the first of those entry
+ * points that needs it (the reference warms cuBLAS's workspaces the same way before it
+ * captures a graph, craftax_full.cu:12094-12122).  Call it before capturing a stream
+ * that uses them.  The workspace has one user at a time: raw seam calls in flight
+ * together must be on one stream.  Trainer objects do not use it (they own theirs).
+ * cfp_set_gemm_bf16 / cfp_set_gemm_split are process-wide and not synchronised: set
+ * them while no other thread is inside the library. */
+int cfp_seam_reserve(void);
 /* bf16 inputs with fp32 accumulation for every GEMM of this seam (cfp_gemm_fwd /
  * enc_fwd / dh / dw, hence the whole PPO update): the reference's process-wide
  * CF_GEMM_BF16 / g_gemm_bf16 switch (craftax_full.cu:11306-11316, wrappers
@@ -350,11 +362,11 @@ int cfp_train_adam(cfp_trainer* tr, void* stream);
  * statistics already in place): epochs x (loss sums reset, minibatches x
  * (cfp_train_backward of the m-th contiguous env slice, cfp_train_adam)), then a
  * synchronisation of the stream, as in the reference.  use_graph != 0 is the
- * reference's graph mode: the first call runs one bare backward as a warm-up
- * (no Adam, parameters untouched; the grads arena is cleared afterwards, so it
- * must hold nothing the caller still needs), captures the iteration once on
- * `stream` (on a stream of the trainer's own when `stream` is NULL, which cannot
- * be captured) and replays it; later calls only replay.  lr, the entropy
+ * reference's graph mode: the first call captures the iteration once on `stream`
+ * (on a stream of the trainer's own when `stream` is NULL, which cannot be
+ * captured) and replays it; later calls only replay.  No warm-up pass is needed
+ * (the reference runs one for cuBLAS's lazy workspaces): the trainer owns every
+ * buffer the iteration touches.  lr, the entropy
  * coefficient and the Adam step counter live in device memory, so replays see
  * their current values.  A change of cfp_set_gemm_split / cfp_set_gemm_bf16 /
  * cfp_policy_set_gemm_bf16 between calls makes the next call capture again.
@@ -368,8 +380,8 @@ int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream);
 
 /* ---- synthetic inputs for parity tests and bench (no reference
  *      counterpart; counter-based so host and device agree bit for bit) ---- */
-/* Records: 792 map bytes, each 0 with prob 0.4 else U{0..40}... see synth.hip;
- * tail floats U[0,1) with 24-bit mantissas.  index = env + n*step. */
+/* Records: 792 map bytes, each U{0..40}; 51 tail floats U[0,1) on a 24-bit grid.
+ * Dword d of env e at step s is a function of (seed, s, 249 e + d) alone. */
 int cfp_synth_records(uint8_t* d_rec, int n, uint64_t seed, uint64_t step,
                       void* stream);
 
