@@ -53,6 +53,7 @@ PROTOTYPES = {
     "cfp_gemm_enc_fwd": (C.c_int, [C.c_int, vp, vp, vp, vp]),
     "cfp_seam_reserve": (C.c_int, []),
     "cfp_gemm_dh": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),
+    "cfp_gemm_dh_noalloc": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),
     "cfp_gemm_dw": (C.c_int, [C.c_int, C.c_int, vp, vp, vp, vp]),
     "cfp_gemv_dwv": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "cfp_expand_obs": (C.c_int, [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int,

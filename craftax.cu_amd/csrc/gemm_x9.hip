@@ -25,7 +25,14 @@
 //               split in registers.  Same software pipeline as the record-fed
 //               encoder kernel.
 //   output    : per-split partial sums, folded in a fixed order.
+#include <mutex>
+
 #include "policy_tile.h"
+
+// W mirror of cfp_gemm_dh_noalloc (below): the split, MFMA-ordered copy of W that
+// k_dh_x9 reads, for K up to 768 rows -- 48 K steps x 24 fragments x 64 lanes x 16 bytes.
+// Every GPU the library runs on holds its own copy until the process ends.
+static __device__ __align__(256) unsigned char scratch[(CFP_GRU / 16) * 24 * 64 * 16];
 
 namespace cfp {
 namespace {
@@ -358,6 +365,49 @@ int gemm_fwd_x9(int m, int cols, int k, const float* W, const float* x, float* y
             return 1;
     return 0;
 }
+
+}  // namespace cfp
+
+// Device address of `scratch` on each GPU, resolved on the first call made with that GPU
+// current: the array's name is only a host-side handle, each device has its own copy.
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+}  // namespace
+
+extern "C" int cfp_gemm_dh_noalloc(int m3, int cols, const float* d_W, const float* d_dpre,
+                                   float* d_dh, void* stream) {
+    using namespace cfp;
+    static_assert(sizeof(scratch) == kDhMirrorBytes, "scratch holds one W mirror");
+    CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh_noalloc: bad argument");
+    CFP_REQUIRE(m3 <= kDhMaxK, "cfp_gemm_dh_noalloc: m3 = %d exceeds the %d rows its W mirror holds",
+                m3, kDhMaxK);
+    CFP_REQUIRE(gemm_dh_x9_ok(m3, cols, d_dpre),
+                "cfp_gemm_dh_noalloc: m3 must be a multiple of 16, cols of 32 and dpre 16-byte "
+                "aligned (got m3 = %d, cols = %d)", m3, cols);
+    int dev = -1;
+    CFP_HIP_TRY(hipGetDevice(&dev));
+    CFP_REQUIRE(dev >= 0 && dev < kMaxDevices, "cfp_gemm_dh_noalloc: device index %d out of range", dev);
+    void* ptr = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        if (!g_scratch_ptr[dev]) {
+            void* p = nullptr;
+            CFP_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            CFP_REQUIRE(p, "cfp_gemm_dh_noalloc: no device address for the W mirror");
+            g_scratch_ptr[dev] = p;
+        }
+        ptr = g_scratch_ptr[dev];
+    }
+    // same arithmetic as cfp_gemm_dh runs for this shape: nine exact partial products
+    // unless the process-wide switches ask for six, or for bf16 inputs
+    const int terms = gemm_split_terms() ? gemm_split_terms() : 9;
+    return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, false, terms, reinterpret_cast<u4*>(ptr),
+                      (hipStream_t)stream);
+}
+
+namespace cfp {
 
 bool gemm_dw_x9_ok(int rows, int cols) {
     return rows > 0 && cols >= 8 && cols % 8 == 0;

@@ -328,6 +328,14 @@ def gemm_dh(W, dpre, dh=None):
     return dh
 
 
+def gemm_dh_noalloc(W, dpre, dh):
+    """cfp_gemm_dh_noalloc: as gemm_dh, the W mirror in the library's own device array;
+    the caller brings the output (nothing is allocated on the way)."""
+    _check(lib().cfp_gemm_dh_noalloc(W.shape[0], dpre.shape[0], _ptr(W), _ptr(dpre), _ptr(dh),
+                                     _stream()))
+    return dh
+
+
 def seam_reserve():
     _check(lib().cfp_seam_reserve())
 

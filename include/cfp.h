@@ -211,6 +211,15 @@ int cfp_gemm_enc_fwd(int cols, const float* d_W_enc, const float* d_xobs,
 /* cu_gemm_dh (:11629): dh[cols][256] = dpre[cols][m3] . W[m3][256]. */
 int cfp_gemm_dh(int m3, int cols, const float* d_W, const float* d_dpre,
                 float* d_dh, void* stream);
+/* cfp_gemm_dh for callers that cannot allocate (code under graph capture, serving loops,
+ * harnesses that forbid hipMalloc); no counterpart in the reference.  Same result as
+ * cfp_gemm_dh, but the split mirror of W sits in a 1.125 MiB array inside the library's
+ * device image instead of the process-wide workspace, so the call never allocates.
+ * Limits: m3 a multiple of 16 up to 768, cols a multiple of 32, d_dpre 16-byte aligned;
+ * anything else is an error.  Calls on one GPU share that GPU's array: calls that overlap
+ * (two streams, two threads) race on it. */
+int cfp_gemm_dh_noalloc(int m3, int cols, const float* d_W, const float* d_dpre,
+                        float* d_dh, void* stream);
 /* cu_gemm_dw (:11642): dW[rows][256] += dpre[cols][rows]^T . x[cols][256]. */
 int cfp_gemm_dw(int rows, int cols, const float* d_x, const float* d_dpre,
                 float* d_dW, void* stream);
