@@ -11,11 +11,13 @@ launch per step; the 16 x 16 384 chunked schedule is timed beside it.
 
 Prints ONE JSON line (metric = env-steps/s) with two extra objects:
   roofline     algorithmic FLOPs per launch / measured launch time (HIP events on
-               the launch stream) vs the matrix-pipe bound of the kernel's
-               instruction mix: fp32 MFMA (157.3 TFLOP/s) for all but the
+               the launch stream) against the fp32 MFMA peak (157.3 TFLOP/s).
+               Beside it, as extra keys, the bound of the kernel's actual
+               instruction mix: all FLOPs issue on the fp32 MFMA except the
                encoder's byte-valued features, which issue as three bf16 MFMAs
-               per product (2.5 PFLOP/s); the fraction of the plain fp32 MFMA
-               peak is reported beside it
+               per product (2.5 PFLOP/s).  `traffic` is read from the tracked
+               counter summary under profiles/ and is null when that summary
+               was taken from other kernel sources than the ones present
   cpu_baseline the CPU oracle's scalar fp32 forward timed on this host's cores
                on a bounded sample of the same workload
 """
@@ -45,11 +47,36 @@ T_BOUND_PER_ENV_STEP = (FLOP_FP32_PIPE / (PEAK_FP32_MFMA_TFLOPS * 1e12) +
                         FLOP_BF16_PIPE_ISSUED / (PEAK_BF16_MFMA_TFLOPS * 1e12))
 PEAK_MIX_TFLOPS = FLOP_PER_ENV_STEP / T_BOUND_PER_ENV_STEP / 1e12   # 196.9
 LAYERS = 3
-# HBM bytes per launch at 262 144 envs from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/policy_forward_262144_pmc.txt), scaled by the factors the same counters
-# show for a plain 1 GiB copy (FETCH_SIZE x2.0, WRITE_SIZE x1.0); None until
-# measured for another size.
-MEASURED_TRAFFIC_BYTES = {262144: 2220562918}
+KERNEL_SOURCES = ("policy_forward.hip", "policy_tile.h", "cfp_common.h")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "policy_forward_262144_pmc.txt")
+
+
+def kernel_source_id():
+    """sha1 over the sources of k_policy_forward: ties a counter summary to a build."""
+    import hashlib
+    h = hashlib.sha1()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "craftax.cu_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def measured_traffic(n):
+    """HBM bytes per launch from the tracked rocprofv3 FETCH_SIZE / WRITE_SIZE summary
+    (already scaled by what the counters read for a plain copy), or None when the
+    summary is missing, was taken at another batch size or from other kernel sources."""
+    import re
+    try:
+        text = open(TRAFFIC_PROFILE).read()
+    except OSError:
+        return None
+    def field(key):
+        m = re.search(r"^" + key + r"\s*=\s*(\S+)", text, flags=re.M)
+        return m.group(1) if m else None
+    if field("envs") != str(n) or field("kernel_source_sha1") != kernel_source_id():
+        return None
+    t = field("traffic_bytes_per_launch")
+    return int(t) if t and t.isdigit() else None
 
 
 def parse():
@@ -198,15 +225,17 @@ def main():
         "pct_fp32_mfma_peak": 100.0 * achieved / PEAK_FP32_MFMA_TFLOPS,
         "chunked_16x16384": results.get("chunked_16x16384"),
         "bf16_in_fp32_acc_unchunked": bf16,
-        # peak = algorithmic FLOPs / matrix-pipe time bound of the kernel's instruction
-        # mix (fp32 pipe at 157.3, the encoder's byte features on the bf16 pipe at 2500)
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MIX_TFLOPS,
-                     "unit": "TFLOP/s", "frac": achieved / PEAK_MIX_TFLOPS,
-                     "frac_of_fp32_mfma_peak": achieved / PEAK_FP32_MFMA_TFLOPS,
+        "kernel_source_sha1": kernel_source_id(),
+        # algorithmic FLOPs per launch / launch time against the fp32 MFMA peak; the
+        # mixed-pipe keys price the same launch against the bound of its instruction mix
+        # (fp32 pipe at 157.3, the encoder's byte features on the bf16 pipe at 2500)
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_FP32_MFMA_TFLOPS,
+                     "mixed_pipe_peak": PEAK_MIX_TFLOPS,
+                     "frac_of_mixed_pipe_bound": achieved / PEAK_MIX_TFLOPS,
                      "fp32_pipe_flops_per_launch": FLOP_FP32_PIPE * n // launches,
                      "bf16_pipe_issued_flops_per_launch": FLOP_BF16_PIPE_ISSUED * n // launches,
-                     "traffic": (MEASURED_TRAFFIC_BYTES[n] // launches
-                                 if n in MEASURED_TRAFFIC_BYTES else None),
+                     "traffic": measured_traffic(n) if launches == 1 else None,
                      "kernel": "k_policy_forward",
                      "flops_per_launch": FLOP_PER_ENV_STEP * n // launches,
                      "algorithmic_hbm_bytes_per_launch": BYTES_PER_ENV_STEP * n // launches,

@@ -6,9 +6,10 @@
 // draws its uniform from cuRAND: curand_init(seed ^ 0xA5A5..., subsequence = env,
 // offset = device step counter) of a Philox4_32_10 state, then curand_uniform.
 // Here the same draw is computed directly (philox_uniform in cfp_common.h): the
-// Philox4x32-10 block function is pinned by the published known-answer vectors;
-// the mapping of (seed, subsequence, offset) onto key and counter follows cuRAND's
-// documented state layout and could only be confirmed against a CUDA run.  Given
+// Philox4x32-10 block function is pinned by the published known-answer vectors,
+// the mapping of (seed, subsequence, offset) onto key, counter and output word by
+// rocRAND's engine (same three arguments; CPU test of the oracle's twin of
+// philox_uniform), the conversion to a float is cuRAND's x * 2^-32 + 2^-33.  Given
 // the uniform, the action and its log-probability follow the reference's
 // arithmetic exactly (max-shifted expf, ascending cumulative sum, first index
 // with target <= cum, last action as the fall-through).

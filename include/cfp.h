@@ -106,8 +106,9 @@ int cfp_policy_get_params(const cfp_policy* p, float* host_params, size_t count)
  * rest, u = the first curand_uniform of a Philox4_32_10 state after
  * curand_init(seed, s, i) (the reference passes seed 1234).  Replaces the
  * Xavier-uniform weights cfp_policy_create made and refreshes the mirrors.  The
- * Philox block function is checked against published vectors; cuRAND's mapping of
- * (seed, subsequence, offset) onto it is taken from its documentation. */
+ * Philox block function is checked against published vectors, the mapping of
+ * (seed, subsequence, offset) onto it against rocRAND's engine, which takes the same
+ * three arguments; the float is cuRAND's x * 2^-32 + 2^-33. */
 int cfp_policy_init_reference(cfp_policy* p, uint64_t seed);
 /* Rebuild the MFMA-ordered weight mirrors from the params arena after the
  * arena changed on device: the role of cu_params_refresh_bf16 + cu_pack_wav

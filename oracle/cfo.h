@@ -20,11 +20,13 @@
  *                           normalisation of exp(logprob))
  *   cfo_philox4x32_10       pinned: the three known-answer vectors published with
  *                           the generator (Random123 kat_vectors, philox4x32 10)
- *   cfo_philox_uniform      "parity unpinned": how cuRAND maps (seed, subsequence,
- *                           offset) onto Philox key / counter / output word is
- *                           restated from its documentation; only a CUDA run could
- *                           confirm it.  The reference's weight-init stream
- *                           (k_nn_init_weights) is not restated.
+ *   cfo_philox_draw         pinned: rocRAND's Philox4x32-10 engine on the host
+ *                           (rocrand_init(seed, subsequence, offset) + rocrand), the
+ *                           ROCm routine with curand_init's three arguments, over
+ *                           thousands of triples (oracle/rocrand_check.cpp)
+ *   cfo_philox_uniform      the draw through cuRAND's published conversion
+ *                           x * 2^-32 + 2^-33 (rocRAND adds 2^-32, so the float
+ *                           itself has no library to be held to: closed form only)
  */
 #ifndef CFO_H_
 #define CFO_H_
@@ -89,6 +91,7 @@ int cfo_sample_action(const float* logits, int actions, float u, float* logprob)
 /* Philox4x32-10 and the uniform of the reference's sampler (k_value_sample,
  * craftax_full.cu:9732-9736: curand_init(seed ^ 0xA5A5.., env, step) + curand_uniform). */
 void cfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+uint32_t cfo_philox_draw(uint64_t seed, uint64_t subsequence, uint64_t offset);
 float cfo_philox_uniform(uint64_t seed, uint64_t subsequence, uint64_t offset);
 float cfo_sample_margin(const float* logits, int actions, float u);
 

@@ -237,18 +237,25 @@ void cfo_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t ou
     out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
 }
 
-/* First curand_uniform() after curand_init(seed, subsequence, offset) of a Philox
- * state, by cuRAND's documented layout: key = seed, counter = subsequence * 2^64 +
- * offset / 4, output word offset % 4, uniform = x * 2^-32 + 2^-33 (one fused
- * multiply-add, as nvcc contracts it). */
-float cfo_philox_uniform(uint64_t seed, uint64_t subsequence, uint64_t offset) {
+/* First 32-bit draw after curand_init(seed, subsequence, offset) of a Philox state:
+ * key = seed, counter = subsequence * 2^64 + offset / 4, output word offset % 4.
+ * Pinned against rocRAND's rocrand_init + rocrand (tests/test_oracle_policy.py). */
+uint32_t cfo_philox_draw(uint64_t seed, uint64_t subsequence, uint64_t offset) {
     const uint64_t blk = offset >> 2;
     const uint32_t ctr[4] = {(uint32_t)blk, (uint32_t)(blk >> 32), (uint32_t)subsequence,
                              (uint32_t)(subsequence >> 32)};
     const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
     uint32_t out[4];
     cfo_philox4x32_10(ctr, key, out);
-    return fmaf((float)out[offset & 3], 2.3283064365386963e-10f, 1.1641532182693481e-10f);
+    return out[offset & 3];
+}
+
+/* curand_uniform of that draw: x * 2^-32 + 2^-33, in (0, 1] (cuRAND's _curand_uniform;
+ * the product is exact, so fused or not gives the same float).  rocRAND adds 2^-32
+ * instead, which is why the float is not what the rocRAND check compares. */
+float cfo_philox_uniform(uint64_t seed, uint64_t subsequence, uint64_t offset) {
+    return fmaf((float)cfo_philox_draw(seed, subsequence, offset), 2.3283064365386963e-10f,
+                1.1641532182693481e-10f);
 }
 
 /* Distance of u*total from the nearest cumulative-sum boundary, relative to

@@ -3,8 +3,9 @@ sampling (cfp_value_sample), reward/done recording (cfp_record_rd), the policy
 half of a rollout step (cfp_rollout_step) and the bootstrap value
 (cfp_train_bootstrap).
 
-The uniform behind each draw is this library's counter generator (the reference's
-cuRAND Philox stream cannot be reproduced without CUDA: parity unpinned); given
+The uniform behind each draw is computed directly from Philox4x32-10 with curand_init's
+(seed, subsequence, offset) mapping; the CPU oracle's version of it is held to rocRAND's
+engine in tests/test_oracle_policy.py, and the device's to the oracle's here.  Given
 the uniform, actions and log-probabilities follow cf_nn_sample_action
 (craftax_full.cu:9147-9165) and are checked against its C restatement.  Actions
 must agree except where u*total lies within 1e-6 (relative) of a cumulative-sum

@@ -340,8 +340,8 @@ def test_philox_known_answer_vectors():
 def test_philox_uniform_state_layout():
     """cfo_philox_uniform against the block function: key = seed, counter low half =
     offset / 4, high half = subsequence, word = offset % 4, uniform = x * 2^-32 +
-    2^-33 in (0, 1].  (That cuRAND lays its state out this way is taken from its
-    documentation: parity unpinned.)"""
+    2^-33 in (0, 1] (cuRAND's conversion; the state layout itself is held to rocRAND's
+    engine in test_philox_draw_matches_rocrand)."""
     seed, sub = 0x0123456789ABCDEF, (7 << 32) | 99
     lib = ob.cfo()
     for off in (0, 1, 2, 3, 4, 5, 11, (1 << 34) + 2):
@@ -354,3 +354,86 @@ def test_philox_uniform_state_layout():
     u = ob.philox_uniforms(1234, range(20000), 5)
     assert abs(u.mean() - 0.5) < 0.01 and abs(u.var() - 1.0 / 12.0) < 0.005
     assert len(np.unique(u)) > 19900
+
+
+def test_philox_draw_matches_rocrand():
+    """cfo_philox_draw(seed, subsequence, offset) -- the 32-bit word behind the sampler's
+    uniform -- against a library routine with the same three arguments: ROCm's rocRAND
+    Philox4x32-10 engine on the host (rocrand_init followed by one rocrand), built by
+    oracle/Makefile.  Offsets cover every residue mod 4, values past 2^32 and the carry
+    of offset / 4 into the counter's second word; subsequences and seeds use all 64
+    bits.  A wrong word order, swapped counter halves or an off-by-one in the output
+    word fails here.  The float conversion is cuRAND's x * 2^-32 + 2^-33 (rocRAND adds
+    2^-32 instead): closed form, test_philox_uniform_state_layout."""
+    import ctypes as C
+    import os
+    path = os.path.join(os.path.dirname(ob.CFO_PATH), "librocrand_check.so")
+    if not os.path.exists(path):
+        pytest.skip("oracle/librocrand_check.so not built (needs hipcc)")
+    lib = C.CDLL(path)
+    lib.cfo_rocrand_draws.argtypes = [C.c_uint64, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p]
+    mine = ob.cfo()
+    mine.cfo_philox_draw.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64]
+    mine.cfo_philox_draw.restype = C.c_uint32
+    rng = np.random.default_rng(77)
+    total = 0
+    for seed in (0, 1234, 1234 ^ 0xA5A5A5A5A5A5A5A5, 0xFFFFFFFFFFFFFFFF, 0x0123456789ABCDEF):
+        sub = np.concatenate([np.arange(8, dtype=np.uint64),
+                              rng.integers(0, 1 << 63, 600, dtype=np.uint64) * np.uint64(2) + np.uint64(1),
+                              np.array([(1 << 32) - 1, 1 << 32, (1 << 64) - 1], dtype=np.uint64)])
+        off = np.concatenate([np.arange(16, dtype=np.uint64),
+                              rng.integers(0, 1 << 40, 580, dtype=np.uint64),
+                              np.array([(1 << 34) - 1, 1 << 34, (1 << 34) + 1, (1 << 34) + 2, (1 << 34) + 3,
+                                        (1 << 62) + 1, (1 << 63) + 2, (1 << 64) - 1, (1 << 64) - 4],
+                                       dtype=np.uint64)])[: sub.size]
+        sub = sub[: off.size]
+        want = np.zeros(sub.size, dtype=np.uint32)
+        lib.cfo_rocrand_draws(seed, sub.ctypes.data, off.ctypes.data, sub.size, want.ctypes.data)
+        got = np.array([mine.cfo_philox_draw(seed, int(s), int(o)) for s, o in zip(sub, off)],
+                       dtype=np.uint32)
+        assert np.array_equal(got, want), (hex(seed), np.flatnonzero(got != want)[:5])
+        assert set(int(o) & 3 for o in off) == {0, 1, 2, 3}
+        # and the uniform is that draw through cuRAND's conversion
+        u = np.array([mine.cfo_philox_uniform(seed, int(s), int(o)) for s, o in zip(sub[:64], off[:64])],
+                     dtype=np.float32)
+        assert np.array_equal(u, (want[:64].astype(np.float32).astype(np.float64) * 2.0 ** -32
+                                  + 2.0 ** -33).astype(np.float32))
+        total += sub.size
+    assert total >= 3000
+
+
+def test_ppo_loss_closed_form_with_zero_head_weights():
+    """cfo_ppo_loss_f64's value, not only its derivative: with W_a = 0, b_a = 0, W_v = 0
+    the policy is uniform whatever the trunk computes, so per sample
+        H = ln 43,  ratio = exp(-ln 43 - old_logp),  v = b_v,
+        pg = -min(ratio * A, clip(ratio, 1 - eps, 1 + eps) * A),  value term = (b_v - ret)^2 / 2
+    with A the advantage normalised by the whole batch's mean and 1 / (std + 1e-8)."""
+    params = random_params(L, 61)
+    W_enc, b_enc, W_gru, W_a, b_a, W_v, b_v = split_params(params, L)
+    o_wa = OBS * HIDDEN + HIDDEN + L * GRU * HIDDEN
+    p = params.copy()
+    p[o_wa: o_wa + ACTIONS * HIDDEN + ACTIONS + HIDDEN] = 0.0     # W_a, b_a, W_v
+    bv = float(p[-1])
+    n, T = 5, 4
+    ro = _consistent_rollout(p, n, T, 62, done_p=0.2)
+    rng = np.random.default_rng(63)
+    ro["r_logprob"] = (-np.log(ACTIONS) + 0.4 * rng.standard_normal((T, n))).astype(np.float32)
+    clip, vf, ent = 0.2, 0.5, 0.01
+    batch, keep = ob.make_batch(T, n, 0, n, L, T, **ro, clip=clip, vf=vf, ent=ent)
+    total, l3 = ob.ppo_loss_f64(p, batch)
+    adv = ro["adv"].astype(np.float64)
+    mean = adv.mean()
+    std = np.sqrt(max((adv * adv).mean() - mean * mean, 0.0))
+    A = (adv - np.float32(mean)) * (1.0 / (np.float32(std) + np.float32(1e-8)))
+    ratio = np.exp(-np.log(ACTIONS) - ro["r_logprob"].astype(np.float64))
+    pg = -np.minimum(ratio * A, np.clip(ratio, 1 - clip, 1 + clip) * A)
+    assert (np.abs(ratio - 1) > clip).any() and (np.abs(ratio - 1) < clip).any()   # both branches
+    vterm = 0.5 * (bv - ro["ret"].astype(np.float64)) ** 2
+    want = np.array([pg.sum(), vterm.sum(), n * T * np.log(ACTIONS)])
+    assert np.allclose(l3, want, rtol=1e-6, atol=1e-9), (l3, want)
+    # the total is that combination of the three sums (the coefficients travel as fp32)
+    assert abs(total - (l3[0] + float(np.float32(vf)) * l3[1] - float(np.float32(ent)) * l3[2]) / (n * T)) < 1e-12
+    assert abs(total - (want[0] + vf * want[1] - ent * want[2]) / (n * T)) < 1e-7
+    # the backward pass reports the same sums
+    g, l3b = ob.ppo_backward_f64(p, batch)
+    assert np.allclose(l3b, want, rtol=1e-6, atol=1e-9)
