@@ -99,10 +99,15 @@ def ppo_update(pkg, torch, reps):
     pkg.policy.set_gemm_bf16(True)       # same update with bf16 GEMM inputs
     try:
         ms16 = _time(torch, step, reps, warm=1)
+        tr.set_bf16_storage(True)        # ... and the window workspace stored as bf16
+        ms16s = _time(torch, step, reps, warm=1)
     finally:
+        tr.set_bf16_storage(False)
         pkg.policy.set_gemm_bf16(False)
     out["bf16_in"] = {"ms_per_update": ms16, "samples_per_s": samples / ms16 * 1e3,
                       "tflops": UPD_FLOP * samples / ms16 / 1e9}
+    out["bf16_in_bf16_storage"] = {"ms_per_update": ms16s, "samples_per_s": samples / ms16s * 1e3,
+                                   "tflops": UPD_FLOP * samples / ms16s / 1e9}
     assert torch.isfinite(pol.params).all()
     tr.close()
     pol.close()

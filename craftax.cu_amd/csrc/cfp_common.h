@@ -132,6 +132,7 @@ struct FwdArgs {
     // every layer's gate pre-activations and output are written out for the
     // reverse pass.  tr_x[0] is filled through h_enc_out.
     int train;
+    int tr_bf16;             // bf16-input kernel only: tr_pre / tr_x (tr_x[0] included) are bf16 arrays
     int tr_t0, tr_mb, tr_n_all, tr_env_start;
     float* tr_pre[CFP_MAX_LAYERS];   // [cols][768]: zh | zg | zp
     float* tr_x[CFP_MAX_LAYERS + 1]; // [cols][256]: tr_x[l+1] = output of layer l
@@ -189,7 +190,7 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
 bool gemm_dw_x9_ok(int rows, int cols);
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
                int terms, const SeamWork& sw, hipStream_t st, int rows_first = 0,
-               float* dW_rest = nullptr);
+               float* dW_rest = nullptr, bool dpre_bf16 = false, bool x_bf16 = false);
 // partial products per product the split kernels run with now (9, 6, or 1 with bf16
 // inputs); 0 when they are switched off
 int gemm_split_terms();
@@ -202,7 +203,7 @@ int gemm_dw_two(int rows_a, int rows_b, int cols, const float* x, const float* d
 // cols % 32 == 0, dpre 16-byte aligned)
 bool gemm_dh_x9_ok(int m3, int cols, const float* dpre);
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               int terms, u4* w_mirror, hipStream_t st);
+               int terms, u4* w_mirror, hipStream_t st, bool dpre_bf16 = false);
 size_t dh_mirror_bytes();   // size of the split mirror of W (K up to 768)
 
 // y[cols][m] = x[cols][k] . W[m][k]^T on the same kernel (m % 256 == 0, k % 16 == 0,

@@ -60,10 +60,18 @@ constexpr int kX9GroupRows = 32 * kX9Blocks;
 constexpr int kX9IterCols = 64;
 constexpr int kX9Xcds = 8;
 
-template <int TERMS>
+// DP16 / X16: that operand is stored as bf16 (bf16-input mode only, TERMS = 1).  A dword
+// then holds two adjacent rows (units) of one column, so a lane that loads dword n of a
+// 64-row span gets rows 2n and 2n+1: the even rows form one 32-row MFMA block and the
+// odd rows the next -- a permutation of rows (units), undone where the result is stored.
+//   dpre: wave w loads K step w/2 of the row-block pair w%2 (one load set instead of two)
+//   x   : waves 2m and 2m+1 both load the 64 units 64m .. 64m+63 and keep the even /
+//         the odd ones
+template <int TERMS, bool DP16 = false, bool X16 = false>
 __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
     const float* __restrict__ dpre, int ldp, int rows, const float* __restrict__ x,
     float* __restrict__ part, int cols, int iters_per_split, int n_wg, int groups) {
+    static_assert(TERMS == 1 || (!DP16 && !X16), "bf16 storage goes with bf16 inputs");
     // [buffer][K step][3 * row block + part][lane]: 96 KiB
     __shared__ u4 stage[2][4][3 * kX9Blocks][64];
     const int xcd = (int)(blockIdx.x % kX9Xcds), q = (int)(blockIdx.x / kX9Xcds);
@@ -74,8 +82,9 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
     const int total_iters = (cols + kX9IterCols - 1) / kX9IterCols;
     const int it0 = split * iters_per_split;
     const int it1 = min(total_iters, it0 + iters_per_split);
-    // this wave stages row block pb of K steps pk and pk + 2
-    const int pk = w >> 2, pb = w & 3;
+    // this wave stages row block pb of K steps pk and pk + 2 (DP16: K step w / 2 of the
+    // row-block pair w % 2)
+    const int pk = DP16 ? w >> 1 : w >> 2, pb = DP16 ? 2 * (w & 1) : w & 3;
 
     // Branch-free body: loads past the last column go to the last 8 columns and the
     // dpre side of such columns is zeroed (cols % 8 == 0, so 8-column groups are all
@@ -101,12 +110,47 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
             stage[buf][ks][3 * pb + 2][lane] = p[2];
         }
     };
-    const float* x_lane = x + 32 * w + n;
+    // bf16 dpre: dword n of the pair's 64 rows, eight columns
+    const uint32_t* dp16_lane = reinterpret_cast<const uint32_t*>(dpre) +
+                                (gi * kX9GroupRows + 32 * pb) / 2 + n;
+    auto dp_load16 = [&](int it, float (&v)[8]) {
+        const int cc = min(it * kX9IterCols + pk * 16 + 8 * g, cols - 8);
+        const uint32_t* p = dp16_lane + (size_t)cc * (ldp / 2);
+#pragma unroll
+        for (int j = 0; j < 8; j++) v[j] = __uint_as_float(p[(size_t)j * (ldp / 2)]);
+    };
+    // eight dwords of bf16 pairs -> the fragment of the even (odd) halves
+    auto pack16 = [&](const float (&v)[8], bool odd, bool in) {
+        uint32_t d[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+            d[p] = __builtin_amdgcn_perm(__float_as_uint(v[2 * p + 1]), __float_as_uint(v[2 * p]),
+                                         odd ? 0x07060302u : 0x05040100u);
+        return in ? u4{d[0], d[1], d[2], d[3]} : u4{0u, 0u, 0u, 0u};
+    };
+    auto dp_store16 = [&](int it, int buf, const float (&v)[8]) {
+        const bool in = it * kX9IterCols + pk * 16 + 8 * g < cols;
+        stage[buf][pk][3 * pb][lane] = pack16(v, false, in);
+        stage[buf][pk][3 * (pb + 1)][lane] = pack16(v, true, in);
+    };
+    const float* x_lane = X16 ? reinterpret_cast<const float*>(
+                                    reinterpret_cast<const uint32_t*>(x) + 32 * (w >> 1) + n)
+                              : x + 32 * w + n;
+    constexpr int kXRow = X16 ? CFP_HIDDEN / 2 : CFP_HIDDEN;   // dwords per column of x
     auto x_load = [&](int it, int ks, float (&v)[8]) {
         const int cc = min(it * kX9IterCols + ks * 16 + 8 * g, cols - 8);
-        const float* p = x_lane + (size_t)cc * CFP_HIDDEN;
+        const float* p = x_lane + (size_t)cc * kXRow;
 #pragma unroll
-        for (int j = 0; j < 8; j++) v[j] = p[j * CFP_HIDDEN];
+        for (int j = 0; j < 8; j++) v[j] = p[j * kXRow];
+    };
+    auto x_parts = [&](const float (&v)[8], u4 (&p)[3]) {
+        if (X16) {
+            p[0] = pack16(v, (w & 1) != 0, true);
+            p[1] = p[0];
+            p[2] = p[0];
+        } else {
+            parts_of<TERMS>(v, p);
+        }
     };
     auto frag_load = [&](int buf, int ks, int pair, u4 (&a)[6]) {
 #pragma unroll
@@ -122,29 +166,41 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
     if (it0 < it1) {
         float d0[8], d1[8];
         float raw[4][8];
-        dp_load(it0, pk, d0);
-        dp_load(it0, pk + 2, d1);
+        if (DP16) {
+            dp_load16(it0, d0);
+        } else {
+            dp_load(it0, pk, d0);
+            dp_load(it0, pk + 2, d1);
+        }
         x_load(it0, 0, raw[0]);
         x_load(it0, 1, raw[1]);
         x_load(it0, 2, raw[2]);
-        dp_store(it0, pk, 0, d0);
-        dp_store(it0, pk + 2, 0, d1);
+        if (DP16) {
+            dp_store16(it0, 0, d0);
+        } else {
+            dp_store(it0, pk, 0, d0);
+            dp_store(it0, pk + 2, 0, d1);
+        }
         __syncthreads();
         u4 a[2][6];
         frag_load(0, 0, 0, a[0]);
         u4 bs[3];
-        parts_of<TERMS>(raw[0], bs);
+        x_parts(raw[0], bs);
         for (int it = it0; it < it1; it++) {
             const int buf = (it - it0) & 1;
             const int itn = min(it + 1, it1 - 1);
-            dp_load(itn, pk, d0);
-            dp_load(itn, pk + 2, d1);
+            if (DP16) {
+                dp_load16(itn, d0);
+            } else {
+                dp_load(itn, pk, d0);
+                dp_load(itn, pk + 2, d1);
+            }
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
                 if (ks < 1) x_load(it, ks + 3, raw[ks + 3]);
                 else x_load(itn, ks - 1, raw[ks - 1]);
                 u4 ns[3];
-                parts_of<TERMS>(raw[(ks + 1) & 3], ns);
+                x_parts(raw[(ks + 1) & 3], ns);
 #pragma unroll
                 for (int pr = 0; pr < 2; pr++) {
                     const int cur = pr, nxt = pr ^ 1;
@@ -155,8 +211,12 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
                     } else {
                         // this wave's last read of the current buffer is in flight or
                         // done; the barrier's wait covers it
-                        dp_store(itn, pk, buf ^ 1, d0);
-                        dp_store(itn, pk + 2, buf ^ 1, d1);
+                        if (DP16) {
+                            dp_store16(itn, buf ^ 1, d0);
+                        } else {
+                            dp_store(itn, pk, buf ^ 1, d0);
+                            dp_store(itn, pk + 2, buf ^ 1, d1);
+                        }
                         __syncthreads();
                         frag_load(buf ^ 1, 0, 0, a[nxt]);
                     }
@@ -174,12 +234,15 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
             }
         }
     }
-    float* o = part + ((size_t)split * rows + gi * kX9GroupRows) * CFP_HIDDEN + 32 * w + n;
+    // undo the even / odd permutations of bf16-stored operands
+    const int unit = X16 ? 64 * (w >> 1) + 2 * n + (w & 1) : 32 * w + n;
+    float* o = part + ((size_t)split * rows + gi * kX9GroupRows) * CFP_HIDDEN + unit;
 #pragma unroll
     for (int b = 0; b < kX9Blocks; b++)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const int row = 32 * b + acc_row(r) + 4 * g;
+            const int i = acc_row(r) + 4 * g;
+            const int row = DP16 ? 64 * (b >> 1) + 2 * i + (b & 1) : 32 * b + i;
             if (gi * kX9GroupRows + row < rows) o[(size_t)row * CFP_HIDDEN] = acc[b][r];
         }
 }
@@ -214,7 +277,9 @@ __global__ void k_pack_w_x9(const float* __restrict__ W, long sk, long su,
     out[idx] = part == 0 ? h : (part == 1 ? m : l);
 }
 
-template <int TERMS>
+// A16: dpre is stored as bf16 (bf16-input mode): a lane's eight values of a K step are
+// the MFMA operand as they lie in memory.
+template <int TERMS, bool A16 = false>
 __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ dpre, int m3,
                                                       const u4* __restrict__ wm,
                                                       float* __restrict__ dh, int ldc, int cols,
@@ -225,12 +290,31 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     const int cb = (int)blockIdx.x * kDhTileCols + 32 * w;
     const bool live = cb < cols;               // cols % 32 == 0: blocks are whole
     const int cbc = live ? cb : cols - 32;     // idle waves still stage W and meet the barriers
+    static_assert(TERMS == 1 || !A16, "bf16 storage goes with bf16 inputs");
     const float* a_lane = dpre + (size_t)(cbc + n) * m3 + 8 * g;
+    const u4* a16_lane = reinterpret_cast<const u4*>(
+        reinterpret_cast<const uint16_t*>(dpre) + (size_t)(cbc + n) * m3 + 8 * g);
     auto a_load = [&](int s, float (&v)[8]) {
+        if (A16) {   // eight bf16 = 16 bytes, kept as raw bits in the first four slots
+            const u4 q = a16_lane[2 * s];
+            v[0] = __uint_as_float(q.x); v[1] = __uint_as_float(q.y);
+            v[2] = __uint_as_float(q.z); v[3] = __uint_as_float(q.w);
+            return;
+        }
         const f4* p = reinterpret_cast<const f4*>(a_lane + 16 * s);
         const f4 x0 = p[0], x1 = p[1];
 #pragma unroll
         for (int j = 0; j < 4; j++) { v[j] = x0[j]; v[4 + j] = x1[j]; }
+    };
+    auto a_parts = [&](const float (&v)[8], u4 (&p)[3]) {
+        if (A16) {
+            p[0] = u4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]),
+                      __float_as_uint(v[3])};
+            p[1] = p[0];
+            p[2] = p[0];
+        } else {
+            parts_of<TERMS>(v, p);
+        }
     };
     const u4* w_lane = wm + (size_t)3 * w * 64 + lane;
     auto w_load = [&](int s, u4 (&b)[3]) {
@@ -267,7 +351,7 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     w_store(0, wb);
     w_load(min(1, last), wb);
     u4 as[3];
-    parts_of<TERMS>(raw[0], as);
+    a_parts(raw[0], as);
     __syncthreads();
     u4 b[2][2];
     frag_load(0, 0, b[0]);
@@ -277,8 +361,8 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
         if (s & 1) a_load(min(s + 2, last), raw[1]);
         else a_load(min(s + 2, last), raw[0]);
         u4 ns[3];
-        if (s & 1) parts_of<TERMS>(raw[0], ns);
-        else parts_of<TERMS>(raw[1], ns);
+        if (s & 1) a_parts(raw[0], ns);
+        else a_parts(raw[1], ns);
 #pragma unroll
         for (int q = 0; q < 12; q++) {
             const int cur = q & 1, nxt = cur ^ 1;
@@ -323,14 +407,17 @@ bool gemm_dh_x9_ok(int m3, int cols, const float* dpre) {
 // out[cols][ldc] (+)= A[cols][K] . B, B(k, u) = B[k*sk + u*su] for 256 units
 static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const float* A,
                         float* out, int ldc, bool accumulate, int terms, u4* g_w_x9,
-                        hipStream_t st) {
+                        hipStream_t st, bool a16 = false) {
+    CFP_REQUIRE(!a16 || terms == 1, "k_dh_x9: bf16-stored operands need the bf16-input mode");
     CFP_REQUIRE(g_w_x9, "k_dh_x9: no mirror buffer for W");
     const int total = (K / 16) * kDhFrags * 64;
     hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, B, sk, su, g_w_x9,
                        total, terms == 1 ? 1 : 0);
     const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
     const int acc = accumulate ? 1 : 0;
-    if (terms == 1)
+    if (a16)
+        hipLaunchKernelGGL((k_dh_x9<1, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+    else if (terms == 1)
         hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
     else if (terms == 6)
         hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
@@ -343,11 +430,11 @@ static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const
 size_t dh_mirror_bytes() { return kDhMirrorBytes; }
 
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               int terms, u4* w_mirror, hipStream_t st) {
+               int terms, u4* w_mirror, hipStream_t st, bool dpre_bf16) {
     CFP_REQUIRE(gemm_dh_x9_ok(m3, cols, dpre) && W && dh,
                 "gemm_dh_x9: K must be a multiple of 16 up to %d and columns of 32", kDhMaxK);
     return launch_dh_x9(m3, cols, W, CFP_HIDDEN, 1, dpre, dh, CFP_HIDDEN, accumulate, terms, w_mirror,
-                        st);
+                        st, dpre_bf16);
 }
 
 // y[cols][m] = x[cols][k] . W[m][k]^T in slices of 256 output rows of W
@@ -414,7 +501,12 @@ bool gemm_dw_x9_ok(int rows, int cols) {
 }
 
 int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpre, float* dW,
-               int terms, const SeamWork& sw, hipStream_t st, int rows_first, float* dW_rest) {
+               int terms, const SeamWork& sw, hipStream_t st, int rows_first, float* dW_rest,
+               bool dpre_bf16, bool x_bf16) {
+    CFP_REQUIRE((!dpre_bf16 && !x_bf16) || terms == 1,
+                "gemm_dw_x9: bf16-stored operands need the bf16-input mode");
+    CFP_REQUIRE(!dpre_bf16 || (rows % kX9GroupRows == 0 && ld_dpre % 2 == 0),
+                "gemm_dw_x9: bf16-stored dpre needs whole groups of %d rows", kX9GroupRows);
     CFP_REQUIRE(gemm_dw_x9_ok(rows, cols) && x && dpre && dW && ld_dpre >= rows &&
                     (!dW_rest || (rows_first > 0 && rows_first < rows)),
                 "gemm_dw_x9: columns must be a multiple of 8");
@@ -433,7 +525,16 @@ int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpr
     splits = (total_iters + ips - 1) / ips;
     const int n_wg = splits * groups;
     const int grid = (n_wg + kX9Xcds - 1) / kX9Xcds * kX9Xcds;
-    if (terms == 1)
+    if (dpre_bf16 && x_bf16)
+        hipLaunchKernelGGL((k_dw_x9<1, true, true>), dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre,
+                           rows, x, work, cols, ips, n_wg, groups);
+    else if (x_bf16)
+        hipLaunchKernelGGL((k_dw_x9<1, false, true>), dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre,
+                           rows, x, work, cols, ips, n_wg, groups);
+    else if (dpre_bf16)
+        hipLaunchKernelGGL((k_dw_x9<1, true, false>), dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre,
+                           rows, x, work, cols, ips, n_wg, groups);
+    else if (terms == 1)
         hipLaunchKernelGGL(k_dw_x9<1>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
                            work, cols, ips, n_wg, groups);
     else if (terms == 6)

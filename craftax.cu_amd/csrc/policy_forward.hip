@@ -741,6 +741,8 @@ int launch_forward(const FwdArgs& a, hipStream_t st) {
                 "MinGRU layers need a state buffer");
     CFP_REQUIRE(!a.do_head || a.av_out != nullptr,
                 "head requested without an output buffer");
+    CFP_REQUIRE(!a.tr_bf16 || (a.bf16 && a.train),
+                "bf16 storage of the window recompute needs the bf16-input kernel");
     if (a.bf16) return launch_forward_bf16(a, st);
     // persistent: one workgroup per CU, each walking tile pairs round-robin; a full-game
     // batch of at most one tile per CU runs one tile per workgroup instead

@@ -7,7 +7,9 @@
 // loaded into the A operand.  Everything else stays fp32: accumulators, biases,
 // the gate/blend epilogue, the recurrent state and every output.  This is the
 // counterpart of the reference's CF_GEMM_BF16 mode (craftax_full.cu:11306-11316,
-// bf16 GEMM wrappers :11688-11756), without its bf16 storage of activations.
+// bf16 GEMM wrappers :11688-11756).  Its bf16 storage of activations exists for the
+// window recompute of the update only (TR16: gate pre-activations and layer outputs
+// leave as bf16, half the bytes of a kernel that is bound by its HBM writes there).
 //
 // At bf16 MFMA rates the matrix pipe is no longer the bound (a layer's gate GEMM
 // is 96 MFMAs of 32 cycles per wave); the kernel is bound by the epilogue's
@@ -53,7 +55,17 @@ __device__ __forceinline__ u4 a_frag(const f4* xs4, int l32, int g, int kb) {
 // one step of the slabs (records in r_obs, the stored post-zero state of every layer
 // as the state input), every layer's gate pre-activations and output written out,
 // nothing written back to the state.
-template <int VARIANT, bool HAS_RS, bool TRAIN>
+// LDS x tile [32][XS] -> dense bf16 [32][256] in HBM, 8 bytes per thread per step.
+__device__ __forceinline__ void copy_tile_out_bf16(const float* lds, uint16_t* dst, int tid) {
+    typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+    typedef unsigned int u2_t __attribute__((ext_vector_type(2)));
+    const f4* xs4 = reinterpret_cast<const f4*>(lds);
+    u2_t* d2 = reinterpret_cast<u2_t*>(dst);
+    for (int i = tid; i < kTileEnvs * CFP_HIDDEN / 4; i += kFwdThreads)
+        d2[i] = __builtin_bit_cast(u2_t, __builtin_convertvector(xs4[(i >> 6) * XS4 + (i & 63)], bf16x4_t));
+}
+
+template <int VARIANT, bool HAS_RS, bool TRAIN, bool TR16 = false>
 __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     __shared__ float term_s[kTileEnvs];
@@ -229,7 +241,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
         }
     }
     __syncthreads();
-    if (a.rec && a.h_enc_out) copy_tile_out(lds, a.h_enc_out + e0 * CFP_HIDDEN, tid);
+    if (a.rec && a.h_enc_out) {
+        if (TR16)
+            copy_tile_out_bf16(lds, reinterpret_cast<uint16_t*>(a.h_enc_out) + e0 * CFP_HIDDEN, tid);
+        else
+            copy_tile_out(lds, a.h_enc_out + e0 * CFP_HIDDEN, tid);
+    }
 
     // ---- MinGRU layers ------------------------------------------------------------
     constexpr int KB_STRIDE = 4 * 6 * 64;   // u4 per K block of the gate mirror
@@ -287,6 +304,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
                                 : nullptr;
         float* out_base = TRAIN ? a.tr_x[l + 1] + e0 * CFP_HIDDEN + wave * 64 : nullptr;
         float* pre_base = TRAIN ? a.tr_pre[l] + e0 * CFP_GRU + wave * 64 : nullptr;
+        __bf16* out16 = TR16 ? reinterpret_cast<__bf16*>(a.tr_x[l + 1]) + e0 * CFP_HIDDEN + wave * 64 : nullptr;
+        __bf16* pre16 = TR16 ? reinterpret_cast<__bf16*>(a.tr_pre[l]) + e0 * CFP_GRU + wave * 64 : nullptr;
 #pragma unroll
         for (int e = 0; e < 32; e++) {
             const int ut = e / 16, r = e % 16;
@@ -297,7 +316,12 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
             const float zh = acc[0 + ut][r];
             const float zg = acc[2 + ut][r];
             const float zp = acc[4 + ut][r];
-            if (TRAIN) {
+            if (TR16) {
+                __bf16* pp = pre16 + (acc_row(r) * CFP_GRU + ut * 32);
+                __builtin_nontemporal_store((__bf16)zh, pp + loff3);
+                __builtin_nontemporal_store((__bf16)zg, (pp + CFP_HIDDEN) + loff3);
+                __builtin_nontemporal_store((__bf16)zp, (pp + 2 * CFP_HIDDEN) + loff3);
+            } else if (TRAIN) {
                 float* pp = pre_base + (acc_row(r) * CFP_GRU + ut * 32);
                 __builtin_nontemporal_store(zh, pp + loff3);
                 __builtin_nontemporal_store(zg, (pp + CFP_HIDDEN) + loff3);
@@ -314,7 +338,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
             const float xv = *xp;
             const float hn = __builtin_fmaf(p, out - xv, xv);
             *xp = hn;
-            if (TRAIN) __builtin_nontemporal_store(hn, (out_base + soff) + loff);
+            if (TR16) __builtin_nontemporal_store((__bf16)hn, (out16 + soff) + loff);
+            else if (TRAIN) __builtin_nontemporal_store(hn, (out_base + soff) + loff);
             else __builtin_nontemporal_store(out, (st_base + soff) + loff);
         }
 #pragma unroll
@@ -356,7 +381,8 @@ int launch_forward_bf16(const FwdArgs& a, hipStream_t st) {
                         !a.terminals && a.tr_mb > 0 && a.tr_mb % kTileEnvs == 0 &&
                         a.h_enc_out == a.tr_x[0],
                     "window recompute: bad arguments");
-        hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true>), g, b, 0, st, a);
+        if (a.tr_bf16) hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true, true>), g, b, 0, st, a);
+        else hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true>), g, b, 0, st, a);
     } else if (a.variant == 1) {
         if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<1, true, false>), g, b, 0, st, a);
         else hipLaunchKernelGGL((k_policy_forward_bf16<1, false, false>), g, b, 0, st, a);

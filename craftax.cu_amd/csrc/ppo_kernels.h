@@ -29,6 +29,7 @@ struct ReverseArgs {
     int steps;                 // steps in this window
     int layer, layers;
     int horizon, seg;          // rollout length, BPTT segment length
+    int gates_bf16;            // gates and layer_in are bf16 arrays (the update's bf16 storage)
 };
 int launch_gru_reverse(const ReverseArgs& a, hipStream_t st);
 

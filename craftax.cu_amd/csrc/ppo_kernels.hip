@@ -49,17 +49,68 @@ __device__ __forceinline__ double wave_sum(double v) {
 // issue order, so "the set fetched three stages ago has landed" is "at most N younger
 // operations are outstanding".  Three register sets rotate through a loop unrolled by
 // three (a set is never copied: a copy would read registers whose loads are in flight).
-struct StepIn {
-    f4 zh, zg, zp, ga, gb, s, x;
+// G16: the gate rows and the layer input are stored as bf16 (8 bytes per lane and row).
+typedef unsigned int u2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+template <bool G16>
+struct StepIn;
+template <>
+struct StepIn<false> {
+    f4 zh, zg, zp, x, ga, gb, s;
+    unsigned done;
+};
+template <>
+struct StepIn<true> {
+    u2 zh, zg, zp, x;
+    f4 ga, gb, s;
     unsigned done;
 };
 
-template <bool TWO_GRADS>
-__device__ __forceinline__ void sweep_fetch(StepIn& r, unsigned lane_off, const f4* gates,
-                                            const f4* ga, const f4* gb, const f4* state,
-                                            const f4* xin, const uint8_t* done) {
+__device__ __forceinline__ f4 widen(const f4& v) { return v; }
+__device__ __forceinline__ f4 widen(const u2& v) {   // four bf16 -> four fp32
+    return f4{__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u),
+              __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u)};
+}
+__device__ __forceinline__ u2 narrow(const f4& v) {   // round to nearest even
+    return __builtin_bit_cast(u2, __builtin_convertvector(v, bf16x4));
+}
+
+// lo: byte offset of the lane inside an fp32 row (16 q), lo8: inside a bf16 row (8 q)
+template <bool TWO_GRADS, bool G16>
+__device__ __forceinline__ void sweep_fetch(StepIn<G16>& r, unsigned lo, unsigned lo8,
+                                            const void* gates, const f4* ga, const f4* gb,
+                                            const f4* state, const void* xin, const uint8_t* done) {
     const unsigned zero = 0u;
-    if (TWO_GRADS)
+    if (G16 && TWO_GRADS)
+        asm volatile(
+            "global_load_dwordx2 %0, %9, %11 nt\n\t"
+            "global_load_dwordx2 %1, %9, %11 offset:512 nt\n\t"
+            "global_load_dwordx2 %2, %9, %11 offset:1024 nt\n\t"
+            "global_load_dwordx4 %3, %8, %12 nt\n\t"
+            "global_load_dwordx4 %4, %8, %13 nt\n\t"
+            "global_load_dwordx4 %5, %8, %14 nt\n\t"
+            "global_load_dwordx2 %6, %9, %15 nt\n\t"
+            "global_load_ubyte %7, %10, %16"
+            : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.gb), "=&v"(r.s),
+              "=&v"(r.x), "=&v"(r.done)
+            : "v"(lo), "v"(lo8), "v"(zero), "s"(gates), "s"(ga), "s"(gb), "s"(state), "s"(xin),
+              "s"(done)
+            : "memory");
+    else if (G16)
+        asm volatile(
+            "global_load_dwordx2 %0, %8, %10 nt\n\t"
+            "global_load_dwordx2 %1, %8, %10 offset:512 nt\n\t"
+            "global_load_dwordx2 %2, %8, %10 offset:1024 nt\n\t"
+            "global_load_dwordx4 %3, %7, %11 nt\n\t"
+            "global_load_dwordx4 %4, %7, %12 nt\n\t"
+            "global_load_dwordx2 %5, %8, %13 nt\n\t"
+            "global_load_ubyte %6, %9, %14"
+            : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.s), "=&v"(r.x),
+              "=&v"(r.done)
+            : "v"(lo), "v"(lo8), "v"(zero), "s"(gates), "s"(ga), "s"(state), "s"(xin), "s"(done)
+            : "memory");
+    else if (TWO_GRADS)
         asm volatile(
             "global_load_dwordx4 %0, %8, %10 nt\n\t"
             "global_load_dwordx4 %1, %8, %10 offset:1024 nt\n\t"
@@ -71,7 +122,7 @@ __device__ __forceinline__ void sweep_fetch(StepIn& r, unsigned lane_off, const 
             "global_load_ubyte %7, %9, %15"
             : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.gb), "=&v"(r.s),
               "=&v"(r.x), "=&v"(r.done)
-            : "v"(lane_off), "v"(zero), "s"(gates), "s"(ga), "s"(gb), "s"(state), "s"(xin), "s"(done)
+            : "v"(lo), "v"(zero), "s"(gates), "s"(ga), "s"(gb), "s"(state), "s"(xin), "s"(done)
             : "memory");
     else
         asm volatile(
@@ -84,14 +135,14 @@ __device__ __forceinline__ void sweep_fetch(StepIn& r, unsigned lane_off, const 
             "global_load_ubyte %6, %8, %13"
             : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.s), "=&v"(r.x),
               "=&v"(r.done)
-            : "v"(lane_off), "v"(zero), "s"(gates), "s"(ga), "s"(state), "s"(xin), "s"(done)
+            : "v"(lo), "v"(zero), "s"(gates), "s"(ga), "s"(state), "s"(xin), "s"(done)
             : "memory");
 }
 
 // Every later use of the set depends on this statement's outputs, so none can be moved
 // in front of the wait.
-template <int N, bool TWO_GRADS>
-__device__ __forceinline__ void sweep_wait(StepIn& r) {
+template <int N, bool TWO_GRADS, bool G16>
+__device__ __forceinline__ void sweep_wait(StepIn<G16>& r) {
     if (TWO_GRADS)
         asm volatile("s_waitcnt vmcnt(%8)"
                      : "+v"(r.zh), "+v"(r.zg), "+v"(r.zp), "+v"(r.ga), "+v"(r.gb), "+v"(r.s),
@@ -104,34 +155,9 @@ __device__ __forceinline__ void sweep_wait(StepIn& r) {
                      : "n"(N));
 }
 
-template <bool HIGHWAY>
-__device__ __forceinline__ void sweep_store(unsigned lane_off, f4* gates, f4* hw, const f4& dzh,
-                                            const f4& dzg, const f4& dzp, const f4& hwv) {
-    // the trailing s_nop keeps the next instruction clear of the store data registers
-    if (HIGHWAY)
-        asm volatile(
-            "global_store_dwordx4 %0, %1, %5 nt\n\t"
-            "global_store_dwordx4 %0, %2, %5 offset:1024 nt\n\t"
-            "global_store_dwordx4 %0, %3, %5 offset:2048 nt\n\t"
-            "global_store_dwordx4 %0, %4, %6 nt\n\t"
-            "s_nop 0"
-            :
-            : "v"(lane_off), "v"(dzh), "v"(dzg), "v"(dzp), "v"(hwv), "s"(gates), "s"(hw)
-            : "memory");
-    else
-        asm volatile(
-            "global_store_dwordx4 %0, %1, %4 nt\n\t"
-            "global_store_dwordx4 %0, %2, %4 offset:1024 nt\n\t"
-            "global_store_dwordx4 %0, %3, %4 offset:2048 nt\n\t"
-            "s_nop 0"
-            :
-            : "v"(lane_off), "v"(dzh), "v"(dzg), "v"(dzp), "s"(gates)
-            : "memory");
-}
-
 // Drain the queue; every set is an output, so nothing of any set is read before it.
-template <bool TWO_GRADS>
-__device__ __forceinline__ void sweep_drain(StepIn& p, StepIn& q, StepIn& r) {
+template <bool TWO_GRADS, bool G16>
+__device__ __forceinline__ void sweep_drain(StepIn<G16>& p, StepIn<G16>& q, StepIn<G16>& r) {
     if (TWO_GRADS)
         asm volatile("s_waitcnt vmcnt(0)"
                      : "+v"(p.zh), "+v"(p.zg), "+v"(p.zp), "+v"(p.ga), "+v"(p.gb), "+v"(p.s),
@@ -146,19 +172,70 @@ __device__ __forceinline__ void sweep_drain(StepIn& p, StepIn& q, StepIn& r) {
                        "+v"(r.s), "+v"(r.x), "+v"(r.done));
 }
 
+// the trailing s_nop keeps the next instruction clear of the store data registers
+template <bool HIGHWAY>
+__device__ __forceinline__ void sweep_store(unsigned lo, unsigned, void* gates, f4* hw, const f4& dzh,
+                                            const f4& dzg, const f4& dzp, const f4& hwv) {
+    if (HIGHWAY)
+        asm volatile(
+            "global_store_dwordx4 %0, %1, %5 nt\n\t"
+            "global_store_dwordx4 %0, %2, %5 offset:1024 nt\n\t"
+            "global_store_dwordx4 %0, %3, %5 offset:2048 nt\n\t"
+            "global_store_dwordx4 %0, %4, %6 nt\n\t"
+            "s_nop 0"
+            :
+            : "v"(lo), "v"(dzh), "v"(dzg), "v"(dzp), "v"(hwv), "s"(gates), "s"(hw)
+            : "memory");
+    else
+        asm volatile(
+            "global_store_dwordx4 %0, %1, %4 nt\n\t"
+            "global_store_dwordx4 %0, %2, %4 offset:1024 nt\n\t"
+            "global_store_dwordx4 %0, %3, %4 offset:2048 nt\n\t"
+            "s_nop 0"
+            :
+            : "v"(lo), "v"(dzh), "v"(dzg), "v"(dzp), "s"(gates)
+            : "memory");
+}
+template <bool HIGHWAY>
+__device__ __forceinline__ void sweep_store(unsigned lo, unsigned lo8, void* gates, f4* hw,
+                                            const u2& dzh, const u2& dzg, const u2& dzp,
+                                            const f4& hwv) {
+    if (HIGHWAY)
+        asm volatile(
+            "global_store_dwordx2 %1, %2, %6 nt\n\t"
+            "global_store_dwordx2 %1, %3, %6 offset:512 nt\n\t"
+            "global_store_dwordx2 %1, %4, %6 offset:1024 nt\n\t"
+            "global_store_dwordx4 %0, %5, %7 nt\n\t"
+            "s_nop 0"
+            :
+            : "v"(lo), "v"(lo8), "v"(dzh), "v"(dzg), "v"(dzp), "v"(hwv), "s"(gates), "s"(hw)
+            : "memory");
+    else
+        asm volatile(
+            "global_store_dwordx2 %0, %1, %4 nt\n\t"
+            "global_store_dwordx2 %0, %2, %4 offset:512 nt\n\t"
+            "global_store_dwordx2 %0, %3, %4 offset:1024 nt\n\t"
+            "s_nop 0"
+            :
+            : "v"(lo8), "v"(dzh), "v"(dzg), "v"(dzp), "s"(gates)
+            : "memory");
+}
+
 #ifndef CFP_SWEEP_EPB
 #define CFP_SWEEP_EPB 1
 #endif
 constexpr int kSweepEnvs = CFP_SWEEP_EPB;   // envs (wavefronts) per workgroup
-template <bool TWO_GRADS, bool HIGHWAY>
+template <bool TWO_GRADS, bool HIGHWAY, bool G16>
 __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int env = (int)blockIdx.x * kSweepEnvs + wave;   // mb % 32 == 0: whole wavefronts only
-    const unsigned lane_off = (threadIdx.x & 63u) * 16u;   // units 4q .. 4q+3 of a 1 KiB row
+    const unsigned lane_off = (threadIdx.x & 63u) * 16u;   // units 4q .. 4q+3 of a 1 KiB fp32 row
+    const unsigned lane_off8 = (threadIdx.x & 63u) * 8u;   // ... of a 512-byte bf16 row
     // wavefront-uniform row pointers of this env; a step back in time is one stride
     const size_t mbz = (size_t)a.w.mb;
-    f4* const gates = reinterpret_cast<f4*>(a.gates) + (size_t)env * G4;
-    const f4* const xin = reinterpret_cast<const f4*>(a.layer_in) + (size_t)env * H4;
+    constexpr size_t kGateRow = G16 ? G * 2 : G * 4, kInRow = G16 ? H * 2 : H * 4;   // bytes
+    char* const gates = reinterpret_cast<char*>(a.gates) + (size_t)env * kGateRow;
+    const char* const xin = reinterpret_cast<const char*>(a.layer_in) + (size_t)env * kInRow;
     const f4* const ga = reinterpret_cast<const f4*>(a.grad_a) + (size_t)env * H4;
     const f4* const gb = TWO_GRADS ? reinterpret_cast<const f4*>(a.grad_b) + (size_t)env * H4 : nullptr;
     f4* const hw = HIGHWAY ? reinterpret_cast<f4*>(a.highway_out) + (size_t)env * H4 : nullptr;
@@ -173,13 +250,15 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
     const f4* const idle = reinterpret_cast<const f4*>(a.carry) +
                            (size_t)(env < a.w.mb - 2 ? env : a.w.mb - 3) * H4;
 
-    auto fetch = [&](int s, StepIn& r) {   // s < 0: nothing left, an idle fetch
+    auto fetch = [&](int s, StepIn<G16>& r) {   // s < 0: nothing left, an idle fetch
         const bool real = s >= 0;
         const size_t c = (size_t)(real ? s : 0) * mbz;
-        sweep_fetch<TWO_GRADS>(r, lane_off, real ? gates + c * G4 : idle, real ? ga + c * H4 : idle,
-                               TWO_GRADS ? (real ? gb + c * H4 : idle) : nullptr,
-                               real ? state + (size_t)s * state_step : idle,
-                               real ? xin + c * H4 : idle, done + (size_t)(real ? s : 0) * a.w.n_all);
+        sweep_fetch<TWO_GRADS, G16>(
+            r, lane_off, lane_off8, real ? (const void*)(gates + c * kGateRow) : (const void*)idle,
+            real ? ga + c * H4 : idle, TWO_GRADS ? (real ? gb + c * H4 : idle) : nullptr,
+            real ? state + (size_t)s * state_step : idle,
+            real ? (const void*)(xin + c * kInRow) : (const void*)idle,
+            done + (size_t)(real ? s : 0) * a.w.n_all);
     };
 
     f4* const carry_p = reinterpret_cast<f4*>(a.carry) + (size_t)env * H4 + (threadIdx.x & 63u);
@@ -189,31 +268,37 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
     const int last = a.steps - 1;
     int phase = (a.w.t0 + last + 1) % a.seg;
 
-    auto consume = [&](int s, const StepIn& in) {
+    auto consume = [&](int s, const StepIn<G16>& in) {
         if (a.w.t0 + s == a.horizon - 1 || phase == 0) carry = f4{0.0f, 0.0f, 0.0f, 0.0f};
         phase = (phase == 0 ? a.seg : phase) - 1;
         const float pass = (in.done & 0xffu) ? 0.0f : 1.0f;   // a terminal step hands nothing back
+        const f4 zh = widen(in.zh), zg = widen(in.zg), zp = widen(in.zp), x = widen(in.x);
         f4 dzh, dzg, dzp, hwv;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const float sg = sigmoid_fast(in.zg[j]);
-            const float mix = sigmoid_fast(in.zp[j]);
-            const float sh = sigmoid_fast(in.zh[j]);
-            const bool lin = in.zh[j] >= 0.0f;
-            const float cand = lin ? in.zh[j] + 0.5f : sh;           // g(zh)
+            const float sg = sigmoid_fast(zg[j]);
+            const float mix = sigmoid_fast(zp[j]);
+            const float sh = sigmoid_fast(zh[j]);
+            const bool lin = zh[j] >= 0.0f;
+            const float cand = lin ? zh[j] + 0.5f : sh;              // g(zh)
             const float dcand = lin ? 1.0f : sh * (1.0f - sh);       // g'(zh)
             const float gap = cand - in.s[j];
             const float h_new = in.s[j] + sg * gap;
             const float g_top = TWO_GRADS ? in.ga[j] + in.gb[j] : in.ga[j];
             const float g_h = g_top * mix + pass * carry[j];
-            dzp[j] = g_top * (h_new - in.x[j]) * mix * (1.0f - mix);
+            dzp[j] = g_top * (h_new - x[j]) * mix * (1.0f - mix);
             hwv[j] = g_top * (1.0f - mix);
             carry[j] = g_h * (1.0f - sg);
             dzg[j] = g_h * gap * sg * (1.0f - sg);
             dzh[j] = g_h * sg * dcand;
         }
         const size_t c = (size_t)s * mbz;
-        sweep_store<HIGHWAY>(lane_off, gates + c * G4, HIGHWAY ? hw + c * H4 : nullptr, dzh, dzg, dzp, hwv);
+        if constexpr (G16)
+            sweep_store<HIGHWAY>(lane_off, lane_off8, gates + c * kGateRow, HIGHWAY ? hw + c * H4 : nullptr,
+                                 narrow(dzh), narrow(dzg), narrow(dzp), hwv);
+        else
+            sweep_store<HIGHWAY>(lane_off, lane_off8, gates + c * kGateRow, HIGHWAY ? hw + c * H4 : nullptr,
+                                 dzh, dzg, dzp, hwv);
     };
 
     // Operations per stage: NL loads then (after the step's arithmetic) NS stores.
@@ -222,21 +307,21 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
     // stores in the first round.  A round is straight-line code: no control flow ever
     // merges registers whose loads are in flight.
     constexpr int NL = TWO_GRADS ? 8 : 7, NS = HIGHWAY ? 4 : 3;
-    StepIn b0, b1, b2;
+    StepIn<G16> b0, b1, b2;
     fetch(last, b0);
     fetch(last - 1, b1);
     fetch(last - 2, b2);
-#define CFP_SWEEP_ROUND(s_, N0, N1, N2)                 \
-    do {                                                \
-        sweep_wait<(N0), TWO_GRADS>(b0);                \
-        consume((s_), b0);                              \
-        fetch((s_) - 3, b0);                            \
-        sweep_wait<(N1), TWO_GRADS>(b1);                \
-        consume((s_) - 1, b1);                          \
-        fetch((s_) - 4, b1);                            \
-        sweep_wait<(N2), TWO_GRADS>(b2);                \
-        consume((s_) - 2, b2);                          \
-        fetch((s_) - 5, b2);                            \
+#define CFP_SWEEP_ROUND(s_, N0, N1, N2)                      \
+    do {                                                     \
+        sweep_wait<(N0), TWO_GRADS, G16>(b0);                \
+        consume((s_), b0);                                   \
+        fetch((s_) - 3, b0);                                 \
+        sweep_wait<(N1), TWO_GRADS, G16>(b1);                \
+        consume((s_) - 1, b1);                               \
+        fetch((s_) - 4, b1);                                 \
+        sweep_wait<(N2), TWO_GRADS, G16>(b2);                \
+        consume((s_) - 2, b2);                               \
+        fetch((s_) - 5, b2);                                 \
     } while (0)
     int s = last;
     if (s >= 2) {
@@ -246,7 +331,7 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
     }
 #undef CFP_SWEEP_ROUND
     // at most two steps are left, in b0 then b1; everything in flight lands first
-    sweep_drain<TWO_GRADS>(b0, b1, b2);
+    sweep_drain<TWO_GRADS, G16>(b0, b1, b2);
     if (s >= 0) consume(s, b0);
     if (s >= 1) consume(s - 1, b1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -530,8 +615,6 @@ __device__ __forceinline__ f4 adam_four(const AdamArgs& a, const AdamCoef& k, si
     return w;
 }
 
-typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-
 __device__ __forceinline__ void put_bf16x4(__bf16* dst, const f4& w) {
     *reinterpret_cast<bf16x4*>(dst) = __builtin_convertvector(w, bf16x4);
 }
@@ -628,10 +711,19 @@ int launch_gru_reverse(const ReverseArgs& a, hipStream_t st) {
                     a.steps > 0 && a.w.mb > 0 && a.w.mb % kSweepEnvs == 0 && a.seg > 0,
                 "reverse MinGRU sweep: bad arguments");
     const dim3 grid(a.w.mb / kSweepEnvs), blk(64 * kSweepEnvs);
-    if (a.grad_b && a.highway_out) hipLaunchKernelGGL((k_gru_reverse<true, true>), grid, blk, 0, st, a);
-    else if (a.grad_b) hipLaunchKernelGGL((k_gru_reverse<true, false>), grid, blk, 0, st, a);
-    else if (a.highway_out) hipLaunchKernelGGL((k_gru_reverse<false, true>), grid, blk, 0, st, a);
-    else hipLaunchKernelGGL((k_gru_reverse<false, false>), grid, blk, 0, st, a);
+    CFP_REQUIRE(a.w.mb >= 3, "reverse MinGRU sweep: at least three envs");
+#define CFP_SWEEP_LAUNCH(G16)                                                                         \
+    do {                                                                                              \
+        if (a.grad_b && a.highway_out)                                                                \
+            hipLaunchKernelGGL((k_gru_reverse<true, true, G16>), grid, blk, 0, st, a);                \
+        else if (a.grad_b) hipLaunchKernelGGL((k_gru_reverse<true, false, G16>), grid, blk, 0, st, a); \
+        else if (a.highway_out)                                                                       \
+            hipLaunchKernelGGL((k_gru_reverse<false, true, G16>), grid, blk, 0, st, a);               \
+        else hipLaunchKernelGGL((k_gru_reverse<false, false, G16>), grid, blk, 0, st, a);             \
+    } while (0)
+    if (a.gates_bf16) CFP_SWEEP_LAUNCH(true);
+    else CFP_SWEEP_LAUNCH(false);
+#undef CFP_SWEEP_LAUNCH
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }

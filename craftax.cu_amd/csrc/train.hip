@@ -162,7 +162,10 @@ struct cfp_trainer {
     // the process-wide GEMM modes it was captured under
     hipGraph_t tgraph = nullptr;
     hipGraphExec_t texec = nullptr;
-    int graph_split = -1, graph_bf16 = -1, graph_pol_bf16 = -1;
+    int graph_split = -1, graph_bf16 = -1, graph_pol_bf16 = -1, graph_store16 = -1;
+    // bf16 storage of the window's gate pre-activations / their gradients and of the
+    // layer inputs (in effect with bf16 GEMM inputs on the split kernels only)
+    int bf16_store = 0;
     hipStream_t st_own = nullptr;   // capture stream when the caller passes the null stream
 };
 
@@ -313,6 +316,13 @@ void* cfp_train_buffer(cfp_trainer* tr, int which) {
     }
 }
 
+int cfp_train_set_bf16_storage(cfp_trainer* tr, int on) {
+    CFP_REQUIRE(tr, "cfp_train_set_bf16_storage: NULL trainer");
+    tr->bf16_store = on ? 1 : 0;
+    return 0;
+}
+int cfp_train_bf16_storage(const cfp_trainer* tr) { return tr ? tr->bf16_store : -1; }
+
 int cfp_train_window(const cfp_trainer* tr) { return tr ? tr->win : 0; }
 int cfp_train_minibatch(const cfp_trainer* tr) { return tr ? tr->mb : 0; }
 
@@ -445,6 +455,9 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         // state in, pre-activations and layer outputs out.  The unfused chain below is
         // what bf16 inputs run with the split kernels switched off.
         const bool fused = cfp_get_gemm_bf16() == 0 || cfp_get_gemm_split() != 0;
+        // bf16 storage: pre / dpre and the layer inputs x[0..L] are bf16 arrays inside
+        // the same buffers; needs mb % 32 (the record-fed dW_enc) and the split kernels
+        const bool st16 = tr->bf16_store && cfp_get_gemm_bf16() != 0 && cfp_get_gemm_split() != 0;
         if (fused) {
             FwdArgs fa{};
             fill_forward_weights(p, fa);
@@ -457,6 +470,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             fa.layers = L;
             fa.do_head = 1;
             fa.train = 1;
+            fa.tr_bf16 = st16 ? 1 : 0;
             fa.tr_t0 = t0; fa.tr_mb = mb; fa.tr_n_all = n; fa.tr_env_start = env_start;
             for (int l = 0; l < L; l++) fa.tr_pre[l] = tr->preb[l];
             for (int l = 0; l <= L; l++) fa.tr_x[l] = tr->x[l];
@@ -498,9 +512,14 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         if (launch_fold_f64(tr->block_loss, head_blocks(cols), 3, tr->loss_acc, true, st)) return 1;
         // dh3 = [dlogits | dvalue] . [W_a ; W_v]; dW_a and dW_v from one GEMM; bias sums
         if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, tr->sw, st)) return 1;
-        if (gemm_dw_two(A, 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L),
-                        g + CFP_OFF_W_V(L), tr->sw, st))
+        if (st16) {
+            if (gemm_dw_x9(A + 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L), 1, tr->sw,
+                           st, A, g + CFP_OFF_W_V(L), false, true))
+                return 1;
+        } else if (gemm_dw_two(A, 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L),
+                               g + CFP_OFF_W_V(L), tr->sw, st)) {
             return 1;
+        }
         if (colsum_into(tr, tr->dlogits, kHeadLd, g + CFP_OFF_B_A(L), A, cols, st)) return 1;
         if (colsum_into(tr, tr->dlogits + A, kHeadLd, g + CFP_OFF_B_V(L), 1, cols, st)) return 1;
         // ---- reverse MinGRU layers
@@ -511,7 +530,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         // reverse kernel of the next layer then fills the wave slots that are left and
         // runs under it.  Every dW has a split workspace of its own.
         const int terms = gemm_split_terms();
-        const bool overlap = terms > 1 && gemm_dw_x9_ok(G, cols);
+        const bool overlap = terms >= 1 && gemm_dw_x9_ok(G, cols);
         hipStream_t chain = st, other = tr->st2;
         const float* dh_gemm = tr->dh3b;
         const float* dh_extra = nullptr;
@@ -521,19 +540,26 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             ra.grad_a = dh_gemm; ra.grad_b = dh_extra; ra.highway_out = tr->dhX;
             ra.slab_state = tr->r_state; ra.slab_done = tr->r_done; ra.carry = tr->dcarry[l];
             ra.w = wm; ra.steps = Tw; ra.layer = l; ra.layers = L; ra.horizon = T; ra.seg = seg;
+            ra.gates_bf16 = st16 ? 1 : 0;
             if (launch_gru_reverse(ra, chain)) return 1;
             if (!overlap &&
                 gemm_dw_ld(G, cols, tr->x[l], tr->preb[l], G, g + CFP_OFF_W_GRU + (size_t)l * G * H,
                            tr->sw, chain))
                 return 1;
             // layer 0: dh_enc = W_0^T dpre + highway, accumulated onto the highway term
-            if (gemm_dh_acc(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
-                            l == 0 ? tr->dhX : tr->dhG, l == 0, tr->sw, chain))
+            if (st16) {
+                if (gemm_dh_x9(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
+                               l == 0 ? tr->dhX : tr->dhG, l == 0, 1, tr->sw.w_mirror, chain, true))
+                    return 1;
+            } else if (gemm_dh_acc(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
+                                   l == 0 ? tr->dhX : tr->dhG, l == 0, tr->sw, chain)) {
                 return 1;
+            }
             if (overlap) {
                 CFP_HIP_TRY(hipEventRecord(tr->ev_dh[l], chain));
                 if (gemm_dw_x9(G, cols, tr->x[l], tr->preb[l], G,
-                               g + CFP_OFF_W_GRU + (size_t)l * G * H, terms, tr->sw_layer[l], chain))
+                               g + CFP_OFF_W_GRU + (size_t)l * G * H, terms, tr->sw_layer[l], chain, 0,
+                               nullptr, st16, st16))
                     return 1;
                 CFP_HIP_TRY(hipStreamWaitEvent(other, tr->ev_dh[l], 0));
                 hipStream_t t = chain; chain = other; other = t;
@@ -613,7 +639,7 @@ int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
     const int split = cfp_get_gemm_split(), bf = cfp_get_gemm_bf16(),
               pbf = cfp_policy_gemm_bf16(tr->p);
     if (tr->texec && (split != tr->graph_split || bf != tr->graph_bf16 ||
-                      pbf != tr->graph_pol_bf16)) {
+                      pbf != tr->graph_pol_bf16 || tr->bf16_store != tr->graph_store16)) {
         (void)hipGraphExecDestroy(tr->texec);
         (void)hipGraphDestroy(tr->tgraph);
         tr->texec = nullptr;
@@ -644,6 +670,7 @@ int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
         tr->graph_split = split;
         tr->graph_bf16 = bf;
         tr->graph_pol_bf16 = pbf;
+        tr->graph_store16 = tr->bf16_store;
     }
     CFP_HIP_TRY(hipGraphLaunch(tr->texec, st));
     CFP_HIP_TRY(hipStreamSynchronize(st));

@@ -247,6 +247,10 @@ class Trainer:
         """V(s_T) on a copy of the live state -> v_boot."""
         _check(lib().cfp_train_bootstrap(self._h, _ptr(rec), _ptr(terminals), _stream()))
 
+    def set_bf16_storage(self, on=True):
+        """bf16 storage of the window workspace (in effect with bf16 GEMM inputs only)."""
+        _check(lib().cfp_train_set_bf16_storage(self._h, 1 if on else 0))
+
     def gae(self):
         _check(lib().cfp_train_gae(self._h, _stream()))
 

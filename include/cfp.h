@@ -331,6 +331,17 @@ enum cfp_train_buf {
 };
 /* Borrowed device pointer to one of the trainer's buffers (NULL if unknown). */
 void* cfp_train_buffer(cfp_trainer* tr, int which);
+/* bf16 storage of the update's window workspace, the reference's CF_GEMM_BF16 storage
+ * (craftax_full.cu:12694-12727: bf16 shadows of the gate pre-activations / their
+ * gradients and of the layer inputs feed its bf16 GEMMs, reverse kernel's bf16 paths
+ * :9538-9590).  In effect only while cfp_set_gemm_bf16(1) is on with the split kernels
+ * (cfp_set_gemm_split != 0): the window recompute then writes the gate pre-activations
+ * and layer inputs as bf16, the reverse sweep reads them and leaves the gate gradients
+ * as bf16, and the dW / dh GEMMs take those as their operands unconverted -- half the
+ * bytes of the kernels that bound the bf16 update.  r_state, the dh buffers, head rows
+ * and every gradient stay fp32.  Off by default. */
+int cfp_train_set_bf16_storage(cfp_trainer* tr, int on);
+int cfp_train_bf16_storage(const cfp_trainer* tr);
 int cfp_train_window(const cfp_trainer* tr);
 int cfp_train_minibatch(const cfp_trainer* tr);
 

@@ -433,3 +433,55 @@ def test_adam_writes_every_weight_mirror(pkg, cuda):
         assert torch.equal(av_a, av_b), f"bf16={bf16}: head rows differ"
         assert torch.equal(sa, sb), f"bf16={bf16}: states differ"
     tr.close(); pol.close(); twin.close()
+
+
+@pytest.mark.parametrize("n,T,minibatches,bwd_win,done_p", [(64, 8, 1, 0, 0.1), (128, 6, 2, 4, 0.15)])
+def test_backward_with_bf16_storage(pkg, cuda, n, T, minibatches, bwd_win, done_p):
+    """bf16 GEMM inputs with the window workspace stored as bf16 (cfp_train_set_bf16_storage:
+    gate pre-activations, their gradients and the layer inputs; the reference's
+    CF_GEMM_BF16 storage) against the fp64 oracle, every gradient segment within 2e-2 in
+    the relative Frobenius norm -- the tolerance of the bf16-input mode -- and close to
+    the same update with fp32 storage.  Behaviour log-probabilities are the current
+    policy's own plus noise, so no sample sits on the clip discontinuity (see
+    test_backward_with_bf16_gemms)."""
+    import torch
+    from parity_util import TOL_BF16, fro_err, expand_records
+    params, pol, tr, host = _collect(pkg, cuda, n, T, 170 + n, done_p, minibatches=minibatches,
+                                     bwd_win=bwd_win)
+    rng = np.random.default_rng(171)
+    for t in range(T):
+        ref = ob.forward_f64(params, L, expand_records(host["r_obs"][t]), host["r_state"][t], None)
+        z = ref["logits"] - ref["logits"].max(axis=1, keepdims=True)
+        logp = z - np.log(np.exp(z).sum(axis=1, keepdims=True))
+        host["r_logprob"][t] = (logp[np.arange(n), host["r_act"][t]]
+                                + 0.02 * rng.standard_normal(n)).astype(np.float32)
+    tr.buf("r_logprob").copy_(_t(host["r_logprob"], cuda))
+    mb = n // minibatches
+    pkg.policy.set_gemm_bf16(True)
+    try:
+        for m in range(minibatches):
+            batch, keep = ob.make_batch(T, n, m * mb, mb, L, T, **host)
+            g_ref, l3_ref = ob.ppo_backward_f64(params, batch)
+            got = {}
+            for store16 in (False, True):
+                tr.set_bf16_storage(store16)
+                outs = []
+                for _ in range(2):
+                    tr.buf("grads").zero_(); tr.zero_loss()
+                    tr.backward(m * mb, mb)
+                    torch.cuda.synchronize()
+                    outs.append(tr.buf("grads").cpu().numpy().copy())
+                assert np.array_equal(outs[0], outs[1]), "bitwise reproducible"
+                got[store16] = outs[0]
+                l3 = tr.buf("loss_acc").cpu().numpy()
+                assert np.allclose(l3, l3_ref, rtol=1e-2, atol=1e-2 * np.abs(l3_ref).max()), (store16, l3, l3_ref)
+            for name, sl in _segments(L):
+                e16 = fro_err(got[True][sl], g_ref[sl])
+                e32 = fro_err(got[False][sl], g_ref[sl])
+                assert e16 <= TOL_BF16, f"minibatch {m} d{name}: bf16 storage, relative Frobenius error {e16:.3e}"
+                assert e16 <= 3.0 * e32 + 2e-3, f"minibatch {m} d{name}: {e16:.3e} vs {e32:.3e} with fp32 storage"
+            assert not np.array_equal(got[True], got[False]), "the storage mode did not take effect"
+    finally:
+        pkg.policy.set_gemm_bf16(False)
+        tr.set_bf16_storage(False)
+    tr.close(); pol.close()
