@@ -45,6 +45,8 @@ PROTOTYPES = {
     "cfp_head": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "cfp_policy_forward": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int,
                                      C.c_int, vp]),
+    "cfp_policy_forward_features": (C.c_int, [vp, vp, vp, vp, vp, vp, vp, vp, C.c_int,
+                                              C.c_int, vp]),
     "cfp_set_gemm_bf16": (C.c_int, [C.c_int]),
     "cfp_get_gemm_bf16": (C.c_int, []),
     "cfp_set_gemm_split": (C.c_int, [C.c_int]),

@@ -43,18 +43,36 @@ def _time(torch, fn, reps, warm=2):
 
 
 def forward_65536(pkg, torch, reps):
+    """Second baseline configuration: 65 536 envs, one step, prior state N(0, 0.5); from
+    records (fused kernel, fp32 and bf16-input) and from the fp32 feature matrix as the
+    configuration states it (encoder GEMM of the seam + fused layers and heads)."""
     n = 65536
     pol = pkg.Policy(n, 3, seed=1)
     rec = pkg.policy.synth_records(n, 1234, 0)
     term = torch.zeros(n, device="cuda")
     av = torch.empty(n, 44, device="cuda")
+    st0 = torch.randn(3, n, 256, device="cuda") * 0.5
+    state = st0.clone()
     out = {"workload": "forward_65536", "envs": n}
+
+    def rate(ms):
+        return {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3, "tflops": FWD_FLOP * n / ms / 1e9,
+                "frac_fp32_mfma_peak": FWD_FLOP * n / ms / 1e9 / PEAK_FP32}
     for name, on in (("fp32", False), ("bf16_in", True)):
         pol.set_gemm_bf16(on)
-        ms = _time(torch, lambda: pol.forward(rec, term, pol.state, av=av), reps)
-        out[name] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
-                     "tflops": FWD_FLOP * n / ms / 1e9,
-                     "frac_fp32_mfma_peak": FWD_FLOP * n / ms / 1e9 / PEAK_FP32}
+        state.copy_(st0)
+        out[name] = rate(_time(torch, lambda: pol.forward(rec, term, state, av=av), reps))
+    pol.set_gemm_bf16(False)
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.where(torch.rand(n, 843, device="cuda", generator=g) < 0.6,
+                    torch.randint(0, 41, (n, 843), device="cuda", generator=g).float(),
+                    torch.rand(n, 843, device="cuda", generator=g))
+    state.copy_(st0)
+    out["fp32_from_feature_matrix"] = rate(_time(torch, lambda: pol.forward_features(x, term, state, av=av), reps))
+    h = torch.empty(n, 256, device="cuda")
+    W = pol.params[: 843 * 256].view(843, 256)
+    out["fp32_from_feature_matrix"]["encoder_gemm_ms"] = _time(
+        torch, lambda: pkg.policy.gemm_enc_fwd(W, x, h), reps)
     pol.close()
     return out
 

@@ -396,6 +396,39 @@ int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
     return run_chunked(a, n, chunk, (hipStream_t)stream);
 }
 
+// The same step fed by the fp32 feature matrix instead of records: the reference's
+// cu_gemm_enc_fwd on xobs (craftax_full.cu:11616) + k_add_bias (:10056), then the fused
+// layers and heads from the encoder output.  fp32 features are not exact in bf16, so the
+// encoder cannot run on the record path's three-term byte products; it goes through the
+// seam's encoder GEMM (and follows the seam's process-wide GEMM switches).
+int cfp_policy_forward_features(cfp_policy* p, const float* d_xobs, const float* d_terminals,
+                                float* d_state, float* d_r_state_t, float* d_h_enc, float* d_h3,
+                                float* d_av, int n, int chunk, void* stream) {
+    CFP_REQUIRE(p && d_xobs, "cfp_policy_forward_features: NULL argument");
+    CFP_REQUIRE(p->variant == 0, "cfp_policy_forward_features covers the full-game policy");
+    CFP_REQUIRE(d_state != nullptr || n == p->n,
+                "cfp_policy_forward_features: the object's live state covers %d envs, n=%d needs "
+                "an explicit state buffer", p->n, n);
+    CFP_REQUIRE((d_h_enc != nullptr && d_av != nullptr) || n <= p->n,
+                "cfp_policy_forward_features: n=%d exceeds the object's buffers (%d envs)", n, p->n);
+    float* h_enc = d_h_enc ? d_h_enc : p->h_enc;
+    const Arena ar = arena_of(0, p->layers);
+    if (gemm_enc_fwd_ld(n, p->params + ar.w_enc, d_xobs, CFP_OBS, h_enc, (hipStream_t)stream)) return 1;
+    if (cfp_add_bias(h_enc, p->params + ar.b_enc, n, stream)) return 1;
+    FwdArgs a{};
+    fill_weights(p, a);
+    a.x0 = h_enc;
+    a.terminals = d_terminals;
+    a.state = d_state ? d_state : p->h_state;
+    a.r_state = d_r_state_t;
+    a.h3_out = d_h3;
+    a.av_out = d_av ? d_av : p->logits;
+    a.layer_stride = (size_t)n * CFP_HIDDEN;
+    a.layers = p->layers;
+    a.do_head = 1;
+    return run_chunked(a, n, chunk, (hipStream_t)stream);
+}
+
 }  // extern "C"
 
 // ---- synthetic records -------------------------------------------------------

@@ -191,6 +191,19 @@ class Policy:
         return av
 
 
+    def forward_features(self, xobs, terminals, state, r_state_t=None, h_enc=None, h3=None,
+                         av=None, chunk=0):
+        """The same step from the fp32 feature matrix xobs[n][843] (cu_gemm_enc_fwd on
+        xobs + bias, then the fused layers and heads)."""
+        n = xobs.shape[0]
+        if av is None:
+            av = torch.empty((n, self.av_width), dtype=torch.float32, device=xobs.device)
+        _check(lib().cfp_policy_forward_features(self._h, _ptr(xobs), _ptr(terminals), _ptr(state),
+                                                 _ptr(r_state_t), _ptr(h_enc), _ptr(h3), _ptr(av),
+                                                 n, chunk, _stream()))
+        return av
+
+
 class Trainer:
     """cfp_trainer handle (CuTrain, craftax_full.cu:12688): rollout slabs, windowed
     recompute backward, GAE, Adam."""

@@ -171,6 +171,16 @@ int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
                        float* d_r_state_t, float* d_h_enc, float* d_h3,
                        float* d_av, int n, int chunk, void* stream);
 
+/* The same step from the fp32 feature matrix xobs[n][843] (ld 843) instead of records:
+ * cu_gemm_enc_fwd on xobs + k_add_bias (craftax_full.cu:11616, :10056; what
+ * cu_encode_step runs after k_expand_obs), then the fused MinGRU layers and heads.
+ * d_h_enc (NULL = the object's buffer) receives the encoder output.  The encoder GEMM is
+ * the seam's (cfp_gemm_enc_fwd), not the record path's fused one: fp32 features are not
+ * exact in bf16. */
+int cfp_policy_forward_features(cfp_policy* p, const float* d_xobs, const float* d_terminals,
+                                float* d_state, float* d_r_state_t, float* d_h_enc, float* d_h3,
+                                float* d_av, int n, int chunk, void* stream);
+
 /* ---- the dense-math seam (craftax_full.cu:11604-11666) ------------------- */
 /* Workspace of the raw entry points below (cfp_gemm_fwd / dh / dw, cfp_gemv_dwv):
  * 1.1 MB for the split mirror of W, 110 MB of split-K partial sums, 256 KB of gemv

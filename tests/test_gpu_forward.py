@@ -283,6 +283,77 @@ def test_full_size_properties(pkg, cuda):
     small.close(); pol.close()
 
 
+def _config2_features(n, cuda, seed):
+    """The second baseline configuration's feature matrix: each entry an integer U{0..40}
+    cast to float with probability 0.6, else U[0, 1)."""
+    import torch
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    ints = torch.randint(0, 41, (n, 843), generator=g).float()
+    cont = torch.rand(n, 843, generator=g)
+    pick = torch.rand(n, 843, generator=g) < 0.6
+    return torch.where(pick, ints, cont).to(cuda)
+
+
+def test_config2_feature_matrix_at_65536(pkg, cuda):
+    """The second baseline configuration as stated: 65 536 envs, an fp32 feature matrix
+    [65536][843] (60 % small integers, 40 % U[0,1) in every column), prior hidden state
+    N(0, 0.5), one step, through cfp_policy_forward_features.  Sampled 32-env tiles
+    (first, last, spread) against the fp64 oracle on the same rows; the whole batch is
+    finite and reproduces, rows of the sampled tiles run alone give the same bits."""
+    import torch
+    n = 65536
+    pol = pkg.Policy(n, L, seed=1)
+    params = pol.get_params()
+    x = _config2_features(n, cuda, 21)
+    assert 0.35 < float((x != x.floor()).float().mean()) < 0.45
+    term = torch.zeros(n, device=cuda)
+    st0 = torch.randn(L, n, HIDDEN, device=cuda, generator=torch.Generator(device=cuda).manual_seed(22)) * 0.5
+    st_a = st0.clone()
+    h_enc = torch.empty(n, HIDDEN, device=cuda); h3 = torch.empty(n, HIDDEN, device=cuda)
+    av_a = pol.forward_features(x, term, st_a, h_enc=h_enc, h3=h3).clone()
+    st_b = st0.clone()
+    av_b = pol.forward_features(x, term, st_b)
+    torch.cuda.synchronize()
+    assert torch.equal(av_a, av_b) and torch.equal(st_a, st_b) and torch.isfinite(av_a).all()
+    tiles = [0, 1, 2047, 1024, 777, 1500]
+    idx = torch.cat([torch.arange(t * 32, t * 32 + 32) for t in tiles]).to(cuda)
+    ref = ob.forward_f64(params, L, x[idx].cpu().numpy(), st0[:, idx].cpu().numpy(), None)
+    assert_close(h_enc[idx].cpu().numpy(), ref["h_enc"], TOL_FP32, "config 2 h_enc")
+    assert_close(av_a[idx].cpu().numpy()[:, :ACTIONS], ref["logits"], TOL_FP32, "config 2 logits")
+    assert_close(av_a[idx].cpu().numpy()[:, ACTIONS], ref["values"], TOL_FP32, "config 2 values")
+    assert_close(st_a[:, idx].cpu().numpy(), ref["state"], TOL_FP32, "config 2 state")
+    assert_close(h3[idx].cpu().numpy(), ref["h3"], TOL_FP32, "config 2 h3")
+    pol.close()
+
+
+def test_config2_records_at_65536(pkg, cuda):
+    """The record-typed equivalent of the second configuration on the fused kernel:
+    65 536 envs of synthetic records, prior state N(0, 0.5), sampled tiles against the
+    fp64 oracle; rows of a sampled tile run alone reproduce bit for bit."""
+    import torch
+    n = 65536
+    pol = pkg.Policy(n, L, seed=1)
+    params = pol.get_params()
+    rec = pkg.policy.synth_records(n, 31, 0)
+    term = torch.zeros(n, device=cuda)
+    st0 = torch.randn(L, n, HIDDEN, device=cuda, generator=torch.Generator(device=cuda).manual_seed(32)) * 0.5
+    st = st0.clone()
+    av = pol.forward(rec, term, st).clone()
+    torch.cuda.synchronize()
+    tiles = [0, 2047, 1023, 311, 1999]
+    idx = torch.cat([torch.arange(t * 32, t * 32 + 32) for t in tiles]).to(cuda)
+    ref = ob.forward_f64(params, L, expand_records(rec[idx].cpu().numpy()), st0[:, idx].cpu().numpy(), None)
+    assert_close(av[idx].cpu().numpy()[:, :ACTIONS], ref["logits"], TOL_FP32, "config 2 (records) logits")
+    assert_close(av[idx].cpu().numpy()[:, ACTIONS], ref["values"], TOL_FP32, "config 2 (records) values")
+    assert_close(st[:, idx].cpu().numpy(), ref["state"], TOL_FP32, "config 2 (records) state")
+    small = pkg.Policy(len(idx), L, seed=1)
+    sub_st = st0[:, idx].contiguous()
+    av_s = small.forward(rec[idx].contiguous(), term[idx].contiguous(), sub_st)
+    torch.cuda.synchronize()
+    assert torch.equal(av_s, av[idx]) and torch.equal(sub_st, st[:, idx])
+    small.close(); pol.close()
+
+
 def test_forward_is_bitwise_reproducible_under_memory_pressure(pkg, cuda):
     """The kernel waits for its LDS-direct weight loads by counting its own vector
     memory operations; a miscount would read a ring slot before it has landed, and
