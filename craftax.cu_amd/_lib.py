@@ -33,6 +33,8 @@ PROTOTYPES = {
     "cfp_load_weights": (C.c_int, [vp, C.c_char_p]),
     "cfp_policy_set_gemm_bf16": (C.c_int, [vp, C.c_int]),
     "cfp_policy_gemm_bf16": (C.c_int, [vp]),
+    "cfp_policy_set_small_tiles": (C.c_int, [vp, C.c_int]),
+    "cfp_policy_small_tiles": (C.c_int, [vp]),
     "cfp_policy_params": (vp, [vp]),
     "cfp_policy_state": (vp, [vp]),
     "cfp_policy_rec": (vp, [vp]),

@@ -191,6 +191,18 @@ def rollout_policy_side(pkg, torch, reps):
         out["sizes"][str(n)] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
                                 "frac_fp32_mfma_peak": FWD_FLOP * n / ms / 1e9 / PEAK_FP32}
         if n <= 8192:
+            # 16-env tiles (opt-in): twice the CUs at work at these sizes
+            pol.set_small_tiles(True)
+            ms_t = _time(torch, round_, max(2, reps // 2), warm=1) / T
+            st = pol.state.clone()
+            av = torch.empty(n, 44, device="cuda")
+            ms_f = _time(torch, lambda: pol.forward(recs[0], term, st, av=av), reps)
+            pol.set_small_tiles(False)
+            ms_f32 = _time(torch, lambda: pol.forward(recs[0], term, st, av=av), reps)
+            out["sizes"][str(n)]["small_tiles"] = {
+                "ms_per_step": ms_t, "env_steps_per_s": n / ms_t * 1e3,
+                "frac_fp32_mfma_peak": FWD_FLOP * n / ms_t / 1e9 / PEAK_FP32,
+                "forward_only_ms": ms_f, "forward_only_ms_32_env_tiles": ms_f32}
             # the same round captured once into a graph and replayed, as the reference does
             # with its rollout (the device step counter keeps the draws fresh)
             side = torch.cuda.Stream()

@@ -43,6 +43,7 @@ static void policy_release(cfp_policy* p) {
     (void)hipFree(p->we_bf);
     (void)hipFree(p->wg_bf);
     (void)hipFree(p->wav_bf);
+    (void)hipFree(p->t16);
     (void)hipFree(p->h_state);
     (void)hipFree(p->rec);
     (void)hipFree(p->h_enc);
@@ -126,6 +127,7 @@ static int policy_create(cfp_policy** out, int num_envs, int layers, uint64_t se
     CFP_ALLOC(p->we_bf, kEncPackFloats * sizeof(uint16_t));
     CFP_ALLOC(p->wg_bf, (size_t)layers * kGruPackFloats * sizeof(uint16_t));
     CFP_ALLOC(p->wav_bf, kAvPackFloats * sizeof(uint16_t));
+    if (variant == 0) CFP_ALLOC(p->t16, t16_mirror_bytes(layers));
     CFP_ALLOC(p->h_state, (size_t)layers * hn * sizeof(float));
     CFP_ALLOC(p->rec, (size_t)num_envs * rec_bytes);
     CFP_ALLOC(p->h_enc, hn * sizeof(float));
@@ -255,9 +257,20 @@ int cfp_policy_refresh_weights(cfp_policy* p, void* stream) {
         return 1;
     if (launch_pack_enc_split(p->params, p->layers, p->variant, p->we_s3, (hipStream_t)stream) != 0)
         return 1;
-    return launch_pack_weights_bf16(p->params, p->layers, p->variant, p->we_bf, p->wg_bf,
-                                    p->wav_bf, (hipStream_t)stream);
+    if (launch_pack_weights_bf16(p->params, p->layers, p->variant, p->we_bf, p->wg_bf, p->wav_bf,
+                                 (hipStream_t)stream) != 0)
+        return 1;
+    if (p->t16) return launch_pack_weights_t16(p->params, p->layers, p->t16, (hipStream_t)stream);
+    return 0;
 }
+
+int cfp_policy_set_small_tiles(cfp_policy* p, int on) {
+    CFP_REQUIRE(p, "cfp_policy_set_small_tiles: NULL policy");
+    CFP_REQUIRE(!on || p->t16, "16-env tiles exist for the full-game policy only");
+    p->small_tiles = on ? 1 : 0;
+    return 0;
+}
+int cfp_policy_small_tiles(const cfp_policy* p) { return p ? p->small_tiles : -1; }
 
 int cfp_policy_set_gemm_bf16(cfp_policy* p, int on) {
     CFP_REQUIRE(p, "cfp_policy_set_gemm_bf16: NULL policy");
@@ -294,6 +307,8 @@ void cfp::fill_forward_weights(const cfp_policy* p, FwdArgs& a) {
     a.wg_bf = reinterpret_cast<const u4*>(p->wg_bf);
     a.wav_bf = reinterpret_cast<const u4*>(p->wav_bf);
     a.bf16 = p->gemm_bf16;
+    if (p->small_tiles && p->t16)
+        t16_mirror_layout(p->t16, p->layers, &a.t16_enc_s, &a.t16_enc_t, &a.t16_wg, &a.t16_wav);
 }
 
 extern "C" {

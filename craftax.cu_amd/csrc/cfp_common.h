@@ -125,6 +125,11 @@ struct FwdArgs {
     const u4* wg_bf;
     const u4* wav_bf;
     int bf16;                // bf16-input / fp32-accumulate kernel
+    // mirrors of the 16-env-tile kernel (policy_forward_t16.hip); null = not in use
+    const u4* t16_enc_s;
+    const f4* t16_enc_t;
+    const f4* t16_wg;
+    const f4* t16_wav;
     // Window recompute of the PPO update (fp32 full game only): "env" c of this
     // launch is window column c = (t0 + c / mb, env_start + c % mb); `rec` is the
     // r_obs slab, `state` the r_state slab [T][layers][n_all][256] whose stored
@@ -139,6 +144,13 @@ struct FwdArgs {
 };
 int launch_forward(const FwdArgs& a, hipStream_t st);
 int launch_forward_bf16(const FwdArgs& a, hipStream_t st);   // called by launch_forward
+// 16-env tiles for small batches (opt-in per policy); called by launch_forward
+bool forward_t16_ok(const FwdArgs& a);
+int launch_forward_t16(const FwdArgs& a, hipStream_t st);
+size_t t16_mirror_bytes(int layers);
+void t16_mirror_layout(void* base, int layers, const u4** enc_s, const f4** enc_t, const f4** gru,
+                       const f4** av);
+int launch_pack_weights_t16(const float* params, int layers, void* mirrors, hipStream_t st);
 int launch_pack_weights_bf16(const float* params, int layers, int variant, uint16_t* we_bf,
                              uint16_t* wg_bf, uint16_t* wav_bf, hipStream_t st);
 

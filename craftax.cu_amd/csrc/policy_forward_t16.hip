@@ -1,0 +1,360 @@
+// Fused policy forward on 16-env tiles, for batches too small to give every CU a
+// 32-env tile (the rollout of a PPO run: a few thousand envs).  Same path as
+// policy_forward.hip -- records -> Linear(843->256) -> MinGRU x L -> actor/value heads,
+// replacing the reference's per-step chain (craftax_full.cu:11954-11962, 11988-12008,
+// 12044) in one launch -- on the 16 x 16 matrix instructions:
+//   v_mfma_f32_16x16x4_f32   gates, heads, the encoder's 51 fp32 tail features
+//   v_mfma_f32_16x16x32_bf16 the encoder's 792 byte-valued features against the exact
+//                            three-term bf16 split of the fp32 weights
+// A tile's matrix-pipe time is half that of a 32-env tile, and 4096 envs are 256 tiles:
+// one per CU instead of one per two.  Opt-in (cfp_policy_set_small_tiles): another MFMA
+// shape adds its products up in another order, so the last bits differ from the 32-env
+// kernels', which every other entry point and batch size share.
+//
+// Workgroup: 512 threads = 8 waves, two per SIMD (one wave's weight loads and epilogue
+// issue while the other's MFMAs run); wave w owns units [32w, 32w+32) as two 16-wide
+// unit tiles.  Operand layout of the 16 x 16 instructions: lane l supplies row (A) /
+// column (B) l%16 and k group l/16; accumulator register r of lane l holds env
+// 4*(l/16) + r, unit l%16.  Weights come from mirrors in that order (k_pack_t16): one
+// 16-byte element per lane feeds four k steps, a wave's fragment is a contiguous 1 KiB.
+#include "policy_tile.h"
+
+namespace cfp {
+namespace {
+
+constexpr int kT16Envs = 16;
+constexpr int kT16Threads = 512;
+constexpr int kT16EncSteps = (CFP_OBS_MAP + 31) / 32;   // 25 K steps of 32 map bytes
+constexpr int kT16TailBlocks = 4;                       // 64 >= 51 fp32 tail features
+constexpr int kT16GateBlocks = CFP_HIDDEN / 16;         // 16 K blocks of 16
+constexpr int kT16HeadTiles = 3;                        // 48 >= 44 head rows
+constexpr int kT16RecV4 = kT16Envs * REC_DW / 4;        // 996 16-byte chunks of records
+constexpr int kT16LdsFloats = kT16Envs * XS;            // x tile [16][260] >= records [16][255]
+static_assert(kT16Envs * RS <= kT16LdsFloats, "records fit the x tile");
+static_assert((kT16Envs * REC_DW) % 4 == 0, "a tile's records are whole 16-byte chunks");
+
+// mirror sizes in 16-byte elements
+constexpr size_t kT16EncS = (size_t)kT16EncSteps * 16 * 3 * 64;
+constexpr size_t kT16EncT = (size_t)kT16TailBlocks * 16 * 64;
+constexpr size_t kT16Gru = (size_t)kT16GateBlocks * 8 * 6 * 64;   // per layer
+constexpr size_t kT16Av = (size_t)kT16GateBlocks * kT16HeadTiles * 64;
+
+__device__ __forceinline__ f4 mfma4(float a, float b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f4 mfma32b(const u4& a, const u4& b, f4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// One 16-byte element of the mirrors per thread.
+//   encoder, map bytes : [step s][unit tile T][term][lane]  eight bf16: feature 32 s + 8 (l/16) + j,
+//                        unit 16 T + l%16, term = hi / mid / lo of the fp32 weight
+//   encoder, fp32 tail : [block B][unit tile T][lane]       feature 792 + 16 B + 4 (l/16) + m
+//   gates              : [layer][K][wave][gate*2 + ut][lane] row gate*256 + 32 wave + 16 ut + l%16,
+//                        k = 16 K + 4 (l/16) + m
+//   heads              : [K][row tile][lane]                 row 16 tile + l%16 (43 = value, then zeros)
+__global__ void k_pack_t16(const float* __restrict__ W_enc, const float* __restrict__ W_gru,
+                           const float* __restrict__ W_a, const float* __restrict__ W_v, int layers,
+                           u4* __restrict__ enc_s, f4* __restrict__ enc_t, f4* __restrict__ gru,
+                           f4* __restrict__ av) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = (int)(i & 63), q = lane >> 4, c = lane & 15;
+    if (i < kT16EncS) {
+        const int term = (int)((i >> 6) % 3), T = (int)((i / 192) % 16), s = (int)(i / (192 * 16));
+        uint32_t d[4];
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+            uint32_t pair = 0;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int f = 32 * s + 8 * q + 2 * p + h;
+                const float w = f < CFP_OBS_MAP ? W_enc[(size_t)f * CFP_HIDDEN + 16 * T + c] : 0.0f;
+                const __bf16 hi = (__bf16)w;
+                const float r1 = w - (float)hi;
+                const __bf16 mid = (__bf16)r1;
+                const __bf16 lo = (__bf16)(r1 - (float)mid);
+                const __bf16 v = term == 0 ? hi : (term == 1 ? mid : lo);
+                pair |= (uint32_t)__builtin_bit_cast(uint16_t, v) << (16 * h);
+            }
+            d[p] = pair;
+        }
+        enc_s[i] = u4{d[0], d[1], d[2], d[3]};
+        return;
+    }
+    i -= kT16EncS;
+    if (i < kT16EncT) {
+        const int T = (int)((i >> 6) % 16), B = (int)(i / (64 * 16));
+        f4 v;
+#pragma unroll
+        for (int m = 0; m < 4; m++) {
+            const int f = CFP_OBS_MAP + 16 * B + 4 * q + m;
+            v[m] = f < CFP_OBS ? W_enc[(size_t)f * CFP_HIDDEN + 16 * T + c] : 0.0f;
+        }
+        enc_t[i] = v;
+        return;
+    }
+    i -= kT16EncT;
+    if (i < (size_t)layers * kT16Gru) {
+        const int layer = (int)(i / kT16Gru);
+        const size_t j = i - (size_t)layer * kT16Gru;
+        const int t = (int)((j >> 6) % 6), wave = (int)((j / 384) % 8), K = (int)(j / (384 * 8));
+        const int row = (t >> 1) * CFP_HIDDEN + 32 * wave + 16 * (t & 1) + c;
+        const float* src = W_gru + ((size_t)layer * CFP_GRU + row) * CFP_HIDDEN + 16 * K + 4 * q;
+        gru[i] = f4{src[0], src[1], src[2], src[3]};
+        return;
+    }
+    i -= (size_t)layers * kT16Gru;
+    if (i < kT16Av) {
+        const int tile = (int)((i >> 6) % kT16HeadTiles), K = (int)(i / (64 * kT16HeadTiles));
+        const int row = 16 * tile + c;
+        const float* src = row < CFP_ACTIONS ? W_a + (size_t)row * CFP_HIDDEN
+                                             : (row == CFP_ACTIONS ? W_v : nullptr);
+        f4 v = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (src) {
+            src += 16 * K + 4 * q;
+            v = f4{src[0], src[1], src[2], src[3]};
+        }
+        av[i] = v;
+    }
+}
+
+// MODE 0: inference; MODE 1: also records the post-zero state (r_state).
+template <int MODE>
+__global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a) {
+    __shared__ __attribute__((aligned(16))) float lds[kT16LdsFloats];
+    __shared__ float term_s[kT16Envs];
+    const int tid = threadIdx.x;
+    const unsigned lane = (unsigned)(tid & 63);
+    const int q = (tid & 63) >> 4;     // k group of the operands, env group of the accumulators
+    const int c = tid & 15;            // row (A) / column (B) / unit within a 16-wide tile
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const size_t e0 = (size_t)blockIdx.x * kT16Envs;
+    const f4* xs4 = reinterpret_cast<const f4*>(lds);
+
+    // ---- stage the tile's records: contiguous 16-byte loads, rows re-strided to RS dwords
+    {
+        uint32_t* rs = reinterpret_cast<uint32_t*>(lds);
+        const u4* src = reinterpret_cast<const u4*>(a.rec + e0 * CFP_REC_BYTES);
+        for (int i = tid; i < kT16RecV4; i += kT16Threads) {
+            const u4 v = __builtin_nontemporal_load(src + i);
+            const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int d = 4 * i + k, row = d / REC_DW;
+                rs[row * RS + (d - row * REC_DW)] = w[k];
+            }
+        }
+        if (tid < kT16Envs * (RS - REC_DW)) {
+            const int row = tid / (RS - REC_DW);
+            rs[row * RS + REC_DW + (tid - row * (RS - REC_DW))] = 0u;
+        }
+        if (tid < kT16Envs) term_s[tid] = a.terminals ? a.terminals[e0 + tid] : 0.0f;
+    }
+    __syncthreads();
+    unsigned tmask = 0u;
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+        if (term_s[4 * q + r] != 0.0f) tmask |= 1u << r;
+
+    // element e = 4 ut + r of a lane: env 4 q + r, unit 32 wave + 16 ut + c
+    const unsigned soff = (unsigned)((4 * q) * CFP_HIDDEN + 32 * wave + c);
+    auto state_fetch = [&](const float* base, float (&v)[8]) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            v[e] = __builtin_nontemporal_load((base + ((e & 3) * CFP_HIDDEN + (e >> 2) * 16)) + soff);
+    };
+    float st[8], stn[8];
+    state_fetch(a.state + e0 * CFP_HIDDEN, st);   // layer 0's state lands under the encoder
+    // gate weights travel kAhead K blocks ahead through a register ring of kAhead + 1 slots;
+    // the first blocks of a layer are requested before the phase in front of it ends
+    constexpr int kAhead = 3;
+    constexpr size_t kBlock = 8 * 6 * 64;
+    f4 bq[kAhead + 1][6];
+    auto gate_preload = [&](int l) {
+        const f4* wp = a.t16_wg + ((size_t)l * kT16GateBlocks * 8 + wave) * 6 * 64 + lane;
+#pragma unroll
+        for (int i = 0; i < kAhead; i++)
+#pragma unroll
+            for (int t = 0; t < 6; t++) bq[i][t] = wp[(size_t)i * kBlock + t * 64];
+    };
+
+    // ---- encoder ----------------------------------------------------------------------
+    {
+        f4 eacc[2] = {f4{0, 0, 0, 0}, f4{0, 0, 0, 0}};
+        const uint32_t* rrow = reinterpret_cast<const uint32_t*>(lds) + c * RS;
+        const u4* ws = a.t16_enc_s + (size_t)(2 * wave) * 3 * 64 + lane;
+        constexpr size_t kStep = 16 * 3 * 64;
+        // weights requested kAhead steps ahead in program order; the compiler spreads the
+        // requests between the MFMAs (pinning them in front of each step measured slower:
+        // six requests in a row stall the wave's own MFMA issue)
+        u4 b[kAhead + 1][6];
+#pragma unroll
+        for (int i = 0; i < kAhead; i++)
+#pragma unroll
+            for (int t = 0; t < 6; t++) b[i][t] = ws[(size_t)i * kStep + t * 64];
+#pragma unroll
+        for (int s = 0; s < kT16EncSteps; s++) {
+            const int cb = s % (kAhead + 1);
+            if (s + kAhead < kT16EncSteps) {
+#pragma unroll
+                for (int t = 0; t < 6; t++)
+                    b[(s + kAhead) % (kAhead + 1)][t] = ws[(size_t)(s + kAhead) * kStep + t * 64];
+            }
+                u4 av = bytes_to_bf16x8(rrow[8 * s + 2 * q], rrow[8 * s + 2 * q + 1]);
+            if (s == kT16EncSteps - 1 && q == 3) av = u4{0u, 0u, 0u, 0u};   // 792..799: not map bytes
+#pragma unroll
+            for (int term = 0; term < 3; term++) {
+                eacc[0] = mfma32b(av, b[cb][term], eacc[0]);
+                eacc[1] = mfma32b(av, b[cb][3 + term], eacc[1]);
+            }
+            }
+        const float* frow = reinterpret_cast<const float*>(rrow) + CFP_OBS_MAP / 4;
+#pragma unroll
+        for (int B = 0; B < kT16TailBlocks; B++) {
+            const f4 w0 = a.t16_enc_t[(size_t)(B * 16 + 2 * wave) * 64 + lane];
+            const f4 w1 = a.t16_enc_t[(size_t)(B * 16 + 2 * wave + 1) * 64 + lane];
+#pragma unroll
+            for (int m = 0; m < 4; m++) {
+                const int k = 16 * B + 4 * q + m;
+                const float x = k < CFP_OBS_TAIL ? frow[k] : 0.0f;   // past the record: not read as a float
+                eacc[0] = mfma4(x, w0[m], eacc[0]);
+                eacc[1] = mfma4(x, w1[m], eacc[1]);
+            }
+        }
+        gate_preload(0);
+        __syncthreads();   // every wave is done with the record bytes
+#pragma unroll
+        for (int ut = 0; ut < 2; ut++) {
+            const float bias = a.b_enc[32 * wave + 16 * ut + c];
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                lds[(4 * q + r) * XS + 32 * wave + 16 * ut + c] = eacc[ut][r] + bias;
+        }
+    }
+    __syncthreads();
+    auto tile_out = [&](float* dst) {
+        f4* d4 = reinterpret_cast<f4*>(dst + e0 * CFP_HIDDEN);
+        for (int i = tid; i < kT16Envs * CFP_HIDDEN / 4; i += kT16Threads)
+            d4[i] = xs4[(i >> 6) * XS4 + (i & 63)];
+    };
+    if (a.h_enc_out) tile_out(a.h_enc_out);
+
+    // ---- MinGRU layers -------------------------------------------------------------------
+#pragma unroll 1
+    for (int l = 0; l < a.layers; l++) {
+        f4 acc[6];
+#pragma unroll
+        for (int t = 0; t < 6; t++) acc[t] = f4{0, 0, 0, 0};
+        const f4* wp = a.t16_wg + ((size_t)l * kT16GateBlocks * 8 + wave) * 6 * 64 + lane;
+        f4 av = xs4[c * XS4 + q];
+#pragma unroll
+        for (int K = 0; K < kT16GateBlocks; K++) {
+            if (K + kAhead < kT16GateBlocks) {
+#pragma unroll
+                for (int t = 0; t < 6; t++)
+                    bq[(K + kAhead) % (kAhead + 1)][t] = wp[(size_t)(K + kAhead) * kBlock + t * 64];
+            }
+            const f4 avn = xs4[c * XS4 + 4 * (K + 1 < kT16GateBlocks ? K + 1 : K) + q];
+#pragma unroll
+            for (int m = 0; m < 4; m++)
+#pragma unroll
+                for (int t = 0; t < 6; t++) acc[t] = mfma4(av[m], bq[K % (kAhead + 1)][t][m], acc[t]);
+            av = avn;
+            }
+        if (l + 1 < a.layers) gate_preload(l + 1);   // ahead of the epilogue's stores
+        __syncthreads();   // every wave has read the layer input
+        if (l + 1 < a.layers)
+            state_fetch(a.state + (size_t)(l + 1) * a.layer_stride + e0 * CFP_HIDDEN, stn);
+        float* st_base = a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN;
+        float* rs_base = MODE == 1 ? a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN : nullptr;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const int ut = e >> 2, r = e & 3;
+            const unsigned off = (unsigned)(r * CFP_HIDDEN + ut * 16);
+            const float s = ((tmask >> r) & 1u) ? 0.0f : st[e];
+            if (MODE == 1) __builtin_nontemporal_store(s, (rs_base + off) + soff);
+            const float zh = acc[0 + ut][r], zg = acc[2 + ut][r], zp = acc[4 + ut][r];
+            const float sg = sigmoid_fast(zg);
+            const float sh = sigmoid_fast(zh);
+            const float gh = zh >= 0.0f ? zh + 0.5f : sh;
+            const float out = __builtin_fmaf(sg, gh - s, s);
+            const float p = sigmoid_fast(zp);
+            float* xp = lds + (4 * q + r) * XS + 32 * wave + 16 * ut + c;
+            const float xv = *xp;
+            *xp = __builtin_fmaf(p, out - xv, xv);
+            __builtin_nontemporal_store(out, (st_base + off) + soff);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) st[e] = stn[e];
+        __syncthreads();
+    }
+    if (a.h3_out) tile_out(a.h3_out);
+
+    // ---- heads: waves 0..2 take one 16-row tile each over the full K ----------------------
+    if (wave < kT16HeadTiles) {
+        f4 hacc = {0, 0, 0, 0};
+        const f4* wp = a.t16_wav + (size_t)wave * 64 + lane;
+#pragma unroll
+        for (int K = 0; K < kT16GateBlocks; K++) {
+            const f4 hb = wp[(size_t)K * kT16HeadTiles * 64];
+            const f4 av = xs4[c * XS4 + 4 * K + q];
+#pragma unroll
+            for (int m = 0; m < 4; m++) hacc = mfma4(av[m], hb[m], hacc);
+        }
+        const int row = 16 * wave + c;
+        if (row < CFP_AV) {
+            const float bias = row < CFP_ACTIONS ? a.b_a[row] : a.b_v[0];
+            float* o = a.av_out + (e0 + 4 * q) * CFP_AV + row;
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[r * CFP_AV] = hacc[r] + bias;
+        }
+    }
+}
+
+}  // namespace
+
+size_t t16_mirror_bytes(int layers) {
+    return (kT16EncS + kT16EncT + (size_t)layers * kT16Gru + kT16Av) * 16;
+}
+
+void t16_mirror_layout(void* base, int layers, const u4** enc_s, const f4** enc_t, const f4** gru,
+                       const f4** av) {
+    char* p = static_cast<char*>(base);
+    *enc_s = reinterpret_cast<const u4*>(p);
+    p += kT16EncS * 16;
+    *enc_t = reinterpret_cast<const f4*>(p);
+    p += kT16EncT * 16;
+    *gru = reinterpret_cast<const f4*>(p);
+    p += (size_t)layers * kT16Gru * 16;
+    *av = reinterpret_cast<const f4*>(p);
+}
+
+int launch_pack_weights_t16(const float* params, int layers, void* mirrors, hipStream_t st) {
+    const u4* es; const f4 *et, *g, *av;
+    t16_mirror_layout(mirrors, layers, &es, &et, &g, &av);
+    const size_t total = kT16EncS + kT16EncT + (size_t)layers * kT16Gru + kT16Av;
+    const Arena ar = arena_of(0, layers);
+    hipLaunchKernelGGL(k_pack_t16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       params + ar.w_enc, params + ar.w_gru, params + ar.w_a, params + ar.w_v, layers,
+                       const_cast<u4*>(es), const_cast<f4*>(et), const_cast<f4*>(g),
+                       const_cast<f4*>(av));
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+bool forward_t16_ok(const FwdArgs& a) {
+    return a.t16_wg && a.variant == 0 && a.rec && !a.train && !a.bf16 && a.layers > 0 && a.do_head &&
+           a.state && a.av_out && a.n % kT16Envs == 0 && a.n <= kT16Envs * 256;
+}
+
+int launch_forward_t16(const FwdArgs& a, hipStream_t st) {
+    CFP_REQUIRE(forward_t16_ok(a), "16-env tiles: records -> heads of the full game, at most 4096 envs");
+    const dim3 g(a.n / kT16Envs), b(kT16Threads);
+    if (a.r_state) hipLaunchKernelGGL(k_policy_forward_t16<1>, g, b, 0, st, a);
+    else hipLaunchKernelGGL(k_policy_forward_t16<0>, g, b, 0, st, a);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+}  // namespace cfp

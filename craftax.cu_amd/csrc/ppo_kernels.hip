@@ -809,6 +809,8 @@ int launch_adam(cfp_policy* p, float* grads, float* m, float* v, const uint64_t*
     const int items = a.enc_items + a.mid_items + a.tail_items;
     hipLaunchKernelGGL(k_adam_mirrors, dim3((items + 255) / 256), dim3(256), 0, st, a);
     CFP_HIP_TRY(hipGetLastError());
+    // the 16-env-tile kernel's mirrors, when that mode is on, take one pack launch
+    if (p->small_tiles && p->t16) return launch_pack_weights_t16(p->params, L, p->t16, st);
     return 0;
 }
 

@@ -125,6 +125,10 @@ class Policy:
         (the reference's CF_GEMM_BF16 mode, craftax_full.cu:11306-11316)."""
         _check(lib().cfp_policy_set_gemm_bf16(self._h, 1 if on else 0))
 
+    def set_small_tiles(self, on=True):
+        """16-env tiles for batches of at most 4096 envs (cfp_policy_set_small_tiles)."""
+        _check(lib().cfp_policy_set_small_tiles(self._h, 1 if on else 0))
+
     @property
     def gemm_bf16(self):
         return bool(lib().cfp_policy_gemm_bf16(self._h))

@@ -130,6 +130,17 @@ int cfp_load_weights(cfp_policy* p, const char* path);
 int cfp_policy_set_gemm_bf16(cfp_policy* p, int on);
 int cfp_policy_gemm_bf16(const cfp_policy* p);
 
+/* 16-env tiles for small batches (no counterpart in the reference, whose cuBLAS GEMMs
+ * take any width): with the flag on, cfp_policy_forward (and the trainer's rollout
+ * steps built on it) runs batches of at most 4096 envs of the full game on 16-env
+ * tiles -- 4096 envs then occupy every CU instead of every other one.  Same path, same
+ * tolerance against the fp64 evaluation; the last bits differ from the 32-env kernels
+ * (another MFMA shape sums its products in another order), which is why it is opt-in:
+ * with the flag off every entry point and batch size produce the same bits for the
+ * same env.  fp32 only; ignored by the bf16-input kernel. */
+int cfp_policy_set_small_tiles(cfp_policy* p, int on);
+int cfp_policy_small_tiles(const cfp_policy* p);
+
 /* Borrowed device pointers owned by the policy object. */
 float* cfp_policy_params(cfp_policy* p);    /* [param_count]                 */
 float* cfp_policy_state(cfp_policy* p);     /* live h_state [layers][n][256] */

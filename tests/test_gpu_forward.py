@@ -399,3 +399,60 @@ def test_error_paths_on_device(pkg, cuda):
     with pytest.raises(pkg._lib.CfpError, match="param count"):
         pol.set_params(np.zeros(10, np.float32))
     pol.close()
+
+
+@pytest.mark.parametrize("n,layers,term_p", [(32, 3, 0.0), (96, 3, 0.3), (1024, 3, 0.1), (64, 1, 1.0),
+                                             (4096, 2, 0.05)])
+def test_small_tiles_match_oracle(pkg, cuda, n, layers, term_p):
+    """cfp_policy_set_small_tiles: the 16-env-tile kernel (16 x 16 matrix instructions, own
+    weight mirrors) against the fp64 oracle, plain and recording; its r_state record is a
+    copy / zero (exact); against the 32-env kernel it agrees to rounding but not in bits."""
+    import torch
+    params = random_params(layers, 300 + n)
+    pol = pkg.Policy(n, layers, seed=1)
+    pol.set_params(params)
+    pol.set_small_tiles(True)
+    rng = np.random.default_rng(n + 1)
+    rec_h = synth_records_host(n, 6, n)
+    state_h = (0.5 * rng.standard_normal((layers, n, HIDDEN))).astype(np.float32)
+    term_h = (rng.random(n) < term_p).astype(np.float32)
+    k = min(n, 512)     # the oracle takes the first rows
+    ref = ob.forward_f64(params, layers, expand_records(rec_h[:k]), state_h[:, :k], term_h[:k])
+    rec, term = _t(rec_h, cuda), _t(term_h, cuda)
+    for record in (False, True):
+        state = _t(state_h, cuda)
+        out = {"h_enc": torch.zeros(n, HIDDEN, device=cuda), "h3": torch.zeros(n, HIDDEN, device=cuda),
+               "r_state": torch.zeros(layers, n, HIDDEN, device=cuda) if record else None}
+        out["av"] = pol.forward(rec, term, state, r_state_t=out["r_state"], h_enc=out["h_enc"],
+                                h3=out["h3"])
+        torch.cuda.synchronize()
+        sub = {key: (v[:k] if v.dim() == 2 else v[:, :k]) if v is not None else None for key, v in out.items()}
+        _check_all(sub, ref, state[:, :k], f"small tiles n={n} L={layers} record={record}")
+        if record:
+            assert np.array_equal(out["r_state"].cpu().numpy()[:, :k], ref["r_state"].astype(np.float32))
+        assert torch.isfinite(out["av"]).all()
+    # the 32-env kernel on the same inputs: same result to rounding
+    pol.set_small_tiles(False)
+    state_b = _t(state_h, cuda)
+    av_b = pol.forward(rec, term, state_b)
+    torch.cuda.synchronize()
+    assert rel_err(out["av"].cpu().numpy(), av_b.cpu().numpy().astype(np.float64)) < 1e-4
+    assert rel_err(state.cpu().numpy(), state_b.cpu().numpy().astype(np.float64)) < 1e-4
+    pol.close()
+
+
+def test_small_tiles_leave_large_batches_alone(pkg, cuda):
+    """Above 4096 envs the flag changes nothing: the 32-env kernels run and the bits are
+    those of a policy without the flag."""
+    import torch
+    n = 16384
+    pol = pkg.Policy(n, L, seed=2)
+    rec = pkg.policy.synth_records(n, 41, 0)
+    term = torch.zeros(n, device=cuda)
+    st0 = torch.randn(L, n, HIDDEN, device=cuda) * 0.5
+    sa = st0.clone(); av_a = pol.forward(rec, term, sa).clone()
+    pol.set_small_tiles(True)
+    sb = st0.clone(); av_b = pol.forward(rec, term, sb)
+    torch.cuda.synchronize()
+    assert torch.equal(av_a, av_b) and torch.equal(sa, sb)
+    pol.close()

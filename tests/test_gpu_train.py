@@ -485,3 +485,30 @@ def test_backward_with_bf16_storage(pkg, cuda, n, T, minibatches, bwd_win, done_
         pkg.policy.set_gemm_bf16(False)
         tr.set_bf16_storage(False)
     tr.close(); pol.close()
+
+
+def test_small_tile_mirrors_follow_adam(pkg, cuda):
+    """With 16-env tiles on, cfp_train_adam also repacks that kernel's weight mirrors: after
+    two steps the trained policy's small-tile forward equals, bit for bit, that of a fresh
+    policy given the same parameters."""
+    import torch
+    n = 64
+    pol = pkg.Policy(n, L, seed=31)
+    pol.set_small_tiles(True)
+    tr = pkg.Trainer(pol, 4)
+    rng = np.random.default_rng(32)
+    for _ in range(2):
+        g = (rng.standard_normal(pol.param_count) * 0.1).astype(np.float32)
+        tr.buf("grads").copy_(_t(g, cuda))
+        tr.adam()
+    torch.cuda.synchronize()
+    twin = pkg.Policy(n, L, seed=98)
+    twin.set_params(pol.get_params())
+    twin.set_small_tiles(True)
+    rec = _t(synth_records_host(n, 33, 0), cuda)
+    term = torch.zeros(n, device=cuda)
+    s0 = (0.5 * rng.standard_normal((L, n, HIDDEN))).astype(np.float32)
+    sa, sb = _t(s0, cuda), _t(s0, cuda)
+    assert torch.equal(pol.forward(rec, term, sa), twin.forward(rec, term, sb))
+    assert torch.equal(sa, sb)
+    tr.close(); pol.close(); twin.close()
