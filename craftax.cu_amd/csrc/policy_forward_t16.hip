@@ -11,9 +11,13 @@
 // shape adds its products up in another order, so the last bits differ from the 32-env
 // kernels', which every other entry point and batch size share.
 //
-// Workgroup: 512 threads = 8 waves, two per SIMD (one wave's weight loads and epilogue
-// issue while the other's MFMAs run); wave w owns units [32w, 32w+32) as two 16-wide
-// unit tiles.  Operand layout of the 16 x 16 instructions: lane l supplies row (A) /
+// Workgroup: 512 threads = 8 waves, two per SIMD (one wave's weight requests and
+// epilogue issue while the other's MFMAs run); wave w owns units [32w, 32w+32) as two
+// 16-wide unit tiles.  Weights stream L2 -> per-wave LDS ring (LDS-direct loads, two K
+// blocks ahead, no registers written) -> registers (one block ahead): a 16-byte global
+// load into registers costs the issuing wave several times the matrix-pipe time of an
+// LDS-direct request plus the LDS read, and a 16-env tile needs twice the weight bytes
+// per MFMA cycle of a 32-env one.  Operand layout of the 16 x 16 instructions: lane l supplies row (A) /
 // column (B) l%16 and k group l/16; accumulator register r of lane l holds env
 // 4*(l/16) + r, unit l%16.  Weights come from mirrors in that order (k_pack_t16): one
 // 16-byte element per lane feeds four k steps, a wave's fragment is a contiguous 1 KiB.
@@ -38,6 +42,50 @@ constexpr size_t kT16EncS = (size_t)kT16EncSteps * 16 * 3 * 64;
 constexpr size_t kT16EncT = (size_t)kT16TailBlocks * 16 * 64;
 constexpr size_t kT16Gru = (size_t)kT16GateBlocks * 8 * 6 * 64;   // per layer
 constexpr size_t kT16Av = (size_t)kT16GateBlocks * kT16HeadTiles * 64;
+
+// ---- weight stream: global -> LDS ring -> registers ---------------------------------
+// One K block of a wave = six 1 KiB fragments = one ring slot.  The LDS-direct loads are
+// issued from inline assembly (lane l's 16 bytes land at M0 base + 16 l + offset); the
+// compiler does not know of them, so the wait that makes a slot readable is an explicit
+// s_waitcnt vmcnt(N), N = the number of vector-memory operations this lane's wave issued
+// after the slot's six (they complete in issue order).  The compiler's own waits then
+// only ever over-wait.  `after`: a register the slot's previous contents were last read
+// into; as an operand it keeps the request behind the completion of those reads.
+constexpr int kT16RingSlots = 2;
+constexpr int kT16SlotF4 = 6 * 64;
+
+__device__ __forceinline__ void t16_dma(const f4* src, f4* slot, unsigned lane, float after = 0.0f) {
+    const unsigned lds_lo = (unsigned)(size_t)slot;
+    const unsigned voff = lane * 16u;
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:1024\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:2048\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:3072"
+        :
+        : "v"(voff), "s"(src), "s"(lds_lo), "v"(after)
+        : "memory", "m0");
+    asm volatile(
+        "s_mov_b32 m0, %2\n\t"
+        "s_nop 0\n\t"
+        "global_load_lds_dwordx4 %0, %1\n\t"
+        "global_load_lds_dwordx4 %0, %1 offset:1024"
+        :
+        : "v"(voff), "s"(src + 4 * 64), "s"(lds_lo + 4096u)
+        : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n); n folds to a constant or to one of a few values chosen at run time
+__device__ __forceinline__ void t16_wait(int n) {
+#define CFP_T16_W(N) case N: asm volatile("s_waitcnt vmcnt(" #N ")" ::: "memory"); break;
+    switch (n) {
+        CFP_T16_W(6) CFP_T16_W(8) CFP_T16_W(14) CFP_T16_W(16) CFP_T16_W(22) CFP_T16_W(24) CFP_T16_W(30)
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+#undef CFP_T16_W
+}
 
 __device__ __forceinline__ f4 mfma4(float a, float b, f4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
@@ -123,6 +171,7 @@ __global__ void k_pack_t16(const float* __restrict__ W_enc, const float* __restr
 template <int MODE>
 __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[kT16LdsFloats];
+    __shared__ __attribute__((aligned(16))) f4 ring_all[8 * kT16RingSlots * kT16SlotF4];   // 96 KiB
     __shared__ float term_s[kT16Envs];
     const int tid = threadIdx.x;
     const unsigned lane = (unsigned)(tid & 63);
@@ -131,6 +180,19 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const size_t e0 = (size_t)blockIdx.x * kT16Envs;
     const f4* xs4 = reinterpret_cast<const f4*>(lds);
+    f4* const ring = ring_all + wave * (kT16RingSlots * kT16SlotF4);   // this wave's ring
+
+    // element e = 4 ut + r of a lane: env 4 q + r, unit 32 wave + 16 ut + c
+    const unsigned soff = (unsigned)((4 * q) * CFP_HIDDEN + 32 * wave + c);
+    auto state_fetch = [&](const float* base, float (&v)[8]) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+            v[e] = __builtin_nontemporal_load((base + ((e & 3) * CFP_HIDDEN + (e >> 2) * 16)) + soff);
+    };
+    // layer 0's state first: it travels beside the records and is older than every
+    // weight request (requests return in order: a later one would be held up behind it)
+    float st[8], stn[8];
+    state_fetch(a.state + e0 * CFP_HIDDEN, st);
 
     // ---- stage the tile's records: contiguous 16-byte loads, rows re-strided to RS dwords
     {
@@ -157,88 +219,98 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
     for (int r = 0; r < 4; r++)
         if (term_s[4 * q + r] != 0.0f) tmask |= 1u << r;
 
-    // element e = 4 ut + r of a lane: env 4 q + r, unit 32 wave + 16 ut + c
-    const unsigned soff = (unsigned)((4 * q) * CFP_HIDDEN + 32 * wave + c);
-    auto state_fetch = [&](const float* base, float (&v)[8]) {
-#pragma unroll
-        for (int e = 0; e < 8; e++)
-            v[e] = __builtin_nontemporal_load((base + ((e & 3) * CFP_HIDDEN + (e >> 2) * 16)) + soff);
+    constexpr size_t kBlock = 8 * 6 * 64;   // f4 per K block of the gate mirror
+    auto gate_base = [&](int l) { return a.t16_wg + ((size_t)l * kT16GateBlocks * 8 + wave) * 6 * 64; };
+    // the first two K blocks of a layer are requested before the phase in front of it ends
+    // (after0 / after1: registers the slots' last contents were read into)
+    auto gate_preload = [&](int l, float after0, float after1) {
+        t16_dma(gate_base(l), ring, lane, after0);
+        t16_dma(gate_base(l) + kBlock, ring + kT16SlotF4, lane, after1);
     };
-    float st[8], stn[8];
-    state_fetch(a.state + e0 * CFP_HIDDEN, st);   // layer 0's state lands under the encoder
-    // gate weights travel kAhead K blocks ahead through a register ring of kAhead + 1 slots;
-    // the first blocks of a layer are requested before the phase in front of it ends
-    constexpr int kAhead = 3;
-    constexpr size_t kBlock = 8 * 6 * 64;
-    f4 bq[kAhead + 1][6];
-    auto gate_preload = [&](int l) {
-        const f4* wp = a.t16_wg + ((size_t)l * kT16GateBlocks * 8 + wave) * 6 * 64 + lane;
-#pragma unroll
-        for (int i = 0; i < kAhead; i++)
-#pragma unroll
-            for (int t = 0; t < 6; t++) bq[i][t] = wp[(size_t)i * kBlock + t * 64];
-    };
+    constexpr int kStores = MODE == 1 ? 16 : 8;   // an epilogue's stores per lane: state (+ r_state)
 
     // ---- encoder ----------------------------------------------------------------------
     {
         f4 eacc[2] = {f4{0, 0, 0, 0}, f4{0, 0, 0, 0}};
         const uint32_t* rrow = reinterpret_cast<const uint32_t*>(lds) + c * RS;
-        const u4* ws = a.t16_enc_s + (size_t)(2 * wave) * 3 * 64 + lane;
+        // this wave's six fragments of a step: unit tiles 2 wave, 2 wave + 1 x (hi, mid, lo)
+        const f4* ws = reinterpret_cast<const f4*>(a.t16_enc_s) + (size_t)(2 * wave) * 3 * 64;
         constexpr size_t kStep = 16 * 3 * 64;
-        // weights requested kAhead steps ahead in program order; the compiler spreads the
-        // requests between the MFMAs (pinning them in front of each step measured slower:
-        // six requests in a row stall the wave's own MFMA issue)
-        u4 b[kAhead + 1][6];
+        // the fp32 tail's weights first: older than every ring request, used last
+        f4 tw[kT16TailBlocks][2];
 #pragma unroll
-        for (int i = 0; i < kAhead; i++)
+        for (int B = 0; B < kT16TailBlocks; B++) {
+            tw[B][0] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave) * 64 + lane];
+            tw[B][1] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave + 1) * 64 + lane];
+        }
+        asm volatile("" ::: "memory");
+        t16_dma(ws, ring, lane);
+        t16_dma(ws + kStep, ring + kT16SlotF4, lane);
+        u4 b[2][6];
+        t16_wait(6);   // step 0 landed; step 1 may be in flight
 #pragma unroll
-            for (int t = 0; t < 6; t++) b[i][t] = ws[(size_t)i * kStep + t * 64];
+        for (int t = 0; t < 6; t++) b[0][t] = __builtin_bit_cast(u4, ring[t * 64 + lane]);
 #pragma unroll
         for (int s = 0; s < kT16EncSteps; s++) {
-            const int cb = s % (kAhead + 1);
-            if (s + kAhead < kT16EncSteps) {
+            const int cb = s & 1, nb = cb ^ 1;
+            if (s + 2 < kT16EncSteps)
+                t16_dma(ws + (size_t)(s + 2) * kStep, ring + (s % kT16RingSlots) * kT16SlotF4, lane,
+                        __uint_as_float(b[cb][5].w));
+            if (s + 1 < kT16EncSteps) {
+                t16_wait(s + 2 < kT16EncSteps ? 6 : 0);   // step s+1 landed; younger: step s+2
+                const f4* slot = ring + ((s + 1) % kT16RingSlots) * kT16SlotF4 + lane;
 #pragma unroll
-                for (int t = 0; t < 6; t++)
-                    b[(s + kAhead) % (kAhead + 1)][t] = ws[(size_t)(s + kAhead) * kStep + t * 64];
+                for (int t = 0; t < 6; t++) b[nb][t] = __builtin_bit_cast(u4, slot[t * 64]);
             }
-                u4 av = bytes_to_bf16x8(rrow[8 * s + 2 * q], rrow[8 * s + 2 * q + 1]);
+            u4 av = bytes_to_bf16x8(rrow[8 * s + 2 * q], rrow[8 * s + 2 * q + 1]);
             if (s == kT16EncSteps - 1 && q == 3) av = u4{0u, 0u, 0u, 0u};   // 792..799: not map bytes
 #pragma unroll
             for (int term = 0; term < 3; term++) {
                 eacc[0] = mfma32b(av, b[cb][term], eacc[0]);
                 eacc[1] = mfma32b(av, b[cb][3 + term], eacc[1]);
             }
-            }
+        }
         const float* frow = reinterpret_cast<const float*>(rrow) + CFP_OBS_MAP / 4;
 #pragma unroll
         for (int B = 0; B < kT16TailBlocks; B++) {
-            const f4 w0 = a.t16_enc_t[(size_t)(B * 16 + 2 * wave) * 64 + lane];
-            const f4 w1 = a.t16_enc_t[(size_t)(B * 16 + 2 * wave + 1) * 64 + lane];
 #pragma unroll
             for (int m = 0; m < 4; m++) {
                 const int k = 16 * B + 4 * q + m;
                 const float x = k < CFP_OBS_TAIL ? frow[k] : 0.0f;   // past the record: not read as a float
-                eacc[0] = mfma4(x, w0[m], eacc[0]);
-                eacc[1] = mfma4(x, w1[m], eacc[1]);
+                eacc[0] = mfma4(x, tw[B][0][m], eacc[0]);
+                eacc[1] = mfma4(x, tw[B][1][m], eacc[1]);
             }
         }
-        gate_preload(0);
+        // biases before the preload: a load behind it would have to wait for it
+        float bias[2];
+#pragma unroll
+        for (int ut = 0; ut < 2; ut++) bias[ut] = a.b_enc[32 * wave + 16 * ut + c];
+        asm volatile("" ::: "memory");
+        // the ring is idle: its last two slots were read into b[0] and b[1]
+        if (a.layers > 0) gate_preload(0, __uint_as_float(b[0][5].w), __uint_as_float(b[1][5].w));
         __syncthreads();   // every wave is done with the record bytes
 #pragma unroll
-        for (int ut = 0; ut < 2; ut++) {
-            const float bias = a.b_enc[32 * wave + 16 * ut + c];
+        for (int ut = 0; ut < 2; ut++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                lds[(4 * q + r) * XS + 32 * wave + 16 * ut + c] = eacc[ut][r] + bias;
-        }
+                lds[(4 * q + r) * XS + 32 * wave + 16 * ut + c] = eacc[ut][r] + bias[ut];
     }
     __syncthreads();
-    auto tile_out = [&](float* dst) {
+    auto tile_out = [&](float* dst) {   // two 16-byte stores per lane
         f4* d4 = reinterpret_cast<f4*>(dst + e0 * CFP_HIDDEN);
-        for (int i = tid; i < kT16Envs * CFP_HIDDEN / 4; i += kT16Threads)
+#pragma unroll
+        for (int j = 0; j < kT16Envs * CFP_HIDDEN / 4 / kT16Threads; j++) {
+            const int i = tid + j * kT16Threads;
             d4[i] = xs4[(i >> 6) * XS4 + (i & 63)];
+        }
     };
-    if (a.h_enc_out) tile_out(a.h_enc_out);
+    // vector-memory operations this lane issued after the pending preload of layer 0:
+    // the stores of tile_out, if any
+    int pending = 0;
+    if (a.h_enc_out) {
+        tile_out(a.h_enc_out);
+        pending = 2;
+    }
 
     // ---- MinGRU layers -------------------------------------------------------------------
 #pragma unroll 1
@@ -246,26 +318,44 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
         f4 acc[6];
 #pragma unroll
         for (int t = 0; t < 6; t++) acc[t] = f4{0, 0, 0, 0};
-        const f4* wp = a.t16_wg + ((size_t)l * kT16GateBlocks * 8 + wave) * 6 * 64 + lane;
+        const f4* wp = gate_base(l);
+        // On entry blocks 0 and 1 have been requested, followed by `pending` other
+        // operations of this lane: block 0 has landed when at most 6 + pending are left.
+        f4 bl[2][6];
+        t16_wait(6 + pending);
+#pragma unroll
+        for (int t = 0; t < 6; t++) bl[0][t] = ring[t * 64 + lane];
         f4 av = xs4[c * XS4 + q];
 #pragma unroll
         for (int K = 0; K < kT16GateBlocks; K++) {
-            if (K + kAhead < kT16GateBlocks) {
+            const int cb = K & 1, nb = cb ^ 1;
+            if (K + 2 < kT16GateBlocks)
+                t16_dma(wp + (size_t)(K + 2) * kBlock, ring + (K % kT16RingSlots) * kT16SlotF4, lane,
+                        bl[cb][5][3]);
+            f4 avn = av;
+            if (K + 1 < kT16GateBlocks) {
+                // block K+1 landed; younger: block K+2 and, at K = 0, what followed the preload
+                if (K == 0) t16_wait(6 + pending);
+                else t16_wait(K + 2 < kT16GateBlocks ? 6 : 0);
+                const f4* slot = ring + ((K + 1) % kT16RingSlots) * kT16SlotF4 + lane;
 #pragma unroll
-                for (int t = 0; t < 6; t++)
-                    bq[(K + kAhead) % (kAhead + 1)][t] = wp[(size_t)(K + kAhead) * kBlock + t * 64];
+                for (int t = 0; t < 6; t++) bl[nb][t] = slot[t * 64];
+                avn = xs4[c * XS4 + 4 * (K + 1) + q];
             }
-            const f4 avn = xs4[c * XS4 + 4 * (K + 1 < kT16GateBlocks ? K + 1 : K) + q];
 #pragma unroll
             for (int m = 0; m < 4; m++)
 #pragma unroll
-                for (int t = 0; t < 6; t++) acc[t] = mfma4(av[m], bq[K % (kAhead + 1)][t][m], acc[t]);
+                for (int t = 0; t < 6; t++) acc[t] = mfma4(av[m], bl[cb][t][m], acc[t]);
             av = avn;
-            }
-        if (l + 1 < a.layers) gate_preload(l + 1);   // ahead of the epilogue's stores
+        }
+        // next layer's first blocks, ahead of this epilogue's loads and stores
+        if (l + 1 < a.layers) gate_preload(l + 1, bl[0][5][3], bl[1][5][3]);
         __syncthreads();   // every wave has read the layer input
-        if (l + 1 < a.layers)
+        pending = kStores;
+        if (l + 1 < a.layers) {
             state_fetch(a.state + (size_t)(l + 1) * a.layer_stride + e0 * CFP_HIDDEN, stn);
+            pending += 8;
+        }
         float* st_base = a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN;
         float* rs_base = MODE == 1 ? a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN : nullptr;
 #pragma unroll
