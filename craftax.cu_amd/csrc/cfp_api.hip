@@ -446,6 +446,50 @@ int cfp_policy_forward_features(cfp_policy* p, const float* d_xobs, const float*
 
 }  // extern "C"
 
+namespace cfp {
+namespace {
+__global__ void k_add_one_u64(uint64_t* ctr) { *ctr += 1; }
+}  // namespace
+
+int forward_and_sample(cfp_policy* p, const uint8_t* d_rec_row, const float* d_terminals,
+                       float* d_r_state_t, int n, const SampleOut& s, hipStream_t st) {
+    CFP_REQUIRE(p && d_rec_row && s.act && s.logp && s.step_ctr && s.ticket,
+                "forward_and_sample: NULL argument");
+    CFP_REQUIRE(n == p->n, "forward_and_sample: the policy's live state covers %d envs, not %d",
+                p->n, n);
+    FwdArgs a{};
+    fill_weights(p, a);
+    a.rec = d_rec_row;
+    a.terminals = d_terminals;
+    a.state = p->h_state;
+    a.r_state = d_r_state_t;
+    a.av_out = p->logits;
+    a.layer_stride = (size_t)n * CFP_HIDDEN;
+    a.layers = p->layers;
+    a.do_head = 1;
+    a.n = n;
+    FwdArgs f = a;
+    f.s_act = s.act;
+    f.s_logp = s.logp;
+    f.s_value = s.value;
+    f.s_env_actions = s.env_actions;
+    f.s_seed = s.seed;
+    f.s_step = s.step_ctr;
+    f.s_ticket = s.ticket;
+    if (forward_t16_ok(f)) return launch_forward_t16(f, st);
+    if (run_chunked(a, n, 0, st) != 0) return 1;
+    const bool ride = n < kSampleRowsFrom;   // the sampler's launch bumps the counter itself
+    if (value_sample(p->logits, n, a.actions, s.env_actions, s.act, s.logp, s.value, s.seed,
+                     s.step_ctr, ride ? s.ticket : nullptr, st) != 0)
+        return 1;
+    if (!ride) {
+        hipLaunchKernelGGL(k_add_one_u64, dim3(1), dim3(1), 0, st, s.step_ctr);
+        CFP_HIP_TRY(hipGetLastError());
+    }
+    return 0;
+}
+}  // namespace cfp
+
 // ---- synthetic records -------------------------------------------------------
 namespace cfp {
 // One thread per (env, dword): dwords 0..197 are four map bytes U{0..40},

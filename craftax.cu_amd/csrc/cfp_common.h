@@ -130,6 +130,15 @@ struct FwdArgs {
     const f4* t16_enc_t;
     const f4* t16_wg;
     const f4* t16_wav;
+    // 16-env-tile kernel only: the draw behind the heads (s_act null = no sampling).
+    // Offset *s_step, bumped by the last workgroup through the tickets at *s_ticket.
+    int32_t* s_act;
+    float* s_logp;
+    float* s_value;
+    float* s_env_actions;    // or null
+    uint64_t s_seed;
+    uint64_t* s_step;
+    unsigned* s_ticket;
     // Window recompute of the PPO update (fp32 full game only): "env" c of this
     // launch is window column c = (t0 + c / mb, env_start + c % mb); `rec` is the
     // r_obs slab, `state` the r_state slab [T][layers][n_all][256] whose stored

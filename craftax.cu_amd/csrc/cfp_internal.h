@@ -30,4 +30,29 @@ struct cfp_policy {
 namespace cfp {
 // weight pointers, variant and action count of a policy into launch arguments
 void fill_forward_weights(const cfp_policy* p, FwdArgs& a);
+
+// Sampler behind cfp_value_sample.  From kSampleRowsFrom envs on it runs one thread per
+// env; below, sixteen lanes per env, and there `ticket` (one zeroed word of device
+// memory, or null) makes the launch bump *d_step_ctr itself once every workgroup has
+// read it.
+constexpr int kSampleRowsFrom = 16384;
+int value_sample(const float* d_av, int n, int actions, float* d_env_actions, int32_t* d_actions,
+                 float* d_logprobs, float* d_values, uint64_t seed, const uint64_t* d_step_ctr,
+                 unsigned* ticket, hipStream_t st);
+
+// One rollout step's policy side for the trainer: records -> heads into the policy's
+// live state and logits (r_state recorded), then the draw into act / logp / value
+// (and env_actions when not null) with offset *step_ctr, then *step_ctr += 1.  One
+// launch where the 16-env-tile kernel applies, forward + sampler otherwise.
+struct SampleOut {
+    int32_t* act;
+    float* logp;
+    float* value;
+    float* env_actions;
+    uint64_t seed;
+    uint64_t* step_ctr;
+    unsigned* ticket;   // one zeroed word, left zeroed
+};
+int forward_and_sample(cfp_policy* p, const uint8_t* d_rec_row, const float* d_terminals,
+                       float* d_r_state_t, int n, const SampleOut& s, hipStream_t st);
 }  // namespace cfp

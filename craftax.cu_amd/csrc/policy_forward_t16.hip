@@ -22,6 +22,7 @@
 // 4*(l/16) + r, unit l%16.  Weights come from mirrors in that order (k_pack_t16): one
 // 16-byte element per lane feeds four k steps, a wave's fragment is a contiguous 1 KiB.
 #include "policy_tile.h"
+#include "sample_row.h"
 
 namespace cfp {
 namespace {
@@ -382,6 +383,8 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
     if (a.h3_out) tile_out(a.h3_out);
 
     // ---- heads: waves 0..2 take one 16-row tile each over the full K ----------------------
+    __shared__ float s_logit[kT16Envs * CFP_AV];
+    __shared__ float s_expo[kT16Envs * kMaxActions];
     if (wave < kT16HeadTiles) {
         f4 hacc = {0, 0, 0, 0};
         const f4* wp = a.t16_wav + (size_t)wave * 64 + lane;
@@ -397,8 +400,27 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
             const float bias = row < CFP_ACTIONS ? a.b_a[row] : a.b_v[0];
             float* o = a.av_out + (e0 + 4 * q) * CFP_AV + row;
 #pragma unroll
-            for (int r = 0; r < 4; r++) o[r * CFP_AV] = hacc[r] + bias;
+            for (int r = 0; r < 4; r++) {
+                const float v = hacc[r] + bias;
+                o[r * CFP_AV] = v;
+                s_logit[(4 * q + r) * CFP_AV + row] = v;
+            }
         }
+    }
+    // ---- the draw, sixteen lanes per env (sample_row.h), and the step counter's bump ---------
+    if (a.s_act) {   // uniform over the launch
+        __syncthreads();
+        const int sub = tid % kSampleLanes, slot = tid / kSampleLanes;
+        const bool live = slot < kT16Envs;
+        const float* lp = s_logit + (live ? slot : 0) * CFP_AV;
+        float* px = s_expo + (live ? slot : 0) * kMaxActions;
+        const float mx = sample_spread(lp, px, CFP_ACTIONS, sub, live);
+        __syncthreads();
+        if (live && sub == 0)
+            sample_draw<CFP_ACTIONS>(lp, px, mx, CFP_ACTIONS, (int)e0 + slot, a.s_seed, *a.s_step,
+                        a.s_env_actions, a.s_act, a.s_logp, a.s_value);
+        __syncthreads();
+        if (tid == 0) bump_by_last_group(a.s_ticket, a.s_step, gridDim.x);
     }
 }
 
@@ -434,6 +456,7 @@ int launch_pack_weights_t16(const float* params, int layers, void* mirrors, hipS
 }
 
 bool forward_t16_ok(const FwdArgs& a) {
+    if (a.s_act && !(a.s_logp && a.s_step && a.s_ticket)) return false;
     return a.t16_wg && a.variant == 0 && a.rec && !a.train && !a.bf16 && a.layers > 0 && a.do_head &&
            a.state && a.av_out && a.n % kT16Envs == 0 && a.n <= kT16Envs * 256;
 }

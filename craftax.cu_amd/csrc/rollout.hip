@@ -13,12 +13,11 @@
 // the uniform, the action and its log-probability follow the reference's
 // arithmetic exactly (max-shifted expf, ascending cumulative sum, first index
 // with target <= cum, last action as the fall-through).
-#include "cfp_common.h"
+#include "cfp_internal.h"
+#include "sample_row.h"
 
 namespace cfp {
 namespace {
-
-constexpr int kMaxActions = 64;
 
 // Sixteen lanes per env, sixteen envs per workgroup.  The workgroup's logits rows are
 // one contiguous piece of av and are staged through LDS with coalesced loads (a thread
@@ -27,13 +26,12 @@ constexpr int kMaxActions = 64;
 // exponentials -- are spread over the env's lanes; the two sums, whose rounding
 // depends on their order, are then run by one lane in the reference's ascending
 // order over the exponentials in LDS, so the draw is the sequential kernel's bit for bit.
-constexpr int kSampleLanes = 16;
 constexpr int kSampleEnvs = 256 / kSampleLanes;
 
 __global__ __launch_bounds__(256) void k_value_sample(
     const float* __restrict__ av, int avs, int actions, float* __restrict__ env_actions,
     int32_t* __restrict__ act, float* __restrict__ logprobs, float* __restrict__ values, int n,
-    uint64_t seed, const uint64_t* __restrict__ step_ctr) {
+    uint64_t seed, const uint64_t* step_ctr, unsigned* ticket) {
     __shared__ float logit[kSampleEnvs * (kMaxActions + 1)];
     __shared__ float expo[kSampleEnvs * kMaxActions];
     const int e0 = (int)blockIdx.x * kSampleEnvs;
@@ -45,31 +43,22 @@ __global__ __launch_bounds__(256) void k_value_sample(
     const bool live = slot < nb;
     const float* lp = logit + slot * avs;
     float* px = expo + slot * kMaxActions;
-    float m = -INFINITY;
-    if (live)
-        for (int a = sub; a < actions; a += kSampleLanes) m = fmaxf(m, lp[a]);
-#pragma unroll
-    for (int d = kSampleLanes / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, kSampleLanes));
-    if (live)
-        for (int a = sub; a < actions; a += kSampleLanes) px[a] = expf(lp[a] - m);
+    const float m = sample_spread(lp, px, actions, sub, live);
     __syncthreads();
-    if (!live || sub != 0) return;
-    const int e = e0 + slot;
-    if (values) values[e] = lp[actions];
-    float total = 0.0f;
-    for (int a = 0; a < actions; a++) total += px[a];
-    const uint64_t step = step_ctr ? *step_ctr : 0;
-    const float u = philox_uniform(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)e, step);
-    const float target = u * total;
-    float cum = 0.0f;
-    int action = actions - 1;
-    for (int a = 0; a < actions; a++) {
-        cum += px[a];
-        if (target <= cum) { action = a; break; }
+    if (live && sub == 0) {
+        const uint64_t step = step_ctr ? *step_ctr : 0;
+        if (actions == CFP_ACTIONS)
+            sample_draw<CFP_ACTIONS>(lp, px, m, actions, e0 + slot, seed, step, env_actions, act,
+                                     logprobs, values);
+        else
+            sample_draw(lp, px, m, actions, e0 + slot, seed, step, env_actions, act, logprobs,
+                        values);
     }
-    if (env_actions) env_actions[e] = (float)action;
-    act[e] = action;
-    logprobs[e] = lp[action] - m - logf(total);
+    if (ticket) {   // the counter's bump rides on this launch (uniform branch)
+        __syncthreads();
+        if (threadIdx.x == 0)
+            bump_by_last_group(ticket, const_cast<uint64_t*>(step_ctr), gridDim.x);
+    }
 }
 
 // Large batches: one thread per env, 128 envs per workgroup (every lane busy through
@@ -132,6 +121,30 @@ __global__ void k_record_rd(const float* __restrict__ rewards, const float* __re
 }
 
 }  // namespace
+
+// ticket not null (batches below kSampleRowsFrom envs only): the launch also bumps
+// *d_step_ctr once every workgroup has read it; *ticket is zero before and after.
+int value_sample(const float* d_av, int n, int actions, float* d_env_actions, int32_t* d_actions,
+                 float* d_logprobs, float* d_values, uint64_t seed, const uint64_t* d_step_ctr,
+                 unsigned* ticket, hipStream_t st) {
+    CFP_REQUIRE(d_av && d_actions && d_logprobs && n > 0, "cfp_value_sample: bad argument");
+    CFP_REQUIRE(actions > 0 && actions <= kMaxActions, "cfp_value_sample: actions must be in 1..%d",
+                kMaxActions);
+    CFP_REQUIRE(!ticket || (d_step_ctr && n < kSampleRowsFrom),
+                "value_sample: the in-launch counter bump covers batches below %d envs",
+                kSampleRowsFrom);
+    if (n >= kSampleRowsFrom)
+        hipLaunchKernelGGL(k_value_sample_rows, dim3((n + kSampleRowEnvs - 1) / kSampleRowEnvs),
+                           dim3(kSampleRowEnvs), 0, st, d_av, actions + 1, actions, d_env_actions,
+                           d_actions, d_logprobs, d_values, n, seed, d_step_ctr);
+    else
+        hipLaunchKernelGGL(k_value_sample, dim3((n + kSampleEnvs - 1) / kSampleEnvs), dim3(256), 0,
+                           st, d_av, actions + 1, actions, d_env_actions, d_actions, d_logprobs,
+                           d_values, n, seed, d_step_ctr, ticket);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
 }  // namespace cfp
 
 using namespace cfp;
@@ -141,19 +154,8 @@ extern "C" {
 int cfp_value_sample(const float* d_av, int n, int actions, float* d_env_actions,
                      int32_t* d_actions, float* d_logprobs, float* d_values, uint64_t seed,
                      const uint64_t* d_step_ctr, void* stream) {
-    CFP_REQUIRE(d_av && d_actions && d_logprobs && n > 0, "cfp_value_sample: bad argument");
-    CFP_REQUIRE(actions > 0 && actions <= kMaxActions, "cfp_value_sample: actions must be in 1..%d",
-                kMaxActions);
-    if (n >= 16384)
-        hipLaunchKernelGGL(k_value_sample_rows, dim3((n + kSampleRowEnvs - 1) / kSampleRowEnvs),
-                           dim3(kSampleRowEnvs), 0, (hipStream_t)stream, d_av, actions + 1, actions,
-                           d_env_actions, d_actions, d_logprobs, d_values, n, seed, d_step_ctr);
-    else
-        hipLaunchKernelGGL(k_value_sample, dim3((n + kSampleEnvs - 1) / kSampleEnvs), dim3(256), 0,
-                           (hipStream_t)stream, d_av, actions + 1, actions, d_env_actions,
-                           d_actions, d_logprobs, d_values, n, seed, d_step_ctr);
-    CFP_HIP_TRY(hipGetLastError());
-    return 0;
+    return value_sample(d_av, n, actions, d_env_actions, d_actions, d_logprobs, d_values, seed,
+                        d_step_ctr, nullptr, (hipStream_t)stream);
 }
 
 int cfp_record_rd(const float* d_rewards, const float* d_terminals, float* d_r_reward_row,

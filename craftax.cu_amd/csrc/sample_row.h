@@ -1,0 +1,82 @@
+// Categorical draw from one env's staged head row (actions logits, then the value),
+// shared by the stand-alone sampler (rollout.hip) and the small-batch forward kernel
+// that samples behind its heads (policy_forward_t16.hip): the same operations in the
+// same order in both, so both give the reference's draw (k_value_sample with
+// cf_nn_sample_action, craftax_full.cu:9714-9741, :9147-9165) bit for bit.
+#pragma once
+
+#include "cfp_common.h"
+
+namespace cfp {
+
+constexpr int kMaxActions = 64;
+constexpr int kSampleLanes = 16;   // lanes that share one env's row
+
+// Order-independent part, spread over the env's sixteen lanes (consecutive lanes of one
+// wave): the row maximum, returned to each of them, and px[a] = expf(lp[a] - max).
+// A workgroup barrier must follow before sample_draw reads px.
+__device__ __forceinline__ float sample_spread(const float* lp, float* px, int actions, int sub,
+                                               bool live) {
+    float m = -INFINITY;
+    if (live)
+        for (int a = sub; a < actions; a += kSampleLanes) m = fmaxf(m, lp[a]);
+#pragma unroll
+    for (int d = kSampleLanes / 2; d > 0; d >>= 1) m = fmaxf(m, __shfl_xor(m, d, kSampleLanes));
+    if (live)
+        for (int a = sub; a < actions; a += kSampleLanes) px[a] = expf(lp[a] - m);
+    return m;
+}
+
+// Order-dependent part, run by one lane of the env: the two sums in ascending action
+// order, the uniform of (seed, env, step), the first action whose cumulative sum
+// reaches the target (the last action as the fall-through), and the outputs.
+// ACTIONS > 0 fixes the action count at compile time: both loops unroll, the
+// exponentials are read from LDS once, in one batch, and what is left in sequence is
+// the two chains of additions.  The scan carries no early exit (a flag keeps the
+// first hit), which changes no result: the sums past the hit are not used.
+template <int ACTIONS = 0>
+__device__ __forceinline__ void sample_draw(const float* lp, const float* px, float m, int actions,
+                                            int e, uint64_t seed, uint64_t step,
+                                            float* __restrict__ env_actions,
+                                            int32_t* __restrict__ act,
+                                            float* __restrict__ logprobs,
+                                            float* __restrict__ values) {
+    const int na = ACTIONS > 0 ? ACTIONS : actions;
+    if (values) values[e] = lp[na];
+    const float u = philox_uniform(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)e, step);
+    float total = 0.0f;
+#pragma unroll
+    for (int a = 0; a < na; a++) total += px[a];
+    const float target = u * total;
+    float cum = 0.0f;
+    int action = na - 1;
+    bool open = true;
+#pragma unroll
+    for (int a = 0; a < na; a++) {
+        cum += px[a];
+        if (open && target <= cum) {
+            action = a;
+            open = false;
+        }
+    }
+    if (env_actions) env_actions[e] = (float)action;
+    act[e] = action;
+    logprobs[e] = lp[action] - m - logf(total);
+}
+
+// The step counter's bump without a launch of its own: every workgroup takes a ticket
+// once its lanes have used the counter, and the one that takes the last ticket writes
+// counter + 1 and clears the tickets for the next launch.  Called by one thread of
+// each workgroup, after a barrier that follows the workgroup's last read of the
+// counter.  Meant for launches of at most a few thousand workgroups (the tickets are
+// atomics on one word).
+__device__ __forceinline__ void bump_by_last_group(unsigned* ticket, uint64_t* ctr, unsigned groups) {
+    const uint64_t step = *ctr;   // unchanged until every ticket, this one included, is taken
+    __threadfence();
+    if (atomicAdd(ticket, 1u) == groups - 1) {
+        *ctr = step + 1;
+        *ticket = 0u;
+    }
+}
+
+}  // namespace cfp

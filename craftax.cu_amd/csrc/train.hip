@@ -136,6 +136,7 @@ struct cfp_trainer {
     float *grads = nullptr, *adam_m = nullptr, *adam_v = nullptr;
     uint64_t* adam_ctr = nullptr;
     uint64_t* step_ctr = nullptr;   // rollout steps taken (the sampler's offset), device side
+    unsigned* ticket = nullptr;     // workgroup tickets of the in-launch counter bump; zero between launches
     float* boot_state = nullptr;    // [L][n][256] copy of the live state for the bootstrap value
     float *d_lr = nullptr, *d_ent = nullptr;
     // window workspace
@@ -250,6 +251,7 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     TA(adam_v, pc * sizeof(float));
     TA(adam_ctr, sizeof(uint64_t));
     TA(step_ctr, sizeof(uint64_t));
+    TA(ticket, sizeof(unsigned));
     TA(boot_state, (size_t)tr->L * hn * sizeof(float));
     TA(d_lr, sizeof(float));
     TA(d_ent, sizeof(float));
@@ -357,16 +359,11 @@ int cfp_rollout_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
     if (d_rec_row != row)
         CFP_HIP_TRY(hipMemcpyAsync(row, d_rec_row, n * CFP_REC_BYTES, hipMemcpyDeviceToDevice,
                                    st));
-    if (cfp_policy_forward(tr->p, row, d_prev_terminals, nullptr, tr->r_state + o * tr->L * H,
-                           nullptr, nullptr, nullptr, tr->n, 0, stream) != 0)
-        return 1;
-    if (cfp_value_sample(tr->p->logits, tr->n, A, d_env_actions, tr->r_act + o, tr->r_logprob + o,
-                         tr->r_value + o, seed, tr->step_ctr, stream) != 0)
-        return 1;
-    hipLaunchKernelGGL(k_bump_ctr, dim3(1), dim3(1), 0, st, tr->step_ctr);
-    CFP_HIP_TRY(hipGetLastError());
+    const SampleOut so{tr->r_act + o,  tr->r_logprob + o, tr->r_value + o, d_env_actions,
+                       seed,           tr->step_ctr,      tr->ticket};
     (void)hn;
-    return 0;
+    return forward_and_sample(tr->p, row, d_prev_terminals, tr->r_state + o * tr->L * H, tr->n, so,
+                              st);
 }
 
 int cfp_train_bootstrap(cfp_trainer* tr, const uint8_t* d_rec_row, const float* d_terminals,

@@ -118,17 +118,22 @@ def test_record_rd(pkg, cuda):
     assert np.array_equal(r_done.cpu().numpy(), (term != 0).astype(np.uint8))
 
 
-def test_rollout_step_and_bootstrap(pkg, cuda):
+@pytest.mark.parametrize("n,small", [(256, False), (256, True), (4096, True), (16416, False)])
+def test_rollout_step_and_bootstrap(pkg, cuda, n, small):
     """cfp_rollout_step == forward on the live state + sampling with the device step
     counter, written into the slab rows; cfp_train_bootstrap values the next
-    records on a copy of the live state."""
+    records on a copy of the live state.  The cases cover the three forms of the step:
+    forward + sampler that bumps the counter in its own launch (256), the 16-env-tile
+    kernel that also draws and bumps (small), forward + row sampler + bump (16 416)."""
     import torch
-    n, T, seed = 256, 4, 4321
+    T, seed = 4, 4321
     params = random_params(L, 21, scale=0.5)
     pol = pkg.Policy(n, L, seed=1)
     pol.set_params(params)
     twin = pkg.Policy(n, L, seed=1)      # same weights, driven by hand
     twin.set_params(params)
+    pol.set_small_tiles(small)
+    twin.set_small_tiles(small)
     tr = pkg.Trainer(pol, T)
     rng = np.random.default_rng(22)
     pol.state.zero_()
