@@ -13,6 +13,7 @@
                   records (fuzzed reference states of tests/golden, tiled) and
                   records -> fp32 features, and the unfused MinGRU gate/blend
                   epilogue of one layer
+  stream_ceilings what plain library copies, fills and reads stream on the GPU
 
 Usage:  python craftax.cu_amd/bench_configs.py [--reps 10] [--only NAME]
 The headline workload (262 144 envs) is bench.py at the repository root."""
@@ -274,6 +275,25 @@ def record_kernels(pkg, torch, reps):
                                "frac_hbm_peak": b_e * n / ms_e / 1e6 / 8000}}
 
 
+def stream_ceilings(pkg, torch, reps):
+    """What plain library kernels stream on this GPU (1 GiB operands, far beyond every
+    cache): the yardstick for the HBM-bound kernels of the update next to the
+    published 8 TB/s.  Rates count bytes read plus bytes written."""
+    n = 1 << 28                                           # floats: 1 GiB
+    a = torch.randn(n, device="cuda")
+    b = torch.randn(n, device="cuda")
+    c = torch.empty(n, device="cuda")
+    gib = n * 4
+    out = {"workload": "stream_ceilings", "bytes_per_operand": gib}
+    for name, fn, moved in (("copy_1r_1w", lambda: c.copy_(a), 2 * gib),
+                            ("fill_1w", lambda: c.fill_(1.0), gib),
+                            ("sum_1r", lambda: a.sum(), gib),
+                            ("add_2r_1w", lambda: torch.add(a, b, out=c), 3 * gib)):
+        ms = _time(torch, fn, reps)
+        out[name] = {"ms": ms, "tb_per_s": moved / ms / 1e9}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=10)
@@ -284,7 +304,7 @@ def main():
     pkg = ge.load_package()
     assert torch.cuda.is_available(), "bench_configs.py needs a GPU"
     for fn in (forward_65536, ppo_update, ppo_update_shapes, rollout_policy_side, classic_1m,
-               record_kernels):
+               record_kernels, stream_ceilings):
         if args.only and fn.__name__ != args.only:
             continue
         print(json.dumps(fn(pkg, torch, args.reps)), flush=True)
