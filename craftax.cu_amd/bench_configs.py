@@ -30,9 +30,18 @@ UPD_FLOP = 4469248                   # per sample: recompute forward + backward
 CLASSIC_FLOP = 1179648 + 9216        # gate GEMMs + 18-row head (gather encoder not counted)
 
 
-def _time(torch, fn, reps, warm=2):
-    for _ in range(warm):
+def _time(torch, fn, reps, warm=2, warm_ms=80.0):
+    """Mean milliseconds of fn over reps calls (HIP events), after at least `warm` calls
+    and `warm_ms` of untimed work: the shader clock needs some tens of milliseconds of
+    load to rise from idle to its steady value, and a few short launches timed before
+    that read 10-25 % slow."""
+    import time
+    t0, calls = time.perf_counter(), 0
+    while calls < warm or (time.perf_counter() - t0) * 1e3 < warm_ms:
         fn()
+        calls += 1
+        if calls % 4 == 0:
+            torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     e0.record()

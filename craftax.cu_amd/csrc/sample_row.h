@@ -71,8 +71,11 @@ __device__ __forceinline__ void sample_draw(const float* lp, const float* px, fl
 // counter.  Meant for launches of at most a few thousand workgroups (the tickets are
 // atomics on one word).
 __device__ __forceinline__ void bump_by_last_group(unsigned* ticket, uint64_t* ctr, unsigned groups) {
-    const uint64_t step = *ctr;   // unchanged until every ticket, this one included, is taken
-    __threadfence();
+    // The counter is unchanged until every ticket, this one included, is taken.  No fence
+    // is needed in front of the ticket: the workgroup's reads of the counter have
+    // returned (their values were used before the barrier), and the two stores below
+    // become visible to the next launch at the end of this one.
+    const uint64_t step = *ctr;
     if (atomicAdd(ticket, 1u) == groups - 1) {
         *ctr = step + 1;
         *ticket = 0u;
