@@ -7,9 +7,10 @@
 // with one accumulator rounding per 16 products instead of per 2 -- and take 9/16 of
 // its pipe time.  The reference runs these GEMMs as cublasSgemm behind cu_gemm_dw
 // and cu_gemm_dh (craftax_full.cu:11642-11666).
-// TERMS = 6 leaves out mid*lo, lo*mid and lo*lo: at most 2^-23 of |a*b| per product
-// (2^-25 on average, always towards zero since the parts are truncations), i.e. below
-// one fp32 rounding of the product, for two thirds of the MFMAs.  Opt-in.
+// TERMS = 6 leaves out mid*lo, lo*mid and lo*lo: with truncated parts |mid| < 2^-7 |a|
+// and |lo| < 2^-15 |a|, so at most 2^-21 of |a*b| per product (about 2^-24 on average,
+// always towards zero), the size of the roundings the fp32 accumulation of those
+// products makes anyway, for two thirds of the MFMAs.  Opt-in.
 // TERMS = 1 is the seam's bf16-input mode (operands rounded to nearest even, one
 // product) on the same kernels: same loads and pipeline, a ninth of the MFMAs.
 //

@@ -217,8 +217,8 @@ int cfp_get_gemm_bf16(void);
  * craftax_full.cu:11642-11666, in 9/16 of the fp32 pipe time).  Used by cfp_gemm_dw and
  * cfp_gemm_dh for the shapes of the PPO update when bf16 inputs are off; other shapes
  * take the fp32 MFMA kernel.  mode 1 (default): all nine partial products; mode 2: the
- * six largest (mid*lo, lo*mid, lo*lo left out: at most 2^-23 of |a*b| per product,
- * below one fp32 rounding of it; opt-in); mode 0: fp32 MFMA everywhere (and, with bf16
+ * six largest (mid*lo, lo*mid, lo*lo left out: at most 2^-21 of |a*b| per product,
+ * about 2^-24 on average, the size of the roundings of the fp32 accumulation; opt-in); mode 0: fp32 MFMA everywhere (and, with bf16
  * inputs on, the generic bf16 kernel).  With cfp_set_gemm_bf16(1) and mode 1 or 2 the same
  * kernels run with both operands rounded to bf16 and one product. */
 int cfp_set_gemm_split(int mode);
