@@ -170,7 +170,7 @@ __global__ void k_pack_t16(const float* __restrict__ W_enc, const float* __restr
 
 // MODE 0: inference; MODE 1: also records the post-zero state (r_state).
 template <int MODE>
-__global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a) {
+__global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[kT16LdsFloats];
     __shared__ __attribute__((aligned(16))) f4 ring_all[8 * kT16RingSlots * kT16SlotF4];   // 96 KiB
     __shared__ float term_s[kT16Envs];
@@ -190,10 +190,27 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
         for (int e = 0; e < 8; e++)
             v[e] = __builtin_nontemporal_load((base + ((e & 3) * CFP_HIDDEN + (e >> 2) * 16)) + soff);
     };
-    // layer 0's state first: it travels beside the records and is older than every
-    // weight request (requests return in order: a later one would be held up behind it)
-    float st[8], stn[8];
-    state_fetch(a.state + e0 * CFP_HIDDEN, st);
+    // Every layer's state first: it travels beside the records, is older than every weight
+    // request (requests return in order: a state load issued later would hold the weight
+    // stream up behind its HBM latency) and has long landed when its epilogue comes.
+    float st[CFP_MAX_LAYERS][8];
+#pragma unroll
+    for (int l = 0; l < CFP_MAX_LAYERS; l++)
+        if (l < a.layers) state_fetch(a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN, st[l]);
+    // The encoder's first weights next, ahead of the records: the fp32 tail's rows (used
+    // last) and the first two steps of the ring.  The record loads that follow are the
+    // compiler's; its waits for them only over-wait for these older requests.
+    const f4* ws = reinterpret_cast<const f4*>(a.t16_enc_s) + (size_t)(2 * wave) * 3 * 64;
+    constexpr size_t kStep = 16 * 3 * 64;
+    f4 tw[kT16TailBlocks][2];
+#pragma unroll
+    for (int B = 0; B < kT16TailBlocks; B++) {
+        tw[B][0] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave) * 64 + lane];
+        tw[B][1] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave + 1) * 64 + lane];
+    }
+    asm volatile("" ::: "memory");
+    t16_dma(ws, ring, lane);
+    t16_dma(ws + kStep, ring + kT16SlotF4, lane);
 
     // ---- stage the tile's records: contiguous 16-byte loads, rows re-strided to RS dwords
     {
@@ -234,19 +251,9 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
     {
         f4 eacc[2] = {f4{0, 0, 0, 0}, f4{0, 0, 0, 0}};
         const uint32_t* rrow = reinterpret_cast<const uint32_t*>(lds) + c * RS;
-        // this wave's six fragments of a step: unit tiles 2 wave, 2 wave + 1 x (hi, mid, lo)
-        const f4* ws = reinterpret_cast<const f4*>(a.t16_enc_s) + (size_t)(2 * wave) * 3 * 64;
-        constexpr size_t kStep = 16 * 3 * 64;
-        // the fp32 tail's weights first: older than every ring request, used last
-        f4 tw[kT16TailBlocks][2];
-#pragma unroll
-        for (int B = 0; B < kT16TailBlocks; B++) {
-            tw[B][0] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave) * 64 + lane];
-            tw[B][1] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave + 1) * 64 + lane];
-        }
-        asm volatile("" ::: "memory");
-        t16_dma(ws, ring, lane);
-        t16_dma(ws + kStep, ring + kT16SlotF4, lane);
+        // (this wave's six fragments of a step: unit tiles 2 wave, 2 wave + 1 x (hi, mid, lo);
+        // steps 0 and 1 were requested before the records; every request of this lane
+        // since then has been consumed)
         u4 b[2][6];
         t16_wait(6);   // step 0 landed; step 1 may be in flight
 #pragma unroll
@@ -314,8 +321,9 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
     }
 
     // ---- MinGRU layers -------------------------------------------------------------------
-#pragma unroll 1
-    for (int l = 0; l < a.layers; l++) {
+#pragma unroll
+    for (int l = 0; l < CFP_MAX_LAYERS; l++) {
+        if (l >= a.layers) break;
         f4 acc[6];
 #pragma unroll
         for (int t = 0; t < 6; t++) acc[t] = f4{0, 0, 0, 0};
@@ -353,17 +361,13 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
         if (l + 1 < a.layers) gate_preload(l + 1, bl[0][5][3], bl[1][5][3]);
         __syncthreads();   // every wave has read the layer input
         pending = kStores;
-        if (l + 1 < a.layers) {
-            state_fetch(a.state + (size_t)(l + 1) * a.layer_stride + e0 * CFP_HIDDEN, stn);
-            pending += 8;
-        }
         float* st_base = a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN;
         float* rs_base = MODE == 1 ? a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN : nullptr;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const int ut = e >> 2, r = e & 3;
             const unsigned off = (unsigned)(r * CFP_HIDDEN + ut * 16);
-            const float s = ((tmask >> r) & 1u) ? 0.0f : st[e];
+            const float s = ((tmask >> r) & 1u) ? 0.0f : st[l][e];
             if (MODE == 1) __builtin_nontemporal_store(s, (rs_base + off) + soff);
             const float zh = acc[0 + ut][r], zg = acc[2 + ut][r], zp = acc[4 + ut][r];
             const float sg = sigmoid_fast(zg);
@@ -376,8 +380,6 @@ __global__ __launch_bounds__(kT16Threads, 2) void k_policy_forward_t16(FwdArgs a
             *xp = __builtin_fmaf(p, out - xv, xv);
             __builtin_nontemporal_store(out, (st_base + off) + soff);
         }
-#pragma unroll
-        for (int e = 0; e < 8; e++) st[e] = stn[e];
         __syncthreads();
     }
     if (a.h3_out) tile_out(a.h3_out);

@@ -387,6 +387,40 @@ def test_forward_is_bitwise_reproducible_under_memory_pressure(pkg, cuda):
         pol.close()
 
 
+def test_small_tiles_are_bitwise_reproducible_under_memory_pressure(pkg, cuda):
+    """The same guard for the 16-env-tile kernel, whose weight ring is waited for with
+    counted s_waitcnt as well: plain and r_state-recording forms at 4096 envs (all 256
+    CUs), one run alone and two racing a large device copy."""
+    import torch
+    n = 4096
+    side = torch.cuda.Stream()
+    big = torch.empty(1 << 28, dtype=torch.uint8, device=cuda)
+    pol = pkg.Policy(n, L, seed=5)
+    pol.set_small_tiles(True)
+    rec = pkg.policy.synth_records(n, 3, 1)
+    term = (torch.rand(n, device=cuda) < 0.1).float()
+    st0 = torch.randn(L, n, HIDDEN, device=cuda) * 0.5
+    for record in (False, True):
+        outs = []
+        for run in range(3):
+            st = st0.clone()
+            rs = torch.zeros_like(st0) if record else None
+            h_enc = torch.zeros(n, HIDDEN, device=cuda)
+            torch.cuda.synchronize()
+            if run:
+                with torch.cuda.stream(side):
+                    for _ in range(2):
+                        big[: 1 << 27].copy_(big[1 << 27:])
+            av = pol.forward(rec, term, st, r_state_t=rs, h_enc=h_enc if run != 1 else None).clone()
+            torch.cuda.synchronize()
+            outs.append((av, st, rs))
+        for av, st, rs in outs[1:]:
+            assert torch.equal(av, outs[0][0]) and torch.equal(st, outs[0][1]), record
+            if record:
+                assert torch.equal(rs, outs[0][2])
+    pol.close()
+
+
 def test_error_paths_on_device(pkg, cuda):
     import torch
     pol = pkg.Policy(64, L, seed=1)

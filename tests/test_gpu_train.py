@@ -191,7 +191,8 @@ def test_config4_shape_properties(pkg, cuda):
     """The PPO-update config at full size (4096 envs x 64 steps = 262 144 samples):
     too large for the oracle, so size-independent properties: the update is
     linear over envs (full-batch gradient = mean of the two half-batch
-    gradients, each normalised by its own size), finite and reproducible."""
+    gradients, each normalised by its own size), finite and reproducible, also while
+    other work competes for the memory system."""
     import torch
     n, T = 4096, 64
     pol = pkg.Policy(n, L, seed=1)
@@ -209,6 +210,17 @@ def test_config4_shape_properties(pkg, cuda):
     tr.buf("grads").zero_(); tr.backward(0, n); torch.cuda.synchronize()
     g_full = tr.buf("grads").clone()
     assert torch.isfinite(g_full).all()
+    # the reverse sweep waits for its own loads with counted s_waitcnt: the same backward
+    # racing a long run of device copies on another stream must give the same bits
+    side = torch.cuda.Stream()
+    big = torch.empty(1 << 28, dtype=torch.uint8, device=cuda)
+    tr.buf("grads").zero_(); torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(150):
+            big[: 1 << 27].copy_(big[1 << 27:])
+    tr.backward(0, n); torch.cuda.synchronize()
+    assert torch.equal(tr.buf("grads"), g_full), "backward depends on timing"
+    del big
     tr.buf("grads").zero_(); tr.backward(0, n // 2); tr.backward(n // 2, n // 2)
     torch.cuda.synchronize()
     g_halves = tr.buf("grads").clone() * 0.5
