@@ -66,6 +66,9 @@ PROTOTYPES = {
     "cfp_mingru_epi_fwd": (C.c_int, [vp, vp, vp, vp, vp, vp, C.c_int, vp]),
     "cfp_record_obs": (C.c_int, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp,
                                  C.c_int, vp]),
+    "cfp_record_obs_soa": (C.c_int, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp, vp, C.c_int, vp]),
+    "cfp_record_obs_soa_list": (C.c_int, [vp, vp, vp, vp, C.c_size_t, C.c_size_t, vp, C.c_size_t,
+                                          vp, C.c_int, vp, C.c_int, vp]),
     "cfp_ppo_defaults": (C.c_int, [vp]),
     "cfp_train_create": (C.c_int, [C.POINTER(vp), vp, C.c_int, vp]),
     "cfp_train_destroy": (None, [vp]),

@@ -261,6 +261,49 @@ def record_kernels(pkg, torch, reps):
     ms_r = _time(torch, lambda: P.record_obs(scalars, planes, planes[plane:], planes[2 * plane:],
                                              n, 3 * plane, 0, rec=rec), reps)
     ms_x = _time(torch, lambda: P.expand_obs(rec, n, xobs=xobs), reps)
+    # the same records from the reference's per-field device arrays (cfp_record_obs_soa): the
+    # fixture states scattered into [sub_index][env] arrays, mobs at the player's level
+    s32 = torch.from_numpy(np.ascontiguousarray(sc[idx]).view(np.int32).copy()).cuda()
+    names = ["player_position", "player_level", "player_direction", "player_health", "player_food",
+             "player_drink", "player_energy", "player_mana", "player_xp", "player_dexterity",
+             "player_strength", "player_intelligence", "is_sleeping", "is_resting", "inv_wood",
+             "inv_stone", "inv_coal", "inv_iron", "inv_diamond", "inv_sapphire", "inv_ruby",
+             "inv_sapling", "inv_torches", "inv_arrows", "inv_books", "inv_pickaxe", "inv_sword",
+             "inv_bow", "inv_potions", "inv_armour", "sword_enchantment", "bow_enchantment",
+             "armour_enchantments", "light_level", "learned_spells"]
+    arrays, w = {}, 0
+    kinds = dict(P.ENV_SOA_FIELDS)
+    for name in names:
+        k = kinds[name]
+        cols = s32[:, w:w + k].t().contiguous()
+        if name in ("player_health", "light_level"):
+            cols = cols.view(torch.float32)
+        elif name in ("is_sleeping", "is_resting", "learned_spells"):
+            cols = (cols != 0).to(torch.uint8)
+        arrays[name] = cols
+        w += k
+    level = s32[:, 2].clamp(0, 8).long()
+    env = torch.arange(n, device="cuda")
+    mk = torch.zeros(9, n, dtype=torch.int32, device="cuda")
+    mk[level, env] = s32[:, w]
+    arrays["monsters_killed"] = mk
+    arrays["boss_timesteps_to_spawn_this_round"] = s32[:, w + 1].contiguous()
+    w += 2
+    mt = torch.zeros(135, n, dtype=torch.int32, device="cuda")
+    mm = torch.zeros(135, n, dtype=torch.uint8, device="cuda")
+    mp = torch.zeros(270, n, dtype=torch.int32, device="cuda")
+    first, cls = (0, 3, 6, 8, 11), (0, 0, 0, 1, 1, 1, 2, 2, 3, 3, 3, 4, 4, 4)
+    for m in range(14):
+        cfm = (cls[m] * 9 + level) * 3 + (m - first[cls[m]])
+        mt[cfm, env] = s32[:, w + m]
+        mm[cfm, env] = (s32[:, w + 14 + m] != 0).to(torch.uint8)
+        mp[2 * cfm, env] = s32[:, w + 28 + 2 * m]
+        mp[2 * cfm + 1, env] = s32[:, w + 28 + 2 * m + 1]
+    arrays.update(mob_type_id=mt, mob_mask=mm, mob_position=mp)
+    rec2 = torch.empty_like(rec)
+    ms_s = _time(torch, lambda: P.record_obs_soa(arrays, n, planes, planes[plane:], planes[2 * plane:],
+                                                 n, 3 * plane, 0, rec=rec2), reps)
+    assert torch.equal(rec, rec2), "records from the field arrays differ from the staged form"
     # the unfused gate/blend epilogue of one MinGRU layer (k_mingru_epi_fwd), recording form
     pre = torch.randn(n, 768, device="cuda")
     xin = torch.randn(n, 256, device="cuda")
@@ -277,6 +320,7 @@ def record_kernels(pkg, torch, reps):
     return {"workload": "record_kernels", "envs": n,
             "record_obs": {"ms": ms_r, "envs_per_s": n / ms_r * 1e3, "bytes_per_env": b_r,
                            "gb_per_s": b_r * n / ms_r / 1e6, "frac_hbm_peak": b_r * n / ms_r / 1e6 / 8000},
+            "record_obs_soa": {"ms": ms_s, "envs_per_s": n / ms_s * 1e3},
             "expand_obs": {"ms": ms_x, "envs_per_s": n / ms_x * 1e3, "bytes_per_env": b_x,
                            "gb_per_s": b_x * n / ms_x / 1e6, "frac_hbm_peak": b_x * n / ms_x / 1e6 / 8000},
             "mingru_epi_fwd": {"ms": ms_e, "envs_per_s": n / ms_e * 1e3, "bytes_per_env": b_e,

@@ -8,6 +8,8 @@
 // passive+1, ranged+1, mob-projectile+1, player-projectile+1}, then 51 raw
 // little-endian fp32 scalars.  All of it is integer/byte work bound by HBM
 // gathers; sixteen lanes encode one env.
+#include <cstring>
+
 #include "cfp_common.h"
 
 namespace cfp {
@@ -83,100 +85,240 @@ __constant__ uint8_t kSlotClass[CFP_MOB_SLOTS] = {0, 0, 0, 1, 1, 1, 2, 2,
 constexpr int kRecLanes = 16;                   // lanes per env: four envs per wavefront,
 constexpr int kRecEnvsPerWg = 256 / kRecLanes;  // more gathers in flight than with one (85 -> 42 us)
 
+// Where an env's scalars come from.  SOA: the reference's device state (one array per
+// field laid out [sub_index][env], craftax_full.cu:613-723); the kernel asks for the words
+// of cfp_env_scalars it needs and a table says which array holds each.
+constexpr int kSoaPtrs = 40;
+struct SoaArgs {
+    const void* p[kSoaPtrs];   // the pointer fields of cfp_env_soa, in declaration order
+    size_t n_stride;
+};
+static_assert(sizeof(cfp_env_soa) == sizeof(SoaArgs), "cfp_env_soa is forty pointers and a stride");
+constexpr int kScalarWords = (int)(sizeof(cfp_env_scalars) / 4);
+
+// One descriptor per 4-byte word of cfp_env_scalars: the array it comes from, how its
+// element is typed and how the sub-index is formed.
+enum : uint8_t { K_I32 = 0, K_F32 = 1, K_BOOL = 2 };
+enum : uint8_t { R_SUB = 0, R_LEVEL = 1, R_MOB = 2, R_MOBPOS0 = 3, R_MOBPOS1 = 4 };
+struct SoaWord { uint8_t ptr, kind, rule, aux; };
+// Mob words: the reference's arrays hold three slots per class and level, CFM(c, l, i) =
+// (c * 9 + l) * 3 + i (craftax_full.cu:706-712); aux = c * 27 + i, so the element is
+// aux + 3 * level (mob_position: twice that, plus the axis).  The 14 slots in class order:
+// melee 0..2, passive 3..5, ranged 6..7, mob projectiles 8..10, player projectiles 11..13.
+#define SW(ptr, kind, rule, aux) {ptr, kind, rule, aux}
+#define SW_SLOTS(ptr, kind, rule)                                                               \
+    SW(ptr, kind, rule, 0), SW(ptr, kind, rule, 1), SW(ptr, kind, rule, 2),                     \
+    SW(ptr, kind, rule, 27), SW(ptr, kind, rule, 28), SW(ptr, kind, rule, 29),                  \
+    SW(ptr, kind, rule, 54), SW(ptr, kind, rule, 55),                                           \
+    SW(ptr, kind, rule, 81), SW(ptr, kind, rule, 82), SW(ptr, kind, rule, 83),                  \
+    SW(ptr, kind, rule, 108), SW(ptr, kind, rule, 109), SW(ptr, kind, rule, 110)
+#define SW_POS(aux) SW(39, K_I32, R_MOBPOS0, aux), SW(39, K_I32, R_MOBPOS1, aux)
+__constant__ SoaWord kSoaWords[kScalarWords] = {
+    SW(0, K_I32, R_SUB, 0), SW(0, K_I32, R_SUB, 1),            // player_position
+    SW(1, K_I32, R_SUB, 0), SW(2, K_I32, R_SUB, 0),            // player_level, player_direction
+    SW(3, K_F32, R_SUB, 0),                                    // player_health
+    SW(4, K_I32, R_SUB, 0), SW(5, K_I32, R_SUB, 0), SW(6, K_I32, R_SUB, 0), SW(7, K_I32, R_SUB, 0),
+    SW(8, K_I32, R_SUB, 0), SW(9, K_I32, R_SUB, 0), SW(10, K_I32, R_SUB, 0), SW(11, K_I32, R_SUB, 0),
+    SW(12, K_BOOL, R_SUB, 0), SW(13, K_BOOL, R_SUB, 0),        // is_sleeping, is_resting
+    // wood stone coal iron diamond sapphire ruby sapling torches arrows books pickaxe sword bow
+    SW(14, K_I32, R_SUB, 0), SW(15, K_I32, R_SUB, 0), SW(16, K_I32, R_SUB, 0), SW(17, K_I32, R_SUB, 0),
+    SW(18, K_I32, R_SUB, 0), SW(19, K_I32, R_SUB, 0), SW(20, K_I32, R_SUB, 0), SW(21, K_I32, R_SUB, 0),
+    SW(22, K_I32, R_SUB, 0), SW(23, K_I32, R_SUB, 0), SW(24, K_I32, R_SUB, 0), SW(25, K_I32, R_SUB, 0),
+    SW(26, K_I32, R_SUB, 0), SW(27, K_I32, R_SUB, 0),
+    SW(28, K_I32, R_SUB, 0), SW(28, K_I32, R_SUB, 1), SW(28, K_I32, R_SUB, 2),   // potions
+    SW(28, K_I32, R_SUB, 3), SW(28, K_I32, R_SUB, 4), SW(28, K_I32, R_SUB, 5),
+    SW(29, K_I32, R_SUB, 0), SW(29, K_I32, R_SUB, 1), SW(29, K_I32, R_SUB, 2), SW(29, K_I32, R_SUB, 3),
+    SW(30, K_I32, R_SUB, 0), SW(31, K_I32, R_SUB, 0),          // sword / bow enchantment
+    SW(32, K_I32, R_SUB, 0), SW(32, K_I32, R_SUB, 1), SW(32, K_I32, R_SUB, 2), SW(32, K_I32, R_SUB, 3),
+    SW(33, K_F32, R_SUB, 0),                                   // light_level
+    SW(34, K_BOOL, R_SUB, 0), SW(34, K_BOOL, R_SUB, 1),        // learned_spells
+    SW(35, K_I32, R_LEVEL, 0),                                 // monsters_killed[player_level]
+    SW(36, K_I32, R_SUB, 0),                                   // boss_timesteps_to_spawn_this_round
+    SW_SLOTS(37, K_I32, R_MOB),                                // mob_type_id[slot]
+    SW_SLOTS(38, K_BOOL, R_MOB),                               // mob_mask[slot]
+    SW_POS(0), SW_POS(1), SW_POS(2), SW_POS(27), SW_POS(28), SW_POS(29), SW_POS(54), SW_POS(55),
+    SW_POS(81), SW_POS(82), SW_POS(83), SW_POS(108), SW_POS(109), SW_POS(110),   // mob_position
+};
+#undef SW_POS
+#undef SW_SLOTS
+#undef SW
+
+// Which envs a launch records.  skip (or null): envs whose byte is set are left alone
+// (the reference's k_record_obs, craftax_full.cu:9284-9296).  list (or null): only the envs
+// named by *count entries of an index list are recorded, grid-strided
+// (k_record_obs_list, :9303-9320); entry i is the int32 at list + i * list_stride.
+struct RecWhich {
+    const uint8_t* skip;
+    const unsigned char* list;
+    size_t list_stride;
+    const int* count;
+};
+
+constexpr int kWPos = (int)(offsetof(cfp_env_scalars, player_position) / 4);
+constexpr int kWLevel = (int)(offsetof(cfp_env_scalars, player_level) / 4);
+constexpr int kWBossTimer = (int)(offsetof(cfp_env_scalars, boss_timesteps_to_spawn_this_round) / 4);
+constexpr int kWMobType = (int)(offsetof(cfp_env_scalars, mob_type_id) / 4);
+constexpr int kWMobMask = (int)(offsetof(cfp_env_scalars, mob_mask) / 4);
+constexpr int kWMobPos = (int)(offsetof(cfp_env_scalars, mob_position) / 4);
+
+// SOA: the env's scalars are first gathered into an LDS copy of cfp_env_scalars, transposed:
+// thread (word group gw, env ge) fetches words gw, gw + 16, ... of env ge, so the sixteen
+// lanes of a word read sixteen adjacent envs of one field array -- one 64-byte piece --
+// and all of a thread's seven elements are in flight together.  The rest of the kernel then
+// reads that copy exactly as it reads a caller-staged struct.
+struct WordSrc {
+    const uint32_t* w;
+    __device__ __forceinline__ uint32_t word(int i) const { return w[i]; }
+};
+
+template <bool SOA>
 __global__ __launch_bounds__(256) void k_record_obs(
-    const cfp_env_scalars* __restrict__ scalars,
+    const cfp_env_scalars* __restrict__ scalars, SoaArgs soa, RecWhich which,
     const uint8_t* __restrict__ map, const uint8_t* __restrict__ item_map,
     const uint8_t* __restrict__ light_map, size_t env_stride,
     size_t level_stride, uint8_t* __restrict__ rec_row, int n) {
     __shared__ uint32_t stage_all[kRecEnvsPerWg][CFP_REC_BYTES / 4 + 3];
+    __shared__ uint32_t sc_all[SOA ? kRecEnvsPerWg : 1][kScalarWords + 1];
+    __shared__ const void* ptrs[SOA ? kSoaPtrs : 1];
+    __shared__ SoaWord words[SOA ? kScalarWords : 1];
     const int lane = threadIdx.x % kRecLanes;
     const int slot = threadIdx.x / kRecLanes;
-    const int env = (int)blockIdx.x * kRecEnvsPerWg + slot;
-    if (env >= n) return;
-    uint32_t* stage = stage_all[slot];
-    const cfp_env_scalars* s = scalars + env;
-    const int pr = s->player_position[0], pc = s->player_position[1];
-    const int level = s->player_level;
-    const int mlevel = jax_index(level, 9);
-    const size_t cell_plane = (size_t)env * env_stride + (size_t)level * level_stride;
-    const size_t mob_plane = (size_t)env * env_stride + (size_t)mlevel * level_stride;
-
-    for (int cell = lane; cell < CELLS; cell += kRecLanes) {
-        const int row = cell / COLS, col = cell - row * COLS;
-        const int wr = pr - ROWS / 2 + row, wc = pc - COLS / 2 + col;
-        uint32_t lo = 0;
-        if (wr >= 0 && wr < MAP && wc >= 0 && wc < MAP) {
-            // all three planes requested at once (one memory round trip, not two)
-            const size_t o = cell_plane + (size_t)(wr * MAP + wc);
-            const uint32_t lv = light_map[o], bv = map[o], iv = item_map[o];
-            if (lv > 12) lo = bv | ((uint32_t)(uint8_t)(iv + 1) << 8) | (1u << 16);
-        }
-        stage[2 * cell] = lo;
-        stage[2 * cell + 1] = 0u;
-    }
-
-    // Mob slot m = lane contributes (cell, channel 3 + class, type + 1) when it passes
-    // the predicates of craftax_encode_mobs{3,2}_compact (craftax_full.c:2747-2825).
-    // Within a class the last slot on a cell wins: a slot stands back when one of the
-    // (at most two) later slots of its class sits on the same cell.
-    {
-        const int m = lane < CFP_MOB_SLOTS ? lane : CFP_MOB_SLOTS - 1;
-        const int type = s->mob_type_id[m];
-        const int mr = s->mob_position[m][0], mc = s->mob_position[m][1];
-        const int lr = mr - pr + ROWS / 2, lc = mc - pc + COLS / 2;
-        bool ok = lane < CFP_MOB_SLOTS && type >= 0 && type < 8 && s->mob_mask[m] != 0 &&
-                  lr >= 0 && lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
-                  mc >= 0 && mc < MAP;
-        if (ok) ok = light_map[mob_plane + (size_t)(mr * MAP + mc)] > 12;
-        const int cell = ok ? lr * COLS + lc : -1;
-        const int cls = kSlotClass[m];
-        bool over = false;
+    if (SOA) {
 #pragma unroll
-        for (int d = 1; d <= 2; d++) {
-            const int oc = __shfl_down(cell, d, kRecLanes);
-            const int ocls = __shfl_down(cls, d, kRecLanes);
-            over = over || (lane + d < CFP_MOB_SLOTS && ocls == cls && oc == cell);
-        }
-        if (ok && !over)
-            reinterpret_cast<uint8_t*>(stage)[cell * 8 + 3 + cls] = (uint8_t)(type + 1);
+        for (int i = 0; i < kSoaPtrs; i++)
+            if ((int)threadIdx.x == i) ptrs[i] = soa.p[i];
+        if ((int)threadIdx.x < kScalarWords) words[threadIdx.x] = kSoaWords[threadIdx.x];
     }
-
-    for (int tj = lane; tj < CFP_OBS_TAIL; tj += kRecLanes) {
-        const TailSpec ts = kTail[tj];
-        const int32_t* fi = reinterpret_cast<const int32_t*>(s);
-        const int iv = fi[ts.field];
-        const float fv = __int_as_float(iv);
-        const float xi = (float)iv;
-        float v = 0.0f;
-        switch (ts.kind) {
-            // IEEE sqrt: HIP's __fsqrt_rn is the approximate native sqrt unless
-            // OCML_BASIC_ROUNDED_OPERATIONS is defined; the fp64 root rounded
-            // to fp32 is the correctly rounded fp32 root (53 >= 2*24 + 2).
-            case T_SQRT10: v = (float)sqrt((double)xi) * 0.1f; break;
-            case T_HALF: v = xi * 0.5f; break;
-            case T_QUARTER: v = xi * 0.25f; break;
-            case T_INT: v = xi; break;
-            case T_F10: v = fv * 0.1f; break;
-            case T_I10: v = xi * 0.1f; break;
-            case T_DIR: v = (iv - 1 == (int)ts.aux) ? 1.0f : 0.0f; break;
-            case T_FLOAT: v = fv; break;
-            case T_BOOL: v = iv != 0 ? 1.0f : 0.0f; break;
-            case T_KILLED: v = iv >= 8 ? 1.0f : 0.0f; break;
-            case T_BOSS: {
-                // craftax_wg_is_boss_vulnerable, craftax_full.c:2205: no live
-                // melee (slots 0..2) or ranged (slots 6..7) mob, spawn timer <= 0
-                bool any = false;
-                for (int m = 0; m < 3; m++) any = any || s->mob_mask[m] != 0;
-                for (int m = 6; m < 8; m++) any = any || s->mob_mask[m] != 0;
-                v = (!any && s->boss_timesteps_to_spawn_this_round <= 0) ? 1.0f : 0.0f;
-            } break;
+    const int total = which.list ? *which.count : n;
+    // the trip count is the same for every thread of the workgroup (barriers inside)
+    for (int first = (int)blockIdx.x * kRecEnvsPerWg; first < total;
+         first += (int)gridDim.x * kRecEnvsPerWg) {
+        if (SOA) {
+            __syncthreads();   // tables filled; the previous round's readers are done with sc_all
+            const int ge = threadIdx.x % kRecEnvsPerWg, gw = threadIdx.x / kRecEnvsPerWg;
+            const int gi = first + ge;
+            int genv = gi;
+            if (which.list && gi < total)
+                genv = *reinterpret_cast<const int32_t*>(which.list + (size_t)gi * which.list_stride);
+            if (gi < total && !(which.skip && which.skip[genv])) {
+                const int lvl = static_cast<const int32_t*>(ptrs[1])[genv];
+                const int lvl_c = lvl < 0 ? 0 : (lvl > 8 ? 8 : lvl);   // monsters_killed has nine entries
+                const int ml3 = 3 * jax_index(lvl, 9);
+                constexpr int kRounds = (kScalarWords + 15) / 16;
+                uint32_t val[kRounds];
+#pragma unroll
+                for (int r = 0; r < kRounds; r++) {
+                    const int w = gw + 16 * r;
+                    const SoaWord d = words[w < kScalarWords ? w : 0];
+                    size_t sub = d.aux;
+                    if (d.rule == R_LEVEL) sub = (size_t)lvl_c;
+                    if (d.rule == R_MOB) sub = (size_t)(d.aux + ml3);
+                    if (d.rule >= R_MOBPOS0) sub = (size_t)(2 * (d.aux + ml3) + (d.rule - R_MOBPOS0));
+                    const size_t idx = sub * soa.n_stride + (size_t)genv;
+                    const void* base = ptrs[d.ptr];
+                    val[r] = d.kind == K_BOOL
+                                 ? (uint32_t)(static_cast<const uint8_t*>(base)[idx] != 0)
+                                 : static_cast<const uint32_t*>(base)[idx];
+                }
+#pragma unroll
+                for (int r = 0; r < kRounds; r++)
+                    if (gw + 16 * r < kScalarWords) sc_all[ge][gw + 16 * r] = val[r];
+            }
+            __syncthreads();
         }
-        stage[CFP_OBS_MAP / 4 + tj] = __float_as_uint(v);
-    }
+        const int item = first + slot;
+        if (item >= total) continue;
+        int env = item;
+        if (which.list)
+            env = *reinterpret_cast<const int32_t*>(which.list + (size_t)item * which.list_stride);
+        if (which.skip && which.skip[env]) continue;
+        uint32_t* stage = stage_all[slot];
+        WordSrc s;
+        s.w = SOA ? sc_all[slot] : reinterpret_cast<const uint32_t*>(scalars + env);
+        const int level = (int)s.word(kWLevel);
+        const int mlevel = jax_index(level, 9);
+        const int pr = (int)s.word(kWPos), pc = (int)s.word(kWPos + 1);
+        const size_t cell_plane = (size_t)env * env_stride + (size_t)level * level_stride;
+        const size_t mob_plane = (size_t)env * env_stride + (size_t)mlevel * level_stride;
 
-    __builtin_amdgcn_wave_barrier();
-    uint32_t* out = reinterpret_cast<uint32_t*>(rec_row + (size_t)env * CFP_REC_BYTES);
-    for (int d = lane; d < CFP_REC_BYTES / 4; d += kRecLanes) out[d] = stage[d];
+        for (int cell = lane; cell < CELLS; cell += kRecLanes) {
+            const int row = cell / COLS, col = cell - row * COLS;
+            const int wr = pr - ROWS / 2 + row, wc = pc - COLS / 2 + col;
+            uint32_t lo = 0;
+            if (wr >= 0 && wr < MAP && wc >= 0 && wc < MAP) {
+                // all three planes requested at once (one memory round trip, not two)
+                const size_t o = cell_plane + (size_t)(wr * MAP + wc);
+                const uint32_t lv = light_map[o], bv = map[o], iv = item_map[o];
+                if (lv > 12) lo = bv | ((uint32_t)(uint8_t)(iv + 1) << 8) | (1u << 16);
+            }
+            stage[2 * cell] = lo;
+            stage[2 * cell + 1] = 0u;
+        }
+
+        // Mob slot m = lane contributes (cell, channel 3 + class, type + 1) when it passes
+        // the predicates of craftax_encode_mobs{3,2}_compact (craftax_full.c:2747-2825).
+        // Within a class the last slot on a cell wins: a slot stands back when one of the
+        // (at most two) later slots of its class sits on the same cell.
+        {
+            const int m = lane < CFP_MOB_SLOTS ? lane : CFP_MOB_SLOTS - 1;
+            const int type = (int)s.word(kWMobType + m);
+            const int mr = (int)s.word(kWMobPos + 2 * m), mc = (int)s.word(kWMobPos + 2 * m + 1);
+            const uint32_t mask = s.word(kWMobMask + m);
+            const int lr = mr - pr + ROWS / 2, lc = mc - pc + COLS / 2;
+            bool ok = lane < CFP_MOB_SLOTS && type >= 0 && type < 8 && mask != 0 &&
+                      lr >= 0 && lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
+                      mc >= 0 && mc < MAP;
+            if (ok) ok = light_map[mob_plane + (size_t)(mr * MAP + mc)] > 12;
+            const int cell = ok ? lr * COLS + lc : -1;
+            const int cls = kSlotClass[m];
+            bool over = false;
+#pragma unroll
+            for (int d = 1; d <= 2; d++) {
+                const int oc = __shfl_down(cell, d, kRecLanes);
+                const int ocls = __shfl_down(cls, d, kRecLanes);
+                over = over || (lane + d < CFP_MOB_SLOTS && ocls == cls && oc == cell);
+            }
+            if (ok && !over)
+                reinterpret_cast<uint8_t*>(stage)[cell * 8 + 3 + cls] = (uint8_t)(type + 1);
+        }
+
+        for (int tj = lane; tj < CFP_OBS_TAIL; tj += kRecLanes) {
+            const TailSpec ts = kTail[tj];
+            const int iv = (int)s.word(ts.field);
+            const float fv = __int_as_float(iv);
+            const float xi = (float)iv;
+            float v = 0.0f;
+            switch (ts.kind) {
+                // IEEE sqrt: HIP's __fsqrt_rn is the approximate native sqrt unless
+                // OCML_BASIC_ROUNDED_OPERATIONS is defined; the fp64 root rounded
+                // to fp32 is the correctly rounded fp32 root (53 >= 2*24 + 2).
+                case T_SQRT10: v = (float)sqrt((double)xi) * 0.1f; break;
+                case T_HALF: v = xi * 0.5f; break;
+                case T_QUARTER: v = xi * 0.25f; break;
+                case T_INT: v = xi; break;
+                case T_F10: v = fv * 0.1f; break;
+                case T_I10: v = xi * 0.1f; break;
+                case T_DIR: v = (iv - 1 == (int)ts.aux) ? 1.0f : 0.0f; break;
+                case T_FLOAT: v = fv; break;
+                case T_BOOL: v = iv != 0 ? 1.0f : 0.0f; break;
+                case T_KILLED: v = iv >= 8 ? 1.0f : 0.0f; break;
+                case T_BOSS: {
+                    // craftax_wg_is_boss_vulnerable, craftax_full.c:2205: no live
+                    // melee (slots 0..2) or ranged (slots 6..7) mob, spawn timer <= 0
+                    bool any = false;
+                    for (int m = 0; m < 3; m++) any = any || s.word(kWMobMask + m) != 0;
+                    for (int m = 6; m < 8; m++) any = any || s.word(kWMobMask + m) != 0;
+                    v = (!any && (int)s.word(kWBossTimer) <= 0) ? 1.0f : 0.0f;
+                } break;
+            }
+            stage[CFP_OBS_MAP / 4 + tj] = __float_as_uint(v);
+        }
+
+        __builtin_amdgcn_wave_barrier();
+        uint32_t* out = reinterpret_cast<uint32_t*>(rec_row + (size_t)env * CFP_REC_BYTES);
+        for (int d = lane; d < CFP_REC_BYTES / 4; d += kRecLanes) out[d] = stage[d];
+        __builtin_amdgcn_wave_barrier();   // the staging row is reused by the next item
+    }
 }
 
 __global__ void k_expand_obs(const uint8_t* __restrict__ r_obs,
@@ -355,11 +497,61 @@ int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
                 "record rows must be 4-byte aligned");
     CFP_REQUIRE(env_stride >= (size_t)MAP * MAP,
                 "cfp_record_obs: env_stride smaller than one 48x48 plane");
-    hipLaunchKernelGGL(k_record_obs, dim3((n + kRecEnvsPerWg - 1) / kRecEnvsPerWg), dim3(256), 0,
-                       (hipStream_t)stream, d_scalars, d_map, d_item_map,
+    hipLaunchKernelGGL(k_record_obs<false>, dim3((n + kRecEnvsPerWg - 1) / kRecEnvsPerWg),
+                       dim3(256), 0, (hipStream_t)stream, d_scalars, SoaArgs{}, RecWhich{}, d_map,
+                       d_item_map, d_light_map, env_stride, level_stride, d_rec_row, n);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+static int record_obs_soa(const cfp_env_soa* soa, const uint8_t* d_map, const uint8_t* d_item_map,
+                          const uint8_t* d_light_map, size_t env_stride, size_t level_stride,
+                          const RecWhich& which, int items, uint8_t* d_rec_row, int n,
+                          void* stream) {
+    CFP_REQUIRE(soa && d_map && d_item_map && d_light_map && d_rec_row,
+                "cfp_record_obs_soa: NULL argument");
+    CFP_REQUIRE(n > 0 && items > 0, "cfp_record_obs_soa: nothing to record");
+    CFP_REQUIRE((reinterpret_cast<uintptr_t>(d_rec_row) & 3u) == 0,
+                "record rows must be 4-byte aligned");
+    CFP_REQUIRE(env_stride >= (size_t)MAP * MAP,
+                "cfp_record_obs_soa: env_stride smaller than one 48x48 plane");
+    CFP_REQUIRE(soa->n_stride >= (size_t)n, "cfp_record_obs_soa: n_stride %zu below the env count %d",
+                soa->n_stride, n);
+    SoaArgs a;
+    std::memcpy(&a, soa, sizeof(a));
+    for (int i = 0; i < kSoaPtrs; i++)
+        CFP_REQUIRE(a.p[i] != nullptr, "cfp_record_obs_soa: field array %d of the view is NULL", i);
+    hipLaunchKernelGGL(k_record_obs<true>, dim3((items + kRecEnvsPerWg - 1) / kRecEnvsPerWg),
+                       dim3(256), 0, (hipStream_t)stream, nullptr, a, which, d_map, d_item_map,
                        d_light_map, env_stride, level_stride, d_rec_row, n);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
+}
+
+int cfp_record_obs_soa(const cfp_env_soa* soa, const uint8_t* d_map, const uint8_t* d_item_map,
+                       const uint8_t* d_light_map, size_t env_stride, size_t level_stride,
+                       const uint8_t* d_skip, uint8_t* d_rec_row, int n, void* stream) {
+    RecWhich w{};
+    w.skip = d_skip;
+    return record_obs_soa(soa, d_map, d_item_map, d_light_map, env_stride, level_stride, w, n,
+                          d_rec_row, n, stream);
+}
+
+int cfp_record_obs_soa_list(const cfp_env_soa* soa, const uint8_t* d_map,
+                            const uint8_t* d_item_map, const uint8_t* d_light_map,
+                            size_t env_stride, size_t level_stride, const void* d_env_list,
+                            size_t list_stride, const int* d_count, int max_count,
+                            uint8_t* d_rec_row, int n, void* stream) {
+    CFP_REQUIRE(d_env_list && d_count && list_stride >= 4 && list_stride % 4 == 0,
+                "cfp_record_obs_soa_list: bad list (entries are int32, stride a multiple of 4)");
+    CFP_REQUIRE(max_count > 0 && max_count <= n,
+                "cfp_record_obs_soa_list: max_count must be in 1..n (got %d)", max_count);
+    RecWhich w{};
+    w.list = static_cast<const unsigned char*>(d_env_list);
+    w.list_stride = list_stride;
+    w.count = d_count;
+    return record_obs_soa(soa, d_map, d_item_map, d_light_map, env_stride, level_stride, w,
+                          max_count, d_rec_row, n, stream);
 }
 
 int cfp_expand_obs(const uint8_t* d_r_obs, float* d_xobs, int t0, int count,

@@ -413,6 +413,57 @@ def record_obs(scalars_u8, maps, item_maps, light_maps, n, env_stride, level_str
     return rec
 
 
+# field arrays of cfp_env_soa in declaration order: (name, entries per env)
+ENV_SOA_FIELDS = (
+    ("player_position", 2), ("player_level", 1), ("player_direction", 1), ("player_health", 1),
+    ("player_food", 1), ("player_drink", 1), ("player_energy", 1), ("player_mana", 1),
+    ("player_xp", 1), ("player_dexterity", 1), ("player_strength", 1), ("player_intelligence", 1),
+    ("is_sleeping", 1), ("is_resting", 1), ("inv_wood", 1), ("inv_stone", 1), ("inv_coal", 1),
+    ("inv_iron", 1), ("inv_diamond", 1), ("inv_sapphire", 1), ("inv_ruby", 1), ("inv_sapling", 1),
+    ("inv_torches", 1), ("inv_arrows", 1), ("inv_books", 1), ("inv_pickaxe", 1), ("inv_sword", 1),
+    ("inv_bow", 1), ("inv_potions", 6), ("inv_armour", 4), ("sword_enchantment", 1),
+    ("bow_enchantment", 1), ("armour_enchantments", 4), ("light_level", 1), ("learned_spells", 2),
+    ("monsters_killed", 9), ("boss_timesteps_to_spawn_this_round", 1), ("mob_type_id", 135),
+    ("mob_mask", 135), ("mob_position", 270))
+
+
+def _env_soa_view(arrays, n_stride):
+    """cfp_env_soa for a dict of device tensors, one per field, each [entries][n_stride]."""
+    import ctypes as C
+    fields = [(name, C.c_void_p) for name, _ in ENV_SOA_FIELDS] + [("n_stride", C.c_size_t)]
+    view = type("cfp_env_soa", (C.Structure,), {"_fields_": fields})()
+    for name, k in ENV_SOA_FIELDS:
+        t = arrays[name]
+        assert t.is_contiguous() and t.numel() == k * n_stride, name
+        setattr(view, name, t.data_ptr())
+    view.n_stride = n_stride
+    return view
+
+
+def record_obs_soa(arrays, n_stride, maps, item_maps, light_maps, n, env_stride, level_stride,
+                   skip=None, rec=None):
+    """k_record_obs (:9284) from the reference's per-field device arrays."""
+    import ctypes as C
+    if rec is None:
+        rec = torch.empty((n, REC_BYTES), dtype=torch.uint8, device=maps.device)
+    view = _env_soa_view(arrays, n_stride)
+    _check(lib().cfp_record_obs_soa(C.addressof(view), _ptr(maps), _ptr(item_maps), _ptr(light_maps),
+                                    env_stride, level_stride, _ptr(skip), _ptr(rec), n, _stream()))
+    return rec
+
+
+def record_obs_soa_list(arrays, n_stride, maps, item_maps, light_maps, n, env_stride, level_stride,
+                        env_list, list_stride, count, max_count, rec):
+    """k_record_obs_list (:9303): only the envs named by the first *count list entries."""
+    import ctypes as C
+    view = _env_soa_view(arrays, n_stride)
+    _check(lib().cfp_record_obs_soa_list(C.addressof(view), _ptr(maps), _ptr(item_maps),
+                                         _ptr(light_maps), env_stride, level_stride, _ptr(env_list),
+                                         list_stride, _ptr(count), max_count, _ptr(rec), n,
+                                         _stream()))
+    return rec
+
+
 def value_sample(av, seed, step_ctr=None, env_actions=None):
     """k_value_sample (:9714): av [n][A+1] -> (actions i32[n], logprobs f32[n], values f32[n])."""
     n, w = av.shape

@@ -300,6 +300,78 @@ int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
                    size_t env_stride, size_t level_stride, uint8_t* d_rec_row,
                    int n, void* stream);
 
+/* The same records straight from the reference's device state, so that cu_encode_step
+ * (craftax_full.cu:11931-11955) needs no staging kernel in front of this library.
+ * cfp_env_soa is a view of the reference's per-field arrays (CF_SOA_FIELDS,
+ * craftax_full.cu:620-690; the device pointers g_cf_<field> :703-705): every array is
+ * laid out [sub_index][env] with stride n_stride (= g_cf_n) elements, bool fields are
+ * one byte, and the mob arrays are indexed CFM(class, level, slot) = (class * 9 +
+ * level) * 3 + slot (:706-712; mob_position: that * 2 + axis), classes in the order
+ * melee, passive, ranged, mob projectiles, player projectiles.  Only the fields the
+ * record encoder reads are listed; all forty pointers must be set.  The planes are the
+ * map / item_map / light_map members of the reference's state block: pass their
+ * addresses inside the first env's block, env_stride = sizeof(CraftaxState),
+ * level_stride = 48 * 48. */
+typedef struct cfp_env_soa {
+    const int32_t* player_position;            /* 2 */
+    const int32_t* player_level;
+    const int32_t* player_direction;
+    const float* player_health;
+    const int32_t* player_food;
+    const int32_t* player_drink;
+    const int32_t* player_energy;
+    const int32_t* player_mana;
+    const int32_t* player_xp;
+    const int32_t* player_dexterity;
+    const int32_t* player_strength;
+    const int32_t* player_intelligence;
+    const uint8_t* is_sleeping;                /* bool */
+    const uint8_t* is_resting;                 /* bool */
+    const int32_t* inv_wood;
+    const int32_t* inv_stone;
+    const int32_t* inv_coal;
+    const int32_t* inv_iron;
+    const int32_t* inv_diamond;
+    const int32_t* inv_sapphire;
+    const int32_t* inv_ruby;
+    const int32_t* inv_sapling;
+    const int32_t* inv_torches;
+    const int32_t* inv_arrows;
+    const int32_t* inv_books;
+    const int32_t* inv_pickaxe;
+    const int32_t* inv_sword;
+    const int32_t* inv_bow;
+    const int32_t* inv_potions;                /* 6 */
+    const int32_t* inv_armour;                 /* 4 */
+    const int32_t* sword_enchantment;
+    const int32_t* bow_enchantment;
+    const int32_t* armour_enchantments;        /* 4 */
+    const float* light_level;
+    const uint8_t* learned_spells;             /* bool, 2 */
+    const int32_t* monsters_killed;            /* 9 */
+    const int32_t* boss_timesteps_to_spawn_this_round;
+    const int32_t* mob_type_id;                /* 135 */
+    const uint8_t* mob_mask;                   /* bool, 135 */
+    const int32_t* mob_position;               /* 270 */
+    size_t n_stride;
+} cfp_env_soa;
+/* k_record_obs (craftax_full.cu:9284-9296).  `soa` is a host struct, read during the call.
+ * d_skip (or NULL): u8[n]; envs whose byte is non-zero are left untouched (the envs whose
+ * reset has not joined yet, recorded afterwards by the list form). */
+int cfp_record_obs_soa(const cfp_env_soa* soa, const uint8_t* d_map, const uint8_t* d_item_map,
+                       const uint8_t* d_light_map, size_t env_stride, size_t level_stride,
+                       const uint8_t* d_skip, uint8_t* d_rec_row, int n, void* stream);
+/* k_record_obs_list (craftax_full.cu:9303-9320): records only the envs named by the
+ * first *d_count entries of a device index list; entry i is the int32 at d_env_list +
+ * i * list_stride bytes (a CraftaxResetRec array with its .env member: pass the address
+ * of the first .env and sizeof(CraftaxResetRec)).  max_count (<= n) bounds *d_count and
+ * sizes the launch; n is the env count the rows and arrays are laid out for. */
+int cfp_record_obs_soa_list(const cfp_env_soa* soa, const uint8_t* d_map,
+                            const uint8_t* d_item_map, const uint8_t* d_light_map,
+                            size_t env_stride, size_t level_stride, const void* d_env_list,
+                            size_t list_stride, const int* d_count, int max_count,
+                            uint8_t* d_rec_row, int n, void* stream);
+
 /* k_value_sample (craftax_full.cu:9714-9741) on the fused head's output
  * av[n][actions+1] (biases already added): values[e] = av[e][actions] (d_values
  * may be NULL), action ~ softmax(av[e][0..actions)) by inversion of the cumulative

@@ -217,3 +217,104 @@ def test_record_obs_live_fuzzed_states(pkg, cuda):
             assert mobs > 0, "the fuzzed states put no mob into view"
     finally:
         env.close()
+
+
+# ---- records straight from the reference's per-field device arrays ----------------------
+_SOA_DTYPES = {"player_health": np.float32, "light_level": np.float32, "is_sleeping": np.uint8,
+               "is_resting": np.uint8, "learned_spells": np.uint8, "mob_mask": np.uint8}
+_SLOT_CLASS = (0, 0, 0, 1, 1, 1, 2, 2, 3, 3, 3, 4, 4, 4)
+_CLASS_FIRST = (0, 3, 6, 8, 11)
+
+
+def _soa_from_scalars(pkg, sc, n_stride, seed):
+    """cfp_env_scalars rows -> the reference's layout (craftax_full.cu:620-712): one array
+    per field, [sub_index][env] with stride n_stride; the env's 14 mob slots go to level
+    jax_index(player_level, 9) of the 9-level mob arrays and its monsters_killed entry to
+    index player_level; every other entry holds random values the encoder must not read."""
+    n = sc.shape[0]
+    s32, f32 = sc.view(np.int32), sc.view(np.float32)
+    off = {f[0]: getattr(ob.EnvScalars, f[0]).offset // 4 for f in ob.EnvScalars._fields_}
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, k in pkg.policy.ENV_SOA_FIELDS:
+        dt = _SOA_DTYPES.get(name, np.int32)
+        if dt is np.float32:
+            out[name] = rng.random((k, n_stride)).astype(np.float32)
+        elif dt is np.uint8:
+            out[name] = rng.integers(0, 2, (k, n_stride)).astype(np.uint8)
+        else:
+            out[name] = rng.integers(-3, 60, (k, n_stride)).astype(np.int32)
+    level = s32[:, off["player_level"]]
+    mlevel = np.where(level < 0, level + 9, level).clip(0, 8)          # jax_index(level, 9)
+    env = np.arange(n)
+    rename = {"wood": "inv_wood", "stone": "inv_stone", "coal": "inv_coal", "iron": "inv_iron",
+              "diamond": "inv_diamond", "sapphire": "inv_sapphire", "ruby": "inv_ruby",
+              "sapling": "inv_sapling", "torches": "inv_torches", "arrows": "inv_arrows",
+              "books": "inv_books", "pickaxe": "inv_pickaxe", "sword": "inv_sword", "bow": "inv_bow",
+              "potions": "inv_potions", "armour": "inv_armour"}
+    for fname, ftype in ob.EnvScalars._fields_:
+        o = off[fname]
+        if fname in ("mob_type_id", "mob_mask", "mob_position", "monsters_killed_level"):
+            continue
+        name = rename.get(fname, fname)
+        k = dict(pkg.policy.ENV_SOA_FIELDS)[name]
+        src = f32 if _SOA_DTYPES.get(name) is np.float32 else s32
+        for i in range(k):
+            v = src[:, o + i]
+            out[name][i, :n] = (v != 0) if _SOA_DTYPES.get(name) is np.uint8 else v
+    out["monsters_killed"][level.clip(0, 8), env] = s32[:, off["monsters_killed_level"]]
+    for m in range(14):
+        c = _SLOT_CLASS[m]
+        cfm = (c * 9 + mlevel) * 3 + (m - _CLASS_FIRST[c])
+        out["mob_type_id"][cfm, env] = s32[:, off["mob_type_id"] + m]
+        out["mob_mask"][cfm, env] = s32[:, off["mob_mask"] + m] != 0
+        for a in range(2):
+            out["mob_position"][cfm * 2 + a, env] = s32[:, off["mob_position"] + 2 * m + a]
+    return out
+
+
+def test_record_obs_from_reference_soa_layout(pkg, cuda, golden):
+    """cfp_record_obs_soa on the fuzzed reference states scattered into the reference's
+    own device layout (field arrays [sub_index][env], 9-level mob arrays, stride > n):
+    the golden records bit for bit, the skip mask honoured, and the list form writing
+    exactly the listed rows."""
+    import torch
+    sc, pl, want = golden["fuzz_scalars"], golden["fuzz_planes"], golden["fuzz_records"]
+    n = sc.shape[0]
+    n_stride = n + 7
+    host = _soa_from_scalars(pkg, sc, n_stride, 11)
+    arrays = {k: _t(v, cuda) for k, v in host.items()}
+    planes = _t(pl, cuda).view(-1)
+    P3 = 3 * P
+    rec = pkg.policy.record_obs_soa(arrays, n_stride, planes, planes[P:], planes[2 * P:], n, P3, 0)
+    torch.cuda.synchronize()
+    got = rec.cpu().numpy()
+    bad = np.nonzero((got != want).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} of {n} records differ, first {bad[:5]}"
+    # skip mask: flagged rows stay as they were
+    skip = (np.arange(n) % 3 == 1).astype(np.uint8)
+    rec2 = torch.full((n, 996), 0xEE, dtype=torch.uint8, device=cuda)
+    pkg.policy.record_obs_soa(arrays, n_stride, planes, planes[P:], planes[2 * P:], n, P3, 0,
+                              skip=_t(skip, cuda), rec=rec2)
+    torch.cuda.synchronize()
+    got2 = rec2.cpu().numpy()
+    assert np.array_equal(got2[skip == 0], want[skip == 0])
+    assert np.all(got2[skip == 1] == 0xEE)
+    # list form: entries are the .env members of 12-byte structs; count < max_count
+    listed = np.nonzero(skip)[0][::-1].copy()
+    recs = np.full((n, 3), -1, np.int32)
+    recs[: listed.size, 1] = listed
+    d_list = _t(recs, cuda)
+    count = torch.tensor([listed.size], dtype=torch.int32, device=cuda)
+    pkg.policy.record_obs_soa_list(arrays, n_stride, planes, planes[P:], planes[2 * P:], n, P3, 0,
+                                   d_list.view(-1)[1:], 12, count, n, rec2)
+    torch.cuda.synchronize()
+    assert np.array_equal(rec2.cpu().numpy(), want)
+    # a one-env list and a launch far larger than the count
+    rec3 = torch.full((n, 996), 0xEE, dtype=torch.uint8, device=cuda)
+    one = torch.tensor([5], dtype=torch.int32, device=cuda)
+    pkg.policy.record_obs_soa_list(arrays, n_stride, planes, planes[P:], planes[2 * P:], n, P3, 0,
+                                   one, 4, torch.tensor([1], dtype=torch.int32, device=cuda), n, rec3)
+    torch.cuda.synchronize()
+    got3 = rec3.cpu().numpy()
+    assert np.array_equal(got3[5], want[5]) and np.all(np.delete(got3, 5, axis=0) == 0xEE)
