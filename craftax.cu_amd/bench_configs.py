@@ -28,6 +28,11 @@ PEAK_FP32 = 157.3                    # TFLOP/s, fp32 MFMA
 FWD_FLOP = 1633792                   # per env-step: encoder + 3 gate GEMMs + head
 UPD_FLOP = 4469248                   # per sample: recompute forward + backward
 CLASSIC_FLOP = 1179648 + 9216        # gate GEMMs + 18-row head (gather encoder not counted)
+# what the fp32 classic kernel issues per env: the above plus 3 K blocks of scalar features on the
+# fp32 pipe, and 83 K blocks of 16 cell features x 256 units x 3 bf16 terms on the bf16 pipe
+CLASSIC_ISSUE_FP32 = CLASSIC_FLOP + 24 * 256 * 2
+CLASSIC_ISSUE_BF16 = 83 * 16 * 256 * 2 * 3
+PEAK_BF16 = 2500.0
 
 
 def _time(torch, fn, reps, warm=2, warm_ms=80.0):
@@ -241,6 +246,9 @@ def classic_1m(pkg, torch, reps):
         out[name] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
                      "mfma_tflops": CLASSIC_FLOP * n / ms / 1e9,
                      "frac_fp32_mfma_peak": CLASSIC_FLOP * n / ms / 1e9 / PEAK_FP32}
+    bound_ms = (CLASSIC_ISSUE_FP32 / PEAK_FP32 + CLASSIC_ISSUE_BF16 / PEAK_BF16) * n / 1e9
+    out["fp32"]["mixed_pipe_bound_ms"] = bound_ms
+    out["fp32"]["frac_of_mixed_pipe_bound"] = bound_ms / out["fp32"]["ms_per_step"]
     pol.close()
     return out
 
