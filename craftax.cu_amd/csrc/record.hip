@@ -89,6 +89,7 @@ constexpr int kRecEnvsPerWg = 256 / kRecLanes;  // more gathers in flight than w
 // field laid out [sub_index][env], craftax_full.cu:613-723); the kernel asks for the words
 // of cfp_env_scalars it needs and a table says which array holds each.
 constexpr int kSoaPtrs = 40;
+constexpr int kSoaGather = 32;   // envs per gather round: one 128-byte line of an int32 field array (64 envs: slower)
 struct SoaArgs {
     const void* p[kSoaPtrs];   // the pointer fields of cfp_env_soa, in declaration order
     size_t n_stride;
@@ -161,10 +162,10 @@ constexpr int kWMobType = (int)(offsetof(cfp_env_scalars, mob_type_id) / 4);
 constexpr int kWMobMask = (int)(offsetof(cfp_env_scalars, mob_mask) / 4);
 constexpr int kWMobPos = (int)(offsetof(cfp_env_scalars, mob_position) / 4);
 
-// SOA: the env's scalars are first gathered into an LDS copy of cfp_env_scalars, transposed:
-// thread (word group gw, env ge) fetches words gw, gw + 16, ... of env ge, so the sixteen
-// lanes of a word read sixteen adjacent envs of one field array -- one 64-byte piece --
-// and all of a thread's seven elements are in flight together.  The rest of the kernel then
+// SOA: the scalars of 32 envs are first gathered into LDS copies of cfp_env_scalars,
+// transposed: thread (word group gw, env ge) fetches words gw, gw + 8, ... of env ge, so the
+// 32 lanes of a word read 32 adjacent envs of one field array -- one 128-byte line -- and
+// all of a thread's fourteen elements are in flight together.  The rest of the kernel then
 // reads that copy exactly as it reads a caller-staged struct.
 struct WordSrc {
     const uint32_t* w;
@@ -178,7 +179,9 @@ __global__ __launch_bounds__(256) void k_record_obs(
     const uint8_t* __restrict__ light_map, size_t env_stride,
     size_t level_stride, uint8_t* __restrict__ rec_row, int n) {
     __shared__ uint32_t stage_all[kRecEnvsPerWg][CFP_REC_BYTES / 4 + 3];
-    __shared__ uint32_t sc_all[SOA ? kRecEnvsPerWg : 1][kScalarWords + 1];
+    // SOA rounds take 32 envs: a 128-byte line of every field array is used by one workgroup
+    constexpr int kGather = SOA ? kSoaGather : kRecEnvsPerWg;
+    __shared__ uint32_t sc_all[SOA ? kGather : 1][kScalarWords + 1];
     __shared__ const void* ptrs[SOA ? kSoaPtrs : 1];
     __shared__ SoaWord words[SOA ? kScalarWords : 1];
     const int lane = threadIdx.x % kRecLanes;
@@ -191,11 +194,11 @@ __global__ __launch_bounds__(256) void k_record_obs(
     }
     const int total = which.list ? *which.count : n;
     // the trip count is the same for every thread of the workgroup (barriers inside)
-    for (int first = (int)blockIdx.x * kRecEnvsPerWg; first < total;
-         first += (int)gridDim.x * kRecEnvsPerWg) {
+    for (int first = (int)blockIdx.x * kGather; first < total; first += (int)gridDim.x * kGather) {
         if (SOA) {
             __syncthreads();   // tables filled; the previous round's readers are done with sc_all
-            const int ge = threadIdx.x % kRecEnvsPerWg, gw = threadIdx.x / kRecEnvsPerWg;
+            constexpr int kGroups = 256 / kGather;
+            const int ge = threadIdx.x % kGather, gw = threadIdx.x / kGather;
             const int gi = first + ge;
             int genv = gi;
             if (which.list && gi < total)
@@ -204,11 +207,11 @@ __global__ __launch_bounds__(256) void k_record_obs(
                 const int lvl = static_cast<const int32_t*>(ptrs[1])[genv];
                 const int lvl_c = lvl < 0 ? 0 : (lvl > 8 ? 8 : lvl);   // monsters_killed has nine entries
                 const int ml3 = 3 * jax_index(lvl, 9);
-                constexpr int kRounds = (kScalarWords + 15) / 16;
+                constexpr int kRounds = (kScalarWords + kGroups - 1) / kGroups;
                 uint32_t val[kRounds];
 #pragma unroll
                 for (int r = 0; r < kRounds; r++) {
-                    const int w = gw + 16 * r;
+                    const int w = gw + kGroups * r;
                     const SoaWord d = words[w < kScalarWords ? w : 0];
                     size_t sub = d.aux;
                     if (d.rule == R_LEVEL) sub = (size_t)lvl_c;
@@ -222,102 +225,104 @@ __global__ __launch_bounds__(256) void k_record_obs(
                 }
 #pragma unroll
                 for (int r = 0; r < kRounds; r++)
-                    if (gw + 16 * r < kScalarWords) sc_all[ge][gw + 16 * r] = val[r];
+                    if (gw + kGroups * r < kScalarWords) sc_all[ge][gw + kGroups * r] = val[r];
             }
             __syncthreads();
         }
-        const int item = first + slot;
-        if (item >= total) continue;
-        int env = item;
-        if (which.list)
-            env = *reinterpret_cast<const int32_t*>(which.list + (size_t)item * which.list_stride);
-        if (which.skip && which.skip[env]) continue;
-        uint32_t* stage = stage_all[slot];
-        WordSrc s;
-        s.w = SOA ? sc_all[slot] : reinterpret_cast<const uint32_t*>(scalars + env);
-        const int level = (int)s.word(kWLevel);
-        const int mlevel = jax_index(level, 9);
-        const int pr = (int)s.word(kWPos), pc = (int)s.word(kWPos + 1);
-        const size_t cell_plane = (size_t)env * env_stride + (size_t)level * level_stride;
-        const size_t mob_plane = (size_t)env * env_stride + (size_t)mlevel * level_stride;
+        for (int part = 0; part < kGather / kRecEnvsPerWg; part++) {
+            const int item = first + part * kRecEnvsPerWg + slot;
+            if (item >= total) continue;
+            int env = item;
+            if (which.list)
+                env = *reinterpret_cast<const int32_t*>(which.list + (size_t)item * which.list_stride);
+            if (which.skip && which.skip[env]) continue;
+            uint32_t* stage = stage_all[slot];
+            WordSrc s;
+            s.w = SOA ? sc_all[part * kRecEnvsPerWg + slot] : reinterpret_cast<const uint32_t*>(scalars + env);
+            const int level = (int)s.word(kWLevel);
+            const int mlevel = jax_index(level, 9);
+            const int pr = (int)s.word(kWPos), pc = (int)s.word(kWPos + 1);
+            const size_t cell_plane = (size_t)env * env_stride + (size_t)level * level_stride;
+            const size_t mob_plane = (size_t)env * env_stride + (size_t)mlevel * level_stride;
 
-        for (int cell = lane; cell < CELLS; cell += kRecLanes) {
-            const int row = cell / COLS, col = cell - row * COLS;
-            const int wr = pr - ROWS / 2 + row, wc = pc - COLS / 2 + col;
-            uint32_t lo = 0;
-            if (wr >= 0 && wr < MAP && wc >= 0 && wc < MAP) {
-                // all three planes requested at once (one memory round trip, not two)
-                const size_t o = cell_plane + (size_t)(wr * MAP + wc);
-                const uint32_t lv = light_map[o], bv = map[o], iv = item_map[o];
-                if (lv > 12) lo = bv | ((uint32_t)(uint8_t)(iv + 1) << 8) | (1u << 16);
+            for (int cell = lane; cell < CELLS; cell += kRecLanes) {
+                const int row = cell / COLS, col = cell - row * COLS;
+                const int wr = pr - ROWS / 2 + row, wc = pc - COLS / 2 + col;
+                uint32_t lo = 0;
+                if (wr >= 0 && wr < MAP && wc >= 0 && wc < MAP) {
+                    // all three planes requested at once (one memory round trip, not two)
+                    const size_t o = cell_plane + (size_t)(wr * MAP + wc);
+                    const uint32_t lv = light_map[o], bv = map[o], iv = item_map[o];
+                    if (lv > 12) lo = bv | ((uint32_t)(uint8_t)(iv + 1) << 8) | (1u << 16);
+                }
+                stage[2 * cell] = lo;
+                stage[2 * cell + 1] = 0u;
             }
-            stage[2 * cell] = lo;
-            stage[2 * cell + 1] = 0u;
-        }
 
-        // Mob slot m = lane contributes (cell, channel 3 + class, type + 1) when it passes
-        // the predicates of craftax_encode_mobs{3,2}_compact (craftax_full.c:2747-2825).
-        // Within a class the last slot on a cell wins: a slot stands back when one of the
-        // (at most two) later slots of its class sits on the same cell.
-        {
-            const int m = lane < CFP_MOB_SLOTS ? lane : CFP_MOB_SLOTS - 1;
-            const int type = (int)s.word(kWMobType + m);
-            const int mr = (int)s.word(kWMobPos + 2 * m), mc = (int)s.word(kWMobPos + 2 * m + 1);
-            const uint32_t mask = s.word(kWMobMask + m);
-            const int lr = mr - pr + ROWS / 2, lc = mc - pc + COLS / 2;
-            bool ok = lane < CFP_MOB_SLOTS && type >= 0 && type < 8 && mask != 0 &&
-                      lr >= 0 && lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
-                      mc >= 0 && mc < MAP;
-            if (ok) ok = light_map[mob_plane + (size_t)(mr * MAP + mc)] > 12;
-            const int cell = ok ? lr * COLS + lc : -1;
-            const int cls = kSlotClass[m];
-            bool over = false;
-#pragma unroll
-            for (int d = 1; d <= 2; d++) {
-                const int oc = __shfl_down(cell, d, kRecLanes);
-                const int ocls = __shfl_down(cls, d, kRecLanes);
-                over = over || (lane + d < CFP_MOB_SLOTS && ocls == cls && oc == cell);
+            // Mob slot m = lane contributes (cell, channel 3 + class, type + 1) when it passes
+            // the predicates of craftax_encode_mobs{3,2}_compact (craftax_full.c:2747-2825).
+            // Within a class the last slot on a cell wins: a slot stands back when one of the
+            // (at most two) later slots of its class sits on the same cell.
+            {
+                const int m = lane < CFP_MOB_SLOTS ? lane : CFP_MOB_SLOTS - 1;
+                const int type = (int)s.word(kWMobType + m);
+                const int mr = (int)s.word(kWMobPos + 2 * m), mc = (int)s.word(kWMobPos + 2 * m + 1);
+                const uint32_t mask = s.word(kWMobMask + m);
+                const int lr = mr - pr + ROWS / 2, lc = mc - pc + COLS / 2;
+                bool ok = lane < CFP_MOB_SLOTS && type >= 0 && type < 8 && mask != 0 &&
+                          lr >= 0 && lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
+                          mc >= 0 && mc < MAP;
+                if (ok) ok = light_map[mob_plane + (size_t)(mr * MAP + mc)] > 12;
+                const int cell = ok ? lr * COLS + lc : -1;
+                const int cls = kSlotClass[m];
+                bool over = false;
+    #pragma unroll
+                for (int d = 1; d <= 2; d++) {
+                    const int oc = __shfl_down(cell, d, kRecLanes);
+                    const int ocls = __shfl_down(cls, d, kRecLanes);
+                    over = over || (lane + d < CFP_MOB_SLOTS && ocls == cls && oc == cell);
+                }
+                if (ok && !over)
+                    reinterpret_cast<uint8_t*>(stage)[cell * 8 + 3 + cls] = (uint8_t)(type + 1);
             }
-            if (ok && !over)
-                reinterpret_cast<uint8_t*>(stage)[cell * 8 + 3 + cls] = (uint8_t)(type + 1);
-        }
 
-        for (int tj = lane; tj < CFP_OBS_TAIL; tj += kRecLanes) {
-            const TailSpec ts = kTail[tj];
-            const int iv = (int)s.word(ts.field);
-            const float fv = __int_as_float(iv);
-            const float xi = (float)iv;
-            float v = 0.0f;
-            switch (ts.kind) {
-                // IEEE sqrt: HIP's __fsqrt_rn is the approximate native sqrt unless
-                // OCML_BASIC_ROUNDED_OPERATIONS is defined; the fp64 root rounded
-                // to fp32 is the correctly rounded fp32 root (53 >= 2*24 + 2).
-                case T_SQRT10: v = (float)sqrt((double)xi) * 0.1f; break;
-                case T_HALF: v = xi * 0.5f; break;
-                case T_QUARTER: v = xi * 0.25f; break;
-                case T_INT: v = xi; break;
-                case T_F10: v = fv * 0.1f; break;
-                case T_I10: v = xi * 0.1f; break;
-                case T_DIR: v = (iv - 1 == (int)ts.aux) ? 1.0f : 0.0f; break;
-                case T_FLOAT: v = fv; break;
-                case T_BOOL: v = iv != 0 ? 1.0f : 0.0f; break;
-                case T_KILLED: v = iv >= 8 ? 1.0f : 0.0f; break;
-                case T_BOSS: {
-                    // craftax_wg_is_boss_vulnerable, craftax_full.c:2205: no live
-                    // melee (slots 0..2) or ranged (slots 6..7) mob, spawn timer <= 0
-                    bool any = false;
-                    for (int m = 0; m < 3; m++) any = any || s.word(kWMobMask + m) != 0;
-                    for (int m = 6; m < 8; m++) any = any || s.word(kWMobMask + m) != 0;
-                    v = (!any && (int)s.word(kWBossTimer) <= 0) ? 1.0f : 0.0f;
-                } break;
+            for (int tj = lane; tj < CFP_OBS_TAIL; tj += kRecLanes) {
+                const TailSpec ts = kTail[tj];
+                const int iv = (int)s.word(ts.field);
+                const float fv = __int_as_float(iv);
+                const float xi = (float)iv;
+                float v = 0.0f;
+                switch (ts.kind) {
+                    // IEEE sqrt: HIP's __fsqrt_rn is the approximate native sqrt unless
+                    // OCML_BASIC_ROUNDED_OPERATIONS is defined; the fp64 root rounded
+                    // to fp32 is the correctly rounded fp32 root (53 >= 2*24 + 2).
+                    case T_SQRT10: v = (float)sqrt((double)xi) * 0.1f; break;
+                    case T_HALF: v = xi * 0.5f; break;
+                    case T_QUARTER: v = xi * 0.25f; break;
+                    case T_INT: v = xi; break;
+                    case T_F10: v = fv * 0.1f; break;
+                    case T_I10: v = xi * 0.1f; break;
+                    case T_DIR: v = (iv - 1 == (int)ts.aux) ? 1.0f : 0.0f; break;
+                    case T_FLOAT: v = fv; break;
+                    case T_BOOL: v = iv != 0 ? 1.0f : 0.0f; break;
+                    case T_KILLED: v = iv >= 8 ? 1.0f : 0.0f; break;
+                    case T_BOSS: {
+                        // craftax_wg_is_boss_vulnerable, craftax_full.c:2205: no live
+                        // melee (slots 0..2) or ranged (slots 6..7) mob, spawn timer <= 0
+                        bool any = false;
+                        for (int m = 0; m < 3; m++) any = any || s.word(kWMobMask + m) != 0;
+                        for (int m = 6; m < 8; m++) any = any || s.word(kWMobMask + m) != 0;
+                        v = (!any && (int)s.word(kWBossTimer) <= 0) ? 1.0f : 0.0f;
+                    } break;
+                }
+                stage[CFP_OBS_MAP / 4 + tj] = __float_as_uint(v);
             }
-            stage[CFP_OBS_MAP / 4 + tj] = __float_as_uint(v);
-        }
 
-        __builtin_amdgcn_wave_barrier();
-        uint32_t* out = reinterpret_cast<uint32_t*>(rec_row + (size_t)env * CFP_REC_BYTES);
-        for (int d = lane; d < CFP_REC_BYTES / 4; d += kRecLanes) out[d] = stage[d];
-        __builtin_amdgcn_wave_barrier();   // the staging row is reused by the next item
+            __builtin_amdgcn_wave_barrier();
+            uint32_t* out = reinterpret_cast<uint32_t*>(rec_row + (size_t)env * CFP_REC_BYTES);
+            for (int d = lane; d < CFP_REC_BYTES / 4; d += kRecLanes) out[d] = stage[d];
+            __builtin_amdgcn_wave_barrier();   // the staging row is reused by the next item
+        }
     }
 }
 
@@ -521,7 +526,7 @@ static int record_obs_soa(const cfp_env_soa* soa, const uint8_t* d_map, const ui
     std::memcpy(&a, soa, sizeof(a));
     for (int i = 0; i < kSoaPtrs; i++)
         CFP_REQUIRE(a.p[i] != nullptr, "cfp_record_obs_soa: field array %d of the view is NULL", i);
-    hipLaunchKernelGGL(k_record_obs<true>, dim3((items + kRecEnvsPerWg - 1) / kRecEnvsPerWg),
+    hipLaunchKernelGGL(k_record_obs<true>, dim3((items + kSoaGather - 1) / kSoaGather),
                        dim3(256), 0, (hipStream_t)stream, nullptr, a, which, d_map, d_item_map,
                        d_light_map, env_stride, level_stride, d_rec_row, n);
     CFP_HIP_TRY(hipGetLastError());
