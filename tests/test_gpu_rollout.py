@@ -203,3 +203,55 @@ def test_reference_weight_init(pkg, cuda, classic):
     torch.cuda.synchronize()
     assert torch.isfinite(av).all()
     pol.close()
+
+
+@pytest.mark.parametrize("n,small", [(256, False), (512, True)])
+def test_rollout_round_replays_from_a_graph(pkg, cuda, n, small):
+    """A round of rollout steps captured once and replayed (the reference captures its
+    rollout the same way): the step counter lives in device memory and is bumped inside
+    the launch that draws, so every replay must continue the eager twin's stream of
+    draws -- same actions, log-probabilities, values, state and counter after each
+    replay, with eager work and synchronisations in between."""
+    import torch
+    T, seed = 3, 99
+    params = random_params(L, 31, scale=0.5)
+    twins = []
+    for _ in range(2):
+        pol = pkg.Policy(n, L, seed=1)
+        pol.set_params(params)
+        pol.set_small_tiles(small)
+        pol.state.zero_()
+        twins.append((pol, pkg.Trainer(pol, T)))
+    (pol_e, tr_e), (pol_g, tr_g) = twins
+    recs = [_t(synth_records_host(n, 7, t), cuda) for t in range(T)]
+    term = _t((np.random.default_rng(3).random(n) < 0.2).astype(np.float32), cuda)
+    acts = [torch.zeros(n, device=cuda) for _ in range(2)]
+
+    def round_(tr, a):
+        for t in range(T):
+            tr.rollout_step(t, recs[t], term, seed, env_actions=a)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            round_(tr_g, acts[1])
+    torch.cuda.synchronize()
+    for i in range(3):
+        round_(tr_e, acts[0])
+        with torch.cuda.stream(side):
+            graph.replay()
+        torch.cuda.synchronize()
+        junk = torch.randn(1 << 16, device=cuda).sum().item()   # eager work between replays
+        assert np.isfinite(junk)
+        assert int(tr_g.buf("step_ctr").cpu()[0]) == (i + 1) * T == int(tr_e.buf("step_ctr").cpu()[0])
+        for name in ("r_act", "r_logprob", "r_value", "r_state"):
+            assert torch.equal(tr_e.buf(name), tr_g.buf(name)), f"replay {i}: {name}"
+        assert torch.equal(pol_e.state, pol_g.state) and torch.equal(acts[0], acts[1])
+    # successive rounds drew from different offsets of the stream
+    first = tr_e.buf("r_act").clone()
+    round_(tr_e, acts[0]); torch.cuda.synchronize()
+    assert not torch.equal(first, tr_e.buf("r_act"))
+    for pol, tr in twins:
+        tr.close(); pol.close()
