@@ -59,7 +59,10 @@ def _collect(pkg, cuda, n, T, seed, done_p, scale=0.3, **cfg):
 
 
 @pytest.mark.parametrize("n,T,minibatches,bptt_split,bwd_win,done_p",
-                         [(64, 8, 1, 1, 0, 0.1), (64, 8, 2, 2, 3, 0.15), (32, 6, 1, 3, 1, 0.0)])
+                         [(64, 8, 1, 1, 0, 0.1), (64, 8, 2, 2, 3, 0.15), (32, 6, 1, 3, 1, 0.0),
+                          # window lengths 7, 4 and 5: every remainder of the reverse sweep's
+                          # three-step rounds after at least one full round
+                          (32, 7, 1, 1, 0, 0.2), (32, 8, 1, 2, 4, 0.1), (32, 5, 1, 1, 0, 0.1)])
 def test_backward_matches_oracle(pkg, cuda, n, T, minibatches, bptt_split, bwd_win, done_p):
     import torch
     params, pol, tr, host = _collect(pkg, cuda, n, T, 50 + n + T, done_p,
