@@ -477,6 +477,7 @@ int forward_and_sample(cfp_policy* p, const uint8_t* d_rec_row, const float* d_t
     f.s_step = s.step_ctr;
     f.s_ticket = s.ticket;
     if (forward_t16_ok(f)) return launch_forward_t16(f, st);
+    if (forward_draws(f)) return launch_forward(f, st);
     if (run_chunked(a, n, 0, st) != 0) return 1;
     const bool ride = n < kSampleRowsFrom;   // the sampler's launch bumps the counter itself
     if (value_sample(p->logits, n, a.actions, s.env_actions, s.act, s.logp, s.value, s.seed,

@@ -40,6 +40,10 @@ int value_sample(const float* d_av, int n, int actions, float* d_env_actions, in
                  float* d_logprobs, float* d_values, uint64_t seed, const uint64_t* d_step_ctr,
                  unsigned* ticket, hipStream_t st);
 
+// launch_forward also draws the actions (FwdArgs::s_act ...) when this holds: full-game
+// records in recording mode on 32-env tiles, one tile per workgroup (at most one per CU).
+bool forward_draws(const FwdArgs& a);
+
 // One rollout step's policy side for the trainer: records -> heads into the policy's
 // live state and logits (r_state recorded), then the draw into act / logp / value
 // (and env_actions when not null) with offset *step_ctr, then *step_ctr += 1.  One

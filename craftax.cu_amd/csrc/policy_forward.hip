@@ -48,6 +48,8 @@
 //   heads:   2 row tiles x 2 K halves over the 4 waves, each weight fragment used for
 //            both tiles, partial sums reduced through LDS.
 #include "policy_tile.h"
+#include "cfp_internal.h"
+#include "sample_row.h"
 
 namespace cfp {
 
@@ -696,10 +698,42 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
                         float* av_base = a.av_out + e0[s] * avs;
                         const int aoff = (4 * L.half) * avs + arow;
 #pragma unroll
-                        for (int r = 0; r < 16; r++)
-                            (av_base + acc_row(r) * avs)[aoff] = hacc[s][r] + red[r * 64] + bias;
+                        for (int r = 0; r < 16; r++) {
+                            const float v = hacc[s][r] + red[r * 64] + bias;
+                            (av_base + acc_row(r) * avs)[aoff] = v;
+                            // rollout step in one launch: the rows stay in LDS for the draw
+                            // (the x tiles are free: every wave is past its head MFMAs)
+                            if (SINGLE && MODE == kModeRecord && a.s_act)
+                                lds_all[0][(acc_row(r) + 4 * L.half) * avs + arow] = v;
+                        }
                     }
                 }
+            }
+            // ---- the draw behind the heads (one tile per workgroup, recording mode): sixteen
+            // lanes per env run the sampler's code (sample_row.h: same operations in the same
+            // order as k_value_sample), lanes 0 and 1 of a group each finish one of the tile's
+            // two halves, and the last workgroup bumps the step counter
+            if (SINGLE && MODE == kModeRecord && a.s_act) {   // uniform over the launch
+                __syncthreads();
+                const int sub = tid % kSampleLanes, grp = tid / kSampleLanes;   // 16 groups
+                const int avs = a.actions + 1;
+                float mx[2];
+#pragma unroll
+                for (int part = 0; part < 2; part++) {
+                    const int env = grp + 16 * part;
+                    mx[part] = sample_spread(lds_all[0] + env * avs, lds_all[1] + env * kMaxActions,
+                                             a.actions, sub, true);
+                }
+                __syncthreads();
+                if (sub < 2) {
+                    const int env = grp + 16 * sub;
+                    sample_draw<CFP_ACTIONS>(lds_all[0] + env * avs, lds_all[1] + env * kMaxActions,
+                                             sub == 0 ? mx[0] : mx[1], a.actions, (int)e0[0] + env,
+                                             a.s_seed, *a.s_step, a.s_env_actions, a.s_act, a.s_logp,
+                                             a.s_value);
+                }
+                __syncthreads();
+                if (tid == 0) bump_by_last_group(a.s_ticket, a.s_step, gridDim.x);
             }
         }
         __syncthreads();   // LDS tiles and partials are free for the next pair
@@ -718,6 +752,14 @@ static int num_cus() {
             cus = 256;
     }
     return cus;
+}
+
+// Does launch_forward run the instantiation that also draws the actions (FwdArgs::s_act)?
+bool forward_draws(const FwdArgs& a) {
+    const int tiles = a.n / kTileEnvs;
+    return a.s_act && a.s_logp && a.s_step && a.s_ticket && a.variant == 0 && !a.train &&
+           !a.bf16 && a.rec && a.r_state && a.do_head && a.layers > 0 && a.n % kTileEnvs == 0 &&
+           tiles > 1 && tiles <= num_cus();
 }
 
 int launch_forward(const FwdArgs& a, hipStream_t st) {
@@ -752,6 +794,8 @@ int launch_forward(const FwdArgs& a, hipStream_t st) {
     const int grid = pairs < num_cus() ? pairs : num_cus();
     const dim3 g(grid), b(kFwdThreads);
     const bool single = a.variant == 0 && !a.train && tiles <= num_cus() && tiles > 1;
+    CFP_REQUIRE(!a.s_act || forward_draws(a),
+                "the draw behind the heads needs full-game records, r_state and one tile per CU");
     if (a.train) {
         CFP_REQUIRE(a.variant == 0 && a.rec && a.state && a.layers > 0 && !a.r_state &&
                         a.tr_mb > 0 && a.tr_mb % kTileEnvs == 0 && a.h_enc_out == a.tr_x[0],

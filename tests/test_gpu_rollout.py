@@ -118,13 +118,16 @@ def test_record_rd(pkg, cuda):
     assert np.array_equal(r_done.cpu().numpy(), (term != 0).astype(np.uint8))
 
 
-@pytest.mark.parametrize("n,small", [(256, False), (256, True), (4096, True), (16416, False)])
+@pytest.mark.parametrize("n,small", [(256, False), (8192, False), (256, True), (4096, True),
+                                     (8224, False), (16416, False)])
 def test_rollout_step_and_bootstrap(pkg, cuda, n, small):
     """cfp_rollout_step == forward on the live state + sampling with the device step
     counter, written into the slab rows; cfp_train_bootstrap values the next
-    records on a copy of the live state.  The cases cover the three forms of the step:
-    forward + sampler that bumps the counter in its own launch (256), the 16-env-tile
-    kernel that also draws and bumps (small), forward + row sampler + bump (16 416)."""
+    records on a copy of the live state.  The cases cover the four forms of the step:
+    one launch on 32-env tiles, one per workgroup, that also draws and bumps (256 and
+    8192 envs: at most one tile per CU), the same on 16-env tiles (small), forward +
+    sampler that bumps the counter in its own launch (8224 envs = 257 tiles), forward +
+    row sampler + bump kernel (16 416)."""
     import torch
     T, seed = 4, 4321
     params = random_params(L, 21, scale=0.5)
