@@ -449,6 +449,10 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
     uint8_t* const cbase = reinterpret_cast<uint8_t*>(&lds_all[0][0]);
     uint8_t* const crec_all[2] = {cbase, cbase + kClsOffRecY};
 
+    // rollout step in one launch: the draw's offset, requested before anything else (older
+    // than every weight request, so no wait of the ring protocol depends on it)
+    uint64_t draw_step = 0;
+    if (SINGLE && MODE == kModeRecord && a.s_act) draw_step = *a.s_step;
     const int tiles = a.n / kTileEnvs;
     constexpr int TS = SINGLE ? 1 : 2;   // tiles per unit of work ("pair")
     const int pairs = (tiles + TS - 1) / TS;
@@ -729,7 +733,7 @@ __global__ __launch_bounds__(kFwdThreads, 1) void k_policy_forward(FwdArgs a) {
                     const int env = grp + 16 * sub;
                     sample_draw<CFP_ACTIONS>(lds_all[0] + env * avs, lds_all[1] + env * kMaxActions,
                                              sub == 0 ? mx[0] : mx[1], a.actions, (int)e0[0] + env,
-                                             a.s_seed, *a.s_step, a.s_env_actions, a.s_act, a.s_logp,
+                                             a.s_seed, draw_step, a.s_env_actions, a.s_act, a.s_logp,
                                              a.s_value);
                 }
                 __syncthreads();

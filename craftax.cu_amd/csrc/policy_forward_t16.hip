@@ -190,6 +190,8 @@ __global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a
         for (int e = 0; e < 8; e++)
             v[e] = __builtin_nontemporal_load((base + ((e & 3) * CFP_HIDDEN + (e >> 2) * 16)) + soff);
     };
+    // the draw's offset (rollout step in one launch), requested before anything else
+    const uint64_t draw_step = a.s_act ? *a.s_step : 0;
     // Every layer's state first: it travels beside the records, is older than every weight
     // request (requests return in order: a state load issued later would hold the weight
     // stream up behind its HBM latency) and has long landed when its epilogue comes.
@@ -419,7 +421,7 @@ __global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a
         const float mx = sample_spread(lp, px, CFP_ACTIONS, sub, live);
         __syncthreads();
         if (live && sub == 0)
-            sample_draw<CFP_ACTIONS>(lp, px, mx, CFP_ACTIONS, (int)e0 + slot, a.s_seed, *a.s_step,
+            sample_draw<CFP_ACTIONS>(lp, px, mx, CFP_ACTIONS, (int)e0 + slot, a.s_seed, draw_step,
                         a.s_env_actions, a.s_act, a.s_logp, a.s_value);
         __syncthreads();
         if (tid == 0) bump_by_last_group(a.s_ticket, a.s_step, gridDim.x);

@@ -27,13 +27,14 @@ __device__ __forceinline__ float sample_spread(const float* lp, float* px, int a
     return m;
 }
 
-// Order-dependent part, run by one lane of the env: the two sums in ascending action
-// order, the uniform of (seed, env, step), the first action whose cumulative sum
-// reaches the target (the last action as the fall-through), and the outputs.
-// ACTIONS > 0 fixes the action count at compile time: both loops unroll, the
-// exponentials are read from LDS once, in one batch, and what is left in sequence is
-// the two chains of additions.  The scan carries no early exit (a flag keeps the
-// first hit), which changes no result: the sums past the hit are not used.
+// Order-dependent part, run by one lane of the env: the sum of the exponentials in
+// ascending action order, the uniform of (seed, env, step), the first action whose
+// cumulative sum reaches the target (the last action as the fall-through), and the outputs.
+// The reference adds the exponentials up twice in the same order (once for the total, once
+// for the scan: cf_nn_sample_action, craftax_full.cu:9147-9165), so the scan's cumulative sums
+// are the partial sums of the total.  ACTIONS > 0 fixes the action count at compile time:
+// the partial sums are then kept (one chain of additions instead of two, the exponentials
+// read from LDS once, in one batch) and the scan is 43 independent comparisons.
 template <int ACTIONS = 0>
 __device__ __forceinline__ void sample_draw(const float* lp, const float* px, float m, int actions,
                                             int e, uint64_t seed, uint64_t step,
@@ -45,18 +46,25 @@ __device__ __forceinline__ void sample_draw(const float* lp, const float* px, fl
     if (values) values[e] = lp[na];
     const float u = philox_uniform(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)e, step);
     float total = 0.0f;
-#pragma unroll
-    for (int a = 0; a < na; a++) total += px[a];
-    const float target = u * total;
-    float cum = 0.0f;
     int action = na - 1;
-    bool open = true;
+    if (ACTIONS > 0) {
+        float cum[ACTIONS > 0 ? ACTIONS : 1];
 #pragma unroll
-    for (int a = 0; a < na; a++) {
-        cum += px[a];
-        if (open && target <= cum) {
-            action = a;
-            open = false;
+        for (int a = 0; a < ACTIONS; a++) {
+            total += px[a];
+            cum[a] = total;
+        }
+        const float target = u * total;
+#pragma unroll
+        for (int a = ACTIONS - 1; a >= 0; a--)
+            if (target <= cum[a]) action = a;   // descending: the smallest hit is kept
+    } else {
+        for (int a = 0; a < na; a++) total += px[a];
+        const float target = u * total;
+        float cum = 0.0f;
+        for (int a = 0; a < na; a++) {
+            cum += px[a];
+            if (target <= cum) { action = a; break; }
         }
     }
     if (env_actions) env_actions[e] = (float)action;
