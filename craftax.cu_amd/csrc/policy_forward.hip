@@ -188,6 +188,8 @@ __device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const 
     ring_preload(ring, wp, L);
     EncDw cur = encs_bytes(rx, ry, 0, L.half);
     EncS bl[2];
+    // block 0 landed: the preload's blocks 1 and 2 (6 requests each) are the only younger
+    // operations -- the tail fragments above were requested before the preload
     vm_wait(12);
 #pragma unroll
     for (int i = 0; i < 6; i++)
@@ -200,6 +202,8 @@ __device__ __forceinline__ void encoder_gemm_split_ring(const FwdArgs& a, const 
                      __uint_as_float(bl[cb].b[5].w));
         EncDw nxt = cur;
         if (kb + 1 < kKb16Split) {
+            // block kb+1 landed; younger: blocks kb+2 and kb+3 (12), near the end the one
+            // block still to come (6) or nothing -- the loop issues no other vector memory
             vm_wait(kb + 3 < kKb16Split ? 12 : (kb + 2 < kKb16Split ? 6 : 0));
             const f4* slot = ring + ((kb + 1) % kRingSlots) * kRingSlotF4 + L.lane_u;
 #pragma unroll
@@ -277,7 +281,7 @@ __device__ __forceinline__ void classic_encoder_gemm(const FwdArgs& a, const uin
     mx = bx[2];
     my = by[2];
     EncS bl[2];
-    vm_wait(12);
+    vm_wait(12);   // block 0 landed; younger: the preload's blocks 1 and 2
 #pragma unroll
     for (int i = 0; i < 6; i++) bl[0].b[i] = __builtin_bit_cast(u4, ring[i * 64 + L.lane_u]);
 #pragma unroll
@@ -288,6 +292,7 @@ __device__ __forceinline__ void classic_encoder_gemm(const FwdArgs& a, const uin
                      __uint_as_float(bl[cb].b[5].w));
         u4 nx = ax, ny = ay;
         if (kb + 1 < kClsKb16) {
+            // block kb+1 landed; younger: the blocks requested since (12, 6 or none)
             vm_wait(kb + 3 < kClsKb16 ? 12 : (kb + 2 < kClsKb16 ? 6 : 0));
             const f4* slot = ring + ((kb + 1) % kRingSlots) * kRingSlotF4 + L.lane_u;
 #pragma unroll
