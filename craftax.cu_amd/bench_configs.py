@@ -352,6 +352,19 @@ def stream_ceilings(pkg, torch, reps):
                             ("add_2r_1w", lambda: torch.add(a, b, out=c), 3 * gib)):
         ms = _time(torch, fn, reps)
         out[name] = {"ms": ms, "tb_per_s": moved / ms / 1e9}
+    del a, b, c
+    # one of this library's own streaming kernels at a size far beyond the last-level cache:
+    # the unfused MinGRU epilogue (5 rows read, 3 written per env and layer) at 262 144 envs
+    n_env = 262144
+    pre = torch.randn(n_env, 768, device="cuda")
+    xin = torch.randn(n_env, 256, device="cuda")
+    state = torch.randn(n_env, 256, device="cuda") * 0.5
+    rs = torch.empty(n_env, 256, device="cuda")
+    hout = torch.empty(n_env, 256, device="cuda")
+    term = torch.zeros(n_env, device="cuda")
+    ms = _time(torch, lambda: pkg.policy.mingru_epi_fwd(pre, xin, state, term, r_state_store=rs,
+                                                        h_out=hout), reps)
+    out["mingru_epi_fwd_5r_3w_262144_envs"] = {"ms": ms, "tb_per_s": 8196 * n_env / ms / 1e9}
     return out
 
 
