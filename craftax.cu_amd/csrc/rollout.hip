@@ -68,6 +68,10 @@ __global__ __launch_bounds__(256) void k_value_sample(
 // replace the logits in the row.  Same operations in the same order: same bits.
 constexpr int kSampleRowEnvs = 128;
 
+// ACTIONS > 0 fixes the action count at compile time: the row is read from LDS once into
+// registers, and the partial sums of the total serve as the scan's cumulative sums (the
+// reference adds the same terms up in the same order twice).
+template <int ACTIONS>
 __global__ __launch_bounds__(kSampleRowEnvs) void k_value_sample_rows(
     const float* __restrict__ av, int avs, int actions, float* __restrict__ env_actions,
     int32_t* __restrict__ act, float* __restrict__ logprobs, float* __restrict__ values, int n,
@@ -89,26 +93,49 @@ __global__ __launch_bounds__(kSampleRowEnvs) void k_value_sample_rows(
     if (e >= n) return;
     float* lp = rows + threadIdx.x * stride;
     if (values) values[e] = lp[actions];
-    float m = lp[0];
-    for (int a = 1; a < actions; a++) m = fmaxf(m, lp[a]);
-    float total = 0.0f;
-    for (int a = 0; a < actions; a++) {
-        const float p = expf(lp[a] - m);
-        lp[a] = p;
-        total += p;
-    }
     const uint64_t step = step_ctr ? *step_ctr : 0;
     const float u = philox_uniform(seed ^ 0xA5A5A5A5A5A5A5A5ULL, (uint64_t)e, step);
-    const float target = u * total;
-    float cum = 0.0f;
+    float m, total = 0.0f, chosen;
     int action = actions - 1;
-    for (int a = 0; a < actions; a++) {
-        cum += lp[a];
-        if (target <= cum) { action = a; break; }
+    if (ACTIONS > 0) {
+        float z[ACTIONS > 0 ? ACTIONS : 1], cum[ACTIONS > 0 ? ACTIONS : 1];
+#pragma unroll
+        for (int a = 0; a < ACTIONS; a++) z[a] = lp[a];
+        m = z[0];
+#pragma unroll
+        for (int a = 1; a < ACTIONS; a++) m = fmaxf(m, z[a]);
+#pragma unroll
+        for (int a = 0; a < ACTIONS; a++) {
+            total += expf(z[a] - m);
+            cum[a] = total;
+        }
+        const float target = u * total;
+        chosen = z[ACTIONS - 1];
+#pragma unroll
+        for (int a = ACTIONS - 1; a >= 0; a--)
+            if (target <= cum[a]) {   // descending: the smallest hit is kept
+                action = a;
+                chosen = z[a];
+            }
+    } else {
+        m = lp[0];
+        for (int a = 1; a < actions; a++) m = fmaxf(m, lp[a]);
+        for (int a = 0; a < actions; a++) {
+            const float p = expf(lp[a] - m);
+            lp[a] = p;
+            total += p;
+        }
+        const float target = u * total;
+        float cum = 0.0f;
+        for (int a = 0; a < actions; a++) {
+            cum += lp[a];
+            if (target <= cum) { action = a; break; }
+        }
+        chosen = av[(size_t)e * avs + action];
     }
     if (env_actions) env_actions[e] = (float)action;
     act[e] = action;
-    logprobs[e] = av[(size_t)e * avs + action] - m - logf(total);
+    logprobs[e] = chosen - m - logf(total);
 }
 
 __global__ void k_record_rd(const float* __restrict__ rewards, const float* __restrict__ terminals,
@@ -133,8 +160,13 @@ int value_sample(const float* d_av, int n, int actions, float* d_env_actions, in
     CFP_REQUIRE(!ticket || (d_step_ctr && n < kSampleRowsFrom),
                 "value_sample: the in-launch counter bump covers batches below %d envs",
                 kSampleRowsFrom);
-    if (n >= kSampleRowsFrom)
-        hipLaunchKernelGGL(k_value_sample_rows, dim3((n + kSampleRowEnvs - 1) / kSampleRowEnvs),
+    if (n >= kSampleRowsFrom && actions == CFP_ACTIONS)
+        hipLaunchKernelGGL(k_value_sample_rows<CFP_ACTIONS>,
+                           dim3((n + kSampleRowEnvs - 1) / kSampleRowEnvs), dim3(kSampleRowEnvs), 0,
+                           st, d_av, actions + 1, actions, d_env_actions, d_actions, d_logprobs,
+                           d_values, n, seed, d_step_ctr);
+    else if (n >= kSampleRowsFrom)
+        hipLaunchKernelGGL(k_value_sample_rows<0>, dim3((n + kSampleRowEnvs - 1) / kSampleRowEnvs),
                            dim3(kSampleRowEnvs), 0, st, d_av, actions + 1, actions, d_env_actions,
                            d_actions, d_logprobs, d_values, n, seed, d_step_ctr);
     else
