@@ -134,6 +134,19 @@ def cpu_baseline(params, seed):
            "sample": f"{n} envs x {steps} steps of the same forward (oracle/policy_ref.c "
                      f"cfo_forward_f32, OpenMP, {dt:.1f} s)",
            "gflops": FLOP_PER_ENV_STEP * n * steps / dt / 1e9}
+    # the record encoder's CPU restatement (state -> 996-byte record, one thread), on the
+    # fuzzed reference states of tests/golden tiled to 65 536 envs
+    try:
+        g = np.load(os.path.join(ROOT, "tests", "golden", "record_fixtures.npz"))
+        idx = np.arange(65536) % g["fuzz_scalars"].shape[0]
+        sc, pl = g["fuzz_scalars"][idx], g["fuzz_planes"][idx]
+        m, it, li = (np.ascontiguousarray(pl[:, k]) for k in range(3))
+        ob.encode_compact(sc[:256], m[:256], it[:256], li[:256])
+        t0 = time.perf_counter()
+        ob.encode_compact(sc, m, it, li)
+        out["record_encode_envs_per_s_1_thread"] = 65536 / (time.perf_counter() - t0)
+    except OSError:
+        pass
     if ob.have_ref():
         # the reference's own CPU env (random actions), for orientation only: a
         # different path (env step, not policy forward)
