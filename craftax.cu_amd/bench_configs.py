@@ -205,6 +205,11 @@ def rollout_policy_side(pkg, torch, reps):
         ms = _time(torch, round_, max(2, reps // 2), warm=1) / T
         out["sizes"][str(n)] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
                                 "frac_fp32_mfma_peak": FWD_FLOP * n / ms / 1e9 / PEAK_FP32}
+        # the same round with the bf16-input forward kernel (cfp_policy_set_gemm_bf16)
+        pol.set_gemm_bf16(True)
+        ms_b = _time(torch, round_, max(2, reps // 2), warm=1) / T
+        pol.set_gemm_bf16(False)
+        out["sizes"][str(n)]["bf16_in"] = {"ms_per_step": ms_b, "env_steps_per_s": n / ms_b * 1e3}
         if n <= 8192:
             # 16-env tiles (opt-in): twice the CUs at work at these sizes
             pol.set_small_tiles(True)
