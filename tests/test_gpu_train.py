@@ -233,6 +233,46 @@ def test_config4_shape_properties(pkg, cuda):
     tr.close(); pol.close()
 
 
+def test_config4_shape_bf16_storage_properties(pkg, cuda):
+    """bf16 GEMM inputs with bf16 storage of the window workspace at the full size of the
+    PPO-update config (4096 envs x 64 steps, one 262 144-column window): finite, the same
+    bits twice, and every gradient segment within the bf16 tolerance (relative Frobenius
+    norm) of the same update with fp32 storage."""
+    import torch
+    from parity_util import TOL_BF16, fro_err
+    n, T = 4096, 64
+    pol = pkg.Policy(n, L, seed=1)
+    tr = pkg.Trainer(pol, T)
+    term0 = torch.zeros(n, device=cuda)
+    for t in range(T):
+        tr.record_step(t, pkg.policy.synth_records(n, 5, t), term0)
+    g = torch.Generator(device="cpu").manual_seed(1)
+    tr.buf("r_act").copy_(torch.randint(0, ACTIONS, (T, n), generator=g, dtype=torch.int32).to(cuda))
+    tr.buf("r_logprob").fill_(float(-np.log(ACTIONS)))
+    tr.buf("adv").copy_(torch.randn(T, n, generator=g).to(cuda))
+    tr.buf("ret").copy_(torch.randn(T, n, generator=g).to(cuda))
+    tr.adv_stats()
+    pkg.policy.set_gemm_bf16(True)
+    try:
+        grads = {}
+        for store16 in (False, True):
+            tr.set_bf16_storage(store16)
+            runs = []
+            for _ in range(2):
+                tr.buf("grads").zero_(); tr.backward(0, n); torch.cuda.synchronize()
+                runs.append(tr.buf("grads").clone())
+            assert torch.isfinite(runs[0]).all()
+            assert torch.equal(runs[0], runs[1]), f"bf16 storage {store16}: not reproducible"
+            grads[store16] = runs[0].cpu().numpy()
+        for name, sl in _segments(L):
+            e = fro_err(grads[True][sl], grads[False][sl])
+            assert e <= TOL_BF16, f"d{name}: bf16 vs fp32 storage, relative Frobenius error {e:.3e}"
+    finally:
+        tr.set_bf16_storage(False)
+        pkg.policy.set_gemm_bf16(False)
+    tr.close(); pol.close()
+
+
 def test_update_iteration_replays_from_a_graph(pkg, cuda):
     """backward + Adam captured once (after the lazily allocated GEMM workspaces
     exist) and replayed: every replay, with eager work and synchronisations in
