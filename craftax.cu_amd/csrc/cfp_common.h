@@ -201,10 +201,11 @@ int launch_splitk_reduce(float* dst, const float* part, long count, long stride,
                          hipStream_t st);
 // dW_enc[843][256] += features^T dh over the window columns, read from the records
 // (bf16 MFMA on the map bytes); needs envs per minibatch % 8 == 0.  tail_scratch:
-// cols * 76 floats.
+// cols * 76 floats.  dh_bf16: dh holds bf16 (one-product mode only).
 bool dw_enc_records_ok(int mb);
 int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
-                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st);
+                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
+                   bool dh_bf16 = false);
 
 // dW[rows][256] += dpre^T x with both fp32 operands split into bf16 triples
 // (cols % 8 == 0)
@@ -221,10 +222,12 @@ int gemm_dw_two(int rows_a, int rows_b, int cols, const float* x, const float* d
                 float* dW_a, float* dW_b, const SeamWork& sw, hipStream_t st);
 
 // dh[cols][256] (+)= dpre[cols][m3] . W[m3][256], same splitting (m3 % 16 == 0,
-// cols % 32 == 0, dpre 16-byte aligned)
+// cols % 32 == 0, dpre 16-byte aligned); dpre_bf16 / dh_bf16: that array holds bf16
+// (one-product mode only)
 bool gemm_dh_x9_ok(int m3, int cols, const float* dpre);
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               int terms, u4* w_mirror, hipStream_t st, bool dpre_bf16 = false);
+               int terms, u4* w_mirror, hipStream_t st, bool dpre_bf16 = false,
+               bool dh_bf16 = false);
 size_t dh_mirror_bytes();   // size of the split mirror of W (K up to 768)
 
 // y[cols][m] = x[cols][k] . W[m][k]^T on the same kernel (m % 256 == 0, k % 16 == 0,

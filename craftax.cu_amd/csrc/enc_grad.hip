@@ -58,6 +58,8 @@ __device__ __forceinline__ u4 byte_frag(const uint32_t (&d)[8]) {
     return f;
 }
 
+// D16: dh is a bf16 array (the update's bf16 storage): one product per byte.
+template <bool D16>
 __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
     const uint8_t* __restrict__ r_obs, const float* __restrict__ dh, float* __restrict__ part,
     int t0, int cols, int mb, int n_all, int env_start, int iters_per_split, int n_wg) {
@@ -98,11 +100,29 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
         stage[buf][pks][psb * 4 + 3][lane] = byte_frag<3>(e);
     };
     const float* dh_lane = dh + 32 * w + n;
+    const uint16_t* dh16_lane = reinterpret_cast<const uint16_t*>(dh) + 32 * w + n;
     auto dh_load = [&](int it, int ks, float (&v)[8]) {
         const int cc = min(it * kEgIterCols + ks * 16 + 8 * g, cols - 8);
+        if (D16) {
+            const uint16_t* p = dh16_lane + (size_t)cc * CFP_HIDDEN;
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                v[j] = __uint_as_float((uint32_t)p[j * CFP_HIDDEN] << 16);
+            return;
+        }
         const float* p = dh_lane + (size_t)cc * CFP_HIDDEN;
 #pragma unroll
         for (int j = 0; j < 8; j++) v[j] = p[j * CFP_HIDDEN];
+    };
+    // hi / mid / lo parts of eight gradients; bf16 values are their own hi part
+    auto dh_parts = [&](const float (&v)[8], u4& h, u4& m, u4& l) {
+        if (D16) {
+            h = round_bf16x8(v);
+            m = h;
+            l = h;
+        } else {
+            split3(v, h, m, l);
+        }
     };
 
     f16v acc[kEgBlocks];
@@ -130,7 +150,7 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
         a[0][0] = stage[0][0][0][lane];
         a[0][1] = stage[0][0][1][lane];
         u4 bh, bm, bl;
-        split3(raw[0], bh, bm, bl);
+        dh_parts(raw[0], bh, bm, bl);
         for (int it = it0; it < it1; it++) {
             const int buf = (it - it0) & 1;
             const int itn = min(it + 1, it1 - 1);
@@ -140,7 +160,7 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
                 if (ks < 1) dh_load(it, ks + 3, raw[ks + 3]);
                 else dh_load(itn, ks - 1, raw[ks - 1]);
                 u4 nh, nm, nl;
-                split3(raw[(ks + 1) & 3], nh, nm, nl);
+                dh_parts(raw[(ks + 1) & 3], nh, nm, nl);
 #pragma unroll
                 for (int pr = 0; pr < 4; pr++) {
                     const int cur = pr & 1, nxt = cur ^ 1;
@@ -159,10 +179,12 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
                     const int b = 2 * pr;
                     acc[b] = mfma16(a[cur][0], bh, acc[b]);
                     acc[b + 1] = mfma16(a[cur][1], bh, acc[b + 1]);
-                    acc[b] = mfma16(a[cur][0], bm, acc[b]);
-                    acc[b + 1] = mfma16(a[cur][1], bm, acc[b + 1]);
-                    acc[b] = mfma16(a[cur][0], bl, acc[b]);
-                    acc[b + 1] = mfma16(a[cur][1], bl, acc[b + 1]);
+                    if (!D16) {
+                        acc[b] = mfma16(a[cur][0], bm, acc[b]);
+                        acc[b + 1] = mfma16(a[cur][1], bm, acc[b + 1]);
+                        acc[b] = mfma16(a[cur][0], bl, acc[b]);
+                        acc[b + 1] = mfma16(a[cur][1], bl, acc[b + 1]);
+                    }
                 }
                 bh = nh; bm = nm; bl = nl;
             }
@@ -213,7 +235,8 @@ __global__ void k_expand_obs_tail(const uint8_t* __restrict__ r_obs, f4* __restr
 bool dw_enc_records_ok(int mb) { return mb > 0 && mb % 8 == 0; }
 
 int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
-                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st) {
+                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
+                   bool dh_bf16) {
     CFP_REQUIRE(r_obs && dh && dW && tail_scratch && cols > 0 && dw_enc_records_ok(mb) &&
                     cols % 8 == 0,
                 "dw_enc_records: columns and envs per minibatch must be multiples of 8");
@@ -230,8 +253,12 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
     splits = (total_iters + ips - 1) / ips;
     const int n_wg = splits * kEgGroups;
     const int grid = (n_wg + kEgXcds - 1) / kEgXcds * kEgXcds;
-    hipLaunchKernelGGL(k_dw_enc_bytes, dim3(grid), dim3(kEgThreads), 0, st, r_obs, dh, work, t0,
-                       cols, mb, n_all, env_start, ips, n_wg);
+    if (dh_bf16)
+        hipLaunchKernelGGL(k_dw_enc_bytes<true>, dim3(grid), dim3(kEgThreads), 0, st, r_obs, dh, work,
+                           t0, cols, mb, n_all, env_start, ips, n_wg);
+    else
+        hipLaunchKernelGGL(k_dw_enc_bytes<false>, dim3(grid), dim3(kEgThreads), 0, st, r_obs, dh, work,
+                           t0, cols, mb, n_all, env_start, ips, n_wg);
     const long count = (long)kEgFeat * CFP_HIDDEN;
     if (launch_splitk_reduce(dW, work, count, count, splits, st)) return 1;
     const size_t total4 = (size_t)cols * (kEgTailLd / 4);
@@ -239,6 +266,9 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
                        r_obs, reinterpret_cast<f4*>(tail_scratch), t0, total4, mb, n_all,
                        env_start);
     CFP_HIP_TRY(hipGetLastError());
+    if (dh_bf16)   // dh is the 256-wide operand of this GEMM, the 75 tail features its rows
+        return gemm_dw_x9(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, 1, sw, st, 0,
+                          nullptr, false, true);
     return gemm_dw_ld(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, sw, st);
 }
 

@@ -280,7 +280,18 @@ __global__ void k_pack_w_x9(const float* __restrict__ W, long sk, long su,
 
 // A16: dpre is stored as bf16 (bf16-input mode): a lane's eight values of a K step are
 // the MFMA operand as they lie in memory.
-template <int TERMS, bool A16 = false>
+// O16: dh is a bf16 array (ldc counts bf16 elements).  A lane holds unit n of each of
+// the eight 32-unit tiles; neighbouring lanes swap one value per pair of tiles, after
+// which an even lane owns units n, n+1 of the even tile and an odd lane units n-1, n of
+// the odd tile: one 4-byte access per lane, row and pair of tiles.
+__device__ __forceinline__ float swap_with_neighbour(float v) { return __shfl_xor(v, 1, 64); }
+__device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {   // nearest even
+    typedef float f2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{lo, hi}, bf16x2_t));
+}
+
+template <int TERMS, bool A16 = false, bool O16 = false>
 __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ dpre, int m3,
                                                       const u4* __restrict__ wm,
                                                       float* __restrict__ dh, int ldc, int cols,
@@ -335,13 +346,34 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
 
     // accumulating form: the accumulators start from dh, all 128 loads in flight at
     // once under the prologue's own loads, and the epilogue is stores only
+    static_assert(TERMS == 1 || !O16, "bf16 storage goes with bf16 inputs");
     float* o_lane = dh + (size_t)(cbc + 4 * g) * ldc + n;
+    // O16: the lane's dword of a pair of tiles (ldc even, n - odd even: 4-byte aligned)
+    const bool odd = n & 1;
+    uint32_t* o16_lane = reinterpret_cast<uint32_t*>(
+        reinterpret_cast<uint16_t*>(dh) + (size_t)(cbc + 4 * g) * ldc + (odd ? 32 + n - 1 : n));
     f16v acc[8];
+    if (O16) {
 #pragma unroll
-    for (int t = 0; t < 8; t++)
+        for (int tp = 0; tp < 4; tp++)
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-            acc[t][r] = accumulate ? o_lane[(size_t)acc_row(r) * ldc + 32 * t] : 0.0f;
+            for (int r = 0; r < 16; r++) {
+                const uint32_t d =
+                    accumulate ? o16_lane[((size_t)acc_row(r) * ldc + 64 * tp) >> 1] : 0u;
+                const float lo = __uint_as_float(d << 16), hi = __uint_as_float(d & 0xffff0000u);
+                // even lane: lo is its own unit of the even tile, hi the neighbour's;
+                // odd lane: hi is its own unit of the odd tile, lo the neighbour's
+                const float got = swap_with_neighbour(odd ? lo : hi);
+                acc[2 * tp][r] = odd ? got : lo;
+                acc[2 * tp + 1][r] = odd ? hi : got;
+            }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++)
+                acc[t][r] = accumulate ? o_lane[(size_t)acc_row(r) * ldc + 32 * t] : 0.0f;
+    }
 
     float raw[2][8];
     u4 wb[3];
@@ -387,6 +419,20 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
         }
         as[0] = ns[0]; as[1] = ns[1]; as[2] = ns[2];
     }
+    if (O16) {
+        // the swap involves every lane of the wavefront: it comes before the early exit
+#pragma unroll
+        for (int tp = 0; tp < 4; tp++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const float got =
+                    swap_with_neighbour(odd ? acc[2 * tp][r] : acc[2 * tp + 1][r]);
+                const uint32_t d = odd ? pack_bf16_pair(got, acc[2 * tp + 1][r])
+                                       : pack_bf16_pair(acc[2 * tp][r], got);
+                if (live) o16_lane[((size_t)acc_row(r) * ldc + 64 * tp) >> 1] = d;
+            }
+        return;
+    }
     if (!live) return;
 #pragma unroll
     for (int t = 0; t < 8; t++)
@@ -408,15 +454,21 @@ bool gemm_dh_x9_ok(int m3, int cols, const float* dpre) {
 // out[cols][ldc] (+)= A[cols][K] . B, B(k, u) = B[k*sk + u*su] for 256 units
 static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const float* A,
                         float* out, int ldc, bool accumulate, int terms, u4* g_w_x9,
-                        hipStream_t st, bool a16 = false) {
-    CFP_REQUIRE(!a16 || terms == 1, "k_dh_x9: bf16-stored operands need the bf16-input mode");
+                        hipStream_t st, bool a16 = false, bool o16 = false) {
+    CFP_REQUIRE((!a16 && !o16) || terms == 1,
+                "k_dh_x9: bf16-stored operands need the bf16-input mode");
+    CFP_REQUIRE(!o16 || ldc % 2 == 0, "k_dh_x9: a bf16 result needs an even row length");
     CFP_REQUIRE(g_w_x9, "k_dh_x9: no mirror buffer for W");
     const int total = (K / 16) * kDhFrags * 64;
     hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, B, sk, su, g_w_x9,
                        total, terms == 1 ? 1 : 0);
     const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
     const int acc = accumulate ? 1 : 0;
-    if (a16)
+    if (a16 && o16)
+        hipLaunchKernelGGL((k_dh_x9<1, true, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+    else if (o16)
+        hipLaunchKernelGGL((k_dh_x9<1, false, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+    else if (a16)
         hipLaunchKernelGGL((k_dh_x9<1, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
     else if (terms == 1)
         hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
@@ -431,11 +483,11 @@ static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const
 size_t dh_mirror_bytes() { return kDhMirrorBytes; }
 
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
-               int terms, u4* w_mirror, hipStream_t st, bool dpre_bf16) {
+               int terms, u4* w_mirror, hipStream_t st, bool dpre_bf16, bool dh_bf16) {
     CFP_REQUIRE(gemm_dh_x9_ok(m3, cols, dpre) && W && dh,
                 "gemm_dh_x9: K must be a multiple of 16 up to %d and columns of 32", kDhMaxK);
     return launch_dh_x9(m3, cols, W, CFP_HIDDEN, 1, dpre, dh, CFP_HIDDEN, accumulate, terms, w_mirror,
-                        st, dpre_bf16);
+                        st, dpre_bf16, dh_bf16);
 }
 
 // y[cols][m] = x[cols][k] . W[m][k]^T in slices of 256 output rows of W

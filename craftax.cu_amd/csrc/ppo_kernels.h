@@ -29,7 +29,8 @@ struct ReverseArgs {
     int steps;                 // steps in this window
     int layer, layers;
     int horizon, seg;          // rollout length, BPTT segment length
-    int gates_bf16;            // gates and layer_in are bf16 arrays (the update's bf16 storage)
+    int gates_bf16;            // gates, layer_in, grad_a/b and highway_out are bf16 arrays (the
+                               // update's bf16 storage); slab_state and carry stay fp32
 };
 int launch_gru_reverse(const ReverseArgs& a, hipStream_t st);
 

@@ -49,7 +49,8 @@ __device__ __forceinline__ double wave_sum(double v) {
 // issue order, so "the set fetched three stages ago has landed" is "at most N younger
 // operations are outstanding".  Three register sets rotate through a loop unrolled by
 // three (a set is never copied: a copy would read registers whose loads are in flight).
-// G16: the gate rows and the layer input are stored as bf16 (8 bytes per lane and row).
+// G16: the gate rows, the layer input, the incoming gradients and the highway term are
+// stored as bf16 (8 bytes per lane and row); the recorded state stays fp32.
 typedef unsigned int u2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
@@ -62,8 +63,8 @@ struct StepIn<false> {
 };
 template <>
 struct StepIn<true> {
-    u2 zh, zg, zp, x;
-    f4 ga, gb, s;
+    u2 zh, zg, zp, x, ga, gb;
+    f4 s;
     unsigned done;
 };
 
@@ -79,7 +80,7 @@ __device__ __forceinline__ u2 narrow(const f4& v) {   // round to nearest even
 // lo: byte offset of the lane inside an fp32 row (16 q), lo8: inside a bf16 row (8 q)
 template <bool TWO_GRADS, bool G16>
 __device__ __forceinline__ void sweep_fetch(StepIn<G16>& r, unsigned lo, unsigned lo8,
-                                            const void* gates, const f4* ga, const f4* gb,
+                                            const void* gates, const void* ga, const void* gb,
                                             const f4* state, const void* xin, const uint8_t* done) {
     const unsigned zero = 0u;
     if (G16 && TWO_GRADS)
@@ -87,8 +88,8 @@ __device__ __forceinline__ void sweep_fetch(StepIn<G16>& r, unsigned lo, unsigne
             "global_load_dwordx2 %0, %9, %11 nt\n\t"
             "global_load_dwordx2 %1, %9, %11 offset:512 nt\n\t"
             "global_load_dwordx2 %2, %9, %11 offset:1024 nt\n\t"
-            "global_load_dwordx4 %3, %8, %12 nt\n\t"
-            "global_load_dwordx4 %4, %8, %13 nt\n\t"
+            "global_load_dwordx2 %3, %9, %12 nt\n\t"
+            "global_load_dwordx2 %4, %9, %13 nt\n\t"
             "global_load_dwordx4 %5, %8, %14 nt\n\t"
             "global_load_dwordx2 %6, %9, %15 nt\n\t"
             "global_load_ubyte %7, %10, %16"
@@ -102,7 +103,7 @@ __device__ __forceinline__ void sweep_fetch(StepIn<G16>& r, unsigned lo, unsigne
             "global_load_dwordx2 %0, %8, %10 nt\n\t"
             "global_load_dwordx2 %1, %8, %10 offset:512 nt\n\t"
             "global_load_dwordx2 %2, %8, %10 offset:1024 nt\n\t"
-            "global_load_dwordx4 %3, %7, %11 nt\n\t"
+            "global_load_dwordx2 %3, %8, %11 nt\n\t"
             "global_load_dwordx4 %4, %7, %12 nt\n\t"
             "global_load_dwordx2 %5, %8, %13 nt\n\t"
             "global_load_ubyte %6, %9, %14"
@@ -174,8 +175,9 @@ __device__ __forceinline__ void sweep_drain(StepIn<G16>& p, StepIn<G16>& q, Step
 
 // the trailing s_nop keeps the next instruction clear of the store data registers
 template <bool HIGHWAY>
-__device__ __forceinline__ void sweep_store(unsigned lo, unsigned, void* gates, f4* hw, const f4& dzh,
-                                            const f4& dzg, const f4& dzp, const f4& hwv) {
+__device__ __forceinline__ void sweep_store(unsigned lo, unsigned, void* gates, void* hw,
+                                            const f4& dzh, const f4& dzg, const f4& dzp,
+                                            const f4& hwv) {
     if (HIGHWAY)
         asm volatile(
             "global_store_dwordx4 %0, %1, %5 nt\n\t"
@@ -197,18 +199,18 @@ __device__ __forceinline__ void sweep_store(unsigned lo, unsigned, void* gates, 
             : "memory");
 }
 template <bool HIGHWAY>
-__device__ __forceinline__ void sweep_store(unsigned lo, unsigned lo8, void* gates, f4* hw,
+__device__ __forceinline__ void sweep_store(unsigned, unsigned lo8, void* gates, void* hw,
                                             const u2& dzh, const u2& dzg, const u2& dzp,
-                                            const f4& hwv) {
+                                            const u2& hwv) {
     if (HIGHWAY)
         asm volatile(
-            "global_store_dwordx2 %1, %2, %6 nt\n\t"
-            "global_store_dwordx2 %1, %3, %6 offset:512 nt\n\t"
-            "global_store_dwordx2 %1, %4, %6 offset:1024 nt\n\t"
-            "global_store_dwordx4 %0, %5, %7 nt\n\t"
+            "global_store_dwordx2 %0, %1, %5 nt\n\t"
+            "global_store_dwordx2 %0, %2, %5 offset:512 nt\n\t"
+            "global_store_dwordx2 %0, %3, %5 offset:1024 nt\n\t"
+            "global_store_dwordx2 %0, %4, %6 nt\n\t"
             "s_nop 0"
             :
-            : "v"(lo), "v"(lo8), "v"(dzh), "v"(dzg), "v"(dzp), "v"(hwv), "s"(gates), "s"(hw)
+            : "v"(lo8), "v"(dzh), "v"(dzg), "v"(dzp), "v"(hwv), "s"(gates), "s"(hw)
             : "memory");
     else
         asm volatile(
@@ -236,9 +238,10 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
     constexpr size_t kGateRow = G16 ? G * 2 : G * 4, kInRow = G16 ? H * 2 : H * 4;   // bytes
     char* const gates = reinterpret_cast<char*>(a.gates) + (size_t)env * kGateRow;
     const char* const xin = reinterpret_cast<const char*>(a.layer_in) + (size_t)env * kInRow;
-    const f4* const ga = reinterpret_cast<const f4*>(a.grad_a) + (size_t)env * H4;
-    const f4* const gb = TWO_GRADS ? reinterpret_cast<const f4*>(a.grad_b) + (size_t)env * H4 : nullptr;
-    f4* const hw = HIGHWAY ? reinterpret_cast<f4*>(a.highway_out) + (size_t)env * H4 : nullptr;
+    const char* const ga = reinterpret_cast<const char*>(a.grad_a) + (size_t)env * kInRow;
+    const char* const gb =
+        TWO_GRADS ? reinterpret_cast<const char*>(a.grad_b) + (size_t)env * kInRow : nullptr;
+    char* const hw = HIGHWAY ? reinterpret_cast<char*>(a.highway_out) + (size_t)env * kInRow : nullptr;
     const size_t slab_env = (size_t)a.w.env_start + env;
     const size_t state_step = (size_t)a.layers * a.w.n_all * H4;
     const f4* const state = reinterpret_cast<const f4*>(a.slab_state) +
@@ -255,7 +258,8 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
         const size_t c = (size_t)(real ? s : 0) * mbz;
         sweep_fetch<TWO_GRADS, G16>(
             r, lane_off, lane_off8, real ? (const void*)(gates + c * kGateRow) : (const void*)idle,
-            real ? ga + c * H4 : idle, TWO_GRADS ? (real ? gb + c * H4 : idle) : nullptr,
+            real ? (const void*)(ga + c * kInRow) : (const void*)idle,
+            TWO_GRADS ? (real ? (const void*)(gb + c * kInRow) : (const void*)idle) : nullptr,
             real ? state + (size_t)s * state_step : idle,
             real ? (const void*)(xin + c * kInRow) : (const void*)idle,
             done + (size_t)(real ? s : 0) * a.w.n_all);
@@ -273,6 +277,9 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
         phase = (phase == 0 ? a.seg : phase) - 1;
         const float pass = (in.done & 0xffu) ? 0.0f : 1.0f;   // a terminal step hands nothing back
         const f4 zh = widen(in.zh), zg = widen(in.zg), zp = widen(in.zp), x = widen(in.x);
+        const f4 ga_v = widen(in.ga);
+        f4 gb_v = f4{0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (TWO_GRADS) gb_v = widen(in.gb);
         f4 dzh, dzg, dzp, hwv;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
@@ -284,7 +291,7 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
             const float dcand = lin ? 1.0f : sh * (1.0f - sh);       // g'(zh)
             const float gap = cand - in.s[j];
             const float h_new = in.s[j] + sg * gap;
-            const float g_top = TWO_GRADS ? in.ga[j] + in.gb[j] : in.ga[j];
+            const float g_top = TWO_GRADS ? ga_v[j] + gb_v[j] : ga_v[j];
             const float g_h = g_top * mix + pass * carry[j];
             dzp[j] = g_top * (h_new - x[j]) * mix * (1.0f - mix);
             hwv[j] = g_top * (1.0f - mix);
@@ -294,11 +301,12 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
         }
         const size_t c = (size_t)s * mbz;
         if constexpr (G16)
-            sweep_store<HIGHWAY>(lane_off, lane_off8, gates + c * kGateRow, HIGHWAY ? hw + c * H4 : nullptr,
-                                 narrow(dzh), narrow(dzg), narrow(dzp), hwv);
+            sweep_store<HIGHWAY>(lane_off, lane_off8, gates + c * kGateRow,
+                                 HIGHWAY ? hw + c * kInRow : nullptr, narrow(dzh), narrow(dzg),
+                                 narrow(dzp), narrow(hwv));
         else
-            sweep_store<HIGHWAY>(lane_off, lane_off8, gates + c * kGateRow, HIGHWAY ? hw + c * H4 : nullptr,
-                                 dzh, dzg, dzp, hwv);
+            sweep_store<HIGHWAY>(lane_off, lane_off8, gates + c * kGateRow,
+                                 HIGHWAY ? hw + c * kInRow : nullptr, dzh, dzg, dzp, hwv);
     };
 
     // Operations per stage: NL loads then (after the step's arithmetic) NS stores.

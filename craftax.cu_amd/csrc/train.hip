@@ -46,7 +46,14 @@ __global__ void k_head_mirror(const float* __restrict__ W_a, const float* __rest
 // with CL = 256 / RB threads each; a thread walks every CL-th column of the slice with
 // four independent running sums (loads in flight instead of one dependent chain) and
 // the CL sums of a row are added in thread order: a fixed order throughout.
-template <int RB>
+// S16: src is a bf16 array (ld counts its elements).
+template <bool S16>
+__device__ __forceinline__ float colsum_at(const float* src, size_t i) {
+    if (S16)
+        return __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(src)[i] << 16);
+    return src[i];
+}
+template <int RB, bool S16 = false>
 __global__ __launch_bounds__(256) void k_colsum_partial(
     const float* __restrict__ src, int ld, float* __restrict__ part, int rows, int cols,
     int cols_per_slice) {
@@ -58,15 +65,14 @@ __global__ __launch_bounds__(256) void k_colsum_partial(
     const int c1 = min(cols, c0 + cols_per_slice);
     float s0 = 0.0f, s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
     if (r < rows) {
-        const float* p = src + r;
         int c = c0 + cl;
         for (; c + 3 * CL < c1; c += 4 * CL) {
-            s0 += p[(size_t)c * ld];
-            s1 += p[(size_t)(c + CL) * ld];
-            s2 += p[(size_t)(c + 2 * CL) * ld];
-            s3 += p[(size_t)(c + 3 * CL) * ld];
+            s0 += colsum_at<S16>(src, (size_t)c * ld + r);
+            s1 += colsum_at<S16>(src, (size_t)(c + CL) * ld + r);
+            s2 += colsum_at<S16>(src, (size_t)(c + 2 * CL) * ld + r);
+            s3 += colsum_at<S16>(src, (size_t)(c + 3 * CL) * ld + r);
         }
-        for (; c < c1; c += CL) s0 += p[(size_t)c * ld];
+        for (; c < c1; c += CL) s0 += colsum_at<S16>(src, (size_t)c * ld + r);
     }
     red[cl][rl] = (s0 + s1) + (s2 + s3);
     __syncthreads();
@@ -397,12 +403,15 @@ int cfp_train_adv_stats(cfp_trainer* tr, void* stream) {
 }
 
 static int colsum_into(cfp_trainer* tr, const float* src, int ld, float* out, int rows,
-                       int cols, hipStream_t st) {
+                       int cols, hipStream_t st, bool src_bf16 = false) {
     int slices = kColsumSlices;
     if (slices > cols) slices = cols;
     const int per = (cols + slices - 1) / slices;
     slices = (cols + per - 1) / per;
-    if (rows <= 64)
+    if (src_bf16)
+        hipLaunchKernelGGL((k_colsum_partial<256, true>), dim3(slices, (rows + 255) / 256), dim3(256),
+                           0, st, src, ld, tr->colsum_part, rows, cols, per);
+    else if (rows <= 64)
         hipLaunchKernelGGL(k_colsum_partial<64>, dim3(slices, 1), dim3(256), 0, st, src, ld,
                            tr->colsum_part, rows, cols, per);
     else
@@ -452,9 +461,11 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         // state in, pre-activations and layer outputs out.  The unfused chain below is
         // what bf16 inputs run with the split kernels switched off.
         const bool fused = cfp_get_gemm_bf16() == 0 || cfp_get_gemm_split() != 0;
-        // bf16 storage: pre / dpre and the layer inputs x[0..L] are bf16 arrays inside
-        // the same buffers; needs mb % 32 (the record-fed dW_enc) and the split kernels
-        const bool st16 = tr->bf16_store && cfp_get_gemm_bf16() != 0 && cfp_get_gemm_split() != 0;
+        // bf16 storage: pre / dpre, the layer inputs x[0..L] and the three dh buffers are
+        // bf16 arrays inside the same buffers; needs the record-fed dW_enc and the split
+        // kernels
+        const bool st16 = tr->bf16_store && cfp_get_gemm_bf16() != 0 && cfp_get_gemm_split() != 0 &&
+                          dw_enc_records_ok(mb);
         if (fused) {
             FwdArgs fa{};
             fill_forward_weights(p, fa);
@@ -508,7 +519,14 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         if (launch_head(ha, st)) return 1;
         if (launch_fold_f64(tr->block_loss, head_blocks(cols), 3, tr->loss_acc, true, st)) return 1;
         // dh3 = [dlogits | dvalue] . [W_a ; W_v]; dW_a and dW_v from one GEMM; bias sums
-        if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, tr->sw, st)) return 1;
+        // (bf16 storage: the three dh buffers hold bf16 as well)
+        if (st16) {
+            if (gemm_dh_x9(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, 1,
+                           tr->sw.w_mirror, st, false, true))
+                return 1;
+        } else if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, tr->sw, st)) {
+            return 1;
+        }
         if (st16) {
             if (gemm_dw_x9(A + 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L), 1, tr->sw,
                            st, A, g + CFP_OFF_W_V(L), false, true))
@@ -546,7 +564,8 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             // layer 0: dh_enc = W_0^T dpre + highway, accumulated onto the highway term
             if (st16) {
                 if (gemm_dh_x9(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
-                               l == 0 ? tr->dhX : tr->dhG, l == 0, 1, tr->sw.w_mirror, chain, true))
+                               l == 0 ? tr->dhX : tr->dhG, l == 0, 1, tr->sw.w_mirror, chain, true,
+                               true))
                     return 1;
             } else if (gemm_dh_acc(G, cols, W_gru + (size_t)l * G * H, tr->preb[l],
                                    l == 0 ? tr->dhX : tr->dhG, l == 0, tr->sw, chain)) {
@@ -565,12 +584,12 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             dh_extra = tr->dhX;
         }
         // ---- encoder: db_enc; dW_enc += xobs^T dh_enc (dh_enc sits in dhX)
-        if (colsum_into(tr, tr->dhX, H, g + CFP_OFF_B_ENC, H, cols, chain)) return 1;
+        if (colsum_into(tr, tr->dhX, H, g + CFP_OFF_B_ENC, H, cols, chain, st16)) return 1;
         if (dw_enc_records_ok(mb)) {
             // map bytes straight from the records; xobs is free by now and takes the
             // 76-float rows of the fp32 remainder
             if (dw_enc_records(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
-                               env_start, tr->sw, chain))
+                               env_start, tr->sw, chain, st16))
                 return 1;
         } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, tr->sw,
                               chain)) {

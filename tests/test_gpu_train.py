@@ -493,8 +493,8 @@ def test_adam_writes_every_weight_mirror(pkg, cuda):
 @pytest.mark.parametrize("n,T,minibatches,bwd_win,done_p", [(64, 8, 1, 0, 0.1), (128, 6, 2, 4, 0.15)])
 def test_backward_with_bf16_storage(pkg, cuda, n, T, minibatches, bwd_win, done_p):
     """bf16 GEMM inputs with the window workspace stored as bf16 (cfp_train_set_bf16_storage:
-    gate pre-activations, their gradients and the layer inputs; the reference's
-    CF_GEMM_BF16 storage) against the fp64 oracle, every gradient segment within 2e-2 in
+    gate pre-activations, their gradients, the layer inputs and the hidden-state gradients
+    between the layers; the reference's CF_GEMM_BF16 storage) against the fp64 oracle, every gradient segment within 2e-2 in
     the relative Frobenius norm -- the tolerance of the bf16-input mode -- and close to
     the same update with fp32 storage.  Behaviour log-probabilities are the current
     policy's own plus noise, so no sample sits on the clip discontinuity (see
