@@ -201,11 +201,14 @@ int launch_splitk_reduce(float* dst, const float* part, long count, long stride,
                          hipStream_t st);
 // dW_enc[843][256] += features^T dh over the window columns, read from the records
 // (bf16 MFMA on the map bytes); needs envs per minibatch % 8 == 0.  tail_scratch:
-// cols * 76 floats.  dh_bf16: dh holds bf16 (one-product mode only).
+// cols * 76 floats.  dh_bf16: dh holds bf16 (one-product mode only).  sw_tail / st_tail:
+// workspace and stream for the GEMM of the last 75 features (both must be ordered behind
+// dh; default: the same as the first 768).
 bool dw_enc_records_ok(int mb);
 int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
                    int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
-                   bool dh_bf16 = false);
+                   bool dh_bf16 = false, const SeamWork* sw_tail = nullptr,
+                   hipStream_t st_tail = nullptr);
 
 // dW[rows][256] += dpre^T x with both fp32 operands split into bf16 triples
 // (cols % 8 == 0)

@@ -236,7 +236,7 @@ bool dw_enc_records_ok(int mb) { return mb > 0 && mb % 8 == 0; }
 
 int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
                    int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
-                   bool dh_bf16) {
+                   bool dh_bf16, const SeamWork* sw_tail, hipStream_t st_tail) {
     CFP_REQUIRE(r_obs && dh && dW && tail_scratch && cols > 0 && dw_enc_records_ok(mb) &&
                     cols % 8 == 0,
                 "dw_enc_records: columns and envs per minibatch must be multiples of 8");
@@ -261,15 +261,19 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
                            t0, cols, mb, n_all, env_start, ips, n_wg);
     const long count = (long)kEgFeat * CFP_HIDDEN;
     if (launch_splitk_reduce(dW, work, count, count, splits, st)) return 1;
+    // rows 768..842: a GEMM of its own on other rows of dW, on the second stream and
+    // workspace when the caller has one to spare
+    const SeamWork& swt = sw_tail ? *sw_tail : sw;
+    hipStream_t stt = sw_tail ? st_tail : st;
     const size_t total4 = (size_t)cols * (kEgTailLd / 4);
-    hipLaunchKernelGGL(k_expand_obs_tail, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, st,
+    hipLaunchKernelGGL(k_expand_obs_tail, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stt,
                        r_obs, reinterpret_cast<f4*>(tail_scratch), t0, total4, mb, n_all,
                        env_start);
     CFP_HIP_TRY(hipGetLastError());
     if (dh_bf16)   // dh is the 256-wide operand of this GEMM, the 75 tail features its rows
-        return gemm_dw_x9(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, 1, sw, st, 0,
+        return gemm_dw_x9(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, 1, swt, stt, 0,
                           nullptr, false, true);
-    return gemm_dw_ld(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, sw, st);
+    return gemm_dw_ld(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, swt, stt);
 }
 
 }  // namespace cfp

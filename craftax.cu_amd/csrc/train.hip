@@ -589,7 +589,8 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             // map bytes straight from the records; xobs is free by now and takes the
             // 76-float rows of the fp32 remainder
             if (dw_enc_records(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
-                               env_start, tr->sw, chain, st16))
+                               env_start, tr->sw, chain, st16, overlap ? &tr->sw_layer[0] : nullptr,
+                               other))
                 return 1;
         } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, tr->sw,
                               chain)) {
