@@ -430,9 +430,11 @@ void* cfp_train_buffer(cfp_trainer* tr, int which);
  * :9538-9590).  In effect only while cfp_set_gemm_bf16(1) is on with the split kernels
  * (cfp_set_gemm_split != 0): the window recompute then writes the gate pre-activations
  * and layer inputs as bf16, the reverse sweep reads them and leaves the gate gradients
- * as bf16, and the dW / dh GEMMs take those as their operands unconverted -- half the
- * bytes of the kernels that bound the bf16 update.  r_state, the dh buffers, head rows
- * and every gradient stay fp32.  Off by default. */
+ * as bf16, the dW / dh GEMMs take those as their operands unconverted, and the
+ * hidden-state gradients between the layers (the dh buffers) are bf16 as well -- half
+ * the bytes of the kernels that bound the bf16 update.  r_state, the head rows and
+ * every weight gradient stay fp32.  Needs envs per minibatch % 8 == 0 (otherwise the
+ * update runs with fp32 storage).  Off by default. */
 int cfp_train_set_bf16_storage(cfp_trainer* tr, int on);
 int cfp_train_bf16_storage(const cfp_trainer* tr);
 int cfp_train_window(const cfp_trainer* tr);
