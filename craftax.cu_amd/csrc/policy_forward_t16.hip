@@ -210,6 +210,18 @@ __global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a
         tw[B][0] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave) * 64 + lane];
         tw[B][1] = a.t16_enc_t[(size_t)(B * 16 + 2 * wave + 1) * 64 + lane];
     }
+    // ... and the heads' weights: a wave takes K blocks 2 wave and 2 wave + 1 of the three
+    // row tiles
+    f4 hw[2][kT16HeadTiles];
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int t = 0; t < kT16HeadTiles; t++)
+            hw[kb][t] = a.t16_wav[((size_t)(2 * wave + kb) * kT16HeadTiles + t) * 64 + lane];
+    // (waves 0..2 finish head row 16 wave + c: its bias)
+    const int head_row = 16 * wave + c;
+    float head_bias = 0.0f;
+    if (head_row < CFP_AV) head_bias = head_row < CFP_ACTIONS ? a.b_a[head_row] : a.b_v[0];
     asm volatile("" ::: "memory");
     t16_dma(ws, ring, lane);
     t16_dma(ws + kStep, ring + kT16SlotF4, lane);
@@ -386,26 +398,42 @@ __global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a
     }
     if (a.h3_out) tile_out(a.h3_out);
 
-    // ---- heads: waves 0..2 take one 16-row tile each over the full K ----------------------
+    // ---- heads: every wave takes two of the sixteen K blocks of all three 16-row tiles;
+    // the eight partial sums meet in LDS and are added in wave order
     __shared__ float s_logit[kT16Envs * CFP_AV];
     __shared__ float s_expo[kT16Envs * kMaxActions];
-    if (wave < kT16HeadTiles) {
-        f4 hacc = {0, 0, 0, 0};
-        const f4* wp = a.t16_wav + (size_t)wave * 64 + lane;
+    __shared__ __attribute__((aligned(16))) f4 s_hpart[8][kT16HeadTiles][64];   // 24 KiB
+    static_assert(kT16GateBlocks == 16, "two K blocks per wave");
+    {
+        f4 hacc[kT16HeadTiles];
 #pragma unroll
-        for (int K = 0; K < kT16GateBlocks; K++) {
-            const f4 hb = wp[(size_t)K * kT16HeadTiles * 64];
-            const f4 av = xs4[c * XS4 + 4 * K + q];
+        for (int t = 0; t < kT16HeadTiles; t++) hacc[t] = f4{0, 0, 0, 0};
 #pragma unroll
-            for (int m = 0; m < 4; m++) hacc = mfma4(av[m], hb[m], hacc);
+        for (int kb = 0; kb < 2; kb++) {
+            const f4 av = xs4[c * XS4 + 4 * (2 * wave + kb) + q];
+#pragma unroll
+            for (int m = 0; m < 4; m++)
+#pragma unroll
+                for (int t = 0; t < kT16HeadTiles; t++) hacc[t] = mfma4(av[m], hw[kb][t][m], hacc[t]);
         }
-        const int row = 16 * wave + c;
+#pragma unroll
+        for (int t = 0; t < kT16HeadTiles; t++) s_hpart[wave][t][lane] = hacc[t];
+    }
+    __syncthreads();
+    if (wave < kT16HeadTiles) {
+        f4 hacc = s_hpart[0][wave][lane];
+#pragma unroll
+        for (int w = 1; w < 8; w++) {
+            const f4 part = s_hpart[w][wave][lane];
+#pragma unroll
+            for (int r = 0; r < 4; r++) hacc[r] += part[r];
+        }
+        const int row = head_row;
         if (row < CFP_AV) {
-            const float bias = row < CFP_ACTIONS ? a.b_a[row] : a.b_v[0];
             float* o = a.av_out + (e0 + 4 * q) * CFP_AV + row;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                const float v = hacc[r] + bias;
+                const float v = hacc[r] + head_bias;
                 o[r * CFP_AV] = v;
                 s_logit[(4 * q + r) * CFP_AV + row] = v;
             }
@@ -414,6 +442,11 @@ __global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a
     // ---- the draw, sixteen lanes per env (sample_row.h), and the step counter's bump ---------
     if (a.s_act) {   // uniform over the launch
         __syncthreads();
+        // The ticket first: its round trip runs under the draw.  Every lane's read of the
+        // counter (draw_step, the kernel's first load) has returned: loads return in
+        // order, and younger ones fed the MFMAs in front of the barriers above.
+        unsigned ticket_no = 0u;
+        if (tid == 0) ticket_no = take_ticket(a.s_ticket);
         const int sub = tid % kSampleLanes, slot = tid / kSampleLanes;
         const bool live = slot < kT16Envs;
         const float* lp = s_logit + (live ? slot : 0) * CFP_AV;
@@ -423,8 +456,7 @@ __global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a
         if (live && sub == 0)
             sample_draw<CFP_ACTIONS>(lp, px, mx, CFP_ACTIONS, (int)e0 + slot, a.s_seed, draw_step,
                         a.s_env_actions, a.s_act, a.s_logp, a.s_value);
-        __syncthreads();
-        if (tid == 0) bump_by_last_group(a.s_ticket, a.s_step, gridDim.x);
+        if (tid == 0) bump_if_last(ticket_no, gridDim.x, a.s_ticket, a.s_step, draw_step);
     }
 }
 

@@ -89,5 +89,16 @@ __device__ __forceinline__ void bump_by_last_group(unsigned* ticket, uint64_t* c
         *ticket = 0u;
     }
 }
+// The same in two halves, for a workgroup that holds the counter's value in registers
+// (`step`): the ticket can be taken as soon as all its reads of the counter have returned,
+// and the atomic's round trip then runs under whatever work is left.
+__device__ __forceinline__ unsigned take_ticket(unsigned* ticket) { return atomicAdd(ticket, 1u); }
+__device__ __forceinline__ void bump_if_last(unsigned no, unsigned groups, unsigned* ticket,
+                                             uint64_t* ctr, uint64_t step) {
+    if (no == groups - 1) {
+        *ctr = step + 1;
+        *ticket = 0u;
+    }
+}
 
 }  // namespace cfp
