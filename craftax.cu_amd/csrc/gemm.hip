@@ -474,7 +474,7 @@ const SeamWork* seam_default() {
 int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* d_dh,
                 bool accumulate, const SeamWork& sw, hipStream_t st) {
     CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh: bad argument");
-    if (g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre))
+    if (g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre) && (!accumulate || m3 >= 160))
         return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, split_terms(), sw.w_mirror, st);
     GemmArgs g{};
     g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;

@@ -352,28 +352,65 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     const bool odd = n & 1;
     uint32_t* o16_lane = reinterpret_cast<uint32_t*>(
         reinterpret_cast<uint16_t*>(dh) + (size_t)(cbc + 4 * g) * ldc + (odd ? 32 + n - 1 : n));
+    // The accumulators start at zero; the old contents of dh are fetched one 32-unit tile
+    // (O16: one pair of tiles) per K step during the first steps and added a step later, so
+    // that the fetch runs under the MFMAs instead of in front of them.  Short K: all of
+    // it up front.
+    constexpr int kSpreadMax = O16 ? 4 : 8;
+    constexpr int spread_steps = kSpreadMax;
+    const bool spread = accumulate != 0;   // the launcher asks for steps > spread_steps
     f16v acc[8];
-    if (O16) {
 #pragma unroll
-        for (int tp = 0; tp < 4; tp++)
+    for (int t = 0; t < 8; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t d =
-                    accumulate ? o16_lane[((size_t)acc_row(r) * ldc + 64 * tp) >> 1] : 0u;
-                const float lo = __uint_as_float(d << 16), hi = __uint_as_float(d & 0xffff0000u);
-                // even lane: lo is its own unit of the even tile, hi the neighbour's;
-                // odd lane: hi is its own unit of the odd tile, lo the neighbour's
-                const float got = swap_with_neighbour(odd ? lo : hi);
-                acc[2 * tp][r] = odd ? got : lo;
-                acc[2 * tp + 1][r] = odd ? hi : got;
-            }
-    } else {
+        for (int r = 0; r < 16; r++) acc[t][r] = 0.0f;
+    f16v held;   // O16: sixteen dwords of two bf16 as raw bits
+    auto old_fetch = [&](int i) {   // tile i, or pair of tiles i
 #pragma unroll
-        for (int t = 0; t < 8; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r++)
-                acc[t][r] = accumulate ? o_lane[(size_t)acc_row(r) * ldc + 32 * t] : 0.0f;
+        for (int r = 0; r < 16; r++) {
+            if (O16)
+                held[r] = __uint_as_float(o16_lane[((size_t)acc_row(r) * ldc + 64 * i) >> 1]);
+            else
+                held[r] = o_lane[(size_t)acc_row(r) * ldc + 32 * i];
+        }
+    };
+    // (macros, not lambdas over references: the accumulators must stay in registers)
+#define CFP_DH_OLD_ADD(EVEN, OTHER)                                                                \
+    _Pragma("unroll") for (int r = 0; r < 16; r++) {                                               \
+        if (O16) {                                                                                 \
+            const uint32_t d = __float_as_uint(held[r]);                                           \
+            const float lo = __uint_as_float(d << 16), hi = __uint_as_float(d & 0xffff0000u);      \
+            /* even lane: lo is its own unit of the even tile, hi the neighbour's; */              \
+            /* odd lane: hi is its own unit of the odd tile, lo the neighbour's */                 \
+            const float got = swap_with_neighbour(odd ? lo : hi);                                  \
+            acc[EVEN][r] += odd ? got : lo;                                                        \
+            acc[OTHER][r] += odd ? hi : got;                                                       \
+        } else {                                                                                   \
+            acc[EVEN][r] += held[r];                                                               \
+        }                                                                                          \
     }
+#define CFP_DH_OLD_ADD_AT(I)                                                                       \
+    do {   /* I is uniform over the workgroup */                                                   \
+        if (O16) {                                                                                 \
+            switch (I) {                                                                           \
+                case 0: CFP_DH_OLD_ADD(0, 1) break;                                                \
+                case 1: CFP_DH_OLD_ADD(2, 3) break;                                                \
+                case 2: CFP_DH_OLD_ADD(4, 5) break;                                                \
+                default: CFP_DH_OLD_ADD(6, 7) break;                                               \
+            }                                                                                      \
+        } else {                                                                                   \
+            switch (I) {                                                                           \
+                case 0: CFP_DH_OLD_ADD(0, 0) break;                                                \
+                case 1: CFP_DH_OLD_ADD(1, 1) break;                                                \
+                case 2: CFP_DH_OLD_ADD(2, 2) break;                                                \
+                case 3: CFP_DH_OLD_ADD(3, 3) break;                                                \
+                case 4: CFP_DH_OLD_ADD(4, 4) break;                                                \
+                case 5: CFP_DH_OLD_ADD(5, 5) break;                                                \
+                case 6: CFP_DH_OLD_ADD(6, 6) break;                                                \
+                default: CFP_DH_OLD_ADD(7, 7) break;                                               \
+            }                                                                                      \
+        }                                                                                          \
+    } while (0)
 
     float raw[2][8];
     u4 wb[3];
@@ -388,13 +425,14 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     __syncthreads();
     u4 b[2][2];
     frag_load(0, 0, b[0]);
-    for (int s = 0; s < steps; s++) {
-        const int buf = s & 1;
-        // raw[s & 1] held step s (already split): refill it two steps ahead
-        if (s & 1) a_load(min(s + 2, last), raw[1]);
+    // par = s & 1 as a literal at every call: it selects registers
+    auto k_step = [&](int s, const int par) __attribute__((always_inline)) {
+        const int buf = par;
+        // raw[par] held step s (already split): refill it two steps ahead
+        if (par) a_load(min(s + 2, last), raw[1]);
         else a_load(min(s + 2, last), raw[0]);
         u4 ns[3];
-        if (s & 1) a_parts(raw[0], ns);
+        if (par) a_parts(raw[0], ns);
         else a_parts(raw[1], ns);
 #pragma unroll
         for (int q = 0; q < 12; q++) {
@@ -418,7 +456,29 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             }
         }
         as[0] = ns[0]; as[1] = ns[1]; as[2] = ns[2];
+    };
+    int s0 = 0;
+    if (spread) {
+        // the first steps as straight-line code: the tile an old value is added to is a
+        // compile-time register index
+#pragma unroll
+        for (int i = 0; i <= kSpreadMax; i++) {
+            if (i > spread_steps) break;
+            if (i > 0) CFP_DH_OLD_ADD_AT(i - 1);
+            if (i < spread_steps) old_fetch(i);
+            k_step(i, i & 1);
+        }
+        s0 = spread_steps + 1;
+        static_assert((kSpreadMax + 1) % 2 == 1, "the loop below goes on with an odd step");
+        if (s0 < steps) k_step(s0, 1);
+        s0++;
     }
+    int sr = s0;   // even
+    for (; sr + 1 < steps; sr += 2) {
+        k_step(sr, 0);
+        k_step(sr + 1, 1);
+    }
+    if (sr < steps) k_step(sr, 0);
     if (O16) {
         // the swap involves every lane of the wavefront: it comes before the early exit
 #pragma unroll
@@ -441,6 +501,9 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             o_lane[(size_t)acc_row(r) * ldc + 32 * t] = acc[t][r];
 }
 
+#undef CFP_DH_OLD_ADD_AT
+#undef CFP_DH_OLD_ADD
+
 constexpr int kDhMaxK = CFP_GRU;
 constexpr size_t kDhMirrorBytes = (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4);   // 1.125 MiB
 
@@ -458,6 +521,8 @@ static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const
     CFP_REQUIRE((!a16 && !o16) || terms == 1,
                 "k_dh_x9: bf16-stored operands need the bf16-input mode");
     CFP_REQUIRE(!o16 || ldc % 2 == 0, "k_dh_x9: a bf16 result needs an even row length");
+    // the old contents are fetched during the first nine K steps
+    CFP_REQUIRE(!accumulate || K >= 160, "k_dh_x9: accumulating needs K >= 160 (got %d)", K);
     CFP_REQUIRE(g_w_x9, "k_dh_x9: no mirror buffer for W");
     const int total = (K / 16) * kDhFrags * 64;
     hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, B, sk, su, g_w_x9,
