@@ -442,17 +442,18 @@ __global__ __launch_bounds__(kT16Threads, 1) void k_policy_forward_t16(FwdArgs a
     // ---- the draw, sixteen lanes per env (sample_row.h), and the step counter's bump ---------
     if (a.s_act) {   // uniform over the launch
         __syncthreads();
-        // The ticket first: its round trip runs under the draw.  Every lane's read of the
-        // counter (draw_step, the kernel's first load) has returned: loads return in
-        // order, and younger ones fed the MFMAs in front of the barriers above.
-        unsigned ticket_no = 0u;
-        if (tid == 0) ticket_no = take_ticket(a.s_ticket);
         const int sub = tid % kSampleLanes, slot = tid / kSampleLanes;
         const bool live = slot < kT16Envs;
         const float* lp = s_logit + (live ? slot : 0) * CFP_AV;
         float* px = s_expo + (live ? slot : 0) * kMaxActions;
         const float mx = sample_spread(lp, px, CFP_ACTIONS, sub, live);
         __syncthreads();
+        // The ticket behind the last barrier (a barrier waits for the atomic's return): its
+        // round trip runs under the scan of the draw.  Every lane's read of the counter
+        // (draw_step, the kernel's first load) has returned: loads return in order, and
+        // younger ones fed the MFMAs in front of the barriers above.
+        unsigned ticket_no = 0u;
+        if (tid == 0) ticket_no = take_ticket(a.s_ticket);
         if (live && sub == 0)
             sample_draw<CFP_ACTIONS>(lp, px, mx, CFP_ACTIONS, (int)e0 + slot, a.s_seed, draw_step,
                         a.s_env_actions, a.s_act, a.s_logp, a.s_value);
