@@ -344,8 +344,6 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
         b[1] = stage[buf][6 * tp + 3 + j][lane];
     };
 
-    // accumulating form: the accumulators start from dh, all 128 loads in flight at
-    // once under the prologue's own loads, and the epilogue is stores only
     static_assert(TERMS == 1 || !O16, "bf16 storage goes with bf16 inputs");
     float* o_lane = dh + (size_t)(cbc + 4 * g) * ldc + n;
     // O16: the lane's dword of a pair of tiles (ldc even, n - odd even: 4-byte aligned)
@@ -354,11 +352,12 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
         reinterpret_cast<uint16_t*>(dh) + (size_t)(cbc + 4 * g) * ldc + (odd ? 32 + n - 1 : n));
     // The accumulators start at zero; the old contents of dh are fetched one 32-unit tile
     // (O16: one pair of tiles) per K step during the first steps and added a step later, so
-    // that the fetch runs under the MFMAs instead of in front of them.  Short K: all of
-    // it up front.
+    // that the fetch runs under the MFMAs instead of in front of them (every workgroup of
+    // a round starts at once: loads in front of the loop are a phase nothing runs beside).
+    // The epilogue is stores only.  The launcher asks for enough K steps.
     constexpr int kSpreadMax = O16 ? 4 : 8;
     constexpr int spread_steps = kSpreadMax;
-    const bool spread = accumulate != 0;   // the launcher asks for steps > spread_steps
+    const bool spread = accumulate != 0;
     f16v acc[8];
 #pragma unroll
     for (int t = 0; t < 8; t++)
