@@ -223,10 +223,7 @@ __device__ __forceinline__ void sweep_store(unsigned, unsigned lo8, void* gates,
             : "memory");
 }
 
-#ifndef CFP_SWEEP_EPB
-#define CFP_SWEEP_EPB 1
-#endif
-constexpr int kSweepEnvs = CFP_SWEEP_EPB;   // envs (wavefronts) per workgroup
+constexpr int kSweepEnvs = 1;   // envs (wavefronts) per workgroup: the best of 1 / 2 / 4
 template <bool TWO_GRADS, bool HIGHWAY, bool G16>
 __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
