@@ -328,14 +328,17 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             parts_of<TERMS>(v, p);
         }
     };
+    // wave w stages the three parts of W for (tile pair w / 2, half w % 2); with one
+    // product only the first part is used
+    constexpr int kWParts = TERMS == 1 ? 1 : 3;
     const u4* w_lane = wm + (size_t)3 * w * 64 + lane;
     auto w_load = [&](int s, u4 (&b)[3]) {
 #pragma unroll
-        for (int i = 0; i < 3; i++) b[i] = w_lane[((size_t)s * kDhFrags + i) * 64];
+        for (int i = 0; i < kWParts; i++) b[i] = w_lane[((size_t)s * kDhFrags + i) * 64];
     };
     auto w_store = [&](int buf, const u4 (&b)[3]) {
 #pragma unroll
-        for (int i = 0; i < 3; i++) stage[buf][3 * w + i][lane] = b[i];
+        for (int i = 0; i < kWParts; i++) stage[buf][3 * w + i][lane] = b[i];
     };
     // group q of a step: unit tiles 2*(q/3), 2*(q/3)+1, part q%3 of W
     auto frag_load = [&](int buf, int q, u4 (&b)[2]) {
@@ -356,7 +359,6 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     // a round starts at once: loads in front of the loop are a phase nothing runs beside).
     // The epilogue is stores only.  The launcher asks for enough K steps.
     constexpr int kSpreadMax = O16 ? 4 : 8;
-    constexpr int spread_steps = kSpreadMax;
     const bool spread = accumulate != 0;
     f16v acc[8];
 #pragma unroll
@@ -411,28 +413,37 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
         }                                                                                          \
     } while (0)
 
-    float raw[2][8];
-    u4 wb[3];
+    // dpre is requested kAhead K steps ahead of its MFMAs.  The split kernels are bound by
+    // the matrix pipe and two steps cover the latency; with one product per operand pair
+    // the kernel is bound by HBM, and a workgroup (the only one on its CU) has to keep
+    // about 48-64 KiB in flight: 6 steps of 8 KiB (bf16 dpre) or 4 of 16 KiB (fp32 dpre).
+    // Loads return in issue order, so W (an L2 hit) comes back no sooner than the dpre
+    // request in front of it: W travels through registers equally far ahead.
+    constexpr int kAhead = TERMS != 1 ? 2 : (A16 ? 6 : 4);
+    constexpr int kWAhead = TERMS != 1 ? 1 : kAhead;   // W(s + 1) is staged during step s
+    static_assert(kAhead % kWAhead == 0, "one literal selects both rings");
+    float raw[kAhead][8];
+    u4 wring[kWAhead][3];
     const int last = steps - 1;
-    w_load(0, wb);
-    a_load(0, raw[0]);
-    a_load(min(1, last), raw[1]);
-    w_store(0, wb);
-    w_load(min(1, last), wb);
+#pragma unroll
+    for (int j = 0; j < kWAhead; j++) w_load(min(j, last), wring[j]);
+#pragma unroll
+    for (int j = 0; j < kAhead; j++) a_load(min(j, last), raw[j]);
+    w_store(0, wring[0]);
+    w_load(min(kWAhead, last), wring[0]);
     u4 as[3];
     a_parts(raw[0], as);
     __syncthreads();
     u4 b[2][2];
     frag_load(0, 0, b[0]);
-    // par = s & 1 as a literal at every call: it selects registers
-    auto k_step = [&](int s, const int par) __attribute__((always_inline)) {
-        const int buf = par;
-        // raw[par] held step s (already split): refill it two steps ahead
-        if (par) a_load(min(s + 2, last), raw[1]);
-        else a_load(min(s + 2, last), raw[0]);
+    // slot = s % kAhead as a literal at every call: it selects registers
+    auto k_step = [&](int s, const int slot) __attribute__((always_inline)) {
+        const int buf = slot & 1;
+        static_assert(kAhead % 2 == 0, "the W stage buffer follows the slot's parity");
+        // raw[slot] held step s (already split): refill it kAhead steps ahead
+        a_load(min(s + kAhead, last), raw[slot]);
         u4 ns[3];
-        if (par) a_parts(raw[0], ns);
-        else a_parts(raw[1], ns);
+        a_parts(raw[(slot + 1) % kAhead], ns);
 #pragma unroll
         for (int q = 0; q < 12; q++) {
             const int cur = q & 1, nxt = cur ^ 1;
@@ -441,9 +452,9 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             } else {
                 // next step's W parts: everyone is past its reads of the other buffer
                 // (they precede the previous barrier)
-                w_store(buf ^ 1, wb);
+                w_store(buf ^ 1, wring[(slot + 1) % kWAhead]);   // W(s + 1)
                 __syncthreads();
-                w_load(min(s + 2, last), wb);
+                w_load(min(s + 1 + kWAhead, last), wring[(slot + 1) % kWAhead]);
                 frag_load(buf ^ 1, 0, b[nxt]);
             }
             const int t = 2 * (q / 3);
@@ -459,25 +470,25 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     int s0 = 0;
     if (spread) {
         // the first steps as straight-line code: the tile an old value is added to is a
-        // compile-time register index
+        // compile-time register index.  The peel runs on to a multiple of kAhead, where
+        // the loop below takes over with slot 0.
+        constexpr int kPeel = (kSpreadMax + 1 + kAhead - 1) / kAhead * kAhead;
 #pragma unroll
-        for (int i = 0; i <= kSpreadMax; i++) {
-            if (i > spread_steps) break;
-            if (i > 0) CFP_DH_OLD_ADD_AT(i - 1);
-            if (i < spread_steps) old_fetch(i);
-            k_step(i, i & 1);
+        for (int i = 0; i < kPeel; i++) {
+            if (i > 0 && i <= kSpreadMax) CFP_DH_OLD_ADD_AT(i - 1);
+            if (i < kSpreadMax) old_fetch(i);
+            if (i <= kSpreadMax || i < steps) k_step(i, i % kAhead);   // steps > kSpreadMax
         }
-        s0 = spread_steps + 1;
-        static_assert((kSpreadMax + 1) % 2 == 1, "the loop below goes on with an odd step");
-        if (s0 < steps) k_step(s0, 1);
-        s0++;
+        s0 = kPeel;
     }
-    int sr = s0;   // even
-    for (; sr + 1 < steps; sr += 2) {
-        k_step(sr, 0);
-        k_step(sr + 1, 1);
+    int sr = s0;   // a multiple of kAhead
+    for (; sr + kAhead <= steps; sr += kAhead) {
+#pragma unroll
+        for (int j = 0; j < kAhead; j++) k_step(sr + j, j);
     }
-    if (sr < steps) k_step(sr, 0);
+#pragma unroll
+    for (int j = 0; j < kAhead - 1; j++)
+        if (sr + j < steps) k_step(sr + j, j);
     if (O16) {
         // the swap involves every lane of the wavefront: it comes before the early exit
 #pragma unroll
