@@ -158,7 +158,7 @@ struct cfp_trainer {
     // it and the caller's, see cfp_train_backward)
     hipStream_t st2 = nullptr;
     hipEvent_t ev_dh[CFP_MAX_LAYERS] = {};
-    hipEvent_t ev_join = nullptr;
+    hipEvent_t ev_join = nullptr, ev_head = nullptr;
     // GEMM scratch owned by this trainer: `sw` for the chain's GEMMs, and a split
     // workspace per layer for the gate dW GEMMs that run beside the chain
     SeamWork sw;
@@ -187,6 +187,7 @@ void cfp_train_destroy(cfp_trainer* tr) {
     for (hipEvent_t e : tr->ev_dh)
         if (e) (void)hipEventDestroy(e);
     if (tr->ev_join) (void)hipEventDestroy(tr->ev_join);
+    if (tr->ev_head) (void)hipEventDestroy(tr->ev_head);
     if (tr->texec) (void)hipGraphExecDestroy(tr->texec);
     if (tr->tgraph) (void)hipGraphDestroy(tr->tgraph);
     if (tr->st2) (void)hipStreamDestroy(tr->st2);
@@ -285,7 +286,8 @@ int cfp_train_create(cfp_trainer** out, cfp_policy* p, int T, const cfp_ppo_conf
     }
     // default priority, as every stream of this library
     if (ok) ok = hipStreamCreateWithFlags(&tr->st2, hipStreamNonBlocking) == hipSuccess &&
-                 hipEventCreateWithFlags(&tr->ev_join, hipEventDisableTiming) == hipSuccess;
+                 hipEventCreateWithFlags(&tr->ev_join, hipEventDisableTiming) == hipSuccess &&
+                 hipEventCreateWithFlags(&tr->ev_head, hipEventDisableTiming) == hipSuccess;
     for (int l = 0; ok && l < tr->L; l++)
         ok = hipEventCreateWithFlags(&tr->ev_dh[l], hipEventDisableTiming) == hipSuccess;
     if (ok) ok = hipMemcpy(tr->d_lr, &cfg->lr, 4, hipMemcpyHostToDevice) == hipSuccess &&
@@ -518,7 +520,17 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         ha.clip = tr->cfg.clip; ha.vf = tr->cfg.vf; ha.ent_coef = tr->d_ent;
         if (launch_head(ha, st)) return 1;
         if (launch_fold_f64(tr->block_loss, head_blocks(cols), 3, tr->loss_acc, true, st)) return 1;
-        // dh3 = [dlogits | dvalue] . [W_a ; W_v]; dW_a and dW_v from one GEMM; bias sums
+        // dh3 = [dlogits | dvalue] . [W_a ; W_v]; dW_a and dW_v from one GEMM; bias sums.
+        // Only dh3 is on the way to the layers: with the split kernels the heads' own
+        // gradients go to the second stream and run beside the top layer's sweep.
+        const int terms = gemm_split_terms();
+        const bool overlap = terms >= 1 && gemm_dw_x9_ok(G, cols);
+        hipStream_t hs = st;
+        if (overlap) {
+            CFP_HIP_TRY(hipEventRecord(tr->ev_head, st));
+            CFP_HIP_TRY(hipStreamWaitEvent(tr->st2, tr->ev_head, 0));
+            hs = tr->st2;
+        }
         // (bf16 storage: the three dh buffers hold bf16 as well)
         if (st16) {
             if (gemm_dh_x9(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, 1,
@@ -529,23 +541,24 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         }
         if (st16) {
             if (gemm_dw_x9(A + 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L), 1, tr->sw,
-                           st, A, g + CFP_OFF_W_V(L), false, true))
+                           hs, A, g + CFP_OFF_W_V(L), false, true))
                 return 1;
         } else if (gemm_dw_two(A, 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L),
-                               g + CFP_OFF_W_V(L), tr->sw, st)) {
+                               g + CFP_OFF_W_V(L), tr->sw, hs)) {
             return 1;
         }
-        if (colsum_into(tr, tr->dlogits, kHeadLd, g + CFP_OFF_B_A(L), A, cols, st)) return 1;
-        if (colsum_into(tr, tr->dlogits + A, kHeadLd, g + CFP_OFF_B_V(L), 1, cols, st)) return 1;
+        if (colsum_into(tr, tr->dlogits, kHeadLd, g + CFP_OFF_B_A(L), A, cols, hs)) return 1;
+        if (colsum_into(tr, tr->dlogits + A, kHeadLd, g + CFP_OFF_B_V(L), 1, cols, hs)) return 1;
         // ---- reverse MinGRU layers
         // With the split kernels the dependent chain  reverse(l) -> dh(l) -> reverse(l-1)
         // hops between two streams: dW(l) is enqueued right behind dh(l) on the stream
         // that ran it, and the next layer's chain on the other stream behind an event.
         // dW(l) so starts first and takes its one workgroup per CU; the HBM-bound
         // reverse kernel of the next layer then fills the wave slots that are left and
-        // runs under it.  Every dW has a split workspace of its own.
-        const int terms = gemm_split_terms();
-        const bool overlap = terms >= 1 && gemm_dw_x9_ok(G, cols);
+        // runs under it.  Every dW has a split workspace of its own.  (The heads' gradients
+        // above share the trainer's workspace and column-sum scratch with dW_enc and
+        // db_enc below: whichever stream those end up on has by then waited for an event
+        // recorded on the second stream behind them.)
         hipStream_t chain = st, other = tr->st2;
         const float* dh_gemm = tr->dh3b;
         const float* dh_extra = nullptr;
