@@ -164,44 +164,58 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
 #pragma unroll
         for (int r = 0; r < 16; r++) acc[b][r] = 0.0f;
 
+    // How far ahead the operands are requested.  The split kernels are bound by the matrix
+    // pipe: x three K steps and dpre one iteration ahead cover the latency.  With one
+    // product per operand pair an iteration is 16 MFMAs and the kernel is bound by HBM:
+    // requests one iteration ahead make an iteration last one memory latency, so x goes
+    // seven K steps and dpre two iterations ahead.
+    constexpr int kXRing = TERMS == 1 ? 8 : 4, kXAhead = kXRing - 1;
+    constexpr int kDpAhead = TERMS == 1 ? 2 : 1;
     if (it0 < it1) {
-        float d0[8], d1[8];
-        float raw[4][8];
-        if (DP16) {
-            dp_load16(it0, d0);
-        } else {
-            dp_load(it0, pk, d0);
-            dp_load(it0, pk + 2, d1);
-        }
-        x_load(it0, 0, raw[0]);
-        x_load(it0, 1, raw[1]);
-        x_load(it0, 2, raw[2]);
-        if (DP16) {
-            dp_store16(it0, 0, d0);
-        } else {
-            dp_store(it0, pk, 0, d0);
-            dp_store(it0, pk + 2, 0, d1);
-        }
+        const int itl = it1 - 1;
+        float d0[kDpAhead][8], d1[kDpAhead][8];   // dpre of iteration it0 + r in slot r % kDpAhead
+        float raw[kXRing][8];                     // x of K step G = 4 r + ks in slot G % kXRing
+        auto dp_fetch = [&](int it, float (&e0)[8], float (&e1)[8]) __attribute__((always_inline)) {
+            if (DP16) {
+                dp_load16(it, e0);
+            } else {
+                dp_load(it, pk, e0);
+                dp_load(it, pk + 2, e1);
+            }
+        };
+        auto dp_stage = [&](int it, int buf, const float (&e0)[8], const float (&e1)[8])
+                            __attribute__((always_inline)) {
+            if (DP16) {
+                dp_store16(it, buf, e0);
+            } else {
+                dp_store(it, pk, buf, e0);
+                dp_store(it, pk + 2, buf, e1);
+            }
+        };
+#pragma unroll
+        for (int j = 0; j < kDpAhead; j++) dp_fetch(min(it0 + j, itl), d0[j], d1[j]);
+#pragma unroll
+        for (int j = 0; j < kXAhead; j++) x_load(min(it0 + j / 4, itl), j % 4, raw[j]);
+        dp_stage(it0, 0, d0[0], d1[0]);
         __syncthreads();
         u4 a[2][6];
         frag_load(0, 0, 0, a[0]);
         u4 bs[3];
         x_parts(raw[0], bs);
-        for (int it = it0; it < it1; it++) {
-            const int buf = (it - it0) & 1;
-            const int itn = min(it + 1, it1 - 1);
-            if (DP16) {
-                dp_load16(itn, d0);
-            } else {
-                dp_load(itn, pk, d0);
-                dp_load(itn, pk + 2, d1);
-            }
+        // par = (it - it0) & 1, a literal at every call of the one-product kernels, where it
+        // selects registers; the LDS buffer everywhere
+        auto iteration = [&](int it, const int par) __attribute__((always_inline)) {
+            const int buf = par;
+            const int itn = min(it + 1, itl);
+            // the slot of this iteration's dpre (staged during the previous one)
+            dp_fetch(min(it + kDpAhead, itl), d0[par % kDpAhead], d1[par % kDpAhead]);
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                if (ks < 1) x_load(it, ks + 3, raw[ks + 3]);
-                else x_load(itn, ks - 1, raw[ks - 1]);
+                const int G = 4 * par + ks;   // K step modulo the ring
+                x_load(min(it + (ks + kXAhead) / 4, itl), (ks + kXAhead) % 4,
+                       raw[(G + kXAhead) % kXRing]);
                 u4 ns[3];
-                x_parts(raw[(ks + 1) & 3], ns);
+                x_parts(raw[(G + 1) % kXRing], ns);
 #pragma unroll
                 for (int pr = 0; pr < 2; pr++) {
                     const int cur = pr, nxt = pr ^ 1;
@@ -212,12 +226,7 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
                     } else {
                         // this wave's last read of the current buffer is in flight or
                         // done; the barrier's wait covers it
-                        if (DP16) {
-                            dp_store16(itn, buf ^ 1, d0);
-                        } else {
-                            dp_store(itn, pk, buf ^ 1, d0);
-                            dp_store(itn, pk + 2, buf ^ 1, d1);
-                        }
+                        dp_stage(itn, buf ^ 1, d0[(par + 1) % kDpAhead], d1[(par + 1) % kDpAhead]);
                         __syncthreads();
                         frag_load(buf ^ 1, 0, 0, a[nxt]);
                     }
@@ -233,6 +242,19 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
                 }
                 bs[0] = ns[0]; bs[1] = ns[1]; bs[2] = ns[2];
             }
+        };
+        if (TERMS == 1) {
+            int it = it0;
+            for (; it + 1 < it1; it += 2) {
+                iteration(it, 0);
+                iteration(it + 1, 1);
+            }
+            if (it < it1) iteration(it, 0);
+        } else {
+            // four ring slots and one dpre slot: the parity only selects the LDS buffer.
+            // (Not unrolled: the split kernels have to stay within 208 registers, or
+            // the reverse sweep that runs under them finds no room on the CU.)
+            for (int it = it0; it < it1; it++) iteration(it, (it - it0) & 1);
         }
     }
     // undo the even / odd permutations of bf16-stored operands
