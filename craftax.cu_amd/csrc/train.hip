@@ -465,9 +465,10 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         const bool fused = cfp_get_gemm_bf16() == 0 || cfp_get_gemm_split() != 0;
         // bf16 storage: pre / dpre, the layer inputs x[0..L] and the three dh buffers are
         // bf16 arrays inside the same buffers; needs the record-fed dW_enc and the split
-        // kernels
+        // kernels (whole 32-column blocks); a window that does not fit runs with fp32
+        // storage
         const bool st16 = tr->bf16_store && cfp_get_gemm_bf16() != 0 && cfp_get_gemm_split() != 0 &&
-                          dw_enc_records_ok(mb);
+                          dw_enc_records_ok(mb) && cols % 32 == 0;
         if (fused) {
             FwdArgs fa{};
             fill_forward_weights(p, fa);

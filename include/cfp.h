@@ -433,8 +433,9 @@ void* cfp_train_buffer(cfp_trainer* tr, int which);
  * as bf16, the dW / dh GEMMs take those as their operands unconverted, and the
  * hidden-state gradients between the layers (the dh buffers) are bf16 as well -- half
  * the bytes of the kernels that bound the bf16 update.  r_state, the head rows and
- * every weight gradient stay fp32.  Needs envs per minibatch % 8 == 0 (otherwise the
- * update runs with fp32 storage).  Off by default. */
+ * every weight gradient stay fp32.  Needs envs per minibatch % 8 == 0 and window
+ * columns (steps x envs) % 32 == 0; a window that does not fit runs with fp32 storage.
+ * Off by default. */
 int cfp_train_set_bf16_storage(cfp_trainer* tr, int on);
 int cfp_train_bf16_storage(const cfp_trainer* tr);
 int cfp_train_window(const cfp_trainer* tr);
