@@ -241,6 +241,10 @@ __global__ __launch_bounds__(kX9Threads) void k_dw_x9(
                         }
                 }
                 bs[0] = ns[0]; bs[1] = ns[1]; bs[2] = ns[2];
+                // six products: left free, the scheduler hoists enough of the next K steps'
+                // LDS reads to take 215 registers, and above 208 the reverse sweep that
+                // runs under this kernel finds no room on the CU
+                if (TERMS == 6) __builtin_amdgcn_sched_barrier(0);
             }
         };
         if (TERMS == 1) {
