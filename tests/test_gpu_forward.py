@@ -323,6 +323,13 @@ def test_config2_feature_matrix_at_65536(pkg, cuda):
     assert_close(av_a[idx].cpu().numpy()[:, ACTIONS], ref["values"], TOL_FP32, "config 2 values")
     assert_close(st_a[:, idx].cpu().numpy(), ref["state"], TOL_FP32, "config 2 state")
     assert_close(h3[idx].cpu().numpy(), ref["h3"], TOL_FP32, "config 2 h3")
+    # the sampled rows alone, as a batch of their own: the same bits
+    st_c = st0[:, idx].contiguous().clone()
+    h_c = torch.empty(idx.numel(), HIDDEN, device=cuda)
+    av_c = torch.empty(idx.numel(), av_a.shape[1], device=cuda)
+    pol.forward_features(x[idx].contiguous(), term[idx].contiguous(), st_c, h_enc=h_c, av=av_c)
+    torch.cuda.synchronize()
+    assert torch.equal(av_c, av_a[idx]) and torch.equal(st_c, st_a[:, idx]) and torch.equal(h_c, h_enc[idx])
     pol.close()
 
 
