@@ -58,8 +58,9 @@ __device__ __forceinline__ u4 byte_frag(const uint32_t (&d)[8]) {
     return f;
 }
 
-// D16: dh is a bf16 array (the update's bf16 storage): one product per byte.
-template <bool D16>
+// ONE: the bf16-input mode of the seam: the gradient is rounded to bf16 (nearest even), one
+// product per byte.  D16: dh is a bf16 array (the update's bf16 storage), which implies ONE.
+template <bool D16, bool ONE>
 __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
     const uint8_t* __restrict__ r_obs, const float* __restrict__ dh, float* __restrict__ part,
     int t0, int cols, int mb, int n_all, int env_start, int iters_per_split, int n_wg) {
@@ -116,7 +117,7 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
     };
     // hi / mid / lo parts of eight gradients; bf16 values are their own hi part
     auto dh_parts = [&](const float (&v)[8], u4& h, u4& m, u4& l) {
-        if (D16) {
+        if (ONE) {
             h = round_bf16x8(v);
             m = h;
             l = h;
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(kEgThreads) void k_dw_enc_bytes(
                     const int b = 2 * pr;
                     acc[b] = mfma16(a[cur][0], bh, acc[b]);
                     acc[b + 1] = mfma16(a[cur][1], bh, acc[b + 1]);
-                    if (!D16) {
+                    if (!ONE) {
                         acc[b] = mfma16(a[cur][0], bm, acc[b]);
                         acc[b + 1] = mfma16(a[cur][1], bm, acc[b + 1]);
                         acc[b] = mfma16(a[cur][0], bl, acc[b]);
@@ -254,11 +255,14 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
     const int n_wg = splits * kEgGroups;
     const int grid = (n_wg + kEgXcds - 1) / kEgXcds * kEgXcds;
     if (dh_bf16)
-        hipLaunchKernelGGL(k_dw_enc_bytes<true>, dim3(grid), dim3(kEgThreads), 0, st, r_obs, dh, work,
-                           t0, cols, mb, n_all, env_start, ips, n_wg);
+        hipLaunchKernelGGL((k_dw_enc_bytes<true, true>), dim3(grid), dim3(kEgThreads), 0, st, r_obs, dh,
+                           work, t0, cols, mb, n_all, env_start, ips, n_wg);
+    else if (gemm_split_terms() == 1)   // bf16 GEMM inputs: like every other GEMM of that mode
+        hipLaunchKernelGGL((k_dw_enc_bytes<false, true>), dim3(grid), dim3(kEgThreads), 0, st, r_obs,
+                           dh, work, t0, cols, mb, n_all, env_start, ips, n_wg);
     else
-        hipLaunchKernelGGL(k_dw_enc_bytes<false>, dim3(grid), dim3(kEgThreads), 0, st, r_obs, dh, work,
-                           t0, cols, mb, n_all, env_start, ips, n_wg);
+        hipLaunchKernelGGL((k_dw_enc_bytes<false, false>), dim3(grid), dim3(kEgThreads), 0, st, r_obs,
+                           dh, work, t0, cols, mb, n_all, env_start, ips, n_wg);
     const long count = (long)kEgFeat * CFP_HIDDEN;
     if (launch_splitk_reduce(dW, work, count, count, splits, st)) return 1;
     // rows 768..842: a GEMM of its own on other rows of dW, on the second stream and
