@@ -1,0 +1,141 @@
+"""ctypes/numpy helpers for the env-step tests: the exchange struct cfp_env_state
+(include/cfp_env.h) as a numpy dtype, the compiled reference (oracle/_ref) stepped env by
+env, and the host build of the library's step text (oracle/libcfenvhost.so).  Test
+infrastructure only."""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+
+L, M = 9, 48
+STATE_DTYPE = np.dtype([
+    ("player_position", "<i4", (2,)), ("player_level", "<i4"), ("player_direction", "<i4"),
+    ("player_health", "<f4"), ("player_food", "<i4"), ("player_drink", "<i4"),
+    ("player_energy", "<i4"), ("player_mana", "<i4"), ("is_sleeping", "<i4"), ("is_resting", "<i4"),
+    ("player_recover", "<f4"), ("player_hunger", "<f4"), ("player_thirst", "<f4"),
+    ("player_fatigue", "<f4"), ("player_recover_mana", "<f4"),
+    ("player_xp", "<i4"), ("player_dexterity", "<i4"), ("player_strength", "<i4"),
+    ("player_intelligence", "<i4"),
+    ("wood", "<i4"), ("stone", "<i4"), ("coal", "<i4"), ("iron", "<i4"), ("diamond", "<i4"),
+    ("sapling", "<i4"), ("pickaxe", "<i4"), ("sword", "<i4"), ("bow", "<i4"), ("arrows", "<i4"),
+    ("armour", "<i4", (4,)), ("torches", "<i4"), ("ruby", "<i4"), ("sapphire", "<i4"),
+    ("potions", "<i4", (6,)), ("books", "<i4"),
+    ("mob_position", "<i4", (5, L, 3, 2)), ("mob_health", "<f4", (5, L, 3)),
+    ("mob_attack_cooldown", "<i4", (5, L, 3)), ("mob_type_id", "<i4", (5, L, 3)),
+    ("mob_mask", "<i4", (5, L, 3)),
+    ("mob_projectile_directions", "<i4", (L, 3, 2)), ("player_projectile_directions", "<i4", (L, 3, 2)),
+    ("growing_plants_positions", "<i4", (10, 2)), ("growing_plants_age", "<i4", (10,)),
+    ("growing_plants_mask", "<i4", (10,)),
+    ("potion_mapping", "<i4", (6,)), ("learned_spells", "<i4", (2,)),
+    ("sword_enchantment", "<i4"), ("bow_enchantment", "<i4"), ("armour_enchantments", "<i4", (4,)),
+    ("boss_progress", "<i4"), ("boss_timesteps_to_spawn_this_round", "<i4"),
+    ("light_level", "<f4"), ("state_rng", "<u4", (2,)), ("timestep", "<i4"),
+    ("down_ladders", "<i4", (L, 2)), ("up_ladders", "<i4", (L, 2)),
+    ("monsters_killed", "<i4", (L,)), ("chests_opened", "<i4", (L,)),
+    ("rng_key", "<u4", (2,)),
+    ("achievements", "u1", (67,)), ("pad_", "u1", (5,)),
+    ("mob_bits", "<u8", (L, M)), ("spawn_all_bits", "<u8", (L, M)),
+    ("spawn_grave_bits", "<u8", (L, M)), ("spawn_water_bits", "<u8", (L, M)),
+    ("map", "u1", (L, M, M)), ("item_map", "u1", (L, M, M)), ("light_map", "u1", (L, M, M)),
+])
+FLOAT_FIELDS = [n for n in STATE_DTYPE.names if STATE_DTYPE[n].base == np.dtype("<f4")]
+
+
+def ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def diff_fields(a, b):
+    """Names of the fields in which two state arrays differ (floats by bit pattern)."""
+    out = []
+    for n in STATE_DTYPE.names:
+        if n == "pad_":
+            continue
+        x, y = a[n], b[n]
+        if x.dtype == np.float32:
+            x, y = x.view(np.uint32), y.view(np.uint32)
+        if not np.array_equal(x, y):
+            out.append(n)
+    return out
+
+
+class Ref:
+    """oracle/_ref/libcfref.so: the reference's own env, one global vector of envs."""
+
+    def __init__(self):
+        path = os.path.join(ROOT, "oracle", "_ref", "libcfref.so")
+        if not os.path.exists(path):
+            raise FileNotFoundError(path)
+        self.lib = lib = C.CDLL(path)
+        lib.cfref_init.argtypes = [C.c_int, C.c_uint64]
+        lib.cfref_exchange_bytes.restype = C.c_size_t
+        lib.cfref_export_state.argtypes = [C.c_int, C.c_void_p]
+        lib.cfref_import_state.argtypes = [C.c_int, C.c_void_p]
+        lib.cfref_next_action.argtypes = [C.c_int]
+        lib.cfref_next_action.restype = C.c_float
+        lib.cfref_step_env.argtypes = [C.c_int, C.c_float, C.c_void_p, C.POINTER(C.c_float), C.c_void_p]
+        lib.cfref_step_env.restype = C.c_int
+        lib.cfref_light_level.argtypes = [C.c_int]
+        lib.cfref_light_level.restype = C.c_float
+        lib.cfref_fuzz_state.argtypes = [C.c_int, C.c_uint64]
+        assert lib.cfref_exchange_bytes() == STATE_DTYPE.itemsize
+
+    def init(self, n, seed):
+        self.n = n
+        self.lib.cfref_init(n, seed)
+
+    def export(self, envs=None):
+        envs = range(self.n) if envs is None else envs
+        out = np.zeros(len(envs), STATE_DTYPE)
+        for k, e in enumerate(envs):
+            self.lib.cfref_export_state(e, C.c_void_p(out[k:k + 1].ctypes.data))
+        return out
+
+    def import_(self, env, state):
+        s = np.ascontiguousarray(state.reshape(1))
+        self.lib.cfref_import_state(env, ptr(s))
+
+    def next_actions(self):
+        return np.array([self.lib.cfref_next_action(e) for e in range(self.n)], np.float32)
+
+    def step(self, actions):
+        """Steps every env; returns (final states before any reset, rewards, terminals,
+        reset keys).  Afterwards the reference holds the post-reset states."""
+        final = np.zeros(self.n, STATE_DTYPE)
+        rew = np.zeros(self.n, np.float32)
+        term = np.zeros(self.n, np.float32)
+        keys = np.zeros((self.n, 2), np.uint32)
+        r = C.c_float()
+        for e in range(self.n):
+            d = self.lib.cfref_step_env(e, float(actions[e]), C.c_void_p(final[e:e + 1].ctypes.data),
+                                        C.byref(r), C.c_void_p(keys[e:e + 1].ctypes.data))
+            rew[e] = r.value
+            term[e] = d
+        return final, rew, term, keys
+
+
+class HostStep:
+    """oracle/libcfenvhost.so: env_logic.h compiled for the host."""
+
+    def __init__(self):
+        path = os.path.join(ROOT, "oracle", "libcfenvhost.so")
+        self.lib = lib = C.CDLL(path)
+        lib.cfhost_state_bytes.restype = C.c_size_t
+        assert lib.cfhost_state_bytes() == STATE_DTYPE.itemsize
+        lib.cfhost_light_table.argtypes = [C.c_void_p, C.c_int]
+        lib.cfhost_step.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5
+        lib.cfhost_derive_spawn_planes.argtypes = [C.c_void_p, C.c_int]
+        self.light = np.zeros(100001, np.float32)
+        lib.cfhost_light_table(ptr(self.light), len(self.light))
+
+    def step(self, states, actions):
+        n = len(states)
+        rew = np.zeros(n, np.float32)
+        term = np.zeros(n, np.float32)
+        keys = np.zeros((n, 2), np.uint32)
+        a = np.ascontiguousarray(actions, np.float32)
+        self.lib.cfhost_step(ptr(states), n, ptr(a), ptr(self.light), ptr(rew), ptr(term), ptr(keys))
+        return rew, term, keys
