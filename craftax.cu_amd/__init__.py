@@ -8,7 +8,9 @@ the shared library and fails if it has not been built.
 from . import _lib
 from . import policy
 from .policy import Policy, Trainer, lib
+from . import env
+from .env import Env
 
 lib()  # fail at import time, not at first use, when the HIP library is missing
 
-__all__ = ["Policy", "Trainer", "policy", "lib", "_lib"]
+__all__ = ["Policy", "Trainer", "Env", "policy", "env", "lib", "_lib"]

@@ -91,6 +91,25 @@ PROTOTYPES = {
     "cfp_train_loss": (C.c_int, [vp, vp, vp]),
     "cfp_synth_classic_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),
     "cfp_synth_records": (C.c_int, [vp, C.c_int, C.c_uint64, C.c_uint64, vp]),
+    # include/cfp_env.h
+    "cfp_env_state_bytes": (C.c_size_t, []),
+    "cfp_env_create": (C.c_int, [C.POINTER(vp), C.c_int, C.c_int]),
+    "cfp_env_destroy": (None, [vp]),
+    "cfp_env_num_envs": (C.c_int, [vp]),
+    "cfp_env_pool_size": (C.c_int, [vp]),
+    "cfp_env_import": (C.c_int, [vp, C.c_int, C.c_int, vp]),
+    "cfp_env_export": (C.c_int, [vp, C.c_int, C.c_int, vp]),
+    "cfp_env_pool_import": (C.c_int, [vp, C.c_int, C.c_int, vp]),
+    "cfp_env_light_table": (C.c_int, [vp, C.c_int]),
+    "cfp_env_step": (C.c_int, [vp, vp, vp, vp, vp]),
+    "cfp_env_seed_actions": (C.c_int, [vp, C.c_uint64, vp]),
+    "cfp_env_reset_count": (vp, [vp]),
+    "cfp_env_reset_list": (vp, [vp]),
+    "cfp_env_fetch_resets": (C.c_int, [vp, vp, C.c_int, C.POINTER(C.c_int), vp]),
+    "cfp_env_reset_from_pool": (C.c_int, [vp, vp]),
+    "cfp_env_view": (C.c_int, [vp, vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp),
+                               C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "cfp_env_record_obs": (C.c_int, [vp, vp, vp]),
 }
 
 

@@ -7,7 +7,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libcfpolicy.so")
-SOURCES = ["policy_forward.hip", "policy_forward_bf16.hip", "policy_forward_t16.hip", "cfp_api.hip", "gemm.hip", "record.hip", "train.hip", "ppo_kernels.hip", "rollout.hip", "enc_grad.hip", "gemm_x9.hip"]
+SOURCES = ["policy_forward.hip", "policy_forward_bf16.hip", "policy_forward_t16.hip", "cfp_api.hip", "gemm.hip", "record.hip", "train.hip", "ppo_kernels.hip", "rollout.hip", "enc_grad.hip", "gemm_x9.hip", "env_step.hip"]
 ARCH = "gfx950"
 
 

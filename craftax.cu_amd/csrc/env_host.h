@@ -203,7 +203,7 @@ struct HostStore {
     }
     void set_plant_age(int i, int a) { st->growing_plants_age[i] = a; }
     void open_level(int l) { lvl = l; }
-    float light_at(int t) const { return light[t]; }
+    float light_at(int t) const { return light[t < kMaxTimesteps ? t : kMaxTimesteps]; }
 };
 
 // c_step_gameplay (craftax_full.c:3981-4011) without the reset, on one host state

@@ -22,6 +22,11 @@
 
 #include <stdint.h>
 
+#if defined(__clang__)
+// strict per-operation fp32 from here to the end of the translation unit (gcc: -ffp-contract=off)
+#pragma clang fp contract(off)
+#endif
+
 #if defined(__HIPCC__)
 #define CFE_FN __host__ __device__ __forceinline__
 #else
@@ -1006,7 +1011,7 @@ CFE_FN Vec2 random_step(uint64_t key, int choices) {  // craftax_update_mobs_dir
 template <class S>
 CFE_FN void move_melee(S& s, Hot& h, uint64_t& rng, int i) {
     if (!s.m_mask(P_MELEE, i)) return;
-    const int l = h.level;
+    const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_MELEE, i), c0 = s.m_col(P_MELEE, i), cd = s.m_cd(P_MELEE, i), type = s.m_type(P_MELEE, i);
     const Vec2 rnd = random_step(next_key(rng), 4);
     const Vec2 to = step_towards_player(h, next_key(rng), r0, c0);
@@ -1045,7 +1050,7 @@ CFE_FN void move_melee(S& s, Hot& h, uint64_t& rng, int i) {
 template <class S>
 CFE_FN void move_passive(S& s, Hot& h, uint64_t& rng, int i) {
     if (!s.m_mask(P_PASSIVE, i)) return;
-    const int l = h.level;
+    const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_PASSIVE, i), c0 = s.m_col(P_PASSIVE, i), type = s.m_type(P_PASSIVE, i);
     const Vec2 rnd = random_step(next_key(rng), 8);
     int r1 = r0 + rnd.r, c1 = c0 + rnd.c;
@@ -1063,7 +1068,7 @@ CFE_FN void move_passive(S& s, Hot& h, uint64_t& rng, int i) {
 template <class S>
 CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
     if (!s.m_mask(P_RANGED, i)) return;
-    const int l = h.level;
+    const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_RANGED, i), c0 = s.m_col(P_RANGED, i), cd = s.m_cd(P_RANGED, i), type = s.m_type(P_RANGED, i);
     const Vec2 rnd = random_step(next_key(rng), 4);
     const Vec2 to = step_towards_player(h, next_key(rng), r0, c0);
@@ -1114,7 +1119,7 @@ CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
 template <class S>
 CFE_FN void move_mob_projectile(S& s, Hot& h, int i) {
     if (!s.m_mask(P_MOB_PROJ, i)) return;
-    const int l = h.level;
+    const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_MOB_PROJ, i), c0 = s.m_col(P_MOB_PROJ, i);
     const int r1 = r0 + s.pd_r(P_MOB_PROJ, i), c1 = c0 + s.pd_c(P_MOB_PROJ, i);
     const int b = s.blk(wrap_clamp(l, kLevels), wrap_clamp(r1, kMap), wrap_clamp(c1, kMap));
@@ -1138,7 +1143,7 @@ CFE_FN void move_mob_projectile(S& s, Hot& h, int i) {
 template <class S>
 CFE_FN void move_player_projectile(S& s, Hot& h, int i) {
     if (!s.m_mask(P_PLAYER_PROJ, i)) return;
-    const int l = h.level;
+    const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_PLAYER_PROJ, i), c0 = s.m_col(P_PLAYER_PROJ, i);
     const int r1 = r0 + s.pd_r(P_PLAYER_PROJ, i), c1 = c0 + s.pd_c(P_PLAYER_PROJ, i);
     const int type = s.m_type(P_PLAYER_PROJ, i);

@@ -1,0 +1,86 @@
+"""Host-side mirror of the reference's env vector (CuVec, craftax_full.cu:10688-10946) over
+the C ABI of include/cfp_env.h.  PyTorch owns the caller-side device buffers; every
+computation is a call into libcfpolicy.so."""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import _lib
+from .policy import REC_BYTES, _check, _ptr, _stream, lib
+
+
+class Env:
+    """cfp_env handle: `n` envs resident on the GPU, optionally with a pool of reset states."""
+
+    def __init__(self, num_envs, pool=0):
+        self._h = C.c_void_p()
+        _check(lib().cfp_env_create(C.byref(self._h), num_envs, pool))
+        self.n = num_envs
+        self.pool = pool
+        dev = torch.device("cuda", torch.cuda.current_device())
+        self.rewards = torch.zeros(num_envs, dtype=torch.float32, device=dev)
+        self.terminals = torch.zeros(num_envs, dtype=torch.float32, device=dev)
+
+    def close(self):
+        if self._h:
+            lib().cfp_env_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @staticmethod
+    def state_bytes():
+        return lib().cfp_env_state_bytes()
+
+    def import_states(self, states, first=0):
+        """states: contiguous numpy structured array of cfp_env_state records."""
+        s = np.ascontiguousarray(states)
+        assert s.dtype.itemsize == self.state_bytes()
+        _check(lib().cfp_env_import(self._h, first, len(s), C.c_void_p(s.ctypes.data)))
+
+    def import_pool(self, states, first=0):
+        s = np.ascontiguousarray(states)
+        assert s.dtype.itemsize == self.state_bytes()
+        _check(lib().cfp_env_pool_import(self._h, first, len(s), C.c_void_p(s.ctypes.data)))
+
+    def export_states(self, dtype, first=0, count=None):
+        count = self.n - first if count is None else count
+        out = np.zeros(count, dtype)
+        assert out.dtype.itemsize == self.state_bytes()
+        _check(lib().cfp_env_export(self._h, first, count, C.c_void_p(out.ctypes.data)))
+        return out
+
+    def seed_actions(self, seed):
+        _check(lib().cfp_env_seed_actions(self._h, seed, _stream()))
+
+    def step(self, actions=None):
+        """k_step: one game step; actions float32[n] on the device, or None for the env's own
+        xorshift32 % 43 stream.  Results land in self.rewards / self.terminals."""
+        _check(lib().cfp_env_step(self._h, _ptr(actions), _ptr(self.rewards), _ptr(self.terminals), _stream()))
+
+    def reset_list(self):
+        """(count, records[count] as int32 (env, key0, key1) rows) of the last step, on the host."""
+        recs = np.zeros((self.n, 3), np.int32)
+        cnt = C.c_int(0)
+        _check(lib().cfp_env_fetch_resets(self._h, C.c_void_p(recs.ctypes.data), self.n, C.byref(cnt), _stream()))
+        return cnt.value, recs[:cnt.value]
+
+    def reset_from_pool(self):
+        _check(lib().cfp_env_reset_from_pool(self._h, _stream()))
+
+    def record_obs(self, rec_row=None):
+        if rec_row is None:
+            rec_row = torch.empty(self.n, REC_BYTES, dtype=torch.uint8, device=self.rewards.device)
+        _check(lib().cfp_env_record_obs(self._h, _ptr(rec_row), _stream()))
+        return rec_row
+
+
+def light_table(count=100001):
+    out = np.zeros(count, np.float32)
+    _check(lib().cfp_env_light_table(C.c_void_p(out.ctypes.data), count))
+    return out

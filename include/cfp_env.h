@@ -132,6 +132,10 @@ int cfp_env_seed_actions(cfp_env* e, uint64_t seed, void* stream);
 /* The reset list of the last step: device count and records (d_resets of CuVec). */
 const int* cfp_env_reset_count(const cfp_env* e);
 const cfp_env_reset_rec* cfp_env_reset_list(const cfp_env* e);
+/* Host copy of the list (synchronises `stream`): up to max records into out, the full
+ * count into *count.  For callers that produce the new states on the host and hand them
+ * to cfp_env_import. */
+int cfp_env_fetch_resets(const cfp_env* e, cfp_env_reset_rec* out, int max, int* count, void* stream);
 /* craftax_reset_state_on_done with a static pool (craftax_full.c:3738-3741): every env
  * on the reset list becomes a copy of pool entry key0 % pool. */
 int cfp_env_reset_from_pool(cfp_env* e, void* stream);

@@ -1,0 +1,65 @@
+"""The env step's game logic without a GPU: the text the kernel compiles
+(craftax.cu_amd/csrc/env_logic.h), built for the host (oracle/libcfenvhost.so), against
+the compiled reference env (oracle/_ref) on the same actions -- every state field,
+reward, terminal and reset key after every step, bit for bit.  Also the light-level
+table the library uploads against the reference's own function for every timestep."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import env_bind as eb
+
+
+@pytest.fixture(scope="module")
+def ref():
+    try:
+        return eb.Ref()
+    except FileNotFoundError:
+        pytest.skip("oracle/_ref/libcfref.so is not built (reference source absent)")
+
+
+def test_exchange_struct_layout(pkg):
+    assert pkg.lib().cfp_env_state_bytes() == eb.STATE_DTYPE.itemsize
+    assert eb.HostStep().lib.cfhost_state_bytes() == eb.STATE_DTYPE.itemsize
+
+
+def test_light_table_matches_reference_for_every_timestep(pkg, ref):
+    """craftax_calculate_light_level_native (craftax_full.c:3760-3767) as the checker's
+    -ffast-math build evaluates it, t = 0..100000."""
+    mine = pkg.env.light_table()
+    want = np.array([ref.lib.cfref_light_level(t) for t in range(len(mine))], np.float32)
+    assert np.array_equal(mine.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(mine.view(np.uint32), eb.HostStep().light.view(np.uint32))
+
+
+@pytest.mark.parametrize("n,steps,seed", [(64, 400, 0), (32, 400, 42)])
+def test_host_build_of_the_step_matches_reference(ref, n, steps, seed):
+    ref.init(n, seed)
+    host = eb.HostStep()
+    mine = ref.export()
+    terminals = 0
+    for t in range(steps):
+        act = ref.next_actions()
+        final, rew, term, keys = ref.step(act)
+        r2, t2, k2 = host.step(mine, act)
+        d = eb.diff_fields(final, mine)
+        assert not d, f"step {t}: fields differ: {d}"
+        assert np.array_equal(rew.view(np.uint32), r2.view(np.uint32)), f"step {t}: reward"
+        assert np.array_equal(term, t2) and np.array_equal(keys, k2), f"step {t}: terminal / reset key"
+        done = np.nonzero(term)[0]
+        if len(done):
+            mine[done] = ref.export(list(done))
+            terminals += len(done)
+    assert terminals > 0
+
+
+def test_import_derives_spawn_planes_like_the_reference(ref):
+    """craftax_refresh_spawn_bits_level (craftax_full.c:3336-3355)."""
+    ref.init(8, 5)
+    s = ref.export()
+    t = s.copy()
+    for f in ("spawn_all_bits", "spawn_grave_bits", "spawn_water_bits"):
+        t[f] = 0
+    eb.HostStep().lib.cfhost_derive_spawn_planes(eb.ptr(t), len(t))
+    assert not eb.diff_fields(s, t)

@@ -1,0 +1,126 @@
+"""The env step on the GPU (cfp_env_step) against the compiled reference env
+(oracle/_ref: the reference's craftax_full.c, stepped env by env with the same actions):
+every state field, reward, terminal flag and reset key after every step, bit for bit
+(floats by bit pattern).  Resets are supplied: when an env finishes, the reference's
+freshly generated state is uploaded, so world generation is not on this test's path.
+Reference functions: craftax_gameplay_step_native and what it calls
+(craftax_full.c:3798-3878, 4210-8225), c_step_gameplay (:3981-4011), k_step
+(craftax_full.cu:8760-8779)."""
+import numpy as np
+import pytest
+import torch
+
+import env_bind as eb
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ref():
+    try:
+        return eb.Ref()
+    except FileNotFoundError:
+        pytest.skip("oracle/_ref/libcfref.so is not built")
+
+
+def _compare(tag, final, mine, rew, rew_gpu, term, term_gpu):
+    d = eb.diff_fields(final, mine)
+    msg = []
+    for f in d[:8]:
+        idx = np.argwhere(final[f] != mine[f])
+        msg.append(f"{f}{idx[0].tolist()}: ref {final[f][tuple(idx[0])]} gpu {mine[f][tuple(idx[0])]}")
+    assert not d, f"{tag}: state fields differ: " + "; ".join(msg)
+    assert np.array_equal(rew.view(np.uint32), rew_gpu.view(np.uint32)), f"{tag}: rewards differ"
+    assert np.array_equal(term, term_gpu), f"{tag}: terminals differ"
+
+
+def _rollout(pkg, ref, n, steps, seed, own_actions):
+    ref.init(n, seed)
+    env = pkg.Env(n)
+    env.import_states(ref.export())
+    assert not eb.diff_fields(ref.export(), env.export_states(eb.STATE_DTYPE)), "import/export round trip"
+    if own_actions:
+        env.seed_actions(seed)
+    terminals_seen = 0
+    for t in range(steps):
+        act = ref.next_actions()
+        final, rew, term, keys = ref.step(act)
+        env.step(None if own_actions else torch.from_numpy(act).cuda())
+        mine = env.export_states(eb.STATE_DTYPE)
+        _compare(f"step {t}", final, mine, rew, env.rewards.cpu().numpy(), term, env.terminals.cpu().numpy())
+        cnt, recs = env.reset_list()
+        done = np.nonzero(term)[0]
+        assert cnt == len(done)
+        if cnt:
+            order = np.argsort(recs[:, 0])
+            assert np.array_equal(recs[order, 0], done)
+            assert np.array_equal(recs[order, 1:].view(np.uint32), keys[done])
+            fresh = ref.export(list(done))
+            for k, e in enumerate(done):   # resets supplied by the reference
+                env.import_states(fresh[k:k + 1], first=int(e))
+            terminals_seen += cnt
+    return terminals_seen
+
+
+def test_env_step_matches_reference_256x600(pkg, cuda, ref):
+    """256 envs x 600 steps with the reference's xorshift32 % 43 actions, seed 0."""
+    seen = _rollout(pkg, ref, 256, 600, 0, own_actions=False)
+    assert seen > 0   # the run went through episode ends
+
+
+def test_env_step_own_action_stream(pkg, cuda, ref):
+    """The kernel's own xorshift32 % 43 stream (d_actions = NULL) is the reference's."""
+    _rollout(pkg, ref, 64, 200, 7, own_actions=True)
+
+
+def test_records_from_stepped_state(pkg, cuda, ref):
+    """cfp_env_record_obs on the stepped device state equals the reference's own encoder
+    on its state (craftax_encode_compact_observation, craftax_full.c:2830)."""
+    import ctypes as C
+    n = 128
+    ref.init(n, 3)
+    env = pkg.Env(n)
+    env.import_states(ref.export())
+    ref.lib.cfref_observations.restype = C.POINTER(C.c_uint8)
+    for t in range(120):
+        act = ref.next_actions()
+        final, rew, term, keys = ref.step(act)
+        env.step(torch.from_numpy(act).cuda())
+        done = np.nonzero(term)[0]
+        if len(done):
+            fresh = ref.export(list(done))
+            for k, e in enumerate(done):
+                env.import_states(fresh[k:k + 1], first=int(e))
+        if t % 10 == 9:
+            rec = env.record_obs().cpu().numpy()
+            want = np.ctypeslib.as_array(ref.lib.cfref_observations(), shape=(n, 996))
+            assert np.array_equal(rec, want), f"records differ at step {t}"
+
+
+def test_reset_from_pool(pkg, cuda, ref):
+    """Envs on the reset list become copies of pool entry key0 % pool; the env key and
+    the action stream survive (craftax_full.c:3738-3741)."""
+    n, pool = 64, 8
+    ref.init(n, 11)
+    states = ref.export()
+    env = pkg.Env(n, pool=pool)
+    dying = states.copy()
+    dying["player_health"][::3] = 0.05   # these die at the next damage or starve tick
+    dying["player_food"][::3] = 0
+    dying["player_drink"][::3] = 0
+    dying["player_recover"][::3] = -15.0
+    env.import_states(dying)
+    env.import_pool(states[:pool])
+    env.step(torch.zeros(n, dtype=torch.float32, device="cuda"))
+    before = env.export_states(eb.STATE_DTYPE)
+    cnt, recs = env.reset_list()
+    assert cnt == len(range(0, n, 3))
+    env.reset_from_pool()
+    after = env.export_states(eb.STATE_DTYPE)
+    hit = np.zeros(n, bool)
+    for e, k0, _ in recs:
+        hit[e] = True
+        want = states[(int(k0) & 0xFFFFFFFF) % pool].copy()
+        want["rng_key"] = before["rng_key"][e]
+        assert not eb.diff_fields(want.reshape(1), after[e:e + 1]), f"env {e}"
+    assert not eb.diff_fields(before[~hit], after[~hit])
