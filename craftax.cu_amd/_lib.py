@@ -110,6 +110,11 @@ PROTOTYPES = {
     "cfp_env_view": (C.c_int, [vp, vp, C.POINTER(vp), C.POINTER(vp), C.POINTER(vp),
                                C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "cfp_env_record_obs": (C.c_int, [vp, vp, vp]),
+    "cfp_env_actions": (vp, [vp]),
+    "cfp_env_rewards": (vp, [vp]),
+    "cfp_env_terminals": (vp, [vp]),
+    "cfp_env_rollout_step": (C.c_int, [vp, vp, C.c_int, C.c_uint64, vp]),
+    "cfp_train_collect": (C.c_int, [vp, vp, C.c_uint64, vp]),
 }
 
 

@@ -666,6 +666,7 @@ struct cfp_env {
     float* light = nullptr;
     cfp_env_reset_rec* resets = nullptr;
     int* reset_count = nullptr;
+    float* slots = nullptr;   // actions | rewards | terminals, n floats each
 };
 
 static_assert(sizeof(cfp_env_state) % 8 == 0, "exchange struct is 8-byte aligned");
@@ -713,6 +714,8 @@ int cfp_env_create(cfp_env** out, int n, int pool) {
     if ((err = hipMalloc((void**)&e->resets, sizeof(cfp_env_reset_rec) * (size_t)n)) != hipSuccess) return fail(err, "hipMalloc(resets)");
     if ((err = hipMalloc((void**)&e->reset_count, sizeof(int))) != hipSuccess) return fail(err, "hipMalloc(reset_count)");
     if ((err = hipMemset(e->reset_count, 0, sizeof(int))) != hipSuccess) return fail(err, "hipMemset(reset_count)");
+    if ((err = hipMalloc((void**)&e->slots, sizeof(float) * 3 * (size_t)n)) != hipSuccess) return fail(err, "hipMalloc(slots)");
+    if ((err = hipMemset(e->slots, 0, sizeof(float) * 3 * (size_t)n)) != hipSuccess) return fail(err, "hipMemset(slots)");
     *out = e;
     return 0;
 }
@@ -724,10 +727,14 @@ void cfp_env_destroy(cfp_env* e) {
     (void)hipFree(e->light);
     (void)hipFree(e->resets);
     (void)hipFree(e->reset_count);
+    (void)hipFree(e->slots);
     delete e;
 }
 
 int cfp_env_num_envs(const cfp_env* e) { return e ? e->live.n : 0; }
+float* cfp_env_actions(const cfp_env* e) { return e ? e->slots : nullptr; }
+float* cfp_env_rewards(const cfp_env* e) { return e ? e->slots + e->live.n : nullptr; }
+float* cfp_env_terminals(const cfp_env* e) { return e ? e->slots + 2 * (size_t)e->live.n : nullptr; }
 int cfp_env_pool_size(const cfp_env* e) { return e ? e->pool_size : 0; }
 
 int cfp_env_import(cfp_env* e, int first, int count, const cfp_env_state* states) {

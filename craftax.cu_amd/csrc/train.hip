@@ -13,6 +13,7 @@
 #include "cfp_common.h"
 #include "cfp_internal.h"
 #include "ppo_kernels.h"
+#include "../../include/cfp_env.h"
 
 namespace cfp {
 namespace {
@@ -372,6 +373,30 @@ int cfp_rollout_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
     (void)hn;
     return forward_and_sample(tr->p, row, d_prev_terminals, tr->r_state + o * tr->L * H, tr->n, so,
                               st);
+}
+
+int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void* stream) {
+    CFP_REQUIRE(tr && e, "cfp_env_rollout_step: NULL argument");
+    CFP_REQUIRE(cfp_env_num_envs(e) == tr->n, "cfp_env_rollout_step: the env object holds %d envs, the trainer %d",
+                cfp_env_num_envs(e), tr->n);
+    CFP_REQUIRE(t >= 0 && t < tr->T, "step %d outside the horizon %d", t, tr->T);
+    const size_t o = (size_t)t * tr->n;
+    uint8_t* row = tr->r_obs + o * CFP_REC_BYTES;
+    if (cfp_env_record_obs(e, row, stream)) return 1;
+    if (cfp_rollout_step(tr, t, row, cfp_env_terminals(e), seed, cfp_env_actions(e), stream)) return 1;
+    if (cfp_env_step(e, cfp_env_actions(e), cfp_env_rewards(e), cfp_env_terminals(e), stream)) return 1;
+    if (cfp_record_rd(cfp_env_rewards(e), cfp_env_terminals(e), tr->r_reward + o, tr->r_done + o, tr->n, stream)) return 1;
+    if (cfp_env_pool_size(e) > 0 && cfp_env_reset_from_pool(e, stream)) return 1;
+    return 0;
+}
+
+int cfp_train_collect(cfp_trainer* tr, cfp_env* e, uint64_t seed, void* stream) {
+    CFP_REQUIRE(tr && e, "cfp_train_collect: NULL argument");
+    for (int t = 0; t < tr->T; t++)
+        if (cfp_env_rollout_step(tr, e, t, seed, stream)) return 1;
+    if (cfp_env_record_obs(e, tr->p->rec, stream)) return 1;
+    if (cfp_train_bootstrap(tr, tr->p->rec, cfp_env_terminals(e), stream)) return 1;
+    return cfp_train_gae(tr, stream);
 }
 
 int cfp_train_bootstrap(cfp_trainer* tr, const uint8_t* d_rec_row, const float* d_terminals,

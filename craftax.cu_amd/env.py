@@ -7,7 +7,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .policy import REC_BYTES, _check, _ptr, _stream, lib
+from .policy import REC_BYTES, _check, _ptr, _stream, _wrap, lib
 
 
 class Env:
@@ -18,9 +18,10 @@ class Env:
         _check(lib().cfp_env_create(C.byref(self._h), num_envs, pool))
         self.n = num_envs
         self.pool = pool
-        dev = torch.device("cuda", torch.cuda.current_device())
-        self.rewards = torch.zeros(num_envs, dtype=torch.float32, device=dev)
-        self.terminals = torch.zeros(num_envs, dtype=torch.float32, device=dev)
+        # the env vector's own slots (CuVec.d_actions / d_rewards / d_terminals)
+        self.actions = _wrap(lib().cfp_env_actions(self._h), (num_envs,), "<f4")
+        self.rewards = _wrap(lib().cfp_env_rewards(self._h), (num_envs,), "<f4")
+        self.terminals = _wrap(lib().cfp_env_terminals(self._h), (num_envs,), "<f4")
 
     def close(self):
         if self._h:
@@ -72,6 +73,15 @@ class Env:
 
     def reset_from_pool(self):
         _check(lib().cfp_env_reset_from_pool(self._h, _stream()))
+
+    def rollout_step(self, trainer, t, seed):
+        """cu_rollout_step with this env vector: record, policy forward + sample, env step,
+        reward / done rows, pool reset."""
+        _check(lib().cfp_env_rollout_step(trainer._h, self._h, t, seed, _stream()))
+
+    def collect(self, trainer, seed):
+        """cu_train_collect: T rollout steps, bootstrap value, GAE."""
+        _check(lib().cfp_train_collect(trainer._h, self._h, seed, _stream()))
 
     def record_obs(self, rec_row=None):
         if rec_row is None:

@@ -112,6 +112,13 @@ int cfp_env_export(cfp_env* e, int first, int count, cfp_env_state* states);
  * craftax_full.c:3568-3581: worlds generated once, copied in on reset). */
 int cfp_env_pool_import(cfp_env* e, int first, int count, const cfp_env_state* states);
 
+/* The env vector's own action / reward / terminal slots, float[n] each on the device
+ * (CuVec.d_actions / d_rewards / d_terminals, craftax_full.cu:10693-10695), zeroed at
+ * creation.  cfp_env_step accepts any buffers; these are the ones the collect loop uses. */
+float* cfp_env_actions(const cfp_env* e);
+float* cfp_env_rewards(const cfp_env* e);
+float* cfp_env_terminals(const cfp_env* e);
+
 /* calculate_light_level(timestep) for timestep 0..CFP_ENV_MAX_TIMESTEPS as the step uses
  * it (craftax_full.c:3760-3767 under the reference's build flags; the reference's GPU
  * port also computes this table on the host, craftax_full.cu:10714-10729).  Host only. */
@@ -148,6 +155,18 @@ int cfp_env_view(const cfp_env* e, cfp_env_soa* soa, const uint8_t** d_map,
 /* k_record_obs on this env's state: n records into d_rec_row (cfp_record_obs_soa on
  * cfp_env_view). */
 int cfp_env_record_obs(const cfp_env* e, uint8_t* d_rec_row, void* stream);
+
+/* cu_rollout_step (craftax_full.cu:12022-12087) with the env on the device: record the
+ * envs' observations into r_obs[t], run the policy half (cfp_rollout_step: forward on the
+ * live state with the env's terminals as the state-zeroing flags, sample into r_act /
+ * r_logprob / r_value and the env's action slots), step the envs, store rewards and
+ * terminals into r_reward[t] / r_done[t], reset finished envs from the pool when the env
+ * object has one.  The trainer's env count must equal the env object's. */
+int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void* stream);
+/* cu_train_collect (craftax_full.cu:12980-13016): T rollout steps as above, the bootstrap
+ * value on a copy of the live state from the post-rollout observations, GAE and the
+ * advantage statistics. */
+int cfp_train_collect(cfp_trainer* tr, cfp_env* e, uint64_t seed, void* stream);
 
 #ifdef __cplusplus
 }

@@ -124,3 +124,53 @@ def test_reset_from_pool(pkg, cuda, ref):
         want["rng_key"] = before["rng_key"][e]
         assert not eb.diff_fields(want.reshape(1), after[e:e + 1]), f"env {e}"
     assert not eb.diff_fields(before[~hit], after[~hit])
+
+
+def test_collect_with_the_env_on_the_device(pkg, cuda, ref):
+    """cfp_train_collect (cu_train_collect, craftax_full.cu:12980-13016): policy and envs
+    both on the device for T steps.  The stored actions are replayed through the reference
+    env on the CPU; observations, rewards and done flags of every step must be the slabs',
+    bit for bit, including envs that finish and are refilled from the reset pool."""
+    import ctypes as C
+    n, T, pool, seed = 64, 40, 4, 5
+    ref.init(n, seed)
+    states = ref.export()
+    pool_states = states[8:8 + pool].copy()
+    weak = states.copy()
+    for e in range(0, n, 4):            # a quarter of the envs starve within the horizon
+        weak["player_health"][e] = 1.0 + (e % 3)
+        weak["player_food"][e] = 0
+        weak["player_recover"][e] = -14.0 + (e % 5)
+        ref.import_(e, weak[e])
+    env = pkg.Env(n, pool=pool)
+    env.import_states(weak)
+    env.import_pool(pool_states)
+    pol = pkg.Policy(n, layers=3, seed=1)
+    tr = pkg.Trainer(pol, T)
+    env.collect(tr, seed=1234)
+    torch.cuda.synchronize()
+    r_obs = tr.buf("r_obs").cpu().numpy()
+    r_act = tr.buf("r_act").cpu().numpy()
+    r_rew = tr.buf("r_reward").cpu().numpy()
+    r_done = tr.buf("r_done").cpu().numpy()
+    ref.lib.cfref_observations.restype = C.POINTER(C.c_uint8)
+    ref.lib.cfref_encode.argtypes = [C.c_int, C.c_void_p]
+    rec = np.zeros((n, 996), np.uint8)
+    finished = 0
+    for t in range(T):
+        for e in range(n):
+            ref.lib.cfref_encode(e, C.c_void_p(rec[e].ctypes.data))
+        assert np.array_equal(rec, r_obs[t]), f"observations of step {t}"
+        final, rew, term, keys = ref.step(r_act[t].astype(np.float32))
+        assert np.array_equal(rew.view(np.uint32), r_rew[t].view(np.uint32)), f"rewards of step {t}"
+        assert np.array_equal(term.astype(np.uint8), r_done[t]), f"done flags of step {t}"
+        for e in np.nonzero(term)[0]:   # the device refilled these from the pool
+            fresh = pool_states[int(keys[e, 0]) % pool].copy()
+            fresh["rng_key"] = final["rng_key"][e]
+            ref.import_(int(e), fresh)
+            finished += 1
+    assert finished >= 4
+    mine = env.export_states(eb.STATE_DTYPE)
+    assert not eb.diff_fields(ref.export(), mine), "states after the rollout"
+    adv = tr.buf("adv").cpu().numpy()
+    assert np.isfinite(adv).all() and np.abs(adv).max() > 0
