@@ -97,6 +97,10 @@ PROTOTYPES = {
     "cfp_env_destroy": (None, [vp]),
     "cfp_env_num_envs": (C.c_int, [vp]),
     "cfp_env_pool_size": (C.c_int, [vp]),
+    "cfp_env_init": (C.c_int, [vp, C.c_uint64, vp]),
+    "cfp_env_reset": (C.c_int, [vp, vp]),
+    "cfp_env_pool_fill": (C.c_int, [vp, C.c_uint64, vp]),
+    "cfp_env_generate_host": (C.c_int, [C.c_uint32, C.c_int, vp]),
     "cfp_env_import": (C.c_int, [vp, C.c_int, C.c_int, vp]),
     "cfp_env_export": (C.c_int, [vp, C.c_int, C.c_int, vp]),
     "cfp_env_pool_import": (C.c_int, [vp, C.c_int, C.c_int, vp]),

@@ -8,6 +8,7 @@
 
 #include "../../include/cfp_env.h"
 #include "env_logic.h"
+#include "env_worldgen.h"
 
 namespace cfenv {
 
@@ -205,6 +206,71 @@ struct HostStore {
     void open_level(int l) { lvl = l; }
     float light_at(int t) const { return light[t < kMaxTimesteps ? t : kMaxTimesteps]; }
 };
+
+// a group of one thread for env_worldgen.h; cos / sin are the C library's
+struct HostGroup {
+    int tid() const { return 0; }
+    int nt() const { return 1; }
+    void sync() {}
+    float gmin(float v) { return v; }
+    float gmax(float v) { return v; }
+    int gmaxi(int v) { return v; }
+    int gscan(int v, int& total) {
+        total = v;
+        return 0;
+    }
+    float cosine(float x) { return cosf(x); }
+    float sine(float x) { return sinf(x); }
+};
+
+// craftax_generate_world_from_key (craftax_full.c:2050-2142): a fresh state from a world key.
+// rng_key is left alone (it belongs to the env, not to the world).
+inline void generate_world_host(uint64_t world_key, cfp_env_state& st, FloorScratch& sc) {
+    const uint32_t keep0 = st.rng_key[0], keep1 = st.rng_key[1];
+    memset(&st, 0, sizeof(st));
+    st.rng_key[0] = keep0;
+    st.rng_key[1] = keep1;
+    HostGroup g;
+    for (int l = 0; l < kLevels; l++) {
+        generate_floor(g, sc, world_key, l);
+        memcpy(st.map[l], sc.map, kCells);
+        memcpy(st.item_map[l], sc.item, kCells);
+        memcpy(st.light_map[l], sc.light, kCells);
+        for (int a = 0; a < 2; a++) {
+            st.down_ladders[l][a] = sc.ladder_down[a];
+            st.up_ladders[l][a] = sc.ladder_up[a];
+        }
+    }
+    for (int p = 0; p < CFP_ENV_MOB_CLASSES; p++)
+        for (int l = 0; l < kLevels; l++)
+            for (int i = 0; i < (p == P_RANGED ? 2 : 3); i++) st.mob_health[p][l][i] = 1.0f;
+    for (int l = 0; l < kLevels; l++)
+        for (int i = 0; i < 3; i++)
+            for (int a = 0; a < 2; a++) st.mob_projectile_directions[l][i][a] = st.player_projectile_directions[l][i][a] = 1;
+    int32_t perm[6];
+    potion_permutation(world_key, perm);
+    for (int i = 0; i < 6; i++) st.potion_mapping[i] = perm[i];
+    const uint64_t sk = world_state_key(world_key);
+    st.state_rng[0] = (uint32_t)sk;
+    st.state_rng[1] = (uint32_t)(sk >> 32);
+    st.monsters_killed[0] = 10;
+    st.player_position[0] = st.player_position[1] = kMap / 2;
+    st.player_direction = A_UP;
+    st.player_health = 9.0f;
+    st.player_food = st.player_drink = st.player_energy = st.player_mana = 9;
+    st.player_dexterity = st.player_strength = st.player_intelligence = 1;
+    st.boss_timesteps_to_spawn_this_round = 7;
+    st.light_level = light_level(0);
+    derive_spawn_planes(st);
+}
+// c_init's state for an env created with `seed` (craftax_reset_state_from_seed, :3601-3614)
+inline void generate_env_host(uint32_t seed, cfp_env_state& st, FloorScratch& sc) {
+    const uint64_t k = seed_key(seed);
+    const uint64_t env_key = lcg(k), reset_key = lcg(env_key);
+    generate_world_host(world_key_of_reset(reset_key), st, sc);
+    st.rng_key[0] = (uint32_t)env_key;
+    st.rng_key[1] = (uint32_t)(env_key >> 32);
+}
 
 // c_step_gameplay (craftax_full.c:3981-4011) without the reset, on one host state
 inline void host_step(cfp_env_state& st, float action, const float* light, float* reward, float* terminal,

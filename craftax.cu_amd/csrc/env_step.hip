@@ -574,6 +574,174 @@ __global__ __launch_bounds__(256) void k_env_reset_from_pool(CopyTable t, EnvArr
     }
 }
 
+// ---- world generation on the device ------------------------------------------------------------
+constexpr int kGenThreads = 256;
+// the group of env_worldgen.h: one 256-thread workgroup, reductions through wave shuffles
+// and four LDS words; cos / sin in double precision, rounded to float
+struct BlockGroup {
+    int t;
+    float* fred;   // LDS, 4 floats
+    int* ired;     // LDS, 4 ints
+    __device__ __forceinline__ int tid() const { return t; }
+    __device__ __forceinline__ int nt() const { return kGenThreads; }
+    __device__ __forceinline__ void sync() { __syncthreads(); }
+    __device__ __forceinline__ float gmin(float v) {
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) v = fminf(v, __shfl_xor(v, d));
+        if ((t & 63) == 0) fred[t >> 6] = v;
+        __syncthreads();
+        v = fminf(fminf(fred[0], fred[1]), fminf(fred[2], fred[3]));
+        __syncthreads();
+        return v;
+    }
+    __device__ __forceinline__ float gmax(float v) {
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) v = fmaxf(v, __shfl_xor(v, d));
+        if ((t & 63) == 0) fred[t >> 6] = v;
+        __syncthreads();
+        v = fmaxf(fmaxf(fred[0], fred[1]), fmaxf(fred[2], fred[3]));
+        __syncthreads();
+        return v;
+    }
+    __device__ __forceinline__ int gmaxi(int v) {
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) v = max(v, __shfl_xor(v, d));
+        if ((t & 63) == 0) ired[t >> 6] = v;
+        __syncthreads();
+        v = max(max(ired[0], ired[1]), max(ired[2], ired[3]));
+        __syncthreads();
+        return v;
+    }
+    __device__ __forceinline__ int gscan(int v, int& total) {
+        const int lane = t & 63, wave = t >> 6;
+        int incl = v;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        if (lane == 63) ired[wave] = incl;
+        __syncthreads();
+        int before = 0;
+        total = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            before += w < wave ? ired[w] : 0;
+            total += ired[w];
+        }
+        __syncthreads();
+        return before + incl - v;
+    }
+    __device__ __forceinline__ float cosine(float x) { return (float)cos((double)x); }
+    __device__ __forceinline__ float sine(float x) { return (float)sin((double)x); }
+};
+
+struct FieldList {          // the per-field arrays of one EnvArrays, for table-driven fills
+    void* ptr[kNumFields];
+    int elem[kNumFields];
+    int count[kNumFields];
+};
+
+// k_env_init / k_reset_list_block (craftax_full.cu:8669-8706, 8957-8975): one workgroup per
+// env.  LIST: the envs of the reset list, world key from each record's reset key, the env's
+// own key kept.  Otherwise: envs [0, A.n), env i created from seed0 + i as c_init does.
+template <bool LIST>
+__global__ __launch_bounds__(kGenThreads) void k_env_worldgen(EnvArrays A, FieldList fl, const float* __restrict__ light,
+                                                              const cfp_env_reset_rec* __restrict__ resets,
+                                                              const int* __restrict__ reset_count, uint64_t seed0,
+                                                              int zero_fields) {
+    __shared__ FloorScratch sc;
+    __shared__ float fred[4];
+    __shared__ int ired[4];
+    BlockGroup g{(int)threadIdx.x, fred, ired};
+    const int t = threadIdx.x;
+    const size_t n = (size_t)A.n;
+    const int total = LIST ? *reset_count : A.n;
+    for (int idx = blockIdx.x; idx < total; idx += gridDim.x) {
+        size_t e;
+        uint64_t world_key, env_key = 0;
+        if (LIST) {
+            e = (size_t)resets[idx].env;
+            world_key = world_key_of_reset((uint64_t)resets[idx].key1 << 32 | resets[idx].key0);
+        } else {
+            e = (size_t)idx;
+            env_key = lcg(seed_key((uint32_t)(seed0 + (uint64_t)idx)));
+            world_key = world_key_of_reset(lcg(env_key));
+        }
+        // scalars: the fields of `fl` are zero in a fresh state; the others are written below
+        for (int f = 0; f < zero_fields; f++) {
+            const int el = fl.elem[f];
+            for (int k = t; k < fl.count[f]; k += kGenThreads) {
+                const size_t at = (size_t)k * n + e;
+                if (el == 4) ((uint32_t*)fl.ptr[f])[at] = 0u;
+                else if (el == 8) ((uint64_t*)fl.ptr[f])[at] = 0ull;
+                else ((uint8_t*)fl.ptr[f])[at] = 0;
+            }
+        }
+        for (int k = t; k < kMobSlots; k += kGenThreads) A.mob_health[(size_t)k * n + e] = (k / 27 == P_RANGED && k % 3 == 2) ? 0.0f : 1.0f;
+        for (int k = t; k < 54; k += kGenThreads) {
+            A.mob_projectile_directions[(size_t)k * n + e] = 1;
+            A.player_projectile_directions[(size_t)k * n + e] = 1;
+        }
+        if (t < kLevels) A.monsters_killed[(size_t)t * n + e] = t == 0 ? 10 : 0;
+        if (t == 0) {
+            int32_t perm[6];
+            potion_permutation(world_key, perm);
+            for (int i = 0; i < 6; i++) A.potion_mapping[(size_t)i * n + e] = perm[i];
+            const uint64_t sk = world_state_key(world_key);
+            A.state_rng[e] = (uint32_t)sk;
+            A.state_rng[n + e] = (uint32_t)(sk >> 32);
+            A.player_position[e] = kMap / 2;
+            A.player_position[n + e] = kMap / 2;
+            A.player_direction[e] = A_UP;
+            A.player_health[e] = 9.0f;
+            A.player_food[e] = 9;
+            A.player_drink[e] = 9;
+            A.player_energy[e] = 9;
+            A.player_mana[e] = 9;
+            A.player_dexterity[e] = 1;
+            A.player_strength[e] = 1;
+            A.player_intelligence[e] = 1;
+            A.boss_timesteps_to_spawn_this_round[e] = 7;
+            A.light_level[e] = light[0];
+            if (!LIST) {
+                A.rng_key[e] = (uint32_t)env_key;
+                A.rng_key[n + e] = (uint32_t)(env_key >> 32);
+            }
+        }
+        uint8_t* planes = A.planes + e * kEnvPlaneBytes;
+        for (int level = 0; level < kLevels; level++) {
+            generate_floor(g, sc, world_key, level);
+            // the three byte planes, 16 bytes a thread
+            for (int k = t; k < 3 * (int)(kPlaneBytes / 16); k += kGenThreads) {
+                const int plane = k / (int)(kPlaneBytes / 16), off = k % (int)(kPlaneBytes / 16);
+                const uint8_t* src = plane == 0 ? sc.map : (plane == 1 ? sc.item : sc.light);
+                ((u4*)(planes + ((size_t)plane * kLevels + level) * kPlaneBytes))[off] = ((const u4*)src)[off];
+            }
+            // spawn bit planes of the level (craftax_refresh_spawn_bits_level), no mobs yet
+            if (t < kMap) {
+                uint64_t all = 0, grave = 0, water = 0;
+                for (int c = 0; c < kMap; c++) {
+                    const int b = sc.map[t * kMap + c];
+                    all |= (uint64_t)in_set(kSpawnAll, b) << c;
+                    grave |= (uint64_t)in_set(kSpawnGrave, b) << c;
+                    water |= (uint64_t)in_set(kSpawnWater, b) << c;
+                }
+                const size_t at = (size_t)(level * kMap + t) * n + e;
+                A.spawn_all_bits[at] = all;
+                A.spawn_grave_bits[at] = grave;
+                A.spawn_water_bits[at] = water;
+                A.mob_bits[at] = 0;
+            }
+            if (t < 2) {
+                A.down_ladders[(size_t)(level * 2 + t) * n + e] = sc.ladder_down[t];
+                A.up_ladders[(size_t)(level * 2 + t) * n + e] = sc.ladder_up[t];
+            }
+            __syncthreads();
+        }
+    }
+}
+
 int alloc_arrays(EnvArrays& A, int n) {
     memset(&A, 0, sizeof(A));
     A.n = n;
@@ -779,6 +947,73 @@ int cfp_env_step(cfp_env* e, const float* d_actions, float* d_rewards, float* d_
 
 const int* cfp_env_reset_count(const cfp_env* e) { return e ? e->reset_count : nullptr; }
 const cfp_env_reset_rec* cfp_env_reset_list(const cfp_env* e) { return e ? e->resets : nullptr; }
+
+namespace cfp {
+namespace {
+// fields a fresh state holds zero in and that the generator kernel does not write itself
+int zero_field_list(const EnvArrays& A, FieldList& fl) {
+    const size_t skip[] = {offsetof(EnvArrays, rng_key), offsetof(EnvArrays, mob_health),
+                           offsetof(EnvArrays, mob_projectile_directions), offsetof(EnvArrays, player_projectile_directions),
+                           offsetof(EnvArrays, potion_mapping), offsetof(EnvArrays, state_rng),
+                           offsetof(EnvArrays, monsters_killed), offsetof(EnvArrays, player_position),
+                           offsetof(EnvArrays, mob_bits), offsetof(EnvArrays, spawn_all_bits),
+                           offsetof(EnvArrays, spawn_grave_bits), offsetof(EnvArrays, spawn_water_bits),
+                           offsetof(EnvArrays, down_ladders), offsetof(EnvArrays, up_ladders)};
+    int m = 0;
+    for (int f = 0; f < kNumFields; f++) {
+        bool skipped = false;
+        for (size_t off : skip) skipped = skipped || off == kFieldTable[f].offset;
+        if (skipped) continue;
+        fl.ptr[m] = *reinterpret_cast<void* const*>(reinterpret_cast<const char*>(&A) + kFieldTable[f].offset);
+        fl.elem[m] = (int)kFieldTable[f].elem;
+        fl.count[m] = kFieldTable[f].count;
+        m++;
+    }
+    return m;
+}
+}  // namespace
+}  // namespace cfp
+
+int cfp_env_init(cfp_env* e, uint64_t seed, void* stream) {
+    CFP_REQUIRE(e != nullptr, "cfp_env_init: NULL env");
+    cfp::FieldList fl;
+    const int m = cfp::zero_field_list(e->live, fl);
+    const int grid = e->live.n < 4096 ? e->live.n : 4096;
+    hipLaunchKernelGGL(cfp::k_env_worldgen<false>, dim3(grid), dim3(cfp::kGenThreads), 0, (hipStream_t)stream, e->live, fl,
+                       e->light, nullptr, nullptr, seed, m);
+    CFP_HIP_TRY(hipGetLastError());
+    return cfp_env_seed_actions(e, seed, stream);
+}
+
+int cfp_env_pool_fill(cfp_env* e, uint64_t seed, void* stream) {
+    CFP_REQUIRE(e != nullptr, "cfp_env_pool_fill: NULL env");
+    CFP_REQUIRE(e->pool_size > 0, "cfp_env_pool_fill: this env object was created without a reset pool");
+    cfp::FieldList fl;
+    const int m = cfp::zero_field_list(e->pool, fl);
+    hipLaunchKernelGGL(cfp::k_env_worldgen<false>, dim3(e->pool_size < 4096 ? e->pool_size : 4096), dim3(cfp::kGenThreads), 0,
+                       (hipStream_t)stream, e->pool, fl, e->light, nullptr, nullptr, seed, m);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int cfp_env_reset(cfp_env* e, void* stream) {
+    CFP_REQUIRE(e != nullptr, "cfp_env_reset: NULL env");
+    cfp::FieldList fl;
+    const int m = cfp::zero_field_list(e->live, fl);
+    // the list is short (a fraction of a percent of the envs per step): a fixed grid strides it
+    const int grid = e->live.n < 1024 ? e->live.n : 1024;
+    hipLaunchKernelGGL(cfp::k_env_worldgen<true>, dim3(grid), dim3(cfp::kGenThreads), 0, (hipStream_t)stream, e->live, fl,
+                       e->light, e->resets, e->reset_count, 0ull, m);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+int cfp_env_generate_host(uint32_t seed, int count, cfp_env_state* states) {
+    CFP_REQUIRE(states != nullptr && count >= 0, "cfp_env_generate_host: bad argument");
+    std::vector<cfenv::FloorScratch> sc(1);
+    for (int i = 0; i < count; i++) cfenv::generate_env_host(seed + (uint32_t)i, states[i], sc[0]);
+    return 0;
+}
 
 int cfp_env_fetch_resets(const cfp_env* e, cfp_env_reset_rec* out, int max, int* count, void* stream) {
     CFP_REQUIRE(e != nullptr && count != nullptr && (out != nullptr || max == 0) && max >= 0,

@@ -386,8 +386,7 @@ int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void
     if (cfp_rollout_step(tr, t, row, cfp_env_terminals(e), seed, cfp_env_actions(e), stream)) return 1;
     if (cfp_env_step(e, cfp_env_actions(e), cfp_env_rewards(e), cfp_env_terminals(e), stream)) return 1;
     if (cfp_record_rd(cfp_env_rewards(e), cfp_env_terminals(e), tr->r_reward + o, tr->r_done + o, tr->n, stream)) return 1;
-    if (cfp_env_pool_size(e) > 0 && cfp_env_reset_from_pool(e, stream)) return 1;
-    return 0;
+    return cfp_env_pool_size(e) > 0 ? cfp_env_reset_from_pool(e, stream) : cfp_env_reset(e, stream);
 }
 
 int cfp_train_collect(cfp_trainer* tr, cfp_env* e, uint64_t seed, void* stream) {

@@ -56,6 +56,17 @@ class Env:
         _check(lib().cfp_env_export(self._h, first, count, C.c_void_p(out.ctypes.data)))
         return out
 
+    def init(self, seed):
+        """k_env_init: env i = the env created from seed + i, worlds generated on the device."""
+        _check(lib().cfp_env_init(self._h, seed, _stream()))
+
+    def reset(self):
+        """k_reset_list_block: new worlds for the envs on the reset list."""
+        _check(lib().cfp_env_reset(self._h, _stream()))
+
+    def pool_fill(self, seed=0):
+        _check(lib().cfp_env_pool_fill(self._h, seed, _stream()))
+
     def seed_actions(self, seed):
         _check(lib().cfp_env_seed_actions(self._h, seed, _stream()))
 
@@ -88,6 +99,14 @@ class Env:
             rec_row = torch.empty(self.n, REC_BYTES, dtype=torch.uint8, device=self.rewards.device)
         _check(lib().cfp_env_record_obs(self._h, _ptr(rec_row), _stream()))
         return rec_row
+
+
+def generate_host(dtype, seed, count):
+    """States of envs created from seed, seed + 1, ... generated on the host."""
+    out = np.zeros(count, dtype)
+    assert out.dtype.itemsize == Env.state_bytes()
+    _check(lib().cfp_env_generate_host(seed, count, C.c_void_p(out.ctypes.data)))
+    return out
 
 
 def light_table(count=100001):

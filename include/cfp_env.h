@@ -104,6 +104,21 @@ void cfp_env_destroy(cfp_env* e);
 int cfp_env_num_envs(const cfp_env* e);
 int cfp_env_pool_size(const cfp_env* e);
 
+/* k_env_init (craftax_full.cu:8669-8699; c_init, craftax_full.c:3883-3893): env i becomes the
+ * env created from seed + i -- its key, the nine floors of its first world generated on the
+ * device (all floors at once, as the reference's C build does; craftax_full.c:2050-2142) --
+ * and its action stream is seeded as cfp_env_seed_actions does. */
+int cfp_env_init(cfp_env* e, uint64_t seed, void* stream);
+/* k_reset_list_block (craftax_full.cu:8957-8975; craftax_reset_state_on_done,
+ * craftax_full.c:3731-3744): every env on the reset list gets a new world generated on the
+ * device from its record's key; its own key and action stream continue. */
+int cfp_env_reset(cfp_env* e, void* stream);
+/* The reset pool filled on the device: entry i = the state of an env created from seed + i
+ * (craftax_set_reset_pool_size, craftax_full.c:3568-3581, uses seeds 0, 1, ...). */
+int cfp_env_pool_fill(cfp_env* e, uint64_t seed, void* stream);
+/* The same states generated on the host, for callers that keep worlds there. */
+int cfp_env_generate_host(uint32_t seed, int count, cfp_env_state* states);
+
 /* Host states -> device arrays of envs [first, first + count) and back.  Both
  * synchronise with the device.  Import derives the spawn bit planes from `map`. */
 int cfp_env_import(cfp_env* e, int first, int count, const cfp_env_state* states);
@@ -160,8 +175,8 @@ int cfp_env_record_obs(const cfp_env* e, uint8_t* d_rec_row, void* stream);
  * envs' observations into r_obs[t], run the policy half (cfp_rollout_step: forward on the
  * live state with the env's terminals as the state-zeroing flags, sample into r_act /
  * r_logprob / r_value and the env's action slots), step the envs, store rewards and
- * terminals into r_reward[t] / r_done[t], reset finished envs from the pool when the env
- * object has one.  The trainer's env count must equal the env object's. */
+ * terminals into r_reward[t] / r_done[t], reset finished envs: from the pool when the env
+ * object has one, with freshly generated worlds otherwise.  The trainer's env count must equal the env object's. */
 int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void* stream);
 /* cu_train_collect (craftax_full.cu:12980-13016): T rollout steps as above, the bootstrap
  * value on a copy of the live state from the post-rollout observations, GAE and the

@@ -25,6 +25,17 @@ void cfhost_step(cfp_env_state* states, int count, const float* actions, const f
         cfenv::host_step(states[i], actions[i], light, &rewards[i], &terminals[i], &reset_keys[2 * i]);
 }
 
+/* States of envs created with seeds seed0, seed0 + 1, ... (c_init), generated on the host. */
+void cfhost_generate(uint32_t seed0, int count, cfp_env_state* states) {
+    static cfenv::FloorScratch sc;
+    for (int i = 0; i < count; i++) cfenv::generate_env_host(seed0 + (uint32_t)i, states[i], sc);
+}
+/* The state a finished env is reset to from its reset key. */
+void cfhost_reset(cfp_env_state* state, const uint32_t reset_key[2]) {
+    static cfenv::FloorScratch sc;
+    cfenv::generate_world_host(cfenv::world_key_of_reset((uint64_t)reset_key[1] << 32 | reset_key[0]), *state, sc);
+}
+
 void cfhost_derive_spawn_planes(cfp_env_state* states, int count) {
     for (int i = 0; i < count; i++) cfenv::derive_spawn_planes(states[i]);
 }

@@ -174,3 +174,80 @@ def test_collect_with_the_env_on_the_device(pkg, cuda, ref):
     assert not eb.diff_fields(ref.export(), mine), "states after the rollout"
     adv = tr.buf("adv").cpu().numpy()
     assert np.isfinite(adv).all() and np.abs(adv).max() > 0
+
+
+def _cell_agreement(a, b):
+    """(differing cells, cells, worlds with any difference) over the three byte maps."""
+    diff = np.zeros(len(a), bool)
+    cells = bad = 0
+    for f in ("map", "item_map", "light_map"):
+        neq = a[f] != b[f]
+        bad += int(neq.sum())
+        cells += neq.size
+        diff |= neq.reshape(len(a), -1).any(axis=1)
+    return bad, cells, int(diff.sum())
+
+
+def test_device_worldgen_against_host_and_reference(pkg, cuda, ref):
+    """cfp_env_init (k_env_init; craftax_generate_world_from_key, craftax_full.c:2050-2142):
+    worlds generated on the GPU against the same generator run on the host and against the
+    compiled reference's c_init.  The three dungeon floors and every scalar are integer work
+    and must be identical; the six noise floors may differ where a Perlin value lies within
+    a rounding of a threshold (the GPU's cos / sin are not the C library's): at most one
+    world in a hundred may show any difference, and at most one cell in a million."""
+    n, seed = 512, 2024
+    env = pkg.Env(n)
+    env.init(seed)
+    gpu = env.export_states(eb.STATE_DTYPE)
+    host = pkg.env.generate_host(eb.STATE_DTYPE, seed, n)
+    ref.init(n, seed)
+    want = ref.export()
+    for other, name in ((host, "host generator"), (want, "compiled reference")):
+        bad, cells, worlds = _cell_agreement(gpu, other)
+        print(f"GPU worldgen vs {name}: {bad} of {cells} cells differ, {worlds} of {n} worlds")
+        assert worlds <= n // 100 and bad <= max(cells // 1000000, 200), name
+        same = ~np.array([bool(eb.diff_fields(gpu[i:i + 1], other[i:i + 1])) for i in range(n)])
+        assert same.sum() >= n - n // 100
+        for f in eb.STATE_DTYPE.names:     # everything that is not a map or derived from one
+            if f in ("map", "item_map", "light_map", "spawn_all_bits", "spawn_grave_bits", "spawn_water_bits",
+                     "down_ladders", "up_ladders", "pad_"):
+                continue
+            x, y = gpu[f], other[f]
+            if x.dtype == np.float32:
+                x, y = x.view(np.uint32), y.view(np.uint32)
+            assert np.array_equal(x, y), f"{f} vs {name}"
+        for lvl in (1, 3, 4):              # dungeons
+            for f in ("map", "item_map", "light_map", "down_ladders", "up_ladders"):
+                assert np.array_equal(gpu[f][:, lvl], other[f][:, lvl]), f"{f}[{lvl}] vs {name}"
+
+
+def test_closed_loop_with_device_resets(pkg, cuda, ref):
+    """256 envs x 500 steps with nothing supplied by the host: envs created by cfp_env_init,
+    stepped with their own action streams, finished envs regenerated by cfp_env_reset.  Every
+    state field, reward and terminal is the compiled reference's after every step.  A reset
+    whose world differs from the reference's in a noise cell (see the worldgen test) is
+    counted and re-synchronised; at most one such reset is tolerated here."""
+    n, steps, seed = 256, 500, 0
+    ref.init(n, seed)
+    env = pkg.Env(n)
+    env.init(seed)
+    start = env.export_states(eb.STATE_DTYPE)
+    assert not eb.diff_fields(ref.export(), start), "initial worlds"
+    resets = resynced = 0
+    for t in range(steps):
+        act = ref.next_actions()
+        final, rew, term, keys = ref.step(act)
+        env.step(None)
+        mine = env.export_states(eb.STATE_DTYPE)
+        _compare(f"step {t}", final, mine, rew, env.rewards.cpu().numpy(), term, env.terminals.cpu().numpy())
+        done = np.nonzero(term)[0]
+        if len(done):
+            env.reset()
+            fresh = ref.export(list(done))
+            got = env.export_states(eb.STATE_DTYPE)[done]
+            for k, e in enumerate(done):
+                resets += 1
+                if eb.diff_fields(fresh[k:k + 1], got[k:k + 1]):
+                    resynced += 1
+                    env.import_states(fresh[k:k + 1], first=int(e))
+    assert resets > 100 and resynced <= 1, (resets, resynced)
