@@ -14,15 +14,21 @@
                   records -> fp32 features, and the unfused MinGRU gate/blend
                   epilogue of one layer
   stream_ceilings what plain library copies, fills and reads stream on the GPU
+  env_step        the env on the device at 8192 / 65 536 / 262 144 envs: game step with the
+                  envs' own random actions + world generation for finished envs (the
+                  reference's "env only" figure, which also writes the observation
+                  records), and the kernels one by one
+  rollout_in_the_loop  policy in the loop: record -> forward + sample -> env step ->
+                  reward/done rows -> reset (cfp_env_rollout_step), steps per second
 
-Usage:  python craftax.cu_amd/bench_configs.py [--reps 10] [--only NAME]
+Usage:  python bench_configs.py [--reps 10] [--only NAME]
 The headline workload (262 144 envs) is bench.py at the repository root."""
 import argparse
 import json
 import os
 import sys
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 PEAK_FP32 = 157.3                    # TFLOP/s, fp32 MFMA
 FWD_FLOP = 1633792                   # per env-step: encoder + 3 gate GEMMs + head
@@ -373,6 +379,67 @@ def stream_ceilings(pkg, torch, reps):
     return out
 
 
+def env_step(pkg, torch, reps):
+    """Env-only steps per second, as the reference's `bench` mode counts them (random
+    actions, auto-reset and observation encode included; README.md:27-52)."""
+    out = {"workload": "env_step", "envs": {}}
+    iters = max(20, 10 * reps)
+    for n in (8192, 65536, 262144):
+        env = pkg.Env(n)
+        env.init(0)
+        rec = torch.empty(n, 996, dtype=torch.uint8, device="cuda")
+
+        def full():
+            env.step(None)
+            env.reset()
+            env.record_obs(rec)
+
+        def play():
+            env.step(None)
+            env.reset()
+
+        for _ in range(300):          # spread the episodes' phases before timing
+            full()
+        torch.cuda.synchronize()
+        ms_full = _time(torch, full, iters)
+        ms_play = _time(torch, play, iters)
+        cnt, _ = env.reset_list()
+        out["envs"][str(n)] = {
+            "us_per_step_all": round(ms_full * 1e3, 1), "M_env_steps_per_s": round(n / ms_full / 1e3, 1),
+            "us_step_and_reset": round(ms_play * 1e3, 1), "M_env_steps_per_s_without_records": round(n / ms_play / 1e3, 1),
+            "finished_envs_last_step": cnt,
+        }
+        env.close()
+    return out
+
+
+def rollout_in_the_loop(pkg, torch, reps):
+    """cu_rollout_step with everything on the device (the reference's `run` mode,
+    craftax_full.cu:12127-12176): h256x3 policy in the loop, fresh worlds on reset."""
+    out = {"workload": "rollout_in_the_loop", "policy": "h256x3 fp32", "envs": {}}
+    T = 8
+    for n in (8192, 65536, 262144):
+        env = pkg.Env(n)
+        env.init(0)
+        pol = pkg.Policy(n, layers=3, seed=1)
+        tr = pkg.Trainer(pol, T)
+        state = {"t": 0}
+
+        def step():
+            env.rollout_step(tr, state["t"] % T, 1234)
+            state["t"] += 1
+
+        for _ in range(40):
+            step()
+        torch.cuda.synchronize()
+        ms = _time(torch, step, max(16, 4 * reps))
+        out["envs"][str(n)] = {"us_per_step": round(ms * 1e3, 1), "M_env_steps_per_s": round(n / ms / 1e3, 2),
+                               "frac_fp32_peak_of_forward_flops": round(FWD_FLOP * n / (ms * 1e-3) / 1e12 / PEAK_FP32, 3)}
+        tr.close()
+        env.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=10)
@@ -383,7 +450,7 @@ def main():
     pkg = ge.load_package()
     assert torch.cuda.is_available(), "bench_configs.py needs a GPU"
     for fn in (forward_65536, ppo_update, ppo_update_shapes, rollout_policy_side, classic_1m,
-               record_kernels, stream_ceilings):
+               record_kernels, stream_ceilings, env_step, rollout_in_the_loop):
         if args.only and fn.__name__ != args.only:
             continue
         print(json.dumps(fn(pkg, torch, args.reps)), flush=True)

@@ -215,20 +215,45 @@ struct Hot {
     uint32_t plant_mask;    // bit i = growing_plants_mask[i]
 };
 
-CFE_FN void unlock(Hot& h, int a) { h.ach[a >> 5] |= 1u << (a & 31); }
-CFE_FN void unlock_if(Hot& h, int a, bool c) { h.ach[a >> 5] |= (uint32_t)c << (a & 31); }
-CFE_FN bool has(const Hot& h, int a) { return (h.ach[a >> 5] >> (a & 31)) & 1u; }
+// An empty asm the value passes through.  Reading element i of a small array of the register
+// struct is a chain of selects over all its elements; the optimiser would rewrite a select of
+// two loads as one load from a selected address, and that runtime address keeps the whole
+// struct in (scratch) memory.  A value that went through here is no longer a load.
+CFE_FN int opaque(int x) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm("" : "+v"(x));
+#else
+    asm("" : "+r"(x));
+#endif
+    return x;
+}
+// (no runtime index into the register struct: a select per word)
+CFE_FN void unlock_if(Hot& h, int a, bool c) {
+    const uint32_t bit = (uint32_t)c << (a & 31);
+    const int w = a >> 5;
+    h.ach[0] |= w == 0 ? bit : 0u;
+    h.ach[1] |= w == 1 ? bit : 0u;
+    h.ach[2] |= w == 2 ? bit : 0u;
+}
+CFE_FN void unlock(Hot& h, int a) { unlock_if(h, a, true); }
+CFE_FN bool has(const Hot& h, int a) {
+    const int w = a >> 5;
+    const uint32_t word = (uint32_t)(w == 0 ? opaque((int)h.ach[0]) : (w == 1 ? opaque((int)h.ach[1]) : opaque((int)h.ach[2])));
+    return (word >> (a & 31)) & 1u;
+}
 template <int N>
 CFE_FN int pick(const int32_t (&a)[N], int i) {
-    int v = a[0];
+    // prvalues on both arms: a conditional between two lvalues is an lvalue, i.e. a select of
+    // addresses, which keeps the whole register struct in memory
+    int v = opaque(a[0]);
 #pragma unroll
-    for (int k = 1; k < N; k++) v = (i == k) ? a[k] : v;
+    for (int k = 1; k < N; k++) v = (i == k) ? opaque(a[k]) : v;
     return v;
 }
 template <int N>
 CFE_FN void put(int32_t (&a)[N], int i, int v) {
 #pragma unroll
-    for (int k = 0; k < N; k++) a[k] = (i == k) ? v : a[k];
+    for (int k = 0; k < N; k++) a[k] = (i == k) ? v : opaque(a[k]);
 }
 
 CFE_FN int max_health(const Hot& h) { return 8 + h.str; }
@@ -504,7 +529,7 @@ CFE_FN void craft(S& s, Hot& h, int action) {
         default: break;
     }
     if (tier != 0) {
-        const int have = is_pickaxe ? h.pickaxe : h.sword;
+        const int have = is_pickaxe ? opaque(h.pickaxe) : opaque(h.sword);
         const int diamonds = is_pickaxe ? 3 : 2;
         bool ok = have < tier && h.wood >= 1;
         if (tier == 2) ok = ok && h.stone >= 1;
@@ -857,7 +882,7 @@ CFE_FN void shoot_or_cast(S& s, Hot& h, int action) {
         }
     } else if (action == A_CAST_FIREBALL || action == A_CAST_ICEBALL) {
         const int which = action - A_CAST_FIREBALL;
-        if (h.mana >= 2 && h.spell[which] && launch_player_projectile(s, h, 2 + which)) {
+        if (h.mana >= 2 && (which ? opaque(h.spell[1]) : opaque(h.spell[0])) && launch_player_projectile(s, h, 2 + which)) {
             unlock(h, which ? ACH_CAST_ICEBALL : ACH_CAST_FIREBALL);
             h.mana -= 2;
         }
@@ -896,7 +921,7 @@ CFE_FN void read_book(Hot& h, uint64_t key, int action) {
     }
     unlock(h, which ? ACH_LEARN_ICEBALL : ACH_LEARN_FIREBALL);
     h.books -= 1;
-    h.spell[which] = 1;
+    if (which) h.spell[1] = 1; else h.spell[0] = 1;
 }
 
 // craftax_enchant_native (:5369-5458)
@@ -907,7 +932,7 @@ CFE_FN void enchant(S& s, Hot& h, int action, uint64_t key) {
     const int b = s.blk(wrap_clamp(h.level, kLevels), wrap_clamp(h.pr + d.r, kMap), wrap_clamp(h.pc + d.c, kMap));
     const bool fire = b == B_ENCH_FIRE, ice = b == B_ENCH_ICE;
     const int kind = fire ? 1 : 2;
-    const int gems = fire ? h.ruby : h.sapphire;
+    const int gems = fire ? opaque(h.ruby) : opaque(h.sapphire);
     if (!(h.mana >= 9 && (fire || ice) && gems >= 1)) return;
     bool done = false;
     if (action == A_ENCHANT_BOW && h.bow > 0) {
@@ -1287,9 +1312,11 @@ CFE_FN SpawnPlan plan_spawns(S& s, const Hot& h, uint64_t rng) {
     const float melee_base = l == 0 ? 0.02f : 0.06f;
     const float night_gain = l == 0 ? 0.1f : 0.0f;
     int count[3], slot[3];
+#pragma unroll
     for (int w = 0; w < 3; w++) {
         const int pool = spawn_pool(w), slots = w == 2 ? 2 : 3;
         int n = 0, first = 0;
+#pragma unroll
         for (int i = slots - 1; i >= 0; i--) {
             const bool m = s.m_mask(pool, i);
             n += (int)m;
@@ -1304,14 +1331,14 @@ CFE_FN SpawnPlan plan_spawns(S& s, const Hot& h, uint64_t rng) {
     p.type[0] = (int8_t)floor_mob_type(l, MC_PASSIVE);
     s.set_m_type(P_PASSIVE, slot[0], p.type[0]);
 
-    p.type[1] = (int8_t)floor_mob_type(boss ? h.boss_progress : l, MC_MELEE);
+    p.type[1] = (int8_t)floor_mob_type(boss ? (int)h.boss_progress : (int)l, MC_MELEE);
     const uint64_t melee_prob = next_key(rng);
     const float night = 1.0f - h.light_level;
     const float melee_chance = melee_base + night_gain * night * night;
     p.key[1] = next_key(rng);
     s.set_m_type(P_MELEE, slot[1], p.type[1]);
 
-    p.type[2] = (int8_t)floor_mob_type(boss ? h.boss_progress : l, MC_RANGED);
+    p.type[2] = (int8_t)floor_mob_type(boss ? (int)h.boss_progress : (int)l, MC_RANGED);
     const uint64_t ranged_prob = next_key(rng);
     p.key[2] = next_key(rng);
     s.set_m_type(P_RANGED, slot[2], p.type[2]);
@@ -1342,6 +1369,7 @@ CFE_FN void place_spawn(S& s, int l, int which, const SpawnPlan& p, int row, int
 template <class S>
 CFE_FN void run_spawns(S& s, const Hot& h, const SpawnPlan& p) {
     const int l = wrap_clamp(h.level, kLevels);
+#pragma unroll
     for (int w = 0; w < 3; w++) {
         if (!((p.tries >> w) & 1)) continue;
         int row, col;
@@ -1433,10 +1461,20 @@ CFE_FN void update_intrinsics(Hot& h, int action) {
 // craftax_clip_inventory_and_intrinsics_native, craftax_calculate_inventory_achievements_native
 // (:4440-4547)
 CFE_FN void clip_and_count(Hot& h) {
-    int32_t* inv[] = {&h.wood, &h.stone, &h.coal, &h.iron, &h.diamond, &h.sapling, &h.pickaxe, &h.sword,
-                      &h.bow, &h.arrows, &h.torches, &h.ruby, &h.sapphire, &h.books};
-#pragma unroll
-    for (int i = 0; i < 14; i++) *inv[i] = imin(*inv[i], 99);
+    h.wood = imin(h.wood, 99);
+    h.stone = imin(h.stone, 99);
+    h.coal = imin(h.coal, 99);
+    h.iron = imin(h.iron, 99);
+    h.diamond = imin(h.diamond, 99);
+    h.sapling = imin(h.sapling, 99);
+    h.pickaxe = imin(h.pickaxe, 99);
+    h.sword = imin(h.sword, 99);
+    h.bow = imin(h.bow, 99);
+    h.arrows = imin(h.arrows, 99);
+    h.torches = imin(h.torches, 99);
+    h.ruby = imin(h.ruby, 99);
+    h.sapphire = imin(h.sapphire, 99);
+    h.books = imin(h.books, 99);
 #pragma unroll
     for (int i = 0; i < 4; i++) h.armour[i] = imin(h.armour[i], 99);
 #pragma unroll

@@ -360,63 +360,61 @@ __device__ __forceinline__ void load_hot_dev(const EnvArrays& A, size_t e, Hot& 
     h.plant_mask = A.plant_mask[e];
 }
 
-// Only what differs from `o` is written: most scalars of an env stay put in a step.
-__device__ __forceinline__ void store_hot_dev(const EnvArrays& A, size_t e, const Hot& h, const Hot& o) {
+// Every scalar is written back: a field is one 256-byte row per wavefront, and keeping the
+// step's input around to compare against would double the registers an env holds.
+__device__ __forceinline__ void store_hot_dev(const EnvArrays& A, size_t e, const Hot& h) {
     const size_t n = (size_t)A.n;
-#define CFE_PUT(arr, idx, a, b) \
-    if ((a) != (b)) A.arr[idx] = (a);
-    CFE_PUT(player_position, e, h.pr, o.pr)
-    CFE_PUT(player_position, n + e, h.pc, o.pc)
-    CFE_PUT(player_level, e, h.level, o.level)
-    CFE_PUT(player_direction, e, h.dir, o.dir)
-    if (__float_as_uint(h.health) != __float_as_uint(o.health)) A.player_health[e] = h.health;
-    CFE_PUT(player_food, e, h.food, o.food)
-    CFE_PUT(player_drink, e, h.drink, o.drink)
-    CFE_PUT(player_energy, e, h.energy, o.energy)
-    CFE_PUT(player_mana, e, h.mana, o.mana)
-    if (h.sleeping != o.sleeping) A.is_sleeping[e] = (uint8_t)h.sleeping;
-    if (h.resting != o.resting) A.is_resting[e] = (uint8_t)h.resting;
+    A.player_position[e] = h.pr;
+    A.player_position[n + e] = h.pc;
+    A.player_level[e] = h.level;
+    A.player_direction[e] = h.dir;
+    A.player_health[e] = h.health;
+    A.player_food[e] = h.food;
+    A.player_drink[e] = h.drink;
+    A.player_energy[e] = h.energy;
+    A.player_mana[e] = h.mana;
+    A.is_sleeping[e] = (uint8_t)h.sleeping;
+    A.is_resting[e] = (uint8_t)h.resting;
     A.player_recover[e] = h.recover;
     A.player_hunger[e] = h.hunger;
     A.player_thirst[e] = h.thirst;
     A.player_fatigue[e] = h.fatigue;
     A.player_recover_mana[e] = h.recover_mana;
-    CFE_PUT(player_xp, e, h.xp, o.xp)
-    CFE_PUT(player_dexterity, e, h.dex, o.dex)
-    CFE_PUT(player_strength, e, h.str, o.str)
-    CFE_PUT(player_intelligence, e, h.intel, o.intel)
-    CFE_PUT(inv_wood, e, h.wood, o.wood)
-    CFE_PUT(inv_stone, e, h.stone, o.stone)
-    CFE_PUT(inv_coal, e, h.coal, o.coal)
-    CFE_PUT(inv_iron, e, h.iron, o.iron)
-    CFE_PUT(inv_diamond, e, h.diamond, o.diamond)
-    CFE_PUT(inv_sapling, e, h.sapling, o.sapling)
-    CFE_PUT(inv_pickaxe, e, h.pickaxe, o.pickaxe)
-    CFE_PUT(inv_sword, e, h.sword, o.sword)
-    CFE_PUT(inv_bow, e, h.bow, o.bow)
-    CFE_PUT(inv_arrows, e, h.arrows, o.arrows)
+    A.player_xp[e] = h.xp;
+    A.player_dexterity[e] = h.dex;
+    A.player_strength[e] = h.str;
+    A.player_intelligence[e] = h.intel;
+    A.inv_wood[e] = h.wood;
+    A.inv_stone[e] = h.stone;
+    A.inv_coal[e] = h.coal;
+    A.inv_iron[e] = h.iron;
+    A.inv_diamond[e] = h.diamond;
+    A.inv_sapling[e] = h.sapling;
+    A.inv_pickaxe[e] = h.pickaxe;
+    A.inv_sword[e] = h.sword;
+    A.inv_bow[e] = h.bow;
+    A.inv_arrows[e] = h.arrows;
 #pragma unroll
-    for (int i = 0; i < 4; i++) CFE_PUT(inv_armour, i * n + e, h.armour[i], o.armour[i])
-    CFE_PUT(inv_torches, e, h.torches, o.torches)
-    CFE_PUT(inv_ruby, e, h.ruby, o.ruby)
-    CFE_PUT(inv_sapphire, e, h.sapphire, o.sapphire)
+    for (int i = 0; i < 4; i++) A.inv_armour[i * n + e] = h.armour[i];
+    A.inv_torches[e] = h.torches;
+    A.inv_ruby[e] = h.ruby;
+    A.inv_sapphire[e] = h.sapphire;
 #pragma unroll
-    for (int i = 0; i < 6; i++) CFE_PUT(inv_potions, i * n + e, h.potions[i], o.potions[i])
-    CFE_PUT(inv_books, e, h.books, o.books)
-    if (h.spell[0] != o.spell[0]) A.learned_spells[e] = (uint8_t)h.spell[0];
-    if (h.spell[1] != o.spell[1]) A.learned_spells[n + e] = (uint8_t)h.spell[1];
-    CFE_PUT(sword_enchantment, e, h.sword_ench, o.sword_ench)
-    CFE_PUT(bow_enchantment, e, h.bow_ench, o.bow_ench)
+    for (int i = 0; i < 6; i++) A.inv_potions[i * n + e] = h.potions[i];
+    A.inv_books[e] = h.books;
+    A.learned_spells[e] = (uint8_t)h.spell[0];
+    A.learned_spells[n + e] = (uint8_t)h.spell[1];
+    A.sword_enchantment[e] = h.sword_ench;
+    A.bow_enchantment[e] = h.bow_ench;
 #pragma unroll
-    for (int i = 0; i < 4; i++) CFE_PUT(armour_enchantments, i * n + e, h.armour_ench[i], o.armour_ench[i])
-    CFE_PUT(boss_progress, e, h.boss_progress, o.boss_progress)
-    CFE_PUT(boss_timesteps_to_spawn_this_round, e, h.boss_timer, o.boss_timer)
+    for (int i = 0; i < 4; i++) A.armour_enchantments[i * n + e] = h.armour_ench[i];
+    A.boss_progress[e] = h.boss_progress;
+    A.boss_timesteps_to_spawn_this_round[e] = h.boss_timer;
     A.light_level[e] = h.light_level;
     A.timestep[e] = h.timestep;
 #pragma unroll
-    for (int w = 0; w < 3; w++) CFE_PUT(ach_bits, w * n + e, h.ach[w], o.ach[w])
-    CFE_PUT(plant_mask, e, h.plant_mask, o.plant_mask)
-#undef CFE_PUT
+    for (int w = 0; w < 3; w++) A.ach_bits[w * n + e] = h.ach[w];
+    A.plant_mask[e] = h.plant_mask;
 }
 
 // run_spawns of env_logic.h by the whole wavefront: for each lane that rolled a spawn, lane
@@ -494,7 +492,6 @@ __global__ __launch_bounds__(kWave) void k_env_step(EnvArrays A, const float* __
 
     Hot h;
     load_hot_dev(A, e, h);
-    const Hot before = h;
     DevStore s{A, lds + lane, A.planes + e * kEnvPlaneBytes, light, (int)e, 0, 0};
 
     int action;
@@ -510,7 +507,7 @@ __global__ __launch_bounds__(kWave) void k_env_step(EnvArrays A, const float* __
     const StepOut out = step(s, h, action, keys.step_rng, plan);
     run_spawns_wave(s, h, plan, lane);
     s.close_level();
-    store_hot_dev(A, e, h, before);
+    store_hot_dev(A, e, h);
     A.state_rng[e] = (uint32_t)out.state_rng;
     A.state_rng[n + e] = (uint32_t)(out.state_rng >> 32);
     A.rng_key[e] = (uint32_t)keys.env_key;
@@ -643,7 +640,7 @@ struct FieldList {          // the per-field arrays of one EnvArrays, for table-
 };
 
 // k_env_init / k_reset_list_block (craftax_full.cu:8669-8706, 8957-8975): one workgroup per
-// env.  LIST: the envs of the reset list, world key from each record's reset key, the env's
+// floor of an env.  LIST: the envs of the reset list, world key from each record's reset key, the env's
 // own key kept.  Otherwise: envs [0, A.n), env i created from seed0 + i as c_init does.
 template <bool LIST>
 __global__ __launch_bounds__(kGenThreads) void k_env_worldgen(EnvArrays A, FieldList fl, const float* __restrict__ light,
@@ -656,8 +653,11 @@ __global__ __launch_bounds__(kGenThreads) void k_env_worldgen(EnvArrays A, Field
     BlockGroup g{(int)threadIdx.x, fred, ired};
     const int t = threadIdx.x;
     const size_t n = (size_t)A.n;
-    const int total = LIST ? *reset_count : A.n;
-    for (int idx = blockIdx.x; idx < total; idx += gridDim.x) {
+    // one workgroup per (env, floor): the nine floors of a world are independent, and a step
+    // waits for its slowest reset
+    const int total = (LIST ? *reset_count : A.n) * kLevels;
+    for (int job = blockIdx.x; job < total; job += gridDim.x) {
+        const int idx = job / kLevels, level = job - idx * kLevels;
         size_t e;
         uint64_t world_key, env_key = 0;
         if (LIST) {
@@ -668,77 +668,78 @@ __global__ __launch_bounds__(kGenThreads) void k_env_worldgen(EnvArrays A, Field
             env_key = lcg(seed_key((uint32_t)(seed0 + (uint64_t)idx)));
             world_key = world_key_of_reset(lcg(env_key));
         }
-        // scalars: the fields of `fl` are zero in a fresh state; the others are written below
-        for (int f = 0; f < zero_fields; f++) {
-            const int el = fl.elem[f];
-            for (int k = t; k < fl.count[f]; k += kGenThreads) {
-                const size_t at = (size_t)k * n + e;
-                if (el == 4) ((uint32_t*)fl.ptr[f])[at] = 0u;
-                else if (el == 8) ((uint64_t*)fl.ptr[f])[at] = 0ull;
-                else ((uint8_t*)fl.ptr[f])[at] = 0;
+        if (level == 0) {
+            // scalars: the fields of `fl` are zero in a fresh state; the others are written below
+            for (int f = 0; f < zero_fields; f++) {
+                const int el = fl.elem[f];
+                for (int k = t; k < fl.count[f]; k += kGenThreads) {
+                    const size_t at = (size_t)k * n + e;
+                    if (el == 4) ((uint32_t*)fl.ptr[f])[at] = 0u;
+                    else if (el == 8) ((uint64_t*)fl.ptr[f])[at] = 0ull;
+                    else ((uint8_t*)fl.ptr[f])[at] = 0;
+                }
             }
-        }
-        for (int k = t; k < kMobSlots; k += kGenThreads) A.mob_health[(size_t)k * n + e] = (k / 27 == P_RANGED && k % 3 == 2) ? 0.0f : 1.0f;
-        for (int k = t; k < 54; k += kGenThreads) {
-            A.mob_projectile_directions[(size_t)k * n + e] = 1;
-            A.player_projectile_directions[(size_t)k * n + e] = 1;
-        }
-        if (t < kLevels) A.monsters_killed[(size_t)t * n + e] = t == 0 ? 10 : 0;
-        if (t == 0) {
-            int32_t perm[6];
-            potion_permutation(world_key, perm);
-            for (int i = 0; i < 6; i++) A.potion_mapping[(size_t)i * n + e] = perm[i];
-            const uint64_t sk = world_state_key(world_key);
-            A.state_rng[e] = (uint32_t)sk;
-            A.state_rng[n + e] = (uint32_t)(sk >> 32);
-            A.player_position[e] = kMap / 2;
-            A.player_position[n + e] = kMap / 2;
-            A.player_direction[e] = A_UP;
-            A.player_health[e] = 9.0f;
-            A.player_food[e] = 9;
-            A.player_drink[e] = 9;
-            A.player_energy[e] = 9;
-            A.player_mana[e] = 9;
-            A.player_dexterity[e] = 1;
-            A.player_strength[e] = 1;
-            A.player_intelligence[e] = 1;
-            A.boss_timesteps_to_spawn_this_round[e] = 7;
-            A.light_level[e] = light[0];
-            if (!LIST) {
-                A.rng_key[e] = (uint32_t)env_key;
-                A.rng_key[n + e] = (uint32_t)(env_key >> 32);
+            for (int k = t; k < kMobSlots; k += kGenThreads)
+                A.mob_health[(size_t)k * n + e] = (k / 27 == P_RANGED && k % 3 == 2) ? 0.0f : 1.0f;
+            for (int k = t; k < 54; k += kGenThreads) {
+                A.mob_projectile_directions[(size_t)k * n + e] = 1;
+                A.player_projectile_directions[(size_t)k * n + e] = 1;
+            }
+            if (t < kLevels) A.monsters_killed[(size_t)t * n + e] = t == 0 ? 10 : 0;
+            if (t == 0) {
+                int32_t perm[6];
+                potion_permutation(world_key, perm);
+                for (int i = 0; i < 6; i++) A.potion_mapping[(size_t)i * n + e] = perm[i];
+                const uint64_t sk = world_state_key(world_key);
+                A.state_rng[e] = (uint32_t)sk;
+                A.state_rng[n + e] = (uint32_t)(sk >> 32);
+                A.player_position[e] = kMap / 2;
+                A.player_position[n + e] = kMap / 2;
+                A.player_direction[e] = A_UP;
+                A.player_health[e] = 9.0f;
+                A.player_food[e] = 9;
+                A.player_drink[e] = 9;
+                A.player_energy[e] = 9;
+                A.player_mana[e] = 9;
+                A.player_dexterity[e] = 1;
+                A.player_strength[e] = 1;
+                A.player_intelligence[e] = 1;
+                A.boss_timesteps_to_spawn_this_round[e] = 7;
+                A.light_level[e] = light[0];
+                if (!LIST) {
+                    A.rng_key[e] = (uint32_t)env_key;
+                    A.rng_key[n + e] = (uint32_t)(env_key >> 32);
+                }
             }
         }
         uint8_t* planes = A.planes + e * kEnvPlaneBytes;
-        for (int level = 0; level < kLevels; level++) {
-            generate_floor(g, sc, world_key, level);
-            // the three byte planes, 16 bytes a thread
-            for (int k = t; k < 3 * (int)(kPlaneBytes / 16); k += kGenThreads) {
-                const int plane = k / (int)(kPlaneBytes / 16), off = k % (int)(kPlaneBytes / 16);
-                const uint8_t* src = plane == 0 ? sc.map : (plane == 1 ? sc.item : sc.light);
-                ((u4*)(planes + ((size_t)plane * kLevels + level) * kPlaneBytes))[off] = ((const u4*)src)[off];
-            }
-            // spawn bit planes of the level (craftax_refresh_spawn_bits_level), no mobs yet
-            if (t < kMap) {
-                uint64_t all = 0, grave = 0, water = 0;
-                for (int c = 0; c < kMap; c++) {
-                    const int b = sc.map[t * kMap + c];
-                    all |= (uint64_t)in_set(kSpawnAll, b) << c;
-                    grave |= (uint64_t)in_set(kSpawnGrave, b) << c;
-                    water |= (uint64_t)in_set(kSpawnWater, b) << c;
-                }
-                const size_t at = (size_t)(level * kMap + t) * n + e;
-                A.spawn_all_bits[at] = all;
-                A.spawn_grave_bits[at] = grave;
-                A.spawn_water_bits[at] = water;
-                A.mob_bits[at] = 0;
-            }
-            if (t < 2) {
-                A.down_ladders[(size_t)(level * 2 + t) * n + e] = sc.ladder_down[t];
-                A.up_ladders[(size_t)(level * 2 + t) * n + e] = sc.ladder_up[t];
-            }
-            __syncthreads();
+        generate_floor(g, sc, world_key, level);
+        // the three byte planes, 16 bytes a thread
+        for (int k = t; k < 3 * (int)(kPlaneBytes / 16); k += kGenThreads) {
+            const int plane = k / (int)(kPlaneBytes / 16), off = k % (int)(kPlaneBytes / 16);
+            const uint8_t* src = plane == 0 ? sc.map : (plane == 1 ? sc.item : sc.light);
+            ((u4*)(planes + ((size_t)plane * kLevels + level) * kPlaneBytes))[off] = ((const u4*)src)[off];
         }
+        // spawn bit planes of the level (craftax_refresh_spawn_bits_level), no mobs yet
+        if (t < kMap) {
+            uint64_t all = 0, grave = 0, water = 0;
+            for (int c = 0; c < kMap; c++) {
+                const int b = sc.map[t * kMap + c];
+                all |= (uint64_t)in_set(kSpawnAll, b) << c;
+                grave |= (uint64_t)in_set(kSpawnGrave, b) << c;
+                water |= (uint64_t)in_set(kSpawnWater, b) << c;
+            }
+            const size_t at = (size_t)(level * kMap + t) * n + e;
+            A.spawn_all_bits[at] = all;
+            A.spawn_grave_bits[at] = grave;
+            A.spawn_water_bits[at] = water;
+            A.mob_bits[at] = 0;
+        }
+        if (t < 2) {
+            A.down_ladders[(size_t)(level * 2 + t) * n + e] = sc.ladder_down[t];
+            A.up_ladders[(size_t)(level * 2 + t) * n + e] = sc.ladder_up[t];
+        }
+        __syncthreads();
     }
 }
 
@@ -978,7 +979,7 @@ int cfp_env_init(cfp_env* e, uint64_t seed, void* stream) {
     CFP_REQUIRE(e != nullptr, "cfp_env_init: NULL env");
     cfp::FieldList fl;
     const int m = cfp::zero_field_list(e->live, fl);
-    const int grid = e->live.n < 4096 ? e->live.n : 4096;
+    const int grid = e->live.n * cfp::kLevels < 8192 ? e->live.n * cfp::kLevels : 8192;
     hipLaunchKernelGGL(cfp::k_env_worldgen<false>, dim3(grid), dim3(cfp::kGenThreads), 0, (hipStream_t)stream, e->live, fl,
                        e->light, nullptr, nullptr, seed, m);
     CFP_HIP_TRY(hipGetLastError());
@@ -990,7 +991,8 @@ int cfp_env_pool_fill(cfp_env* e, uint64_t seed, void* stream) {
     CFP_REQUIRE(e->pool_size > 0, "cfp_env_pool_fill: this env object was created without a reset pool");
     cfp::FieldList fl;
     const int m = cfp::zero_field_list(e->pool, fl);
-    hipLaunchKernelGGL(cfp::k_env_worldgen<false>, dim3(e->pool_size < 4096 ? e->pool_size : 4096), dim3(cfp::kGenThreads), 0,
+    hipLaunchKernelGGL(cfp::k_env_worldgen<false>, dim3(e->pool_size * cfp::kLevels < 8192 ? e->pool_size * cfp::kLevels : 8192),
+                       dim3(cfp::kGenThreads), 0,
                        (hipStream_t)stream, e->pool, fl, e->light, nullptr, nullptr, seed, m);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
@@ -1001,7 +1003,7 @@ int cfp_env_reset(cfp_env* e, void* stream) {
     cfp::FieldList fl;
     const int m = cfp::zero_field_list(e->live, fl);
     // the list is short (a fraction of a percent of the envs per step): a fixed grid strides it
-    const int grid = e->live.n < 1024 ? e->live.n : 1024;
+    const int grid = e->live.n * cfp::kLevels < 4608 ? e->live.n * cfp::kLevels : 4608;
     hipLaunchKernelGGL(cfp::k_env_worldgen<true>, dim3(grid), dim3(cfp::kGenThreads), 0, (hipStream_t)stream, e->live, fl,
                        e->light, e->resets, e->reset_count, 0ull, m);
     CFP_HIP_TRY(hipGetLastError());

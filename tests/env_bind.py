@@ -65,8 +65,9 @@ def diff_fields(a, b):
 class Ref:
     """oracle/_ref/libcfref.so: the reference's own env, one global vector of envs."""
 
-    def __init__(self):
-        path = os.path.join(ROOT, "oracle", "_ref", "libcfref.so")
+    def __init__(self, strict=False):
+        """strict: the same source built with strict per-operation fp32 (oracle/Makefile)."""
+        path = os.path.join(ROOT, "oracle", "_ref", "libcfref_strict.so" if strict else "libcfref.so")
         if not os.path.exists(path):
             raise FileNotFoundError(path)
         self.lib = lib = C.CDLL(path)
@@ -128,8 +129,15 @@ class HostStep:
         lib.cfhost_light_table.argtypes = [C.c_void_p, C.c_int]
         lib.cfhost_step.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 5
         lib.cfhost_derive_spawn_planes.argtypes = [C.c_void_p, C.c_int]
+        lib.cfhost_generate.argtypes = [C.c_uint32, C.c_int, C.c_void_p]
+        lib.cfhost_reset.argtypes = [C.c_void_p, C.c_void_p]
         self.light = np.zeros(100001, np.float32)
         lib.cfhost_light_table(ptr(self.light), len(self.light))
+
+    def generate(self, seed, n):
+        out = np.zeros(n, STATE_DTYPE)
+        self.lib.cfhost_generate(seed, n, ptr(out))
+        return out
 
     def step(self, states, actions):
         n = len(states)

@@ -115,3 +115,52 @@ def test_encoder_matches_reference_live():
             assert np.array_equal(got, env.encode(i % 64)), f"fuzz seed {99000 + i}"
     finally:
         env.close()
+
+
+def test_stock_flag_build_differs_only_in_tail_floats_by_one_ulp():
+    """oracle/Makefile builds the compiled-reference checker with -mno-recip added to the
+    reference's own flags and says what that changes: nothing in the map bytes, rewards and
+    terminals; tail floats by at most one ulp.  Held here against a build with the stock
+    flags over config 1's first 200 steps (1024 envs, seed 0, the xorshift32 % 43 actions)."""
+    import ctypes as C
+    import hashlib
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    stock_path = os.path.join(root, "oracle", "_ref", "libcfref_stock.so")
+    stamp = os.path.join(root, "oracle", "_ref", "stock_build_cpu.txt")
+    if not (os.path.exists(stock_path) and os.path.exists(stamp)):
+        pytest.skip("stock-flag build of the reference not present")
+    flags = next(l for l in open("/proc/cpuinfo") if l.startswith("flags"))
+    if hashlib.md5(flags.encode()).hexdigest() != open(stamp).read().split()[0]:
+        pytest.skip("the stock-flag build (-march=native) was made on another CPU")
+    libs = []
+    for name in ("libcfref.so", "libcfref_stock.so"):
+        lib = C.CDLL(os.path.join(root, "oracle", "_ref", name))
+        lib.cfref_init.argtypes = [C.c_int, C.c_uint64]
+        lib.cfref_observations.restype = C.POINTER(C.c_uint8)
+        lib.cfref_rewards.restype = C.POINTER(C.c_float)
+        lib.cfref_terminals.restype = C.POINTER(C.c_float)
+        lib.cfref_init(1024, 0)
+        libs.append(lib)
+    worst_ulp, moved = 0, set()
+    for t in range(200):
+        out = []
+        for lib in libs:
+            lib.cfref_step()
+            obs = np.ctypeslib.as_array(lib.cfref_observations(), shape=(1024, 996)).copy()
+            rew = np.ctypeslib.as_array(lib.cfref_rewards(), shape=(1024,)).copy()
+            term = np.ctypeslib.as_array(lib.cfref_terminals(), shape=(1024,)).copy()
+            out.append((obs, rew, term))
+        (o0, r0, t0), (o1, r1, t1) = out
+        assert np.array_equal(o0[:, :792], o1[:, :792]), f"map bytes differ at step {t}"
+        assert np.array_equal(r0.view(np.uint32), r1.view(np.uint32)), f"rewards differ at step {t}"
+        assert np.array_equal(t0, t1), f"terminals differ at step {t}"
+        a = o0[:, 792:].copy().view(np.uint32).astype(np.int64)
+        b = o1[:, 792:].copy().view(np.uint32).astype(np.int64)
+        d = np.abs(a - b)
+        worst_ulp = max(worst_ulp, int(d.max()))
+        moved |= set(np.nonzero(d.any(axis=0))[0].tolist())
+    # the square roots of the tail: ten inventory counts (0..9) and six potion counts (16..21)
+    assert worst_ulp <= 1, worst_ulp
+    assert moved <= set(range(0, 10)) | set(range(16, 22)), sorted(moved)
