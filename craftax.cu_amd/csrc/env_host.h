@@ -204,6 +204,7 @@ struct HostStore {
     }
     void set_plant_age(int i, int a) { st->growing_plants_age[i] = a; }
     void open_level(int l) { lvl = l; }
+    void stamp(int) {}
     float light_at(int t) const { return light[t < kMaxTimesteps ? t : kMaxTimesteps]; }
 };
 

@@ -404,6 +404,7 @@ CFE_FN float achievement_reward(int a) {  // CRAFTAX_ACHIEVEMENT_REWARD_MAP, :34
 //   int potion_effect(i); int plant_r(i), plant_c(i), plant_age(i) / set_plant(i, r, c), set_plant_age(i, a)
 //   void open_level(l): called once per step when the step's level is known
 //   float light_at(timestep)
+//   void stamp(k): phase boundary k of the step passed (a hook for timing builds; empty otherwise)
 
 // craftax_set_map_block (:3325-3334): the block and its three spawn bits
 template <class S>
@@ -1229,31 +1230,67 @@ constexpr uint32_t ring_row_const(int ring, int adr) {
     }
     return m;
 }
+// The allowed offsets of a ring row are a centred run minus a centred run: half-widths + 1 (0 =
+// empty), one nibble per |dr|, derived from ring_row_const at compile time.
+constexpr int run_half_width(uint32_t m) {   // widest w with bits 13-w .. 13+w all set, +1; 0 if bit 13 is clear
+    int w = 0;
+    while (w <= kDespawn - 1 && ((m >> (kDespawn - 1 - w)) & 1u) && ((m >> (kDespawn - 1 + w)) & 1u)) w++;
+    return w;
+}
+constexpr uint32_t centred_run(int w1) { return w1 ? ((1u << (2 * w1 - 1)) - 1u) << (kDespawn - w1) : 0u; }
+constexpr uint64_t pack_outer(int ring) {
+    uint64_t t = 0;
+    for (int a = 0; a < kDespawn; a++) {
+        const uint32_t m = ring_row_const(ring, a);
+        int w = 0;   // the row's extent: widest set offset + 1
+        for (int dc = 0; dc < kDespawn; dc++)
+            if ((m >> (kDespawn - 1 + dc)) & 1u) w = dc + 1;
+        t |= (uint64_t)w << (4 * a);
+    }
+    return t;
+}
+constexpr uint64_t pack_inner(int ring, uint64_t outer_table) {   // the hole around dc = 0, as a centred run
+    uint64_t t = 0;
+    for (int a = 0; a < kDespawn; a++) {
+        const uint32_t outer = centred_run((int)((outer_table >> (4 * a)) & 15));
+        t |= (uint64_t)run_half_width(outer & ~ring_row_const(ring, a)) << (4 * a);
+    }
+    return t;
+}
+constexpr uint64_t kRingOuter[3] = {pack_outer(RING_PASSIVE), pack_outer(RING_HOSTILE), pack_outer(RING_BOSS)};
+constexpr uint64_t kRingInner[3] = {pack_inner(RING_PASSIVE, kRingOuter[0]), pack_inner(RING_HOSTILE, kRingOuter[1]),
+                                    pack_inner(RING_BOSS, kRingOuter[2])};
+constexpr bool ring_table_holds(int ring) {
+    for (int a = 0; a < kDespawn; a++)
+        if (ring_row_const(ring, a) != (centred_run((int)((kRingOuter[ring] >> (4 * a)) & 15)) &
+                                        ~centred_run((int)((kRingInner[ring] >> (4 * a)) & 15))))
+            return false;
+    return true;
+}
+static_assert(ring_table_holds(0) && ring_table_holds(1) && ring_table_holds(2),
+              "ring rows are a centred run minus a centred run");
 CFE_FN uint32_t ring_row(int ring, int adr) {
-#define CFE_RING_CASE(k)                                                          \
-    case k: {                                                                     \
-        constexpr uint32_t p = ring_row_const(RING_PASSIVE, k), q = ring_row_const(RING_HOSTILE, k), \
-                           b = ring_row_const(RING_BOSS, k);                      \
-        return ring == RING_PASSIVE ? p : (ring == RING_HOSTILE ? q : b);         \
-    }
-    switch (adr) {
-        CFE_RING_CASE(0) CFE_RING_CASE(1) CFE_RING_CASE(2) CFE_RING_CASE(3) CFE_RING_CASE(4)
-        CFE_RING_CASE(5) CFE_RING_CASE(6) CFE_RING_CASE(7) CFE_RING_CASE(8) CFE_RING_CASE(9)
-        CFE_RING_CASE(10) CFE_RING_CASE(11) CFE_RING_CASE(12) CFE_RING_CASE(13)
-        default: return 0;
-    }
-#undef CFE_RING_CASE
+    constexpr uint64_t o0 = kRingOuter[0], o1 = kRingOuter[1], o2 = kRingOuter[2];
+    constexpr uint64_t i0 = kRingInner[0], i1 = kRingInner[1], i2 = kRingInner[2];
+    const uint64_t outer = ring == RING_PASSIVE ? o0 : (ring == RING_HOSTILE ? o1 : o2);
+    const uint64_t inner = ring == RING_PASSIVE ? i0 : (ring == RING_HOSTILE ? i1 : i2);
+    const int w = (int)((outer >> (4 * adr)) & 15), v = (int)((inner >> (4 * adr)) & 15);
+    const uint32_t a = w ? ((1u << (2 * w - 1)) - 1u) << (kDespawn - w) : 0u;
+    const uint32_t b = v ? ((1u << (2 * v - 1)) - 1u) << (kDespawn - v) : 0u;
+    return a & ~b;
 }
 // open cells of map row pr + dr in the ring: the terrain plane, minus mobs, inside the map
 template <class S>
 CFE_FN uint64_t spawn_candidates(S& s, const Hot& h, int l, int ring, int kind, int dr) {
+    // no branch around the two loads: a row off the map reads row 0 and is masked out, so that
+    // a caller that unrolls over the rows gets all its loads in flight together
     const int r = h.pr + dr;
-    if ((unsigned)r >= (unsigned)kMap) return 0;
+    const bool live = (unsigned)r < (unsigned)kMap;
+    const int rr = live ? r : 0;
     const uint64_t shape = ring_row(ring, iabs(dr));
     const int sh = h.pc - (kDespawn - 1);
-    const uint64_t cols = (sh >= 0 ? shape << sh : shape >> -sh) & kRowMask;
-    if (cols == 0) return 0;
-    return s.spawnrow(kind, l, r) & ~s.mobrow(l, r) & cols;
+    const uint64_t cols = live ? ((sh >= 0 ? shape << sh : shape >> -sh) & kRowMask) : 0ull;
+    return s.spawnrow(kind, l, rr) & ~s.mobrow(l, rr) & cols;
 }
 // craftax_spawn_pick_kth (:7694-7704): the smallest k with k + 1 >= n * (1 - u)
 CFE_FN int pick_index(int n, uint64_t key) {
@@ -1526,9 +1563,11 @@ CFE_FN StepOut step(S& s, Hot& h, int action, uint64_t rng, SpawnPlan& plan) {
 
     change_floor(s, h, action);
     s.open_level(wrap_clamp(h.level, kLevels));
+    s.stamp(2);
     craft(s, h, action);
     uint64_t key = next_key(rng);
     if (action == A_DO) do_action(s, h, key);
+    s.stamp(3);
     place_block(s, h, action);
     shoot_or_cast(s, h, action);
     drink_potion(s, h, action);
@@ -1538,13 +1577,16 @@ CFE_FN StepOut step(S& s, Hot& h, int action, uint64_t rng, SpawnPlan& plan) {
     enchant(s, h, action, key);
     boss_and_attributes(h, action);
     move_player(s, h, action);
+    s.stamp(4);
     key = next_key(rng);
     update_mobs(s, h, key);
+    s.stamp(5);
     key = next_key(rng);
     plan = plan_spawns(s, h, key);
     grow_plants(s, h);
     update_intrinsics(h, action);
     clip_and_count(h);
+    s.stamp(6);
 
     float reward = 0.0f;
 #pragma unroll

@@ -15,10 +15,8 @@
 // slot, the mob standing on a cell, ...); they are staged in LDS as [word][lane] -- 24 KB
 // per wavefront, conflict-free for any per-lane word index -- and written back slot by
 // slot if touched.  The spawn scan (27 rows of 48-bit bitmaps around the player, asked for
-// by ~2 % of the envs per step) would leave 63 lanes idle per request if the asking lane
-// did it alone, so it is run by the wavefront after every lane is through its step: lane j
-// takes row j of the ring, counts candidates with one popcount, a prefix sum over the
-// lanes places the drawn index, the lane that owns the row extracts the column.
+// by 5-15 % of the envs per step) runs after every lane is through its step, with the
+// wavefront converged: the asking lanes scan together, their 54 row loads in flight at once.
 //
 // Arithmetic that the hot path is bound by: each env step moves ~0.3 KB of scalars in and
 // out as whole rows plus ~0.8 KB of mob slots plus a few dozen single-byte map cells (one
@@ -252,6 +250,7 @@ struct DevStore {
         A.plant_pos[at(2 * i + 1)] = c;
     }
     __device__ __forceinline__ void set_plant_age(int i, int a) { A.plant_age[at(i)] = a; }
+    __device__ __forceinline__ void stamp(int) {}
     __device__ __forceinline__ float light_at(int t) const { return light[t < kMaxTimesteps ? t : kMaxTimesteps]; }
 
     __device__ __forceinline__ int global_slot(int g) const {  // CFM(pool, lvl, i) of slot g
@@ -417,66 +416,63 @@ __device__ __forceinline__ void store_hot_dev(const EnvArrays& A, size_t e, cons
     A.plant_mask[e] = h.plant_mask;
 }
 
-// run_spawns of env_logic.h by the whole wavefront: for each lane that rolled a spawn, lane
-// j takes map row pr - 13 + j of that env.
-__device__ __forceinline__ void run_spawns_wave(DevStore& s, const Hot& h, const SpawnPlan& plan, int lane) {
-    const EnvArrays& A = s.A;
-    unsigned long long need = __ballot(plan.tries != 0);
-    while (need != 0) {
-        const int src = __ffsll((long long)need) - 1;
-        need &= need - 1;
-        const int pr = __shfl(h.pr, src), pc = __shfl(h.pc, src);
-        const int l = wrap_clamp(__shfl(h.level, src), kLevels);
-        const int tries = __shfl((int)plan.tries, src);
-        const size_t e_src = (size_t)(s.e - lane + src);
-        const int dr = lane - (kDespawn - 1);
-        const int r = pr + dr;
-        const bool live = lane < 2 * kDespawn - 1 && (unsigned)r < (unsigned)kMap;
-        const size_t row_at = (size_t)(l * kMap + (live ? r : 0)) * (size_t)A.n + e_src;
-        uint64_t mob = live ? A.mob_bits[row_at] : ~0ull;
-        const uint64_t mob0 = mob;
-        const int sh = pc - (kDespawn - 1);
+// run_spawns of env_logic.h with the wavefront kept together.  Some 5-15 % of the lanes roll
+// a spawn in a step, nearly all of them for one kind of mob.  Each such lane scans its own 27
+// bitmap rows (54 independent 8-byte loads in flight at once, then popcounts); lanes asking for
+// different kinds run the same pass, since ring and terrain are per-lane values.  The wavefront
+// repeats the pass only while some lane has a second or third kind pending.
+__device__ __forceinline__ void run_spawns_lanes(DevStore& s, const Hot& h, const SpawnPlan& plan) {
+    const int l = wrap_clamp(h.level, kLevels);
+    uint32_t pending = plan.tries;
+    while (__any(pending != 0)) {
+        if (pending != 0) {
+            const int w = __builtin_ctz(pending);
+            pending &= pending - 1;
+            int ring = 0, kind = 0, slot = 0, type = 0, key_lo = 0, key_hi = 0;
 #pragma unroll
-        for (int w = 0; w < 3; w++) {
-            if (!((tries >> w) & 1)) continue;
-            const int ring = __shfl((int)plan.ring[w], src), kind = __shfl((int)plan.kind[w], src);
-            const uint64_t key = (uint64_t)(uint32_t)__shfl((int)(uint32_t)plan.key[w], src) |
-                                 (uint64_t)(uint32_t)__shfl((int)(uint32_t)(plan.key[w] >> 32), src) << 32;
-            uint64_t cand = 0;
-            if (live) {
-                const uint64_t shape = ring_row(ring, iabs(dr));
-                const uint64_t cols = (sh >= 0 ? shape << sh : shape >> -sh) & kRowMask;
-                cand = s.plane_of(kind)[row_at] & ~mob & cols;
+            for (int v = 0; v < 3; v++) {   // values, not addresses, are selected (see opaque)
+                ring = w == v ? opaque(plan.ring[v]) : ring;
+                kind = w == v ? opaque(plan.kind[v]) : kind;
+                slot = w == v ? opaque(plan.slot[v]) : slot;
+                type = w == v ? opaque(plan.type[v]) : type;
+                key_lo = w == v ? opaque((int)(uint32_t)plan.key[v]) : key_lo;
+                key_hi = w == v ? opaque((int)(uint32_t)(plan.key[v] >> 32)) : key_hi;
             }
-            const int cnt = __popcll(cand);
-            int incl = cnt;   // inclusive prefix sum over lanes 0..31 (27 in use)
+            const uint64_t key = (uint64_t)(uint32_t)key_hi << 32 | (uint32_t)key_lo;
+            // pass 1: candidates per row, one byte each (a row has at most 27)
+            uint64_t counts[4] = {0, 0, 0, 0};
+            int n = 0;
+#pragma unroll 9
+            for (int j = 0; j < 2 * kDespawn - 1; j++) {   // nine rows' loads in flight at a time
+                const int cnt = __popcll(spawn_candidates(s, h, l, ring, kind, j - (kDespawn - 1)));
+                counts[j >> 3] |= (uint64_t)cnt << (8 * (j & 7));
+                n += cnt;
+            }
+            if (n != 0) {
+                // pass 2: the row holding the drawn candidate, then that row once more
+                int k = pick_index(n, key);
+                int jrow = 0;
+                bool found = false;
 #pragma unroll
-            for (int d = 1; d < 32; d <<= 1) {
-                const int up = __shfl_up(incl, d);
-                if (lane >= d) incl += up;
-            }
-            const int total = __shfl(incl, 2 * kDespawn - 2);
-            if (total == 0) continue;
-            const int k = pick_index(total, key);
-            const bool mine = live && k >= incl - cnt && k < incl;
-            int col = 0;
-            if (mine) {
-                uint64_t m = cand;
-                for (int j = k - (incl - cnt); j > 0; j--) m &= m - 1;
-                col = __ffsll((long long)m) - 1;
-                mob |= 1ull << col;
-            }
-            const int owner = __ffsll((long long)__ballot(mine)) - 1;
-            const int row = pr + owner - (kDespawn - 1);
-            col = __shfl(col, owner);
-            if (lane == src) {
+                for (int j = 0; j < 2 * kDespawn - 1; j++) {
+                    const int cnt = (int)((counts[j >> 3] >> (8 * (j & 7))) & 0xff);
+                    if (!found && k < cnt) {
+                        jrow = j;
+                        found = true;
+                    }
+                    k -= found ? 0 : cnt;
+                }
+                uint64_t m = spawn_candidates(s, h, l, ring, kind, jrow - (kDespawn - 1));
+                for (; k > 0; k--) m &= m - 1;
+                const int row = h.pr + jrow - (kDespawn - 1);
+                const int col = __ffsll((long long)m) - 1;
                 const int pool = spawn_pool(w);
-                s.set_m_pos(pool, plan.slot[w], row, col);
-                s.set_m_hp(pool, plan.slot[w], mob_health(plan.type[w], spawn_class(w)));
-                s.set_m_mask(pool, plan.slot[w], true);
+                s.set_m_pos(pool, slot, row, col);
+                s.set_m_hp(pool, slot, mob_health(type, spawn_class(w)));
+                s.set_m_mask(pool, slot, true);
+                s.put_mobrow(l, row, s.mobrow(l, row) | (1ull << col));
             }
         }
-        if (live && mob != mob0) A.mob_bits[row_at] = mob;
     }
 }
 
@@ -505,9 +501,9 @@ __global__ __launch_bounds__(kWave) void k_env_step(EnvArrays A, const float* __
     const StepKeys keys = split_env_key((uint64_t)A.rng_key[n + e] << 32 | A.rng_key[e]);
     SpawnPlan plan;
     const StepOut out = step(s, h, action, keys.step_rng, plan);
-    run_spawns_wave(s, h, plan, lane);
+    store_hot_dev(A, e, h);    // before the scans: they need the position only
+    run_spawns_lanes(s, h, plan);
     s.close_level();
-    store_hot_dev(A, e, h);
     A.state_rng[e] = (uint32_t)out.state_rng;
     A.state_rng[n + e] = (uint32_t)(out.state_rng >> 32);
     A.rng_key[e] = (uint32_t)keys.env_key;
