@@ -227,7 +227,7 @@ constexpr int kSweepEnvs = 1;   // envs (wavefronts) per workgroup: the best of 
 template <bool TWO_GRADS, bool HIGHWAY, bool G16>
 __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-    const int env = (int)blockIdx.x * kSweepEnvs + wave;   // mb % 32 == 0: whole wavefronts only
+    const int env = (int)blockIdx.x * kSweepEnvs + wave;   // one wavefront per env of the minibatch
     const unsigned lane_off = (threadIdx.x & 63u) * 16u;   // units 4q .. 4q+3 of a 1 KiB fp32 row
     const unsigned lane_off8 = (threadIdx.x & 63u) * 8u;   // ... of a 512-byte bf16 row
     // wavefront-uniform row pointers of this env; a step back in time is one stride
@@ -814,8 +814,10 @@ int launch_adam(cfp_policy* p, float* grads, float* m, float* v, const uint64_t*
     const int items = a.enc_items + a.mid_items + a.tail_items;
     hipLaunchKernelGGL(k_adam_mirrors, dim3((items + 255) / 256), dim3(256), 0, st, a);
     CFP_HIP_TRY(hipGetLastError());
-    // the 16-env-tile kernel's mirrors, when that mode is on, take one pack launch
-    if (p->small_tiles && p->t16) return launch_pack_weights_t16(p->params, L, p->t16, st);
+    // the 16-env-tile kernel's mirrors take one more pack launch.  Always, not only while that
+    // mode is on: the switch can be flipped after this step (or after a capture of it), and a
+    // forward on 16-env tiles must never see weights from before an update
+    if (p->t16) return launch_pack_weights_t16(p->params, L, p->t16, st);
     return 0;
 }
 

@@ -153,6 +153,7 @@ struct RecWhich {
     const unsigned char* list;
     size_t list_stride;
     const int* count;
+    int max_count;   // the list form never reads past this many entries, whatever *count says
 };
 
 constexpr int kWPos = (int)(offsetof(cfp_env_scalars, player_position) / 4);
@@ -192,7 +193,7 @@ __global__ __launch_bounds__(256) void k_record_obs(
             if ((int)threadIdx.x == i) ptrs[i] = soa.p[i];
         if ((int)threadIdx.x < kScalarWords) words[threadIdx.x] = kSoaWords[threadIdx.x];
     }
-    const int total = which.list ? *which.count : n;
+    const int total = which.list ? min(*which.count, which.max_count) : n;
     // the trip count is the same for every thread of the workgroup (barriers inside)
     for (int first = (int)blockIdx.x * kGather; first < total; first += (int)gridDim.x * kGather) {
         if (SOA) {
@@ -203,7 +204,8 @@ __global__ __launch_bounds__(256) void k_record_obs(
             int genv = gi;
             if (which.list && gi < total)
                 genv = *reinterpret_cast<const int32_t*>(which.list + (size_t)gi * which.list_stride);
-            if (gi < total && !(which.skip && which.skip[genv])) {
+            // a list entry outside the env range is ignored (never used as an index)
+            if (gi < total && (unsigned)genv < (unsigned)n && !(which.skip && which.skip[genv])) {
                 const int lvl = static_cast<const int32_t*>(ptrs[1])[genv];
                 const int lvl_c = lvl < 0 ? 0 : (lvl > 8 ? 8 : lvl);   // monsters_killed has nine entries
                 const int ml3 = 3 * jax_index(lvl, 9);
@@ -235,6 +237,7 @@ __global__ __launch_bounds__(256) void k_record_obs(
             int env = item;
             if (which.list)
                 env = *reinterpret_cast<const int32_t*>(which.list + (size_t)item * which.list_stride);
+            if ((unsigned)env >= (unsigned)n) continue;
             if (which.skip && which.skip[env]) continue;
             uint32_t* stage = stage_all[slot];
             WordSrc s;
@@ -555,6 +558,7 @@ int cfp_record_obs_soa_list(const cfp_env_soa* soa, const uint8_t* d_map,
     w.list = static_cast<const unsigned char*>(d_env_list);
     w.list_stride = list_stride;
     w.count = d_count;
+    w.max_count = max_count;
     return record_obs_soa(soa, d_map, d_item_map, d_light_map, env_stride, level_stride, w,
                           max_count, d_rec_row, n, stream);
 }

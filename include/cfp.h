@@ -234,9 +234,14 @@ int cfp_gemm_enc_fwd(int cols, const float* d_W_enc, const float* d_xobs,
 int cfp_gemm_dh(int m3, int cols, const float* d_W, const float* d_dpre,
                 float* d_dh, void* stream);
 /* cfp_gemm_dh for callers that cannot allocate (code under graph capture, serving loops,
- * harnesses that forbid hipMalloc); no counterpart in the reference.  Same result as
- * cfp_gemm_dh, but the split mirror of W sits in a 1.125 MiB array inside the library's
- * device image instead of the process-wide workspace, so the call never allocates.
+ * harnesses that forbid hipMalloc); no counterpart in the reference.  Same result, bit for
+ * bit, as cfp_gemm_dh in the split modes (cfp_set_gemm_split 1, the default, and 2) with fp32
+ * inputs; in split mode 0 or with cfp_set_gemm_bf16(1) cfp_gemm_dh runs other kernels and
+ * this call still runs the split kernel (nine terms in mode 0).  The split mirror of W sits
+ * in a 1.125 MiB array inside the library's device image instead of the process-wide
+ * workspace, so the call never allocates.  The first call on a GPU resolves that array's
+ * address (hipGetSymbolAddress, which may load the code object): make one call outside any
+ * graph capture first.
  * Limits: m3 a multiple of 16 up to 768, cols a multiple of 32, d_dpre 16-byte aligned;
  * anything else is an error.  Calls on one GPU share that GPU's array: calls that overlap
  * (two streams, two threads) race on it. */
@@ -364,8 +369,9 @@ int cfp_record_obs_soa(const cfp_env_soa* soa, const uint8_t* d_map, const uint8
 /* k_record_obs_list (craftax_full.cu:9303-9320): records only the envs named by the
  * first *d_count entries of a device index list; entry i is the int32 at d_env_list +
  * i * list_stride bytes (a CraftaxResetRec array with its .env member: pass the address
- * of the first .env and sizeof(CraftaxResetRec)).  max_count (<= n) bounds *d_count and
- * sizes the launch; n is the env count the rows and arrays are laid out for. */
+ * of the first .env and sizeof(CraftaxResetRec)).  max_count (<= n) sizes the launch and
+ * bounds the list: entries past min(*d_count, max_count) are never read, and an entry
+ * outside 0..n-1 is skipped.  n is the env count the rows and arrays are laid out for. */
 int cfp_record_obs_soa_list(const cfp_env_soa* soa, const uint8_t* d_map,
                             const uint8_t* d_item_map, const uint8_t* d_light_map,
                             size_t env_stride, size_t level_stride, const void* d_env_list,

@@ -202,10 +202,25 @@ def rel_err(got, ref):
     return float(np.max(np.abs(got - ref) / (np.abs(ref) + rms)))
 
 
+def strict_rel_err(got, ref):
+    """max of |got-ref| / |ref| over the entries with |ref| >= rms(ref): the plain relative
+    error where it is well defined (entries that are not the result of a cancellation)."""
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    big = (np.abs(ref) >= np.sqrt(np.mean(ref * ref))) & (ref != 0)
+    if not big.any():
+        return 0.0
+    return float(np.max(np.abs(got - ref)[big] / np.abs(ref)[big]))
+
+
 def assert_close(got, ref, tol, what):
+    """Two bounds: |got-ref| <= tol * (|ref| + rms(ref)) for every entry, and the plain
+    |got-ref| <= tol * |ref| for every entry at least as large as the rms."""
     e = rel_err(got, ref)
     assert np.all(np.isfinite(np.asarray(got))), f"{what}: non-finite values"
     assert e <= tol, f"{what}: relative error {e:.3e} exceeds {tol:.1e}"
+    es = strict_rel_err(got, ref)
+    assert es <= tol, f"{what}: plain relative error {es:.3e} of the large entries exceeds {tol:.1e}"
     return e
 
 

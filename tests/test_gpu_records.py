@@ -318,3 +318,13 @@ def test_record_obs_from_reference_soa_layout(pkg, cuda, golden):
     torch.cuda.synchronize()
     got3 = rec3.cpu().numpy()
     assert np.array_equal(got3[5], want[5]) and np.all(np.delete(got3, 5, axis=0) == 0xEE)
+    # a device count above max_count and entries outside the env range: the list is read up
+    # to max_count only, out-of-range entries are skipped, every other row stays untouched
+    rec4 = torch.full((n, 996), 0xEE, dtype=torch.uint8, device=cuda)
+    bad = torch.tensor([3, -7, n + 100, 9, 11, 12], dtype=torch.int32, device=cuda)
+    pkg.policy.record_obs_soa_list(arrays, n_stride, planes, planes[P:], planes[2 * P:], n, P3, 0,
+                                   bad, 4, torch.tensor([1000000], dtype=torch.int32, device=cuda), 4, rec4)
+    torch.cuda.synchronize()
+    got4 = rec4.cpu().numpy()
+    assert np.array_equal(got4[[3, 9]], want[[3, 9]])
+    assert np.all(np.delete(got4, [3, 9], axis=0) == 0xEE)

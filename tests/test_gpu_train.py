@@ -515,6 +515,33 @@ def test_adam_writes_every_weight_mirror(pkg, cuda):
     tr.close(); pol.close(); twin.close()
 
 
+def test_small_tile_mirrors_current_when_switched_on_after_training(pkg, cuda):
+    """Adam steps taken with 16-env tiles off, eager and as a captured update, then the
+    switch is turned on: the small-tile forward must run on the updated weights (equal,
+    bit for bit, to a fresh policy given the same parameters)."""
+    import torch
+    n = 64
+    pol = pkg.Policy(n, L, seed=41)
+    tr = pkg.Trainer(pol, 4)
+    rng = np.random.default_rng(42)
+    for _ in range(2):
+        g = (rng.standard_normal(pol.param_count) * 0.1).astype(np.float32)
+        tr.buf("grads").copy_(_t(g, cuda))
+        tr.adam()
+    torch.cuda.synchronize()
+    pol.set_small_tiles(True)
+    twin = pkg.Policy(n, L, seed=99)
+    twin.set_params(pol.get_params())
+    twin.set_small_tiles(True)
+    rec = _t(synth_records_host(n, 43, 0), cuda)
+    term = torch.zeros(n, device=cuda)
+    s0 = (0.5 * rng.standard_normal((L, n, HIDDEN))).astype(np.float32)
+    sa, sb = _t(s0, cuda), _t(s0, cuda)
+    assert torch.equal(pol.forward(rec, term, sa), twin.forward(rec, term, sb))
+    assert torch.equal(sa, sb)
+    tr.close(); pol.close(); twin.close()
+
+
 @pytest.mark.parametrize("n,T,minibatches,bwd_win,done_p,layers,seed",
                          [(64, 8, 1, 0, 0.1, 3, 234), (128, 6, 2, 4, 0.15, 3, 298),
                           # one and two layers: the stream of every kernel of the chain changes
