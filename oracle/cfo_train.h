@@ -31,6 +31,16 @@ typedef struct cfo_ppo_batch {
 double cfo_ppo_loss_f64(const float* params, const cfo_ppo_batch* b, double* loss3);
 void cfo_ppo_backward_f64(const float* params, const cfo_ppo_batch* b, double* grads,
                           double* loss3);
+/* cfo_ppo_backward_f64 with both operands of every matrix product rounded to bf16 and the
+ * accumulation kept in fp64: the comparator of the bf16-input / fp32-accumulate update.
+ * flags bit 0: also round what cfp_train_set_bf16_storage stores as bf16.
+ * flags bit 1: the 768 leading map-byte rows of dW_enc multiply the unrounded encoder
+ * gradient (the update with the split kernels switched off). */
+void cfo_ppo_backward_bf16ops_f64(const float* params, const cfo_ppo_batch* b, double* grads,
+                                  double* loss3, int flags);
+/* min |zh| over the minibatch's recompute: the distance of the batch from the kink of the
+ * candidate function, where the gradient is discontinuous. */
+double cfo_ppo_min_abs_zh(const float* params, const cfo_ppo_batch* b, int bf16_ops);
 void cfo_gae_f64(const float* values, const float* rewards, const uint8_t* dones,
                  const float* v_boot, double* adv, double* ret, int n, int T,
                  double gamma, double lam);

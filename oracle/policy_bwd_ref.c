@@ -23,6 +23,31 @@
 
 enum { H = CFP_HIDDEN, G = CFP_GRU, F = CFP_OBS, A = CFP_ACTIONS };
 
+/* bf16-operand mode: every operand of a matrix product (encoder, gate and actor GEMMs of
+ * the forward; dW, dh and dW_enc GEMMs of the backward) is rounded to bf16 -- an
+ * activation or gradient from its fp32 value, a weight from its fp32 value -- while
+ * products and sums stay fp64.  This is the arithmetic of the library's bf16-input /
+ * fp32-accumulate update with the accumulation made exact: what remains between it and
+ * the device result is fp32 accumulation order and the fp32 elementwise work.  The value
+ * row rides with the 43 actor rows in one 44-row head GEMM in the forward and in both
+ * backward GEMMs of the head, so W_v, dv and h3 are rounded there as well. */
+static int g_q = 0, g_map_exact = 0;
+#pragma omp threadprivate(g_q, g_map_exact)
+static double qb(double v) {
+    float f = (float)v;
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+    memcpy(&f, &u, 4);
+    return (double)f;
+}
+static double qa(double v) { return g_q ? qb(v) : v; }   /* activation / gradient operand */
+/* g_q == 2: the window workspace of the backward is stored as bf16 as well
+ * (cfp_train_set_bf16_storage): gate pre-activations and layer inputs as the sweep reads
+ * them, gate gradients and the highway term as it writes them, and the outputs of the
+ * dh GEMMs (the layer-0 one adds the stored highway term and rounds the sum). */
+static double qs(double v) { return g_q == 2 ? qb(v) : v; }
+
 static double sig(double x) { return 1.0 / (1.0 + exp(-x)); }
 static double gfun(double x) { return x >= 0.0 ? x + 0.5 : sig(x); }
 static double dgfun(double x) {
@@ -68,22 +93,24 @@ static void step_forward(const Weights* w, int L, const uint8_t* rec, Step* s) {
     cfo_expand_record(rec, s->feat);
     for (int k = 0; k < H; k++) s->x[0][k] = (double)w->b_enc[k];
     for (int f = 0; f < F; f++) {
-        const double xf = (double)s->feat[f];
+        const double xf = qa((double)s->feat[f]);
         if (xf == 0.0) continue;
-        const float* wr = w->W_enc + (size_t)f * H;
+        const float* wr = w->W_enc + (size_t)f * H;   /* W_enc / W_gru / W_a: pre-rounded in bf16 mode */
         for (int k = 0; k < H; k++) s->x[0][k] += xf * (double)wr[k];
     }
     for (int l = 0; l < L; l++) {
         const float* Wl = w->W_gru + (size_t)l * G * H;
+        double xq[H];
+        for (int j = 0; j < H; j++) xq[j] = qa(s->x[l][j]);
         for (int k = 0; k < H; k++) {
             double zh = 0, zg = 0, zp = 0;
             const float* a = Wl + (size_t)k * H;
             const float* bq = Wl + (size_t)(H + k) * H;
             const float* c = Wl + (size_t)(2 * H + k) * H;
             for (int j = 0; j < H; j++) {
-                zh += (double)a[j] * s->x[l][j];
-                zg += (double)bq[j] * s->x[l][j];
-                zp += (double)c[j] * s->x[l][j];
+                zh += (double)a[j] * xq[j];
+                zg += (double)bq[j] * xq[j];
+                zp += (double)c[j] * xq[j];
             }
             s->zh[l][k] = zh; s->zg[l][k] = zg; s->zp[l][k] = zp;
             const double st = s->s_in[l][k];
@@ -103,9 +130,11 @@ static void head_terms(const Weights* w, const cfo_ppo_batch* b, const double* h
                        double* dv) {
     double lg[A], pi[A];
     double mx = -1e300;
+    double h3q[H];
+    for (int j = 0; j < H; j++) h3q[j] = qa(h3[j]);
     for (int a = 0; a < A; a++) {
         double z = (double)w->b_a[a];
-        for (int j = 0; j < H; j++) z += (double)w->W_a[a * H + j] * h3[j];
+        for (int j = 0; j < H; j++) z += (double)w->W_a[a * H + j] * h3q[j];
         lg[a] = z;
         if (z > mx) mx = z;
     }
@@ -125,7 +154,7 @@ static void head_terms(const Weights* w, const cfo_ppo_batch* b, const double* h
     double Hent = 0.0;
     for (int a = 0; a < A; a++) Hent -= pi[a] * (lg[a] - lse);
     double v = (double)w->b_v[0];
-    for (int j = 0; j < H; j++) v += (double)w->W_v[j] * h3[j];
+    for (int j = 0; j < H; j++) v += (double)w->W_v[j] * h3q[j];
     const double dret = v - (double)b->ret[o];
     *l_pg = -(u1 < u2 ? u1 : u2);
     *l_v = 0.5 * dret * dret;
@@ -186,8 +215,35 @@ double cfo_ppo_loss_f64(const float* params, const cfo_ppo_batch* b, double* los
  * recompute from the STORED state at every step, reverse sweep with a live
  * dcarry that is cut at t == T-1 and at BPTT segment ends and blocked by
  * done_t.  grads (param layout, fp64) is overwritten. */
+static void ppo_backward(const float* params, const cfo_ppo_batch* b, double* grads,
+                         double* loss3, int bf16_ops);
+
 void cfo_ppo_backward_f64(const float* params, const cfo_ppo_batch* b, double* grads,
                           double* loss3) {
+    ppo_backward(params, b, grads, loss3, 0);
+}
+
+/* A copy of the parameters with the four weight matrices rounded to bf16 (biases as they are). */
+static float* bf16_weights(const float* params, int L) {
+    const size_t pc = (size_t)CFP_PARAM_COUNT(L);
+    float* pq = (float*)malloc(pc * sizeof(float));
+    memcpy(pq, params, pc * sizeof(float));
+    for (size_t i = CFP_OFF_W_ENC; i < (size_t)CFP_OFF_B_ENC; i++) pq[i] = (float)qb(pq[i]);
+    for (size_t i = CFP_OFF_W_GRU; i < (size_t)CFP_OFF_B_A(L); i++) pq[i] = (float)qb(pq[i]);   /* W_gru, W_a */
+    for (size_t i = CFP_OFF_W_V(L); i < (size_t)CFP_OFF_W_V(L) + CFP_HIDDEN; i++) pq[i] = (float)qb(pq[i]);
+    return pq;
+}
+
+/* The same update with every matrix-product operand rounded to bf16 (see qb above). */
+void cfo_ppo_backward_bf16ops_f64(const float* params, const cfo_ppo_batch* b, double* grads,
+                                  double* loss3, int flags) {
+    float* pq = bf16_weights(params, b->layers);
+    ppo_backward(pq, b, grads, loss3, (flags & 1 ? 2 : 1) | (flags & 2 ? 4 : 0));
+    free(pq);
+}
+
+static void ppo_backward(const float* params, const cfo_ppo_batch* b, double* grads,
+                         double* loss3, int bf16_ops) {
     const int L = b->layers, T = b->T;
     const Weights w = split(params, L);
     const size_t pc = (size_t)CFP_PARAM_COUNT(L);
@@ -208,6 +264,8 @@ void cfo_ppo_backward_f64(const float* params, const cfo_ppo_batch* b, double* g
 #ifdef _OPENMP
         tid = omp_get_thread_num();
 #endif
+        g_q = bf16_ops & 3;
+        g_map_exact = (bf16_ops & 4) != 0;
         double* g = gbuf + pc * (size_t)tid;
         double* gW_enc = g + CFP_OFF_W_ENC;
         double* gb_enc = g + CFP_OFF_B_ENC;
@@ -236,17 +294,20 @@ void cfo_ppo_backward_f64(const float* params, const cfo_ppo_batch* b, double* g
                 head_terms(&w, b, s->x[L], o, amean, ainv, inv_batch, &lp, &lv, &le,
                            dlog, &dv);
                 s_pg += lp; s_v += lv; s_e += le;
-                double dh[H], dhx[H], dhn[H];
-                for (int k = 0; k < H; k++) dh[k] = dv * (double)w.W_v[k];
+                double dh[H], dhx[H], dhn[H], h3q[H];
+                for (int k = 0; k < H; k++) dh[k] = qa(dv) * (double)w.W_v[k];
+                for (int k = 0; k < H; k++) h3q[k] = qa(s->x[L][k]);
                 for (int a = 0; a < A; a++) {
                     gb_a[a] += dlog[a];
+                    const double dq = qa(dlog[a]);
                     for (int k = 0; k < H; k++) {
-                        dh[k] += (double)w.W_a[a * H + k] * dlog[a];
-                        gW_a[a * H + k] += dlog[a] * s->x[L][k];
+                        dh[k] += (double)w.W_a[a * H + k] * dq;
+                        gW_a[a * H + k] += dq * h3q[k];
                     }
                 }
+                for (int k = 0; k < H; k++) dh[k] = qs(dh[k]);
                 gb_v[0] += dv;
-                for (int k = 0; k < H; k++) gW_v[k] += dv * s->x[L][k];
+                for (int k = 0; k < H; k++) gW_v[k] += qa(dv) * h3q[k];
                 memset(dhx, 0, sizeof(dhx));
                 const int cut = (t == T - 1) || ((t + 1) % b->seg_len) == 0;
                 const int done_t = b->r_done[o] != 0;
@@ -257,44 +318,60 @@ void cfo_ppo_backward_f64(const float* params, const cfo_ppo_batch* b, double* g
                     for (int k = 0; k < H; k++) {
                         if (cut) dc[l][k] = 0.0;
                         const double dhout = dh[k] + dhx[k];
-                        const double sgv = sig(s->zg[l][k]);
-                        const double gh = gfun(s->zh[l][k]);
-                        const double p = sig(s->zp[l][k]);
+                        const double zh = qs(s->zh[l][k]);
+                        const double sgv = sig(qs(s->zg[l][k]));
+                        const double gh = gfun(zh);
+                        const double p = sig(qs(s->zp[l][k]));
                         const double s_in = s->s_in[l][k];
                         const double out = s_in + sgv * (gh - s_in);
                         const double dout = dhout * p + (done_t ? 0.0 : dc[l][k]);
-                        dpre[2 * H + k] = dhout * (out - s->x[l][k]) * p * (1.0 - p);
-                        dhx[k] = dhout * (1.0 - p);
+                        dpre[2 * H + k] = qs(dhout * (out - qs(s->x[l][k])) * p * (1.0 - p));
+                        dhx[k] = qs(dhout * (1.0 - p));
                         dc[l][k] = dout * (1.0 - sgv);
-                        dpre[H + k] = dout * (gh - s_in) * sgv * (1.0 - sgv);
-                        dpre[k] = dout * sgv * dgfun(s->zh[l][k]);
+                        dpre[H + k] = qs(dout * (gh - s_in) * sgv * (1.0 - sgv));
+                        dpre[k] = qs(dout * sgv * dgfun(zh));
                     }
                     memset(dhn, 0, sizeof(dhn));
+                    double xq[H];
+                    for (int j = 0; j < H; j++) xq[j] = qa(s->x[l][j]);
                     for (int r = 0; r < G; r++) {
-                        const double d = dpre[r];
+                        const double d = qa(dpre[r]);
                         if (d == 0.0) continue;
                         const float* wr = Wl + (size_t)r * H;
                         double* gr = gWl + (size_t)r * H;
                         for (int j = 0; j < H; j++) {
-                            gr[j] += d * s->x[l][j];
+                            gr[j] += d * xq[j];
                             dhn[j] += (double)wr[j] * d;
                         }
                     }
-                    memcpy(dh, dhn, sizeof(dh));
+                    if (l > 0)
+                        for (int k = 0; k < H; k++) dh[k] = qs(dhn[k]);
+                    else
+                        memcpy(dh, dhn, sizeof(dh));
                 }
                 for (int k = 0; k < H; k++) {
-                    dh[k] += dhx[k];
+                    dh[k] = qs(dh[k] + dhx[k]);
                     gb_enc[k] += dh[k];
                 }
+                /* dW_enc straight from the records: the 768 leading map bytes are exact in
+                 * bf16 and multiply either dh_enc rounded like every other operand of the
+                 * mode (split kernels on) or an exact three-term bf16 split of it (split
+                 * kernels off: g_map_exact); the other 75 features go through the mode's
+                 * GEMM either way. */
+                double dhq[H];
+                for (int k = 0; k < H; k++) dhq[k] = qa(dh[k]);
                 for (int f = 0; f < F; f++) {
-                    const double xf = (double)s->feat[f];
+                    const double xf = qa((double)s->feat[f]);
                     if (xf == 0.0) continue;
                     double* gr = gW_enc + (size_t)f * H;
-                    for (int k = 0; k < H; k++) gr[k] += xf * dh[k];
+                    const double* d = (f < 768 && g_map_exact) ? dh : dhq;
+                    for (int k = 0; k < H; k++) gr[k] += xf * d[k];
                 }
             }
         }
         free(steps);
+        g_q = 0;
+        g_map_exact = 0;
     }
     for (int t = 0; t < nth; t++) {
         const double* g = gbuf + pc * (size_t)t;
@@ -302,6 +379,37 @@ void cfo_ppo_backward_f64(const float* params, const cfo_ppo_batch* b, double* g
     }
     free(gbuf);
     if (loss3) { loss3[0] = s_pg; loss3[1] = s_v; loss3[2] = s_e; }
+}
+
+/* Smallest |zh| over every (step, env of the minibatch, layer, unit) of the recompute.  The
+ * candidate g(zh) = zh + 0.5 (zh >= 0) / sigmoid(zh) (craftax_full.cu:9357) is continuous at
+ * zero but its derivative jumps from 1/4 to 1 there, so the update's gradient is
+ * discontinuous in the parameters wherever a zh is zero: a batch with a zh inside fp32
+ * rounding of zero has two equally valid gradients, and a test that compares an fp32
+ * evaluation with this oracle has to know.  bf16_ops: the zh of the bf16-operand update. */
+double cfo_ppo_min_abs_zh(const float* params, const cfo_ppo_batch* b, int bf16_ops) {
+    const int L = b->layers, T = b->T;
+    float* pq = bf16_ops ? bf16_weights(params, L) : NULL;
+    const Weights w = split(pq ? pq : params, L);
+    double best = 1e300;
+    g_q = bf16_ops ? 1 : 0;
+    Step* s = (Step*)malloc(sizeof(Step));
+    for (int el = 0; el < b->mb; el++) {
+        const int env = b->env_start + el;
+        for (int t = 0; t < T; t++) {
+            for (int l = 0; l < L; l++)
+                for (int k = 0; k < H; k++)
+                    s->s_in[l][k] = (double)b->r_state[rstate_off(b, t, l, env) + k];
+            step_forward(&w, L, b->r_obs + ((size_t)t * b->n + env) * CFP_REC_BYTES, s);
+            for (int l = 0; l < L; l++)
+                for (int k = 0; k < H; k++)
+                    if (fabs(s->zh[l][k]) < best) best = fabs(s->zh[l][k]);
+        }
+    }
+    free(s);
+    free(pq);
+    g_q = 0;
+    return best;
 }
 
 /* k_gae :10617-10634, in fp64 on fp32 inputs. */

@@ -86,6 +86,9 @@ def cfo():
         lib.cfo_ppo_loss_f64.restype = C.c_double
         lib.cfo_ppo_loss_f64.argtypes = [vp, C.POINTER(PpoBatch), vp]
         lib.cfo_ppo_backward_f64.argtypes = [vp, C.POINTER(PpoBatch), vp, vp]
+        lib.cfo_ppo_min_abs_zh.argtypes = [vp, C.POINTER(PpoBatch), C.c_int]
+        lib.cfo_ppo_min_abs_zh.restype = C.c_double
+        lib.cfo_ppo_backward_bf16ops_f64.argtypes = [vp, C.POINTER(PpoBatch), vp, vp, C.c_int]
         lib.cfo_gae_f64.argtypes = [vp, vp, vp, vp, vp, vp, C.c_int, C.c_int,
                                     C.c_double, C.c_double]
         lib.cfo_adam_f64.argtypes = [vp, vp, vp, vp, C.c_size_t, C.c_int, C.c_double,
@@ -230,6 +233,24 @@ def ppo_backward_f64(params, batch):
     g = np.zeros(params.size)
     l3 = np.zeros(3)
     cfo().cfo_ppo_backward_f64(_p(params), C.byref(batch), _p(g), _p(l3))
+    return g, l3
+
+
+def ppo_min_abs_zh(params, batch, bf16_ops=False):
+    """Distance of the batch from the kink of the candidate function (see cfo_train.h)."""
+    params = np.ascontiguousarray(params, dtype=np.float32)
+    return float(cfo().cfo_ppo_min_abs_zh(_p(params), C.byref(batch), int(bool(bf16_ops))))
+
+
+def ppo_backward_bf16ops_f64(params, batch, bf16_storage=False, map_rows_exact=False):
+    """The update's gradients with every matrix-product operand rounded to bf16 (and, with
+    bf16_storage, what the bf16 window storage rounds), sums in fp64.  map_rows_exact: the
+    map-byte rows of dW_enc multiply the unrounded encoder gradient (split kernels off)."""
+    params = np.ascontiguousarray(params, dtype=np.float32)
+    g = np.zeros(params.size)
+    l3 = np.zeros(3)
+    cfo().cfo_ppo_backward_bf16ops_f64(_p(params), C.byref(batch), _p(g), _p(l3),
+                                       int(bool(bf16_storage)) | 2 * int(bool(map_rows_exact)))
     return g, l3
 
 

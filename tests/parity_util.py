@@ -21,6 +21,8 @@ HIDDEN, GRU, OBS, OBS_MAP, OBS_TAIL = 256, 768, 843, 792, 51
 REC_BYTES, ACTIONS, AV = 996, 43, 44
 TOL_FP32 = 1e-4
 TOL_BF16 = 2e-2
+# a bf16-input result against the fp64 evaluation of the same bf16-rounded operands
+TOL_BF16_OPS = 1e-3
 
 _M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
 
@@ -185,6 +187,107 @@ def numpy_forward_bf16_f64(params, layers, x, state, terminals, obs=None, action
     out["logits"] = q(f32(h)) @ q(w["W_a"]).T + w["b_a"]
     out["values"] = q(f32(h)) @ q(w["W_v"]) + w["b_v"][0]
     return out
+
+
+def numpy_ppo_backward_f64(params, layers, feats, r_state, r_act, r_logprob, adv, ret, r_done,
+                           seg_len, clip=0.2, vf=0.5, ent=0.01, mode=0, map_rows_exact=False):
+    """The PPO update's gradients (recompute from the stored state, reverse sweep with the
+    carry cut at segment ends and blocked at terminal steps; k_head_bwd_win,
+    k_mingru_bwd_win and the GEMMs of cu_train_backward, craftax_full.cu:9635-9689,
+    9560-9620, 13230-13330) in fp64 with library matmuls, over all envs at once.
+    feats [T][n][843], r_state [T][L][n][256].
+    mode 0: exact operands.  mode 1: both operands of every matrix product rounded to bf16
+    (activations and gradients from their fp32 value); with map_rows_exact the 768 leading
+    map bytes multiply the unrounded encoder gradient (an exact three-term split of it, what
+    the update does with the split kernels off).  mode 2: also what the bf16 window storage rounds -- the gate
+    pre-activations and layer inputs as the sweep reads them, the gate gradients and the
+    highway term as written, the outputs of the dh GEMMs.
+    Returns (gradient vector, [pg, v, ent] sums)."""
+    T, n = r_act.shape
+    H = HIDDEN
+    w = {k: v.astype(np.float64) for k, v in split_params(params, layers).items()}
+    f32 = lambda a: np.asarray(a, dtype=np.float64).astype(np.float32)
+    q = (lambda a: bf16_round(f32(a))) if mode else (lambda a: np.asarray(a, dtype=np.float64))
+    qs = (lambda a: bf16_round(f32(a))) if mode == 2 else (lambda a: np.asarray(a, dtype=np.float64))
+    We, Wg, Wa, Wv = q(w["W_enc"]), q(w["W_gru"]), q(w["W_a"]), q(w["W_v"])
+    a64 = adv.astype(np.float32).astype(np.float64)
+    mean = a64.sum() / (n * T)
+    var = max((a64 * a64).sum() / (n * T) - mean * mean, 0.0)
+    inv_std = 1.0 / (np.sqrt(var) + 1e-8)
+    inv_batch = 1.0 / (T * n)
+    clip, vf, ent = (float(np.float32(c)) for c in (clip, vf, ent))
+    g = {k: np.zeros_like(v) for k, v in w.items()}
+    loss3 = np.zeros(3)
+    carry = np.zeros((layers, n, H))
+    rows = np.arange(n)
+    for t in range(T - 1, -1, -1):
+        # ---- recompute
+        x = [q(feats[t]) @ We + w["b_enc"]]
+        zs, outs = [], []
+        for l in range(layers):
+            z = q(x[l]) @ Wg[l].T
+            zh, zg, zp = z[:, :H], z[:, H:2 * H], z[:, 2 * H:]
+            st = r_state[t, l].astype(np.float64)
+            gh = np.where(zh >= 0.0, zh + 0.5, sigmoid64(zh))
+            o = st + sigmoid64(zg) * (gh - st)
+            pm = sigmoid64(zp)
+            x.append(pm * o + (1.0 - pm) * x[l])
+            zs.append((zh, zg, zp))
+        h3q = q(x[layers])
+        lg = h3q @ Wa.T + w["b_a"]
+        val = h3q @ Wv + w["b_v"][0]
+        # ---- head
+        lse = np.log(np.exp(lg - lg.max(1, keepdims=True)).sum(1, keepdims=True)) + lg.max(1, keepdims=True)
+        logp = lg - lse
+        pi = np.exp(logp)
+        act = r_act[t]
+        ratio = np.exp(logp[rows, act] - r_logprob[t].astype(np.float64))
+        A = (a64[t] - mean) * inv_std
+        u1 = ratio * A
+        u2 = np.clip(ratio, 1.0 - clip, 1.0 + clip) * A
+        dlogp = np.where(u1 <= u2, -A * ratio, 0.0)
+        Hent = -(pi * logp).sum(1)
+        dret = val - ret[t].astype(np.float64)
+        loss3 += [-np.minimum(u1, u2).sum(), (0.5 * dret * dret).sum(), Hent.sum()]
+        onehot = np.zeros_like(pi); onehot[rows, act] = 1.0
+        dlog = (dlogp[:, None] * (onehot - pi) + ent * pi * (logp + Hent[:, None])) * inv_batch
+        dv = inv_batch * vf * dret
+        g["b_a"] += dlog.sum(0); g["b_v"] += dv.sum()
+        g["W_a"] += q(dlog).T @ h3q
+        g["W_v"] += q(dv) @ h3q
+        dh = qs(q(dlog) @ Wa + q(dv)[:, None] * Wv[None, :])
+        # ---- reverse layers
+        cut = (t == T - 1) or ((t + 1) % seg_len == 0)
+        passes = (r_done[t] == 0).astype(np.float64)[:, None]
+        dhx = np.zeros((n, H))
+        for l in range(layers - 1, -1, -1):
+            if cut:
+                carry[l] = 0.0
+            zh, zg, zp = (qs(z) for z in zs[l])
+            st = r_state[t, l].astype(np.float64)
+            top = dh + dhx
+            sg, pm = sigmoid64(zg), sigmoid64(zp)
+            gh = np.where(zh >= 0.0, zh + 0.5, sigmoid64(zh))
+            dgh = np.where(zh >= 0.0, 1.0, sigmoid64(zh) * (1.0 - sigmoid64(zh)))
+            o = st + sg * (gh - st)
+            dout = top * pm + passes * carry[l]
+            dzp = qs(top * (o - qs(x[l])) * pm * (1.0 - pm))
+            dhx = qs(top * (1.0 - pm))
+            carry[l] = dout * (1.0 - sg)
+            dzg = qs(dout * (gh - st) * sg * (1.0 - sg))
+            dzh = qs(dout * sg * dgh)
+            dpre = q(np.concatenate([dzh, dzg, dzp], axis=1))
+            g["W_gru"][l] += dpre.T @ q(x[l])
+            dh = dpre @ Wg[l]
+            if l > 0:
+                dh = qs(dh)
+        dh = qs(dh + dhx)
+        g["b_enc"] += dh.sum(0)
+        ft = feats[t].astype(np.float64)
+        g["W_enc"][:768] += ft[:, :768].T @ (dh if map_rows_exact else q(dh))
+        g["W_enc"][768:] += q(ft[:, 768:]).T @ q(dh)
+    flat = np.concatenate([g[k].ravel() for k in ("W_enc", "b_enc", "W_gru", "W_a", "b_a", "W_v", "b_v")])
+    return flat, loss3
 
 
 def fro_err(got, ref):

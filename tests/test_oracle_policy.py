@@ -188,6 +188,40 @@ def test_backward_matches_finite_differences():
     assert worst < 1.0
 
 
+@pytest.mark.parametrize("seg_len,layers", [(5, 3), (2, 2), (3, 1)])
+def test_bf16_operand_backward_against_a_numpy_restatement(seg_len, layers):
+    """The bf16-operand comparators of the update (cfo_ppo_backward_bf16ops_f64, with fp32 and
+    with bf16 window storage) against a restatement with numpy matmuls over all envs at once.
+    The restatement is first held, with exact operands, to the gradient that the finite
+    differences above pin; with rounding switched on it then differs from that code only in
+    where an operand is rounded, and the compiled comparator must round in the same places."""
+    from parity_util import numpy_ppo_backward_f64, fro_err
+    params = random_params(layers, 71)
+    n, T = 6, 5
+    ro = _rollout(params, n, T, 72, done_p=0.2, layers=layers)
+    feats = np.stack([expand_records(ro["r_obs"][t]) for t in range(T)])
+    batch, keep = ob.make_batch(T, n, 0, n, layers, seg_len, **ro)
+    kw = dict(seg_len=seg_len)
+    args = (params, layers, feats, ro["r_state"], ro["r_act"], ro["r_logprob"], ro["adv"], ro["ret"],
+            ro["r_done"])
+    g0, l0 = ob.ppo_backward_f64(params, batch)
+    n0, m0 = numpy_ppo_backward_f64(*args, mode=0, **kw)
+    assert np.allclose(m0, l0, rtol=1e-11)
+    assert fro_err(n0, g0) < 1e-12
+    seen = []
+    for mode, exact in ((1, False), (2, False), (1, True)):
+        gc, lc = ob.ppo_backward_bf16ops_f64(params, batch, bf16_storage=(mode == 2), map_rows_exact=exact)
+        gn, ln = numpy_ppo_backward_f64(*args, mode=mode, map_rows_exact=exact, **kw)
+        assert np.allclose(ln, lc, rtol=1e-11)
+        # a sum that lands within an fp64 rounding of a bf16 tie may round the other way in
+        # the two codes: the bound leaves room for a handful of such entries
+        assert fro_err(gc, gn) < 1e-6, mode
+        assert 1e-4 < fro_err(gc, g0) < 1e-1, "rounding took effect"
+        seen.append(gc)
+    assert 1e-5 < fro_err(seen[1], seen[0]), "the storage mode rounds more"
+    assert 1e-5 < fro_err(seen[2], seen[0]), "the map rows of dW_enc follow the switch"
+
+
 def test_backward_truncation_and_done_semantics():
     params = random_params(L, 31)
     n, T = 4, 6
