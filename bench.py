@@ -47,7 +47,7 @@ T_BOUND_PER_ENV_STEP = (FLOP_FP32_PIPE / (PEAK_FP32_MFMA_TFLOPS * 1e12) +
                         FLOP_BF16_PIPE_ISSUED / (PEAK_BF16_MFMA_TFLOPS * 1e12))
 PEAK_MIX_TFLOPS = FLOP_PER_ENV_STEP / T_BOUND_PER_ENV_STEP / 1e12   # 196.9
 LAYERS = 3
-KERNEL_SOURCES = ("policy_forward.hip", "policy_tile.h", "cfp_common.h")
+KERNEL_SOURCES = ("policy_forward.hip", "policy_tile.h", "cfp_common.h", "cfp_internal.h", "sample_row.h")
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "policy_forward_262144_pmc.txt")
 
 

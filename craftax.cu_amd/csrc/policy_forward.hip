@@ -24,8 +24,8 @@
 // latency: per 24 MFMAs, 6 LDS-direct weight requests (no registers written),
 // 7 LDS reads and ~25 epilogue instructions.  (The same instructions issued by a
 // second wave on the SIMD cost the MFMA wave about as much: a two-group variant of
-// this schedule measured no faster.)  The shader clock under this load is
-// 1.9-2.1 GHz, not the 2.4 GHz behind the 157.3 TFLOP/s peak.
+// this schedule measured no faster.)  The shader clock under this load settles at
+// 2.36-2.41 GHz once it has ramped up from idle (some tens of milliseconds of load).
 //
 // Within the workgroup, wave w owns hidden units [64w, 64w+64).  MFMA operand
 // convention (v_mfma_f32_32x32x2_f32): A = activations (row = env), B = weights
