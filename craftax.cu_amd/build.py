@@ -38,6 +38,52 @@ def check_no_scratch(remarks):
         raise RuntimeError("kernels with counted waits spill registers to scratch memory: " + ", ".join(bad))
 
 
+# Register budget and occupancy each of those kernels is scheduled for.  Their waits count
+# the operations the source issues between a load and its use; how many wavefronts share a
+# SIMD decides how far ahead those loads have to be issued (the forward kernels are written
+# for one, respectively two, wavefronts per SIMD; the sweep for at least four, its
+# __launch_bounds__), and a jump in registers is how a compiler change that re-orders or
+# duplicates those loads shows first.  (kernel name part, VGPRs allowed, AGPRs allowed,
+# occupancy [waves/SIMD] lowest, highest)
+COUNTED_WAIT_BUDGET = (
+    ("k_policy_forwardI", 256, 160, 1, 1),
+    ("k_policy_forward_t16I", 192, 0, 2, 2),
+    ("k_gru_reverseI", 128, 0, 4, 8),
+)
+
+
+def resource_usage(remarks):
+    """{mangled kernel name: {"VGPRs", "AGPRs", "Occupancy", "ScratchSize"}} from the
+    -Rpass-analysis=kernel-resource-usage remarks."""
+    import re
+    out, name = {}, None
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+            out[name] = {}
+            continue
+        m = re.search(r"remark:\s+([A-Za-z][\w ]*?)(?: \[[^\]]*\])?:\s+(\d+)", line)
+        if m and name:
+            out[name][m.group(1)] = int(m.group(2))
+    return out
+
+
+def check_counted_wait_budget(remarks):
+    """Refuse a build in which a kernel with counted waits left the register budget or the
+    occupancy it is scheduled for."""
+    bad = []
+    for name, use in resource_usage(remarks).items():
+        for part, vgprs, agprs, occ_lo, occ_hi in COUNTED_WAIT_BUDGET:
+            if part not in name or "VGPRs" not in use:
+                continue
+            occ = use.get("Occupancy", occ_lo)
+            if use["VGPRs"] > vgprs or use.get("AGPRs", 0) > agprs or not occ_lo <= occ <= occ_hi:
+                bad.append(f"{name}: {use['VGPRs']} VGPRs, {use.get('AGPRs', 0)} AGPRs, occupancy {occ} "
+                           f"(allowed: {vgprs}, {agprs}, {occ_lo}..{occ_hi})")
+    if bad:
+        raise RuntimeError("kernels with counted waits outside their register / occupancy budget:\n  " + "\n  ".join(bad))
+
+
 def build(verbose=False):
     """Compile every HIP source into one shared library; always recompiles."""
     cmd = [
@@ -56,6 +102,7 @@ def build(verbose=False):
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{err}")
     check_no_scratch(res.stderr)
+    check_counted_wait_budget(res.stderr)
     if verbose and err.strip():
         print(err, file=sys.stderr)
     return OUT

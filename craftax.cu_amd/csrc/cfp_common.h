@@ -219,6 +219,19 @@ int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpr
 // partial products per product the split kernels run with now (9, 6, or 1 with bf16
 // inputs); 0 when they are switched off
 int gemm_split_terms();
+// The GEMM mode in effect for the calling thread: the process-wide switches
+// (cfp_set_gemm_bf16 / cfp_set_gemm_split) unless a GemmModeScope overrides them.
+int gemm_mode_bf16();
+int gemm_mode_split();
+// Overrides the mode for the calls the current thread issues while the object lives;
+// a negative value leaves that switch as it is.
+struct GemmModeScope {
+    GemmModeScope(int bf16, int split);
+    ~GemmModeScope();
+    GemmModeScope(const GemmModeScope&) = delete;
+    GemmModeScope& operator=(const GemmModeScope&) = delete;
+    int old_bf16, old_split;
+};
 // dW_a[rows_a][256] += and dW_b[rows_b][256] += from adjacent columns of one dpre matrix
 // (one pass over x on the split kernels, two passes otherwise)
 int gemm_dw_two(int rows_a, int rows_b, int cols, const float* x, const float* dpre, int ld_dpre,

@@ -373,13 +373,18 @@ static bool vec_ok(const float* p, long ld, int fast_extent) {
 int g_gemm_bf16 = 0;
 // fp32 operands split into bf16 triples for the update's shapes (gemm_x9.hip)
 int g_gemm_split = 1;
+// A trainer with a mode of its own overrides both for the calls it issues: the override
+// belongs to the issuing thread and lasts for one entry point (GemmModeScope).
+thread_local int t_gemm_bf16 = -1, t_gemm_split = -1;
+inline int eff_bf16() { return t_gemm_bf16 >= 0 ? t_gemm_bf16 : g_gemm_bf16; }
+inline int eff_split() { return t_gemm_split >= 0 ? t_gemm_split : g_gemm_split; }
 // partial products per product on those kernels: bf16 inputs -> 1 (rounded operands)
-inline int split_terms() { return g_gemm_bf16 ? 1 : (g_gemm_split == 2 ? 6 : 9); }
+inline int split_terms() { return eff_bf16() ? 1 : (eff_split() == 2 ? 6 : 9); }
 
 template <bool A_KFAST, bool B_KFAST, bool ACCUM>
 int launch_gemm(const GemmArgs& g, dim3 grid, bool va, bool vb, hipStream_t st) {
     const dim3 blk(GEMM_THREADS);
-    if (g_gemm_bf16) {
+    if (eff_bf16()) {
         if (va && vb) hipLaunchKernelGGL((k_gemm_bf16<A_KFAST, B_KFAST, ACCUM, true, true>), grid, blk, 0, st, g);
         else if (va) hipLaunchKernelGGL((k_gemm_bf16<A_KFAST, B_KFAST, ACCUM, true, false>), grid, blk, 0, st, g);
         else if (vb) hipLaunchKernelGGL((k_gemm_bf16<A_KFAST, B_KFAST, ACCUM, false, true>), grid, blk, 0, st, g);
@@ -474,7 +479,7 @@ const SeamWork* seam_default() {
 int gemm_dh_acc(int m3, int cols, const float* d_W, const float* d_dpre, float* d_dh,
                 bool accumulate, const SeamWork& sw, hipStream_t st) {
     CFP_REQUIRE(m3 > 0 && cols > 0 && d_W && d_dpre && d_dh, "cfp_gemm_dh: bad argument");
-    if (g_gemm_split && gemm_dh_x9_ok(m3, cols, d_dpre) && (!accumulate || m3 >= 160))
+    if (eff_split() && gemm_dh_x9_ok(m3, cols, d_dpre) && (!accumulate || m3 >= 160))
         return gemm_dh_x9(m3, cols, d_W, d_dpre, d_dh, accumulate, split_terms(), sw.w_mirror, st);
     GemmArgs g{};
     g.A = d_dpre; g.sa_i = m3; g.sa_k = 1;
@@ -498,7 +503,7 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
     CFP_REQUIRE(rows > 0 && rows <= CFP_OBS && cols > 0 && d_x && d_dpre && d_dW &&
                     ld_dpre >= rows,
                 "cfp_gemm_dw: bad argument (rows must be in 1..%d)", CFP_OBS);
-    if (g_gemm_split && gemm_dw_x9_ok(rows, cols))
+    if (eff_split() && gemm_dw_x9_ok(rows, cols))
         return gemm_dw_x9(rows, cols, d_x, d_dpre, ld_dpre, d_dW, split_terms(), sw, st);
     // enough workgroups to fill 256 CUs: tiles(M) * tiles(N=2) * splits
     const int tiles = ((rows + BM - 1) / BM) * (CFP_HIDDEN / BN);
@@ -530,13 +535,23 @@ int gemm_dw_ld(int rows, int cols, const float* d_x, const float* d_dpre, int ld
     return launch_splitk_reduce(d_dW, sw.dw_part, count, count, splits, st);
 }
 
-int gemm_split_terms() { return g_gemm_split ? split_terms() : 0; }
+int gemm_split_terms() { return eff_split() ? split_terms() : 0; }
+int gemm_mode_bf16() { return eff_bf16(); }
+int gemm_mode_split() { return eff_split(); }
+GemmModeScope::GemmModeScope(int bf16, int split) : old_bf16(t_gemm_bf16), old_split(t_gemm_split) {
+    if (bf16 >= 0) t_gemm_bf16 = bf16;
+    if (split >= 0) t_gemm_split = split;
+}
+GemmModeScope::~GemmModeScope() {
+    t_gemm_bf16 = old_bf16;
+    t_gemm_split = old_split;
+}
 
 int gemm_dw_two(int rows_a, int rows_b, int cols, const float* d_x, const float* d_dpre,
                 int ld_dpre, float* d_dW_a, float* d_dW_b, const SeamWork& sw, hipStream_t st) {
     CFP_REQUIRE(rows_a > 0 && rows_b > 0 && ld_dpre >= rows_a + rows_b && d_dW_a && d_dW_b,
                 "gemm_dw_two: bad argument");
-    if (g_gemm_split && gemm_dw_x9_ok(rows_a + rows_b, cols))
+    if (eff_split() && gemm_dw_x9_ok(rows_a + rows_b, cols))
         return gemm_dw_x9(rows_a + rows_b, cols, d_x, d_dpre, ld_dpre, d_dW_a, split_terms(), sw, st,
                           rows_a, d_dW_b);
     if (gemm_dw_ld(rows_a, cols, d_x, d_dpre, ld_dpre, d_dW_a, sw, st)) return 1;
@@ -565,7 +580,7 @@ int cfp_gemm_fwd(int m, int cols, int k, const float* d_W, const float* d_x,
                  float* d_y, void* stream) {
     CFP_REQUIRE(m > 0 && cols > 0 && k > 0 && d_W && d_x && d_y,
                 "cfp_gemm_fwd: bad argument");
-    if (g_gemm_split && gemm_fwd_x9_ok(m, cols, k, d_x)) {
+    if (eff_split() && gemm_fwd_x9_ok(m, cols, k, d_x)) {
         const SeamWork* sw = seam_default();
         if (!sw) return 1;
         return gemm_fwd_x9(m, cols, k, d_W, d_x, d_y, split_terms(), sw->w_mirror,

@@ -174,6 +174,8 @@ struct cfp_trainer {
     // bf16 storage of the window's gate pre-activations / their gradients and of the
     // layer inputs (in effect with bf16 GEMM inputs on the split kernels only)
     int bf16_store = 0;
+    // GEMM mode of this trainer's update (cfp_train_set_gemm_mode); -1: the process-wide switch
+    int gemm_bf16 = -1, gemm_split = -1;
     hipStream_t st_own = nullptr;   // capture stream when the caller passes the null stream
 };
 
@@ -334,6 +336,21 @@ int cfp_train_set_bf16_storage(cfp_trainer* tr, int on) {
 }
 int cfp_train_bf16_storage(const cfp_trainer* tr) { return tr ? tr->bf16_store : -1; }
 
+int cfp_train_set_gemm_mode(cfp_trainer* tr, int bf16, int split) {
+    CFP_REQUIRE(tr, "cfp_train_set_gemm_mode: NULL trainer");
+    CFP_REQUIRE(bf16 >= -1 && bf16 <= 1 && split >= -1 && split <= 2,
+                "cfp_train_set_gemm_mode: bf16 must be -1, 0 or 1 and split -1, 0, 1 or 2 (got %d, %d)", bf16, split);
+    tr->gemm_bf16 = bf16;
+    tr->gemm_split = split;
+    return 0;
+}
+int cfp_train_gemm_mode(const cfp_trainer* tr, int* bf16, int* split) {
+    CFP_REQUIRE(tr && bf16 && split, "cfp_train_gemm_mode: NULL argument");
+    *bf16 = tr->gemm_bf16 >= 0 ? tr->gemm_bf16 : cfp_get_gemm_bf16();
+    *split = tr->gemm_split >= 0 ? tr->gemm_split : cfp_get_gemm_split();
+    return 0;
+}
+
 int cfp_train_window(const cfp_trainer* tr) { return tr ? tr->win : 0; }
 int cfp_train_minibatch(const cfp_trainer* tr) { return tr ? tr->mb : 0; }
 
@@ -457,6 +474,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
                 env_start + env_count, tr->n, tr->mb);
     hipStream_t st = (hipStream_t)stream;
     cfp_policy* p = tr->p;
+    const GemmModeScope mode(tr->gemm_bf16, tr->gemm_split);   // the trainer's own mode, if it has one
     const int T = tr->T, n = tr->n, L = tr->L, mb = env_count;
     const int seg = T / tr->cfg.bptt_split;
     const float* W_enc = p->params + CFP_OFF_W_ENC;
@@ -486,17 +504,17 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         // fused forward kernel (fp32, or the bf16-input one) in its window mode: stored
         // state in, pre-activations and layer outputs out.  The unfused chain below is
         // what bf16 inputs run with the split kernels switched off.
-        const bool fused = cfp_get_gemm_bf16() == 0 || cfp_get_gemm_split() != 0;
+        const bool fused = gemm_mode_bf16() == 0 || gemm_mode_split() != 0;
         // bf16 storage: pre / dpre, the layer inputs x[0..L] and the three dh buffers are
         // bf16 arrays inside the same buffers; needs the record-fed dW_enc and the split
         // kernels (whole 32-column blocks); a window that does not fit runs with fp32
         // storage
-        const bool st16 = tr->bf16_store && cfp_get_gemm_bf16() != 0 && cfp_get_gemm_split() != 0 &&
+        const bool st16 = tr->bf16_store && gemm_mode_bf16() != 0 && gemm_mode_split() != 0 &&
                           dw_enc_records_ok(mb) && cols % 32 == 0;
         if (fused) {
             FwdArgs fa{};
             fill_forward_weights(p, fa);
-            fa.bf16 = cfp_get_gemm_bf16();
+            fa.bf16 = gemm_mode_bf16();
             fa.rec = tr->r_obs;
             fa.state = tr->r_state;
             fa.h_enc_out = tr->x[0];
@@ -691,7 +709,8 @@ int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
         if (!tr->st_own) CFP_HIP_TRY(hipStreamCreate(&tr->st_own));
         st = tr->st_own;
     }
-    const int split = cfp_get_gemm_split(), bf = cfp_get_gemm_bf16(),
+    const int split = tr->gemm_split >= 0 ? tr->gemm_split : cfp_get_gemm_split(),
+              bf = tr->gemm_bf16 >= 0 ? tr->gemm_bf16 : cfp_get_gemm_bf16(),
               pbf = cfp_policy_gemm_bf16(tr->p);
     if (tr->texec && (split != tr->graph_split || bf != tr->graph_bf16 ||
                       pbf != tr->graph_pol_bf16 || tr->bf16_store != tr->graph_store16)) {

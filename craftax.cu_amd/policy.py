@@ -268,6 +268,16 @@ class Trainer:
         """bf16 storage of the window workspace (in effect with bf16 GEMM inputs only)."""
         _check(lib().cfp_train_set_bf16_storage(self._h, 1 if on else 0))
 
+    def set_gemm_mode(self, bf16=-1, split=-1):
+        """This trainer's own GEMM mode (cfp_train_set_gemm_mode); -1 follows the process-wide switch."""
+        _check(lib().cfp_train_set_gemm_mode(self._h, int(bf16), int(split)))
+
+    def gemm_mode(self):
+        """(bf16, split) the next update of this trainer runs with."""
+        b, s_ = C.c_int(), C.c_int()
+        _check(lib().cfp_train_gemm_mode(self._h, C.byref(b), C.byref(s_)))
+        return b.value, s_.value
+
     def gae(self):
         _check(lib().cfp_train_gae(self._h, _stream()))
 

@@ -444,6 +444,18 @@ void* cfp_train_buffer(cfp_trainer* tr, int which);
  * Off by default. */
 int cfp_train_set_bf16_storage(cfp_trainer* tr, int on);
 int cfp_train_bf16_storage(const cfp_trainer* tr);
+
+/* GEMM mode of one trainer's update.  The reference has one process-wide switch
+ * (g_gemm_bf16, craftax_full.cu:11306-11316) and one trainer per process; here two trainers
+ * may live in one process, each with a captured update graph, so a trainer can carry its own
+ * mode: bf16 = 0 / 1 and split = 0 / 1 / 2 as in cfp_set_gemm_bf16 / cfp_set_gemm_split, or
+ * -1 to follow the process-wide switch (the default for both).  cfp_train_backward and
+ * cfp_train_update run with the trainer's mode whatever the process-wide switches say, and
+ * cfp_train_update's graph is captured again only when the trainer's effective mode changed.
+ * The raw seam calls (cfp_gemm_*) always follow the process-wide switches. */
+int cfp_train_set_gemm_mode(cfp_trainer* tr, int bf16, int split);
+/* The mode the trainer's next update runs with (its own, or the process-wide one). */
+int cfp_train_gemm_mode(const cfp_trainer* tr, int* bf16, int* split);
 int cfp_train_window(const cfp_trainer* tr);
 int cfp_train_minibatch(const cfp_trainer* tr);
 

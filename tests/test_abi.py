@@ -78,3 +78,34 @@ def test_build_rejects_a_spilling_forward_kernel():
                        other + "remark:     ScratchSize [bytes/lane]: 64 [-R]\n")
     with pytest.raises(RuntimeError, match="scratch"):
         b.check_no_scratch(fn + "remark:     ScratchSize [bytes/lane]: 24 [-R]\n")
+
+
+def test_build_rejects_a_counted_wait_kernel_outside_its_register_budget():
+    """The kernels with counted waits are scheduled for a fixed number of wavefronts per
+    SIMD; the build refuses one whose registers or occupancy left the committed range."""
+    import importlib.util
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                        "craftax.cu_amd", "build.py")
+    spec = importlib.util.spec_from_file_location("cfp_build", path)
+    b = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(b)
+
+    def remarks(fn, vgprs, agprs, occ):
+        return (f"f.hip:1:1: remark: Function Name: {fn} [-Rpass-analysis=kernel-resource-usage]\n"
+                f"f.hip:1:1: remark:     VGPRs: {vgprs} [-Rpass-analysis=kernel-resource-usage]\n"
+                f"f.hip:1:1: remark:     AGPRs: {agprs} [-Rpass-analysis=kernel-resource-usage]\n"
+                f"f.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]\n"
+                f"f.hip:1:1: remark:     Occupancy [waves/SIMD]: {occ} [-Rpass-analysis=kernel-resource-usage]\n")
+    fwd = "_ZN3cfp16k_policy_forwardILi0ELi0ELb0EEEvNS_7FwdArgsE"
+    t16 = "_ZN3cfp12_GLOBAL__N_120k_policy_forward_t16ILi0EEEvNS_7FwdArgsE"
+    rev = "_ZN3cfp12_GLOBAL__N_113k_gru_reverseILb1ELb1ELb0EEEvNS_11ReverseArgsE"
+    other = "_ZN3cfp6k_gemmILb0EEEvNS_8GemmArgsE"
+    use = b.resource_usage(remarks(fwd, 256, 126, 1))
+    assert use[fwd] == {"VGPRs": 256, "AGPRs": 126, "ScratchSize": 0, "Occupancy": 1}
+    # today's figures pass; a kernel without counted waits may use what it likes
+    b.check_counted_wait_budget(remarks(fwd, 256, 126, 1) + remarks(t16, 162, 0, 2) + remarks(rev, 96, 0, 5) +
+                                remarks(other, 512, 0, 1))
+    for bad in (remarks(fwd, 256, 200, 1), remarks(fwd, 128, 0, 2), remarks(t16, 230, 0, 2), remarks(t16, 120, 0, 3),
+                remarks(rev, 140, 0, 3), remarks(rev, 128, 0, 3)):
+        with pytest.raises(RuntimeError, match="budget"):
+            b.check_counted_wait_budget(bad)

@@ -416,6 +416,39 @@ def test_train_update_eager_and_graph_match_the_manual_loop(pkg, cuda, on_side_s
         tr.close(); pol.close()
 
 
+def test_two_trainers_with_their_own_gemm_modes(pkg, cuda):
+    """cfp_train_set_gemm_mode: two trainers in one process, one on the fp32 MFMA kernel and
+    one on bf16 inputs, each with a captured update graph.  Each must equal, bit for bit, a
+    twin that ran the same update eagerly under process-wide switches of the same values --
+    also after the process-wide switches were flipped between the replays, which changes
+    nothing for a trainer that carries its own mode (and triggers no new capture)."""
+    import torch
+    n, T = 64, 6
+    modes = ((0, 0), (1, 1))           # (bf16, split)
+    for own in modes:
+        (_, pol_o, tr_o, _), (_, pol_t, tr_t, _) = [_collect(pkg, cuda, n, T, 421, 0.1) for _ in range(2)]
+        tr_o.set_gemm_mode(*own)
+        assert tr_o.gemm_mode() == own and tr_t.gemm_mode() == (0, 1)
+        for it, ambient in enumerate(((0, 1), (1, 2), (0, 0))):
+            pkg.policy.set_gemm_bf16(own[0]); pkg.policy.set_gemm_split(own[1])
+            try:
+                tr_t.update(use_graph=False)        # the twin follows the process-wide switches
+                torch.cuda.synchronize()
+                pkg.policy.set_gemm_bf16(ambient[0]); pkg.policy.set_gemm_split(ambient[1])
+                tr_o.update(use_graph=True)         # its own mode, whatever the switches say
+                torch.cuda.synchronize()
+            finally:
+                pkg.policy.set_gemm_bf16(False); pkg.policy.set_gemm_split(1)
+            assert torch.equal(pol_o.params, pol_t.params), f"own mode {own}, iteration {it}, ambient {ambient}"
+            assert torch.equal(tr_o.buf("loss_acc"), tr_t.buf("loss_acc"))
+        tr_o.set_gemm_mode(-1, -1)
+        assert tr_o.gemm_mode() == (0, 1)
+        with pytest.raises(pkg._lib.CfpError):
+            tr_o.set_gemm_mode(2, 0)
+        for pol, tr in ((pol_o, tr_o), (pol_t, tr_t)):
+            tr.close(); pol.close()
+
+
 def test_checkpoint_roundtrip(pkg, cuda, tmp_path):
     """CFW1 file: header words, byte-exact params, mirrors refreshed on load, and the
     reference's rejections (wrong shape, truncated file)."""
