@@ -267,7 +267,7 @@ def classic_1m(pkg, torch, reps):
 def record_kernels(pkg, torch, reps):
     import numpy as np
     n = 65536
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    root = os.path.dirname(os.path.abspath(__file__))
     g = np.load(os.path.join(root, "tests", "golden", "record_fixtures.npz"))
     sc, pl = g["fuzz_scalars"], g["fuzz_planes"]          # [384][S], [384][3][2304]
     idx = np.arange(n) % sc.shape[0]

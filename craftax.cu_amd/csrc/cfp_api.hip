@@ -44,6 +44,7 @@ static void policy_release(cfp_policy* p) {
     (void)hipFree(p->wg_bf);
     (void)hipFree(p->wav_bf);
     (void)hipFree(p->t16);
+    (void)hipFree(p->enc_x9);
     (void)hipFree(p->h_state);
     (void)hipFree(p->rec);
     (void)hipFree(p->h_enc);
@@ -128,6 +129,7 @@ static int policy_create(cfp_policy** out, int num_envs, int layers, uint64_t se
     CFP_ALLOC(p->wg_bf, (size_t)layers * kGruPackFloats * sizeof(uint16_t));
     CFP_ALLOC(p->wav_bf, kAvPackFloats * sizeof(uint16_t));
     if (variant == 0) CFP_ALLOC(p->t16, t16_mirror_bytes(layers));
+    if (variant == 0) CFP_ALLOC(p->enc_x9, enc_mirror_bytes());
     CFP_ALLOC(p->h_state, (size_t)layers * hn * sizeof(float));
     CFP_ALLOC(p->rec, (size_t)num_envs * rec_bytes);
     CFP_ALLOC(p->h_enc, hn * sizeof(float));
@@ -428,11 +430,31 @@ int cfp_policy_forward_features(cfp_policy* p, const float* d_xobs, const float*
                 "cfp_policy_forward_features: n=%d exceeds the object's buffers (%d envs)", n, p->n);
     float* h_enc = d_h_enc ? d_h_enc : p->h_enc;
     const Arena ar = arena_of(0, p->layers);
-    if (gemm_enc_fwd_ld(n, p->params + ar.w_enc, d_xobs, CFP_OBS, h_enc, (hipStream_t)stream)) return 1;
-    if (cfp_add_bias(h_enc, p->params + ar.b_enc, n, stream)) return 1;
+    // The encoder product on the split kernels where they are on (every fp32 operand as three
+    // bf16 parts, nine / six exact products, or one with bf16 inputs); its bias is added where
+    // the fused kernel stages h_enc.  Otherwise the fp32 MFMA GEMM and the bias pass.
+    const int terms = gemm_split_terms();
+    const bool split = terms != 0 && gemm_enc_fwd_x9_ok(n, d_xobs) && p->enc_x9;
+    bool bias_at_staging = false;
+    if (split) {
+        if (gemm_enc_fwd_x9(n, p->params + ar.w_enc, d_xobs, CFP_OBS, h_enc, terms,
+                            static_cast<u4*>(p->enc_x9), (hipStream_t)stream))
+            return 1;
+        // a caller who asked for h_enc gets it with the bias (the same fp32 addition, so the
+        // rest of the step sees the same bits either way)
+        if (d_h_enc) {
+            if (cfp_add_bias(h_enc, p->params + ar.b_enc, n, stream)) return 1;
+        } else {
+            bias_at_staging = true;
+        }
+    } else {
+        if (gemm_enc_fwd_ld(n, p->params + ar.w_enc, d_xobs, CFP_OBS, h_enc, (hipStream_t)stream)) return 1;
+        if (cfp_add_bias(h_enc, p->params + ar.b_enc, n, stream)) return 1;
+    }
     FwdArgs a{};
     fill_weights(p, a);
     a.x0 = h_enc;
+    a.x0_add_bias = bias_at_staging ? 1 : 0;
     a.terminals = d_terminals;
     a.state = d_state ? d_state : p->h_state;
     a.r_state = d_r_state_t;

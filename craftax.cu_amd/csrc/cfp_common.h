@@ -101,6 +101,7 @@ __host__ __device__ inline float philox_uniform(uint64_t seed, uint64_t subseque
 struct FwdArgs {
     const uint8_t* rec;      // [n][996] or null (then x0 is the layer-0 input)
     const float* x0;         // [n][256] or null
+    int x0_add_bias;         // x0 is the encoder product without its bias: staging adds b_enc
     const f4* we_pk;         // packed encoder weights
     const u4* we_s3;         // map rows of W_enc as three bf16 terms (hi, mid, lo) per weight
     const float* b_enc;
@@ -219,6 +220,12 @@ int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpr
 // partial products per product the split kernels run with now (9, 6, or 1 with bf16
 // inputs); 0 when they are switched off
 int gemm_split_terms();
+// h[cols][256] = xobs[cols][843] . W_enc on the split kernels (no bias); the mirror is
+// enc_mirror_bytes() of device memory owned by the caller
+size_t enc_mirror_bytes();
+bool gemm_enc_fwd_x9_ok(int cols, const float* xobs);
+int gemm_enc_fwd_x9(int cols, const float* W_enc, const float* xobs, int ldx, float* h, int terms,
+                    u4* enc_mirror, hipStream_t st);
 // The GEMM mode in effect for the calling thread: the process-wide switches
 // (cfp_set_gemm_bf16 / cfp_set_gemm_split) unless a GemmModeScope overrides them.
 int gemm_mode_bf16();

@@ -289,15 +289,18 @@ constexpr int kDhThreads = 512;
 constexpr int kDhTileCols = 256;
 constexpr int kDhFrags = 24;   // 8 unit tiles x 3 parts per K step
 
-__global__ void k_pack_w_x9(const float* __restrict__ W, long sk, long su,
-                            u4* __restrict__ out, int total, int rounded) {   // W(k, u) = W[k*sk + u*su]
+__global__ void k_pack_w_x9(const float* __restrict__ W, long sk, long su, u4* __restrict__ out,
+                            int total, int rounded, int krows) {   // W(k, u) = W[k*sk + u*su], 0 from row krows on
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= total) return;
     const int lane = idx & 63, f = (idx >> 6) % kDhFrags, s = idx / (64 * kDhFrags);
     const int t = f / 3, part = f - 3 * t, n = lane & 31, g = lane >> 5;
     float v[8];
 #pragma unroll
-    for (int j = 0; j < 8; j++) v[j] = W[(long)(16 * s + 8 * g + j) * sk + (long)(32 * t + n) * su];
+    for (int j = 0; j < 8; j++) {
+        const int k = 16 * s + 8 * g + j;
+        v[j] = k < krows ? W[(long)k * sk + (long)(32 * t + n) * su] : 0.0f;
+    }
     u4 h, m, l;
     split3(v, h, m, l);
     if (rounded) h = round_bf16x8(v);   // bf16-input mode: part 0 is the rounded operand
@@ -317,11 +320,15 @@ __device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {   // ne
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(f2_t{lo, hi}, bf16x2_t));
 }
 
-template <int TERMS, bool A16 = false, bool O16 = false>
+// AROW: the rows of dpre are `lda` floats apart with lda any number (rows only 4-byte
+// aligned) and hold kvalid <= m3 values: a lane fetches its eight values of a K step as
+// single dwords and reads what lies past kvalid as zero (the encoder product from an fp32
+// feature matrix: 843 features a row).
+template <int TERMS, bool A16 = false, bool O16 = false, bool AROW = false>
 __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ dpre, int m3,
                                                       const u4* __restrict__ wm,
                                                       float* __restrict__ dh, int ldc, int cols,
-                                                      int accumulate) {
+                                                      int accumulate, int lda, int kvalid) {
     __shared__ u4 stage[2][kDhFrags][64];   // 48 KiB
     const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63, n = lane & 31, g = lane >> 5;
     const int steps = m3 / 16;
@@ -329,7 +336,8 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
     const bool live = cb < cols;               // cols % 32 == 0: blocks are whole
     const int cbc = live ? cb : cols - 32;     // idle waves still stage W and meet the barriers
     static_assert(TERMS == 1 || !A16, "bf16 storage goes with bf16 inputs");
-    const float* a_lane = dpre + (size_t)(cbc + n) * m3 + 8 * g;
+    static_assert(!AROW || (!A16 && !O16), "row-strided A is an fp32 operand");
+    const float* a_lane = dpre + (size_t)(cbc + n) * (AROW ? lda : m3) + 8 * g;
     const u4* a16_lane = reinterpret_cast<const u4*>(
         reinterpret_cast<const uint16_t*>(dpre) + (size_t)(cbc + n) * m3 + 8 * g);
     auto a_load = [&](int s, float (&v)[8]) {
@@ -337,6 +345,13 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
             const u4 q = a16_lane[2 * s];
             v[0] = __uint_as_float(q.x); v[1] = __uint_as_float(q.y);
             v[2] = __uint_as_float(q.z); v[3] = __uint_as_float(q.w);
+            return;
+        }
+        if (AROW) {
+            // rows are only 4-byte aligned: eight dwords (sixteen-byte loads on a dword boundary
+            // measured 4 % slower), what lies past kvalid reads as zero and is never touched
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = 16 * s + 8 * g + j < kvalid ? a_lane[16 * s + j] : 0.0f;
             return;
         }
         const f4* p = reinterpret_cast<const f4*>(a_lane + 16 * s);
@@ -541,7 +556,9 @@ __global__ __launch_bounds__(kDhThreads) void k_dh_x9(const float* __restrict__ 
 #undef CFP_DH_OLD_ADD
 
 constexpr int kDhMaxK = CFP_GRU;
+constexpr int kEncK = (CFP_OBS + 15) / 16 * 16;   // 848: the encoder's K, padded to whole steps
 constexpr size_t kDhMirrorBytes = (size_t)(kDhMaxK / 16) * kDhFrags * 64 * sizeof(u4);   // 1.125 MiB
+constexpr size_t kEncMirrorBytes = (size_t)(kEncK / 16) * kDhFrags * 64 * sizeof(u4);   // 1.24 MiB
 
 }  // namespace
 
@@ -562,26 +579,54 @@ static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const
     CFP_REQUIRE(g_w_x9, "k_dh_x9: no mirror buffer for W");
     const int total = (K / 16) * kDhFrags * 64;
     hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, B, sk, su, g_w_x9,
-                       total, terms == 1 ? 1 : 0);
+                       total, terms == 1 ? 1 : 0, K);
     const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
     const int acc = accumulate ? 1 : 0;
     if (a16 && o16)
-        hipLaunchKernelGGL((k_dh_x9<1, true, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+        hipLaunchKernelGGL((k_dh_x9<1, true, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     else if (o16)
-        hipLaunchKernelGGL((k_dh_x9<1, false, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+        hipLaunchKernelGGL((k_dh_x9<1, false, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     else if (a16)
-        hipLaunchKernelGGL((k_dh_x9<1, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+        hipLaunchKernelGGL((k_dh_x9<1, true>), grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     else if (terms == 1)
-        hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+        hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     else if (terms == 6)
-        hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+        hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     else
-        hipLaunchKernelGGL(k_dh_x9<9>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc);
+        hipLaunchKernelGGL(k_dh_x9<9>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }
 
 size_t dh_mirror_bytes() { return kDhMirrorBytes; }
+size_t enc_mirror_bytes() { return kEncMirrorBytes; }
+
+// Encoder product from an fp32 feature matrix: h[cols][256] = xobs[cols][843] . W_enc[843][256]
+// (cu_gemm_enc_fwd, craftax_full.cu:11616) on the split kernels: K = 848 in 53 steps, rows of
+// xobs ldx floats apart, features 843..847 read as zero on both sides.
+bool gemm_enc_fwd_x9_ok(int cols, const float* xobs) {
+    return cols >= 32 && cols % 32 == 0 && (reinterpret_cast<uintptr_t>(xobs) & 3u) == 0;
+}
+int gemm_enc_fwd_x9(int cols, const float* W_enc, const float* xobs, int ldx, float* h, int terms,
+                    u4* enc_mirror, hipStream_t st) {
+    CFP_REQUIRE(gemm_enc_fwd_x9_ok(cols, xobs) && W_enc && h && enc_mirror && ldx >= CFP_OBS,
+                "gemm_enc_fwd_x9: columns must be a multiple of 32 and the matrix 4-byte aligned");
+    const int total = (kEncK / 16) * kDhFrags * 64;
+    hipLaunchKernelGGL(k_pack_w_x9, dim3((total + 255) / 256), dim3(256), 0, st, W_enc, (long)CFP_HIDDEN, 1L,
+                       enc_mirror, total, terms == 1 ? 1 : 0, CFP_OBS);
+    const dim3 grid((cols + kDhTileCols - 1) / kDhTileCols);
+    if (terms == 1)
+        hipLaunchKernelGGL((k_dh_x9<1, false, false, true>), grid, dim3(kDhThreads), 0, st, xobs, kEncK, enc_mirror, h,
+                           CFP_HIDDEN, cols, 0, ldx, CFP_OBS);
+    else if (terms == 6)
+        hipLaunchKernelGGL((k_dh_x9<6, false, false, true>), grid, dim3(kDhThreads), 0, st, xobs, kEncK, enc_mirror, h,
+                           CFP_HIDDEN, cols, 0, ldx, CFP_OBS);
+    else
+        hipLaunchKernelGGL((k_dh_x9<9, false, false, true>), grid, dim3(kDhThreads), 0, st, xobs, kEncK, enc_mirror, h,
+                           CFP_HIDDEN, cols, 0, ldx, CFP_OBS);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
 
 int gemm_dh_x9(int m3, int cols, const float* W, const float* dpre, float* dh, bool accumulate,
                int terms, u4* w_mirror, hipStream_t st, bool dpre_bf16, bool dh_bf16) {

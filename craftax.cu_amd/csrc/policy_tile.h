@@ -70,8 +70,16 @@ __device__ __forceinline__ void stage_tile(const FwdArgs& a, size_t e0, float* l
     } else {
         const f4* src = reinterpret_cast<const f4*>(a.x0 + e0 * CFP_HIDDEN);
         f4* xs4 = reinterpret_cast<f4*>(lds);
-        for (int i = tid; i < kTileEnvs * CFP_HIDDEN / 4; i += kFwdThreads)
-            xs4[(i >> 6) * XS4 + (i & 63)] = src[i];
+        if (a.x0_add_bias) {   // k_add_bias (craftax_full.cu:10056) folded into the staging
+            const f4* b4 = reinterpret_cast<const f4*>(a.b_enc);
+            for (int i = tid; i < kTileEnvs * CFP_HIDDEN / 4; i += kFwdThreads) {
+                const f4 v = src[i], b = b4[i & 63];
+                xs4[(i >> 6) * XS4 + (i & 63)] = f4{v[0] + b[0], v[1] + b[1], v[2] + b[2], v[3] + b[3]};
+            }
+        } else {
+            for (int i = tid; i < kTileEnvs * CFP_HIDDEN / 4; i += kFwdThreads)
+                xs4[(i >> 6) * XS4 + (i & 63)] = src[i];
+        }
     }
 }
 

@@ -173,13 +173,19 @@ struct WordSrc {
     __device__ __forceinline__ uint32_t word(int i) const { return w[i]; }
 };
 
-template <bool SOA>
+// ROW16: the three byte planes are read as one 16-byte piece per window row and plane (the
+// 11 window bytes of a row lie inside a 4-byte-aligned 16-byte piece of the 48-byte map row)
+// into an LDS strip, and the cells pick their bytes out of the strip: 27 sixteen-byte loads
+// per env instead of 297 single-byte ones.  Needs 4-byte-aligned planes and strides.
+template <bool SOA, bool ROW16>
 __global__ __launch_bounds__(256) void k_record_obs(
     const cfp_env_scalars* __restrict__ scalars, SoaArgs soa, RecWhich which,
     const uint8_t* __restrict__ map, const uint8_t* __restrict__ item_map,
     const uint8_t* __restrict__ light_map, size_t env_stride,
     size_t level_stride, uint8_t* __restrict__ rec_row, int n) {
     __shared__ uint32_t stage_all[kRecEnvsPerWg][CFP_REC_BYTES / 4 + 3];
+    typedef unsigned int strip_u4 __attribute__((ext_vector_type(4)));
+    __shared__ strip_u4 strip_all[ROW16 ? kRecEnvsPerWg : 1][3 * ROWS + 1];   // [plane * 9 + row], odd stride
     // SOA rounds take 32 envs: a 128-byte line of every field array is used by one workgroup
     constexpr int kGather = SOA ? kSoaGather : kRecEnvsPerWg;
     __shared__ uint32_t sc_all[SOA ? kGather : 1][kScalarWords + 1];
@@ -248,14 +254,42 @@ __global__ __launch_bounds__(256) void k_record_obs(
             const size_t cell_plane = (size_t)env * env_stride + (size_t)level * level_stride;
             const size_t mob_plane = (size_t)env * env_stride + (size_t)mlevel * level_stride;
 
+            // first map column of the 16-byte piece of every window row: a multiple of four at or
+            // below the window's first column, inside the map
+            const int wc0 = pc - COLS / 2;
+            int cb = wc0 < 0 ? 0 : (wc0 & ~3);
+            cb = cb > MAP - 16 ? MAP - 16 : cb;
+            const bool strips = ROW16 && level >= 0 && level < 9 && pc >= -64 && pc < 2 * MAP;
+            if (strips) {
+                strip_u4* strip = strip_all[slot];
+                for (int i = lane; i < 3 * ROWS; i += kRecLanes) {
+                    const int plane = i / ROWS, row = i - plane * ROWS;
+                    const int wr = pr - ROWS / 2 + row;
+                    strip_u4 v = {0u, 0u, 0u, 0u};
+                    if (wr >= 0 && wr < MAP) {
+                        const uint8_t* base = plane == 0 ? map : (plane == 1 ? item_map : light_map);
+                        v = *reinterpret_cast<const strip_u4*>(base + cell_plane + (size_t)(wr * MAP + cb));
+                    }
+                    strip[i] = v;
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
             for (int cell = lane; cell < CELLS; cell += kRecLanes) {
                 const int row = cell / COLS, col = cell - row * COLS;
                 const int wr = pr - ROWS / 2 + row, wc = pc - COLS / 2 + col;
                 uint32_t lo = 0;
                 if (wr >= 0 && wr < MAP && wc >= 0 && wc < MAP) {
-                    // all three planes requested at once (one memory round trip, not two)
-                    const size_t o = cell_plane + (size_t)(wr * MAP + wc);
-                    const uint32_t lv = light_map[o], bv = map[o], iv = item_map[o];
+                    uint32_t lv, bv, iv;
+                    if (strips) {
+                        const uint8_t* sb = reinterpret_cast<const uint8_t*>(strip_all[slot]) + row * 16 + (wc - cb);
+                        bv = sb[0];
+                        iv = sb[ROWS * 16];
+                        lv = sb[2 * ROWS * 16];
+                    } else {
+                        // all three planes requested at once (one memory round trip, not two)
+                        const size_t o = cell_plane + (size_t)(wr * MAP + wc);
+                        lv = light_map[o]; bv = map[o]; iv = item_map[o];
+                    }
                     if (lv > 12) lo = bv | ((uint32_t)(uint8_t)(iv + 1) << 8) | (1u << 16);
                 }
                 stage[2 * cell] = lo;
@@ -275,7 +309,13 @@ __global__ __launch_bounds__(256) void k_record_obs(
                 bool ok = lane < CFP_MOB_SLOTS && type >= 0 && type < 8 && mask != 0 &&
                           lr >= 0 && lr < ROWS && lc >= 0 && lc < COLS && mr >= 0 && mr < MAP &&
                           mc >= 0 && mc < MAP;
-                if (ok) ok = light_map[mob_plane + (size_t)(mr * MAP + mc)] > 12;
+                if (ok) {
+                    // a mob that passed the window test sits on a cell of the strip
+                    if (strips && mlevel == level)
+                        ok = reinterpret_cast<const uint8_t*>(strip_all[slot])[(2 * ROWS + lr) * 16 + (mc - cb)] > 12;
+                    else
+                        ok = light_map[mob_plane + (size_t)(mr * MAP + mc)] > 12;
+                }
                 const int cell = ok ? lr * COLS + lc : -1;
                 const int cls = kSlotClass[m];
                 bool over = false;
@@ -492,6 +532,13 @@ int launch_expand_obs(const uint8_t* r_obs, float* xobs, int t0, int count, int 
 }
 }  // namespace cfp
 
+// the 16-byte row pieces need every plane row to start on a 4-byte boundary
+static bool rows16_ok(const uint8_t* m, const uint8_t* im, const uint8_t* lm, size_t env_stride,
+                      size_t level_stride) {
+    return ((reinterpret_cast<uintptr_t>(m) | reinterpret_cast<uintptr_t>(im) |
+             reinterpret_cast<uintptr_t>(lm) | env_stride | level_stride) & 3u) == 0;
+}
+
 extern "C" {
 
 int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
@@ -505,9 +552,14 @@ int cfp_record_obs(const cfp_env_scalars* d_scalars, const uint8_t* d_map,
                 "record rows must be 4-byte aligned");
     CFP_REQUIRE(env_stride >= (size_t)MAP * MAP,
                 "cfp_record_obs: env_stride smaller than one 48x48 plane");
-    hipLaunchKernelGGL(k_record_obs<false>, dim3((n + kRecEnvsPerWg - 1) / kRecEnvsPerWg),
-                       dim3(256), 0, (hipStream_t)stream, d_scalars, SoaArgs{}, RecWhich{}, d_map,
-                       d_item_map, d_light_map, env_stride, level_stride, d_rec_row, n);
+    if (rows16_ok(d_map, d_item_map, d_light_map, env_stride, level_stride))
+        hipLaunchKernelGGL((k_record_obs<false, true>), dim3((n + kRecEnvsPerWg - 1) / kRecEnvsPerWg),
+                           dim3(256), 0, (hipStream_t)stream, d_scalars, SoaArgs{}, RecWhich{}, d_map,
+                           d_item_map, d_light_map, env_stride, level_stride, d_rec_row, n);
+    else
+        hipLaunchKernelGGL((k_record_obs<false, false>), dim3((n + kRecEnvsPerWg - 1) / kRecEnvsPerWg),
+                           dim3(256), 0, (hipStream_t)stream, d_scalars, SoaArgs{}, RecWhich{}, d_map,
+                           d_item_map, d_light_map, env_stride, level_stride, d_rec_row, n);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -529,9 +581,14 @@ static int record_obs_soa(const cfp_env_soa* soa, const uint8_t* d_map, const ui
     std::memcpy(&a, soa, sizeof(a));
     for (int i = 0; i < kSoaPtrs; i++)
         CFP_REQUIRE(a.p[i] != nullptr, "cfp_record_obs_soa: field array %d of the view is NULL", i);
-    hipLaunchKernelGGL(k_record_obs<true>, dim3((items + kSoaGather - 1) / kSoaGather),
-                       dim3(256), 0, (hipStream_t)stream, nullptr, a, which, d_map, d_item_map,
-                       d_light_map, env_stride, level_stride, d_rec_row, n);
+    if (rows16_ok(d_map, d_item_map, d_light_map, env_stride, level_stride))
+        hipLaunchKernelGGL((k_record_obs<true, true>), dim3((items + kSoaGather - 1) / kSoaGather),
+                           dim3(256), 0, (hipStream_t)stream, nullptr, a, which, d_map, d_item_map,
+                           d_light_map, env_stride, level_stride, d_rec_row, n);
+    else
+        hipLaunchKernelGGL((k_record_obs<true, false>), dim3((items + kSoaGather - 1) / kSoaGather),
+                           dim3(256), 0, (hipStream_t)stream, nullptr, a, which, d_map, d_item_map,
+                           d_light_map, env_stride, level_stride, d_rec_row, n);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }

@@ -185,9 +185,13 @@ int cfp_policy_forward(cfp_policy* p, const uint8_t* d_rec_row,
 /* The same step from the fp32 feature matrix xobs[n][843] (ld 843) instead of records:
  * cu_gemm_enc_fwd on xobs + k_add_bias (craftax_full.cu:11616, :10056; what
  * cu_encode_step runs after k_expand_obs), then the fused MinGRU layers and heads.
- * d_h_enc (NULL = the object's buffer) receives the encoder output.  The encoder GEMM is
- * the seam's (cfp_gemm_enc_fwd), not the record path's fused one: fp32 features are not
- * exact in bf16. */
+ * d_h_enc (NULL = the object's buffer) receives the encoder output.  fp32 features are not
+ * exact in bf16, so the record path's three-product encoder does not apply: with the split
+ * kernels on (cfp_set_gemm_split, the default) both operands travel as exact three-term bf16
+ * splits over K = 848 (nine products, or six / one in the other modes) and the bias is added
+ * where the fused kernel stages h_enc (or by k_add_bias when the caller asked for d_h_enc);
+ * with them off it is the seam's fp32 MFMA GEMM (cfp_gemm_enc_fwd) and the bias pass.
+ * n must be a multiple of 32. */
 int cfp_policy_forward_features(cfp_policy* p, const float* d_xobs, const float* d_terminals,
                                 float* d_state, float* d_r_state_t, float* d_h_enc, float* d_h3,
                                 float* d_av, int n, int chunk, void* stream);
