@@ -436,6 +436,14 @@ def rollout_in_the_loop(pkg, torch, reps):
         out["envs"][str(n)] = {"us_per_step": round(ms * 1e3, 1), "M_env_steps_per_s": round(n / ms / 1e3, 2),
                                "frac_fp32_peak_of_forward_flops": round(FWD_FLOP * n / (ms * 1e-3) / 1e12 / PEAK_FP32, 3)}
         tr.close()
+        # cu_train_collect: T steps with the resets overlapped on the second stream, plus the
+        # bootstrap forward and GAE, per step
+        Tc = 32 if n <= 65536 else 16
+        tr = pkg.Trainer(pol, Tc)
+        ms_c = _time(torch, lambda: env.collect(tr, 1234), 3, warm=1) / Tc
+        out["envs"][str(n)]["collect"] = {"T": Tc, "us_per_step": round(ms_c * 1e3, 1),
+                                          "M_env_steps_per_s": round(n / ms_c / 1e3, 2)}
+        tr.close()
         env.close()
     return out
 

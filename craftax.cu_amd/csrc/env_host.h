@@ -213,13 +213,13 @@ struct HostGroup {
     int tid() const { return 0; }
     int nt() const { return 1; }
     void sync() {}
-    float gmin(float v) { return v; }
-    float gmax(float v) { return v; }
     int gmaxi(int v) { return v; }
+    void gminmax4(float (&)[4], float (&)[4]) {}   // one member: its own extrema are the group's
     int gscan(int v, int& total) {
         total = v;
         return 0;
     }
+    void stamp(int) {}
     float cosine(float x) { return cosf(x); }
     float sine(float x) { return sinf(x); }
 };

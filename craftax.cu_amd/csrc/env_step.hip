@@ -568,40 +568,60 @@ __global__ __launch_bounds__(256) void k_env_reset_from_pool(CopyTable t, EnvArr
 }
 
 // ---- world generation on the device ------------------------------------------------------------
-constexpr int kGenThreads = 256;
+// threads of a generator job: 256 where many worlds are made at once (three jobs share a
+// CU), 512 where a step waits for a handful of worlds and a job's latency is what counts
+constexpr int kGenThreads = 256, kGenThreadsFew = 512;
+// jobs of one world: its nine floors and, as a job of its own, the scalar fields
+constexpr int kGenJobs = kLevels + 1;
 // the group of env_worldgen.h: one 256-thread workgroup, reductions through wave shuffles
 // and four LDS words; cos / sin in double precision, rounded to float
+template <int NT>
 struct BlockGroup {
+    static constexpr int kGenWaves = NT / 64;
     int t;
-    float* fred;   // LDS, 4 floats
-    int* ired;     // LDS, 4 ints
+    float* fred;   // LDS, eight floats a wavefront
+    int* ired;     // LDS, one int a wavefront
     __device__ __forceinline__ int tid() const { return t; }
-    __device__ __forceinline__ int nt() const { return kGenThreads; }
+    __device__ __forceinline__ int nt() const { return NT; }
     __device__ __forceinline__ void sync() { __syncthreads(); }
-    __device__ __forceinline__ float gmin(float v) {
+    // minima and maxima of four quantities over the group in one exchange
+    __device__ __forceinline__ void gminmax4(float (&mn)[4], float (&mx)[4]) {
 #pragma unroll
-        for (int d = 32; d > 0; d >>= 1) v = fminf(v, __shfl_xor(v, d));
-        if ((t & 63) == 0) fred[t >> 6] = v;
-        __syncthreads();
-        v = fminf(fminf(fred[0], fred[1]), fminf(fred[2], fred[3]));
-        __syncthreads();
-        return v;
-    }
-    __device__ __forceinline__ float gmax(float v) {
+        for (int f = 0; f < 4; f++) {
 #pragma unroll
-        for (int d = 32; d > 0; d >>= 1) v = fmaxf(v, __shfl_xor(v, d));
-        if ((t & 63) == 0) fred[t >> 6] = v;
+            for (int d = 32; d > 0; d >>= 1) {
+                mn[f] = fminf(mn[f], __shfl_xor(mn[f], d));
+                mx[f] = fmaxf(mx[f], __shfl_xor(mx[f], d));
+            }
+        }
+        if ((t & 63) == 0) {
+#pragma unroll
+            for (int f = 0; f < 4; f++) {
+                fred[8 * (t >> 6) + f] = mn[f];
+                fred[8 * (t >> 6) + 4 + f] = mx[f];
+            }
+        }
         __syncthreads();
-        v = fmaxf(fmaxf(fred[0], fred[1]), fmaxf(fred[2], fred[3]));
+#pragma unroll
+        for (int f = 0; f < 4; f++) {
+            mn[f] = fred[f];
+            mx[f] = fred[4 + f];
+#pragma unroll
+            for (int w = 1; w < kGenWaves; w++) {
+                mn[f] = fminf(mn[f], fred[8 * w + f]);
+                mx[f] = fmaxf(mx[f], fred[8 * w + f + 4]);
+            }
+        }
         __syncthreads();
-        return v;
     }
     __device__ __forceinline__ int gmaxi(int v) {
 #pragma unroll
         for (int d = 32; d > 0; d >>= 1) v = max(v, __shfl_xor(v, d));
         if ((t & 63) == 0) ired[t >> 6] = v;
         __syncthreads();
-        v = max(max(ired[0], ired[1]), max(ired[2], ired[3]));
+        v = ired[0];
+#pragma unroll
+        for (int w = 1; w < kGenWaves; w++) v = max(v, ired[w]);
         __syncthreads();
         return v;
     }
@@ -618,13 +638,14 @@ struct BlockGroup {
         int before = 0;
         total = 0;
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
+        for (int w = 0; w < kGenWaves; w++) {
             before += w < wave ? ired[w] : 0;
             total += ired[w];
         }
         __syncthreads();
         return before + incl - v;
     }
+    __device__ __forceinline__ void stamp(int) {}   // phase marker of a profiling build
     __device__ __forceinline__ float cosine(float x) { return (float)cos((double)x); }
     __device__ __forceinline__ float sine(float x) { return (float)sin((double)x); }
 };
@@ -638,22 +659,22 @@ struct FieldList {          // the per-field arrays of one EnvArrays, for table-
 // k_env_init / k_reset_list_block (craftax_full.cu:8669-8706, 8957-8975): one workgroup per
 // floor of an env.  LIST: the envs of the reset list, world key from each record's reset key, the env's
 // own key kept.  Otherwise: envs [0, A.n), env i created from seed0 + i as c_init does.
-template <bool LIST>
-__global__ __launch_bounds__(kGenThreads) void k_env_worldgen(EnvArrays A, FieldList fl, const float* __restrict__ light,
+template <bool LIST, int NT>
+__global__ __launch_bounds__(NT) void k_env_worldgen(EnvArrays A, FieldList fl, const float* __restrict__ light,
                                                               const cfp_env_reset_rec* __restrict__ resets,
                                                               const int* __restrict__ reset_count, uint64_t seed0,
                                                               int zero_fields) {
     __shared__ FloorScratch sc;
-    __shared__ float fred[4];
-    __shared__ int ired[4];
-    BlockGroup g{(int)threadIdx.x, fred, ired};
+    __shared__ float fred[8 * (NT / 64)];
+    __shared__ int ired[NT / 64];
+    BlockGroup<NT> g{(int)threadIdx.x, fred, ired};
     const int t = threadIdx.x;
     const size_t n = (size_t)A.n;
-    // one workgroup per (env, floor): the nine floors of a world are independent, and a step
-    // waits for its slowest reset
-    const int total = (LIST ? *reset_count : A.n) * kLevels;
+    // one workgroup per (env, floor) and one per env for the scalar fields: the ten jobs of a
+    // world are independent, and a step waits for its slowest reset
+    const int total = (LIST ? *reset_count : A.n) * kGenJobs;
     for (int job = blockIdx.x; job < total; job += gridDim.x) {
-        const int idx = job / kLevels, level = job - idx * kLevels;
+        const int idx = job / kGenJobs, level = job - idx * kGenJobs;
         size_t e;
         uint64_t world_key, env_key = 0;
         if (LIST) {
@@ -664,20 +685,20 @@ __global__ __launch_bounds__(kGenThreads) void k_env_worldgen(EnvArrays A, Field
             env_key = lcg(seed_key((uint32_t)(seed0 + (uint64_t)idx)));
             world_key = world_key_of_reset(lcg(env_key));
         }
-        if (level == 0) {
+        if (level == kLevels) {
             // scalars: the fields of `fl` are zero in a fresh state; the others are written below
             for (int f = 0; f < zero_fields; f++) {
                 const int el = fl.elem[f];
-                for (int k = t; k < fl.count[f]; k += kGenThreads) {
+                for (int k = t; k < fl.count[f]; k += NT) {
                     const size_t at = (size_t)k * n + e;
                     if (el == 4) ((uint32_t*)fl.ptr[f])[at] = 0u;
                     else if (el == 8) ((uint64_t*)fl.ptr[f])[at] = 0ull;
                     else ((uint8_t*)fl.ptr[f])[at] = 0;
                 }
             }
-            for (int k = t; k < kMobSlots; k += kGenThreads)
+            for (int k = t; k < kMobSlots; k += NT)
                 A.mob_health[(size_t)k * n + e] = (k / 27 == P_RANGED && k % 3 == 2) ? 0.0f : 1.0f;
-            for (int k = t; k < 54; k += kGenThreads) {
+            for (int k = t; k < 54; k += NT) {
                 A.mob_projectile_directions[(size_t)k * n + e] = 1;
                 A.player_projectile_directions[(size_t)k * n + e] = 1;
             }
@@ -707,11 +728,12 @@ __global__ __launch_bounds__(kGenThreads) void k_env_worldgen(EnvArrays A, Field
                     A.rng_key[n + e] = (uint32_t)(env_key >> 32);
                 }
             }
+            continue;   // (uniform over the workgroup)
         }
         uint8_t* planes = A.planes + e * kEnvPlaneBytes;
         generate_floor(g, sc, world_key, level);
         // the three byte planes, 16 bytes a thread
-        for (int k = t; k < 3 * (int)(kPlaneBytes / 16); k += kGenThreads) {
+        for (int k = t; k < 3 * (int)(kPlaneBytes / 16); k += NT) {
             const int plane = k / (int)(kPlaneBytes / 16), off = k % (int)(kPlaneBytes / 16);
             const uint8_t* src = plane == 0 ? sc.map : (plane == 1 ? sc.item : sc.light);
             ((u4*)(planes + ((size_t)plane * kLevels + level) * kPlaneBytes))[off] = ((const u4*)src)[off];
@@ -975,8 +997,8 @@ int cfp_env_init(cfp_env* e, uint64_t seed, void* stream) {
     CFP_REQUIRE(e != nullptr, "cfp_env_init: NULL env");
     cfp::FieldList fl;
     const int m = cfp::zero_field_list(e->live, fl);
-    const int grid = e->live.n * cfp::kLevels < 8192 ? e->live.n * cfp::kLevels : 8192;
-    hipLaunchKernelGGL(cfp::k_env_worldgen<false>, dim3(grid), dim3(cfp::kGenThreads), 0, (hipStream_t)stream, e->live, fl,
+    const int grid = e->live.n * cfp::kGenJobs < 8192 ? e->live.n * cfp::kGenJobs : 8192;
+    hipLaunchKernelGGL((cfp::k_env_worldgen<false, cfp::kGenThreads>), dim3(grid), dim3(cfp::kGenThreads), 0, (hipStream_t)stream, e->live, fl,
                        e->light, nullptr, nullptr, seed, m);
     CFP_HIP_TRY(hipGetLastError());
     return cfp_env_seed_actions(e, seed, stream);
@@ -987,7 +1009,7 @@ int cfp_env_pool_fill(cfp_env* e, uint64_t seed, void* stream) {
     CFP_REQUIRE(e->pool_size > 0, "cfp_env_pool_fill: this env object was created without a reset pool");
     cfp::FieldList fl;
     const int m = cfp::zero_field_list(e->pool, fl);
-    hipLaunchKernelGGL(cfp::k_env_worldgen<false>, dim3(e->pool_size * cfp::kLevels < 8192 ? e->pool_size * cfp::kLevels : 8192),
+    hipLaunchKernelGGL((cfp::k_env_worldgen<false, cfp::kGenThreads>), dim3(e->pool_size * cfp::kGenJobs < 8192 ? e->pool_size * cfp::kGenJobs : 8192),
                        dim3(cfp::kGenThreads), 0,
                        (hipStream_t)stream, e->pool, fl, e->light, nullptr, nullptr, seed, m);
     CFP_HIP_TRY(hipGetLastError());
@@ -999,9 +1021,15 @@ int cfp_env_reset(cfp_env* e, void* stream) {
     cfp::FieldList fl;
     const int m = cfp::zero_field_list(e->live, fl);
     // the list is short (a fraction of a percent of the envs per step): a fixed grid strides it
-    const int grid = e->live.n * cfp::kLevels < 4608 ? e->live.n * cfp::kLevels : 4608;
-    hipLaunchKernelGGL(cfp::k_env_worldgen<true>, dim3(grid), dim3(cfp::kGenThreads), 0, (hipStream_t)stream, e->live, fl,
-                       e->light, e->resets, e->reset_count, 0ull, m);
+    const int grid = e->live.n * cfp::kGenJobs < 4608 ? e->live.n * cfp::kGenJobs : 4608;
+    // about one env in 240 finishes per step under random actions: up to 16 384 envs that is
+    // fewer jobs than the GPU holds at once, and the wider workgroup finishes each sooner
+    if (e->live.n <= 16384)
+        hipLaunchKernelGGL((cfp::k_env_worldgen<true, cfp::kGenThreadsFew>), dim3(grid), dim3(cfp::kGenThreadsFew), 0,
+                           (hipStream_t)stream, e->live, fl, e->light, e->resets, e->reset_count, 0ull, m);
+    else
+        hipLaunchKernelGGL((cfp::k_env_worldgen<true, cfp::kGenThreads>), dim3(grid), dim3(cfp::kGenThreads), 0,
+                           (hipStream_t)stream, e->live, fl, e->light, e->resets, e->reset_count, 0ull, m);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }

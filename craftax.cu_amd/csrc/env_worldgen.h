@@ -2,10 +2,10 @@
 // nine floors -- six "smooth" ones from four Perlin fields each (:209-300, 443-503,
 // 1248-1359, 1577-1700) and three dungeons of rooms and corridors (:1733-1944) -- plus the
 // player's starting scalars.  Written once for a cooperating group of threads: the gfx950
-// reset kernel runs it with one 256-thread workgroup per finished env and the floor's
+// reset kernel runs it with one workgroup of 256 or 512 threads per (env, floor) and the floor's
 // working set (four 48x48 float fields, the byte planes, the dungeon's padded canvas) in
 // LDS; the host build runs the same text with a group of one.  `G` supplies the group:
-//   int tid(), nt(); void sync(); float gmin(float), gmax(float); int gmaxi(int);
+//   int tid(), nt(); void sync(); void gminmax4(float (&)[4], float (&)[4]); int gmaxi(int);
 //   int gscan(int v, int& total)   exclusive prefix sum over the threads in tid order
 //   float cosine(float), sine(float)
 // Every per-cell draw is a pure function of (key, cell), so the split of cells over
@@ -89,12 +89,23 @@ CFE_FN SmoothCfg smooth_cfg(int ci) {
     return c;
 }
 
+// what the dungeon's eight rooms and eight corridors are, as numbers (canvas coordinates)
+struct DungeonPlan {
+    int8_t size_r[8], size_c[8], pos_r[8], pos_c[8];
+    int8_t chest_r[8], chest_c[8];
+    int8_t fountain_r[8], fountain_c[8];   // row -1: this room has no fountain
+    int8_t h_row[8], h_c0[8], h_c1[8];     // corridor k: cells (h_row, h_c0..h_c1) ...
+    int8_t v_col[8], v_r0[8], v_r1[8];     // ... and (v_r0..v_r1, v_col); an empty leg has end -1
+};
+// corners of the four noise fields of a smooth floor: 4 x 4, 4 x 4, 7 x 25, 13 x 13
+constexpr int kGradTotal = 16 + 16 + 175 + 169;
 // per-floor working set (LDS on the GPU)
 struct alignas(16) FloorScratch {
     float field[4][kCells];     // water, mountain, path, tree noise
     uint8_t map[kCells], item[kCells], light[kCells], lava[kCells];
-    float gx[176], gy[176];     // gradient table: at most 7 x 25 corners
+    float gx[kGradTotal], gy[kGradTotal];   // gradient tables of the four fields, one after the other
     int32_t ladder_down[2], ladder_up[2];
+    DungeonPlan plan;
 };
 // the dungeon's padded canvas lives where the noise fields are (a dungeon floor has none)
 static_assert(2 * kCanvas * kCanvas <= 4 * (int)sizeof(float) * kCells, "canvas fits in the noise fields");
@@ -146,49 +157,80 @@ CFE_FN int choose_cell(G& g, uint64_t key, F flag) {
     return g.gmaxi(found);
 }
 
-// One normalised Perlin field (craftax_generate_fractal_noise_2d with one octave, :443-503;
-// craftax_generate_perlin_noise_2d_scalar, :209-300).
+// The four normalised Perlin fields of a smooth floor (each craftax_generate_fractal_noise_2d
+// with one octave, :443-503; craftax_generate_perlin_noise_2d_scalar, :209-300), made together:
+// one pass over the gradient corners of all four, one over the cells, one group reduction for
+// the eight extrema.  Field f: subkey[f], res_r[f] x res_c[f] periods, result in sc.field[f].
 template <class G>
-CFE_FN void noise_field(G& g, FloorScratch& sc, uint64_t subkey, int res_r, int res_c, float* out) {
-    const uint64_t angle_key = lcg(lcg(lcg(lcg(subkey))));   // two splits, the right key each time
-    const int gw = res_c + 1, gh = res_r + 1;
-    for (int k = g.tid(); k < gw * gh; k += g.nt()) {
-        const float angle = 6.28318530717958647692f * unit_at(angle_key, (uint64_t)k);
+CFE_FN void noise_fields(G& g, FloorScratch& sc, const uint64_t (&subkey)[4], const int (&res_r)[4],
+                         const int (&res_c)[4]) {
+    int base[4];
+    int corners = 0;
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        base[f] = corners;
+        corners += (res_r[f] + 1) * (res_c[f] + 1);
+    }
+    for (int k = g.tid(); k < corners; k += g.nt()) {
+        // (selects, not indexing: the small tables stay in registers)
+        uint64_t sk = subkey[0];
+        int first = 0;
+#pragma unroll
+        for (int f = 1; f < 4; f++)
+            if (k >= base[f]) {
+                sk = subkey[f];
+                first = base[f];
+            }
+        const uint64_t angle_key = lcg(lcg(lcg(lcg(sk))));   // two splits, the right key each time
+        const float angle = 6.28318530717958647692f * unit_at(angle_key, (uint64_t)(k - first));
         sc.gx[k] = g.cosine(angle);
         sc.gy[k] = g.sine(angle);
     }
     g.sync();
-    const int cr = kMap / res_r, cc = kMap / res_c;
     int lo, hi;
     my_cells(g, lo, hi);
-    float vmin = 3.0e38f, vmax = -3.0e38f;
+    float vmin[4], vmax[4];
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        vmin[f] = 3.0e38f;
+        vmax[f] = -3.0e38f;
+    }
     for (int i = lo; i < hi; i++) {
         const int row = i / kMap, col = i - row * kMap;
-        const int gr = row / cr, gc = col / cc;
-        const float lr = (float)(row - gr * cr) / (float)cr, lc = (float)(col - gc * cc) / (float)cc;
-        const float ir = lr * lr * lr * (lr * (lr * 6.0f - 15.0f) + 10.0f);
-        const float ic = lc * lc * lc * (lc * (lc * 6.0f - 15.0f) + 10.0f);
-        const int i00 = gr * gw + gc, i10 = i00 + gw;
-        float n00 = lr * sc.gx[i00];
-        n00 += lc * sc.gy[i00];
-        float n10 = (lr - 1.0f) * sc.gx[i10];
-        n10 += lc * sc.gy[i10];
-        float n01 = lr * sc.gx[i00 + 1];
-        n01 += (lc - 1.0f) * sc.gy[i00 + 1];
-        float n11 = (lr - 1.0f) * sc.gx[i10 + 1];
-        n11 += (lc - 1.0f) * sc.gy[i10 + 1];
-        const float n0 = n00 * (1.0f - ir) + ir * n10;
-        const float n1 = n01 * (1.0f - ir) + ir * n11;
-        float v = 1.41421356237309504880f * ((1.0f - ic) * n0 + ic * n1);
-        v = 0.0f + 1.0f * v;     // the octave accumulation: out = 0; out += amplitude * perlin
-        out[i] = v;
-        vmin = v < vmin ? v : vmin;
-        vmax = v > vmax ? v : vmax;
+#pragma unroll
+        for (int f = 0; f < 4; f++) {
+            const int gw = res_c[f] + 1;
+            const int cr = kMap / res_r[f], cc = kMap / res_c[f];
+            const float* gx = sc.gx + base[f];
+            const float* gy = sc.gy + base[f];
+            const int gr = row / cr, gc = col / cc;
+            const float lr = (float)(row - gr * cr) / (float)cr, lc = (float)(col - gc * cc) / (float)cc;
+            const float ir = lr * lr * lr * (lr * (lr * 6.0f - 15.0f) + 10.0f);
+            const float ic = lc * lc * lc * (lc * (lc * 6.0f - 15.0f) + 10.0f);
+            const int i00 = gr * gw + gc, i10 = i00 + gw;
+            float n00 = lr * gx[i00];
+            n00 += lc * gy[i00];
+            float n10 = (lr - 1.0f) * gx[i10];
+            n10 += lc * gy[i10];
+            float n01 = lr * gx[i00 + 1];
+            n01 += (lc - 1.0f) * gy[i00 + 1];
+            float n11 = (lr - 1.0f) * gx[i10 + 1];
+            n11 += (lc - 1.0f) * gy[i10 + 1];
+            const float n0 = n00 * (1.0f - ir) + ir * n10;
+            const float n1 = n01 * (1.0f - ir) + ir * n11;
+            float v = 1.41421356237309504880f * ((1.0f - ic) * n0 + ic * n1);
+            v = 0.0f + 1.0f * v;     // the octave accumulation: out = 0; out += amplitude * perlin
+            sc.field[f][i] = v;
+            vmin[f] = v < vmin[f] ? v : vmin[f];
+            vmax[f] = v > vmax[f] ? v : vmax[f];
+        }
     }
-    vmin = g.gmin(vmin);
-    vmax = g.gmax(vmax);
-    const float scale = vmax - vmin;
-    for (int i = lo; i < hi; i++) out[i] = (out[i] - vmin) / scale;
+    g.gminmax4(vmin, vmax);
+#pragma unroll
+    for (int f = 0; f < 4; f++) {
+        const float scale = vmax[f] - vmin[f];
+        for (int i = lo; i < hi; i++) sc.field[f][i] = (sc.field[f][i] - vmin[f]) / scale;
+    }
     g.sync();
 }
 
@@ -200,17 +242,17 @@ CFE_FN void smooth_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
     float* mountain = sc.field[1];
     float* path = sc.field[2];
     float* tree = sc.field[3];
-    uint64_t sub = next_key(rng);
-    noise_field(g, sc, sub, 3, 3, water);
+    uint64_t sub[4];
+    sub[0] = next_key(rng);
     (void)next_key(rng);
-    sub = next_key(rng);
-    noise_field(g, sc, sub, 3, 3, mountain);
-    sub = next_key(rng);
-    noise_field(g, sc, sub, 6, 24, path);
+    sub[1] = next_key(rng);
+    sub[2] = next_key(rng);
     (void)next_key(rng);
-    sub = next_key(rng);
+    sub[3] = next_key(rng);
     const uint64_t tree_key = rng;
-    noise_field(g, sc, sub, 12, 12, tree);
+    const int res_r[4] = {3, 3, 6, 12}, res_c[4] = {3, 3, 24, 12};
+    noise_fields(g, sc, sub, res_r, res_c);
+    g.stamp(1);
 
     uint64_t ore_rng = next_key(rng);
     uint64_t ore_key[5];
@@ -249,6 +291,7 @@ CFE_FN void smooth_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
         sc.lava[i] = lava;
     }
     g.sync();
+    g.stamp(2);
 
     // the diamond draw (:1662-1670) rewrites a stone cell with stone -- or cell 0 when the
     // floor has no stone at all
@@ -270,6 +313,7 @@ CFE_FN void smooth_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
         sc.ladder_up[1] = up % kMap;
         if (c.ladder_down) sc.item[down] = I_LADDER_DOWN;
     }
+    g.stamp(3);
     // craftax_apply_ladder_light (:1148-1169): a 9x9 torch pattern around the up ladder
     int r0 = up / kMap - 4, c0 = up % kMap - 4;
     if (r0 < 0) r0 += kMap;
@@ -307,6 +351,7 @@ CFE_FN void smooth_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
     g.sync();
     if (g.tid() == 0 && c.ladder_up) sc.item[up] = I_LADDER_UP;
     g.sync();
+    g.stamp(4);
 }
 
 // craftax_generate_dungeon_config (:1733-1944).  Rooms and corridors are a few hundred
@@ -318,23 +363,21 @@ CFE_FN void dungeon_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
     const uint8_t rare_path = ci == 1 ? B_WATER : B_PATH;
     uint8_t* canvas = reinterpret_cast<uint8_t*>(sc.field[0]);
     uint8_t* items = canvas + kCanvas * kCanvas;
-    for (int k = g.tid(); k < kCanvas * kCanvas; k += g.nt()) {
-        const int row = k / kCanvas, col = k - row * kCanvas;
-        const bool inner = row >= kPad && row < kPad + kMap && col >= kPad && col < kPad + kMap;
-        canvas[k] = inner ? B_WALL : 0;
-        items[k] = I_NONE;
-    }
-    g.sync();
     // key schedule: split3 -> (rng, ignored, room sizes); split -> room_rng; later path_rng, rare, ladders
     const uint64_t size_key = lcg(lcg(lcg(rng)));
     rng = lcg(rng);
     uint64_t room_rng = next_key(rng);
     uint64_t path_rng = next_key(rng);
+    // The reference draws eight rooms and eight corridors one after the other onto the canvas
+    // (a few hundred dependent byte writes).  Here one thread only draws the numbers -- the
+    // plan below, arithmetic and no memory -- and the group paints from it: the rooms in
+    // order, a cell a thread; then the corridors, which only ever turn wall into path and so
+    // need no order among themselves; then the special block of room 0.
+    DungeonPlan& plan = sc.plan;
     if (g.tid() == 0) {
-        int size_r[8], size_c[8], pos_r[8], pos_c[8];
         for (int k = 0; k < 8; k++) {
-            size_r[k] = int_at(size_key, 2 * k, 5, 10);
-            size_c[k] = int_at(size_key, 2 * k + 1, 5, 10);
+            plan.size_r[k] = (int8_t)int_at(size_key, 2 * k, 5, 10);
+            plan.size_c[k] = (int8_t)int_at(size_key, 2 * k + 1, 5, 10);
         }
         uint32_t free_chunks = 0x1ff;
         for (int k = 0; k < 8; k++) {
@@ -350,21 +393,18 @@ CFE_FN void dungeon_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
             key = next_key(room_rng);
             const int rr = (chunk % 3) * 16 + kPad + int_at(key, 0, 0, 11);
             const int rc = (chunk / 3) * 16 + kPad + int_at(key, 1, 0, 11);
-            pos_r[k] = rr;
-            pos_c[k] = rc;
-            for (int a = 0; a < size_r[k]; a++)
-                for (int b = 0; b < size_c[k]; b++) canvas[(rr + a) * kCanvas + rc + b] = B_PATH;
-            items[rr * kCanvas + rc] = I_TORCH;
-            items[(rr + size_r[k] - 1) * kCanvas + rc] = I_TORCH;
-            items[rr * kCanvas + rc + size_c[k] - 1] = I_TORCH;
-            items[(rr + size_r[k] - 1) * kCanvas + rc + size_c[k] - 1] = I_TORCH;
+            plan.pos_r[k] = (int8_t)rr;
+            plan.pos_c[k] = (int8_t)rc;
             key = next_key(room_rng);
-            canvas[(rr + int_at(key, 0, 1, size_r[k] - 1)) * kCanvas + rc + int_at(key, 1, 1, size_c[k] - 1)] = B_CHEST;
+            plan.chest_r[k] = (int8_t)(rr + int_at(key, 0, 1, plan.size_r[k] - 1));
+            plan.chest_c[k] = (int8_t)(rc + int_at(key, 1, 1, plan.size_c[k] - 1));
             // split3: (room_rng, fountain position, fountain coin)
             const uint64_t fkey = lcg(lcg(room_rng)), coin = lcg(fkey);
             room_rng = lcg(room_rng);
-            const int fr = int_at(fkey, 0, 1, size_r[k] - 1), fc = int_at(fkey, 1, 1, size_c[k] - 1);
-            if (draw_unit(coin) > 0.5f) canvas[(rr + fr) * kCanvas + rc + fc] = fountain;
+            const int fr = int_at(fkey, 0, 1, plan.size_r[k] - 1), fc = int_at(fkey, 1, 1, plan.size_c[k] - 1);
+            const bool has = draw_unit(coin) > 0.5f;
+            plan.fountain_r[k] = (int8_t)(has ? rr + fr : -1);
+            plan.fountain_c[k] = (int8_t)(rc + fc);
         }
         uint32_t linked = 0x80;   // room 7 is the first sink
         for (int k = 0; k < 8; k++) {
@@ -375,23 +415,63 @@ CFE_FN void dungeon_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
             uint32_t m = linked;
             for (int j = 1; j < want; j++) m &= m - 1;
             const int sink = __builtin_ctz(m);
-            const int dc = pos_c[sink] - pos_c[k], dr = pos_r[sink] - pos_r[k];
-            if (dc != 0) {
-                const int c0 = dc > 0 ? pos_c[k] : pos_c[sink], c1 = dc > 0 ? pos_c[sink] : pos_c[k];
-                for (int col = c0; col <= c1; col++)
-                    if (canvas[pos_r[k] * kCanvas + col] == B_WALL) canvas[pos_r[k] * kCanvas + col] = B_PATH;
-            }
-            if (dr != 0) {
-                const int r0 = dr > 0 ? pos_r[k] : pos_r[sink], r1 = dr > 0 ? pos_r[sink] : pos_r[k];
-                for (int row = r0; row <= r1; row++)
-                    if (canvas[row * kCanvas + pos_c[sink]] == B_WALL) canvas[row * kCanvas + pos_c[sink]] = B_PATH;
-            }
+            // the corridor runs along room k's row to the sink's column, then along that column
+            const int ck = plan.pos_c[k], cs = plan.pos_c[sink], rk = plan.pos_r[k], rs = plan.pos_r[sink];
+            plan.h_row[k] = (int8_t)rk;
+            plan.h_c0[k] = (int8_t)(ck < cs ? ck : cs);
+            plan.h_c1[k] = (int8_t)(ck == cs ? -1 : (ck < cs ? cs : ck));   // empty when the columns agree
+            plan.v_col[k] = (int8_t)cs;
+            plan.v_r0[k] = (int8_t)(rk < rs ? rk : rs);
+            plan.v_r1[k] = (int8_t)(rk == rs ? -1 : (rk < rs ? rs : rk));
             path_rng = lcg(lcg(path_rng));
             linked |= 1u << k;
         }
-        canvas[(pos_r[0] + 2) * kCanvas + pos_c[0] + 2] = special;
     }
     g.sync();
+    g.stamp(1);
+    for (int k = g.tid(); k < kCanvas * kCanvas; k += g.nt()) {
+        const int row = k / kCanvas, col = k - row * kCanvas;
+        const bool inner = row >= kPad && row < kPad + kMap && col >= kPad && col < kPad + kMap;
+        canvas[k] = inner ? B_WALL : 0;
+        items[k] = I_NONE;
+    }
+    g.sync();
+    // rooms one after the other (a later room's floor covers what an earlier one put where
+    // they overlap), each cell of a room written once by its own thread: floor, or the chest,
+    // or the fountain, which is drawn after the chest
+    for (int q = 0; q < 8; q++) {
+        const int rr = plan.pos_r[q], rc = plan.pos_c[q], sr = plan.size_r[q], sz = plan.size_c[q];
+        for (int k = g.tid(); k < sr * sz; k += g.nt()) {
+            const int a = k / sz, b = k - a * sz;
+            const int row = rr + a, col = rc + b;
+            int v = B_PATH;
+            if (row == plan.chest_r[q] && col == plan.chest_c[q]) v = B_CHEST;
+            if (row == plan.fountain_r[q] && col == plan.fountain_c[q]) v = fountain;
+            canvas[row * kCanvas + col] = (uint8_t)v;
+            if ((a == 0 || a == sr - 1) && (b == 0 || b == sz - 1)) items[row * kCanvas + col] = I_TORCH;
+        }
+        g.sync();
+    }
+    // the sixteen corridor legs together: each only turns wall into path
+    for (int k = g.tid(); k < 16 * 64; k += g.nt()) {
+        const int leg = k >> 6, i = k & 63, q = leg & 7;
+        int row, col;
+        bool on;
+        if (leg < 8) {
+            row = plan.h_row[q];
+            col = plan.h_c0[q] + i;
+            on = col <= plan.h_c1[q];
+        } else {
+            col = plan.v_col[q];
+            row = plan.v_r0[q] + i;
+            on = row <= plan.v_r1[q];
+        }
+        if (on && canvas[row * kCanvas + col] == B_WALL) canvas[row * kCanvas + col] = B_PATH;
+    }
+    g.sync();
+    if (g.tid() == 0) canvas[(plan.pos_r[0] + 2) * kCanvas + plan.pos_c[0] + 2] = special;
+    g.sync();
+    g.stamp(2);
     const uint64_t rare_key = next_key(rng);
     int lo, hi;
     my_cells(g, lo, hi);
@@ -414,6 +494,7 @@ CFE_FN void dungeon_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
         sc.lava[i] = 0;
     }
     g.sync();
+    g.stamp(3);
     uint64_t key = next_key(rng);
     const int down = choose_cell(g, key, [&](int i) { return sc.map[i] == B_PATH; });
     key = next_key(rng);
@@ -427,6 +508,7 @@ CFE_FN void dungeon_floor(G& g, FloorScratch& sc, uint64_t rng, int ci) {
         sc.item[up] = I_LADDER_UP;   // written second: wins when both land on one cell
     }
     g.sync();
+    g.stamp(4);
 }
 
 // The key of each floor and of the two trailing draws (craftax_generate_world_from_key_lazy,

@@ -176,6 +176,48 @@ def test_collect_with_the_env_on_the_device(pkg, cuda, ref):
     assert np.isfinite(adv).all() and np.abs(adv).max() > 0
 
 
+def test_collect_regenerating_worlds(pkg, cuda, ref):
+    """cfp_train_collect without a reset pool: finished envs are regenerated from their reset
+    keys on the device.  Replayed through the reference env, which regenerates the same worlds
+    from the same keys: every step's observations, rewards and done flags are the slabs', and
+    the final states agree."""
+    import ctypes as C
+    n, T, seed = 128, 48, 9
+    ref.init(n, seed)
+    states = ref.export()
+    weak = states.copy()
+    for e in range(0, n, 3):            # a third of the envs starve within the horizon
+        weak["player_health"][e] = 1.0 + (e % 4)
+        weak["player_food"][e] = 0
+        weak["player_drink"][e] = 0
+        weak["player_recover"][e] = -14.0 + (e % 7)
+        ref.import_(e, weak[e])
+    env = pkg.Env(n)
+    env.import_states(weak)
+    pol = pkg.Policy(n, layers=3, seed=1)
+    tr = pkg.Trainer(pol, T)
+    env.collect(tr, seed=77)
+    torch.cuda.synchronize()
+    r_obs = tr.buf("r_obs").cpu().numpy()
+    r_act = tr.buf("r_act").cpu().numpy()
+    r_rew = tr.buf("r_reward").cpu().numpy()
+    r_done = tr.buf("r_done").cpu().numpy()
+    ref.lib.cfref_encode.argtypes = [C.c_int, C.c_void_p]
+    rec = np.zeros((n, 996), np.uint8)
+    finished = 0
+    for t in range(T):
+        for e in range(n):
+            ref.lib.cfref_encode(e, C.c_void_p(rec[e].ctypes.data))
+        assert np.array_equal(rec, r_obs[t]), f"observations of step {t}"
+        final, rew, term, keys = ref.step(r_act[t].astype(np.float32))
+        assert np.array_equal(rew.view(np.uint32), r_rew[t].view(np.uint32)), f"rewards of step {t}"
+        assert np.array_equal(term.astype(np.uint8), r_done[t]), f"done flags of step {t}"
+        finished += int(term.sum())
+    assert finished >= 20
+    assert not eb.diff_fields(ref.export(), env.export_states(eb.STATE_DTYPE)), "states after the rollout"
+    tr.close(); pol.close()
+
+
 def _cell_agreement(a, b):
     """(differing cells, cells, worlds with any difference) over the three byte maps."""
     diff = np.zeros(len(a), bool)
