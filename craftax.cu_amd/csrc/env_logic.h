@@ -977,20 +977,6 @@ CFE_FN void boss_and_attributes(Hot& h, int action) {
 }
 
 // ---- mobs (craftax_update_mobs_native, :6269-7377) -----------------------------------------
-// craftax_update_mobs_valid_position (:6625-6648)
-template <class S>
-CFE_FN bool mob_can_stand(S& s, const Hot& h, int r, int c, int collision) {
-    if (!on_map(r, c)) return false;
-    const int b = s.blk(wrap_clamp(h.level, kLevels), r, c);
-    const bool solid = is_solid(b), water = b == B_WATER, lava = b == B_LAVA;
-    const bool ground = !solid && !water && !lava;
-    bool ok = !mob_or_player_at(s, h, r, c) && !solid;
-    ok = ok && (!(collision & 1) || !ground);
-    ok = ok && (!(collision & 2) || !water);
-    ok = ok && (!(collision & 4) || !lava);
-    return ok;
-}
-
 // craftax_update_mobs_damage_done_to_player (:6659-6680)
 CFE_FN float damage_to_player(const Hot& h, const float (&dmg)[3]) {
     float def[3] = {0.0f, 0.0f, 0.0f};
@@ -1007,13 +993,54 @@ CFE_FN float damage_to_player(const Hot& h, const float (&dmg)[3]) {
     return total;
 }
 
-// a mob leaves (r0, c0) and, if it stays alive, occupies (r1, c1) in the level's mob bitmap
-// (craftax_update_mobs_clear_old_map_entry / _enter_new_map_entry, :6389-6421)
+// What a moving mob reads from memory -- the block under its target cell and the two rows of
+// the level's mob bitmap it may leave and enter -- asked for together, so that a mob costs
+// one memory round trip instead of one per dependent read (validity test, bitmap clear,
+// bitmap set).  The indices are always addressable (wrap_clamp); whether a value is used is
+// decided afterwards.
+struct MoverView {
+    int b;                       // block at (i_to, wrap_clamp(c1))
+    uint64_t row_from, row_to;   // bitmap rows i_from = wrap_clamp(r0), i_to = wrap_clamp(r1)
+    int i_from, i_to;
+};
 template <class S>
-CFE_FN void move_in_bitmap(S& s, int l, int r0, int c0, int r1, int c1, bool alive) {
-    int lr, lc;
-    if (wrap_drop(r0, kMap, lr) && wrap_drop(c0, kMap, lc)) s.put_mobrow(l, lr, s.mobrow(l, lr) & ~(1ull << lc));
-    if (alive && wrap_drop(r1, kMap, lr) && wrap_drop(c1, kMap, lc)) s.put_mobrow(l, lr, s.mobrow(l, lr) | (1ull << lc));
+CFE_FN MoverView mover_view(S& s, int l, int r0, int r1, int c1) {
+    MoverView v;
+    v.i_from = wrap_clamp(r0, kMap);
+    v.i_to = wrap_clamp(r1, kMap);
+    v.b = s.blk(l, v.i_to, wrap_clamp(c1, kMap));
+    v.row_from = s.mobrow(l, v.i_from);
+    v.row_to = s.mobrow(l, v.i_to);
+    return v;
+}
+// craftax_update_mobs_valid_position (:6625-6648) for the view's target (r, c)
+CFE_FN bool can_stand_view(const Hot& h, const MoverView& v, int r, int c, int collision) {
+    const bool solid = is_solid(v.b), water = v.b == B_WATER, lava = v.b == B_LAVA;
+    const bool ground = !solid && !water && !lava;
+    const bool mob = (v.row_to >> wrap_clamp(c, kMap)) & 1ull;
+    bool ok = on_map(r, c) && !(mob || (h.pr == r && h.pc == c)) && !solid;
+    ok = ok && (!(collision & 1) || !ground);
+    ok = ok && (!(collision & 2) || !water);
+    ok = ok && (!(collision & 4) || !lava);
+    return ok;
+}
+// A mob leaves (r0, c0) and, if it stays alive, occupies (rf, cf) -- its old cell or the
+// view's target -- in the level's mob bitmap (craftax_update_mobs_clear_old_map_entry /
+// _enter_new_map_entry, :6389-6421: scatter indices, negative wraps, 48 and beyond is
+// dropped).  A valid scatter index equals the clamped one, so the row left is i_from and
+// the row entered i_from or i_to; both changes to one row go out as one write.
+template <class S>
+CFE_FN void settle_in_bitmap(S& s, int l, const MoverView& v, int r0, int c0, int rf, int cf, bool alive) {
+    int lr0, lc0, lrf = 0, lcf = 0;
+    const bool clr = wrap_drop(r0, kMap, lr0) && wrap_drop(c0, kMap, lc0);
+    const bool set = alive && wrap_drop(rf, kMap, lrf) && wrap_drop(cf, kMap, lcf);
+    uint64_t from = v.row_from, to = v.row_to;
+    if (clr) from &= ~(1ull << lc0);
+    const bool into_from = set && lrf == v.i_from;
+    if (into_from) from |= 1ull << lcf;
+    if (set && !into_from) to |= 1ull << lcf;
+    if (clr || into_from) s.put_mobrow(l, v.i_from, from);
+    if (set && !into_from) s.put_mobrow(l, v.i_to, to);
 }
 
 // the step towards the player along the longer axis, drawn when both are equal
@@ -1059,14 +1086,15 @@ CFE_FN void move_melee(S& s, Hot& h, uint64_t& rng, int i) {
     h.health -= damage * (float)(int)attacking;
     unlock_if(h, ACH_WAKE_UP, h.sleeping && attacking);
     if (attacking) h.sleeping = h.resting = 0;
-    const bool ok = mob_can_stand(s, h, r1, c1, mob_collision(type, MC_MELEE));
+    const MoverView view = mover_view(s, l, r0, r1, c1);
+    const bool ok = can_stand_view(h, view, r1, c1, mob_collision(type, MC_MELEE));
     if (!ok) {
         r1 = r0;
         c1 = c0;
     }
     const bool alive = dist < kDespawn || at_boss(h);
     rng = lcg(lcg(rng));
-    move_in_bitmap(s, l, r0, c0, r1, c1, alive);
+    settle_in_bitmap(s, l, view, r0, c0, r1, c1, alive);
     s.set_m_pos(P_MELEE, i, r1, c1);
     s.set_m_cd(P_MELEE, i, attacking ? 5 : cd - 1);
     s.set_m_mask(P_MELEE, i, alive);
@@ -1080,12 +1108,13 @@ CFE_FN void move_passive(S& s, Hot& h, uint64_t& rng, int i) {
     const int r0 = s.m_row(P_PASSIVE, i), c0 = s.m_col(P_PASSIVE, i), type = s.m_type(P_PASSIVE, i);
     const Vec2 rnd = random_step(next_key(rng), 8);
     int r1 = r0 + rnd.r, c1 = c0 + rnd.c;
-    if (!mob_can_stand(s, h, r1, c1, mob_collision(type, MC_PASSIVE))) {
+    const MoverView view = mover_view(s, l, r0, r1, c1);
+    if (!can_stand_view(h, view, r1, c1, mob_collision(type, MC_PASSIVE))) {
         r1 = r0;
         c1 = c0;
     }
     const bool alive = iabs(r0 - h.pr) + iabs(c0 - h.pc) < kDespawn;
-    move_in_bitmap(s, l, r0, c0, r1, c1, alive);
+    settle_in_bitmap(s, l, view, r0, c0, r1, c1, alive);
     s.set_m_pos(P_PASSIVE, i, r1, c1);
     s.set_m_mask(P_PASSIVE, i, alive);
 }
@@ -1110,8 +1139,13 @@ CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
         c1 = c0 + rnd.c;
     }
     const int collision = mob_collision(type, MC_RANGED);
+    // the target's validity is read once: the reference asks for it up to twice (here and
+    // below), for this target or -- when the mob attacks and stays -- for its own cell, which
+    // it occupies itself, so that answer never changes where the mob ends up
+    const MoverView view = mover_view(s, l, r0, r1, c1);
+    const bool can = can_stand_view(h, view, r1, c1, collision);
     bool attacking = dist >= 4 && dist <= 5;
-    attacking = attacking || (close && !mob_can_stand(s, h, r1, c1, collision));
+    attacking = attacking || (close && !can);
     attacking = attacking && cd <= 0;
     if (attacking) {
         // craftax_update_mobs_spawn_mob_projectile (:6682-6723)
@@ -1130,12 +1164,12 @@ CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
         r1 = r0;
         c1 = c0;
     }
-    if (!mob_can_stand(s, h, r1, c1, collision)) {
+    if (!can) {
         r1 = r0;
         c1 = c0;
     }
     const bool alive = dist < kDespawn || at_boss(h);
-    move_in_bitmap(s, l, r0, c0, r1, c1, alive);
+    settle_in_bitmap(s, l, view, r0, c0, r1, c1, alive);
     s.set_m_pos(P_RANGED, i, r1, c1);
     s.set_m_cd(P_RANGED, i, attacking ? 4 : cd - 1);
     s.set_m_mask(P_RANGED, i, alive);
@@ -1150,7 +1184,8 @@ CFE_FN void move_mob_projectile(S& s, Hot& h, int i) {
     const int r1 = r0 + s.pd_r(P_MOB_PROJ, i), c1 = c0 + s.pd_c(P_MOB_PROJ, i);
     const int b = s.blk(wrap_clamp(l, kLevels), wrap_clamp(r1, kMap), wrap_clamp(c1, kMap));
     const bool hit = (r0 == h.pr && c0 == h.pc) || (r1 == h.pr && c1 == h.pc);
-    const bool flying = on_map(r1, c1) && !is_solid(b) && !mob_or_player_at(s, h, r1, c1) && !hit;
+    const bool taken = mob_or_player_at(s, h, r1, c1);   // read beside the block, not after it
+    const bool flying = on_map(r1, c1) && !is_solid(b) && !taken && !hit;
     float dmg[3];
     mob_damage(s.m_type(P_MOB_PROJ, i), MC_PROJECTILE, dmg);
     const float damage = damage_to_player(h, dmg);
