@@ -79,6 +79,32 @@ def measured_traffic(n):
     return int(t) if t and t.isdigit() else None
 
 
+def policy_in_the_loop(pkg, torch, n, steps):
+    """The whole rollout step with the env on the device (record -> forward + sample -> game
+    step -> reward / done rows -> regeneration of finished worlds), reported beside `value`:
+    env-steps/s and the forward's FLOPs over the whole step's time against the fp32 peak."""
+    env = pkg.Env(n)
+    env.init(0)
+    pol = pkg.Policy(n, LAYERS, seed=1)
+    T = 8
+    tr = pkg.Trainer(pol, T)
+    for t in range(48):            # spreads the episodes' phases and settles the clock
+        env.rollout_step(tr, t % T, 1234)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for t in range(steps):
+        env.rollout_step(tr, t % T, 1234)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    out = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3, "steps": steps,
+           "frac_fp32_peak_of_forward_flops": FLOP_PER_ENV_STEP * n / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+           "what": "cfp_env_rollout_step: env, records, h256x3 policy, sampling and resets on the device"}
+    tr.close(); pol.close(); env.close()
+    return out
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -255,6 +281,8 @@ def main():
                      "launch_ms": launch_s * 1e3},
     }
     pol.close()
+    if args.schedule == "both":
+        line["policy_in_the_loop"] = policy_in_the_loop(pkg, torch, n, min(steps, 16))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(params, seed)
     print(json.dumps(line))

@@ -350,3 +350,29 @@ def smoke_forward(pkg):
     assert_close(av_h[:, ACTIONS], ref["values"], TOL_FP32, "smoke values")
     assert_close(state.cpu().numpy(), ref["state"], TOL_FP32, "smoke state")
     pol.close()
+
+
+def smoke_env(pkg):
+    """64 envs generated and stepped 20 times on cuda:0 against the compiled reference env
+    (oracle/_ref), every state field after every step; skipped when the checker is not built."""
+    import torch
+    import env_bind as eb
+    try:
+        ref = eb.Ref()
+    except FileNotFoundError:
+        print("smoke: oracle/_ref/libcfref.so is not built, env check skipped")
+        return
+    n, seed = 64, 5
+    ref.init(n, seed)
+    env = pkg.Env(n)
+    env.init(seed)
+    assert not eb.diff_fields(ref.export(), env.export_states(eb.STATE_DTYPE)), "smoke: generated worlds differ"
+    for t in range(20):
+        act = ref.next_actions()
+        final, rew, term, keys = ref.step(act)
+        env.step(None)
+        bad = eb.diff_fields(final, env.export_states(eb.STATE_DTYPE))
+        assert not bad, f"smoke: env step {t}: fields {bad[:4]} differ from the reference"
+        assert np.array_equal(rew.view(np.uint32), env.rewards.cpu().numpy().view(np.uint32))
+        env.reset()
+    env.close()
