@@ -792,6 +792,11 @@ CFE_FN void add_torch_light(S& s, int l, int r, int c) {
             if ((unsigned)cc >= (unsigned)kMap) continue;
             const float t = torch_light(dr, dc);
             if (t == 0.0f) continue;  // q / 255 * 255 truncates back to q for every byte q
+            // product and sum rounded separately, as the reference's GPU port spells it
+            // (craftax_full.cu:5163-5164, built with -fmad=false).  Its C build under gcc
+            // -ffast-math fuses the two into one multiply-add where the CPU has one, which
+            // gives a byte one higher for a third of the (byte, distance) pairs: that is
+            // the toolchain's choice, not the game's.
             float v = (float)s.lum(l, rr, cc) * (1.0f / 255.0f) + t;
             v = v < 0.0f ? 0.0f : v;
             v = v > 1.0f ? 1.0f : v;

@@ -62,6 +62,54 @@ def diff_fields(a, b):
     return out
 
 
+def deep_states(ref, n, seed):
+    """n reference worlds (ref.init) with the player moved onto floor e % 9 at that floor's
+    up ladder and given what a long episode collects: tools, weapons, arrows, torches, ores,
+    potions, books, armour with enchantments, spells, attribute points, kills on every floor,
+    a boss fight in progress on floor 8, a random hour of the day.  Random-action rollouts from
+    the freshly generated worlds rarely leave floors 0..2; these states put every floor's mob
+    table, the ranged mobs and their projectiles, spells, enchanting and the boss on the path.
+    The states are imported into the reference env (slot e) and returned."""
+    ref.init(n, seed)
+    st = ref.export()
+    rng = np.random.default_rng(seed)
+    for e in range(n):
+        s = st[e]
+        lvl = e % L
+        s["player_level"] = lvl
+        if lvl > 0:
+            s["player_position"] = s["up_ladders"][lvl]
+        s["player_direction"] = rng.integers(1, 5)
+        s["player_health"] = np.float32(rng.integers(4, 10))
+        for f in ("player_food", "player_drink", "player_energy", "player_mana"):
+            s[f] = rng.integers(3, 10)
+        for f in ("player_dexterity", "player_strength", "player_intelligence"):
+            s[f] = rng.integers(1, 6)
+        s["player_xp"] = rng.integers(0, 4)
+        for f in ("wood", "stone", "coal", "iron", "diamond", "sapling", "ruby", "sapphire"):
+            s[f] = rng.integers(0, 10)
+        s["pickaxe"] = rng.integers(0, 5)
+        s["sword"] = rng.integers(0, 5)
+        s["bow"] = rng.integers(0, 2)
+        s["arrows"] = rng.integers(0, 20)
+        s["torches"] = rng.integers(0, 10)
+        s["books"] = rng.integers(0, 3)
+        s["potions"] = rng.integers(0, 4, 6)
+        s["armour"] = rng.integers(0, 3, 4)
+        s["armour_enchantments"] = np.where(s["armour"] > 0, rng.integers(0, 3, 4), 0)
+        s["sword_enchantment"] = rng.integers(0, 3) if s["sword"] > 0 else 0
+        s["bow_enchantment"] = rng.integers(0, 3) if s["bow"] > 0 else 0
+        s["learned_spells"] = rng.integers(0, 2, 2)
+        s["monsters_killed"] = rng.choice([0, 3, 8, 12], L)
+        s["timestep"] = rng.integers(0, 6000)
+        s["light_level"] = ref.lib.cfref_light_level(int(s["timestep"]))
+        if lvl == L - 1:
+            s["boss_progress"] = rng.integers(0, 8)
+            s["boss_timesteps_to_spawn_this_round"] = rng.integers(0, 12)
+        ref.import_(e, s)
+    return st
+
+
 class Ref:
     """oracle/_ref/libcfref.so: the reference's own env, one global vector of envs."""
 

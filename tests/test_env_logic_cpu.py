@@ -54,6 +54,55 @@ def test_host_build_of_the_step_matches_reference(ref, n, steps, seed):
     assert terminals > 0
 
 
+@pytest.mark.parametrize("seed,steps", [(17, 400), (4242, 400)])
+def test_host_build_of_the_step_on_every_floor(seed, steps):
+    """The same comparison from states on all nine floors with full inventories, armour,
+    spells, enchantments and a boss fight under way (env_bind.deep_states), 144 envs x 400
+    steps, two seeds, against the reference source built with strict per-operation fp32 (oracle/Makefile,
+    second recipe) -- the arithmetic of the reference's GPU port (-fmad=false).  The
+    -ffast-math C build is no checker for these states: with armour worn gcc reorders the
+    defence sums of craftax_update_mobs_damage_done_to_player (:6659-6680; player_health one
+    or two ulp off), and it fuses light / 255 + torch into one multiply-add (:5046-5047; a
+    light byte one higher for a third of the byte / distance pairs) -- what a toolchain makes
+    of that source, not what the game defines; random play from fresh worlds wears no armour
+    and places no torch, which is why the 256 x 600 comparisons never see it.
+    The light level is the one place where the GPU port itself adopts the fast-math build's
+    fused form (its host-made table, craftax_full.cu:10715-10728); the table is held to that
+    build for every timestep in the test above, and here the step runs on the strict build's
+    table so that every other field can be compared bit for bit."""
+    try:
+        strict = eb.Ref(strict=True)
+    except FileNotFoundError:
+        pytest.skip("oracle/_ref/libcfref_strict.so is not built (reference source absent)")
+    n = 144
+    mine = eb.deep_states(strict, n, seed)
+    host = eb.HostStep()
+    host.light = np.array([strict.lib.cfref_light_level(t) for t in range(len(host.light))], np.float32)
+    assert not eb.diff_fields(strict.export(), mine), "import / export of the prepared states"
+    levels_seen, terminals, torches, hits_in_armour = set(), 0, 0, 0
+    for t in range(steps):
+        act = strict.next_actions()
+        before = mine.copy()
+        final, rew, term, keys = strict.step(act)
+        r2, t2, k2 = host.step(mine, act)
+        d = eb.diff_fields(final, mine)
+        if d:
+            bad = np.nonzero([bool(eb.diff_fields(final[i:i + 1], mine[i:i + 1])) for i in range(n)])[0]
+            raise AssertionError(f"step {t}: fields {d} differ in envs {bad[:6].tolist()} "
+                                 f"(floors {final['player_level'][bad[:6]].tolist()}, actions {act[bad[:6]].tolist()})")
+        assert np.array_equal(rew.view(np.uint32), r2.view(np.uint32)), f"step {t}: reward"
+        assert np.array_equal(term, t2) and np.array_equal(keys, k2), f"step {t}: terminal / reset key"
+        levels_seen |= set(final["player_level"].tolist())
+        torches += int((final["torches"] < before["torches"]).sum())
+        hits_in_armour += int(((final["player_health"] < before["player_health"] - 0.5) & (before["armour"].sum(axis=1) > 0)).sum())
+        done = np.nonzero(term)[0]
+        if len(done):
+            mine[done] = strict.export(list(done))
+            terminals += len(done)
+    assert levels_seen >= set(range(9)), levels_seen
+    assert terminals > 0 and torches >= 5 and hits_in_armour >= 5, (terminals, torches, hits_in_armour)
+
+
 def test_import_derives_spawn_planes_like_the_reference(ref):
     """craftax_refresh_spawn_bits_level (craftax_full.c:3336-3355)."""
     ref.init(8, 5)

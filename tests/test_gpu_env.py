@@ -218,6 +218,36 @@ def test_collect_regenerating_worlds(pkg, cuda, ref):
     tr.close(); pol.close()
 
 
+def test_env_step_on_every_floor_against_the_host_build(pkg, cuda, ref):
+    """States on all nine floors with full inventories, armour, spells, enchantments and a boss
+    fight under way (env_bind.deep_states): the GPU step against the host build of the same
+    game-logic text (oracle/libcfenvhost.so), every field after every step, 288 envs x 400
+    steps, resets supplied by the host generator.  The host build is held to the reference
+    (strict per-operation fp32 build) on these states by the CPU suite; together: the kernel
+    computes on deep floors what the reference's source defines."""
+    n, steps = 288 - 288 % 64, 400
+    states = eb.deep_states(ref, n, 23)
+    host = eb.HostStep()
+    env = pkg.Env(n)
+    env.import_states(states)
+    mine = states.copy()
+    levels_seen, terminals = set(), 0
+    for t in range(steps):
+        act = ref.next_actions()          # any action stream will do: the reference's own
+        rew, term, keys = host.step(mine, act)
+        env.step(torch.from_numpy(act).cuda())
+        got = env.export_states(eb.STATE_DTYPE)
+        _compare(f"step {t}", mine, got, rew, env.rewards.cpu().numpy(), term, env.terminals.cpu().numpy())
+        levels_seen |= set(mine["player_level"].tolist())
+        for e in np.nonzero(term)[0]:
+            st = mine[e:e + 1].copy()
+            host.lib.cfhost_reset(eb.ptr(st), eb.ptr(np.ascontiguousarray(keys[e])))
+            mine[e] = st[0]
+            env.import_states(st, first=int(e))
+            terminals += 1
+    assert levels_seen >= set(range(9)) and terminals > 0, (levels_seen, terminals)
+
+
 def _cell_agreement(a, b):
     """(differing cells, cells, worlds with any difference) over the three byte maps."""
     diff = np.zeros(len(a), bool)
