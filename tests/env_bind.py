@@ -106,6 +106,20 @@ def deep_states(ref, n, seed):
         if lvl == L - 1:
             s["boss_progress"] = rng.integers(0, 8)
             s["boss_timesteps_to_spawn_this_round"] = rng.integers(0, 12)
+        # every other env of the two dungeons that have an enchantment table stands in front of
+        # it (facing right) with the mana and the gems an enchantment costs
+        tables = np.argwhere((s["map"][lvl] == 30) | (s["map"][lvl] == 31))
+        if len(tables) and (e // L) % 2 == 0:
+            r, c = tables[0]
+            if c > 0 and s["map"][lvl, r, c - 1] == 7 and s["item_map"][lvl, r, c - 1] == 0:   # a free path cell
+                s["player_position"] = (r, c - 1)
+                s["player_direction"] = 2
+                s["player_mana"] = 9
+                s["ruby"] = max(int(s["ruby"]), 3)
+                s["sapphire"] = max(int(s["sapphire"]), 3)
+                s["sword"] = max(int(s["sword"]), 1)
+                s["bow"] = 1
+                s["armour"] = np.maximum(s["armour"], 1)
         ref.import_(e, s)
     return st
 
