@@ -18,6 +18,7 @@
                   envs' own random actions + world generation for finished envs (the
                   reference's "env only" figure, which also writes the observation
                   records), and the kernels one by one
+  train_iteration  collect + update with everything on the device, samples/s
   rollout_in_the_loop  policy in the loop: record -> forward + sample -> env step ->
                   reward/done rows -> reset (cfp_env_rollout_step), steps per second
 
@@ -448,6 +449,41 @@ def rollout_in_the_loop(pkg, torch, reps):
     return out
 
 
+def train_iteration(pkg, torch, reps):
+    """One PPO iteration with everything on the device, as the reference's `train` mode counts
+    it (README.md:348-356, horizon 128): cfp_train_collect (T rollout steps with the env, the
+    bootstrap value, GAE) followed by cfp_train_update (backward + Adam, captured graph)."""
+    out = {"workload": "train_iteration", "policy": "h256x3", "cases": {}}
+    for n, T in ((4096, 128), (8192, 128), (65536, 64)):
+        env = pkg.Env(n)
+        env.init(0)
+        pol = pkg.Policy(n, layers=3, seed=1)
+        if n <= 4096:
+            pol.set_small_tiles(True)
+        tr = pkg.Trainer(pol, T)
+        case = {}
+        for mode in ("fp32", "bf16_in_bf16_storage"):
+            bf = mode != "fp32"
+            pol.set_gemm_bf16(bf)
+            tr.set_gemm_mode(1 if bf else 0, 1)
+            tr.set_bf16_storage(bf)
+
+            def it():
+                env.collect(tr, 1234)
+                tr.update(use_graph=True)
+            ms = _time(torch, it, 3, warm=2)
+            ms_c = _time(torch, lambda: env.collect(tr, 1234), 3, warm=1)
+            case[mode] = {"ms_per_iteration": round(ms, 3), "ms_collect": round(ms_c, 3),
+                          "ms_update": round(ms - ms_c, 3), "M_samples_per_s": round(n * T / ms / 1e3, 2)}
+        pol.set_gemm_bf16(False)
+        assert torch.isfinite(pol.params).all()
+        out["cases"][f"{n}x{T}"] = case
+        tr.close()
+        pol.close()
+        env.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=10)
@@ -458,7 +494,7 @@ def main():
     pkg = ge.load_package()
     assert torch.cuda.is_available(), "bench_configs.py needs a GPU"
     for fn in (forward_65536, ppo_update, ppo_update_shapes, rollout_policy_side, classic_1m,
-               record_kernels, stream_ceilings, env_step, rollout_in_the_loop):
+               record_kernels, stream_ceilings, env_step, rollout_in_the_loop, train_iteration):
         if args.only and fn.__name__ != args.only:
             continue
         print(json.dumps(fn(pkg, torch, args.reps)), flush=True)
