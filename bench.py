@@ -85,10 +85,13 @@ def policy_in_the_loop(pkg, torch, n, steps):
     env-steps/s and the forward's FLOPs over the whole step's time against the fp32 peak."""
     env = pkg.Env(n)
     env.init(0)
+    for _ in range(300):           # random-action steps: the episodes' phases spread out
+        env.step(None)
+        env.reset()
     pol = pkg.Policy(n, LAYERS, seed=1)
     T = 8
     tr = pkg.Trainer(pol, T)
-    for t in range(48):            # spreads the episodes' phases and settles the clock
+    for t in range(16):            # settles the clock
         env.rollout_step(tr, t % T, 1234)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
@@ -99,6 +102,7 @@ def policy_in_the_loop(pkg, torch, n, steps):
     torch.cuda.synchronize()
     ms = e0.elapsed_time(e1) / steps
     out = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3, "steps": steps,
+           "finished_envs_last_step": env.reset_list()[0],
            "frac_fp32_peak_of_forward_flops": FLOP_PER_ENV_STEP * n / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
            "what": "cfp_env_rollout_step: env, records, h256x3 policy, sampling and resets on the device"}
     tr.close(); pol.close(); env.close()
@@ -282,7 +286,7 @@ def main():
     }
     pol.close()
     if args.schedule == "both":
-        line["policy_in_the_loop"] = policy_in_the_loop(pkg, torch, n, min(steps, 16))
+        line["policy_in_the_loop"] = policy_in_the_loop(pkg, torch, n, min(steps, 64))
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(params, seed)
     print(json.dumps(line))

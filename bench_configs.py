@@ -416,36 +416,40 @@ def env_step(pkg, torch, reps):
 
 def rollout_in_the_loop(pkg, torch, reps):
     """cu_rollout_step with everything on the device (the reference's `run` mode,
-    craftax_full.cu:12127-12176): h256x3 policy in the loop, fresh worlds on reset."""
+    craftax_full.cu:12127-12176): h256x3 policy in the loop.  Steady state: 300 random-action
+    steps first, so that the episodes' phases are spread and a step regenerates its share of
+    finished envs (about 0.3 % of them); `fresh_worlds` regenerates those from their reset keys
+    (k_reset_list), `reset_pool` copies them from a pool of 4096 worlds (the reference's pooled
+    reset, craftax_full.c:3738-3741)."""
     out = {"workload": "rollout_in_the_loop", "policy": "h256x3 fp32", "envs": {}}
     T = 8
     for n in (8192, 65536, 262144):
-        env = pkg.Env(n)
-        env.init(0)
-        pol = pkg.Policy(n, layers=3, seed=1)
-        tr = pkg.Trainer(pol, T)
-        state = {"t": 0}
+        res = {}
+        for mode, pool in (("fresh_worlds", 0), ("reset_pool", 4096)):
+            env = pkg.Env(n, pool=pool)
+            env.init(0)
+            if pool:
+                env.pool_fill(99)
+            for _ in range(300):
+                env.step(None)
+                env.reset_from_pool() if pool else env.reset()
+            pol = pkg.Policy(n, layers=3, seed=1)
+            tr = pkg.Trainer(pol, T)
+            state = {"t": 0}
 
-        def step():
-            env.rollout_step(tr, state["t"] % T, 1234)
-            state["t"] += 1
+            def step():
+                env.rollout_step(tr, state["t"] % T, 1234)
+                state["t"] += 1
 
-        for _ in range(40):
-            step()
-        torch.cuda.synchronize()
-        ms = _time(torch, step, max(16, 4 * reps))
-        out["envs"][str(n)] = {"us_per_step": round(ms * 1e3, 1), "M_env_steps_per_s": round(n / ms / 1e3, 2),
-                               "frac_fp32_peak_of_forward_flops": round(FWD_FLOP * n / (ms * 1e-3) / 1e12 / PEAK_FP32, 3)}
-        tr.close()
-        # cu_train_collect: T steps with the resets overlapped on the second stream, plus the
-        # bootstrap forward and GAE, per step
-        Tc = 32 if n <= 65536 else 16
-        tr = pkg.Trainer(pol, Tc)
-        ms_c = _time(torch, lambda: env.collect(tr, 1234), 3, warm=1) / Tc
-        out["envs"][str(n)]["collect"] = {"T": Tc, "us_per_step": round(ms_c * 1e3, 1),
-                                          "M_env_steps_per_s": round(n / ms_c / 1e3, 2)}
-        tr.close()
-        env.close()
+            ms = _time(torch, step, 64)
+            cnt, _ = env.reset_list()
+            res[mode] = {"us_per_step": round(ms * 1e3, 1), "M_env_steps_per_s": round(n / ms / 1e3, 2),
+                         "frac_fp32_peak_of_forward_flops": round(FWD_FLOP * n / (ms * 1e-3) / 1e12 / PEAK_FP32, 3),
+                         "finished_envs_last_step": cnt}
+            tr.close()
+            pol.close()
+            env.close()
+        out["envs"][str(n)] = res
     return out
 
 
@@ -457,6 +461,9 @@ def train_iteration(pkg, torch, reps):
     for n, T in ((4096, 128), (8192, 128), (65536, 64)):
         env = pkg.Env(n)
         env.init(0)
+        for _ in range(300):          # spread the episodes' phases (random actions) before timing
+            env.step(None)
+            env.reset()
         pol = pkg.Policy(n, layers=3, seed=1)
         if n <= 4096:
             pol.set_small_tiles(True)
