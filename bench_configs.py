@@ -150,6 +150,33 @@ def ppo_update(pkg, torch, reps):
                                    "tflops": UPD_FLOP * samples / ms16s / 1e9}
     assert torch.isfinite(pol.params).all()
     tr.close()
+    # ... and the r_state slab as bf16 too (cfp_train_set_bf16_rstate): written by the bf16-input
+    # forward of the rollout, so the slab is recorded again in that mode
+    pol.set_gemm_bf16(True)
+    tr = pkg.Trainer(pol, T)
+    tr.set_bf16_rstate(True)
+    pol.state.zero_()
+    for t in range(T):
+        tr.record_step(t, pkg.policy.synth_records(n, 1234, t), term)
+    tr.buf("r_act").copy_(torch.randint(0, 43, (T, n), device="cuda", generator=g, dtype=torch.int32))
+    tr.buf("r_logprob").fill_(-3.7612)
+    tr.buf("adv").copy_(torch.randn(T, n, device="cuda", generator=g))
+    tr.buf("ret").copy_(torch.randn(T, n, device="cuda", generator=g))
+    tr.buf("r_done").zero_()
+    tr.adv_stats()
+    pkg.policy.set_gemm_bf16(True)
+    tr.set_bf16_storage(True)
+    try:
+        def step16():
+            tr.backward(0, n)
+            tr.adam()
+        ms16r = _time(torch, step16, reps, warm=1)
+    finally:
+        pkg.policy.set_gemm_bf16(False)
+        pol.set_gemm_bf16(False)
+    out["bf16_in_bf16_storage_bf16_rstate"] = {"ms_per_update": ms16r, "samples_per_s": samples / ms16r * 1e3,
+                                               "tflops": UPD_FLOP * samples / ms16r / 1e9}
+    tr.close()
     pol.close()
     return out
 
@@ -469,11 +496,12 @@ def train_iteration(pkg, torch, reps):
             pol.set_small_tiles(True)
         tr = pkg.Trainer(pol, T)
         case = {}
-        for mode in ("fp32", "bf16_in_bf16_storage"):
+        for mode in ("fp32", "bf16_in_bf16_storage", "bf16_in_bf16_storage_bf16_rstate"):
             bf = mode != "fp32"
             pol.set_gemm_bf16(bf)
             tr.set_gemm_mode(1 if bf else 0, 1)
             tr.set_bf16_storage(bf)
+            tr.set_bf16_rstate(mode.endswith("rstate"))
 
             def it():
                 env.collect(tr, 1234)
@@ -482,6 +510,7 @@ def train_iteration(pkg, torch, reps):
             ms_c = _time(torch, lambda: env.collect(tr, 1234), 3, warm=1)
             case[mode] = {"ms_per_iteration": round(ms, 3), "ms_collect": round(ms_c, 3),
                           "ms_update": round(ms - ms_c, 3), "M_samples_per_s": round(n * T / ms / 1e3, 2)}
+        tr.set_bf16_rstate(False)
         pol.set_gemm_bf16(False)
         assert torch.isfinite(pol.params).all()
         out["cases"][f"{n}x{T}"] = case

@@ -309,6 +309,7 @@ void cfp::fill_forward_weights(const cfp_policy* p, FwdArgs& a) {
     a.wg_bf = reinterpret_cast<const u4*>(p->wg_bf);
     a.wav_bf = reinterpret_cast<const u4*>(p->wav_bf);
     a.bf16 = p->gemm_bf16;
+    a.rs_bf16 = p->rs_bf16;   // (the window recompute sets its own)
     if (p->small_tiles && p->t16)
         t16_mirror_layout(p->t16, p->layers, &a.t16_enc_s, &a.t16_enc_t, &a.t16_wg, &a.t16_wav);
 }

@@ -112,6 +112,8 @@ struct FwdArgs {
     float* state;            // [layers][state_envs][256] in/out, or null
     const float* terminals;  // [n] or null (= no terminal)
     float* r_state;          // like state, or null
+    int rs_bf16;             // bf16-input kernel only: r_state (written) and, in the window
+                             // recompute, the stored state (read) are bf16 arrays of the same shape
     float* h_enc_out;        // [n][256] or null
     float* h3_out;           // [n][256] or null
     float* av_out;           // [n][44] or null

@@ -17,6 +17,7 @@ struct cfp_policy {
     uint16_t* wg_bf = nullptr;
     uint16_t* wav_bf = nullptr;
     int gemm_bf16 = 0;            // forward entry points run the bf16-input kernel
+    int rs_bf16 = 0;              // r_state rows leave as bf16 (a trainer with a bf16 state slab)
     void* enc_x9 = nullptr;       // split mirror of W_enc for the forward from a feature matrix
     void* t16 = nullptr;          // mirrors of the 16-env-tile kernel (full game only)
     int small_tiles = 0;          // batches of at most 4096 envs run on 16-env tiles

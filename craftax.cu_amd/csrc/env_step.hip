@@ -35,7 +35,6 @@ using namespace cfenv;
 constexpr int kWave = 64;
 constexpr size_t kPlaneBytes = (size_t)kMap * kMap;                 // 2304
 constexpr size_t kEnvPlaneBytes = 3 * (size_t)kLevels * kPlaneBytes;  // 62 208
-constexpr int kRows = kLevels * kMap;                                // 432 bitmap rows per env
 constexpr int kMobSlots = CFP_ENV_MOB_CLASSES * kLevels * 3;         // 135
 
 // ---- field registry ------------------------------------------------------------------------

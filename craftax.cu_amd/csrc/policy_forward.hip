@@ -795,6 +795,9 @@ int launch_forward(const FwdArgs& a, hipStream_t st) {
     CFP_REQUIRE(!a.tr_bf16 || (a.bf16 && a.train),
                 "bf16 storage of the window recompute needs the bf16-input kernel");
     if (a.bf16) return launch_forward_bf16(a, st);
+    CFP_REQUIRE(!(a.rs_bf16 && (a.r_state || a.train)),
+                "a bf16 state slab is written and read by the bf16-input forward only "
+                "(cfp_policy_set_gemm_bf16 / cfp_set_gemm_bf16)");
     if (forward_t16_ok(a)) return launch_forward_t16(a, st);
     // persistent: one workgroup per CU, each walking tile pairs round-robin; a full-game
     // batch of at most one tile per CU runs one tile per workgroup instead

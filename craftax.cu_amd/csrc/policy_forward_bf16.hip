@@ -65,7 +65,9 @@ __device__ __forceinline__ void copy_tile_out_bf16(const float* lds, uint16_t* d
         d2[i] = __builtin_bit_cast(u2_t, __builtin_convertvector(xs4[(i >> 6) * XS4 + (i & 63)], bf16x4_t));
 }
 
-template <int VARIANT, bool HAS_RS, bool TRAIN, bool TR16 = false>
+// RS16: the recorded state is a bf16 slab -- written as bf16 by the rollout (HAS_RS), read as
+// bf16 by the window recompute (TRAIN).
+template <int VARIANT, bool HAS_RS, bool TRAIN, bool TR16 = false, bool RS16 = false>
 __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs a) {
     __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
     __shared__ float term_s[kTileEnvs];
@@ -103,14 +105,21 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
     u4 bq[kGateAhead + 1][6];
     auto state_fetch = [&](const float* base, float (&v)[32]) {
 #pragma unroll
-        for (int e = 0; e < 32; e++)
-            v[e] = __builtin_nontemporal_load(
-                (base + (acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32)) + loff);
+        for (int e = 0; e < 32; e++) {
+            const int off = acc_row(e % 16) * CFP_HIDDEN + (e / 16) * 32;
+            if (TRAIN && RS16)
+                v[e] = (float)__builtin_nontemporal_load((reinterpret_cast<const __bf16*>(base) + off) + loff);
+            else
+                v[e] = __builtin_nontemporal_load((base + off) + loff);
+        }
     };
     auto state_base = [&](int l) -> float* {
         if (TRAIN) {
             const size_t tt = se / a.tr_n_all, ee = se - tt * a.tr_n_all;
-            return a.state + ((tt * a.layers + l) * a.tr_n_all + ee) * CFP_HIDDEN + wave * 64;
+            const size_t el = ((tt * a.layers + l) * a.tr_n_all + ee) * CFP_HIDDEN + wave * 64;
+            // a bf16 slab: the same element index in 2-byte elements (state_fetch casts back)
+            if (RS16) return reinterpret_cast<float*>(reinterpret_cast<__bf16*>(a.state) + el);
+            return a.state + el;
         }
         return a.state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64;
     };
@@ -302,6 +311,9 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
         if (l + 1 < a.layers) state_fetch(state_base(l + 1), stn);
         float* rs_base = HAS_RS ? a.r_state + (size_t)l * a.layer_stride + e0 * CFP_HIDDEN + wave * 64
                                 : nullptr;
+        __bf16* rs16 = (HAS_RS && RS16) ? reinterpret_cast<__bf16*>(a.r_state) + (size_t)l * a.layer_stride +
+                                              e0 * CFP_HIDDEN + wave * 64
+                                        : nullptr;
         float* out_base = TRAIN ? a.tr_x[l + 1] + e0 * CFP_HIDDEN + wave * 64 : nullptr;
         float* pre_base = TRAIN ? a.tr_pre[l] + e0 * CFP_GRU + wave * 64 : nullptr;
         __bf16* out16 = TR16 ? reinterpret_cast<__bf16*>(a.tr_x[l + 1]) + e0 * CFP_HIDDEN + wave * 64 : nullptr;
@@ -312,7 +324,8 @@ __global__ __launch_bounds__(kFwdThreads, 2) void k_policy_forward_bf16(FwdArgs 
             const int soff = acc_row(r) * CFP_HIDDEN + ut * 32;
             float* xp = lds + (acc_row(r) + 4 * g) * XS + wave * 64 + ut * 32 + l32;
             const float s = (!TRAIN && ((tmask >> r) & 1u)) ? 0.0f : st[e];
-            if (HAS_RS) __builtin_nontemporal_store(s, (rs_base + soff) + loff);
+            if (HAS_RS && RS16) __builtin_nontemporal_store((__bf16)s, (rs16 + soff) + loff);
+            else if (HAS_RS) __builtin_nontemporal_store(s, (rs_base + soff) + loff);
             const float zh = acc[0 + ut][r];
             const float zg = acc[2 + ut][r];
             const float zp = acc[4 + ut][r];
@@ -381,13 +394,19 @@ int launch_forward_bf16(const FwdArgs& a, hipStream_t st) {
                         !a.terminals && a.tr_mb > 0 && a.tr_mb % kTileEnvs == 0 &&
                         a.h_enc_out == a.tr_x[0],
                     "window recompute: bad arguments");
-        if (a.tr_bf16) hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true, true>), g, b, 0, st, a);
+        CFP_REQUIRE(!a.rs_bf16 || a.tr_bf16, "a bf16 state slab goes with the bf16 storage of the window");
+        if (a.tr_bf16 && a.rs_bf16)
+            hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true, true, true>), g, b, 0, st, a);
+        else if (a.tr_bf16) hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true, true>), g, b, 0, st, a);
         else hipLaunchKernelGGL((k_policy_forward_bf16<0, false, true>), g, b, 0, st, a);
     } else if (a.variant == 1) {
+        CFP_REQUIRE(!(a.rs_bf16 && a.r_state), "the classic policy has no bf16 state slab");
         if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<1, true, false>), g, b, 0, st, a);
         else hipLaunchKernelGGL((k_policy_forward_bf16<1, false, false>), g, b, 0, st, a);
     } else {
-        if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<0, true, false>), g, b, 0, st, a);
+        if (a.r_state && a.rs_bf16)
+            hipLaunchKernelGGL((k_policy_forward_bf16<0, true, false, false, true>), g, b, 0, st, a);
+        else if (a.r_state) hipLaunchKernelGGL((k_policy_forward_bf16<0, true, false>), g, b, 0, st, a);
         else hipLaunchKernelGGL((k_policy_forward_bf16<0, false, false>), g, b, 0, st, a);
     }
     CFP_HIP_TRY(hipGetLastError());

@@ -30,7 +30,8 @@ struct ReverseArgs {
     int layer, layers;
     int horizon, seg;          // rollout length, BPTT segment length
     int gates_bf16;            // gates, layer_in, grad_a/b and highway_out are bf16 arrays (the
-                               // update's bf16 storage); slab_state and carry stay fp32
+                               // update's bf16 storage); carry stays fp32
+    int state_bf16;            // slab_state is a bf16 array of the same shape (with gates_bf16 only)
 };
 int launch_gru_reverse(const ReverseArgs& a, hipStream_t st);
 

@@ -50,21 +50,27 @@ __device__ __forceinline__ double wave_sum(double v) {
 // operations are outstanding".  Three register sets rotate through a loop unrolled by
 // three (a set is never copied: a copy would read registers whose loads are in flight).
 // G16: the gate rows, the layer input, the incoming gradients and the highway term are
-// stored as bf16 (8 bytes per lane and row); the recorded state stays fp32.
+// stored as bf16 (8 bytes per lane and row); the recorded state stays fp32 unless G16 = 2.
 typedef unsigned int u2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
-template <bool G16>
+// G16 = 2: the recorded state is a bf16 slab as well (cfp_train_set_bf16_rstate).
+template <int G16>
 struct StepIn;
 template <>
-struct StepIn<false> {
+struct StepIn<0> {
     f4 zh, zg, zp, x, ga, gb, s;
     unsigned done;
 };
 template <>
-struct StepIn<true> {
+struct StepIn<1> {
     u2 zh, zg, zp, x, ga, gb;
     f4 s;
+    unsigned done;
+};
+template <>
+struct StepIn<2> {
+    u2 zh, zg, zp, x, ga, gb, s;
     unsigned done;
 };
 
@@ -78,12 +84,40 @@ __device__ __forceinline__ u2 narrow(const f4& v) {   // round to nearest even
 }
 
 // lo: byte offset of the lane inside an fp32 row (16 q), lo8: inside a bf16 row (8 q)
-template <bool TWO_GRADS, bool G16>
+template <bool TWO_GRADS, int G16>
 __device__ __forceinline__ void sweep_fetch(StepIn<G16>& r, unsigned lo, unsigned lo8,
                                             const void* gates, const void* ga, const void* gb,
-                                            const f4* state, const void* xin, const uint8_t* done) {
+                                            const void* state, const void* xin, const uint8_t* done) {
     const unsigned zero = 0u;
-    if (G16 && TWO_GRADS)
+    if (G16 == 2 && TWO_GRADS)
+        asm volatile(
+            "global_load_dwordx2 %0, %9, %11 nt\n\t"
+            "global_load_dwordx2 %1, %9, %11 offset:512 nt\n\t"
+            "global_load_dwordx2 %2, %9, %11 offset:1024 nt\n\t"
+            "global_load_dwordx2 %3, %9, %12 nt\n\t"
+            "global_load_dwordx2 %4, %9, %13 nt\n\t"
+            "global_load_dwordx2 %5, %9, %14 nt\n\t"
+            "global_load_dwordx2 %6, %9, %15 nt\n\t"
+            "global_load_ubyte %7, %10, %16"
+            : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.gb), "=&v"(r.s),
+              "=&v"(r.x), "=&v"(r.done)
+            : "v"(lo), "v"(lo8), "v"(zero), "s"(gates), "s"(ga), "s"(gb), "s"(state), "s"(xin),
+              "s"(done)
+            : "memory");
+    else if (G16 == 2)
+        asm volatile(
+            "global_load_dwordx2 %0, %8, %10 nt\n\t"
+            "global_load_dwordx2 %1, %8, %10 offset:512 nt\n\t"
+            "global_load_dwordx2 %2, %8, %10 offset:1024 nt\n\t"
+            "global_load_dwordx2 %3, %8, %11 nt\n\t"
+            "global_load_dwordx2 %4, %8, %12 nt\n\t"
+            "global_load_dwordx2 %5, %8, %13 nt\n\t"
+            "global_load_ubyte %6, %9, %14"
+            : "=&v"(r.zh), "=&v"(r.zg), "=&v"(r.zp), "=&v"(r.ga), "=&v"(r.s), "=&v"(r.x),
+              "=&v"(r.done)
+            : "v"(lo), "v"(lo8), "v"(zero), "s"(gates), "s"(ga), "s"(state), "s"(xin), "s"(done)
+            : "memory");
+    else if (G16 && TWO_GRADS)
         asm volatile(
             "global_load_dwordx2 %0, %9, %11 nt\n\t"
             "global_load_dwordx2 %1, %9, %11 offset:512 nt\n\t"
@@ -142,7 +176,7 @@ __device__ __forceinline__ void sweep_fetch(StepIn<G16>& r, unsigned lo, unsigne
 
 // Every later use of the set depends on this statement's outputs, so none can be moved
 // in front of the wait.
-template <int N, bool TWO_GRADS, bool G16>
+template <int N, bool TWO_GRADS, int G16>
 __device__ __forceinline__ void sweep_wait(StepIn<G16>& r) {
     if (TWO_GRADS)
         asm volatile("s_waitcnt vmcnt(%8)"
@@ -157,7 +191,7 @@ __device__ __forceinline__ void sweep_wait(StepIn<G16>& r) {
 }
 
 // Drain the queue; every set is an output, so nothing of any set is read before it.
-template <bool TWO_GRADS, bool G16>
+template <bool TWO_GRADS, int G16>
 __device__ __forceinline__ void sweep_drain(StepIn<G16>& p, StepIn<G16>& q, StepIn<G16>& r) {
     if (TWO_GRADS)
         asm volatile("s_waitcnt vmcnt(0)"
@@ -224,7 +258,7 @@ __device__ __forceinline__ void sweep_store(unsigned, unsigned lo8, void* gates,
 }
 
 constexpr int kSweepEnvs = 1;   // envs (wavefronts) per workgroup: the best of 1 / 2 / 4
-template <bool TWO_GRADS, bool HIGHWAY, bool G16>
+template <bool TWO_GRADS, bool HIGHWAY, int G16>
 __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
     const int env = (int)blockIdx.x * kSweepEnvs + wave;   // one wavefront per env of the minibatch
@@ -240,9 +274,11 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
         TWO_GRADS ? reinterpret_cast<const char*>(a.grad_b) + (size_t)env * kInRow : nullptr;
     char* const hw = HIGHWAY ? reinterpret_cast<char*>(a.highway_out) + (size_t)env * kInRow : nullptr;
     const size_t slab_env = (size_t)a.w.env_start + env;
-    const size_t state_step = (size_t)a.layers * a.w.n_all * H4;
-    const f4* const state = reinterpret_cast<const f4*>(a.slab_state) +
-                            (((size_t)a.w.t0 * a.layers + a.layer) * a.w.n_all + slab_env) * H4;
+    // the recorded state: rows of 256 fp32, or of 256 bf16 (G16 = 2); a step back is one stride
+    constexpr size_t kStateRow = G16 == 2 ? H * 2 : H * 4;   // bytes
+    const size_t state_step = (size_t)a.layers * a.w.n_all * kStateRow;
+    const char* const state = reinterpret_cast<const char*>(a.slab_state) +
+                              (((size_t)a.w.t0 * a.layers + a.layer) * a.w.n_all + slab_env) * kStateRow;
     const uint8_t* const done = a.slab_done + (size_t)a.w.t0 * a.w.n_all + slab_env;
     // Every stage fetches, so that the number of operations in flight is the same at
     // every wait; a stage with no step left to fetch reads rows of the carry array
@@ -257,7 +293,7 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
             r, lane_off, lane_off8, real ? (const void*)(gates + c * kGateRow) : (const void*)idle,
             real ? (const void*)(ga + c * kInRow) : (const void*)idle,
             TWO_GRADS ? (real ? (const void*)(gb + c * kInRow) : (const void*)idle) : nullptr,
-            real ? state + (size_t)s * state_step : idle,
+            real ? (const void*)(state + (size_t)s * state_step) : (const void*)idle,
             real ? (const void*)(xin + c * kInRow) : (const void*)idle,
             done + (size_t)(real ? s : 0) * a.w.n_all);
     };
@@ -274,6 +310,7 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
         phase = (phase == 0 ? a.seg : phase) - 1;
         const float pass = (in.done & 0xffu) ? 0.0f : 1.0f;   // a terminal step hands nothing back
         const f4 zh = widen(in.zh), zg = widen(in.zg), zp = widen(in.zp), x = widen(in.x);
+        const f4 sv = widen(in.s);
         const f4 ga_v = widen(in.ga);
         f4 gb_v = f4{0.0f, 0.0f, 0.0f, 0.0f};
         if constexpr (TWO_GRADS) gb_v = widen(in.gb);
@@ -286,8 +323,8 @@ __global__ __launch_bounds__(64 * kSweepEnvs, 4) void k_gru_reverse(ReverseArgs 
             const bool lin = zh[j] >= 0.0f;
             const float cand = lin ? zh[j] + 0.5f : sh;              // g(zh)
             const float dcand = lin ? 1.0f : sh * (1.0f - sh);       // g'(zh)
-            const float gap = cand - in.s[j];
-            const float h_new = in.s[j] + sg * gap;
+            const float gap = cand - sv[j];
+            const float h_new = sv[j] + sg * gap;
             const float g_top = TWO_GRADS ? ga_v[j] + gb_v[j] : ga_v[j];
             const float g_h = g_top * mix + pass * carry[j];
             dzp[j] = g_top * (h_new - x[j]) * mix * (1.0f - mix);
@@ -726,8 +763,10 @@ int launch_gru_reverse(const ReverseArgs& a, hipStream_t st) {
             hipLaunchKernelGGL((k_gru_reverse<false, true, G16>), grid, blk, 0, st, a);               \
         else hipLaunchKernelGGL((k_gru_reverse<false, false, G16>), grid, blk, 0, st, a);             \
     } while (0)
-    if (a.gates_bf16) CFP_SWEEP_LAUNCH(true);
-    else CFP_SWEEP_LAUNCH(false);
+    CFP_REQUIRE(!a.state_bf16 || a.gates_bf16, "a bf16 state slab goes with the bf16 storage of the window");
+    if (a.gates_bf16 && a.state_bf16) CFP_SWEEP_LAUNCH(2);
+    else if (a.gates_bf16) CFP_SWEEP_LAUNCH(1);
+    else CFP_SWEEP_LAUNCH(0);
 #undef CFP_SWEEP_LAUNCH
     CFP_HIP_TRY(hipGetLastError());
     return 0;

@@ -174,6 +174,9 @@ struct cfp_trainer {
     // bf16 storage of the window's gate pre-activations / their gradients and of the
     // layer inputs (in effect with bf16 GEMM inputs on the split kernels only)
     int bf16_store = 0;
+    // the r_state slab holds bf16 (cfp_train_set_bf16_rstate): written by the bf16-input forward
+    // of the rollout, read by the bf16 window recompute and the bf16-storage sweep
+    int rs16 = 0;
     // GEMM mode of this trainer's update (cfp_train_set_gemm_mode); -1: the process-wide switch
     int gemm_bf16 = -1, gemm_split = -1;
     hipStream_t st_own = nullptr;   // capture stream when the caller passes the null stream
@@ -185,6 +188,7 @@ extern "C" {
 
 void cfp_train_destroy(cfp_trainer* tr) {
     if (!tr) return;
+    if (tr->rs16 && tr->p) tr->p->rs_bf16 = 0;   // the policy no longer writes rows of a bf16 slab
     for (void* q : tr->owned) (void)hipFree(q);
     seam_work_destroy(&tr->sw);
     for (hipEvent_t e : tr->ev_dh)
@@ -336,6 +340,14 @@ int cfp_train_set_bf16_storage(cfp_trainer* tr, int on) {
 }
 int cfp_train_bf16_storage(const cfp_trainer* tr) { return tr ? tr->bf16_store : -1; }
 
+int cfp_train_set_bf16_rstate(cfp_trainer* tr, int on) {
+    CFP_REQUIRE(tr, "cfp_train_set_bf16_rstate: NULL trainer");
+    tr->rs16 = on ? 1 : 0;
+    tr->p->rs_bf16 = tr->rs16;   // the policy's forward writes the rows of this trainer's slab
+    return 0;
+}
+int cfp_train_bf16_rstate(const cfp_trainer* tr) { return tr ? tr->rs16 : -1; }
+
 int cfp_train_set_gemm_mode(cfp_trainer* tr, int bf16, int split) {
     CFP_REQUIRE(tr, "cfp_train_set_gemm_mode: NULL trainer");
     CFP_REQUIRE(bf16 >= -1 && bf16 <= 1 && split >= -1 && split <= 2,
@@ -354,18 +366,23 @@ int cfp_train_gemm_mode(const cfp_trainer* tr, int* bf16, int* split) {
 int cfp_train_window(const cfp_trainer* tr) { return tr ? tr->win : 0; }
 int cfp_train_minibatch(const cfp_trainer* tr) { return tr ? tr->mb : 0; }
 
+// r_state rows of step t: [layers][n][256] fp32, or bf16 in a slab of 2-byte elements
+static float* state_rows(cfp_trainer* tr, int t) {
+    const size_t el = (size_t)t * tr->L * tr->n * H;
+    return tr->rs16 ? reinterpret_cast<float*>(reinterpret_cast<uint16_t*>(tr->r_state) + el) : tr->r_state + el;
+}
+
 int cfp_train_record_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
                           const float* d_terminals, void* stream) {
     CFP_REQUIRE(tr && d_rec_row, "cfp_train_record_step: NULL argument");
     CFP_REQUIRE(t >= 0 && t < tr->T, "step %d outside the horizon %d", t, tr->T);
     hipStream_t st = (hipStream_t)stream;
-    const size_t n = tr->n, hn = (size_t)H * n;
+    const size_t n = tr->n;
     uint8_t* row = tr->r_obs + (size_t)t * n * CFP_REC_BYTES;
     if (d_rec_row != row)
         CFP_HIP_TRY(hipMemcpyAsync(row, d_rec_row, n * CFP_REC_BYTES,
                                    hipMemcpyDeviceToDevice, st));
-    if (cfp_policy_forward(tr->p, row, d_terminals, nullptr,
-                           tr->r_state + (size_t)t * tr->L * hn, nullptr, nullptr,
+    if (cfp_policy_forward(tr->p, row, d_terminals, nullptr, state_rows(tr, t), nullptr, nullptr,
                            nullptr, tr->n, 0, stream) != 0)
         return 1;
     hipLaunchKernelGGL(k_take_value, dim3(grid1(n)), dim3(256), 0, st, tr->p->logits,
@@ -388,8 +405,7 @@ int cfp_rollout_step(cfp_trainer* tr, int t, const uint8_t* d_rec_row,
     const SampleOut so{tr->r_act + o,  tr->r_logprob + o, tr->r_value + o, d_env_actions,
                        seed,           tr->step_ctr,      tr->ticket};
     (void)hn;
-    return forward_and_sample(tr->p, row, d_prev_terminals, tr->r_state + o * tr->L * H, tr->n, so,
-                              st);
+    return forward_and_sample(tr->p, row, d_prev_terminals, state_rows(tr, t), tr->n, so, st);
 }
 
 int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void* stream) {
@@ -516,6 +532,9 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         // storage
         const bool st16 = tr->bf16_store && gemm_mode_bf16() != 0 && gemm_mode_split() != 0 &&
                           dw_enc_records_ok(mb) && cols % 32 == 0;
+        CFP_REQUIRE(!tr->rs16 || st16,
+                    "a bf16 state slab needs the update in its bf16 mode: bf16 GEMM inputs, the split "
+                    "kernels, bf16 storage, and a window of whole 32-column blocks");
         if (fused) {
             FwdArgs fa{};
             fill_forward_weights(p, fa);
@@ -529,6 +548,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             fa.do_head = 1;
             fa.train = 1;
             fa.tr_bf16 = st16 ? 1 : 0;
+            fa.rs_bf16 = tr->rs16;
             fa.tr_t0 = t0; fa.tr_mb = mb; fa.tr_n_all = n; fa.tr_env_start = env_start;
             for (int l = 0; l < L; l++) fa.tr_pre[l] = tr->preb[l];
             for (int l = 0; l <= L; l++) fa.tr_x[l] = tr->x[l];
@@ -617,6 +637,7 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             ra.slab_state = tr->r_state; ra.slab_done = tr->r_done; ra.carry = tr->dcarry[l];
             ra.w = wm; ra.steps = Tw; ra.layer = l; ra.layers = L; ra.horizon = T; ra.seg = seg;
             ra.gates_bf16 = st16 ? 1 : 0;
+            ra.state_bf16 = tr->rs16;
             if (launch_gru_reverse(ra, chain)) return 1;
             if (!overlap &&
                 gemm_dw_ld(G, cols, tr->x[l], tr->preb[l], G, g + CFP_OFF_W_GRU + (size_t)l * G * H,
@@ -718,7 +739,7 @@ int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
               bf = tr->gemm_bf16 >= 0 ? tr->gemm_bf16 : cfp_get_gemm_bf16(),
               pbf = cfp_policy_gemm_bf16(tr->p);
     if (tr->texec && (split != tr->graph_split || bf != tr->graph_bf16 ||
-                      pbf != tr->graph_pol_bf16 || tr->bf16_store != tr->graph_store16)) {
+                      pbf != tr->graph_pol_bf16 || tr->bf16_store + 2 * tr->rs16 != tr->graph_store16)) {
         (void)hipGraphExecDestroy(tr->texec);
         (void)hipGraphDestroy(tr->tgraph);
         tr->texec = nullptr;
@@ -749,7 +770,7 @@ int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
         tr->graph_split = split;
         tr->graph_bf16 = bf;
         tr->graph_pol_bf16 = pbf;
-        tr->graph_store16 = tr->bf16_store;
+        tr->graph_store16 = tr->bf16_store + 2 * tr->rs16;
     }
     CFP_HIP_TRY(hipGraphLaunch(tr->texec, st));
     CFP_HIP_TRY(hipStreamSynchronize(st));
@@ -758,6 +779,7 @@ int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
 
 int cfp_train_loss(cfp_trainer* tr, double* host_loss4, void* stream) {
     CFP_REQUIRE(tr && host_loss4, "cfp_train_loss: NULL argument");
+    CFP_REQUIRE(!tr->rs16, "cfp_train_loss replays from an fp32 state slab (cfp_train_set_bf16_rstate is on)");
     hipStream_t st = (hipStream_t)stream;
     const int T = tr->T, n = tr->n, L = tr->L;
     const int seg = T / tr->cfg.bptt_split;

@@ -268,6 +268,10 @@ class Trainer:
         """bf16 storage of the window workspace (in effect with bf16 GEMM inputs only)."""
         _check(lib().cfp_train_set_bf16_storage(self._h, 1 if on else 0))
 
+    def set_bf16_rstate(self, on=True):
+        """The r_state slab as bf16 (cfp_train_set_bf16_rstate): bf16 forward and bf16 update only."""
+        _check(lib().cfp_train_set_bf16_rstate(self._h, 1 if on else 0))
+
     def set_gemm_mode(self, bf16=-1, split=-1):
         """This trainer's own GEMM mode (cfp_train_set_gemm_mode); -1 follows the process-wide switch."""
         _check(lib().cfp_train_set_gemm_mode(self._h, int(bf16), int(split)))

@@ -449,6 +449,20 @@ void* cfp_train_buffer(cfp_trainer* tr, int which);
 int cfp_train_set_bf16_storage(cfp_trainer* tr, int on);
 int cfp_train_bf16_storage(const cfp_trainer* tr);
 
+/* bf16 r_state slab, the rest of the reference's CF_GEMM_BF16 storage
+ * (craftax_full.cu:12694-12700, read paths :9470-9480, :9538-9590): the rollout's forward
+ * writes the post-zero state rows as bf16 and the update's window recompute and reverse sweep
+ * read them as bf16 -- half of the 805 MB the recompute reads at 262 144 columns and 2 of the
+ * sweep's bytes per element.  The slab keeps its shape [T][layers][n][256] and its buffer
+ * (CFP_BUF_R_STATE then holds bf16 elements in the first half of the allocation).  Both ends
+ * exist on the bf16 path only: set it before the rollout writes the slab, on a policy with
+ * cfp_policy_set_gemm_bf16(1); cfp_train_backward then requires the bf16 update mode
+ * (bf16 GEMM inputs, split kernels, cfp_train_set_bf16_storage(1)) and fails with a clear
+ * error otherwise, as does a forward on the fp32 kernels that is asked to write r_state.
+ * The live state stays fp32.  Off by default. */
+int cfp_train_set_bf16_rstate(cfp_trainer* tr, int on);
+int cfp_train_bf16_rstate(const cfp_trainer* tr);
+
 /* GEMM mode of one trainer's update.  The reference has one process-wide switch
  * (g_gemm_bf16, craftax_full.cu:11306-11316) and one trainer per process; here two trainers
  * may live in one process, each with a captured update graph, so a trainer can carry its own

@@ -449,6 +449,93 @@ def test_two_trainers_with_their_own_gemm_modes(pkg, cuda):
             tr.close(); pol.close()
 
 
+@pytest.mark.parametrize("seed,layers", [(500, 3), (501, 2), (502, 1), (503, 3)])
+def test_bf16_state_slab(pkg, cuda, seed, layers):
+    """cfp_train_set_bf16_rstate: the rollout's bf16-input forward writes the post-zero state
+    rows as bf16 and the bf16 update reads them as bf16.  (a) the slab is, bit for bit, the
+    fp32 slab of a twin trainer rounded to bf16 (nearest even), and the live state and head
+    rows do not change; (b) every gradient segment of the update is within 1e-3 (relative
+    Frobenius norm) of the bf16-operand fp64 update evaluated on that slab, and the update
+    reproduces bit for bit; (c) the two ends that exist on the bf16 path only refuse the others
+    with an error: an fp32 forward asked to write the slab, a backward outside the bf16 mode."""
+    import torch
+    from parity_util import TOL_BF16_OPS, bf16_round, fro_err, expand_records
+    n, T = 64, 8
+    for k in range(16):          # a batch off the candidate function's kink (see _collect_off_the_kink)
+        params = random_params(layers, seed + 1000 * k, scale=0.3)
+        pols = [pkg.Policy(n, layers, seed=1) for _ in range(2)]
+        trs = []
+        for i, pol in enumerate(pols):
+            pol.set_params(params)
+            pol.set_gemm_bf16(True)
+            tr = pkg.Trainer(pol, T)
+            if i == 1:
+                tr.set_bf16_rstate(True)
+            trs.append(tr)
+        rng = np.random.default_rng(seed + 1)
+        r_done = (rng.random((T, n)) < 0.1).astype(np.uint8)
+        for pol, tr in zip(pols, trs):
+            pol.state.zero_()
+            for t in range(T):
+                rec = _t(synth_records_host(n, seed, t), cuda)
+                term = _t(r_done[t - 1].astype(np.float32) if t else np.zeros(n, np.float32), cuda)
+                tr.record_step(t, rec, term)
+        torch.cuda.synchronize()
+        slab32 = trs[0].buf("r_state").cpu().numpy()
+        raw = trs[1].buf("r_state").view(torch.bfloat16).flatten()[: slab32.size]
+        slab16 = raw.float().cpu().numpy().reshape(slab32.shape)
+        assert np.array_equal(slab16.view(np.uint32), bf16_round(slab32).astype(np.float32).view(np.uint32)), "slab rounding"
+        assert torch.equal(pols[0].state, pols[1].state) and torch.equal(trs[0].buf("r_value"), trs[1].buf("r_value"))
+        host = dict(r_act=rng.integers(0, ACTIONS, (T, n)).astype(np.int32),
+                    adv=rng.standard_normal((T, n)).astype(np.float32),
+                    ret=rng.standard_normal((T, n)).astype(np.float32), r_done=r_done)
+        host["r_obs"] = trs[1].buf("r_obs").cpu().numpy()
+        host["r_state"] = slab16
+        host["r_logprob"] = np.zeros((T, n), np.float32)
+        for t in range(T):
+            ref = ob.forward_f64(params, layers, expand_records(host["r_obs"][t]), host["r_state"][t], None)
+            z = ref["logits"] - ref["logits"].max(axis=1, keepdims=True)
+            logp = z - np.log(np.exp(z).sum(axis=1, keepdims=True))
+            host["r_logprob"][t] = (logp[np.arange(n), host["r_act"][t]] + 0.02 * rng.standard_normal(n)).astype(np.float32)
+        batch, keep = ob.make_batch(T, n, 0, n, layers, T, **host)
+        if min(ob.ppo_min_abs_zh(params, batch), ob.ppo_min_abs_zh(params, batch, bf16_ops=True)) >= KINK_MARGIN:
+            break
+        for pol, tr in zip(pols, trs):
+            tr.close(); pol.close()
+    else:
+        raise AssertionError("no batch off the kink")
+    tr, pol = trs[1], pols[1]
+    for name in ("r_act", "r_logprob", "adv", "ret", "r_done"):
+        tr.buf(name).copy_(_t(host[name], cuda))
+    tr.adv_stats()
+    g_q = ob.ppo_backward_bf16ops_f64(params, batch, bf16_storage=True)[0]
+    # (c) outside the bf16 mode the backward refuses the slab
+    with pytest.raises(pkg._lib.CfpError):
+        tr.backward(0, n)
+    pkg.policy.set_gemm_bf16(True)
+    tr.set_bf16_storage(True)
+    try:
+        outs = []
+        for _ in range(2):
+            tr.buf("grads").zero_(); tr.zero_loss()
+            tr.backward(0, n)
+            torch.cuda.synchronize()
+            outs.append(tr.buf("grads").cpu().numpy().copy())
+        assert np.array_equal(outs[0], outs[1]), "bitwise reproducible"
+        for name, sl in _segments(layers):
+            e = fro_err(outs[0][sl], g_q[sl])
+            assert e <= TOL_BF16_OPS, f"d{name} with a bf16 state slab: {e:.3e} from the bf16-operand fp64 update"
+    finally:
+        pkg.policy.set_gemm_bf16(False)
+        tr.set_bf16_storage(False)
+    # (c) the fp32 forward cannot write a bf16 slab
+    pol.set_gemm_bf16(False)
+    with pytest.raises(pkg._lib.CfpError):
+        tr.record_step(0, _t(synth_records_host(n, seed, 0), cuda), torch.zeros(n, device=cuda))
+    for pol, tr in zip(pols, trs):
+        tr.close(); pol.close()
+
+
 def test_checkpoint_roundtrip(pkg, cuda, tmp_path):
     """CFW1 file: header words, byte-exact params, mirrors refreshed on load, and the
     reference's rejections (wrong shape, truncated file)."""
