@@ -77,6 +77,8 @@ PROTOTYPES = {
     "cfp_train_bf16_storage": (C.c_int, [vp]),
     "cfp_train_set_bf16_rstate": (C.c_int, [vp, C.c_int]),
     "cfp_train_bf16_rstate": (C.c_int, [vp]),
+    "cfp_train_set_profile": (C.c_int, [vp, C.c_int]),
+    "cfp_train_profile": (C.c_int, [vp, C.POINTER(C.c_double), C.c_int]),
     "cfp_train_set_gemm_mode": (C.c_int, [vp, C.c_int, C.c_int]),
     "cfp_train_gemm_mode": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "cfp_train_window": (C.c_int, [vp]),

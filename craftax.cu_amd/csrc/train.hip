@@ -8,6 +8,7 @@
 //   :10069 into the layer-0 dh GEMM, which accumulates onto the highway term.
 // All reductions are done in a fixed order (no float atomics), so a backward pass
 // is bitwise reproducible run to run.
+#include <chrono>
 #include <vector>
 
 #include "cfp_common.h"
@@ -177,6 +178,8 @@ struct cfp_trainer {
     // the r_state slab holds bf16 (cfp_train_set_bf16_rstate): written by the bf16-input forward
     // of the rollout, read by the bf16 window recompute and the bf16-storage sweep
     int rs16 = 0;
+    int prof = 0;             // phase timers on: eager update, a sync at every phase boundary
+    double prof_ms[4] = {0.0, 0.0, 0.0, 0.0};   // rollout, gae (+ bootstrap), backward, adam
     // GEMM mode of this trainer's update (cfp_train_set_gemm_mode); -1: the process-wide switch
     int gemm_bf16 = -1, gemm_split = -1;
     hipStream_t st_own = nullptr;   // capture stream when the caller passes the null stream
@@ -348,6 +351,21 @@ int cfp_train_set_bf16_rstate(cfp_trainer* tr, int on) {
 }
 int cfp_train_bf16_rstate(const cfp_trainer* tr) { return tr ? tr->rs16 : -1; }
 
+int cfp_train_set_profile(cfp_trainer* tr, int on) {
+    CFP_REQUIRE(tr, "cfp_train_set_profile: NULL trainer");
+    tr->prof = on ? 1 : 0;
+    return 0;
+}
+
+int cfp_train_profile(cfp_trainer* tr, double* ms4, int reset) {
+    CFP_REQUIRE(tr && ms4, "cfp_train_profile: NULL argument");
+    for (int i = 0; i < 4; i++) {
+        ms4[i] = tr->prof_ms[i];
+        if (reset) tr->prof_ms[i] = 0.0;
+    }
+    return 0;
+}
+
 int cfp_train_set_gemm_mode(cfp_trainer* tr, int bf16, int split) {
     CFP_REQUIRE(tr, "cfp_train_set_gemm_mode: NULL trainer");
     CFP_REQUIRE(bf16 >= -1 && bf16 <= 1 && split >= -1 && split <= 2,
@@ -422,6 +440,18 @@ int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void
     return cfp_env_pool_size(e) > 0 ? cfp_env_reset_from_pool(e, stream) : cfp_env_reset(e, stream);
 }
 
+// cu_prof_mark (craftax_full.cu:12973-12980): with the timers on, the work queued so far is
+// waited for and the host clock read; off, nothing happens.  A failed wait reads as -1.
+static double prof_mark(cfp_trainer* tr, void* stream) {
+    if (!tr->prof) return 0.0;
+    if (hipStreamSynchronize((hipStream_t)stream) != hipSuccess) return -1.0;
+    using clk = std::chrono::steady_clock;
+    return std::chrono::duration<double, std::milli>(clk::now().time_since_epoch()).count();
+}
+static void prof_add(cfp_trainer* tr, int phase, double t0, double t1) {
+    if (tr->prof && t0 >= 0.0 && t1 >= 0.0) tr->prof_ms[phase] += t1 - t0;
+}
+
 // The reference overlaps the regeneration of finished envs (side stream, then a list-form
 // record) with the recording of the others (cu_encode_step, craftax_full.cu:11931-11955).
 // Measured here at 65 536 envs that costs time: next to the record kernel's 2048 workgroups
@@ -429,11 +459,16 @@ int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void
 // 80 us, so the steps run in sequence.
 int cfp_train_collect(cfp_trainer* tr, cfp_env* e, uint64_t seed, void* stream) {
     CFP_REQUIRE(tr && e, "cfp_train_collect: NULL argument");
+    const double t0 = prof_mark(tr, stream);
     for (int t = 0; t < tr->T; t++)
         if (cfp_env_rollout_step(tr, e, t, seed, stream)) return 1;
+    const double t1 = prof_mark(tr, stream);
     if (cfp_env_record_obs(e, tr->p->rec, stream)) return 1;
     if (cfp_train_bootstrap(tr, tr->p->rec, cfp_env_terminals(e), stream)) return 1;
-    return cfp_train_gae(tr, stream);
+    if (cfp_train_gae(tr, stream)) return 1;
+    prof_add(tr, 0, t0, t1);
+    prof_add(tr, 1, t1, prof_mark(tr, stream));
+    return 0;
 }
 
 int cfp_train_bootstrap(cfp_trainer* tr, const uint8_t* d_rec_row, const float* d_terminals,
@@ -714,8 +749,12 @@ static int train_body(cfp_trainer* tr, void* stream) {
     for (int e = 0; e < tr->cfg.epochs; e++) {
         int rc = cfp_train_zero_loss(tr, stream);
         for (int m = 0; m < tr->cfg.minibatches && rc == 0; m++) {
+            const double t0 = prof_mark(tr, stream);
             rc = cfp_train_backward(tr, m * tr->mb, tr->mb, stream);
+            const double t1 = prof_mark(tr, stream);
             if (rc == 0) rc = cfp_train_adam(tr, stream);
+            prof_add(tr, 2, t0, t1);
+            prof_add(tr, 3, t1, prof_mark(tr, stream));
         }
         if (rc != 0) return rc;
     }
@@ -725,7 +764,7 @@ static int train_body(cfp_trainer* tr, void* stream) {
 int cfp_train_update(cfp_trainer* tr, int use_graph, void* stream) {
     CFP_REQUIRE(tr, "cfp_train_update: NULL trainer");
     hipStream_t st = (hipStream_t)stream;
-    if (!use_graph) {
+    if (!use_graph || tr->prof) {   // the timers wait between the phases, which a capture cannot
         const int rc = train_body(tr, st);
         if (rc != 0) return rc;
         CFP_HIP_TRY(hipStreamSynchronize(st));

@@ -272,6 +272,16 @@ class Trainer:
         """The r_state slab as bf16 (cfp_train_set_bf16_rstate): bf16 forward and bf16 update only."""
         _check(lib().cfp_train_set_bf16_rstate(self._h, 1 if on else 0))
 
+    def set_profile(self, on=True):
+        """Phase timers of collect / update (cfp_train_set_profile); the update then runs eagerly."""
+        _check(lib().cfp_train_set_profile(self._h, 1 if on else 0))
+
+    def profile(self, reset=False):
+        """Accumulated milliseconds per phase: rollout, gae, backward, adam."""
+        ms = (C.c_double * 4)()
+        _check(lib().cfp_train_profile(self._h, ms, 1 if reset else 0))
+        return dict(zip(("rollout", "gae", "backward", "adam"), (float(x) for x in ms)))
+
     def set_gemm_mode(self, bf16=-1, split=-1):
         """This trainer's own GEMM mode (cfp_train_set_gemm_mode); -1 follows the process-wide switch."""
         _check(lib().cfp_train_set_gemm_mode(self._h, int(bf16), int(split)))

@@ -463,6 +463,17 @@ int cfp_train_bf16_storage(const cfp_trainer* tr);
 int cfp_train_set_bf16_rstate(cfp_trainer* tr, int on);
 int cfp_train_bf16_rstate(const cfp_trainer* tr);
 
+/* Phase timers of the training loop, the counterpart of CRAFTAX_CU_TRAIN_PROF
+ * (craftax_full.cu:12925-12926, cu_prof_mark :12973-12980, read out at :13374 and :13659):
+ * with the timers on, cfp_train_collect and cfp_train_update wait for the stream at every
+ * phase boundary and add the host-clock time of each phase to four sums -- rollout (the T
+ * steps of cfp_env_rollout_step), gae (last record, bootstrap value, advantages), backward,
+ * adam -- and cfp_train_update runs eagerly whatever use_graph says, as the reference's does.
+ * cfp_train_profile copies the sums (milliseconds) to host memory and, with reset != 0,
+ * clears them.  Off by default; the waits cost throughput, so this is a diagnosis aid. */
+int cfp_train_set_profile(cfp_trainer* tr, int on);
+int cfp_train_profile(cfp_trainer* tr, double* ms4, int reset);
+
 /* GEMM mode of one trainer's update.  The reference has one process-wide switch
  * (g_gemm_bf16, craftax_full.cu:11306-11316) and one trainer per process; here two trainers
  * may live in one process, each with a captured update graph, so a trainer can carry its own

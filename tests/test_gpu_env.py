@@ -218,6 +218,42 @@ def test_collect_regenerating_worlds(pkg, cuda, ref):
     tr.close(); pol.close()
 
 
+def test_phase_timers_change_nothing_but_the_clock(pkg, cuda):
+    """cfp_train_set_profile (the reference's CRAFTAX_CU_TRAIN_PROF, craftax_full.cu:12925):
+    two trainers on equal envs and policies run the same iteration, one with the phase timers
+    on (eager update with waits between the phases), one through the captured graph: slabs and
+    parameters agree bit for bit, the four sums are positive and add up to no more than the
+    wall time of the two calls, and a reset clears them."""
+    import time
+    n, T = 256, 8
+    outs = []
+    for timed in (False, True):
+        env = pkg.Env(n)
+        env.init(5)
+        pol = pkg.Policy(n, layers=2, seed=3)
+        tr = pkg.Trainer(pol, T)
+        tr.set_profile(timed)
+        assert tr.profile() == {"rollout": 0.0, "gae": 0.0, "backward": 0.0, "adam": 0.0}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        env.collect(tr, seed=11)
+        tr.update(use_graph=True)
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        ms = tr.profile(reset=True)
+        if timed:
+            assert all(v > 0.0 for v in ms.values()), ms
+            assert sum(ms.values()) <= wall_ms, (ms, wall_ms)
+            assert ms["rollout"] > ms["gae"], ms
+        else:
+            assert all(v == 0.0 for v in ms.values()), ms
+        assert all(v == 0.0 for v in tr.profile().values())
+        outs.append((tr.buf("r_obs").clone(), tr.buf("adv").clone(), pol.params.clone()))
+        tr.close(); pol.close(); env.close()
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+
+
 def test_env_step_on_every_floor_against_the_host_build(pkg, cuda, ref):
     """States on all nine floors with full inventories, armour, spells, enchantments and a boss
     fight under way (env_bind.deep_states): the GPU step against the host build of the same

@@ -111,6 +111,34 @@ def test_backward_matches_oracle(pkg, cuda, n, T, minibatches, bptt_split, bwd_w
     tr.close(); pol.close()
 
 
+def test_backward_matches_oracle_at_a_mid_size(pkg, cuda):
+    """The largest batch the fp64 oracle is asked for: 256 envs x 8 steps (2048 samples,
+    truncation after 4 steps, two windows of 1024 columns), four times the cases above and on
+    the way to the 4096 x 64 shape that is held by properties only: 256 envs fill a workgroup
+    of the dh GEMM and sixteen of the head kernel's.  The batch is taken off the candidate
+    function's kink like the bf16 ones: with 1.6 million gate pre-activations a batch has a
+    value within the margin of zero more often than not (at 8192 samples every batch has, and
+    a comparison with one fp64 evaluation stops being well-posed: an attempt at 512 x 16
+    differed by 7e-4 in the one row of dW_gru a flipped derivative reaches)."""
+    import torch
+    n, T = 256, 8
+    params, pol, tr, host, seed = _collect_off_the_kink(pkg, cuda, n, T, 4321, 0.08, L,
+                                                        bptt_split=2, bwd_win=4)
+    print(f"batch of seed {seed}")
+    tr.buf("grads").zero_()
+    tr.zero_loss()
+    tr.backward(0, n)
+    torch.cuda.synchronize()
+    g = tr.buf("grads").cpu().numpy()
+    l3 = tr.buf("loss_acc").cpu().numpy()
+    batch, keep = ob.make_batch(T, n, 0, n, L, T // 2, **host)
+    g_ref, l3_ref = ob.ppo_backward_f64(params, batch)
+    for name, sl in _segments(L):
+        assert_close(g[sl], g_ref[sl], TOL_FP32, f"d{name}")
+    assert np.allclose(l3, l3_ref, rtol=1e-4), (l3, l3_ref)
+    tr.close(); pol.close()
+
+
 @pytest.mark.parametrize("layers", [1, 2])
 def test_backward_matches_oracle_with_fewer_layers(pkg, cuda, layers):
     """Which of the trainer's two streams runs the dependent chain, the heads' own
