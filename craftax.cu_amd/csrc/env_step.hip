@@ -160,7 +160,8 @@ const FieldDesc kFieldTable[] = {
 constexpr int kNumFields = (int)(sizeof(kFieldTable) / sizeof(kFieldTable[0]));
 
 // ---- storage object of the kernel -----------------------------------------------------------
-constexpr int kSlotWords = 6;                     // row, col, health, mask, cooldown, type
+constexpr int kSlotWords = 4;                     // (row, col), health, cooldown, (type, mask): 17 KiB a wavefront,
+                                                  // so that registers, not LDS, set the eight wavefronts of a CU
 constexpr int kLevelSlots = 14;                   // 3 + 3 + 2 + 3 + 3
 constexpr int kLdsWords = kSlotWords * kLevelSlots + 12;  // + 6 projectile directions x 2
 __device__ __forceinline__ int slot_of(int pool, int i) { return pool < 2 ? pool * 3 + i : (pool == 2 ? 6 + i : 8 + (pool - 3) * 3 + i); }
@@ -190,37 +191,41 @@ struct DevStore {
     __device__ __forceinline__ void put_spawnrow(int kind, int l, int r, uint64_t v) { plane_of(kind)[at(l * kMap + r)] = v; }
 
     __device__ __forceinline__ uint32_t& word(int f, int g) const { return lds[(f * kLevelSlots + g) * kWave]; }
-    __device__ __forceinline__ int m_row(int p, int i) const { return (int)word(0, slot_of(p, i)); }
-    __device__ __forceinline__ int m_col(int p, int i) const { return (int)word(1, slot_of(p, i)); }
-    __device__ __forceinline__ float m_hp(int p, int i) const { return __uint_as_float(word(2, slot_of(p, i))); }
-    __device__ __forceinline__ bool m_mask(int p, int i) const { return word(3, slot_of(p, i)) != 0; }
-    __device__ __forceinline__ int m_cd(int p, int i) const { return (int)word(4, slot_of(p, i)); }
-    __device__ __forceinline__ int m_type(int p, int i) const { return (int)word(5, slot_of(p, i)); }
+    // word 0: row and column as two int16 (positions stay within a step of the 48 x 48 map),
+    // word 1: health, word 2: attack cooldown (counts down without bound), word 3: type id in
+    // the low half, mask in bit 16
+    static __device__ __forceinline__ int lo16(uint32_t w) { return (int)((int32_t)(w << 16) >> 16); }
+    static __device__ __forceinline__ int hi16(uint32_t w) { return (int)((int32_t)w >> 16); }
+    __device__ __forceinline__ int m_row(int p, int i) const { return lo16(word(0, slot_of(p, i))); }
+    __device__ __forceinline__ int m_col(int p, int i) const { return hi16(word(0, slot_of(p, i))); }
+    __device__ __forceinline__ float m_hp(int p, int i) const { return __uint_as_float(word(1, slot_of(p, i))); }
+    __device__ __forceinline__ bool m_mask(int p, int i) const { return (word(3, slot_of(p, i)) >> 16) != 0; }
+    __device__ __forceinline__ int m_cd(int p, int i) const { return (int)word(2, slot_of(p, i)); }
+    __device__ __forceinline__ int m_type(int p, int i) const { return lo16(word(3, slot_of(p, i))); }
     __device__ __forceinline__ void touch(int g) { dirty |= 1u << g; }
     __device__ __forceinline__ void set_m_pos(int p, int i, int r, int c) {
         const int g = slot_of(p, i);
-        word(0, g) = (uint32_t)r;
-        word(1, g) = (uint32_t)c;
+        word(0, g) = ((uint32_t)r & 0xffffu) | ((uint32_t)c << 16);
         touch(g);
     }
     __device__ __forceinline__ void set_m_hp(int p, int i, float v) {
         const int g = slot_of(p, i);
-        word(2, g) = __float_as_uint(v);
+        word(1, g) = __float_as_uint(v);
         touch(g);
     }
     __device__ __forceinline__ void set_m_mask(int p, int i, bool v) {
         const int g = slot_of(p, i);
-        word(3, g) = (uint32_t)v;
+        word(3, g) = (word(3, g) & 0xffffu) | ((uint32_t)v << 16);
         touch(g);
     }
     __device__ __forceinline__ void set_m_cd(int p, int i, int v) {
         const int g = slot_of(p, i);
-        word(4, g) = (uint32_t)v;
+        word(2, g) = (uint32_t)v;
         touch(g);
     }
     __device__ __forceinline__ void set_m_type(int p, int i, int v) {
         const int g = slot_of(p, i);
-        word(5, g) = (uint32_t)v;
+        word(3, g) = (word(3, g) & ~0xffffu) | ((uint32_t)v & 0xffffu);
         touch(g);
     }
     __device__ __forceinline__ uint32_t& dword(int p, int i, int axis) const {
@@ -264,12 +269,10 @@ struct DevStore {
 #pragma unroll
         for (int g = 0; g < kLevelSlots; g++) {
             const int m = global_slot(g);
-            word(0, g) = (uint32_t)A.mob_position[at(2 * m)];
-            word(1, g) = (uint32_t)A.mob_position[at(2 * m + 1)];
-            word(2, g) = __float_as_uint(A.mob_health[at(m)]);
-            word(3, g) = A.mob_mask[at(m)];
-            word(4, g) = (uint32_t)A.mob_attack_cooldown[at(m)];
-            word(5, g) = (uint32_t)A.mob_type_id[at(m)];
+            word(0, g) = ((uint32_t)A.mob_position[at(2 * m)] & 0xffffu) | ((uint32_t)A.mob_position[at(2 * m + 1)] << 16);
+            word(1, g) = __float_as_uint(A.mob_health[at(m)]);
+            word(2, g) = (uint32_t)A.mob_attack_cooldown[at(m)];
+            word(3, g) = ((uint32_t)A.mob_type_id[at(m)] & 0xffffu) | ((uint32_t)(A.mob_mask[at(m)] != 0) << 16);
         }
 #pragma unroll
         for (int j = 0; j < 6; j++) {
@@ -285,12 +288,12 @@ struct DevStore {
         for (int g = 0; g < kLevelSlots; g++) {
             if (!((dirty >> g) & 1u)) continue;
             const int m = global_slot(g);
-            A.mob_position[at(2 * m)] = (int32_t)word(0, g);
-            A.mob_position[at(2 * m + 1)] = (int32_t)word(1, g);
-            A.mob_health[at(m)] = __uint_as_float(word(2, g));
-            A.mob_mask[at(m)] = (uint8_t)word(3, g);
-            A.mob_attack_cooldown[at(m)] = (int32_t)word(4, g);
-            A.mob_type_id[at(m)] = (int32_t)word(5, g);
+            A.mob_position[at(2 * m)] = lo16(word(0, g));
+            A.mob_position[at(2 * m + 1)] = hi16(word(0, g));
+            A.mob_health[at(m)] = __uint_as_float(word(1, g));
+            A.mob_mask[at(m)] = (uint8_t)(word(3, g) >> 16);
+            A.mob_attack_cooldown[at(m)] = (int32_t)word(2, g);
+            A.mob_type_id[at(m)] = lo16(word(3, g));
         }
 #pragma unroll
         for (int j = 0; j < 6; j++) {
