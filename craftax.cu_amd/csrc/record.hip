@@ -90,6 +90,8 @@ constexpr int kRecEnvsPerWg = 256 / kRecLanes;  // more gathers in flight than w
 // of cfp_env_scalars it needs and a table says which array holds each.
 constexpr int kSoaPtrs = 40;
 constexpr int kSoaGather = 32;   // envs per gather round: one 128-byte line of an int32 field array (64 envs: slower)
+constexpr int kSoaGatherFew = 16;   // up to kSoaFewItems envs: twice the workgroups for a GPU that is not full
+constexpr int kSoaFewItems = 16384;  // (8192 envs: 24 -> 19 us; 65 536 envs: 69 -> 84 us with the small rounds)
 struct SoaArgs {
     const void* p[kSoaPtrs];   // the pointer fields of cfp_env_soa, in declaration order
     size_t n_stride;
@@ -177,7 +179,7 @@ struct WordSrc {
 // 11 window bytes of a row lie inside a 4-byte-aligned 16-byte piece of the 48-byte map row)
 // into an LDS strip, and the cells pick their bytes out of the strip: 27 sixteen-byte loads
 // per env instead of 297 single-byte ones.  Needs 4-byte-aligned planes and strides.
-template <bool SOA, bool ROW16>
+template <bool SOA, bool ROW16, int SOA_GATHER = kSoaGather>
 __global__ __launch_bounds__(256) void k_record_obs(
     const cfp_env_scalars* __restrict__ scalars, SoaArgs soa, RecWhich which,
     const uint8_t* __restrict__ map, const uint8_t* __restrict__ item_map,
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(256) void k_record_obs(
     typedef unsigned int strip_u4 __attribute__((ext_vector_type(4)));
     __shared__ strip_u4 strip_all[ROW16 ? kRecEnvsPerWg : 1][3 * ROWS + 1];   // [plane * 9 + row], odd stride
     // SOA rounds take 32 envs: a 128-byte line of every field array is used by one workgroup
-    constexpr int kGather = SOA ? kSoaGather : kRecEnvsPerWg;
+    constexpr int kGather = SOA ? SOA_GATHER : kRecEnvsPerWg;
     __shared__ uint32_t sc_all[SOA ? kGather : 1][kScalarWords + 1];
     __shared__ const void* ptrs[SOA ? kSoaPtrs : 1];
     __shared__ SoaWord words[SOA ? kScalarWords : 1];
@@ -581,14 +583,17 @@ static int record_obs_soa(const cfp_env_soa* soa, const uint8_t* d_map, const ui
     std::memcpy(&a, soa, sizeof(a));
     for (int i = 0; i < kSoaPtrs; i++)
         CFP_REQUIRE(a.p[i] != nullptr, "cfp_record_obs_soa: field array %d of the view is NULL", i);
-    if (rows16_ok(d_map, d_item_map, d_light_map, env_stride, level_stride))
-        hipLaunchKernelGGL((k_record_obs<true, true>), dim3((items + kSoaGather - 1) / kSoaGather),
-                           dim3(256), 0, (hipStream_t)stream, nullptr, a, which, d_map, d_item_map,
-                           d_light_map, env_stride, level_stride, d_rec_row, n);
-    else
-        hipLaunchKernelGGL((k_record_obs<true, false>), dim3((items + kSoaGather - 1) / kSoaGather),
-                           dim3(256), 0, (hipStream_t)stream, nullptr, a, which, d_map, d_item_map,
-                           d_light_map, env_stride, level_stride, d_rec_row, n);
+    const bool rows16 = rows16_ok(d_map, d_item_map, d_light_map, env_stride, level_stride);
+    const bool few = items <= kSoaFewItems;
+    const dim3 grid((items + (few ? kSoaGatherFew : kSoaGather) - 1) / (few ? kSoaGatherFew : kSoaGather));
+#define CFP_REC_SOA(R16, G)                                                                              \
+    hipLaunchKernelGGL((k_record_obs<true, R16, G>), grid, dim3(256), 0, (hipStream_t)stream, nullptr, a, \
+                       which, d_map, d_item_map, d_light_map, env_stride, level_stride, d_rec_row, n)
+    if (rows16 && few) CFP_REC_SOA(true, kSoaGatherFew);
+    else if (rows16) CFP_REC_SOA(true, kSoaGather);
+    else if (few) CFP_REC_SOA(false, kSoaGatherFew);
+    else CFP_REC_SOA(false, kSoaGather);
+#undef CFP_REC_SOA
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }
