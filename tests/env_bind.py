@@ -120,8 +120,57 @@ def deep_states(ref, n, seed):
                 s["sword"] = max(int(s["sword"]), 1)
                 s["bow"] = 1
                 s["armour"] = np.maximum(s["armour"], 1)
+        # the other half of the envs of floors 0, 7 and 8 stand in front of what random play
+        # does not reach: a ripe plant, a wounded ice elemental, the necromancer one hit from
+        # defeat with no guards and no timer (deep_script forces the DO actions)
+        elif (e // L) % 2 == 1 and lvl in (0, 7, 8):
+            pr, pc = (int(v) for v in s["player_position"])
+            steps_of = {1: (0, -1), 2: (0, 1), 3: (-1, 0), 4: (1, 0)}
+
+            def free(r, c):
+                return (0 <= r < M and 0 <= c < M and s["map"][lvl, r, c] in (2, 7, 25, 26)
+                        and s["item_map"][lvl, r, c] == 0 and not (int(s["mob_bits"][lvl, r]) >> c) & 1)
+            if lvl == L - 1:
+                boss = np.argwhere(s["map"][lvl] == 32)
+                for d, (dr, dc) in steps_of.items():
+                    if len(boss) and free(int(boss[0][0]) - dr, int(boss[0][1]) - dc):
+                        s["player_position"] = (boss[0][0] - dr, boss[0][1] - dc)
+                        s["player_direction"] = d
+                        s["boss_progress"] = 7
+                        s["boss_timesteps_to_spawn_this_round"] = 0
+                        s["mob_mask"][:3, lvl] = 0
+                        s["mob_bits"][lvl] = 0
+                        break
+            else:
+                for d, (dr, dc) in steps_of.items():
+                    r, c = pr + dr, pc + dc
+                    if not free(r, c):
+                        continue
+                    s["player_direction"] = d
+                    if lvl == 0:
+                        s["map"][lvl, r, c] = 16
+                        s["growing_plants_positions"][0] = (r, c)
+                        s["growing_plants_age"][0] = 700
+                        s["growing_plants_mask"][0] = 1
+                    else:
+                        s["mob_position"][2, lvl, 0] = (r, c)
+                        s["mob_health"][2, lvl, 0] = 0.5
+                        s["mob_mask"][2, lvl, 0] = 1
+                        s["mob_type_id"][2, lvl, 0] = 7
+                        s["mob_attack_cooldown"][2, lvl, 0] = 3
+                        s["mob_bits"][lvl, r] |= np.uint64(1) << np.uint64(c)
+                    break
         ref.import_(e, s)
+        st[e] = ref.export([e])[0]      # the spawn bit planes follow the edited map
     return st
+
+
+def deep_script(n):
+    """Actions forced on the first two steps of deep_states' envs (-1: none): DO for the envs
+    that were put in front of a plant, an ice elemental or the necromancer."""
+    e = np.arange(n)
+    special = ((e // L) % 2 == 1) & np.isin(e % L, (0, 7, 8))
+    return np.where(special, 5, -1).astype(np.float32)
 
 
 class Ref:
