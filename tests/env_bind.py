@@ -62,6 +62,10 @@ def diff_fields(a, b):
     return out
 
 
+# floor -> what half of its envs are put in front of (block id where it is a block)
+DEEP_ENCOUNTERS = {0: 16, 2: 10, 3: 21, 4: 22, 5: 29, 7: None, 8: 32}
+
+
 def deep_states(ref, n, seed):
     """n reference worlds (ref.init) with the player moved onto floor e % 9 at that floor's
     up ladder and given what a long episode collects: tools, weapons, arrows, torches, ores,
@@ -120,10 +124,11 @@ def deep_states(ref, n, seed):
                 s["sword"] = max(int(s["sword"]), 1)
                 s["bow"] = 1
                 s["armour"] = np.maximum(s["armour"], 1)
-        # the other half of the envs of floors 0, 7 and 8 stand in front of what random play
-        # does not reach: a ripe plant, a wounded ice elemental, the necromancer one hit from
-        # defeat with no guards and no timer (deep_script forces the DO actions)
-        elif (e // L) % 2 == 1 and lvl in (0, 7, 8):
+        # the other half of the envs of seven floors stand in front of what random play does not
+        # reach: a ripe plant, a diamond, a sapphire, a ruby, an ice shrub (pickaxe 4), a wounded
+        # ice elemental, the necromancer one hit from defeat with no guards and no timer
+        # (deep_script forces the DO actions)
+        elif (e // L) % 2 == 1 and lvl in DEEP_ENCOUNTERS:
             pr, pc = (int(v) for v in s["player_position"])
             steps_of = {1: (0, -1), 2: (0, 1), 3: (-1, 0), 4: (1, 0)}
 
@@ -152,6 +157,9 @@ def deep_states(ref, n, seed):
                         s["growing_plants_positions"][0] = (r, c)
                         s["growing_plants_age"][0] = 700
                         s["growing_plants_mask"][0] = 1
+                    elif lvl != 7:      # a diamond, a sapphire, a ruby, an ice shrub to be mined
+                        s["map"][lvl, r, c] = DEEP_ENCOUNTERS[lvl]
+                        s["pickaxe"] = 4
                     else:
                         s["mob_position"][2, lvl, 0] = (r, c)
                         s["mob_health"][2, lvl, 0] = 0.5
@@ -169,7 +177,7 @@ def deep_script(n):
     """Actions forced on the first two steps of deep_states' envs (-1: none): DO for the envs
     that were put in front of a plant, an ice elemental or the necromancer."""
     e = np.arange(n)
-    special = ((e // L) % 2 == 1) & np.isin(e % L, (0, 7, 8))
+    special = ((e // L) % 2 == 1) & np.isin(e % L, list(DEEP_ENCOUNTERS))
     return np.where(special, 5, -1).astype(np.float32)
 
 
