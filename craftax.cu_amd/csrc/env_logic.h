@@ -422,12 +422,54 @@ CFE_FN void set_block(S& s, int l, int r, int c, int b) {
     }
 }
 
-// craftax_step_is_in_mob (:4319-4330)
+// The level's mob bitmap is, at every point of a step, the set of cells of the live melee,
+// passive and ranged mobs of that level (a mob's bit is set where it appears, moved with it and
+// cleared where it dies or despawns; no two of them share a cell).  The step therefore asks
+// the mob slots -- which the storage holds close by -- where it needs occupancy, and writes a
+// bitmap row as what the slots say; it never waits for a bitmap row from memory.
+// The eight movers' cells as one word each (row in the high half, column in the low half; a
+// dead slot holds a cell no query names), read from the slots with no branch between the
+// reads, so that they travel together, and kept in registers while the mobs move.
+struct MoverKeys {
+    uint32_t key[8];
+};
+constexpr uint32_t kNoCell = 0x80008000u;
+CFE_FN uint32_t cell_key(int r, int c) { return ((uint32_t)r << 16) | ((uint32_t)c & 0xffffu); }
+CFE_FN int mover_pool(int k) { return k < 3 ? P_MELEE : (k < 6 ? P_PASSIVE : P_RANGED); }
+CFE_FN int mover_slot(int k) { return k < 6 ? k % 3 : k - 6; }
+template <class S>
+CFE_FN MoverKeys load_mover_keys(S& s) {
+    MoverKeys m;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const int p = mover_pool(k), i = mover_slot(k);
+        const uint32_t cell = cell_key(s.m_row(p, i), s.m_col(p, i));
+        m.key[k] = s.m_mask(p, i) ? cell : kNoCell;
+    }
+    return m;
+}
+CFE_FN bool keys_at(const MoverKeys& m, int r, int c) {
+    const uint32_t want = cell_key(r, c);
+    bool any = false;
+#pragma unroll
+    for (int k = 0; k < 8; k++) any = any | (m.key[k] == want);
+    return any;
+}
+CFE_FN uint64_t keys_row(const MoverKeys& m, int row) {
+    uint64_t bits = 0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) bits |= (m.key[k] >> 16) == (uint32_t)row ? 1ull << (m.key[k] & 63u) : 0ull;
+    return bits & kRowMask;
+}
+template <class S>
+CFE_FN bool mover_at(S& s, int r, int c) { return keys_at(load_mover_keys(s), r, c); }
+template <class S>
+CFE_FN uint64_t movers_row(S& s, int row) { return keys_row(load_mover_keys(s), row); }
+
+// craftax_step_is_in_mob (:4319-4330): the bitmap's bit at the clamped cell, or the player
 template <class S>
 CFE_FN bool mob_or_player_at(S& s, const Hot& h, int r, int c) {
-    const int l = wrap_clamp(h.level, kLevels);
-    const bool mob = (s.mobrow(l, wrap_clamp(r, kMap)) >> wrap_clamp(c, kMap)) & 1ull;
-    return mob || (h.pr == r && h.pc == c);
+    return mover_at(s, wrap_clamp(r, kMap), wrap_clamp(c, kMap)) || (h.pr == r && h.pc == c);
 }
 
 // craftax_move_player_native (:4332-4379)
@@ -638,7 +680,8 @@ CFE_FN Hit hit_cell(S& s, Hot& h, int r, int c, const float (&dmg)[3], bool can_
     int ur, uc;
     if (killed && wrap_drop(r, kMap, ur) && wrap_drop(c, kMap, uc)) {
         const int l = wrap_clamp(h.level, kLevels);
-        s.put_mobrow(l, ur, s.mobrow(l, ur) & ~(1ull << uc));
+        (void)uc;
+        s.put_mobrow(l, ur, movers_row(s, ur));
     }
     if (monster) {
         const int l = wrap_clamp(h.level, kLevels);
@@ -998,54 +1041,38 @@ CFE_FN float damage_to_player(const Hot& h, const float (&dmg)[3]) {
     return total;
 }
 
-// What a moving mob reads from memory -- the block under its target cell and the two rows of
-// the level's mob bitmap it may leave and enter -- asked for together, so that a mob costs
-// one memory round trip instead of one per dependent read (validity test, bitmap clear,
-// bitmap set).  The indices are always addressable (wrap_clamp); whether a value is used is
-// decided afterwards.
-struct MoverView {
-    int b;                       // block at (i_to, wrap_clamp(c1))
-    uint64_t row_from, row_to;   // bitmap rows i_from = wrap_clamp(r0), i_to = wrap_clamp(r1)
-    int i_from, i_to;
+// A mob's move in two halves.  `plan_*` makes every draw of the mob and fixes the cell it
+// wants to enter -- that needs the mob's own slot, the player's position and the key, nothing
+// an earlier mob of the same step changes.  update_mobs plans all eight movers first and asks
+// for the blocks under their targets together (one memory round trip for the eight instead
+// of one each); `apply_*` then runs mob by mob in the reference's order with that block:
+// damage to the player, the validity of the target against the mobs as they stand by then,
+// the bitmap rows, the slot.
+struct MoverPlan {
+    bool active;      // the slot holds a mob
+    int r1, c1;       // the cell the validity test looks at
+    Vec2 to;          // ranged: the step towards the player (projectile direction, retreat)
 };
-template <class S>
-CFE_FN MoverView mover_view(S& s, int l, int r0, int r1, int c1) {
-    MoverView v;
-    v.i_from = wrap_clamp(r0, kMap);
-    v.i_to = wrap_clamp(r1, kMap);
-    v.b = s.blk(l, v.i_to, wrap_clamp(c1, kMap));
-    v.row_from = s.mobrow(l, v.i_from);
-    v.row_to = s.mobrow(l, v.i_to);
-    return v;
-}
-// craftax_update_mobs_valid_position (:6625-6648) for the view's target (r, c)
-CFE_FN bool can_stand_view(const Hot& h, const MoverView& v, int r, int c, int collision) {
-    const bool solid = is_solid(v.b), water = v.b == B_WATER, lava = v.b == B_LAVA;
+// craftax_update_mobs_valid_position (:6625-6648) for target (r, c) with block b under it
+CFE_FN bool can_stand(const MoverKeys& m, const Hot& h, int b, int r, int c, int collision) {
+    const bool solid = is_solid(b), water = b == B_WATER, lava = b == B_LAVA;
     const bool ground = !solid && !water && !lava;
-    const bool mob = (v.row_to >> wrap_clamp(c, kMap)) & 1ull;
-    bool ok = on_map(r, c) && !(mob || (h.pr == r && h.pc == c)) && !solid;
+    const bool taken = keys_at(m, wrap_clamp(r, kMap), wrap_clamp(c, kMap)) || (h.pr == r && h.pc == c);
+    bool ok = on_map(r, c) && !taken && !solid;
     ok = ok && (!(collision & 1) || !ground);
     ok = ok && (!(collision & 2) || !water);
     ok = ok && (!(collision & 4) || !lava);
     return ok;
 }
-// A mob leaves (r0, c0) and, if it stays alive, occupies (rf, cf) -- its old cell or the
-// view's target -- in the level's mob bitmap (craftax_update_mobs_clear_old_map_entry /
-// _enter_new_map_entry, :6389-6421: scatter indices, negative wraps, 48 and beyond is
-// dropped).  A valid scatter index equals the clamped one, so the row left is i_from and
-// the row entered i_from or i_to; both changes to one row go out as one write.
+// The mob of (pool, i) has left row r0 and stands -- if it is still alive -- where its slot
+// says: the rows it left and entered go out as the slots have them
+// (craftax_update_mobs_clear_old_map_entry / _enter_new_map_entry, :6389-6421).
 template <class S>
-CFE_FN void settle_in_bitmap(S& s, int l, const MoverView& v, int r0, int c0, int rf, int cf, bool alive) {
-    int lr0, lc0, lrf = 0, lcf = 0;
-    const bool clr = wrap_drop(r0, kMap, lr0) && wrap_drop(c0, kMap, lc0);
-    const bool set = alive && wrap_drop(rf, kMap, lrf) && wrap_drop(cf, kMap, lcf);
-    uint64_t from = v.row_from, to = v.row_to;
-    if (clr) from &= ~(1ull << lc0);
-    const bool into_from = set && lrf == v.i_from;
-    if (into_from) from |= 1ull << lcf;
-    if (set && !into_from) to |= 1ull << lcf;
-    if (clr || into_from) s.put_mobrow(l, v.i_from, from);
-    if (set && !into_from) s.put_mobrow(l, v.i_to, to);
+CFE_FN void settle_in_bitmap(S& s, int l, MoverKeys& m, int k, int r0, int r1, int c1, bool alive) {
+    m.key[k] = alive ? cell_key(r1, c1) : kNoCell;
+    const int i_from = wrap_clamp(r0, kMap), i_to = wrap_clamp(r1, kMap);
+    s.put_mobrow(l, i_from, keys_row(m, i_from));
+    if (i_to != i_from) s.put_mobrow(l, i_to, keys_row(m, i_to));
 }
 
 // the step towards the player along the longer axis, drawn when both are equal
@@ -1067,21 +1094,32 @@ CFE_FN Vec2 random_step(uint64_t key, int choices) {  // craftax_update_mobs_dir
 
 // craftax_update_mobs_move_melee (:6856-6987)
 template <class S>
-CFE_FN void move_melee(S& s, Hot& h, uint64_t& rng, int i) {
-    if (!s.m_mask(P_MELEE, i)) return;
-    const int l = wrap_clamp(h.level, kLevels);
-    const int r0 = s.m_row(P_MELEE, i), c0 = s.m_col(P_MELEE, i), cd = s.m_cd(P_MELEE, i), type = s.m_type(P_MELEE, i);
+CFE_FN MoverPlan plan_melee(S& s, const Hot& h, uint64_t& rng, int i) {
+    MoverPlan p{s.m_mask(P_MELEE, i), 0, 0, Vec2{0, 0}};
+    if (!p.active) return p;
+    const int r0 = s.m_row(P_MELEE, i), c0 = s.m_col(P_MELEE, i), cd = s.m_cd(P_MELEE, i);
     const Vec2 rnd = random_step(next_key(rng), 4);
     const Vec2 to = step_towards_player(h, next_key(rng), r0, c0);
     const int dist = iabs(h.pr - r0) + iabs(h.pc - c0);
     bool chase = dist < 10 || at_boss(h);
     chase = (draw_unit(next_key(rng)) < 0.75f) && chase;
-    int r1 = r0 + (chase ? to.r : rnd.r), c1 = c0 + (chase ? to.c : rnd.c);
-    const bool attacking = dist == 1 && cd <= 0;
-    if (attacking) {
-        r1 = r0;
-        c1 = c0;
+    p.r1 = r0 + (chase ? to.r : rnd.r);
+    p.c1 = c0 + (chase ? to.c : rnd.c);
+    if (dist == 1 && cd <= 0) {   // attacking: it stays
+        p.r1 = r0;
+        p.c1 = c0;
     }
+    rng = lcg(lcg(rng));
+    return p;
+}
+template <class S>
+CFE_FN void apply_melee(S& s, Hot& h, MoverKeys& m, const MoverPlan& p, int b, int i) {
+    if (!p.active) return;
+    const int l = wrap_clamp(h.level, kLevels);
+    const int r0 = s.m_row(P_MELEE, i), c0 = s.m_col(P_MELEE, i), cd = s.m_cd(P_MELEE, i), type = s.m_type(P_MELEE, i);
+    const int dist = iabs(h.pr - r0) + iabs(h.pc - c0);
+    const bool attacking = dist == 1 && cd <= 0;
+    int r1 = p.r1, c1 = p.c1;
     float base[3];
     mob_damage(type, MC_MELEE, base);
     const float asleep = 1.0f + 2.5f * (float)(int)(h.sleeping != 0);
@@ -1091,45 +1129,49 @@ CFE_FN void move_melee(S& s, Hot& h, uint64_t& rng, int i) {
     h.health -= damage * (float)(int)attacking;
     unlock_if(h, ACH_WAKE_UP, h.sleeping && attacking);
     if (attacking) h.sleeping = h.resting = 0;
-    const MoverView view = mover_view(s, l, r0, r1, c1);
-    const bool ok = can_stand_view(h, view, r1, c1, mob_collision(type, MC_MELEE));
-    if (!ok) {
+    if (!can_stand(m, h, b, r1, c1, mob_collision(type, MC_MELEE))) {
         r1 = r0;
         c1 = c0;
     }
     const bool alive = dist < kDespawn || at_boss(h);
-    rng = lcg(lcg(rng));
-    settle_in_bitmap(s, l, view, r0, c0, r1, c1, alive);
     s.set_m_pos(P_MELEE, i, r1, c1);
     s.set_m_cd(P_MELEE, i, attacking ? 5 : cd - 1);
     s.set_m_mask(P_MELEE, i, alive);
+    settle_in_bitmap(s, l, m, i, r0, r1, c1, alive);
 }
 
 // craftax_update_mobs_move_passive (:6989-7052)
 template <class S>
-CFE_FN void move_passive(S& s, Hot& h, uint64_t& rng, int i) {
-    if (!s.m_mask(P_PASSIVE, i)) return;
+CFE_FN MoverPlan plan_passive(S& s, const Hot&, uint64_t& rng, int i) {
+    MoverPlan p{s.m_mask(P_PASSIVE, i), 0, 0, Vec2{0, 0}};
+    if (!p.active) return p;
+    const Vec2 rnd = random_step(next_key(rng), 8);
+    p.r1 = s.m_row(P_PASSIVE, i) + rnd.r;
+    p.c1 = s.m_col(P_PASSIVE, i) + rnd.c;
+    return p;
+}
+template <class S>
+CFE_FN void apply_passive(S& s, Hot& h, MoverKeys& m, const MoverPlan& p, int b, int i) {
+    if (!p.active) return;
     const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_PASSIVE, i), c0 = s.m_col(P_PASSIVE, i), type = s.m_type(P_PASSIVE, i);
-    const Vec2 rnd = random_step(next_key(rng), 8);
-    int r1 = r0 + rnd.r, c1 = c0 + rnd.c;
-    const MoverView view = mover_view(s, l, r0, r1, c1);
-    if (!can_stand_view(h, view, r1, c1, mob_collision(type, MC_PASSIVE))) {
+    int r1 = p.r1, c1 = p.c1;
+    if (!can_stand(m, h, b, r1, c1, mob_collision(type, MC_PASSIVE))) {
         r1 = r0;
         c1 = c0;
     }
     const bool alive = iabs(r0 - h.pr) + iabs(c0 - h.pc) < kDespawn;
-    settle_in_bitmap(s, l, view, r0, c0, r1, c1, alive);
     s.set_m_pos(P_PASSIVE, i, r1, c1);
     s.set_m_mask(P_PASSIVE, i, alive);
+    settle_in_bitmap(s, l, m, 3 + i, r0, r1, c1, alive);
 }
 
 // craftax_update_mobs_move_ranged (:7054-7191)
 template <class S>
-CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
-    if (!s.m_mask(P_RANGED, i)) return;
-    const int l = wrap_clamp(h.level, kLevels);
-    const int r0 = s.m_row(P_RANGED, i), c0 = s.m_col(P_RANGED, i), cd = s.m_cd(P_RANGED, i), type = s.m_type(P_RANGED, i);
+CFE_FN MoverPlan plan_ranged(S& s, const Hot& h, uint64_t& rng, int i) {
+    MoverPlan p{s.m_mask(P_RANGED, i), 0, 0, Vec2{0, 0}};
+    if (!p.active) return p;
+    const int r0 = s.m_row(P_RANGED, i), c0 = s.m_col(P_RANGED, i);
     const Vec2 rnd = random_step(next_key(rng), 4);
     const Vec2 to = step_towards_player(h, next_key(rng), r0, c0);
     const int dist = iabs(h.pr - r0) + iabs(h.pc - c0);
@@ -1143,12 +1185,23 @@ CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
         r1 = r0 + rnd.r;
         c1 = c0 + rnd.c;
     }
-    const int collision = mob_collision(type, MC_RANGED);
+    p.r1 = r1;
+    p.c1 = c1;
+    p.to = to;
+    return p;
+}
+template <class S>
+CFE_FN void apply_ranged(S& s, Hot& h, MoverKeys& m, const MoverPlan& p, int b, int i) {
+    if (!p.active) return;
+    const int l = wrap_clamp(h.level, kLevels);
+    const int r0 = s.m_row(P_RANGED, i), c0 = s.m_col(P_RANGED, i), cd = s.m_cd(P_RANGED, i), type = s.m_type(P_RANGED, i);
+    const int dist = iabs(h.pr - r0) + iabs(h.pc - c0);
+    const bool close = dist <= 3;
+    int r1 = p.r1, c1 = p.c1;
     // the target's validity is read once: the reference asks for it up to twice (here and
     // below), for this target or -- when the mob attacks and stays -- for its own cell, which
     // it occupies itself, so that answer never changes where the mob ends up
-    const MoverView view = mover_view(s, l, r0, r1, c1);
-    const bool can = can_stand_view(h, view, r1, c1, collision);
+    const bool can = can_stand(m, h, b, r1, c1, mob_collision(type, MC_RANGED));
     bool attacking = dist >= 4 && dist <= 5;
     attacking = attacking || (close && !can);
     attacking = attacking && cd <= 0;
@@ -1164,7 +1217,7 @@ CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
             s.set_m_pos(P_MOB_PROJ, slot, r0, c0);
             s.set_m_mask(P_MOB_PROJ, slot, true);
             s.set_m_type(P_MOB_PROJ, slot, ranged_projectile(type));
-            s.set_pd(P_MOB_PROJ, slot, to.r, to.c);
+            s.set_pd(P_MOB_PROJ, slot, p.to.r, p.to.c);
         }
         r1 = r0;
         c1 = c0;
@@ -1174,22 +1227,22 @@ CFE_FN void move_ranged(S& s, Hot& h, uint64_t& rng, int i) {
         c1 = c0;
     }
     const bool alive = dist < kDespawn || at_boss(h);
-    settle_in_bitmap(s, l, view, r0, c0, r1, c1, alive);
     s.set_m_pos(P_RANGED, i, r1, c1);
     s.set_m_cd(P_RANGED, i, attacking ? 4 : cd - 1);
     s.set_m_mask(P_RANGED, i, alive);
+    settle_in_bitmap(s, l, m, 6 + i, r0, r1, c1, alive);
 }
 
-// craftax_update_mobs_move_mob_projectile (:7193-7268)
+// craftax_update_mobs_move_mob_projectile (:7193-7268); b = the block under its next cell.
+// Returns true when it destroyed that block (a crafting table or furnace in the way).
 template <class S>
-CFE_FN void move_mob_projectile(S& s, Hot& h, int i) {
-    if (!s.m_mask(P_MOB_PROJ, i)) return;
+CFE_FN bool move_mob_projectile(S& s, Hot& h, const MoverKeys& m, int b, int i) {
+    if (!s.m_mask(P_MOB_PROJ, i)) return false;
     const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_MOB_PROJ, i), c0 = s.m_col(P_MOB_PROJ, i);
     const int r1 = r0 + s.pd_r(P_MOB_PROJ, i), c1 = c0 + s.pd_c(P_MOB_PROJ, i);
-    const int b = s.blk(wrap_clamp(l, kLevels), wrap_clamp(r1, kMap), wrap_clamp(c1, kMap));
     const bool hit = (r0 == h.pr && c0 == h.pc) || (r1 == h.pr && c1 == h.pc);
-    const bool taken = mob_or_player_at(s, h, r1, c1);   // read beside the block, not after it
+    const bool taken = keys_at(m, wrap_clamp(r1, kMap), wrap_clamp(c1, kMap)) || (h.pr == r1 && h.pc == c1);
     const bool flying = on_map(r1, c1) && !is_solid(b) && !taken && !hit;
     float dmg[3];
     mob_damage(s.m_type(P_MOB_PROJ, i), MC_PROJECTILE, dmg);
@@ -1201,15 +1254,17 @@ CFE_FN void move_mob_projectile(S& s, Hot& h, int i) {
     // a crafting table or furnace in the way is destroyed; the write goes through the
     // scatter index (negative wraps, 48 and beyond is dropped) while the read was clamped
     int wl, wr, wc;
-    if ((b == B_FURNACE || b == B_TABLE) && wrap_drop(l, kLevels, wl) && wrap_drop(r1, kMap, wr) && wrap_drop(c1, kMap, wc))
+    if ((b == B_FURNACE || b == B_TABLE) && wrap_drop(l, kLevels, wl) && wrap_drop(r1, kMap, wr) && wrap_drop(c1, kMap, wc)) {
         set_block(s, wl, wr, wc, B_PATH);
+        return true;
+    }
+    return false;
 }
 
-// craftax_update_mobs_move_player_projectile (:6799-6854, 7270-7346)
+// craftax_update_mobs_move_player_projectile (:6799-6854, 7270-7346); b as above
 template <class S>
-CFE_FN void move_player_projectile(S& s, Hot& h, int i) {
+CFE_FN void move_player_projectile(S& s, Hot& h, int b, int i) {
     if (!s.m_mask(P_PLAYER_PROJ, i)) return;
-    const int l = wrap_clamp(h.level, kLevels);
     const int r0 = s.m_row(P_PLAYER_PROJ, i), c0 = s.m_col(P_PLAYER_PROJ, i);
     const int r1 = r0 + s.pd_r(P_PLAYER_PROJ, i), c1 = c0 + s.pd_c(P_PLAYER_PROJ, i);
     const int type = s.m_type(P_PLAYER_PROJ, i);
@@ -1232,7 +1287,6 @@ CFE_FN void move_player_projectile(S& s, Hot& h, int i) {
 #pragma unroll
         for (int k = 0; k < 3; k++) dmg[k] *= coeff;
     }
-    const int b = s.blk(wrap_clamp(l, kLevels), wrap_clamp(r1, kMap), wrap_clamp(c1, kMap));
     const Hit first = hit_cell(s, h, r0, c0, dmg, false);
     float second[3];
 #pragma unroll
@@ -1245,14 +1299,49 @@ CFE_FN void move_player_projectile(S& s, Hot& h, int i) {
 
 template <class S>
 CFE_FN void update_mobs(S& s, Hot& h, uint64_t rng) {
+    const int l = wrap_clamp(h.level, kLevels);
+    MoverPlan plan[8];
     rng = lcg(rng);
-    for (int i = 0; i < 3; i++) move_melee(s, h, rng, i);
+#pragma unroll
+    for (int i = 0; i < 3; i++) plan[i] = plan_melee(s, h, rng, i);
     rng = lcg(rng);
-    for (int i = 0; i < 3; i++) move_passive(s, h, rng, i);
+#pragma unroll
+    for (int i = 0; i < 3; i++) plan[3 + i] = plan_passive(s, h, rng, i);
     rng = lcg(rng);
-    for (int i = 0; i < 2; i++) move_ranged(s, h, rng, i);
-    for (int i = 0; i < 3; i++) move_mob_projectile(s, h, i);
-    for (int i = 0; i < 3; i++) move_player_projectile(s, h, i);
+#pragma unroll
+    for (int i = 0; i < 2; i++) plan[6 + i] = plan_ranged(s, h, rng, i);
+    // the eight blocks, asked for together (an empty slot reads the block under cell (0, 0))
+    int b[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) b[k] = s.blk(l, wrap_clamp(plan[k].r1, kMap), wrap_clamp(plan[k].c1, kMap));
+    MoverKeys m = load_mover_keys(s);
+#pragma unroll
+    for (int i = 0; i < 3; i++) apply_melee(s, h, m, plan[i], b[i], i);
+#pragma unroll
+    for (int i = 0; i < 3; i++) apply_passive(s, h, m, plan[3 + i], b[3 + i], i);
+#pragma unroll
+    for (int i = 0; i < 2; i++) apply_ranged(s, h, m, plan[6 + i], b[6 + i], i);
+    // the six projectiles -- those the ranged mobs just launched among them -- likewise.  A
+    // mob projectile that destroys the block under its next cell changes what a later
+    // projectile with the same next cell finds there.
+    int pr1[6], pc1[6], pb[6];
+#pragma unroll
+    for (int k = 0; k < 6; k++) {
+        const int pool = k < 3 ? P_MOB_PROJ : P_PLAYER_PROJ, i = k % 3;
+        pr1[k] = wrap_clamp(s.m_row(pool, i) + s.pd_r(pool, i), kMap);
+        pc1[k] = wrap_clamp(s.m_col(pool, i) + s.pd_c(pool, i), kMap);
+        pb[k] = s.blk(l, pr1[k], pc1[k]);
+    }
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+        if (move_mob_projectile(s, h, m, pb[i], i)) {
+#pragma unroll
+            for (int k = i + 1; k < 6; k++)
+                if (pr1[k] == pr1[i] && pc1[k] == pc1[i]) pb[k] = B_PATH;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 3; i++) move_player_projectile(s, h, pb[3 + i], i);
 }
 
 // ---- spawning (craftax_spawn_mobs_native, :7397-8225) ---------------------------------------
@@ -1438,7 +1527,7 @@ CFE_FN void place_spawn(S& s, int l, int which, const SpawnPlan& p, int row, int
     s.set_m_pos(pool, p.slot[which], row, col);
     s.set_m_hp(pool, p.slot[which], mob_health(p.type[which], spawn_class(which)));
     s.set_m_mask(pool, p.slot[which], true);
-    s.put_mobrow(l, row, s.mobrow(l, row) | (1ull << col));
+    s.put_mobrow(l, row, movers_row(s, row));
 }
 // second half (:8133-8224): passive, melee, ranged in that order.  The reference scans all
 // three against the bitmap as it was and then excludes the cells just taken; scanning in

@@ -75,6 +75,10 @@ typedef struct cfp_env_state {
     uint32_t rng_key[2];
     uint8_t achievements[CFP_ENV_ACHIEVEMENTS];
     uint8_t pad_[5];
+    /* bit c of row r of a level: a live melee, passive or ranged mob stands on (r, c).  The step
+     * keeps the rows it touches equal to what the mob slots say and asks the slots, not these
+     * rows, whether a cell is taken: an imported state has to hold the two in agreement, as
+     * every state the game produces does (mob positions within the 48 x 48 map). */
     uint64_t mob_bits[CFP_ENV_LEVELS][CFP_ENV_MAP];
     uint64_t spawn_all_bits[CFP_ENV_LEVELS][CFP_ENV_MAP];
     uint64_t spawn_grave_bits[CFP_ENV_LEVELS][CFP_ENV_MAP];

@@ -54,6 +54,51 @@ def test_host_build_of_the_step_matches_reference(ref, n, steps, seed):
     assert terminals > 0
 
 
+def _mob_bits_from_slots(states):
+    """The mob bitmap as the live melee, passive and ranged slots define it."""
+    n = len(states)
+    bits = np.zeros((n, eb.L, eb.M), np.uint64)
+    pos, mask = states["mob_position"], states["mob_mask"]
+    for cls, slots in ((0, 3), (1, 3), (2, 2)):
+        for lvl in range(eb.L):
+            for i in range(slots):
+                live = mask[:, cls, lvl, i] != 0
+                r, c = pos[:, cls, lvl, i, 0], pos[:, cls, lvl, i, 1]
+                assert ((r[live] >= 0) & (r[live] < eb.M) & (c[live] >= 0) & (c[live] < eb.M)).all()
+                e = np.nonzero(live)[0]
+                bits[e, lvl, r[e]] |= np.uint64(1) << c[e].astype(np.uint64)
+    return bits
+
+
+def test_reference_keeps_the_mob_bitmap_equal_to_the_mob_slots():
+    """What the step relies on where it asks the mob slots instead of the bitmap whether a
+    cell is taken, and writes a bitmap row as the slots have it: in the reference's own
+    states -- fresh worlds under random play and the prepared deep states, every step, all
+    nine levels, final states of finished episodes included -- a level's bitmap is exactly
+    the cells of its live melee, passive and ranged mobs, and those are on the map."""
+    try:
+        strict = eb.Ref(strict=True)
+    except FileNotFoundError:
+        pytest.skip("oracle/_ref/libcfref_strict.so is not built (reference source absent)")
+    seen = 0
+    for prepared in (False, True):
+        n = 144
+        if prepared:
+            eb.deep_states(strict, n, 99)
+        else:
+            strict.init(n, 3)
+        script = eb.deep_script(n)
+        for t in range(300):
+            act = strict.next_actions()
+            if prepared and t < 2:
+                act = np.where(script >= 0, script, act).astype(np.float32)
+            final, rew, term, keys = strict.step(act)
+            want = _mob_bits_from_slots(final)
+            assert np.array_equal(final["mob_bits"], want), f"prepared={prepared}, step {t}"
+            seen += int((want != 0).sum())
+    assert seen > 100000
+
+
 @pytest.mark.parametrize("seed,steps", [(17, 400), (4242, 400)])
 def test_host_build_of_the_step_on_every_floor(seed, steps):
     """The same comparison from states on all nine floors with full inventories, armour,
