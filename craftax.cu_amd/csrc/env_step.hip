@@ -487,6 +487,9 @@ __global__ __launch_bounds__(kWave) void k_env_step(EnvArrays A, const float* __
     const int lane = threadIdx.x;
     const size_t e = (size_t)blockIdx.x * kWave + lane;
     const size_t n = (size_t)A.n;
+    // env counts are multiples of 32: the last wavefront may run half empty (the wavefront-wide
+    // votes below count the lanes that are there)
+    if (e >= n) return;
 
     Hot h;
     load_hot_dev(A, e, h);
@@ -877,7 +880,8 @@ int cfp_env_light_table(float* out, int count) {
 int cfp_env_create(cfp_env** out, int n, int pool) {
     CFP_REQUIRE(out != nullptr, "cfp_env_create: NULL out");
     *out = nullptr;
-    CFP_REQUIRE(n > 0 && n % cfp::kWave == 0, "cfp_env_create: env count %d is not a positive multiple of 64", n);
+    // the reference's own constraint (--envs a multiple of 32, craftax_full.cu:11820), the policy's too
+    CFP_REQUIRE(n > 0 && n % 32 == 0, "cfp_env_create: env count %d is not a positive multiple of 32", n);
     CFP_REQUIRE(pool >= 0, "cfp_env_create: pool size %d is negative", pool);
     cfp_env* e = new cfp_env();
     memset(&e->live, 0, sizeof(e->live));
@@ -960,7 +964,7 @@ int cfp_env_step(cfp_env* e, const float* d_actions, float* d_rewards, float* d_
     CFP_REQUIRE(e != nullptr && d_rewards != nullptr && d_terminals != nullptr, "cfp_env_step: NULL argument");
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(cfp::k_env_zero, dim3(1), dim3(1), 0, st, e->reset_count);
-    hipLaunchKernelGGL(cfp::k_env_step, dim3(e->live.n / cfp::kWave), dim3(cfp::kWave), 0, st, e->live, e->light, d_actions,
+    hipLaunchKernelGGL(cfp::k_env_step, dim3((e->live.n + cfp::kWave - 1) / cfp::kWave), dim3(cfp::kWave), 0, st, e->live, e->light, d_actions,
                        d_rewards, d_terminals, e->resets, e->reset_count);
     CFP_HIP_TRY(hipGetLastError());
     return 0;

@@ -101,7 +101,7 @@ typedef struct cfp_env_reset_rec {
 typedef struct cfp_env cfp_env;
 
 /* cu_vec_init without its worldgen (craftax_full.cu:10732-10880): allocates the device
- * arrays of `n` envs (a multiple of 64) and of `pool` reset states (0 = none), zeroed,
+ * arrays of `n` envs (a multiple of 32, as the reference asks of --envs) and of `pool` reset states (0 = none), zeroed,
  * and uploads the light-level table.  No env is playable before cfp_env_import. */
 int cfp_env_create(cfp_env** out, int n, int pool);
 void cfp_env_destroy(cfp_env* e);

@@ -68,6 +68,14 @@ def test_env_step_matches_reference_256x600(pkg, cuda, ref):
     assert seen > 0   # the run went through episode ends
 
 
+def test_env_step_with_a_half_empty_wavefront(pkg, cuda, ref):
+    """Env counts are multiples of 32 like the reference's --envs (craftax_full.cu:11820): 96 envs
+    are one full wavefront of the step kernel and one with 32 lanes, whose votes, shuffles and
+    spawn passes run over the lanes that exist."""
+    seen = _rollout(pkg, ref, 96, 300, 11, own_actions=False)
+    assert seen > 0
+
+
 def test_env_step_own_action_stream(pkg, cuda, ref):
     """The kernel's own xorshift32 % 43 stream (d_actions = NULL) is the reference's."""
     _rollout(pkg, ref, 64, 200, 7, own_actions=True)
@@ -182,7 +190,7 @@ def test_collect_regenerating_worlds(pkg, cuda, ref):
     from the same keys: every step's observations, rewards and done flags are the slabs', and
     the final states agree."""
     import ctypes as C
-    n, T, seed = 128, 48, 9
+    n, T, seed = 96, 48, 9      # one and a half wavefronts of the step kernel, three tiles of the policy
     ref.init(n, seed)
     states = ref.export()
     weak = states.copy()
