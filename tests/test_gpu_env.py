@@ -76,6 +76,32 @@ def test_env_step_with_a_half_empty_wavefront(pkg, cuda, ref):
     assert seen > 0
 
 
+def test_env_calls_reject_bad_arguments(pkg, cuda):
+    """The reference exits on a bad --envs (craftax_full.cu:11820-11825); a library returns an
+    error and says why.  No kernel is launched by any of these calls."""
+    err = pkg._lib.CfpError
+    for n in (0, -32, 33, 48):
+        with pytest.raises(err, match="multiple of 32"):
+            pkg.Env(n)
+    with pytest.raises(err, match="negative"):
+        pkg.Env(64, pool=-1)
+    env = pkg.Env(64)
+    states = np.zeros(4, eb.STATE_DTYPE)
+    with pytest.raises(err, match="outside"):
+        env.import_states(states, first=62)
+    with pytest.raises(err, match="outside"):
+        env.export_states(eb.STATE_DTYPE, first=60, count=8)
+    with pytest.raises(err, match="without a reset pool"):
+        env.reset_from_pool()
+    with pytest.raises(err, match="without a reset pool"):
+        env.pool_fill(0)
+    pol = pkg.Policy(96, layers=1, seed=1)
+    tr = pkg.Trainer(pol, 4)
+    with pytest.raises(err, match="holds 64 envs"):
+        env.rollout_step(tr, 0, 1)
+    tr.close(); pol.close(); env.close()
+
+
 def test_env_step_own_action_stream(pkg, cuda, ref):
     """The kernel's own xorshift32 % 43 stream (d_actions = NULL) is the reference's."""
     _rollout(pkg, ref, 64, 200, 7, own_actions=True)
