@@ -328,3 +328,29 @@ def test_record_obs_from_reference_soa_layout(pkg, cuda, golden):
     got4 = rec4.cpu().numpy()
     assert np.array_equal(got4[[3, 9]], want[[3, 9]])
     assert np.all(np.delete(got4, [3, 9], axis=0) == 0xEE)
+
+
+def test_record_obs_soa_above_the_small_batch_threshold(pkg, cuda, golden):
+    """Up to 16 384 envs the SoA kernel gathers 16 envs a round, above that 32 (a 128-byte line
+    of every field array): the fuzzed reference states tiled to 18 432 envs, every record
+    against the golden bytes, dense and through a list of all envs in reverse order."""
+    import torch
+    reps = 48
+    sc = np.tile(golden["fuzz_scalars"], (reps, 1))
+    pl = np.tile(golden["fuzz_planes"], (reps, 1, 1))
+    want = np.tile(golden["fuzz_records"], (reps, 1))
+    n = sc.shape[0]
+    assert n > 16384
+    n_stride = n + 32
+    arrays = {k: _t(v, cuda) for k, v in _soa_from_scalars(pkg, sc, n_stride, 12).items()}
+    planes = _t(pl, cuda).view(-1)
+    rec = pkg.policy.record_obs_soa(arrays, n_stride, planes, planes[P:], planes[2 * P:], n, 3 * P, 0)
+    torch.cuda.synchronize()
+    bad = np.nonzero((rec.cpu().numpy() != want).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} of {n} records differ, first {bad[:5]}"
+    rec2 = torch.full((n, 996), 0xEE, dtype=torch.uint8, device=cuda)
+    order = torch.arange(n - 1, -1, -1, dtype=torch.int32, device=cuda)
+    pkg.policy.record_obs_soa_list(arrays, n_stride, planes, planes[P:], planes[2 * P:], n, 3 * P, 0,
+                                   order, 4, torch.tensor([n], dtype=torch.int32, device=cuda), n, rec2)
+    torch.cuda.synchronize()
+    assert np.array_equal(rec2.cpu().numpy(), want)
