@@ -396,3 +396,43 @@ def test_closed_loop_with_device_resets(pkg, cuda, ref):
                     resynced += 1
                     env.import_states(fresh[k:k + 1], first=int(e))
     assert resets > 100 and resynced <= 1, (resets, resynced)
+
+
+def test_list_reset_in_a_large_env_vector(pkg, cuda):
+    """Above 16 384 envs cfp_env_reset runs the world generator with 256 threads a floor (below,
+    with 512): 16 448 envs made by cfp_env_init, a few hundred of them weakened so that they
+    starve within sixty steps, every regenerated env against the host build of the same
+    generator from the same reset key, and a sample of the initial worlds likewise."""
+    n, seed = 16384 + 64, 5
+    host = eb.HostStep()
+    env = pkg.Env(n)
+    env.init(seed)
+    for e in (0, 1, 4097, n - 1):
+        want = host.generate(seed + e, 1)
+        assert not eb.diff_fields(want, env.export_states(eb.STATE_DTYPE, first=e, count=1)), f"initial world {e}"
+    weak_envs = list(range(3, n, 53))
+    for k, e in enumerate(weak_envs):
+        st = env.export_states(eb.STATE_DTYPE, first=e, count=1)
+        st["player_health"] = 1.0 + (k % 4)
+        st["player_food"] = 0
+        st["player_drink"] = 0
+        st["player_recover"] = -14.0 + (k % 7)
+        env.import_states(st, first=e)
+    noop = torch.zeros(n, device=cuda)
+    compared = 0
+    for t in range(60):
+        env.step(noop)
+        cnt, recs = env.reset_list()
+        if not cnt:
+            continue
+        before = {int(r[0]): env.export_states(eb.STATE_DTYPE, first=int(r[0]), count=1) for r in recs}
+        env.reset()
+        for r in recs:
+            e = int(r[0])
+            st = before[e]
+            host.lib.cfhost_reset(eb.ptr(st), eb.ptr(np.ascontiguousarray(r[1:3]).view(np.uint32)))
+            got = env.export_states(eb.STATE_DTYPE, first=e, count=1)
+            assert not eb.diff_fields(st, got), f"step {t}: regenerated env {e}: {eb.diff_fields(st, got)}"
+            compared += 1
+    assert compared >= 100, compared
+    env.close()
