@@ -485,7 +485,7 @@ def train_iteration(pkg, torch, reps):
     it (README.md:348-356, horizon 128): cfp_train_collect (T rollout steps with the env, the
     bootstrap value, GAE) followed by cfp_train_update (backward + Adam, captured graph)."""
     out = {"workload": "train_iteration", "policy": "h256x3", "cases": {}}
-    for n, T in ((4096, 128), (8192, 128), (65536, 64)):
+    for n, T in ((1024, 128), (4096, 128), (8192, 128), (16384, 128), (65536, 128)):
         env = pkg.Env(n)
         env.init(0)
         for _ in range(300):          # spread the episodes' phases (random actions) before timing
