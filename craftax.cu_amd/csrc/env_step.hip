@@ -23,6 +23,7 @@
 // 64-byte sector each); it is latency- and divergence-bound, not HBM-bound.
 #include "cfp_common.h"
 #include "env_host.h"
+#include "env_internal.h"
 
 #include <mutex>
 #include <vector>
@@ -482,7 +483,8 @@ __device__ __forceinline__ void run_spawns_lanes(DevStore& s, const Hot& h, cons
 __global__ __launch_bounds__(kWave) void k_env_step(EnvArrays A, const float* __restrict__ light,
                                                     const float* __restrict__ actions, float* __restrict__ rewards,
                                                     float* __restrict__ terminals, cfp_env_reset_rec* __restrict__ resets,
-                                                    int* __restrict__ reset_count) {
+                                                    int* __restrict__ reset_count, float* __restrict__ r_reward_row,
+                                                    uint8_t* __restrict__ r_done_row) {
     __shared__ uint32_t lds[kLdsWords * kWave];
     const int lane = threadIdx.x;
     const size_t e = (size_t)blockIdx.x * kWave + lane;
@@ -515,6 +517,10 @@ __global__ __launch_bounds__(kWave) void k_env_step(EnvArrays A, const float* __
     A.rng_key[n + e] = (uint32_t)(keys.env_key >> 32);
     rewards[e] = out.reward;
     terminals[e] = out.done ? 1.0f : 0.0f;
+    if (r_reward_row != nullptr) {   // a trainer's slab rows (k_record_rd, craftax_full.cu:9758-9767)
+        r_reward_row[e] = out.reward;
+        r_done_row[e] = out.done ? 1 : 0;
+    }
 
     // done list: one atomic per wavefront
     const unsigned long long done = __ballot(out.done);
@@ -965,7 +971,7 @@ int cfp_env_step(cfp_env* e, const float* d_actions, float* d_rewards, float* d_
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(cfp::k_env_zero, dim3(1), dim3(1), 0, st, e->reset_count);
     hipLaunchKernelGGL(cfp::k_env_step, dim3((e->live.n + cfp::kWave - 1) / cfp::kWave), dim3(cfp::kWave), 0, st, e->live, e->light, d_actions,
-                       d_rewards, d_terminals, e->resets, e->reset_count);
+                       d_rewards, d_terminals, e->resets, e->reset_count, (float*)nullptr, (uint8_t*)nullptr);
     CFP_HIP_TRY(hipGetLastError());
     return 0;
 }
@@ -1140,3 +1146,22 @@ int cfp_env_record_obs(const cfp_env* e, uint8_t* d_rec_row, void* stream) {
 }
 
 }  // extern "C"
+
+int cfp::env_record_obs_zero(const cfp_env* e, uint8_t* d_rec_row, void* stream) {
+    CFP_REQUIRE(e != nullptr && d_rec_row != nullptr, "env_record_obs_zero: NULL argument");
+    cfp_env_soa soa;
+    const uint8_t *m, *im, *lm;
+    size_t es, ls;
+    if (cfp_env_view(e, &soa, &m, &im, &lm, &es, &ls)) return 1;
+    return cfp::record_obs_soa_zero(&soa, m, im, lm, es, ls, d_rec_row, e->live.n, e->reset_count, stream);
+}
+
+int cfp::env_step_rows(cfp_env* e, float* d_r_reward_row, uint8_t* d_r_done_row, void* stream) {
+    CFP_REQUIRE(e != nullptr && d_r_reward_row != nullptr && d_r_done_row != nullptr, "env_step_rows: NULL argument");
+    const size_t n = (size_t)e->live.n;
+    hipLaunchKernelGGL(cfp::k_env_step, dim3((e->live.n + cfp::kWave - 1) / cfp::kWave), dim3(cfp::kWave), 0,
+                       (hipStream_t)stream, e->live, e->light, e->slots, e->slots + n, e->slots + 2 * n, e->resets,
+                       e->reset_count, d_r_reward_row, d_r_done_row);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}

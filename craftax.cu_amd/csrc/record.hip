@@ -11,6 +11,7 @@
 #include <cstring>
 
 #include "cfp_common.h"
+#include "env_internal.h"
 
 namespace cfp {
 namespace {
@@ -156,6 +157,7 @@ struct RecWhich {
     size_t list_stride;
     const int* count;
     int max_count;   // the list form never reads past this many entries, whatever *count says
+    int* zero;       // not null: the first thread of the launch stores 0 there
 };
 
 constexpr int kWPos = (int)(offsetof(cfp_env_scalars, player_position) / 4);
@@ -195,6 +197,7 @@ __global__ __launch_bounds__(256) void k_record_obs(
     __shared__ SoaWord words[SOA ? kScalarWords : 1];
     const int lane = threadIdx.x % kRecLanes;
     const int slot = threadIdx.x / kRecLanes;
+    if (which.zero != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *which.zero = 0;
     if (SOA) {
 #pragma unroll
         for (int i = 0; i < kSoaPtrs; i++)
@@ -624,6 +627,19 @@ int cfp_record_obs_soa_list(const cfp_env_soa* soa, const uint8_t* d_map,
     return record_obs_soa(soa, d_map, d_item_map, d_light_map, env_stride, level_stride, w,
                           max_count, d_rec_row, n, stream);
 }
+
+}  // extern "C"
+
+int cfp::record_obs_soa_zero(const cfp_env_soa* soa, const uint8_t* d_map, const uint8_t* d_item_map,
+                             const uint8_t* d_light_map, size_t env_stride, size_t level_stride,
+                             uint8_t* d_rec_row, int n, int* d_zero, void* stream) {
+    RecWhich w{};
+    w.zero = d_zero;
+    return record_obs_soa(soa, d_map, d_item_map, d_light_map, env_stride, level_stride, w, n,
+                               d_rec_row, n, stream);
+}
+
+extern "C" {
 
 int cfp_expand_obs(const uint8_t* d_r_obs, float* d_xobs, int t0, int count,
                    int mb, int n, int env_start, void* stream) {

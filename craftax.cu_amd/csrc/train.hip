@@ -15,6 +15,7 @@
 #include "cfp_internal.h"
 #include "ppo_kernels.h"
 #include "../../include/cfp_env.h"
+#include "env_internal.h"
 
 namespace cfp {
 namespace {
@@ -433,10 +434,13 @@ int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void
     CFP_REQUIRE(t >= 0 && t < tr->T, "step %d outside the horizon %d", t, tr->T);
     const size_t o = (size_t)t * tr->n;
     uint8_t* row = tr->r_obs + o * CFP_REC_BYTES;
-    if (cfp_env_record_obs(e, row, stream)) return 1;
+    // cfp_env_record_obs, cfp_rollout_step, cfp_env_step, cfp_record_rd, reset -- with the two
+    // one-line kernels of that sequence folded into their neighbours: the record kernel leaves the
+    // finished-env counter at zero for the step, the step writes rewards and done flags into the
+    // slab rows as well (two launches of ~5 us less per step, 6 % of a step at 4096 envs)
+    if (cfp::env_record_obs_zero(e, row, stream)) return 1;
     if (cfp_rollout_step(tr, t, row, cfp_env_terminals(e), seed, cfp_env_actions(e), stream)) return 1;
-    if (cfp_env_step(e, cfp_env_actions(e), cfp_env_rewards(e), cfp_env_terminals(e), stream)) return 1;
-    if (cfp_record_rd(cfp_env_rewards(e), cfp_env_terminals(e), tr->r_reward + o, tr->r_done + o, tr->n, stream)) return 1;
+    if (cfp::env_step_rows(e, tr->r_reward + o, tr->r_done + o, stream)) return 1;
     return cfp_env_pool_size(e) > 0 ? cfp_env_reset_from_pool(e, stream) : cfp_env_reset(e, stream);
 }
 
