@@ -27,6 +27,7 @@
 // The last map bytes (768..791) and the 51 fp32 features go through the fp32 GEMM as
 // a 75-row operand (k_expand_obs_tail + gemm_dw_ld).
 #include "policy_tile.h"
+#include "ppo_kernels.h"
 
 namespace cfp {
 namespace {
@@ -235,9 +236,19 @@ __global__ void k_expand_obs_tail(const uint8_t* __restrict__ r_obs, f4* __restr
 
 bool dw_enc_records_ok(int mb) { return mb > 0 && mb % 8 == 0; }
 
-int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
-                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
-                   bool dh_bf16, const SeamWork* sw_tail, hipStream_t st_tail) {
+int dw_enc_tail_expand(const uint8_t* r_obs, float* tail_scratch, int t0, int cols, int mb, int n_all,
+                       int env_start, hipStream_t st) {
+    CFP_REQUIRE(r_obs && tail_scratch && cols > 0 && dw_enc_records_ok(mb), "dw_enc_tail_expand: bad argument");
+    const size_t total4 = (size_t)cols * (kEgTailLd / 4);
+    hipLaunchKernelGGL(k_expand_obs_tail, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, st, r_obs,
+                       reinterpret_cast<f4*>(tail_scratch), t0, total4, mb, n_all, env_start);
+    CFP_HIP_TRY(hipGetLastError());
+    return 0;
+}
+
+static int dw_enc_records_impl(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
+                               int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
+                               bool dh_bf16, const SeamWork* sw_tail, hipStream_t st_tail, bool tail_ready) {
     CFP_REQUIRE(r_obs && dh && dW && tail_scratch && cols > 0 && dw_enc_records_ok(mb) &&
                     cols % 8 == 0,
                 "dw_enc_records: columns and envs per minibatch must be multiples of 8");
@@ -269,15 +280,24 @@ int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail
     // workspace when the caller has one to spare
     const SeamWork& swt = sw_tail ? *sw_tail : sw;
     hipStream_t stt = sw_tail ? st_tail : st;
-    const size_t total4 = (size_t)cols * (kEgTailLd / 4);
-    hipLaunchKernelGGL(k_expand_obs_tail, dim3((unsigned)((total4 + 255) / 256)), dim3(256), 0, stt,
-                       r_obs, reinterpret_cast<f4*>(tail_scratch), t0, total4, mb, n_all,
-                       env_start);
-    CFP_HIP_TRY(hipGetLastError());
+    if (!tail_ready && dw_enc_tail_expand(r_obs, tail_scratch, t0, cols, mb, n_all, env_start, stt)) return 1;
     if (dh_bf16)   // dh is the 256-wide operand of this GEMM, the 75 tail features its rows
         return gemm_dw_x9(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, 1, swt, stt, 0,
                           nullptr, false, true);
     return gemm_dw_ld(kEgTail, cols, dh, tail_scratch, kEgTailLd, dW + count, swt, stt);
+}
+
+int dw_enc_records(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
+                   int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
+                   bool dh_bf16, const SeamWork* sw_tail, hipStream_t st_tail) {
+    return dw_enc_records_impl(r_obs, dh, dW, tail_scratch, t0, cols, mb, n_all, env_start, sw, st, dh_bf16,
+                               sw_tail, st_tail, false);
+}
+int dw_enc_records_tail_ready(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
+                              int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
+                              bool dh_bf16, const SeamWork* sw_tail, hipStream_t st_tail) {
+    return dw_enc_records_impl(r_obs, dh, dW, tail_scratch, t0, cols, mb, n_all, env_start, sw, st, dh_bf16,
+                               sw_tail, st_tail, true);
 }
 
 }  // namespace cfp

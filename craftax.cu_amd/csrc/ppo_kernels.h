@@ -85,4 +85,13 @@ int launch_adv_moments(const float* adv, size_t count, double* part, double* mom
 int launch_adam(cfp_policy* p, float* grads, float* m, float* v, const uint64_t* step_ctr,
                 const float* lr, float beta1, float beta2, float eps, hipStream_t st);
 
+// dW_enc from the records (enc_grad.hip) with the fp32 rows of its 75-feature remainder made
+// ahead of time: the expansion depends on the records only, so the update asks for it at the
+// start of a window, next to the recompute, instead of at the end of the dependent chain.
+int dw_enc_tail_expand(const uint8_t* r_obs, float* tail_scratch, int t0, int cols, int mb, int n_all,
+                       int env_start, hipStream_t st);
+int dw_enc_records_tail_ready(const uint8_t* r_obs, const float* dh, float* dW, float* tail_scratch, int t0,
+                              int cols, int mb, int n_all, int env_start, const SeamWork& sw, hipStream_t st,
+                              bool dh_bf16, const SeamWork* sw_tail, hipStream_t st_tail);
+
 }  // namespace cfp

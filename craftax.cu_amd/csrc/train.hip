@@ -591,6 +591,12 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
             fa.tr_t0 = t0; fa.tr_mb = mb; fa.tr_n_all = n; fa.tr_env_start = env_start;
             for (int l = 0; l < L; l++) fa.tr_pre[l] = tr->preb[l];
             for (int l = 0; l <= L; l++) fa.tr_x[l] = tr->x[l];
+            // the fp32 rows of dW_enc's 75-feature remainder depend on the records only: made here
+            // (40 us alone) instead of behind the last GEMMs of the chain, where the same kernel
+            // shares the GPU and takes 190 us on the critical path; xobs is free in this mode
+            if (dw_enc_records_ok(mb) &&
+                dw_enc_tail_expand(tr->r_obs, tr->xobs, t0, cols, mb, n, env_start, st))
+                return 1;
             if (launch_forward(fa, st)) return 1;
             // without the record-fed dW_enc kernel the reverse pass reads the fp32
             // feature matrix
@@ -709,9 +715,12 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         if (dw_enc_records_ok(mb)) {
             // map bytes straight from the records; xobs is free by now and takes the
             // 76-float rows of the fp32 remainder
-            if (dw_enc_records(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
-                               env_start, tr->sw, chain, st16, overlap ? &tr->sw_layer[0] : nullptr,
-                               other))
+            if (fused ? dw_enc_records_tail_ready(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
+                                                  env_start, tr->sw, chain, st16,
+                                                  overlap ? &tr->sw_layer[0] : nullptr, other)
+                      : dw_enc_records(tr->r_obs, tr->dhX, g + CFP_OFF_W_ENC, tr->xobs, t0, cols, mb, n,
+                                       env_start, tr->sw, chain, st16, overlap ? &tr->sw_layer[0] : nullptr,
+                                       other))
                 return 1;
         } else if (gemm_dw_ld(CFP_OBS, cols, tr->dhX, tr->xobs, kObsPad, g + CFP_OFF_W_ENC, tr->sw,
                               chain)) {
