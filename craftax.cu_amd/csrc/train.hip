@@ -639,11 +639,6 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
         const int terms = gemm_split_terms();
         const bool overlap = terms >= 1 && gemm_dw_x9_ok(G, cols);
         hipStream_t hs = st;
-        if (overlap) {
-            CFP_HIP_TRY(hipEventRecord(tr->ev_head, st));
-            CFP_HIP_TRY(hipStreamWaitEvent(tr->st2, tr->ev_head, 0));
-            hs = tr->st2;
-        }
         // (bf16 storage: the three dh buffers hold bf16 as well)
         if (st16) {
             if (gemm_dh_x9(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, 1,
@@ -651,6 +646,14 @@ int cfp_train_backward(cfp_trainer* tr, int env_start, int env_count, void* stre
                 return 1;
         } else if (gemm_dh_acc(kHeadLd, cols, tr->w_head, tr->dlogits, tr->dh3b, false, tr->sw, st)) {
             return 1;
+        }
+        // the second stream starts behind dh3: next to it the heads' dW doubled its time (90 ->
+        // 190 us) with the top layer's sweep waiting; under that sweep, which is bound by memory,
+        // the same GEMM costs little
+        if (overlap) {
+            CFP_HIP_TRY(hipEventRecord(tr->ev_head, st));
+            CFP_HIP_TRY(hipStreamWaitEvent(tr->st2, tr->ev_head, 0));
+            hs = tr->st2;
         }
         if (st16) {
             if (gemm_dw_x9(A + 1, cols, tr->x[L], tr->dlogits, kHeadLd, g + CFP_OFF_W_A(L), 1, tr->sw,
