@@ -128,7 +128,7 @@ def ppo_update(pkg, torch, reps):
            "tflops": UPD_FLOP * samples / ms / 1e9,
            "frac_fp32_mfma_peak": UPD_FLOP * samples / ms / 1e9 / PEAK_FP32}
     # same update with the GEMMs as fp32 MFMA (mode 0) and as six partial products (mode 2)
-    for mode, key in ((0, "fp32_mfma_gemms"), (2, "split6_gemms")):
+    for mode, key in ((0, "fp32_mfma_gemms"), (2, "split6_gemms"), (3, "split8_gemms")):
         pkg.policy.set_gemm_split(mode)
         try:
             ms_m = _time(torch, step, reps, warm=1)

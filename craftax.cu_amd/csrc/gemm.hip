@@ -379,7 +379,7 @@ thread_local int t_gemm_bf16 = -1, t_gemm_split = -1;
 inline int eff_bf16() { return t_gemm_bf16 >= 0 ? t_gemm_bf16 : g_gemm_bf16; }
 inline int eff_split() { return t_gemm_split >= 0 ? t_gemm_split : g_gemm_split; }
 // partial products per product on those kernels: bf16 inputs -> 1 (rounded operands)
-inline int split_terms() { return eff_bf16() ? 1 : (eff_split() == 2 ? 6 : 9); }
+inline int split_terms() { return eff_bf16() ? 1 : (eff_split() == 2 ? 6 : (eff_split() == 3 ? 8 : 9)); }
 
 template <bool A_KFAST, bool B_KFAST, bool ACCUM>
 int launch_gemm(const GemmArgs& g, dim3 grid, bool va, bool vb, hipStream_t st) {
@@ -570,7 +570,7 @@ int cfp_set_gemm_bf16(int on) {
 }
 int cfp_get_gemm_bf16(void) { return g_gemm_bf16; }
 int cfp_set_gemm_split(int mode) {
-    CFP_REQUIRE(mode >= 0 && mode <= 2, "cfp_set_gemm_split: mode must be 0, 1 or 2 (got %d)", mode);
+    CFP_REQUIRE(mode >= 0 && mode <= 3, "cfp_set_gemm_split: mode must be 0..3 (got %d)", mode);
     g_gemm_split = mode;
     return 0;
 }

@@ -7,7 +7,8 @@
 // with one accumulator rounding per 16 products instead of per 2 -- and take 9/16 of
 // its pipe time.  The reference runs these GEMMs as cublasSgemm behind cu_gemm_dw
 // and cu_gemm_dh (craftax_full.cu:11642-11666).
-// TERMS = 6 leaves out mid*lo, lo*mid and lo*lo: with truncated parts |mid| < 2^-7 |a|
+// TERMS = 8 leaves out lo*lo alone (|lo| < 2^-15 |a| with truncated parts: below 2^-30 of a
+// product).  TERMS = 6 leaves out mid*lo, lo*mid and lo*lo: with truncated parts |mid| < 2^-7 |a|
 // and |lo| < 2^-15 |a|, so at most 2^-21 of |a*b| per product (about 2^-24 on average,
 // always towards zero), the size of the roundings the fp32 accumulation of those
 // products makes anyway, for two thirds of the MFMAs.  Opt-in.
@@ -38,7 +39,7 @@ static __device__ __align__(256) unsigned char scratch[(CFP_GRU / 16) * 24 * 64 
 namespace cfp {
 namespace {
 
-// The operand parts a kernel multiplies: TERMS = 9 or 6 -> the exact triple; TERMS = 1 ->
+// The operand parts a kernel multiplies: TERMS = 9, 8 or 6 -> the exact triple; TERMS = 1 ->
 // the operand rounded to bf16 (the bf16-input mode of the seam), one product.
 template <int TERMS>
 __device__ __forceinline__ void parts_of(const float (&v)[8], u4 (&p)[3]) {
@@ -52,7 +53,7 @@ __device__ __forceinline__ void parts_of(const float (&v)[8], u4 (&p)[3]) {
 }
 template <int TERMS>
 __device__ __forceinline__ constexpr bool term_used(int i, int j) {
-    return TERMS == 9 || (TERMS == 6 && i + j <= 2) || (TERMS == 1 && i == 0 && j == 0);
+    return TERMS == 9 || (TERMS == 8 && i + j <= 3) || (TERMS == 6 && i + j <= 2) || (TERMS == 1 && i == 0 && j == 0);
 }
 
 constexpr int kX9Threads = 512;
@@ -592,6 +593,8 @@ static int launch_dh_x9(int K, int cols, const float* B, long sk, long su, const
         hipLaunchKernelGGL(k_dh_x9<1>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     else if (terms == 6)
         hipLaunchKernelGGL(k_dh_x9<6>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
+    else if (terms == 8)
+        hipLaunchKernelGGL(k_dh_x9<8>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     else
         hipLaunchKernelGGL(k_dh_x9<9>, grid, dim3(kDhThreads), 0, st, A, K, g_w_x9, out, ldc, cols, acc, 0, 0);
     CFP_HIP_TRY(hipGetLastError());
@@ -620,6 +623,9 @@ int gemm_enc_fwd_x9(int cols, const float* W_enc, const float* xobs, int ldx, fl
                            CFP_HIDDEN, cols, 0, ldx, CFP_OBS);
     else if (terms == 6)
         hipLaunchKernelGGL((k_dh_x9<6, false, false, true>), grid, dim3(kDhThreads), 0, st, xobs, kEncK, enc_mirror, h,
+                           CFP_HIDDEN, cols, 0, ldx, CFP_OBS);
+    else if (terms == 8)
+        hipLaunchKernelGGL((k_dh_x9<8, false, false, true>), grid, dim3(kDhThreads), 0, st, xobs, kEncK, enc_mirror, h,
                            CFP_HIDDEN, cols, 0, ldx, CFP_OBS);
     else
         hipLaunchKernelGGL((k_dh_x9<9, false, false, true>), grid, dim3(kDhThreads), 0, st, xobs, kEncK, enc_mirror, h,
@@ -738,6 +744,9 @@ int gemm_dw_x9(int rows, int cols, const float* x, const float* dpre, int ld_dpr
                            work, cols, ips, n_wg, groups);
     else if (terms == 6)
         hipLaunchKernelGGL(k_dw_x9<6>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
+                           work, cols, ips, n_wg, groups);
+    else if (terms == 8)
+        hipLaunchKernelGGL(k_dw_x9<8>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,
                            work, cols, ips, n_wg, groups);
     else
         hipLaunchKernelGGL(k_dw_x9<9>, dim3(grid), dim3(kX9Threads), 0, st, dpre, ld_dpre, rows, x,

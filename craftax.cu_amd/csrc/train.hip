@@ -369,7 +369,7 @@ int cfp_train_profile(cfp_trainer* tr, double* ms4, int reset) {
 
 int cfp_train_set_gemm_mode(cfp_trainer* tr, int bf16, int split) {
     CFP_REQUIRE(tr, "cfp_train_set_gemm_mode: NULL trainer");
-    CFP_REQUIRE(bf16 >= -1 && bf16 <= 1 && split >= -1 && split <= 2,
+    CFP_REQUIRE(bf16 >= -1 && bf16 <= 1 && split >= -1 && split <= 3,
                 "cfp_train_set_gemm_mode: bf16 must be -1, 0 or 1 and split -1, 0, 1 or 2 (got %d, %d)", bf16, split);
     tr->gemm_bf16 = bf16;
     tr->gemm_split = split;

@@ -222,9 +222,11 @@ int cfp_get_gemm_bf16(void);
  * cfp_gemm_dh for the shapes of the PPO update when bf16 inputs are off; other shapes
  * take the fp32 MFMA kernel.  mode 1 (default): all nine partial products; mode 2: the
  * six largest (mid*lo, lo*mid, lo*lo left out: at most 2^-21 of |a*b| per product,
- * about 2^-24 on average, the size of the roundings of the fp32 accumulation; opt-in); mode 0: fp32 MFMA everywhere (and, with bf16
- * inputs on, the generic bf16 kernel).  With cfp_set_gemm_bf16(1) and mode 1 or 2 the same
- * kernels run with both operands rounded to bf16 and one product. */
+ * about 2^-24 on average, the size of the roundings of the fp32 accumulation; opt-in); mode 3:
+ * eight (only lo*lo left out: below 2^-30 of |a*b| per product, 1/64 of one rounding of the
+ * fp32 accumulator; opt-in); mode 0: fp32 MFMA everywhere (and, with bf16 inputs on, the generic
+ * bf16 kernel).  With cfp_set_gemm_bf16(1) and mode 1, 2 or 3 the same kernels run with both
+ * operands rounded to bf16 and one product. */
 int cfp_set_gemm_split(int mode);
 int cfp_get_gemm_split(void);
 
@@ -477,7 +479,7 @@ int cfp_train_profile(cfp_trainer* tr, double* ms4, int reset);
 /* GEMM mode of one trainer's update.  The reference has one process-wide switch
  * (g_gemm_bf16, craftax_full.cu:11306-11316) and one trainer per process; here two trainers
  * may live in one process, each with a captured update graph, so a trainer can carry its own
- * mode: bf16 = 0 / 1 and split = 0 / 1 / 2 as in cfp_set_gemm_bf16 / cfp_set_gemm_split, or
+ * mode: bf16 = 0 / 1 and split = 0 / 1 / 2 / 3 as in cfp_set_gemm_bf16 / cfp_set_gemm_split, or
  * -1 to follow the process-wide switch (the default for both).  cfp_train_backward and
  * cfp_train_update run with the trainer's mode whatever the process-wide switches say, and
  * cfp_train_update's graph is captured again only when the trainer's effective mode changed.

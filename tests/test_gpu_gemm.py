@@ -61,15 +61,18 @@ def test_gemm_dw_accumulates(pkg, cuda, rows, cols):
 def _check_split_errors(errs):
     """errs[mode] = max |got - fp64| / sum_k |a_k b_k|.  Mode 1 (nine exact partial
     products) must sit at the fp32 MFMA kernel's level (mode 0); mode 2 (six) may add
-    its documented 2^-23 per product on top."""
+    its documented 2^-23 per product on top; mode 3 (eight: only lo*lo left out, below
+    2^-30 of a product) is held to the bar of mode 1."""
     assert errs[1] <= 3.0 * errs[0] + 1e-7, errs
     assert errs[1] < 2e-6, errs
+    assert errs[3] <= 3.0 * errs[0] + 1e-7 and errs[3] < 2e-6, errs
+    assert abs(errs[3] - errs[1]) <= 2.0 ** -28, errs
     assert errs[2] <= 3.0 * errs[0] + 1e-7 + 2.0 ** -23, errs
 
 
 def test_gemm_split_mode_is_checked(pkg, cuda):
-    with pytest.raises(pkg._lib.CfpError, match="mode must be 0, 1 or 2"):
-        pkg.policy.set_gemm_split(3)
+    with pytest.raises(pkg._lib.CfpError, match="mode must be 0..3"):
+        pkg.policy.set_gemm_split(4)
     assert pkg.policy.lib().cfp_get_gemm_split() == 1
 
 
@@ -85,7 +88,7 @@ def test_gemm_dw_split_is_as_accurate_as_fp32_mfma(pkg, cuda, rows, cols):
     scale = (d.double().abs().T @ x.double().abs())
     errs = {}
     assert pkg.policy.lib().cfp_get_gemm_split() == 1
-    for mode in (1, 2, 0):
+    for mode in (1, 2, 3, 0):
         pkg.policy.set_gemm_split(mode)
         dW = torch.zeros(rows, HIDDEN, device=cuda)
         pkg.policy.gemm_dw(x, d, dW)
@@ -105,7 +108,7 @@ def test_gemm_dh_split_is_as_accurate_as_fp32_mfma(pkg, cuda, m3, cols):
     want = d.double() @ W.double()
     scale = d.double().abs() @ W.double().abs()
     errs = {}
-    for mode in (1, 2, 0):
+    for mode in (1, 2, 3, 0):
         pkg.policy.set_gemm_split(mode)
         out = pkg.policy.gemm_dh(W, d)
         torch.cuda.synchronize()
@@ -122,7 +125,7 @@ def test_gemm_fwd_split_is_as_accurate_as_fp32_mfma(pkg, cuda, m, cols, k):
     want = x.double() @ W.double().T
     scale = x.double().abs() @ W.double().abs().T
     errs = {}
-    for mode in (1, 2, 0):
+    for mode in (1, 2, 3, 0):
         pkg.policy.set_gemm_split(mode)
         out = pkg.policy.gemm_fwd(W, x)
         torch.cuda.synchronize()
