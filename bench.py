@@ -104,7 +104,19 @@ def policy_in_the_loop(pkg, torch, n, steps):
     out = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3, "steps": steps,
            "finished_envs_last_step": env.reset_list()[0],
            "frac_fp32_peak_of_forward_flops": FLOP_PER_ENV_STEP * n / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
-           "what": "cfp_env_rollout_step: env, records, h256x3 policy, sampling and resets on the device"}
+           "what": "cfp_env_rollout_step: env, records, h256x3 policy, sampling and resets on the device, "
+                   "observations / states / actions / rewards recorded into a trainer's slabs"}
+    # the same step without the slabs (cfp_env_run_step = the reference's `run` mode)
+    e0.record()
+    for t in range(steps):
+        env.run_step(pol, 1234)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    out["run_mode"] = {"ms_per_step": ms, "env_steps_per_s": n / ms * 1e3,
+                       "frac_fp32_peak_of_forward_flops":
+                           FLOP_PER_ENV_STEP * n / (ms * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                       "what": "cfp_env_run_step: the same step with no slabs"}
     tr.close(); pol.close(); env.close()
     return out
 

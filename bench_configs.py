@@ -473,6 +473,11 @@ def rollout_in_the_loop(pkg, torch, reps):
             res[mode] = {"us_per_step": round(ms * 1e3, 1), "M_env_steps_per_s": round(n / ms / 1e3, 2),
                          "frac_fp32_peak_of_forward_flops": round(FWD_FLOP * n / (ms * 1e-3) / 1e12 / PEAK_FP32, 3),
                          "finished_envs_last_step": cnt}
+            # the same step without the trainer's slabs: cu_rollout_step_plain, what the reference's
+            # `run` mode times (craftax_full.cu:12089-12092, 12127-12176)
+            ms_run = _time(torch, lambda: env.run_step(pol, 1234), 64)
+            res[mode]["run_mode"] = {"us_per_step": round(ms_run * 1e3, 1), "M_env_steps_per_s": round(n / ms_run / 1e3, 2),
+                                     "frac_fp32_peak_of_forward_flops": round(FWD_FLOP * n / (ms_run * 1e-3) / 1e12 / PEAK_FP32, 3)}
             tr.close()
             pol.close()
             env.close()

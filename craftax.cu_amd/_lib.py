@@ -124,6 +124,11 @@ PROTOTYPES = {
     "cfp_env_rewards": (vp, [vp]),
     "cfp_env_terminals": (vp, [vp]),
     "cfp_env_rollout_step": (C.c_int, [vp, vp, C.c_int, C.c_uint64, vp]),
+    "cfp_env_run_step": (C.c_int, [vp, vp, C.c_uint64, vp]),
+    "cfp_env_run_actions": (vp, [vp]),
+    "cfp_env_run_logprobs": (vp, [vp]),
+    "cfp_env_run_values": (vp, [vp]),
+    "cfp_env_run_counter": (vp, [vp]),
     "cfp_train_collect": (C.c_int, [vp, vp, C.c_uint64, vp]),
 }
 

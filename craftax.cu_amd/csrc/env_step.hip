@@ -24,6 +24,7 @@
 #include "cfp_common.h"
 #include "env_host.h"
 #include "env_internal.h"
+#include "cfp_internal.h"
 
 #include <mutex>
 #include <vector>
@@ -865,6 +866,10 @@ struct cfp_env {
     cfp_env_reset_rec* resets = nullptr;
     int* reset_count = nullptr;
     float* slots = nullptr;   // actions | rewards | terminals, n floats each
+    // the `run` mode's outputs (CuPolicy.d_act / d_logprob / d_value and step_ctr,
+    // craftax_full.cu:11770-11773): sampled actions (int32) | log-probabilities | values, n each,
+    // then the 8-byte step counter of the draws and a zeroed word for the sampler's ticket
+    float* run = nullptr;
 };
 
 static_assert(sizeof(cfp_env_state) % 8 == 0, "exchange struct is 8-byte aligned");
@@ -915,6 +920,8 @@ int cfp_env_create(cfp_env** out, int n, int pool) {
     if ((err = hipMemset(e->reset_count, 0, sizeof(int))) != hipSuccess) return fail(err, "hipMemset(reset_count)");
     if ((err = hipMalloc((void**)&e->slots, sizeof(float) * 3 * (size_t)n)) != hipSuccess) return fail(err, "hipMalloc(slots)");
     if ((err = hipMemset(e->slots, 0, sizeof(float) * 3 * (size_t)n)) != hipSuccess) return fail(err, "hipMemset(slots)");
+    if ((err = hipMalloc((void**)&e->run, sizeof(float) * 3 * (size_t)n + 16)) != hipSuccess) return fail(err, "hipMalloc(run)");
+    if ((err = hipMemset(e->run, 0, sizeof(float) * 3 * (size_t)n + 16)) != hipSuccess) return fail(err, "hipMemset(run)");
     *out = e;
     return 0;
 }
@@ -927,6 +934,7 @@ void cfp_env_destroy(cfp_env* e) {
     (void)hipFree(e->resets);
     (void)hipFree(e->reset_count);
     (void)hipFree(e->slots);
+    (void)hipFree(e->run);
     delete e;
 }
 
@@ -935,6 +943,12 @@ float* cfp_env_actions(const cfp_env* e) { return e ? e->slots : nullptr; }
 float* cfp_env_rewards(const cfp_env* e) { return e ? e->slots + e->live.n : nullptr; }
 float* cfp_env_terminals(const cfp_env* e) { return e ? e->slots + 2 * (size_t)e->live.n : nullptr; }
 int cfp_env_pool_size(const cfp_env* e) { return e ? e->pool_size : 0; }
+int32_t* cfp_env_run_actions(const cfp_env* e) { return e ? reinterpret_cast<int32_t*>(e->run) : nullptr; }
+float* cfp_env_run_logprobs(const cfp_env* e) { return e ? e->run + e->live.n : nullptr; }
+float* cfp_env_run_values(const cfp_env* e) { return e ? e->run + 2 * (size_t)e->live.n : nullptr; }
+uint64_t* cfp_env_run_counter(const cfp_env* e) {
+    return e ? reinterpret_cast<uint64_t*>(e->run + 3 * (size_t)e->live.n) : nullptr;
+}
 
 int cfp_env_import(cfp_env* e, int first, int count, const cfp_env_state* states) {
     CFP_REQUIRE(e != nullptr && states != nullptr, "cfp_env_import: NULL argument");
@@ -1145,6 +1159,23 @@ int cfp_env_record_obs(const cfp_env* e, uint8_t* d_rec_row, void* stream) {
     return cfp_record_obs_soa(&soa, m, im, lm, es, ls, nullptr, d_rec_row, e->live.n, stream);
 }
 
+// cu_rollout_step_plain (craftax_full.cu:12089-12092): the step of the reference's `run` mode,
+// no slabs.  Records of the current states into the policy's own record buffer, forward on its
+// live state (zeroed where the last step ended an episode) and the draw, the env step with the
+// drawn actions, finished envs replaced.
+int cfp_env_run_step(cfp_policy* p, cfp_env* e, uint64_t seed, void* stream) {
+    CFP_REQUIRE(p != nullptr && e != nullptr, "cfp_env_run_step: NULL argument");
+    CFP_REQUIRE(p->n == e->live.n, "cfp_env_run_step: the policy holds %d envs, the env object %d", p->n, e->live.n);
+    CFP_REQUIRE(p->variant == 0, "cfp_env_run_step: the env on the device is the full game");
+    const size_t n = (size_t)e->live.n;
+    if (cfp::env_record_obs_zero(e, p->rec, stream)) return 1;
+    const cfp::SampleOut so{cfp_env_run_actions(e), cfp_env_run_logprobs(e), cfp_env_run_values(e), e->slots, seed,
+                            cfp_env_run_counter(e), reinterpret_cast<unsigned*>(cfp_env_run_counter(e) + 1)};
+    if (cfp::forward_and_sample(p, p->rec, e->slots + 2 * n, nullptr, e->live.n, so, (hipStream_t)stream)) return 1;
+    if (cfp::env_step_rows(e, nullptr, nullptr, stream)) return 1;
+    return e->pool_size > 0 ? cfp_env_reset_from_pool(e, stream) : cfp_env_reset(e, stream);
+}
+
 }  // extern "C"
 
 int cfp::env_record_obs_zero(const cfp_env* e, uint8_t* d_rec_row, void* stream) {
@@ -1157,7 +1188,7 @@ int cfp::env_record_obs_zero(const cfp_env* e, uint8_t* d_rec_row, void* stream)
 }
 
 int cfp::env_step_rows(cfp_env* e, float* d_r_reward_row, uint8_t* d_r_done_row, void* stream) {
-    CFP_REQUIRE(e != nullptr && d_r_reward_row != nullptr && d_r_done_row != nullptr, "env_step_rows: NULL argument");
+    CFP_REQUIRE(e != nullptr && (d_r_reward_row == nullptr) == (d_r_done_row == nullptr), "env_step_rows: bad argument");
     const size_t n = (size_t)e->live.n;
     hipLaunchKernelGGL(cfp::k_env_step, dim3((e->live.n + cfp::kWave - 1) / cfp::kWave), dim3(cfp::kWave), 0,
                        (hipStream_t)stream, e->live, e->light, e->slots, e->slots + n, e->slots + 2 * n, e->resets,

@@ -90,6 +90,19 @@ class Env:
         reward / done rows, pool reset."""
         _check(lib().cfp_env_rollout_step(trainer._h, self._h, t, seed, _stream()))
 
+    def run_step(self, policy, seed):
+        """cu_rollout_step_plain: the `run` mode's step (no slabs); results in run_actions /
+        run_logprobs / run_values."""
+        _check(lib().cfp_env_run_step(policy._h, self._h, seed, _stream()))
+
+    def run_outputs(self):
+        """(actions int32[n], logprobs f32[n], values f32[n], step counter u64[1]) of the run mode."""
+        n = self.n
+        return (_wrap(lib().cfp_env_run_actions(self._h), (n,), "<i4"),
+                _wrap(lib().cfp_env_run_logprobs(self._h), (n,), "<f4"),
+                _wrap(lib().cfp_env_run_values(self._h), (n,), "<f4"),
+                _wrap(lib().cfp_env_run_counter(self._h), (1,), "<i8"))
+
     def collect(self, trainer, seed):
         """cu_train_collect: T rollout steps, bootstrap value, GAE."""
         _check(lib().cfp_train_collect(trainer._h, self._h, seed, _stream()))

@@ -182,6 +182,18 @@ int cfp_env_record_obs(const cfp_env* e, uint8_t* d_rec_row, void* stream);
  * terminals into r_reward[t] / r_done[t], reset finished envs: from the pool when the env
  * object has one, with freshly generated worlds otherwise.  The trainer's env count must equal the env object's. */
 int cfp_env_rollout_step(cfp_trainer* tr, cfp_env* e, int t, uint64_t seed, void* stream);
+/* cu_rollout_step_plain (craftax_full.cu:12089-12092), the step of the reference's `run` mode
+ * (cu_run_rollout_bench, :12127-12176): the same sequence with no slabs -- records into the
+ * policy's own buffer, forward on its live state, the draw with offset *counter (then
+ * *counter += 1), the env step with the drawn actions, finished envs replaced.  The sampled
+ * actions (int32), log-probabilities and values of the step lie in the env object
+ * (CuPolicy.d_act / d_logprob / d_value, :11770-11773), as does the 8-byte device step counter
+ * of the draws, zero at cfp_env_create.  The policy's env count must equal the env object's. */
+int cfp_env_run_step(cfp_policy* p, cfp_env* e, uint64_t seed, void* stream);
+int32_t* cfp_env_run_actions(const cfp_env* e);
+float* cfp_env_run_logprobs(const cfp_env* e);
+float* cfp_env_run_values(const cfp_env* e);
+uint64_t* cfp_env_run_counter(const cfp_env* e);
 /* cu_train_collect (craftax_full.cu:12980-13016): T rollout steps as above, the bootstrap
  * value on a copy of the live state from the post-rollout observations, GAE and the
  * advantage statistics. */

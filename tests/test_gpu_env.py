@@ -436,3 +436,44 @@ def test_list_reset_in_a_large_env_vector(pkg, cuda):
             compared += 1
     assert compared >= 100, compared
     env.close()
+
+
+@pytest.mark.parametrize("n,small,pool", [(256, False, 0), (512, True, 0), (20480, False, 64)])
+def test_run_step_is_the_rollout_step_without_slabs(pkg, cuda, n, small, pool):
+    """cfp_env_run_step (cu_rollout_step_plain, the reference's `run` mode) against
+    cfp_env_rollout_step on a twin: same worlds, same weights, same seed -- the sampled actions,
+    log-probabilities and values of every step are the slabs' rows, rewards and terminals agree,
+    the device step counter counts the steps, and the env states agree at the end (sampler
+    fused into the 16-env-tile kernel, behind the 32-env-tile forward, and one thread per env
+    above 16 384 envs; regenerated worlds and the pool)."""
+    T = 12
+    twins = []
+    for _ in range(2):
+        env = pkg.Env(n, pool=pool)
+        env.init(3)
+        if pool:
+            env.pool_fill(9)
+        pol = pkg.Policy(n, layers=2, seed=4)
+        if small:
+            pol.set_small_tiles(True)
+        twins.append((env, pol))
+    (env_a, pol_a), (env_b, pol_b) = twins
+    tr = pkg.Trainer(pol_a, T)
+    act, logp, val, ctr = env_b.run_outputs()
+    for t in range(T):
+        env_a.rollout_step(tr, t, 77)
+        env_b.run_step(pol_b, 77)
+        torch.cuda.synchronize()
+        assert torch.equal(tr.buf("r_act")[t], act), f"step {t}: actions"
+        assert torch.equal(tr.buf("r_logprob")[t], logp) and torch.equal(tr.buf("r_value")[t], val), f"step {t}"
+        assert torch.equal(env_a.rewards, env_b.rewards) and torch.equal(env_a.terminals, env_b.terminals), f"step {t}"
+        assert int(ctr[0]) == t + 1
+    assert torch.equal(pol_a.state, pol_b.state)
+    for first in range(0, n, 4096):
+        cnt = min(64, n - first)
+        a = env_a.export_states(eb.STATE_DTYPE, first=first, count=cnt)
+        b = env_b.export_states(eb.STATE_DTYPE, first=first, count=cnt)
+        assert not eb.diff_fields(a, b), f"final states from env {first}"
+    tr.close()
+    for env, pol in twins:
+        pol.close(); env.close()
