@@ -450,7 +450,7 @@ def rollout_in_the_loop(pkg, torch, reps):
     reset, craftax_full.c:3738-3741)."""
     out = {"workload": "rollout_in_the_loop", "policy": "h256x3 fp32", "envs": {}}
     T = 8
-    for n in (8192, 65536, 262144):
+    for n in (1024, 4096, 8192, 65536, 262144):
         res = {}
         for mode, pool in (("fresh_worlds", 0), ("reset_pool", 4096)):
             env = pkg.Env(n, pool=pool)
@@ -461,6 +461,8 @@ def rollout_in_the_loop(pkg, torch, reps):
                 env.step(None)
                 env.reset_from_pool() if pool else env.reset()
             pol = pkg.Policy(n, layers=3, seed=1)
+            if n <= 4096:
+                pol.set_small_tiles(True)
             tr = pkg.Trainer(pol, T)
             state = {"t": 0}
 
@@ -478,6 +480,16 @@ def rollout_in_the_loop(pkg, torch, reps):
             ms_run = _time(torch, lambda: env.run_step(pol, 1234), 64)
             res[mode]["run_mode"] = {"us_per_step": round(ms_run * 1e3, 1), "M_env_steps_per_s": round(n / ms_run / 1e3, 2),
                                      "frac_fp32_peak_of_forward_flops": round(FWD_FLOP * n / (ms_run * 1e-3) / 1e12 / PEAK_FP32, 3)}
+            if n <= 8192:   # ... and replayed from a graph of one step (the reference's graph = 1)
+                side = torch.cuda.Stream()
+                side.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(side):
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph, stream=side):
+                        env.run_step(pol, 1234)
+                    ms_g = _time(torch, graph.replay, 64)
+                torch.cuda.synchronize()
+                res[mode]["run_mode"]["graph_replay_us_per_step"] = round(ms_g * 1e3, 1)
             tr.close()
             pol.close()
             env.close()

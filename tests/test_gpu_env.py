@@ -477,3 +477,56 @@ def test_run_step_is_the_rollout_step_without_slabs(pkg, cuda, n, small, pool):
     tr.close()
     for env, pol in twins:
         pol.close(); env.close()
+
+
+@pytest.mark.parametrize("n,small", [(256, False), (512, True)])
+def test_run_step_replays_from_a_graph(pkg, cuda, n, small):
+    """The reference captures one `run` step into a graph and replays it (cu_run_rollout_bench
+    with graph = 1, craftax_full.cu:12142-12160; "replays are bitwise identical to eager
+    launches").  Same here: one captured cfp_env_run_step replayed twelve times on a side
+    stream, with eager work and synchronisations in between, against an eager twin -- draws,
+    rewards, terminals, the step counter and the policy state after every replay, the env
+    states at the end.  Weakened envs finish inside the run, so replays also regenerate worlds
+    (the finished-env counter is cleared by a kernel of the step, not by a memset node)."""
+    twins = []
+    for _ in range(2):
+        env = pkg.Env(n)
+        env.init(21)
+        weak = env.export_states(eb.STATE_DTYPE)
+        for k, e in enumerate(range(0, n, 5)):
+            weak["player_health"][e] = 1.0 + (k % 3)
+            weak["player_food"][e] = 0
+            weak["player_drink"][e] = 0
+            weak["player_recover"][e] = -14.0 + (k % 5)
+        env.import_states(weak)
+        pol = pkg.Policy(n, layers=2, seed=8)
+        if small:
+            pol.set_small_tiles(True)
+        twins.append((env, pol))
+    (env_e, pol_e), (env_g, pol_g) = twins
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            env_g.run_step(pol_g, 5)
+    torch.cuda.synchronize()
+    out_e, out_g = env_e.run_outputs(), env_g.run_outputs()
+    finished = 0
+    for i in range(12):
+        env_e.run_step(pol_e, 5)
+        with torch.cuda.stream(side):
+            graph.replay()
+        torch.cuda.synchronize()
+        junk = torch.randn(1 << 16, device=cuda).sum().item()   # eager work between replays
+        assert np.isfinite(junk)
+        for a, b, name in zip(out_e, out_g, ("actions", "logprobs", "values", "counter")):
+            assert torch.equal(a, b), f"replay {i}: {name}"
+        assert int(out_g[3][0]) == i + 1       # a capture runs nothing: replay i is step i
+        assert torch.equal(env_e.rewards, env_g.rewards) and torch.equal(env_e.terminals, env_g.terminals)
+        assert torch.equal(pol_e.state, pol_g.state)
+        finished += int(env_g.terminals.sum().item())
+    assert finished > 0
+    assert not eb.diff_fields(env_e.export_states(eb.STATE_DTYPE), env_g.export_states(eb.STATE_DTYPE))
+    for env, pol in twins:
+        pol.close(); env.close()
